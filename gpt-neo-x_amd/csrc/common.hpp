@@ -1,0 +1,200 @@
+// Device-side helpers shared by the softmax and rotary kernels (gfx950, wave64).
+//
+// Everything here assumes a 64-lane wavefront and is compiled for gfx950 only.
+// The translation units are built with -ffp-contract=off: a fused multiply-add
+// appears only where the source says fmaf().
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/neox_hotpath.h"
+
+namespace nhp {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kNegInf = -__builtin_huge_valf();
+
+template <typename To, typename From>
+__device__ __forceinline__ To bitcast(From v)
+{
+    return __builtin_bit_cast(To, v);
+}
+
+// ---------------------------------------------------------------------------
+// 16-bit storage formats. A 32-bit word holds two consecutive elements, the
+// lower-addressed one in bits 0..15.
+// ---------------------------------------------------------------------------
+template <int DT>
+struct Half2;
+
+template <>
+struct Half2<NHP_BF16> {
+    static __device__ __forceinline__ float lo(uint32_t w) { return bitcast<float>(w << 16); }
+    static __device__ __forceinline__ float hi(uint32_t w) { return bitcast<float>(w & 0xffff0000u); }
+    // round-to-nearest-even, v_cvt_pk_bf16_f32 on gfx950
+    static __device__ __forceinline__ uint32_t pack(float a, float b)
+    {
+        f32x2 v = {a, b};
+        return bitcast<uint32_t>(__builtin_convertvector(v, bf16x2));
+    }
+    static __device__ __forceinline__ float round(float a)
+    {
+        return (float)(__bf16)a;
+    }
+    static __device__ __forceinline__ float from_bits(uint16_t h)
+    {
+        return bitcast<float>((uint32_t)h << 16);
+    }
+    static __device__ __forceinline__ uint16_t to_bits(float a)
+    {
+        return bitcast<uint16_t>((__bf16)a);
+    }
+};
+
+template <>
+struct Half2<NHP_F16> {
+    static __device__ __forceinline__ float lo(uint32_t w) { return (float)bitcast<f16x2>(w)[0]; }
+    static __device__ __forceinline__ float hi(uint32_t w) { return (float)bitcast<f16x2>(w)[1]; }
+    // round-to-nearest-even (the wave's default rounding mode), v_cvt_pk_f16_f32
+    static __device__ __forceinline__ uint32_t pack(float a, float b)
+    {
+        f32x2 v = {a, b};
+        return bitcast<uint32_t>(__builtin_convertvector(v, f16x2));
+    }
+    static __device__ __forceinline__ float round(float a)
+    {
+        return (float)(_Float16)a;
+    }
+    static __device__ __forceinline__ float from_bits(uint16_t h)
+    {
+        return (float)bitcast<_Float16>(h);
+    }
+    static __device__ __forceinline__ uint16_t to_bits(float a)
+    {
+        return bitcast<uint16_t>((_Float16)a);
+    }
+};
+
+// Unpack the eight elements of a 16-byte chunk.
+template <int DT>
+__device__ __forceinline__ void unpack8(const u32x4& raw, float (&f)[8])
+{
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        f[2 * i] = Half2<DT>::lo(raw[i]);
+        f[2 * i + 1] = Half2<DT>::hi(raw[i]);
+    }
+}
+
+template <int DT>
+__device__ __forceinline__ u32x4 pack8(const float (&f)[8])
+{
+    u32x4 r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r[i] = Half2<DT>::pack(f[2 * i], f[2 * i + 1]);
+    return r;
+}
+
+// ---------------------------------------------------------------------------
+// Streaming global memory access: every byte of these tensors is touched once,
+// so loads and stores carry the non-temporal hint.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ u32x4 load16_stream(const void* p)
+{
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+}
+__device__ __forceinline__ void store16_stream(void* p, u32x4 v)
+{
+    __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
+}
+__device__ __forceinline__ u32x4 load16(const void* p)
+{
+    return *reinterpret_cast<const u32x4*>(p);
+}
+__device__ __forceinline__ u32x2 load8(const void* p)
+{
+    return *reinterpret_cast<const u32x2*>(p);
+}
+
+// ---------------------------------------------------------------------------
+// Cross-lane reductions over groups of L consecutive lanes (L a power of two,
+// 1..64). Lanes 2^k apart are combined with DPP controls inside a row of 16
+// lanes, ds_swizzle for the 16<->16 exchange and v_readlane for the two
+// halves of the wave. Every lane of the group ends up with the group result.
+// ---------------------------------------------------------------------------
+struct OpMax {
+    static __device__ __forceinline__ float apply(float a, float b) { return fmaxf(a, b); }
+};
+struct OpSum {
+    static __device__ __forceinline__ float apply(float a, float b) { return a + b; }
+};
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v)
+{
+    return bitcast<float>(
+        __builtin_amdgcn_update_dpp(0, bitcast<int>(v), CTRL, 0xF, 0xF, true));
+}
+
+template <typename Op, int L>
+__device__ __forceinline__ float group_reduce(float v)
+{
+    static_assert(L >= 1 && L <= 64 && (L & (L - 1)) == 0, "L must be a power of two <= 64");
+    if constexpr (L >= 2) v = Op::apply(v, dpp_move<0xB1>(v));   // quad_perm [1,0,3,2]
+    if constexpr (L >= 4) v = Op::apply(v, dpp_move<0x4E>(v));   // quad_perm [2,3,0,1]
+    if constexpr (L >= 8) v = Op::apply(v, dpp_move<0x141>(v));  // row_half_mirror
+    if constexpr (L >= 16) v = Op::apply(v, dpp_move<0x140>(v)); // row_mirror
+    if constexpr (L >= 32) {
+        // swap lanes i and i^16 (bit-mode swizzle: and 0x1f, or 0, xor 0x10)
+        v = Op::apply(v, bitcast<float>(__builtin_amdgcn_ds_swizzle(bitcast<int>(v), 0x401F)));
+    }
+    if constexpr (L >= 64) {
+        float a = bitcast<float>(__builtin_amdgcn_readlane(bitcast<int>(v), 0));
+        float b = bitcast<float>(__builtin_amdgcn_readlane(bitcast<int>(v), 32));
+        v = Op::apply(a, b);
+    }
+    return v;
+}
+
+// Combine the per-wave partials of the W waves of a workgroup through LDS.
+// `slots` must hold at least W floats and must not be reused for another
+// reduction before a later barrier.
+template <typename Op, int W>
+__device__ __forceinline__ float block_combine(float v, float* slots, int wave, int lane)
+{
+    if constexpr (W == 1) {
+        return v;
+    } else {
+        if (lane == 0) slots[wave] = v;
+        __syncthreads();
+        float r = slots[0];
+#pragma unroll
+        for (int i = 1; i < W; ++i) r = Op::apply(r, slots[i]);
+        return r;
+    }
+}
+
+// The hardware schedules consecutive workgroup ids round-robin over the 8
+// XCDs, each of which has a private L2. This maps the hardware id to a logical
+// id such that consecutive logical ids share an XCD (and so its L2).
+__device__ __forceinline__ uint32_t xcd_swizzle(uint32_t hw_id, uint32_t total)
+{
+    constexpr uint32_t kXcd = 8;
+    const uint32_t full = total - total % kXcd;
+    if (hw_id >= full) return hw_id;
+    return (hw_id % kXcd) * (full / kXcd) + hw_id / kXcd;
+}
+
+// 2^(x) with the raw v_exp_f32 instruction (about 1 ulp, no denormal results).
+__device__ __forceinline__ float exp2_raw(float x) { return __builtin_amdgcn_exp2f(x); }
+
+}  // namespace nhp

@@ -1,0 +1,105 @@
+"""Extension-module surface of the fused rotary positional embedding.
+
+Same functions as the reference's pybind module
+(megatron/fused_kernels/fused_rotary_positional_embedding.cpp:129-139), served
+by libneox_hotpath.so. The input may have arbitrary strides; the output is a
+new contiguous [s,b,h,d] tensor, or [b,s,h,d] storage viewed as [s,b,h,d] when
+``transpose_output`` is set. Launches are asynchronous on the current stream.
+"""
+import torch
+
+from megatron.fused_kernels import _hotpath as _hp
+
+_FLOATS = (torch.float16, torch.bfloat16, torch.float32)
+
+
+def _check(cond, msg):
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _new_output(t, transpose_output):
+    s, b, h, d = t.shape
+    if transpose_output:
+        return torch.empty((b, s, h, d), dtype=t.dtype, device=t.device).transpose(0, 1)
+    return torch.empty((s, b, h, d), dtype=t.dtype, device=t.device)
+
+
+def _run_freqs(name, fn, t, freqs, transpose_output, what):
+    # argument checks of fused_rotary_positional_embedding.cpp:39-73
+    _check(t.dim() == 4, "expected 4D tensor")
+    _check(freqs.dim() == 4, "expected 4D tensor")
+    _check(t.size(0) == freqs.size(0), f"expected {what} and freqs tensor have the same sequence length")
+    _check(freqs.size(1) == 1 and freqs.size(2) == 1,
+           "expected the second and third dims of the freqs tensor equal 1")
+    _check(t.size(3) >= freqs.size(3),
+           f"expected the last dim of the {what} tensor equals or is greater than the freqs tensor")
+    _check(freqs.dtype == torch.float32, "Dtype of the freqs tensor must be float")
+    _check(t.dtype in _FLOATS, f"{name}: unsupported dtype {t.dtype}")
+    _hp.require_gpu(t, name)
+    _hp.require_gpu(freqs, name)
+    t = t.detach()
+    f = freqs.detach().contiguous()
+    out = _new_output(t, transpose_output)
+    s, b, h, d = t.shape
+    with torch.cuda.device(t.device):
+        rc = fn(out.data_ptr(), t.data_ptr(), f.data_ptr(), s, b, h, d, f.size(3), _hp.strides4(t),
+                _hp.strides4(out), _hp.dtype_code(t, name), _hp.stream_of(t))
+    _hp.check(rc, name)
+    return out
+
+
+def _run_cached(name, fn, t, cos, sin, transpose_output, what):
+    # argument checks of fused_rotary_positional_embedding.cpp:75-125
+    _check(t.dim() == 4, "expected 4D tensor")
+    _check(cos.dim() == 4, "expected 4D tensor")
+    _check(sin.dim() == 4, "expected 4D tensor")
+    _check(t.size(0) == cos.size(0), f"expected {what} and cos tensor have the same sequence length")
+    _check(t.size(0) == sin.size(0), f"expected {what} and sin tensor have the same sequence length")
+    _check(cos.size(1) == 1 and cos.size(2) == 1, "expected the second and third dims of the cos tensor equal 1")
+    _check(sin.size(1) == 1 and sin.size(2) == 1, "expected the second and third dims of the sin tensor equal 1")
+    _check(cos.size(3) == sin.size(3), "expected cos and sin tensor have the same last dim")
+    _check(t.size(3) >= cos.size(3),
+           f"expected the last dim of the {what} tensor equals or is greater than the cos tensor")
+    _check(cos.dtype == sin.dtype, "expected cos and sin tensor have the same dtype")
+    _check(t.dtype in _FLOATS, f"{name}: unsupported dtype {t.dtype}")
+    _check(cos.dtype == torch.float32 or cos.dtype == t.dtype,
+           f"{name}: cos/sin must be float32 or have the dtype of the input")
+    _hp.require_gpu(t, name)
+    _hp.require_gpu(cos, name)
+    _hp.require_gpu(sin, name)
+    t = t.detach()
+    c = cos.detach().contiguous()
+    sn = sin.detach().contiguous()
+    out = _new_output(t, transpose_output)
+    s, b, h, d = t.shape
+    with torch.cuda.device(t.device):
+        rc = fn(out.data_ptr(), t.data_ptr(), c.data_ptr(), sn.data_ptr(), s, b, h, d, c.size(3),
+                _hp.strides4(t), _hp.strides4(out), _hp.dtype_code(t, name), _hp.dtype_code(c, name),
+                _hp.stream_of(t))
+    _hp.check(rc, name)
+    return out
+
+
+def forward(input, freqs, transpose_output):
+    """Rotate ``input`` [s,b,h,d] by the fp32 angles ``freqs`` [s,1,1,d2]."""
+    return _run_freqs("fused_rotary_positional_embedding.forward", _hp.lib().nhp_rope_freqs_fwd, input, freqs,
+                      transpose_output, "input")
+
+
+def backward(output_grads, freqs, transpose_output):
+    """Gradient of ``forward`` w.r.t. its input."""
+    return _run_freqs("fused_rotary_positional_embedding.backward", _hp.lib().nhp_rope_freqs_bwd, output_grads,
+                      freqs, transpose_output, "output_grads")
+
+
+def forward_cached(input, cos, sin, transpose_output):
+    """Rotate ``input`` [s,b,h,d] with cached ``cos``/``sin`` [s,1,1,d2]."""
+    return _run_cached("fused_rotary_positional_embedding.forward_cached", _hp.lib().nhp_rope_cached_fwd, input,
+                       cos, sin, transpose_output, "input")
+
+
+def backward_cached(output_grads, cos, sin, transpose_output):
+    """Gradient of ``forward_cached`` w.r.t. its input."""
+    return _run_cached("fused_rotary_positional_embedding.backward_cached", _hp.lib().nhp_rope_cached_bwd,
+                       output_grads, cos, sin, transpose_output, "output_grads")

@@ -1,0 +1,108 @@
+"""ctypes binding of libneox_hotpath.so (the C ABI declared in include/neox_hotpath.h).
+
+The library is the only implementation: if it cannot be loaded an ImportError
+is raised, there is no fallback of any kind.
+"""
+import ctypes
+import os
+import subprocess
+import threading
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libneox_hotpath.so")
+CSRC_DIR = os.path.normpath(os.path.join(_HERE, "..", "..", "csrc"))
+
+F16, BF16, F32 = 0, 1, 2
+_DTYPE = {torch.float16: F16, torch.bfloat16: BF16, torch.float32: F32}
+
+ABI_VERSION = 1
+
+_lock = threading.Lock()
+_lib = None
+
+
+def build(force=False, verbose=False):
+    """Compile the HIP sources for gfx950 with hipcc (``make`` in csrc/)."""
+    cmd = ["make", "-C", CSRC_DIR, "-j4"] + (["-B"] if force else [])
+    out = None if verbose else subprocess.DEVNULL
+    subprocess.run(cmd, check=True, stdout=out, stderr=None if verbose else subprocess.PIPE)
+    return LIB_PATH
+
+
+def _declare(lib):
+    i64, vp, f32, ci = ctypes.c_int64, ctypes.c_void_p, ctypes.c_float, ctypes.c_int
+    p64 = ctypes.POINTER(i64)
+    sigs = {
+        "nhp_abi_version": ([], ci),
+        "nhp_status_string": ([ci], ctypes.c_char_p),
+        "nhp_softmax_max_resident_row": ([], i64),
+        "nhp_causal_softmax_fwd": ([vp, vp, f32, i64, i64, ci, vp], ci),
+        "nhp_causal_softmax_bwd": ([vp, vp, vp, f32, i64, i64, ci, vp], ci),
+        "nhp_masked_softmax_fwd": ([vp, vp, vp, f32, i64, i64, i64, i64, i64, ci, vp], ci),
+        "nhp_masked_softmax_bwd": ([vp, vp, vp, f32, i64, i64, ci, vp], ci),
+        "nhp_softmax_batch_per_block": ([i64, i64, i64, i64], ci),
+        "nhp_rope_cached_fwd": ([vp, vp, vp, vp, i64, i64, i64, i64, i64, p64, p64, ci, ci, vp], ci),
+        "nhp_rope_cached_bwd": ([vp, vp, vp, vp, i64, i64, i64, i64, i64, p64, p64, ci, ci, vp], ci),
+        "nhp_rope_freqs_fwd": ([vp, vp, vp, i64, i64, i64, i64, i64, p64, p64, ci, vp], ci),
+        "nhp_rope_freqs_bwd": ([vp, vp, vp, i64, i64, i64, i64, i64, p64, p64, ci, vp], ci),
+    }
+    for name, (args, res) in sigs.items():
+        fn = getattr(lib, name)  # AttributeError if the symbol is missing
+        fn.argtypes = args
+        fn.restype = res
+    return sigs
+
+
+EXPORTS = None
+
+
+def lib():
+    """The loaded library; raises ImportError when it is absent or stale."""
+    global _lib, EXPORTS
+    if _lib is None:
+        with _lock:
+            if _lib is None:
+                if not os.path.exists(LIB_PATH):
+                    raise ImportError(
+                        f"{LIB_PATH} not found: the fused kernels are not built. "
+                        "Run `from megatron.fused_kernels import load; load()`."
+                    )
+                try:
+                    handle = ctypes.CDLL(LIB_PATH)
+                    EXPORTS = _declare(handle)
+                except (OSError, AttributeError) as e:
+                    raise ImportError(f"cannot load {LIB_PATH}: {e}") from e
+                if handle.nhp_abi_version() != ABI_VERSION:
+                    raise ImportError(
+                        f"{LIB_PATH} has ABI version {handle.nhp_abi_version()}, expected {ABI_VERSION}; rebuild it"
+                    )
+                _lib = handle
+    return _lib
+
+
+def check(status, what):
+    if status != 0:
+        msg = lib().nhp_status_string(status).decode()
+        raise RuntimeError(f"{what}: {msg} (status {status})")
+
+
+def dtype_code(t, what):
+    try:
+        return _DTYPE[t.dtype]
+    except KeyError:
+        raise RuntimeError(f"{what}: unsupported dtype {t.dtype}") from None
+
+
+def require_gpu(t, what):
+    if t.device.type != "cuda":
+        raise RuntimeError(f"{what}: expected a tensor on the GPU, got device {t.device}")
+
+
+def stream_of(t):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def strides4(t):
+    return (ctypes.c_int64 * 4)(*t.stride())

@@ -1,0 +1,62 @@
+"""Extension-module surface of the causal fused softmax.
+
+Same functions as the reference's pybind module
+(megatron/fused_kernels/scaled_upper_triang_masked_softmax.cpp:62-70), served
+by libneox_hotpath.so. Launches are asynchronous on the current stream.
+"""
+import torch
+
+from megatron.fused_kernels import _hotpath as _hp
+
+_HALF = (torch.float16, torch.bfloat16)
+
+
+def forward(input, scale_factor):
+    """softmax(scale * input) under an upper-triangular mask.
+
+    input: [attn_batches, seq_len, seq_len] fp16/bf16 on the GPU. Returns a new
+    tensor of the same shape and dtype (requires_grad False). Checks follow
+    scaled_upper_triang_masked_softmax.cpp:31-39; seq_len is not limited to 2048.
+    """
+    if input.dim() != 3:
+        raise RuntimeError("expected 3D tensor")
+    if input.dtype not in _HALF:
+        raise RuntimeError("Only fp16 and bf16 are supported")
+    if input.size(1) != input.size(2):
+        raise RuntimeError("expected a square [attn_batches, seq_len, seq_len] tensor")
+    _hp.require_gpu(input, "scaled_upper_triang_masked_softmax_cuda.forward")
+    x = input.detach().contiguous()
+    y = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        rc = _hp.lib().nhp_causal_softmax_fwd(
+            y.data_ptr(), x.data_ptr(), float(scale_factor), x.size(0), x.size(1), _hp.dtype_code(x, "forward"),
+            _hp.stream_of(x))
+    _hp.check(rc, "scaled_upper_triang_masked_softmax_cuda.forward")
+    return y
+
+
+def backward(output_grads, softmax_results, scale_factor):
+    """Gradient w.r.t. the input of ``forward``.
+
+    Works in place: the result is written into (the contiguous version of)
+    ``output_grads`` and that tensor is returned, as in
+    scaled_upper_triang_masked_softmax_cuda.cu:61-90.
+    """
+    if output_grads.dim() != 3 or softmax_results.dim() != 3:
+        raise RuntimeError("expected 3D tensor")
+    if output_grads.dtype not in _HALF or softmax_results.dtype not in _HALF:
+        raise RuntimeError("Only fp16 and bf16 are supported")
+    if output_grads.shape != softmax_results.shape or output_grads.dtype != softmax_results.dtype:
+        raise RuntimeError("output_grads and softmax_results must have the same shape and dtype")
+    if output_grads.size(1) != output_grads.size(2):
+        raise RuntimeError("expected a square [attn_batches, seq_len, seq_len] tensor")
+    _hp.require_gpu(output_grads, "scaled_upper_triang_masked_softmax_cuda.backward")
+    _hp.require_gpu(softmax_results, "scaled_upper_triang_masked_softmax_cuda.backward")
+    g = output_grads.detach().contiguous()
+    y = softmax_results.detach().contiguous()
+    with torch.cuda.device(g.device):
+        rc = _hp.lib().nhp_causal_softmax_bwd(
+            g.data_ptr(), g.data_ptr(), y.data_ptr(), float(scale_factor), g.size(0), g.size(1),
+            _hp.dtype_code(g, "backward"), _hp.stream_of(g))
+    _hp.check(rc, "scaled_upper_triang_masked_softmax_cuda.backward")
+    return g

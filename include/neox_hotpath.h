@@ -1,0 +1,199 @@
+/*
+ * neox_hotpath.h -- C ABI of libneox_hotpath.so
+ *
+ * MI355X (gfx950) implementation of the three GPT-NeoX fused kernels:
+ * scaled upper-triangular (causal) masked softmax, scaled padding-masked
+ * softmax and fused rotary positional embedding, forward and backward.
+ *
+ * Conventions shared by every entry point
+ *   - all tensor arguments are raw DEVICE pointers; the library never
+ *     allocates, frees, retains or synchronises on them;
+ *   - sizes and strides are int64_t, strides are counted in ELEMENTS;
+ *   - `dtype` is an nhp_dtype value; `stream` is a hipStream_t passed as
+ *     void* (NULL = the legacy default stream);
+ *   - the call only enqueues work on `stream` and returns; the return value
+ *     is NHP_OK (0) or a negative nhp_status; nothing is launched when an
+ *     error is returned; no C++ exception crosses the boundary;
+ *   - the library keeps no mutable global state and is safe to call from
+ *     several host threads at once (forward from the main thread, backward
+ *     from autograd worker threads).
+ *
+ * Each declaration cites the reference interface it replaces; paths are
+ * relative to the GPT-NeoX source tree.
+ */
+#ifndef NEOX_HOTPATH_H
+#define NEOX_HOTPATH_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum nhp_dtype {
+    NHP_F16 = 0,  /* IEEE binary16 */
+    NHP_BF16 = 1, /* bfloat16 */
+    NHP_F32 = 2   /* IEEE binary32 (rotary only) */
+} nhp_dtype;
+
+typedef enum nhp_status {
+    NHP_OK = 0,
+    NHP_ERR_DTYPE = -1,     /* dtype not supported by this entry point */
+    NHP_ERR_SHAPE = -2,     /* a size is negative / inconsistent / beyond the supported range */
+    NHP_ERR_NULL = -3,      /* a required pointer is NULL while the tensor is not empty */
+    NHP_ERR_PAD_BATCHES = -4, /* mask batch dimension is neither 1 nor b */
+    NHP_ERR_LAUNCH = -5,    /* hipGetLastError() reported a launch failure */
+    NHP_ERR_ALIAS = -6      /* an output overlaps an input where that is not allowed */
+} nhp_status;
+
+/* Library ABI version (bumped when a signature changes). */
+int nhp_abi_version(void);
+
+/* Static, human readable text for an nhp_status value. Never NULL. */
+const char* nhp_status_string(int status);
+
+/* Longest softmax row (sk) the register-resident kernels accept; longer rows
+ * take a slower streaming kernel but are still supported. */
+int64_t nhp_softmax_max_resident_row(void);
+
+/* ------------------------------------------------------------------------
+ * Scaled upper-triangular (causal) masked softmax
+ * ---------------------------------------------------------------------- */
+
+/*
+ * y[a, q, k] = softmax_k( scale * x[a, q, k] ) over k <= q,  +0 for k > q.
+ * x, y: contiguous [attn_batches, seq_len, seq_len], fp16 or bf16; fp32
+ * accumulation; elements k > q of x are never read.
+ * y may alias x exactly (in-place) but must not partially overlap it.
+ *
+ * Replaces scaled_upper_triang_masked_softmax_cuda.forward
+ *   megatron/fused_kernels/scaled_upper_triang_masked_softmax.cpp:31-39
+ *   megatron/fused_kernels/scaled_upper_triang_masked_softmax_cuda.cu:33-59
+ *   kernel megatron/fused_kernels/scaled_upper_triang_masked_softmax.h:143-260
+ * The reference's seq_len <= 2048 limit does not apply.
+ */
+int nhp_causal_softmax_fwd(void* y, const void* x, float scale,
+                           int64_t attn_batches, int64_t seq_len,
+                           int dtype, void* stream);
+
+/*
+ * dx[a, q, k] = scale * ( dy*y - y * sum_{j<=q} dy[j]*y[j] ) for k <= q,
+ * +0 for k > q.  dy, y, dx: contiguous [attn_batches, seq_len, seq_len].
+ * dx may alias dy exactly (the reference always works in place on dy).
+ *
+ * Replaces scaled_upper_triang_masked_softmax_cuda.backward
+ *   megatron/fused_kernels/scaled_upper_triang_masked_softmax.cpp:41-56
+ *   megatron/fused_kernels/scaled_upper_triang_masked_softmax_cuda.cu:61-90
+ *   kernel megatron/fused_kernels/scaled_upper_triang_masked_softmax.h:262-361
+ */
+int nhp_causal_softmax_bwd(void* dx, const void* dy, const void* y, float scale,
+                           int64_t attn_batches, int64_t seq_len,
+                           int dtype, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Scaled padding-masked softmax
+ * ---------------------------------------------------------------------- */
+
+/*
+ * z = (mask == 1) ? -10000 : scale * x ;  y = softmax over the last dim.
+ * x, y: contiguous [b, np, sq, sk], fp16 or bf16.
+ * mask: contiguous [pad_batches, 1, sq, sk], one byte per element (bool or
+ * uint8; only the value 1 masks), pad_batches is 1 (shared by all batches)
+ * or b. A fully masked row yields the uniform distribution 1/sk.
+ *
+ * Replaces scaled_masked_softmax_cuda.forward
+ *   megatron/fused_kernels/scaled_masked_softmax.cpp:33-42
+ *   megatron/fused_kernels/scaled_masked_softmax_cuda.cu:38-76
+ *   kernel megatron/fused_kernels/scaled_masked_softmax.h:117-238
+ * The reference's sk <= 2048 limit does not apply.
+ */
+int nhp_masked_softmax_fwd(void* y, const void* x, const uint8_t* mask, float scale,
+                           int64_t b, int64_t np, int64_t sq, int64_t sk,
+                           int64_t pad_batches, int dtype, void* stream);
+
+/*
+ * dx = scale * ( dy*y - y * sum_k dy*y ) per row; no mask is applied.
+ * dy, y, dx: contiguous, `rows` rows of `sk` elements (rows = b*np*sq).
+ * dx may alias dy exactly.
+ *
+ * Replaces scaled_masked_softmax_cuda.backward
+ *   megatron/fused_kernels/scaled_masked_softmax.cpp:44-59
+ *   megatron/fused_kernels/scaled_masked_softmax_cuda.cu:78-108
+ *   kernel megatron/fused_kernels/scaled_masked_softmax.h:240-335
+ */
+int nhp_masked_softmax_bwd(void* dx, const void* dy, const void* y, float scale,
+                           int64_t rows, int64_t sk, int dtype, void* stream);
+
+/*
+ * Rows handled per 128-thread block by the reference's launch geometry on a
+ * 64-wide wavefront; only used by FusedScaleMaskSoftmax.is_kernel_available.
+ * Returns a value >= 1, or a negative nhp_status if key_seq_len < 1.
+ *
+ * Replaces scaled_masked_softmax_cuda.get_batch_per_block
+ *   megatron/fused_kernels/scaled_masked_softmax.cpp:61-64
+ *   megatron/fused_kernels/scaled_masked_softmax.h:338-352
+ */
+int nhp_softmax_batch_per_block(int64_t query_seq_len, int64_t key_seq_len,
+                                int64_t batches, int64_t attn_heads);
+
+/* ------------------------------------------------------------------------
+ * Fused rotary positional embedding (rotate-half form), sbhd layout
+ * ---------------------------------------------------------------------- */
+
+/*
+ * For i < d2, h2 = d2/2:
+ *   forward : out_i = in_i (*) c_i (+) rot_i (*) s_i,
+ *             rot_i = (i < d2-h2) ? -in[i+h2] : in[i+h2-d2]
+ *   backward: out_i = in_i (*) c_i (+) in[partner] (*) s'_i,
+ *             s'_i  = (i < d2-h2) ? s[i+h2] : -s[i+h2-d2]
+ * where c = cos[s_idx, i], s = sin[s_idx, i] are first converted to the data
+ * dtype and (*) / (+) round to the data dtype after every operation (the
+ * arithmetic of the 16-bit scalar types in the reference and of eager torch).
+ * For d2 <= i < d the element is copied.
+ *
+ * in : [s, b, h, d] with arbitrary element strides in_stride[4];
+ * out: [s, b, h, d] with arbitrary element strides out_stride[4] (a
+ *      contiguous sbhd or bshd buffer in the reference); must not overlap in;
+ * cos, sin: contiguous [s, d2]; cs_dtype is NHP_F32 or equal to dtype.
+ * dtype: NHP_F16, NHP_BF16 or NHP_F32.
+ *
+ * Replaces fused_rotary_positional_embedding.forward_cached / backward_cached
+ *   megatron/fused_kernels/fused_rotary_positional_embedding.cpp:75-125
+ *   megatron/fused_kernels/fused_rotary_positional_embedding_cuda.cu:218-335
+ *   kernels megatron/fused_kernels/fused_rotary_positional_embedding.h:126-225
+ */
+int nhp_rope_cached_fwd(void* out, const void* in, const void* cos, const void* sin,
+                        int64_t s, int64_t b, int64_t h, int64_t d, int64_t d2,
+                        const int64_t in_stride[4], const int64_t out_stride[4],
+                        int dtype, int cs_dtype, void* stream);
+
+int nhp_rope_cached_bwd(void* out, const void* in, const void* cos, const void* sin,
+                        int64_t s, int64_t b, int64_t h, int64_t d, int64_t d2,
+                        const int64_t in_stride[4], const int64_t out_stride[4],
+                        int dtype, int cs_dtype, void* stream);
+
+/*
+ * Same, with c = cosf(freqs[s_idx, i]) and s = sinf(freqs[s_idx, i]) evaluated
+ * on the device in fp32 and then converted to the data dtype.
+ * freqs: contiguous fp32 [s, d2].
+ *
+ * Replaces fused_rotary_positional_embedding.forward / backward
+ *   megatron/fused_kernels/fused_rotary_positional_embedding.cpp:39-73
+ *   megatron/fused_kernels/fused_rotary_positional_embedding_cuda.cu:24-137
+ *   kernels megatron/fused_kernels/fused_rotary_positional_embedding.h:27-124
+ */
+int nhp_rope_freqs_fwd(void* out, const void* in, const float* freqs,
+                       int64_t s, int64_t b, int64_t h, int64_t d, int64_t d2,
+                       const int64_t in_stride[4], const int64_t out_stride[4],
+                       int dtype, void* stream);
+
+int nhp_rope_freqs_bwd(void* out, const void* in, const float* freqs,
+                       int64_t s, int64_t b, int64_t h, int64_t d, int64_t d2,
+                       const int64_t in_stride[4], const int64_t out_stride[4],
+                       int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* NEOX_HOTPATH_H */

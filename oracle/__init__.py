@@ -1,0 +1,152 @@
+"""TEST INFRASTRUCTURE -- NOT PART OF THE PRODUCT.
+
+CPU oracle for the fused softmax / rotary hot path. Two restatements live here:
+
+* ``kernel_semantics.c`` (this module's ctypes wrappers): what the reference's
+  CUDA kernels compute, element by element, in plain C.
+* ``fallback_semantics.py``: the reference's own torch fallback
+  (``FusedScaleMaskSoftmax.forward_torch_softmax``, the eager rotary functions
+  and the ``RotaryEmbedding`` cache recipe).
+
+Only ``tests/``, ``__graft_entry__.smoke()`` and ``bench.py``'s cpu_baseline leg
+may import this package, and only as the checker. The product package never
+does; it raises when its HIP library is missing.
+
+All wrappers take and return CPU ``torch`` tensors.
+"""
+import ctypes
+import os
+import subprocess
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liboracle.so")
+
+DT_F16, DT_BF16, DT_F32 = 0, 1, 2
+_DT = {torch.float16: DT_F16, torch.bfloat16: DT_BF16, torch.float32: DT_F32}
+
+
+def build(force=False):
+    """Compile liboracle.so with gcc (a few hundred milliseconds)."""
+    cmd = ["make", "-C", _HERE] + (["-B"] if force else [])
+    subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL)
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        L = ctypes.CDLL(_LIB_PATH)
+        i64, vp, f32, ci = ctypes.c_int64, ctypes.c_void_p, ctypes.c_float, ctypes.c_int
+        L.oracle_causal_softmax_fwd.argtypes = [vp, vp, f32, i64, i64, ci]
+        L.oracle_masked_softmax_fwd.argtypes = [vp, vp, vp, f32, i64, i64, i64, i64, i64, ci]
+        L.oracle_softmax_bwd.argtypes = [vp, vp, vp, f32, i64, i64, i64, ci, ci]
+        L.oracle_batch_per_block.argtypes = [i64, ci]
+        p64 = ctypes.POINTER(i64)
+        L.oracle_rope_cached.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, p64, p64, ci, ci, ci]
+        L.oracle_rope_freqs.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, p64, p64, ci, ci]
+        L.oracle_float_to_bf16.argtypes = [f32]
+        L.oracle_float_to_bf16.restype = ctypes.c_uint16
+        L.oracle_float_to_f16.argtypes = [f32]
+        L.oracle_float_to_f16.restype = ctypes.c_uint16
+        L.oracle_bf16_to_float.argtypes = [ctypes.c_uint16]
+        L.oracle_bf16_to_float.restype = f32
+        L.oracle_f16_to_float.argtypes = [ctypes.c_uint16]
+        L.oracle_f16_to_float.restype = f32
+        _lib = L
+    return _lib
+
+
+def _check(rc, what):
+    if rc != 0:
+        raise RuntimeError(f"oracle {what} failed with code {rc}")
+
+
+def _cpu_contig(t):
+    assert t.device.type == "cpu", "the oracle works on CPU tensors"
+    return t.contiguous()
+
+
+def causal_softmax_fwd(x, scale):
+    """x: [attn_batches, s, s] fp16/bf16 -> probabilities, same shape and dtype."""
+    assert x.dim() == 3 and x.size(1) == x.size(2)
+    x = _cpu_contig(x)
+    y = torch.empty_like(x)
+    _check(lib().oracle_causal_softmax_fwd(y.data_ptr(), x.data_ptr(), float(scale), x.size(0), x.size(1),
+                                           _DT[x.dtype]), "causal_softmax_fwd")
+    return y
+
+
+def masked_softmax_fwd(x, mask, scale):
+    """x: [b, np, sq, sk]; mask: [1 or b, 1, sq, sk] bool/uint8 (value 1 masks)."""
+    assert x.dim() == 4 and mask.dim() == 4
+    x = _cpu_contig(x)
+    m = _cpu_contig(mask).view(torch.uint8) if mask.dtype == torch.bool else _cpu_contig(mask)
+    assert m.dtype == torch.uint8
+    b, np_, sq, sk = x.shape
+    assert m.size(1) == 1 and m.size(2) == sq and m.size(3) == sk
+    y = torch.empty_like(x)
+    _check(lib().oracle_masked_softmax_fwd(y.data_ptr(), x.data_ptr(), m.data_ptr(), float(scale), b, np_, sq,
+                                           sk, m.size(0), _DT[x.dtype]), "masked_softmax_fwd")
+    return y
+
+
+def softmax_bwd(dy, y, scale, causal):
+    """Returns dx (a new tensor). dy, y: [..., rows_per_matrix, n]."""
+    dy = _cpu_contig(dy)
+    y = _cpu_contig(y)
+    assert dy.shape == y.shape and dy.dtype == y.dtype
+    n = dy.size(-1)
+    rows = dy.numel() // max(n, 1)
+    dx = torch.empty_like(dy)
+    _check(lib().oracle_softmax_bwd(dx.data_ptr(), dy.data_ptr(), y.data_ptr(), float(scale), rows, n,
+                                    dy.size(-2), 1 if causal else 0, _DT[dy.dtype]), "softmax_bwd")
+    return dx
+
+
+def batch_per_block(sk, warp=64):
+    return lib().oracle_batch_per_block(int(sk), int(warp))
+
+
+def _strides4(t):
+    return (ctypes.c_int64 * 4)(*t.stride())
+
+
+def _rope_out(t, transpose_output):
+    s, b, h, d = t.shape
+    if transpose_output:
+        return torch.empty((b, s, h, d), dtype=t.dtype).transpose(0, 1)
+    return torch.empty((s, b, h, d), dtype=t.dtype)
+
+
+def rope_cached(t, cos, sin, backward=False, transpose_output=False):
+    """t: [s,b,h,d] (any strides); cos, sin: [s,1,1,d2] fp32 or t.dtype."""
+    assert t.device.type == "cpu" and t.dim() == 4
+    cos = _cpu_contig(cos)
+    sin = _cpu_contig(sin)
+    s, b, h, d = t.shape
+    d2 = cos.size(3)
+    out = _rope_out(t, transpose_output)
+    _check(lib().oracle_rope_cached(out.data_ptr(), t.data_ptr(), cos.data_ptr(), sin.data_ptr(), s, b, h, d,
+                                    d2, _strides4(t), _strides4(out), _DT[t.dtype], _DT[cos.dtype],
+                                    1 if backward else 0), "rope_cached")
+    return out
+
+
+def rope_freqs(t, freqs, backward=False, transpose_output=False):
+    """t: [s,b,h,d]; freqs: [s,1,1,d2] fp32 angles."""
+    assert t.device.type == "cpu" and t.dim() == 4 and freqs.dtype == torch.float32
+    freqs = _cpu_contig(freqs)
+    s, b, h, d = t.shape
+    d2 = freqs.size(3)
+    out = _rope_out(t, transpose_output)
+    _check(lib().oracle_rope_freqs(out.data_ptr(), t.data_ptr(), freqs.data_ptr(), s, b, h, d, d2,
+                                   _strides4(t), _strides4(out), _DT[t.dtype], 1 if backward else 0),
+           "rope_freqs")
+    return out

@@ -1,0 +1,332 @@
+/*
+ * TEST INFRASTRUCTURE -- NOT PART OF THE PRODUCT.
+ *
+ * Plain-C, single-threaded restatement of what the GPT-NeoX fused CUDA kernels
+ * compute (scaled causal softmax, scaled padding-masked softmax, fused rotary
+ * embedding; forward and backward). Only tests/, __graft_entry__.smoke() and
+ * bench.py's cpu_baseline leg may load this library, and only as the checker.
+ * Nothing under the product package imports, links or executes it.
+ *
+ * Each function cites the reference source it follows (paths relative to the
+ * GPT-NeoX tree). Storage is fp16/bf16 (raw uint16_t bit patterns) or fp32;
+ * all arithmetic is IEEE binary32, written so that no fused multiply-add is
+ * formed (build with -ffp-contract=off), rounding to storage is to nearest even.
+ *
+ * Two documented choices where the reference leaves freedom or is inconsistent:
+ *   - row sums are accumulated pairwise in fp32 (the reference sums per lane and
+ *     then butterflies across the warp; any order is within a few fp32 ulp);
+ *   - the forward `scale` is applied as the fp32 value handed in. The CUDA
+ *     dispatcher narrows it to the input dtype first
+ *     (scaled_upper_triang_masked_softmax.h:368, scaled_masked_softmax.h:358);
+ *     pass an already narrowed value to reproduce that.
+ *
+ * How this oracle is pinned (tests/test_oracle_*.py): closed forms (row 0 of a
+ * causal softmax is [1,0,...], constant rows give 1/(q+1), fully masked rows
+ * give 1/sk), invariants (rows sum to 1, shift invariance, gradient rows sum to
+ * 0, rotations preserve pair norms and compose to the identity, backward is the
+ * adjoint of forward), brute force in float64 on tiny inputs, and the torch
+ * library routines the reference's own Python fallback is made of.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+enum { DT_F16 = 0, DT_BF16 = 1, DT_F32 = 2 };
+
+/* ------------------------------------------------------------------------ */
+/* storage formats                                                          */
+/* ------------------------------------------------------------------------ */
+static float u32_as_float(uint32_t u)
+{
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+static uint32_t float_as_u32(float f)
+{
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    return u;
+}
+
+static float bf16_to_float(uint16_t h) { return u32_as_float((uint32_t)h << 16); }
+
+static uint16_t float_to_bf16(float f)
+{
+    uint32_t u = float_as_u32(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u); /* quiet NaN */
+    u += 0x7fffu + ((u >> 16) & 1u);                                             /* nearest even */
+    return (uint16_t)(u >> 16);
+}
+
+static float f16_to_float(uint16_t h)
+{
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    const uint32_t exp = (h >> 10) & 0x1fu;
+    const uint32_t man = h & 0x3ffu;
+    if (exp == 0x1fu) return u32_as_float(sign | 0x7f800000u | (man << 13));
+    if (exp == 0) {
+        /* zero or subnormal: man * 2^-24, exact in fp32 */
+        const float v = (float)man * 5.9604644775390625e-08f;
+        return sign ? -v : v;
+    }
+    return u32_as_float(sign | ((exp + 112u) << 23) | (man << 13));
+}
+
+static uint16_t float_to_f16(float f)
+{
+    const uint32_t u = float_as_u32(f);
+    const uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+    const uint32_t a = u & 0x7fffffffu;
+    if (a > 0x7f800000u) return (uint16_t)(sign | 0x7e00u);  /* NaN */
+    if (a >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u); /* >= 65520 rounds to inf */
+    if (a < 0x33000001u) return sign;                        /* <= 2^-25 rounds to zero */
+    const int e = (int)(a >> 23) - 127;
+    uint32_t man = (a & 0x7fffffu) | 0x800000u; /* 24-bit significand */
+    int shift;                                  /* bits dropped from the significand */
+    uint32_t base;
+    if (e < -14) {
+        shift = 13 + (-14 - e); /* subnormal result */
+        base = 0;
+    } else {
+        shift = 13;
+        base = (uint32_t)(e + 15) << 10;
+        man &= 0x7fffffu;
+    }
+    const uint32_t kept = man >> shift;
+    const uint32_t rest = man & ((1u << shift) - 1u);
+    const uint32_t half = 1u << (shift - 1);
+    uint32_t r = base + kept; /* a carry out of the mantissa bumps the exponent, as it should */
+    if (rest > half || (rest == half && (kept & 1u))) r += 1;
+    return (uint16_t)(sign | r);
+}
+
+static float load_elem(const void* p, int64_t i, int dt)
+{
+    if (dt == DT_BF16) return bf16_to_float(((const uint16_t*)p)[i]);
+    if (dt == DT_F16) return f16_to_float(((const uint16_t*)p)[i]);
+    return ((const float*)p)[i];
+}
+static void store_elem(void* p, int64_t i, int dt, float v)
+{
+    if (dt == DT_BF16)
+        ((uint16_t*)p)[i] = float_to_bf16(v);
+    else if (dt == DT_F16)
+        ((uint16_t*)p)[i] = float_to_f16(v);
+    else
+        ((float*)p)[i] = v;
+}
+/* value of v after a round trip through storage type dt */
+static float round_to(float v, int dt)
+{
+    if (dt == DT_BF16) return bf16_to_float(float_to_bf16(v));
+    if (dt == DT_F16) return f16_to_float(float_to_f16(v));
+    return v;
+}
+
+/* exported for the conversion tests */
+uint16_t oracle_float_to_bf16(float f) { return float_to_bf16(f); }
+uint16_t oracle_float_to_f16(float f) { return float_to_f16(f); }
+float oracle_bf16_to_float(uint16_t h) { return bf16_to_float(h); }
+float oracle_f16_to_float(uint16_t h) { return f16_to_float(h); }
+
+static float pairwise_sum(const float* v, int64_t n)
+{
+    if (n <= 8) {
+        float s = 0.0f;
+        for (int64_t i = 0; i < n; ++i) s += v[i];
+        return s;
+    }
+    const int64_t h = n / 2;
+    return pairwise_sum(v, h) + pairwise_sum(v + h, n - h);
+}
+
+/* ------------------------------------------------------------------------ */
+/* softmax of one row of already scaled/filled logits z[0..n) (fp32)         */
+/* scaled_upper_triang_masked_softmax.h:206-233, scaled_masked_softmax.h:198-218 */
+/* ------------------------------------------------------------------------ */
+static void softmax_row(float* z, int64_t n)
+{
+    float m = z[0];
+    for (int64_t k = 1; k < n; ++k) m = (m > z[k]) ? m : z[k];
+    for (int64_t k = 0; k < n; ++k) z[k] = expf(z[k] - m);
+    const float sum = pairwise_sum(z, n);
+    for (int64_t k = 0; k < n; ++k) z[k] = z[k] / sum;
+}
+
+/*
+ * scaled_upper_triang_masked_softmax_warp_forward
+ * (scaled_upper_triang_masked_softmax.h:143-260): for row q of each [s,s]
+ * matrix, softmax over columns k <= q of x*scale, +0 for k > q.
+ * x, y: [batches, s, s].
+ */
+int oracle_causal_softmax_fwd(void* y, const void* x, float scale, int64_t batches, int64_t s, int dt)
+{
+    if (dt != DT_F16 && dt != DT_BF16) return -1;
+    float* z = (float*)malloc(sizeof(float) * (size_t)(s > 0 ? s : 1));
+    if (!z) return -2;
+    for (int64_t a = 0; a < batches; ++a)
+        for (int64_t q = 0; q < s; ++q) {
+            const int64_t base = (a * s + q) * s;
+            for (int64_t k = 0; k <= q; ++k) z[k] = load_elem(x, base + k, dt) * scale;
+            softmax_row(z, q + 1);
+            for (int64_t k = 0; k <= q; ++k) store_elem(y, base + k, dt, z[k]);
+            for (int64_t k = q + 1; k < s; ++k) store_elem(y, base + k, dt, 0.0f);
+        }
+    free(z);
+    return 0;
+}
+
+/*
+ * scaled_masked_softmax_warp_forward (scaled_masked_softmax.h:117-238):
+ * z = (mask == 1) ? -10000 : x*scale. x, y: [b, np, sq, sk];
+ * mask: [pad_batches, 1, sq, sk] bytes, pad_batches in {1, b} (:141-147).
+ */
+int oracle_masked_softmax_fwd(void* y, const void* x, const uint8_t* mask, float scale, int64_t b,
+                              int64_t np, int64_t sq, int64_t sk, int64_t pad_batches, int dt)
+{
+    if (dt != DT_F16 && dt != DT_BF16) return -1;
+    if (pad_batches != 1 && pad_batches != b) return -3;
+    float* z = (float*)malloc(sizeof(float) * (size_t)(sk > 0 ? sk : 1));
+    if (!z) return -2;
+    for (int64_t bi = 0; bi < b; ++bi)
+        for (int64_t h = 0; h < np; ++h)
+            for (int64_t q = 0; q < sq; ++q) {
+                const int64_t base = ((bi * np + h) * sq + q) * sk;
+                const uint8_t* mrow = mask + ((pad_batches == 1 ? 0 : bi) * sq + q) * sk;
+                for (int64_t k = 0; k < sk; ++k)
+                    z[k] = (mrow[k] != 1) ? load_elem(x, base + k, dt) * scale : -10000.0f;
+                softmax_row(z, sk);
+                for (int64_t k = 0; k < sk; ++k) store_elem(y, base + k, dt, z[k]);
+            }
+    free(z);
+    return 0;
+}
+
+/*
+ * scaled_upper_triang_masked_softmax_warp_backward (.h:262-361) when
+ * causal != 0, scaled_masked_softmax_warp_backward (scaled_masked_softmax.h:240-335)
+ * otherwise: g = dy*y on the unmasked columns (0 elsewhere),
+ * dx = scale * (g - y * sum(g)). rows x n elements; rows_per_matrix gives the
+ * causal row index q = row % rows_per_matrix. dx may alias dy.
+ */
+int oracle_softmax_bwd(void* dx, const void* dy, const void* y, float scale, int64_t rows, int64_t n,
+                       int64_t rows_per_matrix, int causal, int dt)
+{
+    if (dt != DT_F16 && dt != DT_BF16) return -1;
+    float* g = (float*)malloc(sizeof(float) * (size_t)(n > 0 ? n : 1));
+    float* p = (float*)malloc(sizeof(float) * (size_t)(n > 0 ? n : 1));
+    if (!g || !p) {
+        free(g);
+        free(p);
+        return -2;
+    }
+    for (int64_t r = 0; r < rows; ++r) {
+        const int64_t valid = causal ? (r % rows_per_matrix) + 1 : n;
+        const int64_t base = r * n;
+        for (int64_t k = 0; k < n; ++k) {
+            if (k < valid) {
+                p[k] = load_elem(y, base + k, dt);
+                g[k] = load_elem(dy, base + k, dt) * p[k];
+            } else {
+                p[k] = 0.0f;
+                g[k] = 0.0f;
+            }
+        }
+        const float sum = pairwise_sum(g, n);
+        for (int64_t k = 0; k < n; ++k) {
+            const float t = p[k] * sum;
+            const float d = g[k] - t;
+            store_elem(dx, base + k, dt, scale * d);
+        }
+    }
+    free(g);
+    free(p);
+    return 0;
+}
+
+/*
+ * get_batch_per_block (scaled_masked_softmax.h:338-352) for a machine whose
+ * warp is `warp` lanes wide (32 on NVIDIA, 64 on gfx9).
+ */
+int oracle_batch_per_block(int64_t key_seq_len, int warp)
+{
+    int64_t pow2 = 1;
+    while (pow2 < key_seq_len) pow2 *= 2;
+    const int64_t ws = pow2 < warp ? pow2 : warp;
+    const int64_t per_warp = pow2 <= 128 ? 2 : 1;
+    return (int)((128 / ws) * per_warp);
+}
+
+/* ------------------------------------------------------------------------ */
+/* rotary embedding                                                          */
+/* ------------------------------------------------------------------------ */
+
+/* a (*) b and a (+) b of the 16-bit scalar types: fp32 operation, then round
+ * (fused_rotary_positional_embedding.h:58,107,158,209 use scalar_t operators). */
+static float mul_t(float a, float b, int dt) { return round_to(a * b, dt); }
+static float add_t(float a, float b, int dt) { return round_to(a + b, dt); }
+
+/*
+ * Shared body of the four rotary kernels
+ * (fused_rotary_positional_embedding.h:27-74 fwd, :76-124 bwd, :126-174 cached
+ * fwd, :176-225 cached bwd).
+ *   cs_mode 0: cos/sin tables of dtype cs_dt, contiguous [s, d2]
+ *   cs_mode 1: freqs fp32 [s, d2] in `cos`; cosf/sinf evaluated here
+ * in/out: [s, b, h, d] with element strides is[4] / os[4].
+ */
+static int rope_any(void* out, const void* in, const void* cos, const void* sin, int64_t s, int64_t b,
+                    int64_t h, int64_t d, int64_t d2, const int64_t* is, const int64_t* os, int dt,
+                    int cs_dt, int cs_mode, int backward)
+{
+    if (dt != DT_F16 && dt != DT_BF16 && dt != DT_F32) return -1;
+    if (d2 > d) return -3;
+    const int64_t h2 = d2 / 2;
+    for (int64_t si = 0; si < s; ++si)
+        for (int64_t bi = 0; bi < b; ++bi)
+            for (int64_t hi = 0; hi < h; ++hi) {
+                const int64_t src = si * is[0] + bi * is[1] + hi * is[2];
+                const int64_t dst = si * os[0] + bi * os[1] + hi * os[2];
+                for (int64_t i = 0; i < d2; ++i) {
+                    const int first = (i + h2 < d2);
+                    const int64_t partner = first ? i + h2 : i + h2 - d2;
+                    /* the index whose sine is used: own index forward, partner's backward */
+                    const int64_t si_idx = backward ? partner : i;
+                    float c, sn;
+                    if (cs_mode == 0) {
+                        c = round_to(load_elem(cos, si * d2 + i, cs_dt), dt);
+                        sn = round_to(load_elem(sin, si * d2 + si_idx, cs_dt), dt);
+                    } else {
+                        c = round_to(cosf(((const float*)cos)[si * d2 + i]), dt);
+                        sn = round_to(sinf(((const float*)cos)[si * d2 + si_idx]), dt);
+                    }
+                    const float x = load_elem(in, src + i * is[3], dt);
+                    float r = load_elem(in, src + partner * is[3], dt);
+                    if (!backward) {
+                        if (first) r = -r; /* rotate_half: (-x2, x1) */
+                    } else {
+                        if (!first) sn = -sn;
+                    }
+                    const float v = add_t(mul_t(x, c, dt), mul_t(r, sn, dt), dt);
+                    store_elem(out, dst + i * os[3], dt, v);
+                }
+                for (int64_t i = d2; i < d; ++i)
+                    store_elem(out, dst + i * os[3], dt, load_elem(in, src + i * is[3], dt));
+            }
+    return 0;
+}
+
+int oracle_rope_cached(void* out, const void* in, const void* cos, const void* sin, int64_t s, int64_t b,
+                       int64_t h, int64_t d, int64_t d2, const int64_t* is, const int64_t* os, int dt,
+                       int cs_dt, int backward)
+{
+    if (cs_dt != DT_F32 && cs_dt != dt) return -1;
+    return rope_any(out, in, cos, sin, s, b, h, d, d2, is, os, dt, cs_dt, 0, backward);
+}
+
+int oracle_rope_freqs(void* out, const void* in, const float* freqs, int64_t s, int64_t b, int64_t h,
+                      int64_t d, int64_t d2, const int64_t* is, const int64_t* os, int dt, int backward)
+{
+    return rope_any(out, in, freqs, freqs, s, b, h, d, d2, is, os, dt, DT_F32, 1, backward);
+}

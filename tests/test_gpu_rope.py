@@ -1,0 +1,161 @@
+"""GPU parity of the rotary kernels, called through the C ABI, against the CPU
+oracle and against eager torch.
+
+Cached tables: bit-exact (the kernel performs the same three roundings as the
+scalar types of the reference). On-device cos/sin (freqs variant): the fp32
+sincos of the device and of the host libm may differ in the last place, which
+after rounding to the data dtype can move one table entry by one ulp, so the
+comparison allows 2 ulp measured at the magnitude of the larger of the two
+products (stated in assert_rope_freqs_close).
+"""
+import pytest
+import torch
+
+import oracle
+import util
+from oracle import fallback_semantics as fb
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def tables(d2, s, dtype, cs_fp32=False):
+    cos, sin, ang = fb.rotary_tables(d2, s, 10000, torch.float32 if cs_fp32 else dtype)
+    return cos.contiguous(), sin.contiguous(), ang.contiguous()
+
+
+# (s, b, h, d, d2)
+SHAPES = [
+    (16, 2, 4, 128, 128), (16, 2, 4, 128, 32), (9, 3, 5, 64, 64), (8, 2, 3, 96, 96), (8, 2, 3, 80, 48),
+    (5, 2, 33, 128, 64), (4, 1, 2, 256, 256), (7, 2, 2, 32, 16), (3, 2, 2, 24, 8), (6, 2, 3, 20, 10),
+    (4, 2, 2, 16, 6), (4, 2, 2, 15, 7), (64, 4, 16, 128, 32), (33, 5, 40, 128, 128),
+]
+DTYPES = [torch.bfloat16, torch.float16, torch.float32]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("cs_fp32", [False, True], ids=["cs_same", "cs_fp32"])
+def test_rope_cached_bit_exact(hotpath, shape, dtype, cs_fp32):
+    s, b, h, d, d2 = shape
+    say(f"rope cached {shape} {dtype} cs_fp32={cs_fp32}")
+    t = util.randn((s, b, h, d), dtype, seed=s + d)
+    cos, sin, _ = tables(d2, s, dtype, cs_fp32)
+    for backward in (False, True):
+        for transpose in (False, True):
+            want = oracle.rope_cached(t, cos, sin, backward=backward, transpose_output=transpose)
+            got = util.abi_rope_cached(hotpath, t.to(DEV), cos.to(DEV), sin.to(DEV), backward, transpose)
+            torch.cuda.synchronize()
+            assert got.stride() == want.stride()
+            assert torch.equal(util.raw_bits(got.cpu()), util.raw_bits(want)), (backward, transpose)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+def test_rope_strided_views_of_fused_qkv(hotpath, dtype):
+    """q, k as NeoX passes them: slices of a [sq, b, np, 3*hn] projection, and
+    the partial-rotary narrowing [..., :rot] on top (transformer.py:852-887)."""
+    s, b, h, hn = 32, 2, 8, 128
+    qkv = util.randn((s, b, h, 3 * hn), dtype, seed=1)
+    qkv_d = qkv.to(DEV)
+    for d2 in (128, 32):
+        cos, sin, _ = tables(d2, s, dtype)
+        for part in range(2):
+            view = qkv[..., part * hn : (part + 1) * hn]
+            view_d = qkv_d[..., part * hn : (part + 1) * hn]
+            for backward in (False, True):
+                # full head vector with in-kernel pass-through
+                want = oracle.rope_cached(view, cos, sin, backward=backward)
+                got = util.abi_rope_cached(hotpath, view_d, cos.to(DEV), sin.to(DEV), backward)
+                assert torch.equal(util.raw_bits(got.cpu()), util.raw_bits(want))
+                # narrowed view, d == d2
+                want = oracle.rope_cached(view[..., :d2], cos, sin, backward=backward)
+                got = util.abi_rope_cached(hotpath, view_d[..., :d2], cos.to(DEV), sin.to(DEV), backward)
+                assert torch.equal(util.raw_bits(got.cpu()), util.raw_bits(want))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32], ids=["bf16", "fp16", "fp32"])
+def test_rope_matches_eager_torch(hotpath, dtype):
+    """Forward equals apply_rotary_pos_emb_torch bit for bit; backward equals
+    autograd through the eager expression when that is evaluated with the same
+    roundings (the adjoint rotation)."""
+    s, b, h, d = 24, 2, 4, 128
+    for d2 in (128, 32):
+        t = util.randn((s, b, h, d), dtype, seed=d2)
+        cos, sin, _ = tables(d2, s, dtype)
+        want = fb.eager_rotary_partial(t, cos, sin)
+        got = util.abi_rope_cached(hotpath, t.to(DEV), cos.to(DEV), sin.to(DEV)).cpu()
+        assert torch.equal(util.raw_bits(got), util.raw_bits(want))
+        # backward: rotation by the negative angle = forward with sin -> -sin
+        g = util.randn((s, b, h, d), dtype, seed=d2 + 1)
+        want_b = fb.eager_rotary_partial(g, cos, -sin)
+        got_b = util.abi_rope_cached(hotpath, g.to(DEV), cos.to(DEV), sin.to(DEV), backward=True).cpu()
+        assert torch.equal(util.raw_bits(got_b), util.raw_bits(want_b))
+
+
+def assert_rope_freqs_close(got, want, t, max_ulp=2):
+    """|got - want| <= max_ulp * ulp(storage dtype at max(|t|) magnitude of the
+    head vector's rotary pair), or 2 representable values apart."""
+    got, want = got.cpu(), want.cpu()
+    near = util.ulp_distance(got, want) <= max_ulp
+    scale_ref = t.cpu().float().abs().amax(dim=-1, keepdim=True).expand_as(got.float())
+    bound = max_ulp * util.ulp_size(scale_ref.to(got.dtype))
+    ok = near | ((got.float() - want.float()).abs() <= bound)
+    assert ok.all(), f"{int((~ok).sum())} elements out of tolerance"
+    return float((~near).float().mean())
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("shape", SHAPES[:8] + SHAPES[-2:], ids=lambda s: "x".join(map(str, s)))
+def test_rope_freqs_vs_oracle(hotpath, shape, dtype):
+    s, b, h, d, d2 = shape
+    say(f"rope freqs {shape} {dtype}")
+    t = util.randn((s, b, h, d), dtype, seed=s + d + 1)
+    _, _, ang = tables(d2, s, dtype)
+    # include large angles (positions in the thousands) to exercise range reduction
+    ang = (ang + 4000.0 * ang[1:2]).contiguous() if s > 1 else ang
+    for backward in (False, True):
+        want = oracle.rope_freqs(t, ang, backward=backward)
+        got = util.abi_rope_freqs(hotpath, t.to(DEV), ang.to(DEV), backward)
+        torch.cuda.synchronize()
+        assert_rope_freqs_close(got, want, t)
+        # pass-through features are copies
+        if d > d2:
+            assert torch.equal(util.raw_bits(got.cpu()[..., d2:]), util.raw_bits(t[..., d2:]))
+
+
+def test_rope_full_size_properties(hotpath):
+    """q, k [4096, 4, 32, 128] bf16 (rotary_pct 1.0 and 0.25) and the
+    Llama-2-7B shape [8192, 2, 32, 128]: bit-exact against eager torch on the
+    GPU (same roundings), position 0 is the identity, tail features are copies,
+    and backward(forward(x)) returns x up to the six roundings involved."""
+    for (s, b, h, d), pcts in (((4096, 4, 32, 128), (1.0, 0.25)), ((8192, 2, 32, 128), (1.0,))):
+        for pct in pcts:
+            d2 = int(d * pct)
+            say(f"rope full size s={s} b={b} h={h} d={d} d2={d2}")
+            g = torch.Generator(device=DEV).manual_seed(s + d2)
+            q = torch.randn((s, b, h, d), generator=g, device=DEV).to(torch.bfloat16)
+            cos, sin, _ = tables(d2, s, torch.bfloat16)
+            cos, sin = cos.to(DEV), sin.to(DEV)
+            y = util.abi_rope_cached(hotpath, q, cos, sin)
+            want = fb.eager_rotary_partial(q, cos, sin)
+            assert torch.equal(y.view(torch.int16), want.view(torch.int16))
+            assert torch.equal(y[0].view(torch.int16), q[0].view(torch.int16))
+            if d2 < d:
+                assert torch.equal(y[..., d2:].contiguous().view(torch.int16), q[..., d2:].contiguous().view(torch.int16))
+            back = util.abi_rope_cached(hotpath, y, cos, sin, backward=True)
+            err = (back.float() - q.float()).abs().max().item()
+            assert err < 0.1, err
+            # adjointness <rope(x), g> == <x, rope_bwd(g)> up to bf16 rounding
+            gy = torch.randn((s, b, h, d), generator=g, device=DEV).to(torch.bfloat16)
+            gx = util.abi_rope_cached(hotpath, gy, cos, sin, backward=True)
+            lhs = (y.double() * gy.double()).sum().item()
+            rhs = (q.double() * gx.double()).sum().item()
+            # each of the ~N products carries a relative rounding error of about 2^-8 with random
+            # sign, so the two sums differ by a few times 2^-8 * sqrt(sum of squared terms);
+            # a wrong sign or index in backward would move rhs by about sqrt(N) instead
+            noise = 2.0**-8 * (y.double() * gy.double()).pow(2).sum().item() ** 0.5
+            assert abs(lhs - rhs) <= 8 * noise, (lhs, rhs, noise)
