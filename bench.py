@@ -1,0 +1,317 @@
+#!/usr/bin/env python3
+"""Throughput of the fused softmax + rotary hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+A step is one pass of the hot path over one batch of synthetic input, through
+the drop-in extension modules (which call libneox_hotpath.so):
+
+  pythia-1.4b (default; the configuration the headline metric is quoted on)
+      rotary fwd on q and k  [s=2048, b=8, h=16, d=128] bf16, rotary_pct 0.25
+      causal softmax fwd     [b*h=128, 2048, 2048] bf16, scale 1/sqrt(128)
+      causal softmax bwd     same shape, in place on the upstream gradient
+      rotary bwd on dq, dk
+  masked-c3      padding-masked softmax fwd+bwd [16,32,1024,2048] fp16
+  rope-c4        rotary fwd+bwd on q,k [4096,4,32,128] bf16, rotary_pct 1.0 and 0.25
+  llama2-7b-c5   rotary on q,k [8192,2,32,128] + causal softmax fwd+bwd [64,8192,8192] bf16
+
+`value` is algorithmic bytes per step / wall time per step (inputs resident in
+HBM, K steps bracketed by device synchronisation). Algorithmic bytes: softmax
+forward reads the lower triangle and writes the dense result; backward reads
+two triangles and writes dense; rotary reads and writes every element once plus
+the cos/sin tables. `roofline` is the same ratio for the dominant kernel alone,
+timed with events on the launch stream. `cpu_baseline` times the reference's
+torch fallback (oracle/fallback_semantics.py) on this machine's host cores on a
+bounded sample of the default workload.
+
+One GPU only: there is no multi-GPU mode, `--gpus N` with N > 1 exits.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "gpt-neo-x_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+METRIC = "achieved HBM GB/s (% of MI355X peak), causal softmax+rotary fwd/bwd, 1.4B shape"
+HBM_PEAK_GBS = 8000.0
+
+# HBM bytes per launch of the dominant kernel of the default workload measured
+# with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), see profiles/; None until measured.
+MEASURED_TRAFFIC_BYTES = {"pythia-1.4b": None}
+
+
+def tri(n):
+    return n * (n + 1) // 2
+
+
+def causal_bytes(a, s, e=2):
+    fwd = a * tri(s) * e + a * s * s * e
+    bwd = 2 * a * tri(s) * e + a * s * s * e
+    return fwd, bwd
+
+
+def rope_bytes(s, b, h, d, d2, e=2, e_cs=2):
+    return 2 * s * b * h * d * e + 2 * s * d2 * e_cs
+
+
+class Timer:
+    """Accumulates event-timed durations of one named kernel on the current stream."""
+
+    def __init__(self, torch):
+        self.torch = torch
+        self.pairs = {}
+
+    def run(self, name, fn):
+        a = self.torch.cuda.Event(enable_timing=True)
+        b = self.torch.cuda.Event(enable_timing=True)
+        a.record()
+        out = fn()
+        b.record()
+        self.pairs.setdefault(name, []).append((a, b))
+        return out
+
+    def averages_ms(self):
+        return {k: sum(a.elapsed_time(b) for a, b in v) / len(v) for k, v in self.pairs.items()}
+
+    def reset(self):
+        self.pairs = {}
+
+
+def make_workload(name, torch, dev):
+    import fused_rotary_positional_embedding as rope_ext
+    import scaled_masked_softmax_cuda as masked_ext
+    import scaled_upper_triang_masked_softmax_cuda as causal_ext
+    from megatron.model.positional_embeddings import RotaryEmbedding
+
+    gen = torch.Generator(device=dev)
+
+    def randn(shape, seed, dtype, std=1.0):
+        gen.manual_seed(seed)
+        return (torch.randn(shape, generator=gen, device=dev) * std).to(dtype)
+
+    def rope_setup(s, b, h, d, d2, seed):
+        q = randn((s, b, h, d), seed, torch.bfloat16)
+        k = randn((s, b, h, d), seed + 1, torch.bfloat16)
+        dq = randn((s, b, h, d), seed + 2, torch.bfloat16)
+        dk = randn((s, b, h, d), seed + 3, torch.bfloat16)
+        cos, sin = RotaryEmbedding(d2, s, base=10000, precision=torch.bfloat16)(q, seq_len=s)
+        return q, k, dq, dk, cos.contiguous(), sin.contiguous()
+
+    if name in ("pythia-1.4b", "llama2-7b-c5"):
+        if name == "pythia-1.4b":
+            s, b, h, d, d2 = 2048, 8, 16, 128, 32
+        else:
+            s, b, h, d, d2 = 8192, 2, 32, 128, 128
+        a = b * h
+        scale = 1.0 / math.sqrt(d)
+        q, k, dq, dk, cos, sin = rope_setup(s, b, h, d, d2, 10)
+        x = randn((a, s, s), 0, torch.bfloat16, 2.0)
+        dy = randn((a, s, s), 1, torch.bfloat16)
+        fwd_b, bwd_b = causal_bytes(a, s)
+        rb = rope_bytes(s, b, h, d, d2)
+        kernel_bytes = {"rope_fwd": 2 * rb, "causal_softmax_fwd": fwd_b, "causal_softmax_bwd": bwd_b,
+                        "rope_bwd": 2 * rb}
+        dense = {"causal_softmax_fwd": 2 * a * s * s * 2, "causal_softmax_bwd": 3 * a * s * s * 2}
+
+        def step(t):
+            def rope_f():
+                rope_ext.forward_cached(q, cos, sin, False)
+                rope_ext.forward_cached(k, cos, sin, False)
+
+            def rope_b():
+                rope_ext.backward_cached(dq, cos, sin, False)
+                rope_ext.backward_cached(dk, cos, sin, False)
+
+            t.run("rope_fwd", rope_f)
+            y = t.run("causal_softmax_fwd", lambda: causal_ext.forward(x, scale))
+            # in place on dy, as the reference does; its values shrink from step
+            # to step, which does not change the work done
+            t.run("causal_softmax_bwd", lambda: causal_ext.backward(dy, y, scale))
+            t.run("rope_bwd", rope_b)
+
+        cfg = {"workload": name, "scores": [a, s, s], "qk": [s, b, h, d], "rotary_dim": d2,
+               "scale": "1/sqrt(%d)" % d, "bytes_convention": "causal-min (reads of the lower triangle, dense writes)"}
+        return step, kernel_bytes, dense, "causal_softmax_bwd", "bf16", cfg
+
+    if name == "masked-c3":
+        b, np_, sq, sk = 16, 32, 1024, 2048
+        scale = 1.0 / math.sqrt(128)
+        x = randn((b, np_, sq, sk), 0, torch.float16, 3.0)
+        gen.manual_seed(5)
+        hit = torch.rand(x.shape, generator=gen, device=dev) < 0.01
+        sign = torch.where(torch.rand(x.shape, generator=gen, device=dev) < 0.5, -60.0, 60.0).half()
+        x = torch.where(hit, sign, x)
+        del hit, sign
+        g = torch.Generator().manual_seed(0)
+        valid = torch.randint(512, sk + 1, (b,), generator=g)
+        kk = torch.arange(sk)
+        mask = (kk[None, :] >= valid[:, None])[:, None, None, :].expand(b, 1, sq, sk).contiguous()
+        mask[7] = True
+        mask = mask.to(dev)
+        dy = randn(x.shape, 1, torch.float16)
+        n = x.numel()
+        kernel_bytes = {"masked_softmax_fwd": 2 * n * 2 + mask.numel(), "masked_softmax_bwd": 3 * n * 2}
+
+        def step(t):
+            y = t.run("masked_softmax_fwd", lambda: masked_ext.forward(x, mask, scale))
+            t.run("masked_softmax_bwd", lambda: masked_ext.backward(dy, y, scale))
+
+        cfg = {"workload": name, "scores": [b, np_, sq, sk], "mask": [b, 1, sq, sk],
+               "bytes_convention": "dense (2x tensor forward + mask once, 3x tensor backward)"}
+        return step, kernel_bytes, {}, "masked_softmax_bwd", "f16", cfg
+
+    if name == "rope-c4":
+        s, b, h, d = 4096, 4, 32, 128
+        sets = []
+        for i, d2 in enumerate((128, 32, 128, 32)):  # rotate through distinct buffers: 128 MiB tensors fit the 256 MB cache
+            sets.append((d2,) + rope_setup(s, b, h, d, d2, 20 + 10 * i))
+        kernel_bytes = {"rope_fwd_d2_128": 2 * rope_bytes(s, b, h, d, 128), "rope_bwd_d2_128": 2 * rope_bytes(s, b, h, d, 128),
+                        "rope_fwd_d2_32": 2 * rope_bytes(s, b, h, d, 32), "rope_bwd_d2_32": 2 * rope_bytes(s, b, h, d, 32)}
+        state = {"i": 0}
+
+        def step(t):
+            for _ in range(2):
+                d2, q, k, dq, dk, cos, sin = sets[state["i"] % len(sets)]
+                state["i"] += 1
+
+                def f():
+                    rope_ext.forward_cached(q, cos, sin, False)
+                    rope_ext.forward_cached(k, cos, sin, False)
+
+                def bw():
+                    rope_ext.backward_cached(dq, cos, sin, False)
+                    rope_ext.backward_cached(dk, cos, sin, False)
+
+                t.run(f"rope_fwd_d2_{d2}", f)
+                t.run(f"rope_bwd_d2_{d2}", bw)
+
+        cfg = {"workload": name, "qk": [s, b, h, d], "rotary_dims": [128, 32]}
+        return step, kernel_bytes, {}, "rope_fwd_d2_128", "bf16", cfg
+
+    raise SystemExit(f"unknown workload {name}")
+
+
+def cpu_baseline(torch):
+    """The reference's torch fallback on the host cores, on 1/8 of the default
+    workload (one batch entry: scores [1,16,2048,2048], q/k [2048,1,16,128])."""
+    from oracle import fallback_semantics as fb
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    s, h, d, d2 = 2048, 16, 128, 32
+    scale = 1.0 / math.sqrt(d)
+    g = torch.Generator().manual_seed(0)
+    x = (torch.randn((1, h, s, s), generator=g) * 2).bfloat16()
+    dy = torch.randn((1, h, s, s), generator=g).bfloat16()
+    q = torch.randn((s, 1, h, d), generator=g).bfloat16()
+    k = torch.randn((s, 1, h, d), generator=g).bfloat16()
+    dq = torch.randn((s, 1, h, d), generator=g).bfloat16()
+    cos, sin, _ = fb.rotary_tables(d2, s, 10000, torch.bfloat16)
+    mask = fb.causal_mask(s)
+
+    def one():
+        qq = q.clone().requires_grad_(True)
+        kk = k.clone().requires_grad_(True)
+        oq = fb.eager_rotary_partial(qq, cos, sin)
+        ok = fb.eager_rotary_partial(kk, cos, sin)
+        xx = x.clone().requires_grad_(True)
+        y = fb.torch_softmax_fallback(xx, mask, scale)
+        y.backward(dy)
+        torch.autograd.backward([oq, ok], [dq, dq])
+
+    one()  # warm-up
+    times = []
+    t_end = time.perf_counter() + 12.0  # about 12 s of CPU work
+    while len(times) < 3 or time.perf_counter() < t_end:
+        t0 = time.perf_counter()
+        one()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    fwd_b, bwd_b = causal_bytes(h, s)
+    nbytes = fwd_b + bwd_b + 4 * rope_bytes(s, 1, h, d, d2)
+    return {"value": round(nbytes / med / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": "reference torch fallback (fp32 softmax via autograd, eager rotary) on 1/8 of the default "
+                      f"workload: scores [1,16,2048,2048], q,k [2048,1,16,128] bf16; median of {len(times)} runs, "
+                      f"{med * 1e3:.1f} ms each, same algorithmic-byte convention"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="pythia-1.4b")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        raise SystemExit("bench.py measures one GPU; this hot path has no multi-GPU mode (run with --gpus 1)")
+
+    import torch
+
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU")
+    from megatron.fused_kernels import load
+
+    load()  # raises if libneox_hotpath.so cannot be loaded; there is no fallback
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    step, kernel_bytes, dense_bytes, dominant, dtype, cfg = make_workload(args.workload, torch, dev)
+    timer = Timer(torch)
+    for _ in range(args.warmup):
+        step(timer)
+    torch.cuda.synchronize()
+    timer.reset()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(timer)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+
+    ms_per_step = elapsed * 1e3 / args.steps
+    step_bytes = sum(kernel_bytes.values())
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+    avg = timer.averages_ms()
+    kernels = {}
+    for name, nbytes in kernel_bytes.items():
+        gbs = nbytes / (avg[name] * 1e-3) / 1e9
+        kernels[name] = {"ms": round(avg[name], 4), "bytes": nbytes, "GB/s": round(gbs, 1),
+                         "frac_of_peak": round(gbs / HBM_PEAK_GBS, 4)}
+        if name in dense_bytes:
+            kernels[name]["GB/s_dense_convention"] = round(dense_bytes[name] / (avg[name] * 1e-3) / 1e9, 1)
+    dom = kernels[dominant]
+    out = {
+        "metric": METRIC,
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": dtype,
+        "data": "synthetic",
+        "config": cfg,
+        "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+        "bytes_per_step": step_bytes,
+        "kernels": kernels,
+        "roofline": {"bound": "hbm", "kernel": dominant, "achieved": dom["GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": dom["frac_of_peak"], "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "algorithmic_bytes": kernel_bytes[dominant], "avg_launch_ms": dom["ms"]},
+    }
+    if args.workload == "pythia-1.4b" and not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(torch)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

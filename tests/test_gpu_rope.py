@@ -24,8 +24,18 @@ def say(*a):
 
 
 def tables(d2, s, dtype, cs_fp32=False):
+    """Tables of the RotaryEmbedding recipe (the two halves of the feature axis share angles)."""
     cos, sin, ang = fb.rotary_tables(d2, s, 10000, torch.float32 if cs_fp32 else dtype)
     return cos.contiguous(), sin.contiguous(), ang.contiguous()
+
+
+def generic_tables(d2, s, dtype, cs_fp32=False, seed=0):
+    """Independent angle for every (position, feature): unlike the recipe above this tells
+    sin[i] from sin[i + d2/2], and it exists for odd d2."""
+    g = torch.Generator().manual_seed(seed)
+    ang = (torch.rand((s, 1, 1, d2), generator=g) * 20.0 - 10.0).contiguous()
+    cs = torch.float32 if cs_fp32 else dtype
+    return ang.cos().to(cs).contiguous(), ang.sin().to(cs).contiguous(), ang
 
 
 # (s, b, h, d, d2)
@@ -44,7 +54,7 @@ def test_rope_cached_bit_exact(hotpath, shape, dtype, cs_fp32):
     s, b, h, d, d2 = shape
     say(f"rope cached {shape} {dtype} cs_fp32={cs_fp32}")
     t = util.randn((s, b, h, d), dtype, seed=s + d)
-    cos, sin, _ = tables(d2, s, dtype, cs_fp32)
+    cos, sin, _ = generic_tables(d2, s, dtype, cs_fp32, seed=d2)
     for backward in (False, True):
         for transpose in (False, True):
             want = oracle.rope_cached(t, cos, sin, backward=backward, transpose_output=transpose)
@@ -114,9 +124,9 @@ def test_rope_freqs_vs_oracle(hotpath, shape, dtype):
     s, b, h, d, d2 = shape
     say(f"rope freqs {shape} {dtype}")
     t = util.randn((s, b, h, d), dtype, seed=s + d + 1)
-    _, _, ang = tables(d2, s, dtype)
+    _, _, ang = generic_tables(d2, s, dtype, seed=d)
     # include large angles (positions in the thousands) to exercise range reduction
-    ang = (ang + 4000.0 * ang[1:2]).contiguous() if s > 1 else ang
+    ang = (ang * torch.where(torch.arange(s) % 2 == 0, 1.0, 700.0).view(s, 1, 1, 1)).contiguous()
     for backward in (False, True):
         want = oracle.rope_freqs(t, ang, backward=backward)
         got = util.abi_rope_freqs(hotpath, t.to(DEV), ang.to(DEV), backward)
