@@ -183,17 +183,6 @@ __device__ __forceinline__ float block_combine(float v, float* slots, int wave, 
     }
 }
 
-// The hardware schedules consecutive workgroup ids round-robin over the 8
-// XCDs, each of which has a private L2. This maps the hardware id to a logical
-// id such that consecutive logical ids share an XCD (and so its L2).
-__device__ __forceinline__ uint32_t xcd_swizzle(uint32_t hw_id, uint32_t total)
-{
-    constexpr uint32_t kXcd = 8;
-    const uint32_t full = total - total % kXcd;
-    if (hw_id >= full) return hw_id;
-    return (hw_id % kXcd) * (full / kXcd) + hw_id / kXcd;
-}
-
 // 2^(x) with the raw v_exp_f32 instruction (about 1 ulp, no denormal results).
 __device__ __forceinline__ float exp2_raw(float x) { return __builtin_amdgcn_exp2f(x); }
 

@@ -6,19 +6,21 @@
 // the remaining d - d2 are copied.
 //
 // Vector kernel. A head vector is cut into 16-byte chunks (V = 8 elements for
-// 16-bit data, 4 for fp32). The rotation pairs element i with i + d2/2, so a
-// lane takes the two chunks [i, i+V) and [i+d2/2, i+d2/2+V) together: every
-// element is loaded once and no data crosses lanes. The pass-through tail is
-// cut into units of two chunks as well. A head vector is thus U units wide and
-// a workgroup is laid out as [heads][U] for one sequence position; it walks
-// over a slice of the batch dimension re-using the cos/sin values it loaded
-// (or computed) once.
+// 16-bit data, 4 for fp32) and every lane owns one chunk, so a wave-wide load
+// or store moves up to 1 KiB of consecutive head vectors. The rotation pairs
+// element i with i + d2/2, i.e. a chunk with the chunk d2/(2V) lanes away in
+// the same wave; the partner's data is fetched with ds_bpermute (no memory
+// traffic). Chunks of the pass-through tail are copied by their lanes. A
+// workgroup stays on one sequence position and walks over the (batch, head)
+// rows, re-using the cos/sin values it loaded (or computed) once.
 //
 // Arithmetic: out = (x (*) c) (+) (r (*) s) where every product and the sum
 // are rounded to the data dtype, which is what the scalar types of the
 // reference kernels and eager torch do.
 
 #include "common.hpp"
+
+#include <cstdlib>
 
 namespace nhp {
 
@@ -165,73 +167,100 @@ struct FreqTable {
 
 // ---------------------------------------------------------------------------
 // Vector kernel
-//   grid  = (s, ceil(b / b_per_block)), block = heads_per_block * U threads (<= 256)
-//   unit u < np : rotary pair of chunks  i = u*V  and  i + h2
-//   unit u >= np: tail chunks 2*(u-np) and 2*(u-np)+1 (the second may not exist)
-// Requires: stride_d == 1 on both sides, d2 % (2V) == 0, (d-d2) % V == 0,
-// every other stride a multiple of V, 16-byte aligned base pointers.
+//   grid  = (s, row_splits), block = 256 threads = 4 waves
+//   lane  = (row within wave) * cpr + chunk,  cpr = d / V chunks per head vector
+//   a wave covers rpw = 64 / cpr rows per step, the workgroup 4 * rpw, and the
+//   workgroups of one position interleave over the b*h rows.
+// Requires: stride_d == 1 on both sides, d % V == 0, d2 % (2V) == 0, d <= 64 V,
+// every other stride a multiple of V, 16-byte aligned base pointers and tables.
 // ---------------------------------------------------------------------------
-template <int DT, bool BWD, typename Tables>
+constexpr int kRopeUnroll = 2;
+
+// FLAT: the batch and head dimensions collapse into one row dimension on both
+// sides (stride_b == h * stride_h), which saves the division by h per row.
+template <int DT, bool BWD, bool FLAT, typename Tables>
 __global__ void __launch_bounds__(256)
-rope_vec_kernel(void* out, const void* in, Tables tab, int b, int h, int d, int d2, int units,
-                int heads_per_block, int b_per_block, int64_t is_s, int64_t is_b, int64_t is_h,
-                int64_t os_s, int64_t os_b, int64_t os_h)
+rope_vec_kernel(void* out, const void* in, Tables tab, int rows, int h, int cpr, int rot_chunks, int rpw,
+                int64_t is_s, int64_t is_b, int64_t is_h, int64_t os_s, int64_t os_b, int64_t os_h)
 {
     constexpr int V = Elt<DT>::kVec;
     using S = typename Elt<DT>::storage;
-    const int u = threadIdx.x % units;
-    const int hl = threadIdx.x / units;
-    if (hl >= heads_per_block) return;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int rl = lane / cpr;        // row within the wave's group
+    const int c = lane - rl * cpr;    // chunk within the head vector
+    const bool lane_on = rl < rpw;
     const int64_t pos = blockIdx.x;
-    const int h2 = d2 / 2;
-    const int np = h2 / V;  // rotary units per head vector
-    const int b0 = blockIdx.y * b_per_block;
-    const int b1 = (b0 + b_per_block < b) ? b0 + b_per_block : b;
 
-    const S* ip = static_cast<const S*>(in) + pos * is_s;
-    S* op = static_cast<S*>(out) + pos * os_s;
+    const int half = rot_chunks / 2;
+    const bool is_rot = c < rot_chunks;
+    const bool first = c < half;
+    const int partner_lane = is_rot ? (first ? lane + half : lane - half) : lane;
 
-    if (u < np) {
-        const int i = u * V;
-        float ca[V], sa[V], cb[V], sb[V];
-        tab.get_vec(pos, i, ca, sa);
-        tab.get_vec(pos, i + h2, cb, sb);
-        for (int hh = hl; hh < h; hh += heads_per_block) {
-            for (int bb = b0; bb < b1; ++bb) {
-                const S* src = ip + bb * is_b + hh * is_h;
-                S* dst = op + bb * os_b + hh * os_h;
-                float xa[V], xb[V], ya[V], yb[V];
-                chunk_to_float<DT>(load16_stream(src + i), xa);
-                chunk_to_float<DT>(load16_stream(src + i + h2), xb);
+    // cos of the own chunk; sin of the own chunk (forward) or of the partner's (backward)
+    float cv[V], sv[V];
 #pragma unroll
-                for (int v = 0; v < V; ++v) {
-                    if (!BWD) {
-                        // y_a = x_a*c_a + (-x_b)*s_a ; y_b = x_b*c_b + x_a*s_b
-                        ya[v] = rot<DT, true>(xa[v], ca[v], xb[v], sa[v]);
-                        yb[v] = rot<DT>(xb[v], cb[v], xa[v], sb[v]);
-                    } else {
-                        // dx_a = g_a*c_a + g_b*s_b ; dx_b = g_b*c_b + g_a*(-s_a)
-                        ya[v] = rot<DT>(xa[v], ca[v], xb[v], sb[v]);
-                        yb[v] = rot<DT, true>(xb[v], cb[v], xa[v], sa[v]);
-                    }
+    for (int v = 0; v < V; ++v) {
+        cv[v] = 0.0f;
+        sv[v] = 0.0f;
+    }
+    if (lane_on && is_rot) {
+        float unused[V];
+        if (!BWD) {
+            tab.get_vec(pos, (int64_t)c * V, cv, sv);
+        } else {
+            tab.get_vec(pos, (int64_t)c * V, cv, unused);
+            tab.get_vec(pos, (int64_t)(first ? c + half : c - half) * V, unused, sv);
+        }
+    }
+    // forward: first half subtracts, backward: second half subtracts
+    const bool negate = BWD ? !first : first;
+
+    const S* ip = static_cast<const S*>(in) + pos * is_s + (int64_t)c * V;
+    S* op = static_cast<S*>(out) + pos * os_s + (int64_t)c * V;
+
+    const int rows_per_step = 4 * rpw;
+    const int stride = rows_per_step * (int)gridDim.y;
+    // All lanes of a row (a lane and its partner included) share r0 and leave the loop together.
+    for (int r0 = (int)blockIdx.y * rows_per_step + wave * rpw + rl; r0 < rows; r0 += stride * kRopeUnroll) {
+        u32x4 raw[kRopeUnroll];
+        int64_t dst_off[kRopeUnroll];
+        bool on[kRopeUnroll];
+#pragma unroll
+        for (int u = 0; u < kRopeUnroll; ++u) {
+            const int r = r0 + u * stride;
+            on[u] = lane_on && r < rows;
+            raw[u] = u32x4{0, 0, 0, 0};
+            dst_off[u] = 0;
+            if (on[u]) {
+                if (FLAT) {
+                    raw[u] = load16_stream(ip + r * is_h);
+                    dst_off[u] = r * os_h;
+                } else {
+                    const int bi = r / h;
+                    const int hi = r - bi * h;
+                    raw[u] = load16_stream(ip + bi * is_b + hi * is_h);
+                    dst_off[u] = bi * os_b + hi * os_h;
                 }
-                store16_stream(dst + i, float_to_chunk<DT>(ya));
-                store16_stream(dst + i + h2, float_to_chunk<DT>(yb));
             }
         }
-    } else {
-        const int c0 = d2 + 2 * (u - np) * V;
-        const bool second = c0 + V < d;
-        for (int hh = hl; hh < h; hh += heads_per_block) {
-            for (int bb = b0; bb < b1; ++bb) {
-                const S* src = ip + bb * is_b + hh * is_h;
-                S* dst = op + bb * os_b + hh * os_h;
-                const u32x4 a = load16_stream(src + c0);
-                u32x4 c = u32x4{0, 0, 0, 0};
-                if (second) c = load16_stream(src + c0 + V);
-                store16_stream(dst + c0, a);
-                if (second) store16_stream(dst + c0 + V, c);
+#pragma unroll
+        for (int u = 0; u < kRopeUnroll; ++u) {
+            u32x4 praw;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                praw[i] = (uint32_t)__builtin_amdgcn_ds_bpermute(partner_lane << 2, (int)raw[u][i]);
+            u32x4 res = raw[u];
+            if (is_rot) {
+                float x[V], pr[V], y[V];
+                chunk_to_float<DT>(raw[u], x);
+                chunk_to_float<DT>(praw, pr);
+#pragma unroll
+                for (int v = 0; v < V; ++v)
+                    y[v] = negate ? rot<DT, true>(x[v], cv[v], pr[v], sv[v]) : rot<DT>(x[v], cv[v], pr[v], sv[v]);
+                res = float_to_chunk<DT>(y);
             }
+            if (on[u]) store16_stream(op + dst_off[u], res);
         }
     }
 }
@@ -300,37 +329,51 @@ static bool vector_ok(const RopeArgs& a, bool tables_ok)
     constexpr int V = Elt<DT>::kVec;
     if (!tables_ok) return false;
     if (a.is[3] != 1 || a.os[3] != 1) return false;
-    if (a.d2 % (2 * V) != 0 || (a.d - a.d2) % V != 0) return false;
+    if (a.d % V != 0 || a.d2 % (2 * V) != 0 || a.d > 64 * V) return false;
     for (int i = 0; i < 3; ++i)
         if (a.is[i] % V != 0 || a.os[i] % V != 0) return false;
     if (!is_aligned16(a.in) || !is_aligned16(a.out)) return false;
-    const int64_t units = a.d2 / (2 * V) + ((a.d - a.d2) / V + 1) / 2;
-    if (units > 256) return false;
-    if (a.s >= ((int64_t)1 << 31) || a.b > 65535 * (int64_t)64 || a.h >= ((int64_t)1 << 30)) return false;
+    if (a.s >= ((int64_t)1 << 31) || a.b * a.h >= ((int64_t)1 << 30)) return false;
     return true;
 }
+
+#ifdef NHP_TUNING
+static int rope_tune(const char* name, int def)
+{
+    const char* v = getenv(name);
+    return v ? atoi(v) : def;
+}
+#else
+static inline int rope_tune(const char*, int def) { return def; }
+#endif
 
 template <int DT, bool BWD, typename Tables>
 static int rope_launch(const RopeArgs& a, const Tables& tab, bool tables_ok)
 {
     constexpr int V = Elt<DT>::kVec;
     if (vector_ok<DT>(a, tables_ok)) {
-        const int units = (int)(a.d2 / (2 * V) + ((a.d - a.d2) / V + 1) / 2);
-        int hpb = 256 / units;
-        if (hpb > a.h) hpb = (int)a.h;
-        // batch entries per workgroup: re-use cos/sin over a few of them, but
-        // keep at least ~16 workgroups per CU in the grid
-        int bpb = 1;
-        const int64_t head_passes = (a.h + hpb - 1) / hpb;
-        while (bpb * 2 <= a.b && bpb * head_passes < 4 &&
-               a.s * ((a.b + bpb * 2 - 1) / (bpb * 2)) >= 4096)
-            bpb *= 2;
-        const int64_t gy = (a.b + bpb - 1) / bpb;
-        if (gy > 65535) return NHP_ERR_SHAPE;
-        dim3 grid((uint32_t)a.s, (uint32_t)gy);
-        rope_vec_kernel<DT, BWD, Tables><<<grid, hpb * units, 0, a.st>>>(
-            a.out, a.in, tab, (int)a.b, (int)a.h, (int)a.d, (int)a.d2, units, hpb, bpb, a.is[0], a.is[1],
-            a.is[2], a.os[0], a.os[1], a.os[2]);
+        const int cpr = (int)(a.d / V);
+        const int rpw = 64 / cpr;
+        const int rows = (int)(a.b * a.h);
+        const int rows_per_step = 4 * rpw;
+        // Workgroups per position: each makes about four steps (two unrolled loop
+        // iterations) with one set of cos/sin values; measured best on MI355X.
+        const int64_t steps = (rows + rows_per_step - 1) / rows_per_step;
+        int64_t splits = (steps + 3) / 4;
+        splits = rope_tune("NHP_ROPE_SPLITS", (int)splits);
+        if (splits > 65535) splits = 65535;
+        dim3 grid((uint32_t)a.s, (uint32_t)splits);
+        const uint32_t lds = (uint32_t)rope_tune("NHP_ROPE_LDS", 0);
+        const bool flat = (a.is[1] == a.h * a.is[2]) && (a.os[1] == a.h * a.os[2]);
+        if (flat) {
+            rope_vec_kernel<DT, BWD, true, Tables><<<grid, 256, lds, a.st>>>(
+                a.out, a.in, tab, rows, (int)a.h, cpr, (int)(a.d2 / V), rpw, a.is[0], a.is[1], a.is[2], a.os[0],
+                a.os[1], a.os[2]);
+        } else {
+            rope_vec_kernel<DT, BWD, false, Tables><<<grid, 256, lds, a.st>>>(
+                a.out, a.in, tab, rows, (int)a.h, cpr, (int)(a.d2 / V), rpw, a.is[0], a.is[1], a.is[2], a.os[0],
+                a.os[1], a.os[2]);
+        }
     } else {
         const int64_t total = a.s * a.b * a.h * a.d;
         const int64_t blocks = (total + 255) / 256;

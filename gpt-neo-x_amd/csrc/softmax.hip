@@ -9,10 +9,10 @@
 // in registers. One wave-wide load therefore reads L*16 contiguous bytes per
 // row, and a row is read from HBM exactly once and written exactly once.
 //
-//   n <= 256        : L = n/8 rounded up to a power of two, K = 1, 64/L rows per wave
-//   n <= 2048       : one wave per row, K = 1..4
-//   n <= 65536      : W = 2..16 waves per row, partial max / sum exchanged
-//                     through 2*W floats of LDS
+//   n <= 512        : L = n/8 rounded up to a power of two, K = 1, 64/L rows per wave
+//   n <= 65536      : W = 1..8 (16 beyond 32768) waves per row with K = 1..8
+//                     chunks per lane; partial max / sum are exchanged through
+//                     2*W floats of LDS (see plan_row for the choice)
 //   otherwise, or if n % 8 != 0 or a pointer is not 16-byte aligned:
 //                     a scalar three-pass kernel (one workgroup per row).
 //
@@ -26,6 +26,8 @@
 // mask bytes are all 1 is not loaded.
 
 #include "common.hpp"
+
+#include <cstdlib>
 
 namespace nhp {
 
@@ -51,6 +53,11 @@ __device__ __forceinline__ uint32_t chunk_col(int k, int w, int l)
 // Row softmax over the register tile z[K][8]; entries that must not take part
 // hold -inf. On return z holds the probabilities (fp32).
 // `nk`: only slots k < nk hold finite values (a wave-uniform count).
+//
+// With several waves per row every wave first reduces its own part against its
+// own maximum m_w, then the (m_w, s_w) pairs are exchanged through LDS once:
+//   M = max m_w,  S = sum s_w * 2^((m_w - M) log2 e),  p = e * 2^((m_w - M) log2 e) / S
+// which needs one barrier instead of one for the maximum and one for the sum.
 template <int L, int K, int W>
 __device__ __forceinline__ void softmax_tile(float (&z)[K][8], int nk, float* lds, int wave, int lane)
 {
@@ -63,7 +70,6 @@ __device__ __forceinline__ void softmax_tile(float (&z)[K][8], int nk, float* ld
         }
     }
     m = group_reduce<OpMax, L>(m);
-    m = block_combine<OpMax, W>(m, lds, wave, lane);
 
     float sum = 0.0f;
 #pragma unroll
@@ -78,9 +84,25 @@ __device__ __forceinline__ void softmax_tile(float (&z)[K][8], int nk, float* ld
         }
     }
     sum = group_reduce<OpSum, L>(sum);
-    sum = block_combine<OpSum, W>(sum, lds + 16, wave, lane);
 
-    const float inv = 1.0f / sum;
+    float inv;
+    if constexpr (W == 1) {
+        inv = 1.0f / sum;
+    } else {
+        if (lane == 0) {
+            lds[wave] = m;
+            lds[16 + wave] = sum;
+        }
+        __syncthreads();
+        float big = lds[0];
+#pragma unroll
+        for (int i = 1; i < W; ++i) big = fmaxf(big, lds[i]);
+        float total = 0.0f;
+#pragma unroll
+        for (int i = 0; i < W; ++i) total = fmaf(lds[16 + i], exp2_raw((lds[i] - big) * kLog2e), total);
+        // a wave without any valid column has m = -inf and never uses inv
+        inv = exp2_raw((m - big) * kLog2e) / total;
+    }
 #pragma unroll
     for (int k = 0; k < K; ++k) {
         if (k < nk) {
@@ -123,7 +145,10 @@ causal_fwd_kernel(uint16_t* y, const uint16_t* x, float scale, uint32_t total_ro
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int l = lane & (L - 1);
-    const int w = (W > 1) ? wave : 0;
+    // Which of the row's W interleaved segment sets this wave takes rotates with
+    // the row: the leftmost segments are the ones most often below the diagonal,
+    // and wave i of every workgroup sits on the same SIMD of its CU.
+    const int w = (W > 1) ? (int)((wave + blockIdx.x) % W) : 0;
 
     uint32_t row, q;
     locate_row<G>(blockIdx.x, n, wave, lane, L, row, q);
@@ -177,6 +202,8 @@ causal_fwd_kernel(uint16_t* y, const uint16_t* x, float scale, uint32_t total_ro
 
     softmax_tile<L, K, W>(z, nk, lds, wave, lane);
 
+    // The whole row is written in one go, zeros above the diagonal included:
+    // splitting a row's stores in time costs DRAM efficiency.
 #pragma unroll
     for (int k = 0; k < K; ++k) {
         const uint32_t col = chunk_col<L, W>(k, w, l);
@@ -199,7 +226,8 @@ template <int DT, int L, int K, int W, int BW>
 __global__ void __launch_bounds__((Geo<L, K, W, BW>::kThreads))
 masked_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float scale,
                   uint32_t bq_rows, uint32_t sq, uint32_t np, uint32_t n,
-                  uint32_t heads_per_wave, uint32_t head_groups, int mask_per_batch)
+                  uint32_t heads_per_wave, uint32_t head_groups, int mask_per_batch, uint32_t row_blocks,
+                  uint32_t tile)
 {
     using G = Geo<L, K, W, BW>;
     __shared__ float lds[2][32];
@@ -208,11 +236,17 @@ masked_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
     const int l = lane & (L - 1);
     const int w = (W > 1) ? wave : 0;
 
-    // head group varies fastest so that the blocks sharing mask rows are
-    // neighbours in logical order, i.e. run on the same XCD back to back.
-    const uint32_t id = xcd_swizzle(blockIdx.x, gridDim.x);
-    const uint32_t hg = id % head_groups;
-    const uint32_t rb = id / head_groups;
+    // Workgroup order: `tile` consecutive row blocks (all query rows of a
+    // sequence), then the next head group on the same rows, then the next tile.
+    // Neighbouring workgroups thus work on consecutive score rows (what HBM
+    // likes best), and a mask row is used again one tile later, from L2.
+    const uint32_t id = blockIdx.x;
+    const uint32_t per_tile = tile * head_groups;
+    const uint32_t t = id / per_tile;
+    const uint32_t r = id - t * per_tile;
+    const uint32_t tile_rows = (t * tile + tile <= row_blocks) ? tile : row_blocks - t * tile;
+    const uint32_t hg = r / tile_rows;
+    const uint32_t rb = t * tile + (r - hg * tile_rows);
 
     uint32_t local;
     if constexpr (G::kRowsPerBlock == 1) {
@@ -229,21 +263,24 @@ masked_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
     const uint8_t* mrow = mask + (size_t)(mask_per_batch ? bq : qi) * n;
 
     // decode the mask once
-    bool inb[K];    // chunk lies inside the row
-    bool dead[K];   // all eight columns masked: the scores are not needed
+    bool live[K];  // chunk inside the row with at least one unmasked column: scores are read
+    bool dead[K];  // chunk inside the row with all eight columns masked: scores are not needed
+    bool any_dead = false;
     uint32_t mb[K][2];
 #pragma unroll
     for (int k = 0; k < K; ++k) {
         const uint32_t col = chunk_col<L, W>(k, w, l);
-        inb[k] = ok && col < n;
+        const bool inb = ok && col < n;
         mb[k][0] = 0;
         mb[k][1] = 0;
-        if (inb[k]) {
+        if (inb) {
             const u32x2 v = load8(mrow + col);
             mb[k][0] = v[0];
             mb[k][1] = v[1];
         }
-        dead[k] = (mb[k][0] == 0x01010101u) && (mb[k][1] == 0x01010101u);
+        dead[k] = inb && (mb[k][0] == 0x01010101u) && (mb[k][1] == 0x01010101u);
+        live[k] = inb && !dead[k];
+        any_dead = any_dead || dead[k];
     }
 
     const uint32_t h_begin = hg * heads_per_wave;
@@ -258,28 +295,60 @@ masked_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
         for (int k = 0; k < K; ++k) {
             const uint32_t col = chunk_col<L, W>(k, w, l);
             raw[k] = u32x4{0, 0, 0, 0};
-            if (inb[k] && !dead[k]) raw[k] = load16_stream(xr + col);
+            if (live[k]) raw[k] = load16_stream(xr + col);
         }
 
+        // Chunks whose eight columns are all masked hold eight copies of the fill value:
+        // they enter the maximum once, and share one exponential and one output value.
         float z[K][8];
+        float m = any_dead ? kMaskFill : kNegInf;
 #pragma unroll
         for (int k = 0; k < K; ++k) {
-            float f[8];
-            unpack8<DT>(raw[k], f);
+            if (live[k]) {
+                float f[8];
+                unpack8<DT>(raw[k], f);
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const uint32_t byte = (mb[k][j >> 2] >> (8 * (j & 3))) & 0xffu;
-                const float v = (byte == 1u) ? kMaskFill : f[j] * scale;
-                z[k][j] = inb[k] ? v : kNegInf;
+                for (int j = 0; j < 8; ++j) {
+                    const uint32_t byte = (mb[k][j >> 2] >> (8 * (j & 3))) & 0xffu;
+                    z[k][j] = (byte == 1u) ? kMaskFill : f[j] * scale;
+                    m = fmaxf(m, z[k][j]);
+                }
             }
         }
+        m = group_reduce<OpMax, L>(m);
+        m = block_combine<OpMax, W>(m, lds[h & 1], wave, lane);
 
-        softmax_tile<L, K, W>(z, K, lds[h & 1], wave, lane);
+        const float e_dead = exp2_raw(fmaf(kMaskFill - m, kLog2e, kExpBias));
+        float sum = 0.0f;
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            if (live[k]) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float e = exp2_raw(fmaf(z[k][j] - m, kLog2e, kExpBias));
+                    z[k][j] = e;
+                    sum += e;
+                }
+            } else if (dead[k]) {
+                sum += 8.0f * e_dead;
+            }
+        }
+        sum = group_reduce<OpSum, L>(sum);
+        sum = block_combine<OpSum, W>(sum, lds[h & 1] + 16, wave, lane);
+        const float inv = 1.0f / sum;
+        const uint32_t pd = Half2<DT>::pack(e_dead * inv, e_dead * inv);
 
 #pragma unroll
         for (int k = 0; k < K; ++k) {
             const uint32_t col = chunk_col<L, W>(k, w, l);
-            if (inb[k]) store16_stream(yr + col, pack8<DT>(z[k]));
+            if (live[k]) {
+                float o[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) o[j] = z[k][j] * inv;
+                store16_stream(yr + col, pack8<DT>(o));
+            } else if (dead[k]) {
+                store16_stream(yr + col, u32x4{pd, pd, pd, pd});
+            }
         }
     }
 }
@@ -298,7 +367,8 @@ softmax_bwd_kernel(uint16_t* dx, const uint16_t* dy, const uint16_t* y, float sc
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int l = lane & (L - 1);
-    const int w = (W > 1) ? wave : 0;
+    // rotate the segment sets over the waves as in the forward kernel
+    const int w = (W > 1) ? (int)((wave + (CAUSAL ? blockIdx.x : 0u)) % W) : 0;
 
     uint32_t row, q;
     locate_row<G>(blockIdx.x, rows_per_matrix, wave, lane, L, row, q);
@@ -353,10 +423,11 @@ softmax_bwd_kernel(uint16_t* dx, const uint16_t* dy, const uint16_t* y, float sc
     s = group_reduce<OpSum, L>(s);
     s = block_combine<OpSum, W>(s, lds, wave, lane);
 
-    // what the formula gives where dy = y = 0 (masked columns): +0 for finite s
+    // what the formula gives where dy = y = 0 (masked columns): +0 for finite s and scale > 0
     const float zv = scale * fmaf(-0.0f, s, 0.0f);
     const uint32_t zw = Half2<DT>::pack(zv, zv);
 
+    // the whole row is written in one go (see the forward kernel)
 #pragma unroll
     for (int k = 0; k < K; ++k) {
         const uint32_t col = chunk_col<L, W>(k, w, l);
@@ -480,66 +551,95 @@ scalar_bwd_kernel(uint16_t* dx, const uint16_t* dy, const uint16_t* y, float sca
 // ---------------------------------------------------------------------------
 struct RowPlan {
     int L, K, W;
+    uint32_t lds;  // dynamic LDS bytes, only used to bound the number of resident workgroups
 };
 
 constexpr int64_t kMaxResidentRow = 65536;
 constexpr int kBlockWaves = 4;  // waves per workgroup when a wave owns whole rows
 
-static bool plan_row(int64_t n, RowPlan& p)
+#ifdef NHP_TUNING
+// Tuning builds read overrides from the environment on every call.
+static int tune(const char* name, int def)
+{
+    const char* v = getenv(name);
+    return v ? atoi(v) : def;
+}
+#else
+static inline int tune(const char*, int def) { return def; }
+#endif
+
+enum RowKind { kCausalFwd, kCausalBwd, kMaskedFwd, kMaskedBwd };
+
+// Geometry for rows of n elements, from measurements on MI355X. HBM efficiency
+// drops when too many different rows are in flight per CU, and a row should be
+// read and written in bursts that are compact in time, so a row is spread over
+// several waves that each load about 2 KiB of it:
+//   forward (one input tensor): K = 2 chunks per lane;
+//   backward (two input tensors): K = 1;
+//   at most 8 waves per row (workgroups of 1024 threads measured slower), so K
+//   doubles for rows beyond 8 * K KiB; rows beyond 32768 elements use 16 waves;
+//   padding-mask forward: one wave per row up to 2048 elements (K <= 4), since
+//   its waves walk over heads and a multi-wave row would synchronise twice
+//   per head.
+static bool plan_row(int64_t n, RowKind kind, RowPlan& p)
 {
     if (n < 8 || n % 8 != 0 || n > kMaxResidentRow) return false;
     const int64_t chunks = n / 8;
-    if (chunks <= 32) {
+    p.lds = (uint32_t)tune("NHP_LDS", 0);
+    if (chunks <= 64) {
         int L = 1;
         while (L < chunks) L *= 2;
-        p = {L, 1, 1};
+        p.L = L;
+        p.K = 1;
+        p.W = 1;
         return true;
     }
-    if (chunks <= 256) {
-        p = {64, (int)((chunks + 63) / 64), 1};
-        return true;
+    p.L = 64;
+    const int64_t segs = (chunks + 63) / 64;  // 1 KiB segments per row
+    int W, K;
+    if (kind == kMaskedFwd && segs <= 4) {
+        W = 1;
+        K = (int)segs;
+    } else if (segs > 64) {
+        W = 16;
+        K = 8;
+    } else {
+        K = (kind == kCausalFwd || kind == kMaskedFwd) ? 2 : 1;
+        while (8 * K < segs) K *= 2;
+        static const int kWaves[] = {1, 2, 3, 4, 6, 8};
+        W = 8;
+        for (int w : kWaves)
+            if ((int64_t)K * w >= segs) {
+                W = w;
+                break;
+            }
     }
-    for (int W = 2; W <= 16; W *= 2) {
-        const int64_t k = (chunks + 64 * W - 1) / (64 * W);
-        if (k <= 4) {
-            p = {64, k < 3 ? 3 : (int)k, W};
-            return true;
-        }
-    }
-    const int64_t k = (chunks + 1023) / 1024;
-    p = {64, k <= 6 ? 6 : 8, 16};
+    p.W = tune("NHP_W", W);
+    p.K = tune("NHP_K", K);
+    if ((int64_t)p.W * p.K < segs) p.K = (int)((segs + p.W - 1) / p.W);
     return true;
 }
 
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-// Invoke F<L, K, W>() for the plan. The list is the set of instantiated geometries.
-#define NHP_FOR_PLAN(PLAN, CALL)                                     \
-    do {                                                             \
-        const int key_ = (PLAN).L * 10000 + (PLAN).K * 100 + (PLAN).W; \
-        switch (key_) {                                              \
-            case 10101: CALL(1, 1, 1); break;                        \
-            case 20101: CALL(2, 1, 1); break;                        \
-            case 40101: CALL(4, 1, 1); break;                        \
-            case 80101: CALL(8, 1, 1); break;                        \
-            case 160101: CALL(16, 1, 1); break;                      \
-            case 320101: CALL(32, 1, 1); break;                      \
-            case 640101: CALL(64, 1, 1); break;                      \
-            case 640201: CALL(64, 2, 1); break;                      \
-            case 640301: CALL(64, 3, 1); break;                      \
-            case 640401: CALL(64, 4, 1); break;                      \
-            case 640302: CALL(64, 3, 2); break;                      \
-            case 640402: CALL(64, 4, 2); break;                      \
-            case 640304: CALL(64, 3, 4); break;                      \
-            case 640404: CALL(64, 4, 4); break;                      \
-            case 640308: CALL(64, 3, 8); break;                      \
-            case 640408: CALL(64, 4, 8); break;                      \
-            case 640316: CALL(64, 3, 16); break;                     \
-            case 640416: CALL(64, 4, 16); break;                     \
-            case 640616: CALL(64, 6, 16); break;                     \
-            case 640816: CALL(64, 8, 16); break;                     \
-            default: return NHP_ERR_SHAPE;                           \
-        }                                                            \
+// The instantiated geometries (L, K, W).
+#define NHP_GEOMETRIES(X)                                                                          \
+    X(1, 1, 1) X(2, 1, 1) X(4, 1, 1) X(8, 1, 1) X(16, 1, 1) X(32, 1, 1) X(64, 1, 1)                \
+    X(64, 2, 1) X(64, 3, 1) X(64, 4, 1)                                                            \
+    X(64, 1, 2) X(64, 1, 3) X(64, 1, 4) X(64, 1, 6) X(64, 1, 8)                                    \
+    X(64, 2, 2) X(64, 2, 3) X(64, 2, 4) X(64, 2, 6) X(64, 2, 8)                                    \
+    X(64, 4, 4) X(64, 4, 6) X(64, 4, 8) X(64, 8, 6) X(64, 8, 8) X(64, 8, 16)
+
+#define NHP_CASE_(L_, K_, W_) \
+    case (L_) * 10000 + (K_) * 100 + (W_): CALL(L_, K_, W_); break;
+
+// Expands CALL(L, K, W) for the plan's geometry; CALL must be defined at the point of use.
+#define NHP_FOR_PLAN(PLAN)                                                 \
+    do {                                                                   \
+        switch ((PLAN).L * 10000 + (PLAN).K * 100 + (PLAN).W) {            \
+            NHP_GEOMETRIES(NHP_CASE_)                                      \
+            default: return NHP_ERR_SHAPE;                                 \
+        }                                                                  \
     } while (0)
 
 static inline int launch_status()
@@ -556,15 +656,15 @@ static int causal_fwd(void* y, const void* x, float scale, int64_t batches, int6
     RowPlan p;
     uint16_t* yp = static_cast<uint16_t*>(y);
     const uint16_t* xp = static_cast<const uint16_t*>(x);
-    if (plan_row(n, p) && aligned16(x) && aligned16(y)) {
+    if (plan_row(n, kCausalFwd, p) && aligned16(x) && aligned16(y)) {
 #define CALL(L_, K_, W_)                                                                   \
     {                                                                                      \
         using G = Geo<L_, K_, W_, kBlockWaves>;                                            \
         const uint32_t blocks = (uint32_t)((rows + G::kRowsPerBlock - 1) / G::kRowsPerBlock); \
-        causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves><<<blocks, G::kThreads, 0, st>>>(    \
+        causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves><<<blocks, G::kThreads, p.lds, st>>>(    \
             yp, xp, scale, (uint32_t)rows, (uint32_t)n);                                   \
     }
-        NHP_FOR_PLAN(p, CALL);
+        NHP_FOR_PLAN(p);
 #undef CALL
     } else {
         scalar_fwd_kernel<DT, 0><<<(uint32_t)rows, kScalarThreads, 0, st>>>(
@@ -581,15 +681,15 @@ static int softmax_bwd(void* dx, const void* dy, const void* y, float scale, int
     uint16_t* dxp = static_cast<uint16_t*>(dx);
     const uint16_t* dyp = static_cast<const uint16_t*>(dy);
     const uint16_t* yp = static_cast<const uint16_t*>(y);
-    if (plan_row(n, p) && aligned16(dx) && aligned16(dy) && aligned16(y)) {
+    if (plan_row(n, CAUSAL ? kCausalBwd : kMaskedBwd, p) && aligned16(dx) && aligned16(dy) && aligned16(y)) {
 #define CALL(L_, K_, W_)                                                                   \
     {                                                                                      \
         using G = Geo<L_, K_, W_, kBlockWaves>;                                            \
         const uint32_t blocks = (uint32_t)((rows + G::kRowsPerBlock - 1) / G::kRowsPerBlock); \
-        softmax_bwd_kernel<DT, L_, K_, W_, kBlockWaves, CAUSAL><<<blocks, G::kThreads, 0, st>>>( \
+        softmax_bwd_kernel<DT, L_, K_, W_, kBlockWaves, CAUSAL><<<blocks, G::kThreads, p.lds, st>>>( \
             dxp, dyp, yp, scale, (uint32_t)rows, (uint32_t)n, (uint32_t)rows_per_matrix);  \
     }
-        NHP_FOR_PLAN(p, CALL);
+        NHP_FOR_PLAN(p);
 #undef CALL
     } else {
         scalar_bwd_kernel<DT, CAUSAL><<<(uint32_t)rows, kScalarThreads, 0, st>>>(
@@ -598,16 +698,9 @@ static int softmax_bwd(void* dx, const void* dy, const void* y, float scale, int
     return launch_status();
 }
 
-// Heads a wave walks over with one decoded mask row: as many as possible
-// while the grid still holds several waves per SIMD of the 256 CUs.
-static uint32_t pick_heads_per_wave(int64_t bq_row_blocks, int64_t np, int waves_per_block)
-{
-    const int64_t want_waves = 256 * 4 * 8 * 4;  // four full rounds of 8 waves per SIMD
-    int64_t hpw = np;
-    while (hpw > 1 && bq_row_blocks * waves_per_block * ((np + hpw - 1) / hpw) < want_waves)
-        hpw = (hpw + 1) / 2;
-    return (uint32_t)hpw;
-}
+// Heads a wave walks over with one decoded mask row. A few are enough to
+// amortise the decoding; more would only make the access order less sequential.
+static uint32_t pick_heads_per_wave(int64_t np) { return (uint32_t)(np < 4 ? np : 4); }
 
 template <int DT>
 static int masked_fwd(void* y, const void* x, const uint8_t* mask, float scale, int64_t b, int64_t np,
@@ -619,19 +712,22 @@ static int masked_fwd(void* y, const void* x, const uint8_t* mask, float scale, 
     uint16_t* yp = static_cast<uint16_t*>(y);
     const uint16_t* xp = static_cast<const uint16_t*>(x);
     const bool mask_ok = (reinterpret_cast<uintptr_t>(mask) & 7u) == 0;
-    if (plan_row(n, p) && aligned16(x) && aligned16(y) && mask_ok) {
+    if (plan_row(n, kMaskedFwd, p) && aligned16(x) && aligned16(y) && mask_ok) {
 #define CALL(L_, K_, W_)                                                                   \
     {                                                                                      \
         using G = Geo<L_, K_, W_, kBlockWaves>;                                            \
         const int64_t rb = (bq_rows + G::kRowsPerBlock - 1) / G::kRowsPerBlock;            \
-        const uint32_t hpw = pick_heads_per_wave(rb, np, G::kThreads / kWave);             \
+        const uint32_t hpw = (uint32_t)tune("NHP_HPW", (int)pick_heads_per_wave(np));       \
         const uint32_t hgs = (uint32_t)((np + hpw - 1) / hpw);                             \
         if (rb * hgs >= kMaxRows) return NHP_ERR_SHAPE;                                    \
-        masked_fwd_kernel<DT, L_, K_, W_, kBlockWaves><<<(uint32_t)(rb * hgs), G::kThreads, 0, st>>>( \
+        int64_t tile = tune("NHP_MASK_TILE", (int)((sq + G::kRowsPerBlock - 1) / G::kRowsPerBlock)); \
+        if (tile < 1) tile = 1;                                                            \
+        if (tile > rb) tile = rb;                                                          \
+        masked_fwd_kernel<DT, L_, K_, W_, kBlockWaves><<<(uint32_t)(rb * hgs), G::kThreads, p.lds, st>>>( \
             yp, xp, mask, scale, (uint32_t)bq_rows, (uint32_t)sq, (uint32_t)np, (uint32_t)n, hpw, hgs, \
-            per_batch);                                                                    \
+            per_batch, (uint32_t)rb, (uint32_t)tile);                                      \
     }
-        NHP_FOR_PLAN(p, CALL);
+        NHP_FOR_PLAN(p);
 #undef CALL
     } else {
         scalar_fwd_kernel<DT, 1><<<(uint32_t)(b * np * sq), kScalarThreads, 0, st>>>(

@@ -38,11 +38,10 @@ def _run_freqs(name, fn, t, freqs, transpose_output, what):
     _check(t.dtype in _FLOATS, f"{name}: unsupported dtype {t.dtype}")
     _hp.require_gpu(t, name)
     _hp.require_gpu(freqs, name)
-    t = t.detach()
-    f = freqs.detach().contiguous()
+    f = freqs.contiguous()
     out = _new_output(t, transpose_output)
     s, b, h, d = t.shape
-    with torch.cuda.device(t.device):
+    with _hp.device_guard(t):
         rc = fn(out.data_ptr(), t.data_ptr(), f.data_ptr(), s, b, h, d, f.size(3), _hp.strides4(t),
                 _hp.strides4(out), _hp.dtype_code(t, name), _hp.stream_of(t))
     _hp.check(rc, name)
@@ -68,12 +67,11 @@ def _run_cached(name, fn, t, cos, sin, transpose_output, what):
     _hp.require_gpu(t, name)
     _hp.require_gpu(cos, name)
     _hp.require_gpu(sin, name)
-    t = t.detach()
-    c = cos.detach().contiguous()
-    sn = sin.detach().contiguous()
+    c = cos.contiguous()
+    sn = sin.contiguous()
     out = _new_output(t, transpose_output)
     s, b, h, d = t.shape
-    with torch.cuda.device(t.device):
+    with _hp.device_guard(t):
         rc = fn(out.data_ptr(), t.data_ptr(), c.data_ptr(), sn.data_ptr(), s, b, h, d, c.size(3),
                 _hp.strides4(t), _hp.strides4(out), _hp.dtype_code(t, name), _hp.dtype_code(c, name),
                 _hp.stream_of(t))

@@ -35,10 +35,10 @@ def forward(input, mask, scale_factor):
         raise RuntimeError("mask must have shape [pad_batches, 1, query_seq_len, key_seq_len]")
     _hp.require_gpu(input, "scaled_masked_softmax_cuda.forward")
     _hp.require_gpu(mask, "scaled_masked_softmax_cuda.forward")
-    x = input.detach().contiguous()
-    m = mask.detach().contiguous()
+    x = input.contiguous()
+    m = mask.contiguous()
     y = torch.empty_like(x)
-    with torch.cuda.device(x.device):
+    with _hp.device_guard(x):
         rc = _hp.lib().nhp_masked_softmax_fwd(
             y.data_ptr(), x.data_ptr(), m.data_ptr(), float(scale_factor), b, np_, sq, sk, m.size(0),
             _hp.dtype_code(x, "forward"), _hp.stream_of(x))
@@ -62,7 +62,7 @@ def backward(output_grads, softmax_results, scale_factor):
     y = softmax_results.detach().contiguous()
     sk = g.size(3)
     rows = g.numel() // sk if sk else 0
-    with torch.cuda.device(g.device):
+    with _hp.device_guard(g):
         rc = _hp.lib().nhp_masked_softmax_bwd(
             g.data_ptr(), g.data_ptr(), y.data_ptr(), float(scale_factor), rows, sk,
             _hp.dtype_code(g, "backward"), _hp.stream_of(g))

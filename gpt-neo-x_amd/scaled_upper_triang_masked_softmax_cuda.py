@@ -25,9 +25,9 @@ def forward(input, scale_factor):
     if input.size(1) != input.size(2):
         raise RuntimeError("expected a square [attn_batches, seq_len, seq_len] tensor")
     _hp.require_gpu(input, "scaled_upper_triang_masked_softmax_cuda.forward")
-    x = input.detach().contiguous()
+    x = input.contiguous()
     y = torch.empty_like(x)
-    with torch.cuda.device(x.device):
+    with _hp.device_guard(x):
         rc = _hp.lib().nhp_causal_softmax_fwd(
             y.data_ptr(), x.data_ptr(), float(scale_factor), x.size(0), x.size(1), _hp.dtype_code(x, "forward"),
             _hp.stream_of(x))
@@ -54,7 +54,7 @@ def backward(output_grads, softmax_results, scale_factor):
     _hp.require_gpu(softmax_results, "scaled_upper_triang_masked_softmax_cuda.backward")
     g = output_grads.detach().contiguous()
     y = softmax_results.detach().contiguous()
-    with torch.cuda.device(g.device):
+    with _hp.device_guard(g):
         rc = _hp.lib().nhp_causal_softmax_bwd(
             g.data_ptr(), g.data_ptr(), y.data_ptr(), float(scale_factor), g.size(0), g.size(1),
             _hp.dtype_code(g, "backward"), _hp.stream_of(g))
