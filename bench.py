@@ -42,8 +42,8 @@ METRIC = "achieved HBM GB/s (% of MI355X peak), causal softmax+rotary fwd/bwd, 1
 HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch of the dominant kernel of the default workload measured
-# with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), see profiles/; None until measured.
-MEASURED_TRAFFIC_BYTES = {"pythia-1.4b": None}
+# with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE; profiles/pythia-1.4b_step_hbm_traffic.txt).
+MEASURED_TRAFFIC_BYTES = {"pythia-1.4b": 2181026543}
 
 
 def tri(n):
@@ -253,6 +253,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="pythia-1.4b")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="run one plain 1 GiB device copy first (reference for scaling rocprofv3 --pmc byte counters)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         raise SystemExit("bench.py measures one GPU; this hot path has no multi-GPU mode (run with --gpus 1)")
@@ -266,6 +268,15 @@ def main():
     load()  # raises if libneox_hotpath.so cannot be loaded; there is no fallback
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.calibration_copy:
+        # 2^29 bf16 elements: the copy kernel reads 1 GiB and writes 1 GiB
+        src = torch.ones(1 << 29, dtype=torch.bfloat16, device=dev)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     step, kernel_bytes, dense_bytes, dominant, dtype, cfg = make_workload(args.workload, torch, dev)
     # Timed region: K steps; only the dominant kernel is bracketed by events
