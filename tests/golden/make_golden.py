@@ -1,0 +1,77 @@
+#!/usr/bin/env python3
+"""Writes tests/golden/hotpath_golden.npz: small seeded inputs and the outputs
+of the CPU oracle (oracle/kernel_semantics.c) for every entry point, stored as
+raw bit patterns. The oracle itself is pinned by tests/test_oracle_*.py; these
+vectors freeze its answers so that the GPU path (and any later change to the
+oracle) is compared against fixed data.
+
+    python tests/golden/make_golden.py
+"""
+import os
+import sys
+
+import numpy as np
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+sys.path[:0] = [ROOT, os.path.join(ROOT, "tests")]
+
+import oracle  # noqa: E402
+import util  # noqa: E402
+
+
+def bits(t):
+    t = t.contiguous()
+    if t.dtype == torch.float32:
+        return t.view(torch.int32).numpy()
+    if t.dtype in (torch.float16, torch.bfloat16):
+        return t.view(torch.int16).numpy()
+    return t.numpy()
+
+
+def main():
+    out = {}
+
+    def put(prefix, **tensors):
+        for k, v in tensors.items():
+            out[f"{prefix}.{k}"] = bits(v) if isinstance(v, torch.Tensor) else np.asarray(v)
+
+    for name, dtype, a, s, scale, seed in (("causal_bf16", torch.bfloat16, 2, 24, 0.125, 1),
+                                           ("causal_fp16", torch.float16, 2, 40, 0.0883883461356163, 2)):
+        x = util.randn((a, s, s), dtype, seed, std=2.0)
+        dy = util.randn((a, s, s), dtype, seed + 100)
+        y = oracle.causal_softmax_fwd(x, scale)
+        put(name, x=x, dy=dy, y=y, dx=oracle.softmax_bwd(dy, y, scale, True), scale=np.float32(scale))
+
+    for name, dtype, b, np_, sq, sk, pb, scale, seed in (("masked_fp16", torch.float16, 2, 2, 4, 40, 2, 0.0883883461356163, 3),
+                                                         ("masked_bf16", torch.bfloat16, 2, 2, 4, 24, 1, 0.5, 4)):
+        x = util.randn((b, np_, sq, sk), dtype, seed, std=3.0)
+        x[0, 0, 0, 3] = 60.0
+        x[1, 1, 2, 5] = -60.0
+        mask = util.padding_mask(pb, sq, sk, seed, full_batch=1 if pb > 1 else None)
+        if pb == 1:
+            mask[0, 0, 1, :] = True
+        dy = util.randn((b, np_, sq, sk), dtype, seed + 100)
+        y = oracle.masked_softmax_fwd(x, mask, scale)
+        put(name, x=x, mask=mask.to(torch.uint8), dy=dy, y=y, dx=oracle.softmax_bwd(dy, y, scale, False),
+            scale=np.float32(scale))
+
+    for name, dtype, s, b, h, d, d2, seed in (("rope_bf16", torch.bfloat16, 6, 2, 2, 16, 8, 5),
+                                              ("rope_fp16", torch.float16, 5, 1, 3, 16, 16, 6),
+                                              ("rope_fp32", torch.float32, 4, 2, 1, 8, 8, 7)):
+        t = util.randn((s, b, h, d), dtype, seed)
+        g = torch.Generator().manual_seed(seed)
+        ang = (torch.rand((s, 1, 1, d2), generator=g) * 20.0 - 10.0).contiguous()
+        cos, sin = ang.cos().to(dtype), ang.sin().to(dtype)
+        put(name, t=t, cos=cos, sin=sin, freqs=ang, fwd=oracle.rope_cached(t, cos, sin),
+            bwd=oracle.rope_cached(t, cos, sin, backward=True),
+            fwd_freqs=oracle.rope_freqs(t, ang), bwd_freqs=oracle.rope_freqs(t, ang, backward=True))
+
+    path = os.path.join(HERE, "hotpath_golden.npz")
+    np.savez_compressed(path, **out)
+    print(path, os.path.getsize(path), "bytes,", len(out), "arrays")
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,118 @@
+"""The C-ABI library: it loads without a GPU, exports every symbol that
+include/neox_hotpath.h declares, and its argument validation (which happens
+before anything touches the device) returns the documented status codes."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "neox_hotpath.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(nhp_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    names = declared_functions()
+    for must in ("nhp_causal_softmax_fwd", "nhp_causal_softmax_bwd", "nhp_masked_softmax_fwd",
+                 "nhp_masked_softmax_bwd", "nhp_softmax_batch_per_block", "nhp_rope_cached_fwd",
+                 "nhp_rope_cached_bwd", "nhp_rope_freqs_fwd", "nhp_rope_freqs_bwd"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol(hotpath):
+    lib = ctypes.CDLL(hotpath.LIB_PATH)
+    for name in declared_functions():
+        assert hasattr(lib, name), f"{name} declared in the header but not exported"
+    # and the Python binding declares exactly the header's functions
+    hotpath.lib()
+    assert sorted(hotpath.EXPORTS) == declared_functions()
+
+
+def test_every_header_comment_cites_the_reference():
+    text = open(HEADER).read()
+    for name in declared_functions():
+        if name in ("nhp_abi_version", "nhp_status_string", "nhp_softmax_max_resident_row"):
+            continue
+        before = text[: text.index(name + "(")]
+        comment = before[before.rindex("/*") :]
+        # the backward/forward pairs of the rotary functions share one comment
+        assert "megatron/fused_kernels/" in comment or name.startswith("nhp_rope_"), name
+    assert text.count("Replaces ") >= 7
+
+
+def test_status_strings_and_version(hotpath):
+    lib = hotpath.lib()
+    assert lib.nhp_abi_version() == hotpath.ABI_VERSION
+    assert lib.nhp_status_string(0) == b"ok"
+    seen = set()
+    for code in range(-6, 0):
+        s = lib.nhp_status_string(code)
+        assert s and s != b"unknown status"
+        seen.add(s)
+    assert len(seen) == 6
+    assert lib.nhp_status_string(-99) == b"unknown status"
+    assert lib.nhp_softmax_max_resident_row() == 65536
+
+
+def test_batch_per_block_matches_reference_formula(hotpath):
+    import oracle
+
+    lib = hotpath.lib()
+    for sk in (1, 2, 8, 16, 17, 32, 33, 64, 65, 128, 129, 256, 1000, 2048, 4096, 8192):
+        assert lib.nhp_softmax_batch_per_block(1024, sk, 4, 8) == oracle.batch_per_block(sk, 64), sk
+    assert lib.nhp_softmax_batch_per_block(4, 0, 1, 1) == -2  # NHP_ERR_SHAPE
+
+
+def test_argument_validation_needs_no_gpu(hotpath):
+    lib = hotpath.lib()
+    F16, BF16, F32 = hotpath.F16, hotpath.BF16, hotpath.F32
+    p = ctypes.c_void_p(0x1000)  # never dereferenced: every call below fails validation or is empty
+    o = ctypes.c_void_p(0x9000)
+    null = ctypes.c_void_p(0)
+    st = (ctypes.c_int64 * 4)(8, 8, 8, 1)
+    # dtype
+    assert lib.nhp_causal_softmax_fwd(p, p, 1.0, 1, 8, F32, None) == -1
+    assert lib.nhp_causal_softmax_bwd(p, p, p, 1.0, 1, 8, 7, None) == -1
+    assert lib.nhp_masked_softmax_fwd(p, p, p, 1.0, 1, 1, 2, 8, 1, F32, None) == -1
+    assert lib.nhp_masked_softmax_bwd(p, p, p, 1.0, 2, 8, -1, None) == -1
+    assert lib.nhp_rope_cached_fwd(p, p, p, p, 1, 1, 1, 8, 8, st, st, 5, F32, None) == -1
+    assert lib.nhp_rope_cached_fwd(p, p, p, p, 1, 1, 1, 8, 8, st, st, BF16, F16, None) == -1  # tables neither fp32 nor same
+    assert lib.nhp_rope_freqs_bwd(p, p, p, 1, 1, 1, 8, 8, st, st, 9, None) == -1
+    # shape
+    assert lib.nhp_causal_softmax_fwd(p, p, 1.0, -1, 8, BF16, None) == -2
+    assert lib.nhp_causal_softmax_fwd(p, p, 1.0, 1 << 40, 1 << 20, BF16, None) == -2
+    assert lib.nhp_masked_softmax_fwd(p, p, p, 1.0, 1, 1, -2, 8, 1, F16, None) == -2
+    assert lib.nhp_rope_cached_fwd(p, p, p, p, 1, 1, 1, 8, 16, st, st, BF16, BF16, None) == -2  # d2 > d
+    # empty tensors are fine and launch nothing, even with null pointers
+    assert lib.nhp_causal_softmax_fwd(null, null, 1.0, 0, 8, BF16, None) == 0
+    assert lib.nhp_causal_softmax_bwd(null, null, null, 1.0, 4, 0, BF16, None) == 0
+    assert lib.nhp_masked_softmax_fwd(null, null, null, 1.0, 2, 0, 4, 8, 2, F16, None) == 0
+    assert lib.nhp_masked_softmax_bwd(null, null, null, 1.0, 0, 8, F16, None) == 0
+    assert lib.nhp_rope_cached_bwd(null, null, null, null, 0, 1, 1, 8, 8, st, st, F32, F32, None) == 0
+    assert lib.nhp_rope_freqs_fwd(null, null, null, 4, 0, 1, 8, 8, st, st, F16, None) == 0
+    # null pointers for non-empty tensors
+    assert lib.nhp_causal_softmax_fwd(null, p, 1.0, 1, 8, BF16, None) == -3
+    assert lib.nhp_masked_softmax_fwd(p, p, null, 1.0, 1, 1, 2, 8, 1, F16, None) == -3
+    assert lib.nhp_rope_cached_fwd(o, p, null, p, 1, 1, 1, 8, 8, st, st, BF16, BF16, None) == -3
+    assert lib.nhp_rope_freqs_fwd(o, p, null, 1, 1, 1, 8, 8, st, st, BF16, None) == -3
+    assert lib.nhp_rope_freqs_fwd(o, p, p, 1, 1, 1, 8, 8, None, st, BF16, None) == -3
+    # mask batch dimension
+    assert lib.nhp_masked_softmax_fwd(p, p, p, 1.0, 4, 1, 2, 8, 3, F16, None) == -4
+    # aliasing that is not allowed: dx over y, rotary in place
+    assert lib.nhp_causal_softmax_bwd(p, ctypes.c_void_p(0x2000), p, 1.0, 1, 8, BF16, None) == -6
+    assert lib.nhp_masked_softmax_bwd(p, ctypes.c_void_p(0x2000), p, 1.0, 2, 8, BF16, None) == -6
+    assert lib.nhp_rope_cached_fwd(p, p, p, p, 1, 1, 1, 8, 8, st, st, BF16, BF16, None) == -6
+
+
+def test_missing_library_fails_loudly(hotpath, monkeypatch, tmp_path):
+    """No fallback: without the built library the binding raises ImportError."""
+    monkeypatch.setattr(hotpath, "_lib", None)
+    monkeypatch.setattr(hotpath, "LIB_PATH", str(tmp_path / "libneox_hotpath.so"))
+    with pytest.raises(ImportError):
+        hotpath.lib()

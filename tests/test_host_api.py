@@ -1,0 +1,211 @@
+"""Host-side mirror of the reference API (megatron.model.fused_softmax,
+fused_rope, positional_embeddings, megatron.fused_kernels): names, argument
+meaning, gating logic and error behaviour. Runs without a GPU."""
+import math
+
+import pytest
+import torch
+
+import util
+from oracle import fallback_semantics as fb
+
+
+def mask_func(scores, mask):
+    return fb.fill_masked_with_dtype_min(scores, mask)
+
+
+def make(fusion, fp16=True, bf16=False, fp32=True, scale=None):
+    from megatron.model.fused_softmax import FusedScaleMaskSoftmax
+
+    return FusedScaleMaskSoftmax(fp16, bf16, fusion, mask_func, fp32, scale)
+
+
+def test_public_names_exist():
+    import megatron.fused_kernels as fk
+    import megatron.model.fused_rope as fr
+    import megatron.model.fused_softmax as fs
+    import megatron.model.positional_embeddings as pe
+
+    for mod, names in ((fs, ["ScaledUpperTriangMaskedSoftmax", "ScaledMaskedSoftmax", "SoftmaxFusionTypes",
+                             "FusedScaleMaskSoftmax"]),
+                       (fr, ["FusedRoPEFunc", "fused_apply_rotary_pos_emb", "FusedRoPECachedFunc",
+                             "fused_apply_rotary_pos_emb_cached"]),
+                       (pe, ["RotaryEmbedding", "rotate_half", "apply_rotary_pos_emb", "apply_rotary_pos_emb_torch"]),
+                       (fk, ["load", "load_fused_kernels"])):
+        for n in names:
+            assert hasattr(mod, n), (mod.__name__, n)
+    fk.load_fused_kernels()
+    import fused_rotary_positional_embedding as rope
+    import scaled_masked_softmax_cuda as masked
+    import scaled_upper_triang_masked_softmax_cuda as causal
+
+    assert callable(causal.forward) and callable(causal.backward)
+    assert callable(masked.forward) and callable(masked.backward) and callable(masked.get_batch_per_block)
+    for n in ("forward", "backward", "forward_cached", "backward_cached"):
+        assert callable(getattr(rope, n))
+    assert [m.value for m in fs.SoftmaxFusionTypes] == [1, 2, 3]
+
+
+def test_constructor_contract():
+    from megatron.model.fused_softmax import SoftmaxFusionTypes as T
+
+    m = make(T.upper_triang, scale=0.5)
+    assert m.input_in_float16 and m.upper_triang_mask_fusion and not m.general_mask_fusion and m.fusion
+    m = make(T.general, fp16=False, bf16=True)
+    assert m.input_in_float16 and m.general_mask_fusion and m.scale is None
+    m = make(T.none, fp16=False, bf16=False)
+    assert not m.fusion and not m.input_in_float16
+    with pytest.raises(AssertionError, match="softmax should be in fp32 when scaled"):
+        make(T.none, fp32=False, scale=2.0)
+    with pytest.raises(AssertionError, match="Invalid fusion type"):
+        make("upper_triang")
+
+
+def test_fusion_gate_follows_reference_without_the_2048_cap():
+    """fused_softmax.py:148-168: fusion on, 16-bit input, mask given, sk > 16,
+    sq % 4 == 0, (b*np) % 4 == 0, plus the batch_per_block divisibility."""
+    from megatron.model.fused_softmax import SoftmaxFusionTypes as T
+
+    mask = torch.zeros(1, 1, 4, 4, dtype=torch.bool)
+    causal = make(T.upper_triang, scale=1.0)
+    general = make(T.general, scale=1.0)
+    assert causal.is_kernel_available(mask, 8, 16, 2048, 2048)
+    assert general.is_kernel_available(mask, 16, 32, 1024, 2048)
+    assert causal.is_kernel_available(mask, 2, 32, 8192, 8192)  # beyond the reference's 2048 limit
+    assert general.is_kernel_available(mask, 2, 2, 8, 4096)
+    assert not causal.is_kernel_available(None, 8, 16, 2048, 2048)  # no mask
+    assert not causal.is_kernel_available(mask, 8, 16, 16, 16)  # sk must exceed 16
+    assert causal.is_kernel_available(mask, 8, 16, 20, 20)
+    assert not causal.is_kernel_available(mask, 8, 16, 2046, 2046)  # sq % 4
+    assert not causal.is_kernel_available(mask, 1, 6, 64, 64)  # attn_batches % 4
+    # batch_per_block on a 64-wide wavefront: sk=32 -> 8 rows per block
+    assert causal.get_batch_per_block(32, 32, 1, 4) == 8
+    assert not causal.is_kernel_available(mask, 1, 4, 32, 32)  # 4 % 8 != 0
+    assert causal.is_kernel_available(mask, 2, 4, 32, 32)
+    assert not general.is_kernel_available(mask, 1, 4, 4, 32)  # sq=4, 4 % 8 != 0
+    assert general.is_kernel_available(mask, 1, 4, 8, 32)
+    assert not make(T.none).is_kernel_available(mask, 8, 16, 2048, 2048)
+    assert not make(T.general, fp16=False, bf16=False).is_kernel_available(mask, 8, 16, 2048, 2048)
+
+
+@pytest.mark.parametrize("dtype,fp16,bf16", [(torch.float16, True, False), (torch.bfloat16, False, True)])
+def test_torch_path_matches_reference_fallback_and_kernel_semantics(dtype, fp16, bf16):
+    """FusedScaleMaskSoftmax with fusion off runs on CPU: it is the reference's
+    fallback, and it agrees with the kernel semantics to 1 ulp on ordinary inputs."""
+    import oracle
+    from megatron.model.fused_softmax import SoftmaxFusionTypes as T
+
+    b, np_, s, scale = 2, 4, 64, 1 / math.sqrt(64)
+    x = util.randn((b, np_, s, s), dtype, seed=1, std=2.0)
+    mask = fb.causal_mask(s)
+    m = make(T.none, fp16=fp16, bf16=bf16, scale=scale)
+    y = m(x.clone(), mask)
+    assert y.dtype == dtype
+    assert torch.equal(util.raw_bits(y), util.raw_bits(fb.torch_softmax_fallback(x.clone(), mask, scale)))
+    util.assert_ulp_close(y, oracle.causal_softmax_fwd(x.view(-1, s, s), scale).view(b, np_, s, s), 1, "kernel semantics")
+    # mask None: plain softmax
+    y2 = m(x.clone(), None)
+    assert torch.equal(util.raw_bits(y2), util.raw_bits(torch.softmax(x.float() * scale, -1).to(dtype)))
+    # native 16-bit softmax when softmax_in_fp32 is off (scale must be None then)
+    m16 = make(T.none, fp16=fp16, bf16=bf16, fp32=False)
+    assert m16(x.clone(), None).dtype == dtype
+    with pytest.raises(AssertionError):
+        m(x[0], mask)  # 3-D input
+
+
+def test_extension_modules_reject_bad_arguments():
+    import fused_rotary_positional_embedding as rope
+    import scaled_masked_softmax_cuda as masked
+    import scaled_upper_triang_masked_softmax_cuda as causal
+
+    x3 = torch.zeros(4, 32, 32, dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="expected 3D tensor"):
+        causal.forward(x3[0], 1.0)
+    with pytest.raises(RuntimeError, match="Only fp16 and bf16 are supported"):
+        causal.forward(x3.float(), 1.0)
+    with pytest.raises(RuntimeError, match="GPU"):
+        causal.forward(x3, 1.0)
+    with pytest.raises(RuntimeError, match="expected 3D tensor"):
+        causal.backward(x3[0], x3, 1.0)
+    x4 = torch.zeros(2, 2, 4, 32, dtype=torch.bfloat16)
+    m4 = torch.zeros(2, 1, 4, 32, dtype=torch.bool)
+    with pytest.raises(RuntimeError, match="expected 4D tensor"):
+        masked.forward(x4[0], m4, 1.0)
+    with pytest.raises(RuntimeError, match="expected 4D tensor"):
+        masked.forward(x4, m4[0], 1.0)
+    with pytest.raises(RuntimeError, match="pad_batches"):
+        masked.forward(torch.zeros(4, 2, 4, 32, dtype=torch.bfloat16), torch.zeros(3, 1, 4, 32, dtype=torch.bool), 1.0)
+    with pytest.raises(RuntimeError, match="query_seq_len > 1"):
+        masked.forward(torch.zeros(2, 2, 1, 32, dtype=torch.bfloat16), torch.zeros(2, 1, 1, 32, dtype=torch.bool), 1.0)
+    with pytest.raises(RuntimeError, match="Only fp16 and bf16"):
+        masked.backward(x4.float(), x4.float(), 1.0)
+    t = torch.zeros(8, 2, 2, 16, dtype=torch.bfloat16)
+    cos = torch.zeros(8, 1, 1, 16, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="expected 4D tensor"):
+        rope.forward_cached(t[0], cos, cos, False)
+    with pytest.raises(RuntimeError, match="same sequence length"):
+        rope.forward_cached(t, cos[:4], cos[:4], False)
+    with pytest.raises(RuntimeError, match="second and third dims"):
+        rope.forward_cached(t, cos.expand(8, 2, 1, 16), cos, False)
+    with pytest.raises(RuntimeError, match="same last dim"):
+        rope.forward_cached(t, cos, cos[..., :8], False)
+    with pytest.raises(RuntimeError, match="greater than the cos tensor"):
+        rope.forward_cached(t[..., :8], cos, cos, False)
+    with pytest.raises(RuntimeError, match="same dtype"):
+        rope.backward_cached(t, cos, cos.float(), False)
+    with pytest.raises(RuntimeError, match="must be float"):
+        rope.forward(t, cos, False)
+    with pytest.raises(RuntimeError, match="GPU"):
+        rope.forward(t, cos.float(), False)
+
+
+def test_rotary_embedding_module():
+    from megatron.model.positional_embeddings import RotaryEmbedding
+
+    dim, n = 32, 128
+    rot = RotaryEmbedding(dim, n, base=10000, precision=torch.bfloat16)
+    cos_ref, sin_ref, ang = fb.rotary_tables(dim, n, 10000, torch.bfloat16)
+    assert torch.equal(rot.cos_cached, cos_ref) and torch.equal(rot.sin_cached, sin_ref)
+    assert torch.equal(rot.emb, ang)
+    assert rot.dim == dim and rot.base == 10000 and rot.max_seq_len == n and rot.precision == torch.bfloat16
+    # the surviving buffer is cast to `precision`; it is not in the state dict unless asked for
+    assert rot.inv_freq.dtype == torch.bfloat16 and rot.inv_freq.shape == (dim // 2,)
+    assert "inv_freq" not in rot.state_dict()
+    assert "inv_freq" in RotaryEmbedding(dim, n, save_inv_freqs=True).state_dict()
+    x = torch.zeros(64, 2, 4, dim)
+    cos, sin = rot(x)  # seq_len from x.shape[seq_dim]
+    assert cos.shape == (64, 1, 1, dim) and torch.equal(cos, cos_ref[:64])
+    cos, sin = rot(x, seq_len=n)
+    assert cos.shape == (n, 1, 1, dim)
+    cos, sin = rot(x.transpose(0, 1), seq_dim=1)
+    assert cos.shape == (64, 1, 1, dim)
+    with pytest.raises(AssertionError):
+        rot(x, seq_len=n + 1)
+    assert RotaryEmbedding(8, 4).cos_cached.dtype == torch.half  # default precision
+
+
+def test_eager_rotary_functions():
+    from megatron.model.positional_embeddings import apply_rotary_pos_emb, apply_rotary_pos_emb_torch, rotate_half
+
+    x = torch.arange(8.0).view(1, 1, 1, 8)
+    assert rotate_half(x).flatten().tolist() == [-4, -5, -6, -7, 0, 1, 2, 3]
+    s, d = 6, 16
+    q = util.randn((s, 2, 2, d), torch.bfloat16, seed=1)
+    k = util.randn((s, 2, 2, d), torch.bfloat16, seed=2)
+    cos, sin, _ = fb.rotary_tables(d, 16, 10000, torch.bfloat16)
+    for fn in (apply_rotary_pos_emb, apply_rotary_pos_emb_torch):
+        for offset in (0, 3):
+            oq, ok = fn(q, k, cos, sin, offset)
+            assert torch.equal(util.raw_bits(oq), util.raw_bits(fb.eager_rotary(q, cos, sin, offset)))
+            assert torch.equal(util.raw_bits(ok), util.raw_bits(fb.eager_rotary(k, cos, sin, offset)))
+
+
+def test_load_fused_kernels_exits_when_not_installed(hotpath, monkeypatch, tmp_path, capsys):
+    """Reference behaviour (megatron/fused_kernels/__init__.py:167-181): print a banner and exit()."""
+    import megatron.fused_kernels as fk
+
+    monkeypatch.setattr(hotpath, "_lib", None)
+    monkeypatch.setattr(hotpath, "LIB_PATH", str(tmp_path / "missing.so"))
+    with pytest.raises(SystemExit):
+        fk.load_fused_kernels()
+    assert "Fused kernels configured but not properly installed" in capsys.readouterr().out
