@@ -174,11 +174,10 @@ struct FreqTable {
 // Requires: stride_d == 1 on both sides, d % V == 0, d2 % (2V) == 0, d <= 64 V,
 // every other stride a multiple of V, 16-byte aligned base pointers and tables.
 // ---------------------------------------------------------------------------
-constexpr int kRopeUnroll = 2;
-
 // FLAT: the batch and head dimensions collapse into one row dimension on both
 // sides (stride_b == h * stride_h), which saves the division by h per row.
-template <int DT, bool BWD, bool FLAT, typename Tables>
+// U: rows in flight per lane (loads of U steps are issued before the first is used).
+template <int DT, bool BWD, bool FLAT, int U, typename Tables>
 __global__ void __launch_bounds__(256)
 rope_vec_kernel(void* out, const void* in, Tables tab, int rows, int h, int cpr, int rot_chunks, int rpw,
                 int64_t is_s, int64_t is_b, int64_t is_h, int64_t os_s, int64_t os_b, int64_t os_h)
@@ -222,12 +221,12 @@ rope_vec_kernel(void* out, const void* in, Tables tab, int rows, int h, int cpr,
     const int rows_per_step = 4 * rpw;
     const int stride = rows_per_step * (int)gridDim.y;
     // All lanes of a row (a lane and its partner included) share r0 and leave the loop together.
-    for (int r0 = (int)blockIdx.y * rows_per_step + wave * rpw + rl; r0 < rows; r0 += stride * kRopeUnroll) {
-        u32x4 raw[kRopeUnroll];
-        int64_t dst_off[kRopeUnroll];
-        bool on[kRopeUnroll];
+    for (int r0 = (int)blockIdx.y * rows_per_step + wave * rpw + rl; r0 < rows; r0 += stride * U) {
+        u32x4 raw[U];
+        int64_t dst_off[U];
+        bool on[U];
 #pragma unroll
-        for (int u = 0; u < kRopeUnroll; ++u) {
+        for (int u = 0; u < U; ++u) {
             const int r = r0 + u * stride;
             on[u] = lane_on && r < rows;
             raw[u] = u32x4{0, 0, 0, 0};
@@ -245,7 +244,7 @@ rope_vec_kernel(void* out, const void* in, Tables tab, int rows, int h, int cpr,
             }
         }
 #pragma unroll
-        for (int u = 0; u < kRopeUnroll; ++u) {
+        for (int u = 0; u < U; ++u) {
             u32x4 praw;
 #pragma unroll
             for (int i = 0; i < 4; ++i)
@@ -365,15 +364,17 @@ static int rope_launch(const RopeArgs& a, const Tables& tab, bool tables_ok)
         dim3 grid((uint32_t)a.s, (uint32_t)splits);
         const uint32_t lds = (uint32_t)rope_tune("NHP_ROPE_LDS", 0);
         const bool flat = (a.is[1] == a.h * a.is[2]) && (a.os[1] == a.h * a.os[2]);
+#define NHP_ROPE_LAUNCH(FLAT_, U_)                                                                         \
+    rope_vec_kernel<DT, BWD, FLAT_, U_, Tables><<<grid, 256, lds, a.st>>>(                                 \
+        a.out, a.in, tab, rows, (int)a.h, cpr, (int)(a.d2 / V), rpw, a.is[0], a.is[1], a.is[2], a.os[0],   \
+        a.os[1], a.os[2])
+        // two rows in flight per lane measured best (one is short of latency cover, four adds nothing)
         if (flat) {
-            rope_vec_kernel<DT, BWD, true, Tables><<<grid, 256, lds, a.st>>>(
-                a.out, a.in, tab, rows, (int)a.h, cpr, (int)(a.d2 / V), rpw, a.is[0], a.is[1], a.is[2], a.os[0],
-                a.os[1], a.os[2]);
+            NHP_ROPE_LAUNCH(true, 2);
         } else {
-            rope_vec_kernel<DT, BWD, false, Tables><<<grid, 256, lds, a.st>>>(
-                a.out, a.in, tab, rows, (int)a.h, cpr, (int)(a.d2 / V), rpw, a.is[0], a.is[1], a.is[2], a.os[0],
-                a.os[1], a.os[2]);
+            NHP_ROPE_LAUNCH(false, 2);
         }
+#undef NHP_ROPE_LAUNCH
     } else {
         const int64_t total = a.s * a.b * a.h * a.d;
         const int64_t blocks = (total + 255) / 256;

@@ -274,3 +274,94 @@ def test_masked_full_size_properties(hotpath):
         sl = (slice(bi, bi + 1), slice(h, h + 1), slice(0, 64))
         want = oracle.softmax_bwd(dy[sl].cpu(), y[sl].cpu(), scale, causal=False)
         util.assert_softmax_bwd_close(dx[sl].cpu(), want, dy[sl].cpu(), y[sl].cpu(), scale, f"bwd {bi},{h}")
+
+
+def test_causal_llama2_7b_full_size_64bit_indexing(hotpath):
+    """[2*32, 8192, 8192] bf16 = 2^32 elements per tensor (8 GiB): element offsets
+    exceed 32 bits. Properties over the whole tensor, and the last matrices (beyond
+    2^31 elements) against torch on the GPU and the oracle on sampled rows."""
+    a, s = 64, 8192
+    scale = 1.0 / math.sqrt(128.0)
+    g = torch.Generator(device=DEV).manual_seed(5)
+    x = torch.empty((a, s, s), dtype=torch.bfloat16, device=DEV)
+    for i in range(0, a, 8):  # generate in slices to bound the fp32 temporaries
+        x[i : i + 8] = (torch.randn((8, s, s), generator=g, device=DEV) * 2).to(torch.bfloat16)
+    say("c5 forward")
+    y = util.abi_causal_fwd(hotpath, x, scale)
+    torch.cuda.synchronize()
+    for m in (0, 31, 32, 63):
+        sums = y[m].float().sum(-1)
+        assert (sums - 1).abs().max().item() < 0.05
+        assert int(y[m].view(torch.int16).triu(1).abs().max()) == 0
+        for r in (0, 511, 512, 4095, 8191):
+            ref = torch.softmax(x[m, r, : r + 1].float() * scale, -1).to(torch.bfloat16)
+            util.assert_ulp_close(y[m, r, : r + 1].cpu(), ref.cpu(), 2, f"matrix {m} row {r}")
+    rows = slice(8000, 8016)
+    want = oracle.causal_softmax_fwd(x[63:64].cpu(), scale)[0, rows]
+    util.assert_ulp_close(y[63, rows].cpu(), want, 2, "oracle rows of the last matrix")
+    say("c5 backward")
+    dy = torch.empty_like(x)
+    for i in range(0, a, 8):
+        dy[i : i + 8] = torch.randn((8, s, s), generator=g, device=DEV).to(torch.bfloat16)
+    keep = dy[63, rows].cpu()
+    dx = util.abi_causal_bwd(hotpath, dy, y, scale, inplace=True)
+    torch.cuda.synchronize()
+    for m in (0, 32, 63):
+        assert int(dx[m].view(torch.int16).triu(1).abs().max()) == 0
+        assert dx[m].float().sum(-1).abs().max().item() < 0.05
+    # rows 8000..8015 of the last matrix against the oracle (the oracle wants whole matrices: build one
+    # whose other rows are zero, which leaves these rows unchanged)
+    yc = torch.zeros((1, s, s), dtype=torch.bfloat16)
+    gc = torch.zeros((1, s, s), dtype=torch.bfloat16)
+    yc[0, rows] = y[63, rows].cpu()
+    gc[0, rows] = keep
+    want_dx = oracle.softmax_bwd(gc, yc, scale, causal=True)[0, rows]
+    util.assert_softmax_bwd_close(dx[63, rows].cpu(), want_dx, gc[0, rows], yc[0, rows], scale, "bwd rows of the last matrix")
+
+
+def test_empty_tensors_through_the_modules():
+    import scaled_masked_softmax_cuda as masked
+    import scaled_upper_triang_masked_softmax_cuda as causal
+
+    e = torch.empty((0, 64, 64), dtype=torch.bfloat16, device=DEV)
+    assert causal.forward(e, 1.0).shape == (0, 64, 64)
+    assert causal.backward(e.clone(), e, 1.0).shape == (0, 64, 64)
+    e4 = torch.empty((0, 4, 8, 64), dtype=torch.float16, device=DEV)
+    m4 = torch.empty((0, 1, 8, 64), dtype=torch.bool, device=DEV)
+    assert masked.forward(e4, m4, 1.0).shape == (0, 4, 8, 64)
+    assert masked.backward(e4.clone(), e4, 1.0).shape == (0, 4, 8, 64)
+
+
+def test_hip_graph_capture_and_replay(hotpath):
+    """The library allocates nothing and never synchronises, so its launches can be
+    captured in a HIP graph. Every replay (with eager work and synchronisation in
+    between) must give the eager result bit for bit."""
+    a, s, scale = 16, 1024, 0.125
+    x = util.randn((a, s, s), torch.bfloat16, seed=1, std=2.0).to(DEV)
+    dy = util.randn((a, s, s), torch.bfloat16, seed=2).to(DEV)
+    y = torch.empty_like(x)
+    dx = torch.empty_like(x)
+    L = hotpath.lib()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm-up on the capture stream
+        L.nhp_causal_softmax_fwd(y.data_ptr(), x.data_ptr(), scale, a, s, hotpath.BF16, side.cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        st = torch.cuda.current_stream().cuda_stream
+        assert L.nhp_causal_softmax_fwd(y.data_ptr(), x.data_ptr(), scale, a, s, hotpath.BF16, st) == 0
+        assert L.nhp_causal_softmax_bwd(dx.data_ptr(), dy.data_ptr(), y.data_ptr(), scale, a, s, hotpath.BF16, st) == 0
+    for rep in range(3):
+        x.copy_(util.randn((a, s, s), torch.bfloat16, seed=10 + rep, std=2.0).to(DEV))
+        y.fill_(7)
+        dx.fill_(7)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want_y = util.abi_causal_fwd(hotpath, x, scale)
+        want_dx = util.abi_causal_bwd(hotpath, dy, want_y, scale)
+        torch.cuda.synchronize()
+        assert torch.equal(y.view(torch.int16), want_y.view(torch.int16)), rep
+        assert torch.equal(dx.view(torch.int16), want_dx.view(torch.int16)), rep
