@@ -14,6 +14,8 @@ the drop-in extension modules (which call libneox_hotpath.so):
   masked-c3      padding-masked softmax fwd+bwd [16,32,1024,2048] fp16
   rope-c4        rotary fwd+bwd on q,k [4096,4,32,128] bf16, rotary_pct 1.0 and 0.25
   llama2-7b-c5   rotary on q,k [8192,2,32,128] + causal softmax fwd+bwd [64,8192,8192] bf16
+  mistral-window causal softmax fwd+bwd [64,8192,8192] bf16 with a 4096-key sliding window applied by index
+  alibi-1.4b     causal softmax fwd+bwd [128,2048,2048] bf16 with the AliBi bias of 16 heads added in the kernel
 
 `value` is algorithmic bytes per step / wall time per step (inputs resident in
 HBM, K steps bracketed by device synchronisation). Algorithmic bytes: softmax
@@ -142,6 +144,34 @@ def make_workload(name, torch, dev):
         cfg = {"workload": name, "scores": [a, s, s], "qk": [s, b, h, d], "rotary_dim": d2,
                "scale": "1/sqrt(%d)" % d, "bytes_convention": "causal-min (reads of the lower triangle, dense writes)"}
         return step, kernel_bytes, dense, "causal_softmax_bwd", "bf16", cfg
+
+    if name in ("mistral-window", "alibi-1.4b"):
+        from oracle import fallback_semantics as fb_
+
+        if name == "mistral-window":
+            a, s, window, heads = 64, 8192, 4096, None
+        else:
+            a, s, window, heads = 128, 2048, None, 16
+        scale = 1.0 / math.sqrt(128)
+        slopes = None if heads is None else torch.tensor(fb_.alibi_slopes(heads), dtype=torch.float32, device=dev)
+        x = torch.empty((a, s, s), dtype=torch.bfloat16, device=dev)
+        dy = torch.empty_like(x)
+        for i in range(0, a, 8):
+            x[i:i + 8] = randn((8, s, s), i, torch.bfloat16, 2.0)
+            dy[i:i + 8] = randn((8, s, s), 1000 + i, torch.bfloat16)
+        w = s if window is None else window
+        band = sum(min(q, w) + 1 for q in range(s))  # keys read per matrix
+        fwd_b = a * band * 2 + a * s * s * 2
+        bwd_b = 2 * a * band * 2 + a * s * s * 2
+        kernel_bytes = {"causal_softmax_fwd": fwd_b, "causal_softmax_bwd": bwd_b}
+
+        def step(t):
+            y = t.run("causal_softmax_fwd", lambda: causal_ext.forward(x, scale, window, slopes))
+            t.run("causal_softmax_bwd", lambda: causal_ext.backward(dy, y, scale, window))
+
+        cfg = {"workload": name, "scores": [a, s, s], "window": window, "alibi_heads": heads,
+               "bytes_convention": "reads of the attended band, dense writes"}
+        return step, kernel_bytes, {}, "causal_softmax_bwd", "bf16", cfg
 
     if name == "masked-c3":
         b, np_, sq, sk = 16, 32, 1024, 2048

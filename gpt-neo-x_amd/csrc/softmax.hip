@@ -52,19 +52,19 @@ __device__ __forceinline__ uint32_t chunk_col(int k, int w, int l)
 
 // Row softmax over the register tile z[K][8]; entries that must not take part
 // hold -inf. On return z holds the probabilities (fp32).
-// `nk`: only slots k < nk hold finite values (a wave-uniform count).
+// `act`: bit k set = slot k holds at least one finite value (wave-uniform).
 //
 // With several waves per row every wave first reduces its own part against its
 // own maximum m_w, then the (m_w, s_w) pairs are exchanged through LDS once:
 //   M = max m_w,  S = sum s_w * 2^((m_w - M) log2 e),  p = e * 2^((m_w - M) log2 e) / S
 // which needs one barrier instead of one for the maximum and one for the sum.
 template <int L, int K, int W>
-__device__ __forceinline__ void softmax_tile(float (&z)[K][8], int nk, float* lds, int wave, int lane)
+__device__ __forceinline__ void softmax_tile(float (&z)[K][8], uint32_t act, float* lds, int wave, int lane)
 {
     float m = kNegInf;
 #pragma unroll
     for (int k = 0; k < K; ++k) {
-        if (k < nk) {
+        if (act >> k & 1u) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) m = fmaxf(m, z[k][j]);
         }
@@ -74,7 +74,7 @@ __device__ __forceinline__ void softmax_tile(float (&z)[K][8], int nk, float* ld
     float sum = 0.0f;
 #pragma unroll
     for (int k = 0; k < K; ++k) {
-        if (k < nk) {
+        if (act >> k & 1u) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const float e = exp2_raw(fmaf(z[k][j] - m, kLog2e, kExpBias));
@@ -105,7 +105,7 @@ __device__ __forceinline__ void softmax_tile(float (&z)[K][8], int nk, float* ld
     }
 #pragma unroll
     for (int k = 0; k < K; ++k) {
-        if (k < nk) {
+        if (act >> k & 1u) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) z[k][j] *= inv;
         }
@@ -113,13 +113,14 @@ __device__ __forceinline__ void softmax_tile(float (&z)[K][8], int nk, float* ld
 }
 
 // Locate the row this lane works on. Rows are numbered over the whole tensor;
-// `q` is the row's index inside its [n_q, n] matrix.
+// `q` is the row's index inside its [n_q, n] matrix and `mat` that matrix.
 template <typename G>
 __device__ __forceinline__ void locate_row(uint32_t block, uint32_t rows_per_matrix, int wave, int lane,
-                                           int lanes_per_row, uint32_t& row, uint32_t& q)
+                                           int lanes_per_row, uint32_t& row, uint32_t& q, uint32_t& mat)
 {
     const uint32_t row0 = block * (uint32_t)G::kRowsPerBlock;
-    const uint32_t q0 = row0 % rows_per_matrix;  // scalar: depends on the block id only
+    mat = row0 / rows_per_matrix;  // scalar: depends on the block id only
+    const uint32_t q0 = row0 - mat * rows_per_matrix;
     uint32_t local;
     if constexpr (G::kRowsPerBlock == 1) {
         local = 0;
@@ -130,7 +131,41 @@ __device__ __forceinline__ void locate_row(uint32_t block, uint32_t rows_per_mat
     }
     row = row0 + local;
     q = q0 + local;
-    while (q >= rows_per_matrix) q -= rows_per_matrix;
+    while (q >= rows_per_matrix) {
+        q -= rows_per_matrix;
+        ++mat;
+    }
+}
+
+// The columns of row q that take part in a causal softmax: [lo, hi) with
+// hi = q + 1 and lo = max(0, q - window) (window = 0xffffffff: no lower bound).
+struct Band {
+    uint32_t lo, hi;
+};
+__device__ __forceinline__ Band causal_band(uint32_t q, uint32_t window, bool ok)
+{
+    Band b;
+    b.hi = ok ? q + 1 : 0;
+    b.lo = (ok && q > window) ? q - window : 0;
+    return b;
+}
+
+// Bit k set: register slot k of wave-slot w holds at least one column of the
+// band. Wave-uniform for full-wave rows; all K bits for rows sharing a wave.
+template <int L, int K, int W>
+__device__ __forceinline__ uint32_t active_slots(const Band& band, int w)
+{
+    if constexpr (L == 64) {
+        uint32_t act = 0;
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            const uint32_t start = (uint32_t)(k * W + w) * 512u;
+            if (start < band.hi && start + 512u > band.lo) act |= 1u << k;
+        }
+        return act;
+    } else {
+        return (1u << K) - 1u;
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -138,7 +173,8 @@ __device__ __forceinline__ void locate_row(uint32_t block, uint32_t rows_per_mat
 // ---------------------------------------------------------------------------
 template <int DT, int L, int K, int W, int BW>
 __global__ void __launch_bounds__((Geo<L, K, W, BW>::kThreads))
-causal_fwd_kernel(uint16_t* y, const uint16_t* x, float scale, uint32_t total_rows, uint32_t n)
+causal_fwd_kernel(uint16_t* y, const uint16_t* x, float scale, uint32_t total_rows, uint32_t n, uint32_t window,
+                  const float* slopes, uint32_t heads)
 {
     using G = Geo<L, K, W, BW>;
     __shared__ float lds[32];
@@ -150,65 +186,70 @@ causal_fwd_kernel(uint16_t* y, const uint16_t* x, float scale, uint32_t total_ro
     // and wave i of every workgroup sits on the same SIMD of its CU.
     const int w = (W > 1) ? (int)((wave + blockIdx.x) % W) : 0;
 
-    uint32_t row, q;
-    locate_row<G>(blockIdx.x, n, wave, lane, L, row, q);
+    uint32_t row, q, mat;
+    locate_row<G>(blockIdx.x, n, wave, lane, L, row, q, mat);
     const bool ok = row < total_rows;
-    const uint32_t valid = ok ? q + 1 : 0;  // columns [0, valid) take part
+    const Band band = causal_band(q, window, ok);  // columns [lo, hi) take part
 
     const uint16_t* xr = x + (size_t)row * n;
     uint16_t* yr = y + (size_t)row * n;
 
-    // Number of register slots that hold at least one valid column. For
-    // full-wave rows this is wave-uniform; for shared waves K == 1.
-    int nk;
-    if constexpr (G::kUniformRow) {
-        const int first = w * 512;
-        nk = ((int)valid > first) ? ((int)valid - first + W * 512 - 1) / (W * 512) : 0;
-        if (nk > K) nk = K;
-    } else {
-        nk = K;
-    }
+    const uint32_t act = active_slots<L, K, W>(band, w);
 
     u32x4 raw[K];
 #pragma unroll
     for (int k = 0; k < K; ++k) {
         const uint32_t col = chunk_col<L, W>(k, w, l);
         raw[k] = u32x4{0, 0, 0, 0};
-        if (k < nk && col < valid) raw[k] = load16_stream(xr + col);
+        if ((act >> k & 1u) && col < band.hi && col + 8 > band.lo) raw[k] = load16_stream(xr + col);
     }
+
+    // AliBi: bias[q][k] = (-(q - k)) * slope in the storage dtype, added to the
+    // score in the storage dtype (what `scores + alibi_matrix` does in eager torch)
+    float slope = 0.0f;
+    if (slopes != nullptr) slope = Half2<DT>::round(slopes[mat % heads]);
 
     float z[K][8];
 #pragma unroll
     for (int k = 0; k < K; ++k) {
-        if (k < nk) {
+        if (act >> k & 1u) {
             const uint32_t col = chunk_col<L, W>(k, w, l);
             float f[8];
             unpack8<DT>(raw[k], f);
+            if (slopes != nullptr) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float dist = Half2<DT>::round(-(float)((int)q - (int)(col + j)));
+                    f[j] = Half2<DT>::round(f[j] + Half2<DT>::round(dist * slope));
+                }
+            }
 #pragma unroll
             for (int j = 0; j < 8; ++j) z[k][j] = f[j] * scale;
-            // only the slot that straddles `valid` (or lies beyond it) needs masking
+            // only slots that straddle an end of the band need masking
             bool edge;
             if constexpr (G::kUniformRow) {
-                edge = (uint32_t)((k * W + w + 1) * 512) > valid;
+                const uint32_t start = (uint32_t)(k * W + w) * 512u;
+                edge = start + 512u > band.hi || start < band.lo;
             } else {
                 edge = true;
             }
             if (edge) {
 #pragma unroll
-                for (int j = 0; j < 8; ++j) z[k][j] = (col + j < valid) ? z[k][j] : kNegInf;
+                for (int j = 0; j < 8; ++j)
+                    z[k][j] = (col + j < band.hi && col + j >= band.lo) ? z[k][j] : kNegInf;
             }
         }
     }
 
-    softmax_tile<L, K, W>(z, nk, lds, wave, lane);
+    softmax_tile<L, K, W>(z, act, lds, wave, lane);
 
-    // The whole row is written in one go, zeros above the diagonal included:
+    // The whole row is written in one go, zeros outside the band included:
     // splitting a row's stores in time costs DRAM efficiency.
 #pragma unroll
     for (int k = 0; k < K; ++k) {
         const uint32_t col = chunk_col<L, W>(k, w, l);
         if (ok && col < n) {
-            if (k < nk && col < valid) {
+            if ((act >> k & 1u) && col < band.hi && col + 8 > band.lo) {
                 store16_stream(yr + col, pack8<DT>(z[k]));
             } else {
                 store16_stream(yr + col, u32x4{0, 0, 0, 0});
@@ -360,7 +401,7 @@ masked_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
 template <int DT, int L, int K, int W, int BW, bool CAUSAL>
 __global__ void __launch_bounds__((Geo<L, K, W, BW>::kThreads))
 softmax_bwd_kernel(uint16_t* dx, const uint16_t* dy, const uint16_t* y, float scale,
-                   uint32_t total_rows, uint32_t n, uint32_t rows_per_matrix)
+                   uint32_t total_rows, uint32_t n, uint32_t rows_per_matrix, uint32_t window)
 {
     using G = Geo<L, K, W, BW>;
     __shared__ float lds[32];
@@ -370,21 +411,19 @@ softmax_bwd_kernel(uint16_t* dx, const uint16_t* dy, const uint16_t* y, float sc
     // rotate the segment sets over the waves as in the forward kernel
     const int w = (W > 1) ? (int)((wave + (CAUSAL ? blockIdx.x : 0u)) % W) : 0;
 
-    uint32_t row, q;
-    locate_row<G>(blockIdx.x, rows_per_matrix, wave, lane, L, row, q);
+    uint32_t row, q, mat;
+    locate_row<G>(blockIdx.x, rows_per_matrix, wave, lane, L, row, q, mat);
     const bool ok = row < total_rows;
-    const uint32_t valid = ok ? (CAUSAL ? q + 1 : n) : 0;
+    Band band;
+    if constexpr (CAUSAL) {
+        band = causal_band(q, window, ok);
+    } else {
+        band.lo = 0;
+        band.hi = ok ? n : 0;
+    }
 
     const size_t base = (size_t)row * n;
-
-    int nk;
-    if constexpr (G::kUniformRow) {
-        const int first = w * 512;
-        nk = ((int)valid > first) ? ((int)valid - first + W * 512 - 1) / (W * 512) : 0;
-        if (nk > K) nk = K;
-    } else {
-        nk = K;
-    }
+    const uint32_t act = active_slots<L, K, W>(band, w);
 
     u32x4 rg[K], ry[K];
 #pragma unroll
@@ -392,16 +431,18 @@ softmax_bwd_kernel(uint16_t* dx, const uint16_t* dy, const uint16_t* y, float sc
         const uint32_t col = chunk_col<L, W>(k, w, l);
         rg[k] = u32x4{0, 0, 0, 0};
         ry[k] = u32x4{0, 0, 0, 0};
-        if (k < nk && col < valid) {
+        if ((act >> k & 1u) && col < band.hi && col + 8 > band.lo) {
             rg[k] = load16_stream(dy + base + col);
             ry[k] = load16_stream(y + base + col);
-            if (CAUSAL && col + 8 > valid) {
-                // zero the elements at and beyond `valid` (both operands)
-                const uint32_t rem = valid - col;  // 1..7
+            if (CAUSAL && (col + 8 > band.hi || col < band.lo)) {
+                // zero the elements outside the band (both operands): keep [a, b) of the chunk
+                const uint32_t b_end = (band.hi - col < 8u) ? band.hi - col : 8u;
+                const uint32_t a_beg = (band.lo > col) ? band.lo - col : 0u;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const uint32_t keep = (rem >= 2u * i + 2u) ? 0xffffffffu
-                                          : (rem == 2u * i + 1u) ? 0x0000ffffu : 0u;
+                    const uint32_t e0 = 2u * i, e1 = 2u * i + 1u;
+                    const uint32_t keep = ((e0 >= a_beg && e0 < b_end) ? 0x0000ffffu : 0u) |
+                                          ((e1 >= a_beg && e1 < b_end) ? 0xffff0000u : 0u);
                     rg[k][i] &= keep;
                     ry[k][i] &= keep;
                 }
@@ -412,7 +453,7 @@ softmax_bwd_kernel(uint16_t* dx, const uint16_t* dy, const uint16_t* y, float sc
     float s = 0.0f;
 #pragma unroll
     for (int k = 0; k < K; ++k) {
-        if (k < nk) {
+        if (act >> k & 1u) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 s = fmaf(Half2<DT>::lo(rg[k][i]), Half2<DT>::lo(ry[k][i]), s);
@@ -423,7 +464,7 @@ softmax_bwd_kernel(uint16_t* dx, const uint16_t* dy, const uint16_t* y, float sc
     s = group_reduce<OpSum, L>(s);
     s = block_combine<OpSum, W>(s, lds, wave, lane);
 
-    // what the formula gives where dy = y = 0 (masked columns): +0 for finite s and scale > 0
+    // what the formula gives where dy = y = 0 (masked columns): +0 for finite s and scale >= 0
     const float zv = scale * fmaf(-0.0f, s, 0.0f);
     const uint32_t zw = Half2<DT>::pack(zv, zv);
 
@@ -433,7 +474,7 @@ softmax_bwd_kernel(uint16_t* dx, const uint16_t* dy, const uint16_t* y, float sc
         const uint32_t col = chunk_col<L, W>(k, w, l);
         if (ok && col < n) {
             u32x4 o;
-            if (k < nk && col < valid) {
+            if ((act >> k & 1u) && col < band.hi && col + 8 > band.lo) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const float g0 = Half2<DT>::lo(rg[k][i]), y0 = Half2<DT>::lo(ry[k][i]);
@@ -469,11 +510,12 @@ __device__ __forceinline__ float block_reduce_256(float v, float* slots)
     return Op::apply(Op::apply(slots[0], slots[1]), Op::apply(slots[2], slots[3]));
 }
 
-// MODE 0: causal, MODE 1: padding mask
+// MODE 0: causal (optional sliding window and AliBi), MODE 1: padding mask
 template <int DT, int MODE>
 __global__ void __launch_bounds__(kScalarThreads)
 scalar_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float scale,
-                  uint64_t n, uint64_t sq, uint64_t np, int mask_per_batch)
+                  uint64_t n, uint64_t sq, uint64_t np, int mask_per_batch, uint32_t window,
+                  const float* slopes, uint32_t heads)
 {
     __shared__ float slots[4];
     const uint64_t row = blockIdx.x;
@@ -481,64 +523,69 @@ scalar_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
     const uint16_t* xr = x + row * n;
     uint16_t* yr = y + row * n;
     const uint8_t* mrow = nullptr;
-    uint64_t valid = n;
+    uint64_t lo = 0, hi = n;
+    float slope = 0.0f;
     if (MODE == 0) {
-        valid = q + 1;
+        hi = q + 1;
+        lo = (q > window) ? q - window : 0;
+        if (slopes != nullptr) slope = Half2<DT>::round(slopes[(row / sq) % heads]);
     } else {
         const uint64_t bi = row / (sq * np);
         mrow = mask + (mask_per_batch ? (bi * sq + q) : q) * n;
     }
+    // scaled logit of column c (lo <= c < hi)
+    auto logit = [&](uint64_t c) {
+        float f = Half2<DT>::from_bits(xr[c]);
+        if (MODE == 0 && slopes != nullptr) {
+            const float dist = Half2<DT>::round(-(float)((int64_t)q - (int64_t)c));
+            f = Half2<DT>::round(f + Half2<DT>::round(dist * slope));
+        }
+        float z = f * scale;
+        if (MODE == 1 && mrow[c] == 1) z = kMaskFill;
+        return z;
+    };
 
     float m = kNegInf;
-    for (uint64_t c = threadIdx.x; c < valid; c += kScalarThreads) {
-        float z = Half2<DT>::from_bits(xr[c]) * scale;
-        if (MODE == 1 && mrow[c] == 1) z = kMaskFill;
-        m = fmaxf(m, z);
-    }
+    for (uint64_t c = lo + threadIdx.x; c < hi; c += kScalarThreads) m = fmaxf(m, logit(c));
     m = block_reduce_256<OpMax>(m, slots);
 
     float sum = 0.0f;
-    for (uint64_t c = threadIdx.x; c < valid; c += kScalarThreads) {
-        float z = Half2<DT>::from_bits(xr[c]) * scale;
-        if (MODE == 1 && mrow[c] == 1) z = kMaskFill;
-        sum += exp2_raw(fmaf(z - m, kLog2e, kExpBias));
-    }
+    for (uint64_t c = lo + threadIdx.x; c < hi; c += kScalarThreads)
+        sum += exp2_raw(fmaf(logit(c) - m, kLog2e, kExpBias));
     sum = block_reduce_256<OpSum>(sum, slots);
     const float inv = 1.0f / sum;
 
-    // all reads of x are done before the first write of y (y may alias x)
-    for (uint64_t c0 = 0; c0 < n; c0 += kScalarThreads) {
-        const uint64_t c = c0 + threadIdx.x;
+    // every thread reads and then writes the columns it owns, after the last
+    // reduction barrier: y may alias x
+    for (uint64_t c = threadIdx.x; c < n; c += kScalarThreads) {
         float p = 0.0f;
-        if (c < valid) {
-            float z = Half2<DT>::from_bits(xr[c]) * scale;
-            if (MODE == 1 && mrow[c] == 1) z = kMaskFill;
-            p = exp2_raw(fmaf(z - m, kLog2e, kExpBias)) * inv;
-        }
-        if (c < n) yr[c] = Half2<DT>::to_bits(p);
+        if (c >= lo && c < hi) p = exp2_raw(fmaf(logit(c) - m, kLog2e, kExpBias)) * inv;
+        yr[c] = Half2<DT>::to_bits(p);
     }
 }
 
 template <int DT, bool CAUSAL>
 __global__ void __launch_bounds__(kScalarThreads)
 scalar_bwd_kernel(uint16_t* dx, const uint16_t* dy, const uint16_t* y, float scale,
-                  uint64_t n, uint64_t rows_per_matrix)
+                  uint64_t n, uint64_t rows_per_matrix, uint32_t window)
 {
     __shared__ float slots[4];
     const uint64_t row = blockIdx.x;
-    const uint64_t valid = CAUSAL ? (row % rows_per_matrix) + 1 : n;
+    const uint64_t q = row % rows_per_matrix;
+    const uint64_t hi = CAUSAL ? q + 1 : n;
+    const uint64_t lo = (CAUSAL && q > window) ? q - window : 0;
     const uint16_t* gr = dy + row * n;
     const uint16_t* yr = y + row * n;
     uint16_t* dr = dx + row * n;
 
     float s = 0.0f;
-    for (uint64_t c = threadIdx.x; c < valid; c += kScalarThreads)
+    for (uint64_t c = lo + threadIdx.x; c < hi; c += kScalarThreads)
         s = fmaf(Half2<DT>::from_bits(gr[c]), Half2<DT>::from_bits(yr[c]), s);
     s = block_reduce_256<OpSum>(s, slots);
 
     for (uint64_t c = threadIdx.x; c < n; c += kScalarThreads) {
         float g = 0.0f, p = 0.0f;
-        if (c < valid) {
+        if (c >= lo && c < hi) {
             g = Half2<DT>::from_bits(gr[c]);
             p = Half2<DT>::from_bits(yr[c]);
         }
@@ -648,9 +695,11 @@ static inline int launch_status()
 }
 
 constexpr int64_t kMaxRows = (int64_t)1 << 31;  // row and block ids are 32-bit on the device
+constexpr uint32_t kNoWindow = 0xffffffffu;
 
 template <int DT>
-static int causal_fwd(void* y, const void* x, float scale, int64_t batches, int64_t n, hipStream_t st)
+static int causal_fwd(void* y, const void* x, float scale, int64_t batches, int64_t n, uint32_t window,
+                      const float* slopes, uint32_t heads, hipStream_t st)
 {
     const int64_t rows = batches * n;
     RowPlan p;
@@ -662,20 +711,20 @@ static int causal_fwd(void* y, const void* x, float scale, int64_t batches, int6
         using G = Geo<L_, K_, W_, kBlockWaves>;                                            \
         const uint32_t blocks = (uint32_t)((rows + G::kRowsPerBlock - 1) / G::kRowsPerBlock); \
         causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves><<<blocks, G::kThreads, p.lds, st>>>(    \
-            yp, xp, scale, (uint32_t)rows, (uint32_t)n);                                   \
+            yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, slopes, heads);            \
     }
         NHP_FOR_PLAN(p);
 #undef CALL
     } else {
         scalar_fwd_kernel<DT, 0><<<(uint32_t)rows, kScalarThreads, 0, st>>>(
-            yp, xp, nullptr, scale, (uint64_t)n, (uint64_t)n, 1, 0);
+            yp, xp, nullptr, scale, (uint64_t)n, (uint64_t)n, 1, 0, window, slopes, heads);
     }
     return launch_status();
 }
 
 template <int DT, bool CAUSAL>
 static int softmax_bwd(void* dx, const void* dy, const void* y, float scale, int64_t rows, int64_t n,
-                       int64_t rows_per_matrix, hipStream_t st)
+                       int64_t rows_per_matrix, uint32_t window, hipStream_t st)
 {
     RowPlan p;
     uint16_t* dxp = static_cast<uint16_t*>(dx);
@@ -687,13 +736,13 @@ static int softmax_bwd(void* dx, const void* dy, const void* y, float scale, int
         using G = Geo<L_, K_, W_, kBlockWaves>;                                            \
         const uint32_t blocks = (uint32_t)((rows + G::kRowsPerBlock - 1) / G::kRowsPerBlock); \
         softmax_bwd_kernel<DT, L_, K_, W_, kBlockWaves, CAUSAL><<<blocks, G::kThreads, p.lds, st>>>( \
-            dxp, dyp, yp, scale, (uint32_t)rows, (uint32_t)n, (uint32_t)rows_per_matrix);  \
+            dxp, dyp, yp, scale, (uint32_t)rows, (uint32_t)n, (uint32_t)rows_per_matrix, window); \
     }
         NHP_FOR_PLAN(p);
 #undef CALL
     } else {
         scalar_bwd_kernel<DT, CAUSAL><<<(uint32_t)rows, kScalarThreads, 0, st>>>(
-            dxp, dyp, yp, scale, (uint64_t)n, (uint64_t)rows_per_matrix);
+            dxp, dyp, yp, scale, (uint64_t)n, (uint64_t)rows_per_matrix, window);
     }
     return launch_status();
 }
@@ -731,7 +780,7 @@ static int masked_fwd(void* y, const void* x, const uint8_t* mask, float scale, 
 #undef CALL
     } else {
         scalar_fwd_kernel<DT, 1><<<(uint32_t)(b * np * sq), kScalarThreads, 0, st>>>(
-            yp, xp, mask, scale, (uint64_t)n, (uint64_t)sq, (uint64_t)np, per_batch);
+            yp, xp, mask, scale, (uint64_t)n, (uint64_t)sq, (uint64_t)np, per_batch, kNoWindow, nullptr, 1);
     }
     return launch_status();
 }
@@ -744,21 +793,31 @@ extern "C" {
 
 int64_t nhp_softmax_max_resident_row(void) { return kMaxResidentRow; }
 
-int nhp_causal_softmax_fwd(void* y, const void* x, float scale, int64_t attn_batches, int64_t seq_len,
-                           int dtype, void* stream)
+int nhp_causal_softmax_ex_fwd(void* y, const void* x, float scale, int64_t attn_batches, int64_t seq_len,
+                              int64_t window, const float* alibi_slopes, int64_t heads, int dtype, void* stream)
 {
     if (dtype != NHP_F16 && dtype != NHP_BF16) return NHP_ERR_DTYPE;
     if (attn_batches < 0 || seq_len < 0) return NHP_ERR_SHAPE;
+    if (alibi_slopes != nullptr && (heads < 1 || attn_batches % heads != 0)) return NHP_ERR_SHAPE;
     if (attn_batches == 0 || seq_len == 0) return NHP_OK;
     if (attn_batches > kMaxRows / seq_len - 1) return NHP_ERR_SHAPE;
     if (!x || !y) return NHP_ERR_NULL;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    return dtype == NHP_BF16 ? causal_fwd<NHP_BF16>(y, x, scale, attn_batches, seq_len, st)
-                             : causal_fwd<NHP_F16>(y, x, scale, attn_batches, seq_len, st);
+    const uint32_t win = (window < 0 || window >= seq_len) ? kNoWindow : (uint32_t)window;
+    const uint32_t hd = alibi_slopes ? (uint32_t)heads : 1u;
+    return dtype == NHP_BF16
+               ? causal_fwd<NHP_BF16>(y, x, scale, attn_batches, seq_len, win, alibi_slopes, hd, st)
+               : causal_fwd<NHP_F16>(y, x, scale, attn_batches, seq_len, win, alibi_slopes, hd, st);
 }
 
-int nhp_causal_softmax_bwd(void* dx, const void* dy, const void* y, float scale, int64_t attn_batches,
-                           int64_t seq_len, int dtype, void* stream)
+int nhp_causal_softmax_fwd(void* y, const void* x, float scale, int64_t attn_batches, int64_t seq_len,
+                           int dtype, void* stream)
+{
+    return nhp_causal_softmax_ex_fwd(y, x, scale, attn_batches, seq_len, -1, nullptr, 1, dtype, stream);
+}
+
+int nhp_causal_softmax_ex_bwd(void* dx, const void* dy, const void* y, float scale, int64_t attn_batches,
+                              int64_t seq_len, int64_t window, int dtype, void* stream)
 {
     if (dtype != NHP_F16 && dtype != NHP_BF16) return NHP_ERR_DTYPE;
     if (attn_batches < 0 || seq_len < 0) return NHP_ERR_SHAPE;
@@ -768,9 +827,16 @@ int nhp_causal_softmax_bwd(void* dx, const void* dy, const void* y, float scale,
     if (dx == y) return NHP_ERR_ALIAS;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int64_t rows = attn_batches * seq_len;
+    const uint32_t win = (window < 0 || window >= seq_len) ? kNoWindow : (uint32_t)window;
     return dtype == NHP_BF16
-               ? softmax_bwd<NHP_BF16, true>(dx, dy, y, scale, rows, seq_len, seq_len, st)
-               : softmax_bwd<NHP_F16, true>(dx, dy, y, scale, rows, seq_len, seq_len, st);
+               ? softmax_bwd<NHP_BF16, true>(dx, dy, y, scale, rows, seq_len, seq_len, win, st)
+               : softmax_bwd<NHP_F16, true>(dx, dy, y, scale, rows, seq_len, seq_len, win, st);
+}
+
+int nhp_causal_softmax_bwd(void* dx, const void* dy, const void* y, float scale, int64_t attn_batches,
+                           int64_t seq_len, int dtype, void* stream)
+{
+    return nhp_causal_softmax_ex_bwd(dx, dy, y, scale, attn_batches, seq_len, -1, dtype, stream);
 }
 
 int nhp_masked_softmax_fwd(void* y, const void* x, const uint8_t* mask, float scale, int64_t b,
@@ -799,8 +865,8 @@ int nhp_masked_softmax_bwd(void* dx, const void* dy, const void* y, float scale,
     if (dx == y) return NHP_ERR_ALIAS;
     hipStream_t st = static_cast<hipStream_t>(stream);
     // rows_per_matrix only matters for the causal variant; any non-zero value works here
-    return dtype == NHP_BF16 ? softmax_bwd<NHP_BF16, false>(dx, dy, y, scale, rows, sk, rows, st)
-                             : softmax_bwd<NHP_F16, false>(dx, dy, y, scale, rows, sk, rows, st);
+    return dtype == NHP_BF16 ? softmax_bwd<NHP_BF16, false>(dx, dy, y, scale, rows, sk, rows, kNoWindow, st)
+                             : softmax_bwd<NHP_F16, false>(dx, dy, y, scale, rows, sk, rows, kNoWindow, st);
 }
 
 int nhp_softmax_batch_per_block(int64_t query_seq_len, int64_t key_seq_len, int64_t batches,

@@ -9,7 +9,13 @@ reference uses. Differences from the reference, all widening:
   * the fused path takes key lengths above 2048 (the kernels keep rows of up
     to 65536 keys in registers, longer ones stream);
   * ``scale`` reaches the forward kernel as an fp32 value; the reference's CUDA
-    dispatcher first narrows it to the input dtype.
+    dispatcher first narrows it to the input dtype;
+  * two optional constructor arguments of ``FusedScaleMaskSoftmax`` let the
+    causal kernel do by index what its caller otherwise does with tensors:
+    ``sliding_window_width`` (the reference's causal kernel ignores the mask
+    contents and so drops a sliding window) and ``alibi_slopes`` (the AliBi
+    bias is added inside the kernel instead of by a separate
+    ``scores + alibi_matrix`` pass). Both default to off.
 """
 import enum
 
@@ -24,12 +30,13 @@ class ScaledUpperTriangMaskedSoftmax(torch.autograd.Function):
     [attn_batches, sq, sk] tensor, fused into one kernel each way."""
 
     @staticmethod
-    def forward(ctx, inputs, scale):
+    def forward(ctx, inputs, scale, window=None, alibi_slopes=None):
         import scaled_upper_triang_masked_softmax_cuda as ext
 
         scale_t = torch.tensor([scale])
-        probs = ext.forward(inputs, scale_t[0])
+        probs = ext.forward(inputs, scale_t[0], window, alibi_slopes)
         ctx.save_for_backward(probs, scale_t)
+        ctx.window = window
         return probs
 
     @staticmethod
@@ -37,7 +44,7 @@ class ScaledUpperTriangMaskedSoftmax(torch.autograd.Function):
         import scaled_upper_triang_masked_softmax_cuda as ext
 
         probs, scale_t = ctx.saved_tensors
-        return ext.backward(output_grads, probs, scale_t[0]), None
+        return ext.backward(output_grads, probs, scale_t[0], ctx.window), None, None, None
 
 
 class ScaledMaskedSoftmax(torch.autograd.Function):
@@ -78,9 +85,16 @@ class FusedScaleMaskSoftmax(nn.Module):
         mask_func: ``mask_func(scores, mask)`` used by the torch path.
         softmax_in_fp32: compute the torch path in fp32.
         scale: factor applied to the scores before the softmax, or None.
+        sliding_window_width: (extension) with upper_triang fusion, restrict row q
+            to keys q-width..q inside the kernel. The mask handed to ``forward``
+            must then be the sliding-window mask, which the torch path uses.
+        alibi_slopes: (extension) fp32 tensor [np]; with upper_triang fusion the
+            AliBi bias is added inside the kernel, and by the torch path with the
+            same roundings, so the caller must not add it itself.
     """
 
-    def __init__(self, input_in_fp16, input_in_bf16, fusion_type, mask_func, softmax_in_fp32, scale):
+    def __init__(self, input_in_fp16, input_in_bf16, fusion_type, mask_func, softmax_in_fp32, scale,
+                 sliding_window_width=None, alibi_slopes=None):
         super().__init__()
         self.input_in_fp16 = input_in_fp16
         self.input_in_bf16 = input_in_bf16
@@ -98,6 +112,12 @@ class FusedScaleMaskSoftmax(nn.Module):
         self.softmax_in_fp32 = softmax_in_fp32
         self.scale = scale
         assert self.scale is None or softmax_in_fp32, "softmax should be in fp32 when scaled"
+
+        self.sliding_window_width = sliding_window_width
+        if alibi_slopes is not None:
+            self.register_buffer("alibi_slopes", alibi_slopes.detach().float().clone(), persistent=False)
+        else:
+            self.alibi_slopes = None
 
     def forward(self, input, mask):
         assert input.dim() == 4  # [b, np, sq, sk]
@@ -124,11 +144,29 @@ class FusedScaleMaskSoftmax(nn.Module):
         if self.upper_triang_mask_fusion:
             assert sq == sk, "causal mask is only for self attention"
             # the causal kernel works on [attn_batches, sq, sk]; the mask is implied
-            probs = ScaledUpperTriangMaskedSoftmax.apply(input.view(-1, sq, sk), scale)
+            slopes = self.alibi_slopes
+            if slopes is not None and slopes.device != input.device:
+                slopes = slopes.to(input.device)
+            probs = ScaledUpperTriangMaskedSoftmax.apply(
+                input.view(-1, sq, sk), scale, self.sliding_window_width, slopes)
             return probs.view(b, np, sq, sk)
+        if self.alibi_slopes is not None:
+            input = self._add_alibi(input)
         return ScaledMaskedSoftmax.apply(input, mask, scale)
 
+    def _add_alibi(self, scores):
+        """scores + AliBi matrix in the scores' dtype, for sq == sk (the arithmetic of
+        megatron/model/positional_embeddings.py:219-257)."""
+        s = scores.shape[-1]
+        assert scores.shape[-2] == s, "in-module AliBi needs sq == sk"
+        i = torch.arange(s, device=scores.device)
+        a = -torch.tril(i.view(s, 1) - i.view(1, s)).to(scores.dtype)
+        slopes = self.alibi_slopes.to(scores.device).to(scores.dtype)
+        return scores + a * slopes.view(-1, 1, 1)
+
     def forward_torch_softmax(self, input, mask):
+        if self.alibi_slopes is not None:
+            input = self._add_alibi(input)
         upcast = self.input_in_float16 and self.softmax_in_fp32
         if upcast:
             input = input.float()

@@ -1,9 +1,10 @@
-"""Rotary cache and the eager (unfused) rotary functions, with the public
-surface of the rotary part of GPT-NeoX's
-``megatron/model/positional_embeddings.py`` (RotaryEmbedding :38-97,
-rotate_half :103-107, apply_rotary_pos_emb :110-116,
-apply_rotary_pos_emb_torch :119-126).
+"""Rotary cache, the eager (unfused) rotary functions and the AliBi slopes, with
+the public surface of GPT-NeoX's ``megatron/model/positional_embeddings.py``
+(RotaryEmbedding :38-97, rotate_half :103-107, apply_rotary_pos_emb :110-116,
+apply_rotary_pos_emb_torch :119-126, AliBi :129-257).
 """
+import math
+
 import torch
 
 
@@ -84,3 +85,64 @@ def apply_rotary_pos_emb_torch(q, k, cos, sin, offset: int = 0):
     # identical to apply_rotary_pos_emb; the reference keeps two names because
     # its first variant is TorchScript-compiled and that fails for bf16
     return apply_rotary_pos_emb(q, k, cos, sin, offset)
+
+
+class AliBi(torch.nn.Module):
+    """Attention with linear biases: head h adds -(q - k) * slope_h to the score of
+    query q and key k <= q.
+
+    Same constructor, ``slopes`` buffer, ``bias`` and ``forward`` as the reference
+    class. ``forward(x)`` is the eager path (one extra pass over the scores);
+    handing ``alibi.slopes`` to ``FusedScaleMaskSoftmax(alibi_slopes=...)`` adds
+    the same bias inside the causal softmax kernel instead.
+    """
+
+    def __init__(self, num_heads, mp_size=1, mp_rank=1):
+        super().__init__()
+        # heads are split across model-parallel ranks: each rank keeps its slice of the slopes
+        assert mp_size <= num_heads and mp_rank <= mp_size
+        self.mp_size = mp_size
+        self.mp_rank = mp_rank
+        self.num_heads = num_heads
+        self.slice_size = num_heads // mp_size
+        self.cached_matrix = None
+        self.cached_seq_len = None
+        slopes = torch.Tensor(self._get_slopes(num_heads))[mp_rank * self.slice_size : (mp_rank + 1) * self.slice_size]
+        self.register_buffer("slopes", slopes)
+
+    def _get_slopes(self, n):
+        """Geometric sequence 2^(-8/n), 2^(-16/n), ... for a power-of-two n; other n
+        take the sequence of the next lower power of two plus every other slope of
+        the next higher one."""
+
+        def power_of_2(m):
+            start = 2 ** (-(2 ** -(math.log2(m) - 3)))
+            return [start * start**i for i in range(m)]
+
+        if math.log2(n).is_integer():
+            return power_of_2(n)
+        closest = 2 ** math.floor(math.log2(n))
+        return power_of_2(closest) + self._get_slopes(2 * closest)[0::2][: n - closest]
+
+    def bias(self, seq_len_q, seq_len_k, device, dtype):
+        """The [np, sq, sk] bias matrix (cached; it grows fourfold when a longer key length shows up)."""
+        if self.cached_seq_len is None or self.cached_seq_len < seq_len_k:
+            target = seq_len_k if self.cached_seq_len is None else self.cached_seq_len * 4
+            i = torch.arange(target)
+            a = -torch.tril(i.view(target, 1).repeat(1, target) + torch.arange(0, -target, -1))
+            a = a.to(device).to(dtype)
+            slopes = self.slopes.to(a.device).to(a.dtype)
+            self.cached_matrix = a * slopes.view(self.slopes.shape[0], 1, 1)
+            self.cached_seq_len = target
+        a = self.cached_matrix
+        if self.cached_seq_len > seq_len_k:
+            a = a[:, :seq_len_k, :seq_len_k]
+        if seq_len_q != seq_len_k:
+            # decoding with a key/value cache: one query, the last position
+            assert seq_len_q == 1, "assumption sq == sk unless at inference time with cache in layer_past with sq == 1"
+            a = a[:, seq_len_k - 1, :].view(a.shape[0], 1, a.shape[2])
+        return a
+
+    def forward(self, x):
+        # x: [b, np, sq, sk]
+        return x + self.bias(x.shape[-2], x.shape[-1], x.device, x.dtype)

@@ -11,12 +11,18 @@ from megatron.fused_kernels import _hotpath as _hp
 _HALF = (torch.float16, torch.bfloat16)
 
 
-def forward(input, scale_factor):
+def forward(input, scale_factor, window=None, alibi_slopes=None):
     """softmax(scale * input) under an upper-triangular mask.
 
     input: [attn_batches, seq_len, seq_len] fp16/bf16 on the GPU. Returns a new
     tensor of the same shape and dtype (requires_grad False). Checks follow
     scaled_upper_triang_masked_softmax.cpp:31-39; seq_len is not limited to 2048.
+
+    Two optional arguments go beyond the reference function:
+    window: sliding-window width; row q attends to keys q-window..q only.
+    alibi_slopes: fp32 tensor [heads] on the GPU (attn_batches % heads == 0);
+        the AliBi bias -(q-k)*slope is added to the scores in the storage dtype
+        before the softmax, as `scores + alibi_matrix` would.
     """
     if input.dim() != 3:
         raise RuntimeError("expected 3D tensor")
@@ -27,16 +33,25 @@ def forward(input, scale_factor):
     _hp.require_gpu(input, "scaled_upper_triang_masked_softmax_cuda.forward")
     x = input.contiguous()
     y = torch.empty_like(x)
+    slopes_ptr, heads = None, 1
+    if alibi_slopes is not None:
+        if alibi_slopes.dtype != torch.float32 or alibi_slopes.dim() != 1:
+            raise RuntimeError("alibi_slopes must be a 1-D float32 tensor")
+        _hp.require_gpu(alibi_slopes, "scaled_upper_triang_masked_softmax_cuda.forward")
+        alibi_slopes = alibi_slopes.contiguous()
+        slopes_ptr, heads = alibi_slopes.data_ptr(), alibi_slopes.numel()
+        if heads == 0 or x.size(0) % heads != 0:
+            raise RuntimeError("attn_batches must be a multiple of the number of AliBi slopes")
     with _hp.device_guard(x):
-        rc = _hp.lib().nhp_causal_softmax_fwd(
-            y.data_ptr(), x.data_ptr(), float(scale_factor), x.size(0), x.size(1), _hp.dtype_code(x, "forward"),
-            _hp.stream_of(x))
+        rc = _hp.lib().nhp_causal_softmax_ex_fwd(
+            y.data_ptr(), x.data_ptr(), float(scale_factor), x.size(0), x.size(1),
+            -1 if window is None else int(window), slopes_ptr, heads, _hp.dtype_code(x, "forward"), _hp.stream_of(x))
     _hp.check(rc, "scaled_upper_triang_masked_softmax_cuda.forward")
     return y
 
 
-def backward(output_grads, softmax_results, scale_factor):
-    """Gradient w.r.t. the input of ``forward``.
+def backward(output_grads, softmax_results, scale_factor, window=None):
+    """Gradient w.r.t. the input of ``forward`` (pass the same ``window``; AliBi needs nothing here).
 
     Works in place: the result is written into (the contiguous version of)
     ``output_grads`` and that tensor is returned, as in
@@ -55,8 +70,8 @@ def backward(output_grads, softmax_results, scale_factor):
     g = output_grads.detach().contiguous()
     y = softmax_results.detach().contiguous()
     with _hp.device_guard(g):
-        rc = _hp.lib().nhp_causal_softmax_bwd(
+        rc = _hp.lib().nhp_causal_softmax_ex_bwd(
             g.data_ptr(), g.data_ptr(), y.data_ptr(), float(scale_factor), g.size(0), g.size(1),
-            _hp.dtype_code(g, "backward"), _hp.stream_of(g))
+            -1 if window is None else int(window), _hp.dtype_code(g, "backward"), _hp.stream_of(g))
     _hp.check(rc, "scaled_upper_triang_masked_softmax_cuda.backward")
     return g

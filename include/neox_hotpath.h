@@ -90,6 +90,39 @@ int nhp_causal_softmax_bwd(void* dx, const void* dy, const void* y, float scale,
                            int64_t attn_batches, int64_t seq_len,
                            int dtype, void* stream);
 
+/*
+ * Causal softmax with the two index-only generalisations its caller needs, so
+ * that neither a mask tensor nor a bias tensor has to be read or written:
+ *
+ *  window >= 0: sliding-window attention. Row q attends to columns
+ *      max(0, q - window) <= k <= q (the mask megatron/utils.py:67-80 builds
+ *      with sliding_window_width = window); everything else is +0 and is never
+ *      read. window < 0 (or >= seq_len): plain causal.
+ *  alibi_slopes != NULL: AliBi. The score of head hd = a % heads (a = index
+ *      along attn_batches, i.e. x is a [b, heads, s, s] tensor) becomes
+ *      x (+) ( dt(-(q - k)) (*) dt(slopes[hd]) ), every operation rounded to
+ *      the storage dtype, which is what `scores + alibi_matrix` computes in
+ *      eager torch (megatron/model/positional_embeddings.py:129-257, applied
+ *      at megatron/model/transformer.py:584-585) before the softmax sees the
+ *      scores. slopes: `heads` fp32 values on the device.
+ *
+ * The backward of the AliBi variant is the plain (windowed) backward: the bias
+ * is constant.
+ *
+ * Extends scaled_upper_triang_masked_softmax_cuda.forward / backward
+ * (megatron/fused_kernels/scaled_upper_triang_masked_softmax.cpp:31-56), whose
+ * kernel ignores the mask contents and therefore drops a sliding window
+ * (megatron/model/fused_softmax.py:148-179).
+ */
+int nhp_causal_softmax_ex_fwd(void* y, const void* x, float scale,
+                              int64_t attn_batches, int64_t seq_len,
+                              int64_t window, const float* alibi_slopes, int64_t heads,
+                              int dtype, void* stream);
+
+int nhp_causal_softmax_ex_bwd(void* dx, const void* dy, const void* y, float scale,
+                              int64_t attn_batches, int64_t seq_len, int64_t window,
+                              int dtype, void* stream);
+
 /* ------------------------------------------------------------------------
  * Scaled padding-masked softmax
  * ---------------------------------------------------------------------- */

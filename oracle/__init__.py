@@ -45,6 +45,8 @@ def lib():
         L = ctypes.CDLL(_LIB_PATH)
         i64, vp, f32, ci = ctypes.c_int64, ctypes.c_void_p, ctypes.c_float, ctypes.c_int
         L.oracle_causal_softmax_fwd.argtypes = [vp, vp, f32, i64, i64, ci]
+        L.oracle_causal_softmax_ex_fwd.argtypes = [vp, vp, f32, i64, i64, i64, vp, i64, ci]
+        L.oracle_softmax_ex_bwd.argtypes = [vp, vp, vp, f32, i64, i64, i64, ci, i64, ci]
         L.oracle_masked_softmax_fwd.argtypes = [vp, vp, vp, f32, i64, i64, i64, i64, i64, ci]
         L.oracle_softmax_bwd.argtypes = [vp, vp, vp, f32, i64, i64, i64, ci, ci]
         L.oracle_batch_per_block.argtypes = [i64, ci]
@@ -73,13 +75,20 @@ def _cpu_contig(t):
     return t.contiguous()
 
 
-def causal_softmax_fwd(x, scale):
-    """x: [attn_batches, s, s] fp16/bf16 -> probabilities, same shape and dtype."""
+def causal_softmax_fwd(x, scale, window=None, alibi_slopes=None):
+    """x: [attn_batches, s, s] fp16/bf16 -> probabilities, same shape and dtype.
+    window: sliding-window width or None; alibi_slopes: fp32 [heads] or None."""
     assert x.dim() == 3 and x.size(1) == x.size(2)
     x = _cpu_contig(x)
     y = torch.empty_like(x)
-    _check(lib().oracle_causal_softmax_fwd(y.data_ptr(), x.data_ptr(), float(scale), x.size(0), x.size(1),
-                                           _DT[x.dtype]), "causal_softmax_fwd")
+    sl_ptr, heads = None, 1
+    if alibi_slopes is not None:
+        alibi_slopes = _cpu_contig(alibi_slopes.float())
+        sl_ptr, heads = alibi_slopes.data_ptr(), alibi_slopes.numel()
+        assert x.size(0) % heads == 0
+    _check(lib().oracle_causal_softmax_ex_fwd(y.data_ptr(), x.data_ptr(), float(scale), x.size(0), x.size(1),
+                                              -1 if window is None else int(window), sl_ptr, heads,
+                                              _DT[x.dtype]), "causal_softmax_fwd")
     return y
 
 
@@ -97,7 +106,7 @@ def masked_softmax_fwd(x, mask, scale):
     return y
 
 
-def softmax_bwd(dy, y, scale, causal):
+def softmax_bwd(dy, y, scale, causal, window=None):
     """Returns dx (a new tensor). dy, y: [..., rows_per_matrix, n]."""
     dy = _cpu_contig(dy)
     y = _cpu_contig(y)
@@ -105,8 +114,9 @@ def softmax_bwd(dy, y, scale, causal):
     n = dy.size(-1)
     rows = dy.numel() // max(n, 1)
     dx = torch.empty_like(dy)
-    _check(lib().oracle_softmax_bwd(dx.data_ptr(), dy.data_ptr(), y.data_ptr(), float(scale), rows, n,
-                                    dy.size(-2), 1 if causal else 0, _DT[dy.dtype]), "softmax_bwd")
+    _check(lib().oracle_softmax_ex_bwd(dx.data_ptr(), dy.data_ptr(), y.data_ptr(), float(scale), rows, n,
+                                       dy.size(-2), 1 if causal else 0, -1 if window is None else int(window),
+                                       _DT[dy.dtype]), "softmax_bwd")
     return dx
 
 

@@ -15,11 +15,41 @@ Follows (paths relative to the GPT-NeoX tree):
 import torch
 
 
-def causal_mask(seq_len, device="cpu"):
-    """Boolean [1,1,s,s], True where the key index exceeds the query index
-    (megatron/utils.py:67-80 without a sliding window)."""
+def causal_mask(seq_len, device="cpu", sliding_window_width=None):
+    """Boolean [1,1,s,s], True = masked: keys after the query, and with a sliding
+    window also keys more than `sliding_window_width` before it
+    (megatron/utils.py:67-80: tril, then triu(diagonal=-width), then `< 0.5`)."""
     idx = torch.arange(seq_len, device=device)
-    return (idx[None, :] > idx[:, None]).view(1, 1, seq_len, seq_len)
+    masked = idx[None, :] > idx[:, None]
+    if sliding_window_width is not None:
+        masked = masked | (idx[None, :] < idx[:, None] - sliding_window_width)
+    return masked.view(1, 1, seq_len, seq_len)
+
+
+def alibi_slopes(n):
+    """Per-head AliBi slopes (megatron/model/positional_embeddings.py:147-168)."""
+    import math
+
+    def power_of_2(m):
+        start = 2 ** (-(2 ** -(math.log2(m) - 3)))
+        return [start * start**i for i in range(m)]
+
+    if math.log2(n).is_integer():
+        return power_of_2(n)
+    closest = 2 ** math.floor(math.log2(n))
+    return power_of_2(closest) + alibi_slopes(2 * closest)[0::2][: n - closest]
+
+
+def alibi_add(scores, slopes):
+    """scores [b, np, s, s] + AliBi matrix, in scores.dtype, as AliBi.forward does for
+    sq == sk (positional_embeddings.py:219-257): a = -tril(i - j), cast, times slopes."""
+    s = scores.shape[-1]
+    i = torch.arange(s, device=scores.device)
+    a = -torch.tril(i.view(s, 1).repeat(1, s) + torch.arange(0, -s, -1, device=scores.device))
+    a = a.to(scores.dtype)
+    sl = slopes.to(a.device).to(a.dtype)
+    a = a * sl.view(sl.shape[0], 1, 1)
+    return scores + a
 
 
 def fill_masked_with_dtype_min(scores, mask):

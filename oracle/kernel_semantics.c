@@ -125,6 +125,12 @@ static float round_to(float v, int dt)
     return v;
 }
 
+/* a (*) b and a (+) b of the 16-bit scalar types (c10::Half / c10::BFloat16 operators, and torch's eager
+ * kernels for these dtypes): the fp32 operation, then rounding to the storage type
+ * (fused_rotary_positional_embedding.h:58,107,158,209 use scalar_t operators). */
+static float mul_t(float a, float b, int dt) { return round_to(a * b, dt); }
+static float add_t(float a, float b, int dt) { return round_to(a + b, dt); }
+
 /* exported for the conversion tests */
 uint16_t oracle_float_to_bf16(float f) { return float_to_bf16(f); }
 uint16_t oracle_float_to_f16(float f) { return float_to_f16(f); }
@@ -160,22 +166,49 @@ static void softmax_row(float* z, int64_t n)
  * (scaled_upper_triang_masked_softmax.h:143-260): for row q of each [s,s]
  * matrix, softmax over columns k <= q of x*scale, +0 for k > q.
  * x, y: [batches, s, s].
+ *
+ * Two generalisations that the callers of the kernel apply around it with
+ * tensors, restated here by index:
+ *   window >= 0: columns k < q - window are masked as well -- the boolean mask
+ *     of megatron/utils.py:67-80 (tril, then triu with diagonal -window);
+ *   slopes != NULL: the AliBi matrix of
+ *     megatron/model/positional_embeddings.py:219-257 is added to the scores
+ *     first, in the storage dtype: a = dt(-(q-k)) (*) dt(slope[head]),
+ *     x' = x (+) a, head = batch index % heads (transformer.py:584-585 adds it
+ *     to the [b, np, sq, sk] scores before scale_mask_softmax).
  */
-int oracle_causal_softmax_fwd(void* y, const void* x, float scale, int64_t batches, int64_t s, int dt)
+int oracle_causal_softmax_ex_fwd(void* y, const void* x, float scale, int64_t batches, int64_t s,
+                                 int64_t window, const float* slopes, int64_t heads, int dt)
 {
     if (dt != DT_F16 && dt != DT_BF16) return -1;
     float* z = (float*)malloc(sizeof(float) * (size_t)(s > 0 ? s : 1));
     if (!z) return -2;
-    for (int64_t a = 0; a < batches; ++a)
+    for (int64_t a = 0; a < batches; ++a) {
+        const float slope = slopes ? round_to(slopes[a % heads], dt) : 0.0f;
         for (int64_t q = 0; q < s; ++q) {
             const int64_t base = (a * s + q) * s;
-            for (int64_t k = 0; k <= q; ++k) z[k] = load_elem(x, base + k, dt) * scale;
-            softmax_row(z, q + 1);
-            for (int64_t k = 0; k <= q; ++k) store_elem(y, base + k, dt, z[k]);
+            const int64_t lo = (window >= 0 && q > window) ? q - window : 0;
+            for (int64_t k = lo; k <= q; ++k) {
+                float v = load_elem(x, base + k, dt);
+                if (slopes) {
+                    const float dist = round_to(-(float)(q - k), dt);
+                    v = add_t(v, mul_t(dist, slope, dt), dt);
+                }
+                z[k - lo] = v * scale;
+            }
+            softmax_row(z, q + 1 - lo);
+            for (int64_t k = 0; k < lo; ++k) store_elem(y, base + k, dt, 0.0f);
+            for (int64_t k = lo; k <= q; ++k) store_elem(y, base + k, dt, z[k - lo]);
             for (int64_t k = q + 1; k < s; ++k) store_elem(y, base + k, dt, 0.0f);
         }
+    }
     free(z);
     return 0;
+}
+
+int oracle_causal_softmax_fwd(void* y, const void* x, float scale, int64_t batches, int64_t s, int dt)
+{
+    return oracle_causal_softmax_ex_fwd(y, x, scale, batches, s, -1, NULL, 1, dt);
 }
 
 /*
@@ -211,8 +244,8 @@ int oracle_masked_softmax_fwd(void* y, const void* x, const uint8_t* mask, float
  * dx = scale * (g - y * sum(g)). rows x n elements; rows_per_matrix gives the
  * causal row index q = row % rows_per_matrix. dx may alias dy.
  */
-int oracle_softmax_bwd(void* dx, const void* dy, const void* y, float scale, int64_t rows, int64_t n,
-                       int64_t rows_per_matrix, int causal, int dt)
+int oracle_softmax_ex_bwd(void* dx, const void* dy, const void* y, float scale, int64_t rows, int64_t n,
+                          int64_t rows_per_matrix, int causal, int64_t window, int dt)
 {
     if (dt != DT_F16 && dt != DT_BF16) return -1;
     float* g = (float*)malloc(sizeof(float) * (size_t)(n > 0 ? n : 1));
@@ -223,10 +256,13 @@ int oracle_softmax_bwd(void* dx, const void* dy, const void* y, float scale, int
         return -2;
     }
     for (int64_t r = 0; r < rows; ++r) {
-        const int64_t valid = causal ? (r % rows_per_matrix) + 1 : n;
+        const int64_t q = r % rows_per_matrix;
+        const int64_t valid = causal ? q + 1 : n;
+        /* sliding window: columns below q - window are masked like those above the diagonal */
+        const int64_t lo = (causal && window >= 0 && q > window) ? q - window : 0;
         const int64_t base = r * n;
         for (int64_t k = 0; k < n; ++k) {
-            if (k < valid) {
+            if (k >= lo && k < valid) {
                 p[k] = load_elem(y, base + k, dt);
                 g[k] = load_elem(dy, base + k, dt) * p[k];
             } else {
@@ -246,6 +282,12 @@ int oracle_softmax_bwd(void* dx, const void* dy, const void* y, float scale, int
     return 0;
 }
 
+int oracle_softmax_bwd(void* dx, const void* dy, const void* y, float scale, int64_t rows, int64_t n,
+                       int64_t rows_per_matrix, int causal, int dt)
+{
+    return oracle_softmax_ex_bwd(dx, dy, y, scale, rows, n, rows_per_matrix, causal, -1, dt);
+}
+
 /*
  * get_batch_per_block (scaled_masked_softmax.h:338-352) for a machine whose
  * warp is `warp` lanes wide (32 on NVIDIA, 64 on gfx9).
@@ -263,10 +305,6 @@ int oracle_batch_per_block(int64_t key_seq_len, int warp)
 /* rotary embedding                                                          */
 /* ------------------------------------------------------------------------ */
 
-/* a (*) b and a (+) b of the 16-bit scalar types: fp32 operation, then round
- * (fused_rotary_positional_embedding.h:58,107,158,209 use scalar_t operators). */
-static float mul_t(float a, float b, int dt) { return round_to(a * b, dt); }
-static float add_t(float a, float b, int dt) { return round_to(a + b, dt); }
 
 /*
  * Shared body of the four rotary kernels

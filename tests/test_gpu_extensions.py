@@ -1,0 +1,107 @@
+"""GPU parity of the sliding-window / AliBi variants of the causal softmax, through
+the C ABI and through FusedScaleMaskSoftmax, against the CPU oracle.
+Tolerances as for the plain kernels: 2 ulp forward, masked positions bit-exact +0,
+backward 2 ulp plus the fp32 row-sum noise."""
+import math
+
+import pytest
+import torch
+
+import oracle
+import util
+from oracle import fallback_semantics as fb
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+DTYPES = [torch.bfloat16, torch.float16]
+
+
+def abi_ex_fwd(hp, x, scale, window, slopes):
+    y = torch.empty_like(x)
+    rc = hp.lib().nhp_causal_softmax_ex_fwd(
+        y.data_ptr(), x.data_ptr(), scale, x.size(0), x.size(1), -1 if window is None else window,
+        None if slopes is None else slopes.data_ptr(), 1 if slopes is None else slopes.numel(),
+        hp.dtype_code(x, "t"), None)
+    assert rc == 0, hp.lib().nhp_status_string(rc)
+    return y
+
+
+def abi_ex_bwd(hp, dy, y, scale, window):
+    dx = torch.empty_like(dy)
+    rc = hp.lib().nhp_causal_softmax_ex_bwd(dx.data_ptr(), dy.data_ptr(), y.data_ptr(), scale, dy.size(0), dy.size(1),
+                                            -1 if window is None else window, hp.dtype_code(dy, "t"), None)
+    assert rc == 0, hp.lib().nhp_status_string(rc)
+    return dx
+
+
+# (attn_batches, seq_len, window, heads or None)
+CASES = [
+    (4, 64, 0, None), (4, 64, 5, 2), (3, 200, 63, None), (2, 512, 100, 2), (2, 1024, 511, None),
+    (2, 1024, 512, 2), (2, 2048, 7, None), (6, 2048, 700, 6), (2, 2048, None, 2), (1, 4096, 1000, None),
+    (2, 4096, 3000, 2), (1, 8192, 2047, 1), (2, 1001, 50, 2), (2, 33, 40, None), (4, 2056, 1024, 4),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
+@pytest.mark.parametrize("case", CASES, ids=lambda c: f"a{c[0]}_s{c[1]}_w{c[2]}_h{c[3]}")
+def test_window_alibi_forward_backward_vs_oracle(hotpath, case, dtype):
+    a, s, window, heads = case
+    print(f"ex case {case} {dtype}", flush=True)
+    scale = 1 / math.sqrt(128)
+    slopes = None if heads is None else torch.tensor(fb.alibi_slopes(max(heads, 2))[:heads], dtype=torch.float32)
+    x = util.randn((a, s, s), dtype, seed=s + (window or 0), std=2.0)
+    dy = util.randn((a, s, s), dtype, seed=s + 1)
+    want_y = oracle.causal_softmax_fwd(x, scale, window=window, alibi_slopes=slopes)
+    got_y = abi_ex_fwd(hotpath, x.to(DEV), scale, window, None if slopes is None else slopes.to(DEV)).cpu()
+    masked = fb.causal_mask(s, sliding_window_width=window)[0, 0]
+    assert int(util.raw_bits(got_y)[:, masked].abs().max() if masked.any() else 0) == 0
+    util.assert_ulp_close(got_y, want_y, 2, "fwd")
+    want_dx = oracle.softmax_bwd(dy, want_y, scale, causal=True, window=window)
+    got_dx = abi_ex_bwd(hotpath, dy.to(DEV), want_y.to(DEV), scale, window).cpu()
+    assert int(util.raw_bits(got_dx)[:, masked].abs().max() if masked.any() else 0) == 0
+    util.assert_softmax_bwd_close(got_dx, want_dx, dy.masked_fill(masked, 0), want_y, scale, "bwd")
+
+
+def test_window_never_reads_outside_the_band(hotpath):
+    """NaNs planted outside the band (and above the diagonal) must not reach the output."""
+    a, s, window = 2, 2048, 300
+    x = util.randn((a, s, s), torch.bfloat16, seed=1, std=2.0)
+    masked = fb.causal_mask(s, sliding_window_width=window)[0, 0]
+    # chunk granularity: a 16-byte chunk that straddles the band edge is loaded, so poison whole chunks only
+    col = torch.arange(s)
+    q = torch.arange(s)[:, None]
+    poison = ((col[None, :] // 8 * 8 + 8) <= (q - window)) | ((col[None, :] // 8 * 8) > q)
+    xp = x.clone()
+    xp[:, poison] = float("nan")
+    y = abi_ex_fwd(hotpath, xp.to(DEV), 0.1, window, None).cpu()
+    assert not torch.isnan(y.float()).any()
+    util.assert_ulp_close(y, oracle.causal_softmax_fwd(x, 0.1, window=window), 2, "poisoned")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
+def test_module_with_window_and_alibi(dtype):
+    from megatron.model.fused_softmax import FusedScaleMaskSoftmax, SoftmaxFusionTypes as T
+    from megatron.model.positional_embeddings import AliBi
+
+    b, np_, s, window, scale = 2, 8, 1024, 256, 0.125
+    alibi = AliBi(np_, mp_size=1, mp_rank=0)
+    x = util.randn((b, np_, s, s), dtype, seed=9, std=2.0)
+    dy = util.randn((b, np_, s, s), dtype, seed=10)
+    mask = fb.causal_mask(s, DEV, sliding_window_width=window)
+    fused = FusedScaleMaskSoftmax(dtype == torch.float16, dtype == torch.bfloat16, T.upper_triang,
+                                  fb.fill_masked_with_dtype_min, True, scale, sliding_window_width=window,
+                                  alibi_slopes=alibi.slopes).to(DEV)
+    xd = x.to(DEV).requires_grad_(True)
+    y = fused(xd, mask)
+    want = oracle.causal_softmax_fwd(x.view(-1, s, s), scale, window=window, alibi_slopes=alibi.slopes).view(b, np_, s, s)
+    util.assert_ulp_close(y.detach().cpu(), want, 2, "module fwd")
+    y.backward(dy.to(DEV))
+    yc = y.detach().cpu()
+    want_dx = oracle.softmax_bwd(dy.view(-1, s, s), yc.view(-1, s, s), scale, True, window=window).view(b, np_, s, s)
+    masked = mask.cpu()[0, 0]
+    util.assert_softmax_bwd_close(xd.grad.cpu(), want_dx, dy.masked_fill(masked, 0), yc, scale, "module bwd")
+    # the unfused route the reference would take: eager AliBi add, then the torch softmax with the window mask
+    plain = FusedScaleMaskSoftmax(dtype == torch.float16, dtype == torch.bfloat16, T.none,
+                                  fb.fill_masked_with_dtype_min, True, scale)
+    ref = plain(alibi.to(DEV)(x.to(DEV)), mask)
+    util.assert_ulp_close(y.detach().cpu(), ref.cpu(), 2, "fused vs eager AliBi + torch softmax")

@@ -1,0 +1,143 @@
+"""Pins the oracle's sliding-window and AliBi variants of the causal softmax and
+the host-side AliBi mirror, without a GPU."""
+import math
+
+import pytest
+import torch
+
+import oracle
+import util
+from oracle import fallback_semantics as fb
+
+DTYPES = [torch.bfloat16, torch.float16]
+IDS = ["bf16", "fp16"]
+
+
+def f64_softmax_rows(z):
+    z = z.double()
+    z = z - z.max(dim=-1, keepdim=True).values
+    e = z.exp()
+    return e / e.sum(dim=-1, keepdim=True)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("s,window", [(16, 0), (16, 3), (33, 8), (100, 31), (100, 99), (64, 200)])
+def test_sliding_window_forward(dtype, s, window):
+    a, scale = 2, 0.3
+    x = util.randn((a, s, s), dtype, seed=s + window, std=2.0)
+    y = oracle.causal_softmax_fwd(x, scale, window=window)
+    masked = fb.causal_mask(s, sliding_window_width=window)[0, 0]
+    # everything outside the band is +0 bit for bit
+    assert int(util.raw_bits(y)[:, masked].abs().max()) == 0
+    # float64 brute force over the band
+    z = (x.double() * float(torch.tensor(scale, dtype=torch.float32))).masked_fill(masked, float("-inf"))
+    util.assert_ulp_close(y, f64_softmax_rows(z).to(dtype), 1, "vs float64")
+    # the reference's torch path with the sliding-window mask of get_attn_mask
+    ref = fb.torch_softmax_fallback(x.view(1, a, s, s), masked.view(1, 1, s, s), scale).view(a, s, s)
+    util.assert_ulp_close(y, ref, 1, "vs torch fallback")
+    # the band of row q holds min(q, window) + 1 keys
+    counts = (~masked).sum(-1)
+    assert torch.equal(counts, torch.clamp(torch.arange(s), max=window) + 1)
+    if window == 0:
+        assert torch.equal(y.float(), torch.eye(s).expand(a, s, s))
+    if window >= s - 1:
+        assert torch.equal(util.raw_bits(y), util.raw_bits(oracle.causal_softmax_fwd(x, scale)))
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_sliding_window_backward(dtype):
+    a, s, window, scale = 2, 40, 9, 0.6
+    x = util.randn((a, s, s), dtype, seed=1, std=2.0)
+    y = oracle.causal_softmax_fwd(x, scale, window=window)
+    dy = util.randn((a, s, s), dtype, seed=2)
+    dx = oracle.softmax_bwd(dy, y, scale, causal=True, window=window)
+    masked = fb.causal_mask(s, sliding_window_width=window)[0, 0]
+    assert int(util.raw_bits(dx)[:, masked].abs().max()) == 0
+    g = (dy.double() * y.double()).masked_fill(masked, 0.0)
+    want = float(torch.tensor(scale, dtype=torch.float32)) * (g - y.double().masked_fill(masked, 0.0) * g.sum(-1, keepdim=True))
+    util.assert_softmax_bwd_close(dx, want.to(dtype), dy.masked_fill(masked, 0), y, scale, "vs float64 JVP")
+    # dy outside the band must not leak into the row sum: garbage there changes nothing
+    dy2 = dy.clone()
+    dy2[:, masked] = 1000.0
+    dx2 = oracle.softmax_bwd(dy2, y, scale, causal=True, window=window)
+    assert torch.equal(util.raw_bits(dx2), util.raw_bits(dx))
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("heads", [4, 6])
+def test_alibi_equals_eager_add_then_plain_softmax(dtype, heads):
+    """softmax_alibi(x) == softmax(x + alibi_matrix) with the sum formed by torch in
+    the storage dtype: pins the sign, the orientation (q - k), the head indexing
+    (batch % heads) and the three roundings."""
+    b, s, scale = 2, 300, 0.2  # distances above 256 are not exact in bf16
+    slopes = torch.tensor(fb.alibi_slopes(heads), dtype=torch.float32)
+    x = util.randn((b, heads, s, s), dtype, seed=heads, std=2.0)
+    fused = oracle.causal_softmax_fwd(x.view(-1, s, s), scale, alibi_slopes=slopes)
+    eager = oracle.causal_softmax_fwd(fb.alibi_add(x, slopes).view(-1, s, s), scale)
+    assert torch.equal(util.raw_bits(fused), util.raw_bits(eager))
+    zero = oracle.causal_softmax_fwd(x.view(-1, s, s), scale, alibi_slopes=torch.zeros(heads))
+    assert torch.equal(util.raw_bits(zero), util.raw_bits(oracle.causal_softmax_fwd(x.view(-1, s, s), scale)))
+    # the bias favours recent keys: with constant scores the probabilities increase towards the diagonal
+    c = torch.zeros((1, heads, 64, 64), dtype=dtype)
+    p = oracle.causal_softmax_fwd(c.view(-1, 64, 64), 1.0, alibi_slopes=slopes).float()
+    assert (p[0, 63, :64].diff() >= 0).all() and p[0, 63, 63] > p[0, 63, 0]
+
+
+def test_alibi_with_window_combined():
+    heads, s, window = 4, 64, 10
+    slopes = torch.tensor(fb.alibi_slopes(heads), dtype=torch.float32)
+    x = util.randn((1, heads, s, s), torch.bfloat16, seed=3, std=2.0)
+    fused = oracle.causal_softmax_fwd(x.view(-1, s, s), 0.5, window=window, alibi_slopes=slopes)
+    eager = oracle.causal_softmax_fwd(fb.alibi_add(x, slopes).view(-1, s, s), 0.5, window=window)
+    assert torch.equal(util.raw_bits(fused), util.raw_bits(eager))
+
+
+def test_alibi_module_mirror():
+    from megatron.model.positional_embeddings import AliBi
+
+    # the reference's default mp_rank=1 with mp_size=1 selects an empty slice; callers pass the 0-based rank
+    assert AliBi(8).slopes.numel() == 0
+    a8 = AliBi(8, mp_size=1, mp_rank=0)
+    assert torch.allclose(a8.slopes, torch.tensor([2.0 ** -(i + 1) for i in range(8)]))
+    a12 = AliBi(12, 1, 0)
+    assert a12.slopes.shape == (12,) and torch.allclose(a12.slopes, torch.tensor(fb.alibi_slopes(12)))
+    assert torch.allclose(a12.slopes[:8], a8.slopes)
+    # model-parallel slicing: rank r keeps heads [r*slice, (r+1)*slice)
+    part = AliBi(8, mp_size=2, mp_rank=1)
+    assert torch.equal(part.slopes, a8.slopes[4:])
+    assert "slopes" in a8.state_dict()
+    # forward adds -(q-k)*slope below the diagonal and nothing above
+    x = torch.zeros(1, 8, 5, 5)
+    y = a8(x)
+    assert y[0, 0, 4, 0].item() == -4 * 0.5 and y[0, 0, 4, 4].item() == 0 and y[0, 0, 0, 4].item() == 0
+    assert y[0, 3, 3, 1].item() == -2 * 2.0**-4
+    # same arithmetic as the restatement, in bf16
+    xb = util.randn((2, 8, 40, 40), torch.bfloat16, seed=1)
+    assert torch.equal(util.raw_bits(AliBi(8, 1, 0)(xb)), util.raw_bits(fb.alibi_add(xb, a8.slopes)))
+    # the cached matrix grows fourfold, is clipped for shorter inputs, and serves single-query decoding
+    al = AliBi(4, 1, 0)
+    al(torch.zeros(1, 4, 6, 6))
+    assert al.cached_seq_len == 6
+    al(torch.zeros(1, 4, 7, 7))
+    assert al.cached_seq_len == 24
+    assert al(torch.zeros(1, 4, 3, 3)).shape == (1, 4, 3, 3)
+    d = al(torch.zeros(1, 4, 1, 9))
+    assert d.shape == (1, 4, 1, 9) and d[0, 0, 0, 8].item() == 0 and d[0, 0, 0, 0].item() == -8 * al.slopes[0].item()
+    with pytest.raises(AssertionError):
+        al(torch.zeros(1, 4, 2, 9))
+
+
+@pytest.mark.parametrize("dtype,fp16,bf16", [(torch.float16, True, False), (torch.bfloat16, False, True)])
+def test_module_torch_path_with_window_and_alibi(dtype, fp16, bf16):
+    """With fusion off the module applies the same semantics with torch ops (CPU here)."""
+    from megatron.model.fused_softmax import FusedScaleMaskSoftmax, SoftmaxFusionTypes as T
+
+    b, np_, s, window, scale = 2, 4, 48, 7, 0.25
+    slopes = torch.tensor(fb.alibi_slopes(np_), dtype=torch.float32)
+    x = util.randn((b, np_, s, s), dtype, seed=5, std=2.0)
+    m = FusedScaleMaskSoftmax(fp16, bf16, T.none, fb.fill_masked_with_dtype_min, True, scale,
+                              sliding_window_width=window, alibi_slopes=slopes)
+    y = m(x.clone(), fb.causal_mask(s, sliding_window_width=window))
+    want = oracle.causal_softmax_fwd(x.view(-1, s, s), scale, window=window, alibi_slopes=slopes).view(b, np_, s, s)
+    util.assert_ulp_close(y, want, 1, "torch path vs oracle")
+    assert "alibi_slopes" not in m.state_dict()
