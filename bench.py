@@ -14,6 +14,7 @@ the drop-in extension modules (which call libneox_hotpath.so):
   masked-c3      padding-masked softmax fwd+bwd [16,32,1024,2048] fp16
   rope-c4        rotary fwd+bwd on q,k [4096,4,32,128] bf16, rotary_pct 1.0 and 0.25
   llama2-7b-c5   rotary on q,k [8192,2,32,128] + causal softmax fwd+bwd [64,8192,8192] bf16
+  rope-qk-1.4b   rotary fwd+bwd on q,k [2048,8,16,128] bf16, rotary_pct 0.25, q and k in one launch
   mistral-window causal softmax fwd+bwd [64,8192,8192] bf16 with a 4096-key sliding window applied by index
   alibi-1.4b     causal softmax fwd+bwd [128,2048,2048] bf16 with the AliBi bias of 16 heads added in the kernel
 
@@ -199,6 +200,22 @@ def make_workload(name, torch, dev):
         cfg = {"workload": name, "scores": [b, np_, sq, sk], "mask": [b, 1, sq, sk],
                "bytes_convention": "dense (2x tensor forward + mask once, 3x tensor backward)"}
         return step, kernel_bytes, {}, "masked_softmax_bwd", "f16", cfg
+
+    if name == "rope-qk-1.4b":
+        s, b, h, d, d2 = 2048, 8, 16, 128, 32
+        sets = [rope_setup(s, b, h, d, d2, 50 + 10 * i) for i in range(4)]  # rotate buffers: 64 MiB tensors fit the cache
+        rb = rope_bytes(s, b, h, d, d2)
+        kernel_bytes = {"rope_qk_fwd": 2 * rb - 2 * s * d2 * 2, "rope_qk_bwd": 2 * rb - 2 * s * d2 * 2}
+        state = {"i": 0}
+
+        def step(t):
+            q, k, dq, dk, cos, sin = sets[state["i"] % len(sets)]
+            state["i"] += 1
+            t.run("rope_qk_fwd", lambda: rope_ext.forward_cached_qk(q, k, cos, sin, False))
+            t.run("rope_qk_bwd", lambda: rope_ext.backward_cached_qk(dq, dk, cos, sin, False))
+
+        cfg = {"workload": name, "qk": [s, b, h, d], "rotary_dim": d2}
+        return step, kernel_bytes, {}, "rope_qk_fwd", "bf16", cfg
 
     if name == "rope-c4":
         s, b, h, d = 4096, 4, 32, 128

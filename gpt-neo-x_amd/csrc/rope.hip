@@ -174,14 +174,31 @@ struct FreqTable {
 // Requires: stride_d == 1 on both sides, d % V == 0, d2 % (2V) == 0, d <= 64 V,
 // every other stride a multiple of V, 16-byte aligned base pointers and tables.
 // ---------------------------------------------------------------------------
+// One tensor of a launch: where it lives and how its (batch, head) rows are strided.
+struct RopeTensor {
+    void* out;
+    const void* in;
+    int rows;  // b * h
+    int h;
+    int64_t is_s, is_b, is_h, os_s, os_b, os_h;
+};
+// A launch rotates one or two tensors (q and k) with the same tables; blockIdx.z picks the tensor.
+struct RopePair {
+    RopeTensor t[2];
+};
+
 // FLAT: the batch and head dimensions collapse into one row dimension on both
 // sides (stride_b == h * stride_h), which saves the division by h per row.
 // U: rows in flight per lane (loads of U steps are issued before the first is used).
 template <int DT, bool BWD, bool FLAT, int U, typename Tables>
 __global__ void __launch_bounds__(256)
-rope_vec_kernel(void* out, const void* in, Tables tab, int rows, int h, int cpr, int rot_chunks, int rpw,
-                int64_t is_s, int64_t is_b, int64_t is_h, int64_t os_s, int64_t os_b, int64_t os_h)
+rope_vec_kernel(RopePair pair, Tables tab, int cpr, int rot_chunks, int rpw)
 {
+    const RopeTensor& T = pair.t[blockIdx.z];
+    void* const out = T.out;
+    const void* const in = T.in;
+    const int rows = T.rows, h = T.h;
+    const int64_t is_s = T.is_s, is_b = T.is_b, is_h = T.is_h, os_s = T.os_s, os_b = T.os_b, os_h = T.os_h;
     constexpr int V = Elt<DT>::kVec;
     using S = typename Elt<DT>::storage;
     const int lane = threadIdx.x & 63;
@@ -347,43 +364,71 @@ static inline int rope_tune(const char*, int def) { return def; }
 #endif
 
 template <int DT, bool BWD, typename Tables>
-static int rope_launch(const RopeArgs& a, const Tables& tab, bool tables_ok)
+static int rope_launch_scalar(const RopeArgs& a, const Tables& tab)
+{
+    const int64_t total = a.s * a.b * a.h * a.d;
+    const int64_t blocks = (total + 255) / 256;
+    if (blocks >= ((int64_t)1 << 24)) return NHP_ERR_SHAPE;  // grid*block must stay below 2^32
+    rope_scalar_kernel<DT, BWD, Tables><<<(uint32_t)blocks, 256, 0, a.st>>>(
+        a.out, a.in, tab, total, a.b, a.h, a.d, a.d2, a.is[0], a.is[1], a.is[2], a.is[3], a.os[0], a.os[1],
+        a.os[2], a.os[3]);
+    return hipGetLastError() == hipSuccess ? NHP_OK : NHP_ERR_LAUNCH;
+}
+
+static RopeTensor rope_tensor(const RopeArgs& a)
+{
+    return RopeTensor{a.out, a.in, (int)(a.b * a.h), (int)a.h, a.is[0], a.is[1], a.is[2], a.os[0], a.os[1], a.os[2]};
+}
+
+static bool rope_flat(const RopeArgs& a) { return (a.is[1] == a.h * a.is[2]) && (a.os[1] == a.h * a.os[2]); }
+
+// Launches the vector kernel for one tensor (b == nullptr) or for two tensors
+// that share s, d, d2 and the tables (q and k; their head counts may differ).
+template <int DT, bool BWD, typename Tables>
+static int rope_launch_vec(const RopeArgs& a, const RopeArgs* b, const Tables& tab)
 {
     constexpr int V = Elt<DT>::kVec;
-    if (vector_ok<DT>(a, tables_ok)) {
-        const int cpr = (int)(a.d / V);
-        const int rpw = 64 / cpr;
-        const int rows = (int)(a.b * a.h);
-        const int rows_per_step = 4 * rpw;
-        // Workgroups per position: each makes about four steps (two unrolled loop
-        // iterations) with one set of cos/sin values; measured best on MI355X.
-        const int64_t steps = (rows + rows_per_step - 1) / rows_per_step;
-        int64_t splits = (steps + 3) / 4;
-        splits = rope_tune("NHP_ROPE_SPLITS", (int)splits);
-        if (splits > 65535) splits = 65535;
-        dim3 grid((uint32_t)a.s, (uint32_t)splits);
-        const uint32_t lds = (uint32_t)rope_tune("NHP_ROPE_LDS", 0);
-        const bool flat = (a.is[1] == a.h * a.is[2]) && (a.os[1] == a.h * a.os[2]);
-#define NHP_ROPE_LAUNCH(FLAT_, U_)                                                                         \
-    rope_vec_kernel<DT, BWD, FLAT_, U_, Tables><<<grid, 256, lds, a.st>>>(                                 \
-        a.out, a.in, tab, rows, (int)a.h, cpr, (int)(a.d2 / V), rpw, a.is[0], a.is[1], a.is[2], a.os[0],   \
-        a.os[1], a.os[2])
-        // two rows in flight per lane measured best (one is short of latency cover, four adds nothing)
-        if (flat) {
-            NHP_ROPE_LAUNCH(true, 2);
-        } else {
-            NHP_ROPE_LAUNCH(false, 2);
-        }
-#undef NHP_ROPE_LAUNCH
+    const int cpr = (int)(a.d / V);
+    const int rpw = 64 / cpr;
+    const int rows_per_step = 4 * rpw;
+    RopePair pair;
+    pair.t[0] = rope_tensor(a);
+    pair.t[1] = b ? rope_tensor(*b) : pair.t[0];
+    const int rows = (b && pair.t[1].rows > pair.t[0].rows) ? pair.t[1].rows : pair.t[0].rows;
+    // Workgroups per position: each makes about four steps (two unrolled loop
+    // iterations) with one set of cos/sin values; measured best on MI355X.
+    const int64_t steps = (rows + rows_per_step - 1) / rows_per_step;
+    int64_t splits = (steps + 3) / 4;
+    splits = rope_tune("NHP_ROPE_SPLITS", (int)splits);
+    if (splits < 1) splits = 1;
+    if (splits > 65535) splits = 65535;
+    dim3 grid((uint32_t)a.s, (uint32_t)splits, b ? 2u : 1u);
+    const uint32_t lds = (uint32_t)rope_tune("NHP_ROPE_LDS", 0);
+    const bool flat = rope_flat(a) && (!b || rope_flat(*b));
+    // two rows in flight per lane measured best (one is short of latency cover, four adds nothing)
+    if (flat) {
+        rope_vec_kernel<DT, BWD, true, 2, Tables><<<grid, 256, lds, a.st>>>(pair, tab, cpr, (int)(a.d2 / V), rpw);
     } else {
-        const int64_t total = a.s * a.b * a.h * a.d;
-        const int64_t blocks = (total + 255) / 256;
-        if (blocks >= ((int64_t)1 << 24)) return NHP_ERR_SHAPE;  // grid*block must stay below 2^32
-        rope_scalar_kernel<DT, BWD, Tables><<<(uint32_t)blocks, 256, 0, a.st>>>(
-            a.out, a.in, tab, total, a.b, a.h, a.d, a.d2, a.is[0], a.is[1], a.is[2], a.is[3], a.os[0],
-            a.os[1], a.os[2], a.os[3]);
+        rope_vec_kernel<DT, BWD, false, 2, Tables><<<grid, 256, lds, a.st>>>(pair, tab, cpr, (int)(a.d2 / V), rpw);
     }
     return hipGetLastError() == hipSuccess ? NHP_OK : NHP_ERR_LAUNCH;
+}
+
+template <int DT, bool BWD, typename Tables>
+static int rope_launch(const RopeArgs& a, const Tables& tab, bool tables_ok)
+{
+    if (vector_ok<DT>(a, tables_ok)) return rope_launch_vec<DT, BWD>(a, nullptr, tab);
+    return rope_launch_scalar<DT, BWD>(a, tab);
+}
+
+// q and k in one launch when both qualify for the vector kernel, otherwise one launch each.
+template <int DT, bool BWD, typename Tables>
+static int rope_launch_pair(const RopeArgs& q, const RopeArgs& k, const Tables& tab, bool tables_ok)
+{
+    if (vector_ok<DT>(q, tables_ok) && vector_ok<DT>(k, tables_ok)) return rope_launch_vec<DT, BWD>(q, &k, tab);
+    const int rc = rope_launch<DT, BWD>(q, tab, tables_ok);
+    if (rc != NHP_OK) return rc;
+    return rope_launch<DT, BWD>(k, tab, tables_ok);
 }
 
 static int check_common(const void* out, const void* in, int64_t s, int64_t b, int64_t h, int64_t d,
@@ -446,6 +491,48 @@ static int rope_freqs(void* out, const void* in, const float* freqs, int64_t s, 
     return rope_launch<NHP_F32, BWD>(a, FreqTable<NHP_F32>{freqs, d2}, true);
 }
 
+template <bool BWD>
+static int rope_cached_qk(void* q_out, void* k_out, const void* q_in, const void* k_in, const void* cos,
+                          const void* sin, int64_t s, int64_t b, int64_t hq, int64_t hk, int64_t d, int64_t d2,
+                          const int64_t* qis, const int64_t* kis, const int64_t* qos, const int64_t* kos, int dtype,
+                          int cs_dtype, void* stream)
+{
+    if (dtype != NHP_F16 && dtype != NHP_BF16 && dtype != NHP_F32) return NHP_ERR_DTYPE;
+    if (cs_dtype != NHP_F32 && cs_dtype != dtype) return NHP_ERR_DTYPE;
+    bool empty_q, empty_k;
+    int rc = check_common(q_out, q_in, s, b, hq, d, d2, qis, qos, empty_q);
+    if (rc != NHP_OK) return rc;
+    rc = check_common(k_out, k_in, s, b, hk, d, d2, kis, kos, empty_k);
+    if (rc != NHP_OK) return rc;
+    if (empty_q || empty_k) {
+        // at most one tensor has work: hand it to the single-tensor path
+        if (!empty_q)
+            return rope_cached<BWD>(q_out, q_in, cos, sin, s, b, hq, d, d2, qis, qos, dtype, cs_dtype, stream);
+        if (!empty_k)
+            return rope_cached<BWD>(k_out, k_in, cos, sin, s, b, hk, d, d2, kis, kos, dtype, cs_dtype, stream);
+        return NHP_OK;
+    }
+    if (q_out == k_in || k_out == q_in || q_out == k_out) return NHP_ERR_ALIAS;
+    if (d2 > 0 && (!cos || !sin)) return NHP_ERR_NULL;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    RopeArgs q{q_out, q_in, s, b, hq, d, d2, {qis[0], qis[1], qis[2], qis[3]}, {qos[0], qos[1], qos[2], qos[3]}, st};
+    RopeArgs k{k_out, k_in, s, b, hk, d, d2, {kis[0], kis[1], kis[2], kis[3]}, {kos[0], kos[1], kos[2], kos[3]}, st};
+    const int cs_size = (cs_dtype == NHP_F32) ? 4 : 2;
+    const bool tab_ok = is_aligned16(cos) && is_aligned16(sin) && (d2 * cs_size) % 16 == 0;
+#define NHP_ROPE_CASE(DT_, CS_)                                         \
+    if (dtype == DT_ && cs_dtype == CS_) {                              \
+        CachedTables<DT_, CS_> tab{cos, sin, d2};                       \
+        return rope_launch_pair<DT_, BWD>(q, k, tab, tab_ok);           \
+    }
+    NHP_ROPE_CASE(NHP_BF16, NHP_BF16)
+    NHP_ROPE_CASE(NHP_BF16, NHP_F32)
+    NHP_ROPE_CASE(NHP_F16, NHP_F16)
+    NHP_ROPE_CASE(NHP_F16, NHP_F32)
+    NHP_ROPE_CASE(NHP_F32, NHP_F32)
+#undef NHP_ROPE_CASE
+    return NHP_ERR_DTYPE;
+}
+
 }  // namespace nhp
 
 using namespace nhp;
@@ -480,6 +567,26 @@ int nhp_rope_freqs_bwd(void* out, const void* in, const float* freqs, int64_t s,
                        int dtype, void* stream)
 {
     return rope_freqs<true>(out, in, freqs, s, b, h, d, d2, in_stride, out_stride, dtype, stream);
+}
+
+int nhp_rope_cached_qk_fwd(void* q_out, void* k_out, const void* q_in, const void* k_in, const void* cos,
+                           const void* sin, int64_t s, int64_t b, int64_t hq, int64_t hk, int64_t d, int64_t d2,
+                           const int64_t q_in_stride[4], const int64_t k_in_stride[4],
+                           const int64_t q_out_stride[4], const int64_t k_out_stride[4], int dtype, int cs_dtype,
+                           void* stream)
+{
+    return rope_cached_qk<false>(q_out, k_out, q_in, k_in, cos, sin, s, b, hq, hk, d, d2, q_in_stride, k_in_stride,
+                                 q_out_stride, k_out_stride, dtype, cs_dtype, stream);
+}
+
+int nhp_rope_cached_qk_bwd(void* q_out, void* k_out, const void* q_in, const void* k_in, const void* cos,
+                           const void* sin, int64_t s, int64_t b, int64_t hq, int64_t hk, int64_t d, int64_t d2,
+                           const int64_t q_in_stride[4], const int64_t k_in_stride[4],
+                           const int64_t q_out_stride[4], const int64_t k_out_stride[4], int dtype, int cs_dtype,
+                           void* stream)
+{
+    return rope_cached_qk<true>(q_out, k_out, q_in, k_in, cos, sin, s, b, hq, hk, d, d2, q_in_stride, k_in_stride,
+                                q_out_stride, k_out_stride, dtype, cs_dtype, stream);
 }
 
 int nhp_abi_version(void) { return 1; }

@@ -101,3 +101,47 @@ def backward_cached(output_grads, cos, sin, transpose_output):
     """Gradient of ``forward_cached`` w.r.t. its input."""
     return _run_cached("fused_rotary_positional_embedding.backward_cached", _hp.lib().nhp_rope_cached_bwd,
                        output_grads, cos, sin, transpose_output, "output_grads")
+
+
+def _run_cached_qk(name, fn, q, k, cos, sin, transpose_output):
+    for t, what in ((q, "q"), (k, "k")):
+        _check(t.dim() == 4, "expected 4D tensor")
+        _check(t.size(0) == cos.size(0), f"expected {what} and cos tensor have the same sequence length")
+        _check(t.size(3) >= cos.size(3),
+               f"expected the last dim of the {what} tensor equals or is greater than the cos tensor")
+        _check(t.dtype in _FLOATS, f"{name}: unsupported dtype {t.dtype}")
+        _hp.require_gpu(t, name)
+    _check(cos.dim() == 4 and sin.dim() == 4, "expected 4D tensor")
+    _check(cos.shape == sin.shape, "expected cos and sin tensor have the same shape")
+    _check(cos.size(1) == 1 and cos.size(2) == 1, "expected the second and third dims of the cos tensor equal 1")
+    _check(cos.dtype == sin.dtype, "expected cos and sin tensor have the same dtype")
+    _check(q.dtype == k.dtype and q.device == k.device, "q and k must have the same dtype and device")
+    _check(q.size(0) == k.size(0) and q.size(1) == k.size(1) and q.size(3) == k.size(3),
+           "q and k must agree in sequence length, batch size and head dimension")
+    _check(cos.dtype == torch.float32 or cos.dtype == q.dtype,
+           f"{name}: cos/sin must be float32 or have the dtype of the input")
+    _hp.require_gpu(cos, name)
+    _hp.require_gpu(sin, name)
+    c = cos.contiguous()
+    sn = sin.contiguous()
+    q_out = _new_output(q, transpose_output)
+    k_out = _new_output(k, transpose_output)
+    s, b, hq, d = q.shape
+    with _hp.device_guard(q):
+        rc = fn(q_out.data_ptr(), k_out.data_ptr(), q.data_ptr(), k.data_ptr(), c.data_ptr(), sn.data_ptr(), s, b, hq,
+                k.size(2), d, c.size(3), _hp.strides4(q), _hp.strides4(k), _hp.strides4(q_out), _hp.strides4(k_out),
+                _hp.dtype_code(q, name), _hp.dtype_code(c, name), _hp.stream_of(q))
+    _hp.check(rc, name)
+    return q_out, k_out
+
+
+def forward_cached_qk(q, k, cos, sin, transpose_output):
+    """(not in the reference module) ``forward_cached`` for q and k in one launch; k may have fewer heads."""
+    return _run_cached_qk("fused_rotary_positional_embedding.forward_cached_qk", _hp.lib().nhp_rope_cached_qk_fwd, q, k,
+                          cos, sin, transpose_output)
+
+
+def backward_cached_qk(grad_q, grad_k, cos, sin, transpose_output):
+    """(not in the reference module) ``backward_cached`` for the gradients of q and k in one launch."""
+    return _run_cached_qk("fused_rotary_positional_embedding.backward_cached_qk", _hp.lib().nhp_rope_cached_qk_bwd,
+                          grad_q, grad_k, cos, sin, transpose_output)

@@ -47,6 +47,8 @@ def _declare(lib):
         "nhp_softmax_batch_per_block": ([i64, i64, i64, i64], ci),
         "nhp_rope_cached_fwd": ([vp, vp, vp, vp, i64, i64, i64, i64, i64, p64, p64, ci, ci, vp], ci),
         "nhp_rope_cached_bwd": ([vp, vp, vp, vp, i64, i64, i64, i64, i64, p64, p64, ci, ci, vp], ci),
+        "nhp_rope_cached_qk_fwd": ([vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, p64, p64, p64, p64, ci, ci, vp], ci),
+        "nhp_rope_cached_qk_bwd": ([vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, p64, p64, p64, p64, ci, ci, vp], ci),
         "nhp_rope_freqs_fwd": ([vp, vp, vp, i64, i64, i64, i64, i64, p64, p64, ci, vp], ci),
         "nhp_rope_freqs_bwd": ([vp, vp, vp, i64, i64, i64, i64, i64, p64, p64, ci, vp], ci),
     }

@@ -81,3 +81,49 @@ def fused_apply_rotary_pos_emb_cached(
         transpose_output_memory: as in ``fused_apply_rotary_pos_emb``.
     """
     return FusedRoPECachedFunc.apply(t, cos_, sin_, transpose_output_memory)
+
+
+class FusedRoPEQKCachedFunc(torch.autograd.Function):
+    """RoPE of q and k from precomputed cos/sin tables in one kernel launch."""
+
+    @staticmethod
+    def forward(ctx, q, k, cos_, sin_, transpose_output_memory=False):
+        import fused_rotary_positional_embedding as ext
+
+        q_out, k_out = ext.forward_cached_qk(q, k, cos_, sin_, transpose_output_memory)
+        ctx.save_for_backward(cos_, sin_)
+        ctx.transpose_output_memory = transpose_output_memory
+        return q_out, k_out
+
+    @staticmethod
+    def backward(ctx, grad_q, grad_k):
+        import fused_rotary_positional_embedding as ext
+
+        cos_, sin_ = ctx.saved_tensors
+        gq, gk = ext.backward_cached_qk(grad_q, grad_k, cos_, sin_, ctx.transpose_output_memory)
+        return gq, gk, None, None, None
+
+
+def fused_apply_rotary_pos_emb_qk_cached(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    cos_: torch.Tensor,
+    sin_: torch.Tensor,
+    offset: int = 0,
+    transpose_output_memory: bool = False,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Fused counterpart of ``apply_rotary_pos_emb(q, k, cos, sin, offset)``
+    (megatron/model/positional_embeddings.py:110-126): both tensors in one launch.
+
+    Args:
+        q: [s, b, hq, d]; k: [s, b, hk, d] (any strides; hk may differ from hq).
+        cos_, sin_: [S, 1, 1, d2] tables with S >= offset + s and d2 <= d; features
+            d2..d pass through, so a partial rotary needs no slicing and no concatenation.
+        offset: position of the first row of q/k (decoding with a key/value cache).
+        transpose_output_memory: as in ``fused_apply_rotary_pos_emb``.
+    Returns (q_rotated, k_rotated).
+    """
+    s = q.shape[0]
+    cos_ = cos_[offset : offset + s, ...]
+    sin_ = sin_[offset : offset + s, ...]
+    return FusedRoPEQKCachedFunc.apply(q, k, cos_, sin_, transpose_output_memory)

@@ -206,6 +206,34 @@ int nhp_rope_cached_bwd(void* out, const void* in, const void* cos, const void* 
                         int dtype, int cs_dtype, void* stream);
 
 /*
+ * q and k of one attention layer rotated by one launch with the same tables:
+ * exactly nhp_rope_cached_fwd / _bwd applied to (q_out, q_in) and (k_out, k_in).
+ * q: [s, b, hq, d], k: [s, b, hk, d] (hk may differ from hq: grouped-query
+ * attention), both with their own element strides. This is the fused form of
+ * the reference's two-operand functions
+ *   apply_rotary_pos_emb / apply_rotary_pos_emb_torch
+ *   megatron/model/positional_embeddings.py:110-126
+ * and of the call site megatron/model/transformer.py:877-914, which calls the
+ * fused kernel once per tensor, slices [..., :d2] before and concatenates the
+ * pass-through features after; with d2 < d the copy happens inside the
+ * kernel. A position `offset` (KV-cache decoding, transformer.py:893-896) is
+ * expressed by passing cos + offset*d2 and sin + offset*d2.
+ */
+int nhp_rope_cached_qk_fwd(void* q_out, void* k_out, const void* q_in, const void* k_in,
+                           const void* cos, const void* sin,
+                           int64_t s, int64_t b, int64_t hq, int64_t hk, int64_t d, int64_t d2,
+                           const int64_t q_in_stride[4], const int64_t k_in_stride[4],
+                           const int64_t q_out_stride[4], const int64_t k_out_stride[4],
+                           int dtype, int cs_dtype, void* stream);
+
+int nhp_rope_cached_qk_bwd(void* q_out, void* k_out, const void* q_in, const void* k_in,
+                           const void* cos, const void* sin,
+                           int64_t s, int64_t b, int64_t hq, int64_t hk, int64_t d, int64_t d2,
+                           const int64_t q_in_stride[4], const int64_t k_in_stride[4],
+                           const int64_t q_out_stride[4], const int64_t k_out_stride[4],
+                           int dtype, int cs_dtype, void* stream);
+
+/*
  * Same, with c = cosf(freqs[s_idx, i]) and s = sinf(freqs[s_idx, i]) evaluated
  * on the device in fp32 and then converted to the data dtype.
  * freqs: contiguous fp32 [s, d2].

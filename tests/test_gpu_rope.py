@@ -169,3 +169,70 @@ def test_rope_full_size_properties(hotpath):
             # a wrong sign or index in backward would move rhs by about sqrt(N) instead
             noise = 2.0**-8 * (y.double() * gy.double()).pow(2).sum().item() ** 0.5
             assert abs(lhs - rhs) <= 8 * noise, (lhs, rhs, noise)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("shape", [(16, 2, 8, 8, 128, 128), (16, 2, 8, 2, 128, 32), (9, 3, 5, 1, 64, 16), (7, 2, 4, 4, 24, 8)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_rope_qk_single_launch_equals_two_calls(hotpath, shape, dtype):
+    """q and k (k possibly with fewer heads) through nhp_rope_cached_qk_* give the
+    bits of two nhp_rope_cached_* calls, forward and backward, for views of a
+    fused projection and for both output layouts."""
+    s, b, hq, hk, d, d2 = shape
+    buf = util.randn((s, b, hq + 2 * hk, d), dtype, seed=s + d).to(DEV)
+    q, k = buf[:, :, :hq], buf[:, :, hq : hq + hk]
+    cos, sin, _ = generic_tables(d2, s, dtype, seed=d2)
+    cos, sin = cos.to(DEV), sin.to(DEV)
+    L = hotpath.lib()
+    for backward in (False, True):
+        for transpose in (False, True):
+            want_q = util.abi_rope_cached(hotpath, q, cos, sin, backward, transpose)
+            want_k = util.abi_rope_cached(hotpath, k, cos, sin, backward, transpose)
+            got_q = util._rope_out(q, transpose)
+            got_k = util._rope_out(k, transpose)
+            fn = L.nhp_rope_cached_qk_bwd if backward else L.nhp_rope_cached_qk_fwd
+            rc = fn(got_q.data_ptr(), got_k.data_ptr(), q.data_ptr(), k.data_ptr(), cos.data_ptr(), sin.data_ptr(), s, b,
+                    hq, hk, d, d2, hotpath.strides4(q), hotpath.strides4(k), hotpath.strides4(got_q),
+                    hotpath.strides4(got_k), hotpath.dtype_code(q, "t"), hotpath.dtype_code(cos, "c"), None)
+            assert rc == 0
+            torch.cuda.synchronize()
+            assert torch.equal(util.raw_bits(got_q.cpu()), util.raw_bits(want_q.cpu()))
+            assert torch.equal(util.raw_bits(got_k.cpu()), util.raw_bits(want_k.cpu()))
+            # and against the oracle directly
+            assert torch.equal(util.raw_bits(got_k.cpu()), util.raw_bits(oracle.rope_cached(k.cpu(), cos.cpu(), sin.cpu(), backward, transpose)))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("offset", [0, 5])
+def test_fused_qk_function_matches_eager_apply_with_offset(dtype, offset):
+    """fused_apply_rotary_pos_emb_qk_cached == apply_rotary_pos_emb_torch on the rotary
+    slice + concatenation of the pass-through slice (what ParallelSelfAttention does),
+    including a position offset, forward and backward."""
+    from megatron.model.fused_rope import fused_apply_rotary_pos_emb_qk_cached
+    from megatron.model.positional_embeddings import RotaryEmbedding, apply_rotary_pos_emb_torch
+
+    sq, b, hq, hk, d, d2, smax = 24, 2, 8, 2, 128, 32, 64
+    rot = RotaryEmbedding(d2, smax, precision=dtype)
+    q = util.randn((sq, b, hq, d), dtype, seed=1)
+    k = util.randn((sq, b, hk, d), dtype, seed=2)
+    gq = util.randn((sq, b, hq, d), dtype, seed=3)
+    gk = util.randn((sq, b, hk, d), dtype, seed=4)
+    # eager reference on the CPU: rotate the first d2 features, pass the rest through
+    qe = q.clone().requires_grad_(True)
+    ke = k.clone().requires_grad_(True)
+    cos_c, sin_c = rot.cos_cached, rot.sin_cached
+    oq = torch.cat((fb.eager_rotary(qe[..., :d2], cos_c, sin_c, offset), qe[..., d2:]), dim=-1)
+    ok = torch.cat((fb.eager_rotary(ke[..., :d2], cos_c, sin_c, offset), ke[..., d2:]), dim=-1)
+    torch.autograd.backward([oq, ok], [gq, gk])
+    # and the two-operand eager function of the module agrees with that on the rotary slice
+    eq, ek = apply_rotary_pos_emb_torch(q[..., :d2], k[..., :d2], cos_c, sin_c, offset)
+    assert torch.equal(util.raw_bits(eq), util.raw_bits(oq[..., :d2].detach().contiguous()))
+    qd = q.to(DEV).requires_grad_(True)
+    kd = k.to(DEV).requires_grad_(True)
+    cos, sin = rot(qd, seq_len=smax)
+    fq, fk = fused_apply_rotary_pos_emb_qk_cached(qd, kd, cos, sin, offset)
+    torch.autograd.backward([fq, fk], [gq.to(DEV), gk.to(DEV)])
+    assert torch.equal(util.raw_bits(fq.detach().cpu()), util.raw_bits(oq.detach()))
+    assert torch.equal(util.raw_bits(fk.detach().cpu()), util.raw_bits(ok.detach()))
+    assert torch.equal(util.raw_bits(qd.grad.cpu()), util.raw_bits(qe.grad))
+    assert torch.equal(util.raw_bits(kd.grad.cpu()), util.raw_bits(ke.grad))
