@@ -689,6 +689,9 @@ static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t
         }                                                                  \
     } while (0)
 
+// The runtime rejects launches of 2^32 or more threads per grid dimension.
+static inline bool launch_fits(int64_t blocks, int threads) { return blocks * threads < ((int64_t)1 << 32); }
+
 static inline int launch_status()
 {
     return hipGetLastError() == hipSuccess ? NHP_OK : NHP_ERR_LAUNCH;
@@ -710,12 +713,14 @@ static int causal_fwd(void* y, const void* x, float scale, int64_t batches, int6
     {                                                                                      \
         using G = Geo<L_, K_, W_, kBlockWaves>;                                            \
         const uint32_t blocks = (uint32_t)((rows + G::kRowsPerBlock - 1) / G::kRowsPerBlock); \
+        if (!launch_fits(blocks, G::kThreads)) return NHP_ERR_SHAPE;                       \
         causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves><<<blocks, G::kThreads, p.lds, st>>>(    \
             yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, slopes, heads);            \
     }
         NHP_FOR_PLAN(p);
 #undef CALL
     } else {
+        if (!launch_fits(rows, kScalarThreads)) return NHP_ERR_SHAPE;
         scalar_fwd_kernel<DT, 0><<<(uint32_t)rows, kScalarThreads, 0, st>>>(
             yp, xp, nullptr, scale, (uint64_t)n, (uint64_t)n, 1, 0, window, slopes, heads);
     }
@@ -735,12 +740,14 @@ static int softmax_bwd(void* dx, const void* dy, const void* y, float scale, int
     {                                                                                      \
         using G = Geo<L_, K_, W_, kBlockWaves>;                                            \
         const uint32_t blocks = (uint32_t)((rows + G::kRowsPerBlock - 1) / G::kRowsPerBlock); \
+        if (!launch_fits(blocks, G::kThreads)) return NHP_ERR_SHAPE;                       \
         softmax_bwd_kernel<DT, L_, K_, W_, kBlockWaves, CAUSAL><<<blocks, G::kThreads, p.lds, st>>>( \
             dxp, dyp, yp, scale, (uint32_t)rows, (uint32_t)n, (uint32_t)rows_per_matrix, window); \
     }
         NHP_FOR_PLAN(p);
 #undef CALL
     } else {
+        if (!launch_fits(rows, kScalarThreads)) return NHP_ERR_SHAPE;
         scalar_bwd_kernel<DT, CAUSAL><<<(uint32_t)rows, kScalarThreads, 0, st>>>(
             dxp, dyp, yp, scale, (uint64_t)n, (uint64_t)rows_per_matrix, window);
     }
@@ -768,7 +775,7 @@ static int masked_fwd(void* y, const void* x, const uint8_t* mask, float scale, 
         const int64_t rb = (bq_rows + G::kRowsPerBlock - 1) / G::kRowsPerBlock;            \
         const uint32_t hpw = (uint32_t)tune("NHP_HPW", (int)pick_heads_per_wave(np));       \
         const uint32_t hgs = (uint32_t)((np + hpw - 1) / hpw);                             \
-        if (rb * hgs >= kMaxRows) return NHP_ERR_SHAPE;                                    \
+        if (rb * hgs >= kMaxRows || !launch_fits(rb * hgs, G::kThreads)) return NHP_ERR_SHAPE; \
         int64_t tile = tune("NHP_MASK_TILE", (int)((sq + G::kRowsPerBlock - 1) / G::kRowsPerBlock)); \
         if (tile < 1) tile = 1;                                                            \
         if (tile > rb) tile = rb;                                                          \
@@ -779,6 +786,7 @@ static int masked_fwd(void* y, const void* x, const uint8_t* mask, float scale, 
         NHP_FOR_PLAN(p);
 #undef CALL
     } else {
+        if (!launch_fits(b * np * sq, kScalarThreads)) return NHP_ERR_SHAPE;
         scalar_fwd_kernel<DT, 1><<<(uint32_t)(b * np * sq), kScalarThreads, 0, st>>>(
             yp, xp, mask, scale, (uint64_t)n, (uint64_t)sq, (uint64_t)np, per_batch, kNoWindow, nullptr, 1);
     }

@@ -310,3 +310,32 @@ def test_batch_per_block_table():
     for sk, w32, w64 in table:
         assert oracle.batch_per_block(sk, 32) == w32, sk
         assert oracle.batch_per_block(sk, 64) == w64, sk
+
+
+# ---------------------------------------------------------------------------
+# the reference's forward narrows `scale` to the input dtype; this build does not
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype,std,outliers", [(torch.bfloat16, 2.0, False), (torch.float16, 3.0, True)],
+                         ids=["bf16_causal_like", "fp16_with_60_outliers"])
+def test_scale_narrowing_quirk_is_small_and_quantified(dtype, std, outliers):
+    """scaled_upper_triang_masked_softmax.h:368 / scaled_masked_softmax.h:358 take the
+    forward scale as `input_t`: 1/sqrt(128) becomes 0.08837890625 in bf16 and fp16
+    (relative error 1.07e-4), while the reference's backward and its torch fallback
+    use the fp32 value, as this build does everywhere. The effect on a probability is
+    about 1.07e-4 * |z - z_max| relative: below one bf16 ulp on N(0,4) scores, and up
+    to about 2 fp16 ulp when +-60 outliers stretch z - z_max to ~10."""
+    scale = 1.0 / math.sqrt(128.0)
+    narrowed = float(torch.tensor(scale).to(dtype))
+    assert narrowed == 0.08837890625
+    assert abs(narrowed / scale - 1) < 1.1e-4
+    x = util.randn((4, 256, 256), dtype, seed=1, std=std)
+    if outliers:
+        g = torch.Generator().manual_seed(2)
+        hit = torch.rand(x.shape, generator=g) < 0.01
+        x = torch.where(hit, torch.where(torch.rand(x.shape, generator=g) < 0.5, -60.0, 60.0).to(dtype), x)
+    full = oracle.causal_softmax_fwd(x, scale)
+    narrow = oracle.causal_softmax_fwd(x, narrowed)
+    d = util.ulp_distance(full, narrow)
+    assert int(d.max()) <= (1 if dtype == torch.bfloat16 else 3)
+    # most elements do not move at all
+    assert (d == 0).float().mean().item() > (0.95 if dtype == torch.bfloat16 else 0.6)
