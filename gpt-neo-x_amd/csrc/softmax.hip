@@ -21,9 +21,11 @@
 // cancels in p, and keeps e out of the range where v_exp_f32 flushes to zero
 // down to 2^-190, so probabilities in the bf16 subnormal range are still produced.
 //
-// Masks are applied by index: in the causal kernels columns k > q are never
-// loaded and are written as zeros; in the padding-mask kernel a chunk whose 8
-// mask bytes are all 1 is not loaded.
+// Masks are applied by index: in the causal kernels only the columns of the
+// band max(0, q - window) <= k <= q are loaded (window = none: 0 <= k <= q),
+// everything else is written as zeros; an AliBi bias is computed from (q - k)
+// and the head's slope; in the padding-mask kernel a chunk whose 8 mask bytes
+// are all 1 is not loaded.
 
 #include "common.hpp"
 
