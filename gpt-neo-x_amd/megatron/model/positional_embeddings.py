@@ -8,39 +8,44 @@ import math
 import torch
 
 
-class RotaryEmbedding(torch.nn.Module):
-    """Precomputed cos/sin tables for rotary position embedding.
+def _rotary_angles(dim, seq_len, base):
+    """fp32 angles ``position * base^(-2j/dim)``; the two halves of the feature axis share them."""
+    inv_freq = 1.0 / (base ** (torch.arange(0, dim, 2).float() / dim))
+    positions = torch.arange(seq_len).type_as(inv_freq)
+    half = torch.einsum("i,j->ij", positions, inv_freq)
+    return inv_freq, torch.cat((half, half), dim=-1)
 
-    The tables are built once, in fp32, for ``max_seq_len`` positions and cast
-    to ``precision``; ``forward`` hands out the first ``seq_len`` rows on the
-    device of ``x``. The reference copies the host tables to the device on
-    every call; here each device's copy is made once and kept.
+
+class RotaryEmbedding(torch.nn.Module):
+    """cos / sin tables for rotary position embedding.
+
+    Built once in fp32 for ``max_seq_len`` positions, then cast to ``precision``;
+    ``forward`` returns the first ``seq_len`` rows on the device of ``x``. The
+    reference copies its host tables to the device on every call; here each
+    device gets its copy once.
+
+    Attributes kept from the reference: ``cos_cached``, ``sin_cached``
+    (``[max_seq_len, 1, 1, dim]`` in ``precision``), ``emb`` (fp32 angles of the same
+    shape), the buffer ``inv_freq`` (cast to ``precision``; in the state dict only
+    with ``save_inv_freqs``), ``dim``, ``base``, ``max_seq_len``, ``precision``.
     """
 
     def __init__(self, dim, max_seq_len, base=10000, precision=torch.half, save_inv_freqs=False):
         super().__init__()
-        self.seq_len_cached = None
-        self.precision = precision
-        self.max_seq_len = max_seq_len
-        self.base = base
         self.dim = dim
-
-        cos_cached, sin_cached, inv_freq = self._prepare_cache(max_seq_len, precision, base)
-        # as in the reference, the buffer that survives is the one cast to `precision`
+        self.base = base
+        self.max_seq_len = max_seq_len
+        self.precision = precision
+        self.seq_len_cached = None
+        self.cos_cached, self.sin_cached, inv_freq = self._prepare_cache(max_seq_len, precision, base)
         self.register_buffer("inv_freq", inv_freq, persistent=save_inv_freqs)
-        self.cos_cached = cos_cached
-        self.sin_cached = sin_cached
-        self._on_device = {}
+        self._per_device = {}
 
     def _prepare_cache(self, seq_len, precision, base):
-        inv_freq = 1.0 / (base ** (torch.arange(0, self.dim, 2).float() / self.dim))
-        t = torch.arange(seq_len).type_as(inv_freq)
-        freqs = torch.einsum("i,j->ij", t, inv_freq)
-        emb = torch.cat((freqs, freqs), dim=-1)
-        self.emb = emb.reshape(emb.size(0), 1, 1, emb.size(1))
-        cos_cached = emb.cos()[:, None, None, :]
-        sin_cached = emb.sin()[:, None, None, :]
-        return cos_cached.to(precision), sin_cached.to(precision), inv_freq.to(precision)
+        inv_freq, angles = _rotary_angles(self.dim, seq_len, base)
+        self.emb = angles.reshape(seq_len, 1, 1, angles.size(1))
+        shape4 = (slice(None), None, None, slice(None))
+        return angles.cos()[shape4].to(precision), angles.sin()[shape4].to(precision), inv_freq.to(precision)
 
     def get_emb(self):
         return self.emb.to(self.precision).cuda()
@@ -49,41 +54,45 @@ class RotaryEmbedding(torch.nn.Module):
         device = torch.device(device)
         if device == self.cos_cached.device:
             return self.cos_cached, self.sin_cached
-        key = str(device)
-        hit = self._on_device.get(key)
-        if hit is None or hit[0] is not self.cos_cached:
-            hit = (self.cos_cached, self.cos_cached.to(device), self.sin_cached.to(device))
-            self._on_device[key] = hit
-        return hit[1], hit[2]
+        entry = self._per_device.get(str(device))
+        if entry is None or entry[0] is not self.cos_cached:  # first use, or the host tables were replaced
+            entry = (self.cos_cached, self.cos_cached.to(device), self.sin_cached.to(device))
+            self._per_device[str(device)] = entry
+        return entry[1], entry[2]
 
     def forward(self, x, seq_dim=0, seq_len=None):
         if seq_len is None:
             seq_len = x.shape[seq_dim]
         assert seq_len <= self.max_seq_len
         cos, sin = self._tables_on(x.device)
-        if seq_len != self.max_seq_len:
-            return cos[:seq_len, ...], sin[:seq_len, ...]
-        return cos, sin
+        if seq_len == self.max_seq_len:
+            return cos, sin
+        return cos[:seq_len, ...], sin[:seq_len, ...]
 
 
 # rotary pos emb helpers:
 
 
 def rotate_half(x):
-    half = x.shape[-1] // 2
-    x1, x2 = x[..., :half], x[..., half:]
-    return torch.cat((-x2, x1), dim=x1.ndim - 1)
+    """``(-x2, x1)`` for ``x = (x1, x2)`` split in halves along the last dimension."""
+    mid = x.shape[-1] // 2
+    return torch.cat((-x[..., mid:], x[..., :mid]), dim=x.ndim - 1)
+
+
+def _rotate(t, cos, sin):
+    return (t * cos) + (rotate_half(t) * sin)
 
 
 def apply_rotary_pos_emb(q, k, cos, sin, offset: int = 0):
-    cos = cos[offset : q.shape[0] + offset, ...]
-    sin = sin[offset : q.shape[0] + offset, ...]
-    return (q * cos) + (rotate_half(q) * sin), (k * cos) + (rotate_half(k) * sin)
+    """Eager RoPE of q and k ``[s, b, h, d]`` with tables ``[S, 1, 1, d]``; row i of
+    q/k takes table row ``offset + i``."""
+    rows = slice(offset, q.shape[0] + offset)
+    cos, sin = cos[rows, ...], sin[rows, ...]
+    return _rotate(q, cos, sin), _rotate(k, cos, sin)
 
 
 def apply_rotary_pos_emb_torch(q, k, cos, sin, offset: int = 0):
-    # identical to apply_rotary_pos_emb; the reference keeps two names because
-    # its first variant is TorchScript-compiled and that fails for bf16
+    # the reference keeps two names: its first variant is TorchScript-compiled, which fails for bf16
     return apply_rotary_pos_emb(q, k, cos, sin, offset)
 
 
