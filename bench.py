@@ -17,6 +17,7 @@ the drop-in extension modules (which call libneox_hotpath.so):
   rope-qk-1.4b   rotary fwd+bwd on q,k [2048,8,16,128] bf16, rotary_pct 0.25, q and k in one launch
   mistral-window causal softmax fwd+bwd [64,8192,8192] bf16 with a 4096-key sliding window applied by index
   alibi-1.4b     causal softmax fwd+bwd [128,2048,2048] bf16 with the AliBi bias of 16 heads added in the kernel
+  rpe-bias-1.4b  causal softmax fwd+bwd [128,2048,2048] bf16 with a bias tensor [16,2048,2048] added in the kernel
 
 `value` is algorithmic bytes per step / wall time per step (inputs resident in
 HBM, K steps bracketed by device synchronisation). Algorithmic bytes: softmax
@@ -146,15 +147,19 @@ def make_workload(name, torch, dev):
                "scale": "1/sqrt(%d)" % d, "bytes_convention": "causal-min (reads of the lower triangle, dense writes)"}
         return step, kernel_bytes, dense, "causal_softmax_bwd", "bf16", cfg
 
-    if name in ("mistral-window", "alibi-1.4b"):
+    if name in ("mistral-window", "alibi-1.4b", "rpe-bias-1.4b"):
         from oracle import fallback_semantics as fb_
 
+        bias = None
         if name == "mistral-window":
             a, s, window, heads = 64, 8192, 4096, None
         else:
             a, s, window, heads = 128, 2048, None, 16
         scale = 1.0 / math.sqrt(128)
         slopes = None if heads is None else torch.tensor(fb_.alibi_slopes(heads), dtype=torch.float32, device=dev)
+        if name == "rpe-bias-1.4b":
+            slopes = None
+            bias = randn((heads, s, s), 77, torch.bfloat16, 1.0)
         x = torch.empty((a, s, s), dtype=torch.bfloat16, device=dev)
         dy = torch.empty_like(x)
         for i in range(0, a, 8):
@@ -164,13 +169,16 @@ def make_workload(name, torch, dev):
         band = sum(min(q, w) + 1 for q in range(s))  # keys read per matrix
         fwd_b = a * band * 2 + a * s * s * 2
         bwd_b = 2 * a * band * 2 + a * s * s * 2
+        if bias is not None:
+            fwd_b += heads * band * 2  # each head's bias triangle once; the batch re-reads it from cache
         kernel_bytes = {"causal_softmax_fwd": fwd_b, "causal_softmax_bwd": bwd_b}
 
         def step(t):
-            y = t.run("causal_softmax_fwd", lambda: causal_ext.forward(x, scale, window, slopes))
+            y = t.run("causal_softmax_fwd", lambda: causal_ext.forward(x, scale, window, slopes, bias))
             t.run("causal_softmax_bwd", lambda: causal_ext.backward(dy, y, scale, window))
 
-        cfg = {"workload": name, "scores": [a, s, s], "window": window, "alibi_heads": heads,
+        cfg = {"workload": name, "scores": [a, s, s], "window": window,
+               "alibi_heads": None if slopes is None else heads, "bias": None if bias is None else list(bias.shape),
                "bytes_convention": "reads of the attended band, dense writes"}
         return step, kernel_bytes, {}, "causal_softmax_bwd", "bf16", cfg
 

@@ -173,10 +173,12 @@ __device__ __forceinline__ uint32_t active_slots(const Band& band, int w)
 // ---------------------------------------------------------------------------
 // Causal forward
 // ---------------------------------------------------------------------------
-template <int DT, int L, int K, int W, int BW>
+// PER_HEAD = false compiles the per-head extras (bias tensor, AliBi) out of the
+// plain kernel, which then keeps its registers for loads in flight.
+template <int DT, int L, int K, int W, int BW, bool PER_HEAD>
 __global__ void __launch_bounds__((Geo<L, K, W, BW>::kThreads))
 causal_fwd_kernel(uint16_t* y, const uint16_t* x, float scale, uint32_t total_rows, uint32_t n, uint32_t window,
-                  const float* slopes, uint32_t heads)
+                  const float* slopes, const uint16_t* bias, uint32_t heads)
 {
     using G = Geo<L, K, W, BW>;
     __shared__ float lds[32];
@@ -206,10 +208,30 @@ causal_fwd_kernel(uint16_t* y, const uint16_t* x, float scale, uint32_t total_ro
         if ((act >> k & 1u) && col < band.hi && col + 8 > band.lo) raw[k] = load16_stream(xr + col);
     }
 
+    // Additive bias [heads, n, n] (e.g. a relative-position bias shared by the batch):
+    // added to the score in the storage dtype, as `scores += bias` does in eager torch.
+    if (PER_HEAD && bias != nullptr) {
+        const uint16_t* br = bias + ((size_t)(mat % heads) * n + q) * n;
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            const uint32_t col = chunk_col<L, W>(k, w, l);
+            if ((act >> k & 1u) && col < band.hi && col + 8 > band.lo) {
+                const u32x4 rb = load16(br + col);  // re-used by every batch entry: keep it cacheable
+                float f[8], g[8];
+                unpack8<DT>(raw[k], f);
+                unpack8<DT>(rb, g);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) f[j] = f[j] + g[j];
+                raw[k] = pack8<DT>(f);
+            }
+        }
+    }
+
     // AliBi: bias[q][k] = (-(q - k)) * slope in the storage dtype, added to the
     // score in the storage dtype (what `scores + alibi_matrix` does in eager torch)
+    const bool alibi = PER_HEAD && slopes != nullptr;
     float slope = 0.0f;
-    if (slopes != nullptr) slope = Half2<DT>::round(slopes[mat % heads]);
+    if (alibi) slope = Half2<DT>::round(slopes[mat % heads]);
 
     float z[K][8];
 #pragma unroll
@@ -218,7 +240,7 @@ causal_fwd_kernel(uint16_t* y, const uint16_t* x, float scale, uint32_t total_ro
             const uint32_t col = chunk_col<L, W>(k, w, l);
             float f[8];
             unpack8<DT>(raw[k], f);
-            if (slopes != nullptr) {
+            if (alibi) {
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     const float dist = Half2<DT>::round(-(float)((int)q - (int)(col + j)));
@@ -517,7 +539,7 @@ template <int DT, int MODE>
 __global__ void __launch_bounds__(kScalarThreads)
 scalar_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float scale,
                   uint64_t n, uint64_t sq, uint64_t np, int mask_per_batch, uint32_t window,
-                  const float* slopes, uint32_t heads)
+                  const float* slopes, const uint16_t* bias, uint32_t heads)
 {
     __shared__ float slots[4];
     const uint64_t row = blockIdx.x;
@@ -527,10 +549,12 @@ scalar_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
     const uint8_t* mrow = nullptr;
     uint64_t lo = 0, hi = n;
     float slope = 0.0f;
+    const uint16_t* br = nullptr;
     if (MODE == 0) {
         hi = q + 1;
         lo = (q > window) ? q - window : 0;
         if (slopes != nullptr) slope = Half2<DT>::round(slopes[(row / sq) % heads]);
+        if (bias != nullptr) br = bias + (((row / sq) % heads) * sq + q) * n;
     } else {
         const uint64_t bi = row / (sq * np);
         mrow = mask + (mask_per_batch ? (bi * sq + q) : q) * n;
@@ -538,6 +562,7 @@ scalar_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
     // scaled logit of column c (lo <= c < hi)
     auto logit = [&](uint64_t c) {
         float f = Half2<DT>::from_bits(xr[c]);
+        if (MODE == 0 && br != nullptr) f = Half2<DT>::round(f + Half2<DT>::from_bits(br[c]));
         if (MODE == 0 && slopes != nullptr) {
             const float dist = Half2<DT>::round(-(float)((int64_t)q - (int64_t)c));
             f = Half2<DT>::round(f + Half2<DT>::round(dist * slope));
@@ -704,27 +729,32 @@ constexpr uint32_t kNoWindow = 0xffffffffu;
 
 template <int DT>
 static int causal_fwd(void* y, const void* x, float scale, int64_t batches, int64_t n, uint32_t window,
-                      const float* slopes, uint32_t heads, hipStream_t st)
+                      const float* slopes, const void* bias, uint32_t heads, hipStream_t st)
 {
     const int64_t rows = batches * n;
     RowPlan p;
     uint16_t* yp = static_cast<uint16_t*>(y);
     const uint16_t* xp = static_cast<const uint16_t*>(x);
-    if (plan_row(n, kCausalFwd, p) && aligned16(x) && aligned16(y)) {
+    const uint16_t* bp = static_cast<const uint16_t*>(bias);
+    if (plan_row(n, kCausalFwd, p) && aligned16(x) && aligned16(y) && aligned16(bias)) {
 #define CALL(L_, K_, W_)                                                                   \
     {                                                                                      \
         using G = Geo<L_, K_, W_, kBlockWaves>;                                            \
         const uint32_t blocks = (uint32_t)((rows + G::kRowsPerBlock - 1) / G::kRowsPerBlock); \
         if (!launch_fits(blocks, G::kThreads)) return NHP_ERR_SHAPE;                       \
-        causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves><<<blocks, G::kThreads, p.lds, st>>>(    \
-            yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, slopes, heads);            \
+        if (slopes != nullptr || bp != nullptr)                                            \
+            causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves, true><<<blocks, G::kThreads, p.lds, st>>>(  \
+                yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, slopes, bp, heads);    \
+        else                                                                               \
+            causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves, false><<<blocks, G::kThreads, p.lds, st>>>( \
+                yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, nullptr, nullptr, 1);  \
     }
         NHP_FOR_PLAN(p);
 #undef CALL
     } else {
         if (!launch_fits(rows, kScalarThreads)) return NHP_ERR_SHAPE;
         scalar_fwd_kernel<DT, 0><<<(uint32_t)rows, kScalarThreads, 0, st>>>(
-            yp, xp, nullptr, scale, (uint64_t)n, (uint64_t)n, 1, 0, window, slopes, heads);
+            yp, xp, nullptr, scale, (uint64_t)n, (uint64_t)n, 1, 0, window, slopes, bp, heads);
     }
     return launch_status();
 }
@@ -790,7 +820,7 @@ static int masked_fwd(void* y, const void* x, const uint8_t* mask, float scale, 
     } else {
         if (!launch_fits(b * np * sq, kScalarThreads)) return NHP_ERR_SHAPE;
         scalar_fwd_kernel<DT, 1><<<(uint32_t)(b * np * sq), kScalarThreads, 0, st>>>(
-            yp, xp, mask, scale, (uint64_t)n, (uint64_t)sq, (uint64_t)np, per_batch, kNoWindow, nullptr, 1);
+            yp, xp, mask, scale, (uint64_t)n, (uint64_t)sq, (uint64_t)np, per_batch, kNoWindow, nullptr, nullptr, 1);
     }
     return launch_status();
 }
@@ -804,26 +834,29 @@ extern "C" {
 int64_t nhp_softmax_max_resident_row(void) { return kMaxResidentRow; }
 
 int nhp_causal_softmax_ex_fwd(void* y, const void* x, float scale, int64_t attn_batches, int64_t seq_len,
-                              int64_t window, const float* alibi_slopes, int64_t heads, int dtype, void* stream)
+                              int64_t window, const float* alibi_slopes, const void* bias, int64_t heads,
+                              int dtype, void* stream)
 {
     if (dtype != NHP_F16 && dtype != NHP_BF16) return NHP_ERR_DTYPE;
     if (attn_batches < 0 || seq_len < 0) return NHP_ERR_SHAPE;
-    if (alibi_slopes != nullptr && (heads < 1 || attn_batches % heads != 0)) return NHP_ERR_SHAPE;
+    const bool per_head = alibi_slopes != nullptr || bias != nullptr;
+    if (per_head && (heads < 1 || attn_batches % heads != 0)) return NHP_ERR_SHAPE;
+    if (bias != nullptr && (bias == y)) return NHP_ERR_ALIAS;
     if (attn_batches == 0 || seq_len == 0) return NHP_OK;
     if (attn_batches > kMaxRows / seq_len - 1) return NHP_ERR_SHAPE;
     if (!x || !y) return NHP_ERR_NULL;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const uint32_t win = (window < 0 || window >= seq_len) ? kNoWindow : (uint32_t)window;
-    const uint32_t hd = alibi_slopes ? (uint32_t)heads : 1u;
+    const uint32_t hd = per_head ? (uint32_t)heads : 1u;
     return dtype == NHP_BF16
-               ? causal_fwd<NHP_BF16>(y, x, scale, attn_batches, seq_len, win, alibi_slopes, hd, st)
-               : causal_fwd<NHP_F16>(y, x, scale, attn_batches, seq_len, win, alibi_slopes, hd, st);
+               ? causal_fwd<NHP_BF16>(y, x, scale, attn_batches, seq_len, win, alibi_slopes, bias, hd, st)
+               : causal_fwd<NHP_F16>(y, x, scale, attn_batches, seq_len, win, alibi_slopes, bias, hd, st);
 }
 
 int nhp_causal_softmax_fwd(void* y, const void* x, float scale, int64_t attn_batches, int64_t seq_len,
                            int dtype, void* stream)
 {
-    return nhp_causal_softmax_ex_fwd(y, x, scale, attn_batches, seq_len, -1, nullptr, 1, dtype, stream);
+    return nhp_causal_softmax_ex_fwd(y, x, scale, attn_batches, seq_len, -1, nullptr, nullptr, 1, dtype, stream);
 }
 
 int nhp_causal_softmax_ex_bwd(void* dx, const void* dy, const void* y, float scale, int64_t attn_batches,

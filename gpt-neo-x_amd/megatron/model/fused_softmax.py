@@ -19,7 +19,10 @@ all of it widening:
   caller otherwise does with tensors: ``sliding_window_width`` (the reference's
   causal kernel never looks at the mask, so a sliding window is lost on its
   fused branch) and ``alibi_slopes`` (the AliBi bias is formed inside the kernel
-  instead of by a separate ``scores + alibi_matrix`` pass). Both default to off.
+  instead of by a separate ``scores + alibi_matrix`` pass). Both default to off;
+* ``forward(input, mask, bias=None)``: an optional additive bias ``[1, np, sq, sk]``
+  (the relative-position bias the caller adds with ``attention_scores += rpe``)
+  is read by the causal kernel instead of being added in a pass of its own.
 """
 import enum
 
@@ -44,17 +47,18 @@ class ScaledUpperTriangMaskedSoftmax(torch.autograd.Function):
     """``softmax(scale * x)`` over the lower triangle of ``[attn_batches, sq, sk]``
     scores (zeros above the diagonal), one kernel forward and one backward.
 
-    ``window`` and ``alibi_slopes`` are the optional index-only extras described
-    in the module docstring; the reference signature is ``apply(inputs, scale)``.
+    ``window``, ``alibi_slopes`` and ``bias`` are the optional extras described in
+    the module docstring; the reference signature is ``apply(inputs, scale)``.
     """
 
     @staticmethod
-    def forward(ctx, inputs, scale, window=None, alibi_slopes=None):
+    def forward(ctx, inputs, scale, window=None, alibi_slopes=None, bias=None):
         import scaled_upper_triang_masked_softmax_cuda as kernels
 
         factor = _scale_tensor(scale)
-        out = kernels.forward(inputs, factor[0], window, alibi_slopes)
+        out = kernels.forward(inputs, factor[0], window, alibi_slopes, bias)
         ctx.window = window
+        ctx.bias_shape = None if bias is None else tuple(bias.shape)
         ctx.save_for_backward(out, factor)
         return out
 
@@ -65,7 +69,12 @@ class ScaledUpperTriangMaskedSoftmax(torch.autograd.Function):
         out, factor = ctx.saved_tensors
         # in place on output_grads, like the reference kernel
         grad = kernels.backward(output_grads, out, factor[0], ctx.window)
-        return grad, None, None, None
+        grad_bias = None
+        if ctx.bias_shape is not None and ctx.needs_input_grad[4]:
+            # the bias is shared by the batch: its gradient is the batch sum of the score gradient
+            heads, sq, sk = ctx.bias_shape[-3:]
+            grad_bias = grad.view(-1, heads, sq, sk).sum(dim=0).view(ctx.bias_shape)
+        return grad, None, None, None, grad_bias
 
 
 class ScaledMaskedSoftmax(torch.autograd.Function):
@@ -135,10 +144,11 @@ class FusedScaleMaskSoftmax(nn.Module):
             self.register_buffer("alibi_slopes", alibi_slopes.detach().float().clone(), persistent=False)
 
     # ------------------------------------------------------------------ dispatch
-    def forward(self, input, mask):
+    def forward(self, input, mask, bias=None):
         assert input.dim() == 4  # [b, np, sq, sk]
-        fused = self.is_kernel_available(mask, *input.size())
-        return self.forward_fused_softmax(input, mask) if fused else self.forward_torch_softmax(input, mask)
+        if self.is_kernel_available(mask, *input.size()):
+            return self.forward_fused_softmax(input, mask, bias)
+        return self.forward_torch_softmax(input, mask, bias)
 
     def is_kernel_available(self, mask, b, np, sq, sk):
         """The reference's conditions (fused_softmax.py:148-168) without ``sk <= 2048``."""
@@ -158,10 +168,12 @@ class FusedScaleMaskSoftmax(nn.Module):
         return scaled_masked_softmax_cuda.get_batch_per_block(sq, sk, b, np)
 
     # ------------------------------------------------------------------ branches
-    def forward_fused_softmax(self, input, mask):
+    def forward_fused_softmax(self, input, mask, bias=None):
         b, np, sq, sk = input.size()
         factor = 1.0 if self.scale is None else self.scale
         if not self.upper_triang_mask_fusion:
+            if bias is not None:
+                input = input + bias
             if self.alibi_slopes is not None:
                 input = self._add_alibi(input)
             return ScaledMaskedSoftmax.apply(input, mask, factor)
@@ -172,10 +184,14 @@ class FusedScaleMaskSoftmax(nn.Module):
             slopes = slopes.to(input.device)
         # the kernel takes [attn_batches, sq, sk]; the causal mask is implied by the indices
         flat = input.view(b * np, sq, sk)
-        probs = ScaledUpperTriangMaskedSoftmax.apply(flat, factor, self.sliding_window_width, slopes)
+        if bias is not None:
+            assert bias.shape[-3:] == (np, sq, sk) and bias.numel() == np * sq * sk, "bias must be [1, np, sq, sk]"
+        probs = ScaledUpperTriangMaskedSoftmax.apply(flat, factor, self.sliding_window_width, slopes, bias)
         return probs.view(b, np, sq, sk)
 
-    def forward_torch_softmax(self, input, mask):
+    def forward_torch_softmax(self, input, mask, bias=None):
+        if bias is not None:
+            input = input + bias
         if self.alibi_slopes is not None:
             input = self._add_alibi(input)
         widen = self.input_in_float16 and self.softmax_in_fp32

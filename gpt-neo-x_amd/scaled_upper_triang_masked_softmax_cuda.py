@@ -11,18 +11,21 @@ from megatron.fused_kernels import _hotpath as _hp
 _HALF = (torch.float16, torch.bfloat16)
 
 
-def forward(input, scale_factor, window=None, alibi_slopes=None):
+def forward(input, scale_factor, window=None, alibi_slopes=None, bias=None):
     """softmax(scale * input) under an upper-triangular mask.
 
     input: [attn_batches, seq_len, seq_len] fp16/bf16 on the GPU. Returns a new
     tensor of the same shape and dtype (requires_grad False). Checks follow
     scaled_upper_triang_masked_softmax.cpp:31-39; seq_len is not limited to 2048.
 
-    Two optional arguments go beyond the reference function:
+    Three optional arguments go beyond the reference function:
     window: sliding-window width; row q attends to keys q-window..q only.
     alibi_slopes: fp32 tensor [heads] on the GPU (attn_batches % heads == 0);
         the AliBi bias -(q-k)*slope is added to the scores in the storage dtype
         before the softmax, as `scores + alibi_matrix` would.
+    bias: [heads, seq_len, seq_len] tensor of the input's dtype (attn_batches %
+        heads == 0), added to the scores in the storage dtype first, as
+        `scores += bias` would (e.g. a relative-position bias shared by the batch).
     """
     if input.dim() != 3:
         raise RuntimeError("expected 3D tensor")
@@ -42,10 +45,24 @@ def forward(input, scale_factor, window=None, alibi_slopes=None):
         slopes_ptr, heads = alibi_slopes.data_ptr(), alibi_slopes.numel()
         if heads == 0 or x.size(0) % heads != 0:
             raise RuntimeError("attn_batches must be a multiple of the number of AliBi slopes")
+    bias_ptr = None
+    if bias is not None:
+        if bias.dim() == 4 and bias.size(0) == 1:
+            bias = bias[0]
+        if bias.dim() != 3 or bias.size(1) != x.size(1) or bias.size(2) != x.size(2) or bias.dtype != x.dtype:
+            raise RuntimeError("bias must be [heads, seq_len, seq_len] in the dtype of the input")
+        _hp.require_gpu(bias, "scaled_upper_triang_masked_softmax_cuda.forward")
+        if alibi_slopes is not None and bias.size(0) != heads:
+            raise RuntimeError("bias and alibi_slopes must have the same number of heads")
+        bias = bias.contiguous()
+        bias_ptr, heads = bias.data_ptr(), bias.size(0)
+        if heads == 0 or x.size(0) % heads != 0:
+            raise RuntimeError("attn_batches must be a multiple of the number of bias heads")
     with _hp.device_guard(x):
         rc = _hp.lib().nhp_causal_softmax_ex_fwd(
             y.data_ptr(), x.data_ptr(), float(scale_factor), x.size(0), x.size(1),
-            -1 if window is None else int(window), slopes_ptr, heads, _hp.dtype_code(x, "forward"), _hp.stream_of(x))
+            -1 if window is None else int(window), slopes_ptr, bias_ptr, heads, _hp.dtype_code(x, "forward"),
+            _hp.stream_of(x))
     _hp.check(rc, "scaled_upper_triang_masked_softmax_cuda.forward")
     return y
 

@@ -91,8 +91,8 @@ int nhp_causal_softmax_bwd(void* dx, const void* dy, const void* y, float scale,
                            int dtype, void* stream);
 
 /*
- * Causal softmax with the two index-only generalisations its caller needs, so
- * that neither a mask tensor nor a bias tensor has to be read or written:
+ * Causal softmax with the generalisations its caller needs, so that no mask
+ * tensor is read and no biased copy of the scores is written:
  *
  *  window >= 0: sliding-window attention. Row q attends to columns
  *      max(0, q - window) <= k <= q (the mask megatron/utils.py:67-80 builds
@@ -105,6 +105,11 @@ int nhp_causal_softmax_bwd(void* dx, const void* dy, const void* y, float scale,
  *      eager torch (megatron/model/positional_embeddings.py:129-257, applied
  *      at megatron/model/transformer.py:584-585) before the softmax sees the
  *      scores. slopes: `heads` fp32 values on the device.
+ *  bias != NULL: an additive bias [heads, seq_len, seq_len] in the storage
+ *      dtype, shared by the batch (the relative-position bias added at
+ *      megatron/model/transformer.py:580-582 as `attention_scores += rpe`):
+ *      the score becomes x (+) bias[hd, q, k], rounded to the storage dtype,
+ *      before AliBi (if any) and the softmax. Only the attended band is read.
  *
  * The backward of the AliBi variant is the plain (windowed) backward: the bias
  * is constant.
@@ -116,8 +121,8 @@ int nhp_causal_softmax_bwd(void* dx, const void* dy, const void* y, float scale,
  */
 int nhp_causal_softmax_ex_fwd(void* y, const void* x, float scale,
                               int64_t attn_batches, int64_t seq_len,
-                              int64_t window, const float* alibi_slopes, int64_t heads,
-                              int dtype, void* stream);
+                              int64_t window, const float* alibi_slopes, const void* bias,
+                              int64_t heads, int dtype, void* stream);
 
 int nhp_causal_softmax_ex_bwd(void* dx, const void* dy, const void* y, float scale,
                               int64_t attn_batches, int64_t seq_len, int64_t window,

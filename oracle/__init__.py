@@ -45,7 +45,7 @@ def lib():
         L = ctypes.CDLL(_LIB_PATH)
         i64, vp, f32, ci = ctypes.c_int64, ctypes.c_void_p, ctypes.c_float, ctypes.c_int
         L.oracle_causal_softmax_fwd.argtypes = [vp, vp, f32, i64, i64, ci]
-        L.oracle_causal_softmax_ex_fwd.argtypes = [vp, vp, f32, i64, i64, i64, vp, i64, ci]
+        L.oracle_causal_softmax_ex_fwd.argtypes = [vp, vp, f32, i64, i64, i64, vp, vp, i64, ci]
         L.oracle_softmax_ex_bwd.argtypes = [vp, vp, vp, f32, i64, i64, i64, ci, i64, ci]
         L.oracle_masked_softmax_fwd.argtypes = [vp, vp, vp, f32, i64, i64, i64, i64, i64, ci]
         L.oracle_softmax_bwd.argtypes = [vp, vp, vp, f32, i64, i64, i64, ci, ci]
@@ -75,9 +75,10 @@ def _cpu_contig(t):
     return t.contiguous()
 
 
-def causal_softmax_fwd(x, scale, window=None, alibi_slopes=None):
+def causal_softmax_fwd(x, scale, window=None, alibi_slopes=None, bias=None):
     """x: [attn_batches, s, s] fp16/bf16 -> probabilities, same shape and dtype.
-    window: sliding-window width or None; alibi_slopes: fp32 [heads] or None."""
+    window: sliding-window width or None; alibi_slopes: fp32 [heads] or None;
+    bias: [heads, s, s] in x.dtype or None."""
     assert x.dim() == 3 and x.size(1) == x.size(2)
     x = _cpu_contig(x)
     y = torch.empty_like(x)
@@ -86,8 +87,15 @@ def causal_softmax_fwd(x, scale, window=None, alibi_slopes=None):
         alibi_slopes = _cpu_contig(alibi_slopes.float())
         sl_ptr, heads = alibi_slopes.data_ptr(), alibi_slopes.numel()
         assert x.size(0) % heads == 0
+    b_ptr = None
+    if bias is not None:
+        bias = _cpu_contig(bias)
+        assert bias.dtype == x.dtype and bias.shape[1:] == x.shape[1:]
+        assert alibi_slopes is None or bias.size(0) == heads
+        b_ptr, heads = bias.data_ptr(), bias.size(0)
+        assert x.size(0) % heads == 0
     _check(lib().oracle_causal_softmax_ex_fwd(y.data_ptr(), x.data_ptr(), float(scale), x.size(0), x.size(1),
-                                              -1 if window is None else int(window), sl_ptr, heads,
+                                              -1 if window is None else int(window), sl_ptr, b_ptr, heads,
                                               _DT[x.dtype]), "causal_softmax_fwd")
     return y
 

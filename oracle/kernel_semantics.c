@@ -175,10 +175,12 @@ static void softmax_row(float* z, int64_t n)
  *     megatron/model/positional_embeddings.py:219-257 is added to the scores
  *     first, in the storage dtype: a = dt(-(q-k)) (*) dt(slope[head]),
  *     x' = x (+) a, head = batch index % heads (transformer.py:584-585 adds it
- *     to the [b, np, sq, sk] scores before scale_mask_softmax).
+ *     to the [b, np, sq, sk] scores before scale_mask_softmax);
+ *   bias != NULL: `attention_scores += rpe` (transformer.py:580-582), a
+ *     [heads, s, s] tensor in the storage dtype added (rounded) before AliBi.
  */
 int oracle_causal_softmax_ex_fwd(void* y, const void* x, float scale, int64_t batches, int64_t s,
-                                 int64_t window, const float* slopes, int64_t heads, int dt)
+                                 int64_t window, const float* slopes, const void* bias, int64_t heads, int dt)
 {
     if (dt != DT_F16 && dt != DT_BF16) return -1;
     float* z = (float*)malloc(sizeof(float) * (size_t)(s > 0 ? s : 1));
@@ -190,6 +192,8 @@ int oracle_causal_softmax_ex_fwd(void* y, const void* x, float scale, int64_t ba
             const int64_t lo = (window >= 0 && q > window) ? q - window : 0;
             for (int64_t k = lo; k <= q; ++k) {
                 float v = load_elem(x, base + k, dt);
+                /* attention_scores += rpe (transformer.py:580-582): bias [heads, s, s] in the storage dtype */
+                if (bias) v = add_t(v, load_elem(bias, ((a % heads) * s + q) * s + k, dt), dt);
                 if (slopes) {
                     const float dist = round_to(-(float)(q - k), dt);
                     v = add_t(v, mul_t(dist, slope, dt), dt);
@@ -208,7 +212,7 @@ int oracle_causal_softmax_ex_fwd(void* y, const void* x, float scale, int64_t ba
 
 int oracle_causal_softmax_fwd(void* y, const void* x, float scale, int64_t batches, int64_t s, int dt)
 {
-    return oracle_causal_softmax_ex_fwd(y, x, scale, batches, s, -1, NULL, 1, dt);
+    return oracle_causal_softmax_ex_fwd(y, x, scale, batches, s, -1, NULL, NULL, 1, dt);
 }
 
 /*

@@ -16,11 +16,12 @@ DEV = "cuda"
 DTYPES = [torch.bfloat16, torch.float16]
 
 
-def abi_ex_fwd(hp, x, scale, window, slopes):
+def abi_ex_fwd(hp, x, scale, window, slopes, bias=None):
     y = torch.empty_like(x)
+    heads = slopes.numel() if slopes is not None else bias.size(0) if bias is not None else 1
     rc = hp.lib().nhp_causal_softmax_ex_fwd(
         y.data_ptr(), x.data_ptr(), scale, x.size(0), x.size(1), -1 if window is None else window,
-        None if slopes is None else slopes.data_ptr(), 1 if slopes is None else slopes.numel(),
+        None if slopes is None else slopes.data_ptr(), None if bias is None else bias.data_ptr(), heads,
         hp.dtype_code(x, "t"), None)
     assert rc == 0, hp.lib().nhp_status_string(rc)
     return y
@@ -105,3 +106,55 @@ def test_module_with_window_and_alibi(dtype):
                                   fb.fill_masked_with_dtype_min, True, scale)
     ref = plain(alibi.to(DEV)(x.to(DEV)), mask)
     util.assert_ulp_close(y.detach().cpu(), ref.cpu(), 2, "fused vs eager AliBi + torch softmax")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
+@pytest.mark.parametrize("s,window,with_alibi", [(64, None, False), (1024, None, True), (2048, 300, False), (1001, None, False)])
+def test_additive_bias_forward_vs_oracle(hotpath, dtype, s, window, with_alibi):
+    import scaled_upper_triang_masked_softmax_cuda as ext
+
+    b, heads, scale = 2, 4, 0.125
+    x = util.randn((b * heads, s, s), dtype, seed=s, std=2.0)
+    bias = util.randn((heads, s, s), dtype, seed=s + 1, std=1.5)
+    masked = fb.causal_mask(s, sliding_window_width=window)[0, 0]
+    slopes = torch.tensor(fb.alibi_slopes(heads), dtype=torch.float32) if with_alibi else None
+    clean = oracle.causal_softmax_fwd(x, scale, window=window, alibi_slopes=slopes, bias=bias)
+    # whatever lies outside the band, in the scores or in the bias, must not reach the result
+    x[:, masked] = float("nan")
+    bias[:, masked] = float("inf")
+    want = oracle.causal_softmax_fwd(x, scale, window=window, alibi_slopes=slopes, bias=bias)
+    assert torch.equal(util.raw_bits(clean), util.raw_bits(want))
+    got = ext.forward(x.to(DEV), scale, window, None if slopes is None else slopes.to(DEV), bias.to(DEV)).cpu()
+    assert int(util.raw_bits(got)[:, masked].abs().max()) == 0
+    util.assert_ulp_close(got, want, 2, "bias fwd")
+    via_abi = abi_ex_fwd(hotpath, x.to(DEV), scale, window, None if slopes is None else slopes.to(DEV), bias.to(DEV)).cpu()
+    assert torch.equal(util.raw_bits(via_abi), util.raw_bits(got))
+
+
+def test_module_with_relative_position_bias_and_its_gradient():
+    """FusedScaleMaskSoftmax(input, mask, bias): probabilities and the gradients of the
+    scores and of the (batch-shared, learned) bias against autograd through the unfused path."""
+    from megatron.model.fused_softmax import FusedScaleMaskSoftmax, SoftmaxFusionTypes as T
+
+    dtype = torch.bfloat16
+    b, np_, s, scale = 3, 4, 512, 0.125
+    x = util.randn((b, np_, s, s), dtype, seed=1, std=2.0)
+    rpe = util.randn((1, np_, s, s), dtype, seed=2, std=1.0)
+    dy = util.randn((b, np_, s, s), dtype, seed=3)
+    mask = fb.causal_mask(s, DEV)
+    out = {}
+    for name, fusion in (("fused", T.upper_triang), ("plain", T.none)):
+        m = FusedScaleMaskSoftmax(False, True, fusion, fb.fill_masked_with_dtype_min, True, scale)
+        xd = x.to(DEV).requires_grad_(True)
+        bd = rpe.to(DEV).requires_grad_(True)
+        y = m(xd, mask, bd)
+        y.backward(dy.to(DEV).clone())
+        out[name] = (y.detach().cpu(), xd.grad.float().cpu(), bd.grad.float().cpu())
+    want = oracle.causal_softmax_fwd(x.view(-1, s, s), scale, bias=rpe[0]).view(b, np_, s, s)
+    util.assert_ulp_close(out["fused"][0], want, 2, "fwd vs oracle")
+    util.assert_ulp_close(out["fused"][0], out["plain"][0], 2, "fwd vs unfused")
+    eps = 2.0**-8
+    for i, what in ((1, "dx"), (2, "dbias")):
+        f, p = out["fused"][i], out["plain"][i]
+        assert (f - p).norm().item() <= 4 * eps * p.norm().item(), what
+    assert out["fused"][2].shape == (1, np_, s, s)

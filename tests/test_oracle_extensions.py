@@ -141,3 +141,21 @@ def test_module_torch_path_with_window_and_alibi(dtype, fp16, bf16):
     want = oracle.causal_softmax_fwd(x.view(-1, s, s), scale, window=window, alibi_slopes=slopes).view(b, np_, s, s)
     util.assert_ulp_close(y, want, 1, "torch path vs oracle")
     assert "alibi_slopes" not in m.state_dict()
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_additive_bias_equals_eager_add_then_plain_softmax(dtype):
+    """softmax_bias(x, bias) == softmax(x + bias) with the sum formed by torch in the
+    storage dtype (`attention_scores += rpe`), the bias being shared by the batch and
+    indexed by head; combined with AliBi the bias comes first."""
+    b, heads, s, scale = 3, 4, 40, 0.3
+    x = util.randn((b, heads, s, s), dtype, seed=1, std=2.0)
+    bias = util.randn((1, heads, s, s), dtype, seed=2, std=1.5)
+    fused = oracle.causal_softmax_fwd(x.view(-1, s, s), scale, bias=bias[0])
+    eager = oracle.causal_softmax_fwd((x + bias).view(-1, s, s), scale)
+    assert torch.equal(util.raw_bits(fused), util.raw_bits(eager))
+    assert not torch.equal(util.raw_bits(fused), util.raw_bits(oracle.causal_softmax_fwd(x.view(-1, s, s), scale)))
+    slopes = torch.tensor(fb.alibi_slopes(heads), dtype=torch.float32)
+    both = oracle.causal_softmax_fwd(x.view(-1, s, s), scale, window=9, alibi_slopes=slopes, bias=bias[0])
+    eager = oracle.causal_softmax_fwd(fb.alibi_add(x + bias, slopes).view(-1, s, s), scale, window=9)
+    assert torch.equal(util.raw_bits(both), util.raw_bits(eager))
