@@ -14,6 +14,8 @@ the drop-in extension modules (which call libneox_hotpath.so):
   masked-c3      padding-masked softmax fwd+bwd [16,32,1024,2048] fp16
   rope-c4        rotary fwd+bwd on q,k [4096,4,32,128] bf16, rotary_pct 1.0 and 0.25
   llama2-7b-c5   rotary on q,k [8192,2,32,128] + causal softmax fwd+bwd [64,8192,8192] bf16
+  rope-c4-qkv-view  rotary fwd+bwd on q,k given as views of one fused [4096,4,32,3*128] bf16 buffer (the layout
+                 the attention layer slices q and k from), rotary_pct 1.0
   rope-qk-1.4b   rotary fwd+bwd on q,k [2048,8,16,128] bf16, rotary_pct 0.25, q and k in one launch
   mistral-window causal softmax fwd+bwd [64,8192,8192] bf16 with a 4096-key sliding window applied by index
   alibi-1.4b     causal softmax fwd+bwd [128,2048,2048] bf16 with the AliBi bias of 16 heads added in the kernel
@@ -148,7 +150,7 @@ def make_workload(name, torch, dev):
         return step, kernel_bytes, dense, "causal_softmax_bwd", "bf16", cfg
 
     if name in ("mistral-window", "alibi-1.4b", "rpe-bias-1.4b"):
-        from oracle import fallback_semantics as fb_
+        from megatron.model.positional_embeddings import AliBi
 
         bias = None
         if name == "mistral-window":
@@ -156,7 +158,7 @@ def make_workload(name, torch, dev):
         else:
             a, s, window, heads = 128, 2048, None, 16
         scale = 1.0 / math.sqrt(128)
-        slopes = None if heads is None else torch.tensor(fb_.alibi_slopes(heads), dtype=torch.float32, device=dev)
+        slopes = None if heads is None else AliBi(heads, mp_size=1, mp_rank=0).slopes.float().to(dev)
         if name == "rpe-bias-1.4b":
             slopes = None
             bias = randn((heads, s, s), 77, torch.bfloat16, 1.0)
@@ -224,6 +226,36 @@ def make_workload(name, torch, dev):
 
         cfg = {"workload": name, "qk": [s, b, h, d], "rotary_dim": d2}
         return step, kernel_bytes, {}, "rope_qk_fwd", "bf16", cfg
+
+    if name == "rope-c4-qkv-view":
+        s, b, h, d, d2 = 4096, 4, 32, 128, 128
+        sets = []
+        for i in range(3):  # rotate through distinct buffers
+            qkv = randn((s, b, h, 3 * d), 80 + i, torch.bfloat16)
+            dqkv = randn((s, b, h, 3 * d), 90 + i, torch.bfloat16)
+            cos, sin = RotaryEmbedding(d2, s, base=10000, precision=torch.bfloat16)(qkv, seq_len=s)
+            sets.append((qkv[..., :d], qkv[..., d:2 * d], dqkv[..., :d], dqkv[..., d:2 * d], cos.contiguous(), sin.contiguous()))
+        rb = rope_bytes(s, b, h, d, d2)
+        kernel_bytes = {"rope_fwd_view": 2 * rb, "rope_bwd_view": 2 * rb}
+        state = {"i": 0}
+
+        def step(t):
+            q, k, dq, dk, cos, sin = sets[state["i"] % len(sets)]
+            state["i"] += 1
+
+            def f():
+                rope_ext.forward_cached(q, cos, sin, False)
+                rope_ext.forward_cached(k, cos, sin, False)
+
+            def bw():
+                rope_ext.backward_cached(dq, cos, sin, False)
+                rope_ext.backward_cached(dk, cos, sin, False)
+
+            t.run("rope_fwd_view", f)
+            t.run("rope_bwd_view", bw)
+
+        cfg = {"workload": name, "qk": [s, b, h, d], "qk_strides": list(sets[0][0].stride()), "rotary_dim": d2}
+        return step, kernel_bytes, {}, "rope_fwd_view", "bf16", cfg
 
     if name == "rope-c4":
         s, b, h, d = 4096, 4, 32, 128

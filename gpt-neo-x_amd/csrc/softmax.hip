@@ -140,16 +140,27 @@ __device__ __forceinline__ void locate_row(uint32_t block, uint32_t rows_per_mat
 }
 
 // The columns of row q that take part in a causal softmax: [lo, hi) with
-// hi = q + 1 and lo = max(0, q - window) (window = 0xffffffff: no lower bound).
+// hi = min(q + 1, limit) and lo = max(0, q - window) (window = 0xffffffff: no
+// lower bound; limit = the number of real keys of the row's batch entry).
+// hi <= lo is an empty band: the row is written as zeros.
 struct Band {
     uint32_t lo, hi;
 };
-__device__ __forceinline__ Band causal_band(uint32_t q, uint32_t window, bool ok)
+__device__ __forceinline__ Band causal_band(uint32_t q, uint32_t window, bool ok, uint32_t limit = 0xffffffffu)
 {
     Band b;
-    b.hi = ok ? q + 1 : 0;
+    b.hi = ok ? min(q + 1, limit) : 0;
     b.lo = (ok && q > window) ? q - window : 0;
+    if (b.hi <= b.lo) b.hi = b.lo = 0;  // one form for the empty band: no chunk straddles it
     return b;
+}
+
+// Number of real keys of matrix `mat` ([batch * heads] matrices, one length per batch entry).
+__device__ __forceinline__ uint32_t key_limit(const int32_t* key_lengths, uint32_t mat, uint32_t heads)
+{
+    if (key_lengths == nullptr) return 0xffffffffu;
+    const int32_t len = key_lengths[mat / heads];
+    return len < 0 ? 0u : (uint32_t)len;
 }
 
 // Bit k set: register slot k of wave-slot w holds at least one column of the
@@ -173,12 +184,12 @@ __device__ __forceinline__ uint32_t active_slots(const Band& band, int w)
 // ---------------------------------------------------------------------------
 // Causal forward
 // ---------------------------------------------------------------------------
-// PER_HEAD = false compiles the per-head extras (bias tensor, AliBi) out of the
-// plain kernel, which then keeps its registers for loads in flight.
+// PER_HEAD = false compiles the per-head extras (bias tensor, AliBi, key
+// lengths) out of the plain kernel, which then keeps its registers for loads in flight.
 template <int DT, int L, int K, int W, int BW, bool PER_HEAD>
 __global__ void __launch_bounds__((Geo<L, K, W, BW>::kThreads))
 causal_fwd_kernel(uint16_t* y, const uint16_t* x, float scale, uint32_t total_rows, uint32_t n, uint32_t window,
-                  const float* slopes, const uint16_t* bias, uint32_t heads)
+                  const float* slopes, const uint16_t* bias, const int32_t* key_lengths, uint32_t heads)
 {
     using G = Geo<L, K, W, BW>;
     __shared__ float lds[32];
@@ -193,7 +204,8 @@ causal_fwd_kernel(uint16_t* y, const uint16_t* x, float scale, uint32_t total_ro
     uint32_t row, q, mat;
     locate_row<G>(blockIdx.x, n, wave, lane, L, row, q, mat);
     const bool ok = row < total_rows;
-    const Band band = causal_band(q, window, ok);  // columns [lo, hi) take part
+    // columns [lo, hi) take part
+    const Band band = causal_band(q, window, ok, (PER_HEAD && ok) ? key_limit(key_lengths, mat, heads) : 0xffffffffu);
 
     const uint16_t* xr = x + (size_t)row * n;
     uint16_t* yr = y + (size_t)row * n;
@@ -422,10 +434,11 @@ masked_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
 // Backward (causal and unmasked). dx = scale * (dy*y - y * sum(dy*y)).
 // dy and y stay packed in registers between the two passes.
 // ---------------------------------------------------------------------------
-template <int DT, int L, int K, int W, int BW, bool CAUSAL>
+template <int DT, int L, int K, int W, int BW, bool CAUSAL, bool LENGTHS>
 __global__ void __launch_bounds__((Geo<L, K, W, BW>::kThreads))
 softmax_bwd_kernel(uint16_t* dx, const uint16_t* dy, const uint16_t* y, float scale,
-                   uint32_t total_rows, uint32_t n, uint32_t rows_per_matrix, uint32_t window)
+                   uint32_t total_rows, uint32_t n, uint32_t rows_per_matrix, uint32_t window,
+                   const int32_t* key_lengths, uint32_t heads)
 {
     using G = Geo<L, K, W, BW>;
     __shared__ float lds[32];
@@ -440,7 +453,7 @@ softmax_bwd_kernel(uint16_t* dx, const uint16_t* dy, const uint16_t* y, float sc
     const bool ok = row < total_rows;
     Band band;
     if constexpr (CAUSAL) {
-        band = causal_band(q, window, ok);
+        band = causal_band(q, window, ok, (LENGTHS && ok) ? key_limit(key_lengths, mat, heads) : 0xffffffffu);
     } else {
         band.lo = 0;
         band.hi = ok ? n : 0;
@@ -539,7 +552,7 @@ template <int DT, int MODE>
 __global__ void __launch_bounds__(kScalarThreads)
 scalar_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float scale,
                   uint64_t n, uint64_t sq, uint64_t np, int mask_per_batch, uint32_t window,
-                  const float* slopes, const uint16_t* bias, uint32_t heads)
+                  const float* slopes, const uint16_t* bias, const int32_t* key_lengths, uint32_t heads)
 {
     __shared__ float slots[4];
     const uint64_t row = blockIdx.x;
@@ -551,7 +564,7 @@ scalar_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
     float slope = 0.0f;
     const uint16_t* br = nullptr;
     if (MODE == 0) {
-        hi = q + 1;
+        hi = min(q + 1, (uint64_t)key_limit(key_lengths, (uint32_t)(row / sq), heads));
         lo = (q > window) ? q - window : 0;
         if (slopes != nullptr) slope = Half2<DT>::round(slopes[(row / sq) % heads]);
         if (bias != nullptr) br = bias + (((row / sq) % heads) * sq + q) * n;
@@ -580,7 +593,7 @@ scalar_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
     for (uint64_t c = lo + threadIdx.x; c < hi; c += kScalarThreads)
         sum += exp2_raw(fmaf(logit(c) - m, kLog2e, kExpBias));
     sum = block_reduce_256<OpSum>(sum, slots);
-    const float inv = 1.0f / sum;
+    const float inv = 1.0f / sum;  // an empty band (hi <= lo) never uses it
 
     // every thread reads and then writes the columns it owns, after the last
     // reduction barrier: y may alias x
@@ -594,12 +607,13 @@ scalar_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
 template <int DT, bool CAUSAL>
 __global__ void __launch_bounds__(kScalarThreads)
 scalar_bwd_kernel(uint16_t* dx, const uint16_t* dy, const uint16_t* y, float scale,
-                  uint64_t n, uint64_t rows_per_matrix, uint32_t window)
+                  uint64_t n, uint64_t rows_per_matrix, uint32_t window, const int32_t* key_lengths, uint32_t heads)
 {
     __shared__ float slots[4];
     const uint64_t row = blockIdx.x;
     const uint64_t q = row % rows_per_matrix;
-    const uint64_t hi = CAUSAL ? q + 1 : n;
+    const uint64_t hi =
+        CAUSAL ? min(q + 1, (uint64_t)key_limit(key_lengths, (uint32_t)(row / rows_per_matrix), heads)) : n;
     const uint64_t lo = (CAUSAL && q > window) ? q - window : 0;
     const uint16_t* gr = dy + row * n;
     const uint16_t* yr = y + row * n;
@@ -729,7 +743,7 @@ constexpr uint32_t kNoWindow = 0xffffffffu;
 
 template <int DT>
 static int causal_fwd(void* y, const void* x, float scale, int64_t batches, int64_t n, uint32_t window,
-                      const float* slopes, const void* bias, uint32_t heads, hipStream_t st)
+                      const float* slopes, const void* bias, const int32_t* kl, uint32_t heads, hipStream_t st)
 {
     const int64_t rows = batches * n;
     RowPlan p;
@@ -742,26 +756,26 @@ static int causal_fwd(void* y, const void* x, float scale, int64_t batches, int6
         using G = Geo<L_, K_, W_, kBlockWaves>;                                            \
         const uint32_t blocks = (uint32_t)((rows + G::kRowsPerBlock - 1) / G::kRowsPerBlock); \
         if (!launch_fits(blocks, G::kThreads)) return NHP_ERR_SHAPE;                       \
-        if (slopes != nullptr || bp != nullptr)                                            \
+        if (slopes != nullptr || bp != nullptr || kl != nullptr)                           \
             causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves, true><<<blocks, G::kThreads, p.lds, st>>>(  \
-                yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, slopes, bp, heads);    \
+                yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, slopes, bp, kl, heads); \
         else                                                                               \
             causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves, false><<<blocks, G::kThreads, p.lds, st>>>( \
-                yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, nullptr, nullptr, 1);  \
+                yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, nullptr, nullptr, nullptr, 1); \
     }
         NHP_FOR_PLAN(p);
 #undef CALL
     } else {
         if (!launch_fits(rows, kScalarThreads)) return NHP_ERR_SHAPE;
         scalar_fwd_kernel<DT, 0><<<(uint32_t)rows, kScalarThreads, 0, st>>>(
-            yp, xp, nullptr, scale, (uint64_t)n, (uint64_t)n, 1, 0, window, slopes, bp, heads);
+            yp, xp, nullptr, scale, (uint64_t)n, (uint64_t)n, 1, 0, window, slopes, bp, kl, heads);
     }
     return launch_status();
 }
 
 template <int DT, bool CAUSAL>
 static int softmax_bwd(void* dx, const void* dy, const void* y, float scale, int64_t rows, int64_t n,
-                       int64_t rows_per_matrix, uint32_t window, hipStream_t st)
+                       int64_t rows_per_matrix, uint32_t window, const int32_t* kl, uint32_t heads, hipStream_t st)
 {
     RowPlan p;
     uint16_t* dxp = static_cast<uint16_t*>(dx);
@@ -773,15 +787,19 @@ static int softmax_bwd(void* dx, const void* dy, const void* y, float scale, int
         using G = Geo<L_, K_, W_, kBlockWaves>;                                            \
         const uint32_t blocks = (uint32_t)((rows + G::kRowsPerBlock - 1) / G::kRowsPerBlock); \
         if (!launch_fits(blocks, G::kThreads)) return NHP_ERR_SHAPE;                       \
-        softmax_bwd_kernel<DT, L_, K_, W_, kBlockWaves, CAUSAL><<<blocks, G::kThreads, p.lds, st>>>( \
-            dxp, dyp, yp, scale, (uint32_t)rows, (uint32_t)n, (uint32_t)rows_per_matrix, window); \
+        if (CAUSAL && kl != nullptr)                                                       \
+            softmax_bwd_kernel<DT, L_, K_, W_, kBlockWaves, CAUSAL, CAUSAL><<<blocks, G::kThreads, p.lds, st>>>( \
+                dxp, dyp, yp, scale, (uint32_t)rows, (uint32_t)n, (uint32_t)rows_per_matrix, window, kl, heads); \
+        else                                                                               \
+            softmax_bwd_kernel<DT, L_, K_, W_, kBlockWaves, CAUSAL, false><<<blocks, G::kThreads, p.lds, st>>>( \
+                dxp, dyp, yp, scale, (uint32_t)rows, (uint32_t)n, (uint32_t)rows_per_matrix, window, nullptr, 1); \
     }
         NHP_FOR_PLAN(p);
 #undef CALL
     } else {
         if (!launch_fits(rows, kScalarThreads)) return NHP_ERR_SHAPE;
         scalar_bwd_kernel<DT, CAUSAL><<<(uint32_t)rows, kScalarThreads, 0, st>>>(
-            dxp, dyp, yp, scale, (uint64_t)n, (uint64_t)rows_per_matrix, window);
+            dxp, dyp, yp, scale, (uint64_t)n, (uint64_t)rows_per_matrix, window, CAUSAL ? kl : nullptr, heads);
     }
     return launch_status();
 }
@@ -820,7 +838,7 @@ static int masked_fwd(void* y, const void* x, const uint8_t* mask, float scale, 
     } else {
         if (!launch_fits(b * np * sq, kScalarThreads)) return NHP_ERR_SHAPE;
         scalar_fwd_kernel<DT, 1><<<(uint32_t)(b * np * sq), kScalarThreads, 0, st>>>(
-            yp, xp, mask, scale, (uint64_t)n, (uint64_t)sq, (uint64_t)np, per_batch, kNoWindow, nullptr, nullptr, 1);
+            yp, xp, mask, scale, (uint64_t)n, (uint64_t)sq, (uint64_t)np, per_batch, kNoWindow, nullptr, nullptr, nullptr, 1);
     }
     return launch_status();
 }
@@ -834,12 +852,12 @@ extern "C" {
 int64_t nhp_softmax_max_resident_row(void) { return kMaxResidentRow; }
 
 int nhp_causal_softmax_ex_fwd(void* y, const void* x, float scale, int64_t attn_batches, int64_t seq_len,
-                              int64_t window, const float* alibi_slopes, const void* bias, int64_t heads,
-                              int dtype, void* stream)
+                              int64_t window, const float* alibi_slopes, const void* bias,
+                              const int32_t* key_lengths, int64_t heads, int dtype, void* stream)
 {
     if (dtype != NHP_F16 && dtype != NHP_BF16) return NHP_ERR_DTYPE;
     if (attn_batches < 0 || seq_len < 0) return NHP_ERR_SHAPE;
-    const bool per_head = alibi_slopes != nullptr || bias != nullptr;
+    const bool per_head = alibi_slopes != nullptr || bias != nullptr || key_lengths != nullptr;
     if (per_head && (heads < 1 || attn_batches % heads != 0)) return NHP_ERR_SHAPE;
     if (bias != nullptr && (bias == y)) return NHP_ERR_ALIAS;
     if (attn_batches == 0 || seq_len == 0) return NHP_OK;
@@ -849,21 +867,24 @@ int nhp_causal_softmax_ex_fwd(void* y, const void* x, float scale, int64_t attn_
     const uint32_t win = (window < 0 || window >= seq_len) ? kNoWindow : (uint32_t)window;
     const uint32_t hd = per_head ? (uint32_t)heads : 1u;
     return dtype == NHP_BF16
-               ? causal_fwd<NHP_BF16>(y, x, scale, attn_batches, seq_len, win, alibi_slopes, bias, hd, st)
-               : causal_fwd<NHP_F16>(y, x, scale, attn_batches, seq_len, win, alibi_slopes, bias, hd, st);
+               ? causal_fwd<NHP_BF16>(y, x, scale, attn_batches, seq_len, win, alibi_slopes, bias, key_lengths, hd, st)
+               : causal_fwd<NHP_F16>(y, x, scale, attn_batches, seq_len, win, alibi_slopes, bias, key_lengths, hd, st);
 }
 
 int nhp_causal_softmax_fwd(void* y, const void* x, float scale, int64_t attn_batches, int64_t seq_len,
                            int dtype, void* stream)
 {
-    return nhp_causal_softmax_ex_fwd(y, x, scale, attn_batches, seq_len, -1, nullptr, nullptr, 1, dtype, stream);
+    return nhp_causal_softmax_ex_fwd(y, x, scale, attn_batches, seq_len, -1, nullptr, nullptr, nullptr, 1, dtype,
+                                     stream);
 }
 
 int nhp_causal_softmax_ex_bwd(void* dx, const void* dy, const void* y, float scale, int64_t attn_batches,
-                              int64_t seq_len, int64_t window, int dtype, void* stream)
+                              int64_t seq_len, int64_t window, const int32_t* key_lengths, int64_t heads,
+                              int dtype, void* stream)
 {
     if (dtype != NHP_F16 && dtype != NHP_BF16) return NHP_ERR_DTYPE;
     if (attn_batches < 0 || seq_len < 0) return NHP_ERR_SHAPE;
+    if (key_lengths != nullptr && (heads < 1 || attn_batches % heads != 0)) return NHP_ERR_SHAPE;
     if (attn_batches == 0 || seq_len == 0) return NHP_OK;
     if (attn_batches > kMaxRows / seq_len - 1) return NHP_ERR_SHAPE;
     if (!dx || !dy || !y) return NHP_ERR_NULL;
@@ -871,15 +892,16 @@ int nhp_causal_softmax_ex_bwd(void* dx, const void* dy, const void* y, float sca
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int64_t rows = attn_batches * seq_len;
     const uint32_t win = (window < 0 || window >= seq_len) ? kNoWindow : (uint32_t)window;
+    const uint32_t hd = key_lengths != nullptr ? (uint32_t)heads : 1u;
     return dtype == NHP_BF16
-               ? softmax_bwd<NHP_BF16, true>(dx, dy, y, scale, rows, seq_len, seq_len, win, st)
-               : softmax_bwd<NHP_F16, true>(dx, dy, y, scale, rows, seq_len, seq_len, win, st);
+               ? softmax_bwd<NHP_BF16, true>(dx, dy, y, scale, rows, seq_len, seq_len, win, key_lengths, hd, st)
+               : softmax_bwd<NHP_F16, true>(dx, dy, y, scale, rows, seq_len, seq_len, win, key_lengths, hd, st);
 }
 
 int nhp_causal_softmax_bwd(void* dx, const void* dy, const void* y, float scale, int64_t attn_batches,
                            int64_t seq_len, int dtype, void* stream)
 {
-    return nhp_causal_softmax_ex_bwd(dx, dy, y, scale, attn_batches, seq_len, -1, dtype, stream);
+    return nhp_causal_softmax_ex_bwd(dx, dy, y, scale, attn_batches, seq_len, -1, nullptr, 1, dtype, stream);
 }
 
 int nhp_masked_softmax_fwd(void* y, const void* x, const uint8_t* mask, float scale, int64_t b,
@@ -908,8 +930,8 @@ int nhp_masked_softmax_bwd(void* dx, const void* dy, const void* y, float scale,
     if (dx == y) return NHP_ERR_ALIAS;
     hipStream_t st = static_cast<hipStream_t>(stream);
     // rows_per_matrix only matters for the causal variant; any non-zero value works here
-    return dtype == NHP_BF16 ? softmax_bwd<NHP_BF16, false>(dx, dy, y, scale, rows, sk, rows, kNoWindow, st)
-                             : softmax_bwd<NHP_F16, false>(dx, dy, y, scale, rows, sk, rows, kNoWindow, st);
+    return dtype == NHP_BF16 ? softmax_bwd<NHP_BF16, false>(dx, dy, y, scale, rows, sk, rows, kNoWindow, nullptr, 1, st)
+                             : softmax_bwd<NHP_F16, false>(dx, dy, y, scale, rows, sk, rows, kNoWindow, nullptr, 1, st);
 }
 
 int nhp_softmax_batch_per_block(int64_t query_seq_len, int64_t key_seq_len, int64_t batches,

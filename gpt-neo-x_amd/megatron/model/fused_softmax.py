@@ -22,7 +22,11 @@ all of it widening:
   instead of by a separate ``scores + alibi_matrix`` pass). Both default to off;
 * ``forward(input, mask, bias=None)``: an optional additive bias ``[1, np, sq, sk]``
   (the relative-position bias the caller adds with ``attention_scores += rpe``)
-  is read by the causal kernel instead of being added in a pass of its own.
+  is read by the causal kernel instead of being added in a pass of its own;
+* ``forward(..., key_lengths=None)``: an integer tensor ``[b]`` of real key counts for
+  right-padded batches. The causal kernel masks the padding keys by index (the
+  reference's ignores the mask, so padding is attended to on its fused branch); the
+  other branches merge ``k >= key_lengths[b]`` into the mask they are given.
 """
 import enum
 
@@ -47,17 +51,18 @@ class ScaledUpperTriangMaskedSoftmax(torch.autograd.Function):
     """``softmax(scale * x)`` over the lower triangle of ``[attn_batches, sq, sk]``
     scores (zeros above the diagonal), one kernel forward and one backward.
 
-    ``window``, ``alibi_slopes`` and ``bias`` are the optional extras described in
+    ``window``, ``alibi_slopes``, ``bias`` and ``key_lengths`` are the optional extras described in
     the module docstring; the reference signature is ``apply(inputs, scale)``.
     """
 
     @staticmethod
-    def forward(ctx, inputs, scale, window=None, alibi_slopes=None, bias=None):
+    def forward(ctx, inputs, scale, window=None, alibi_slopes=None, bias=None, key_lengths=None):
         import scaled_upper_triang_masked_softmax_cuda as kernels
 
         factor = _scale_tensor(scale)
-        out = kernels.forward(inputs, factor[0], window, alibi_slopes, bias)
+        out = kernels.forward(inputs, factor[0], window, alibi_slopes, bias, key_lengths)
         ctx.window = window
+        ctx.key_lengths = key_lengths
         ctx.bias_shape = None if bias is None else tuple(bias.shape)
         ctx.save_for_backward(out, factor)
         return out
@@ -68,13 +73,13 @@ class ScaledUpperTriangMaskedSoftmax(torch.autograd.Function):
 
         out, factor = ctx.saved_tensors
         # in place on output_grads, like the reference kernel
-        grad = kernels.backward(output_grads, out, factor[0], ctx.window)
+        grad = kernels.backward(output_grads, out, factor[0], ctx.window, ctx.key_lengths)
         grad_bias = None
         if ctx.bias_shape is not None and ctx.needs_input_grad[4]:
             # the bias is shared by the batch: its gradient is the batch sum of the score gradient
             heads, sq, sk = ctx.bias_shape[-3:]
             grad_bias = grad.view(-1, heads, sq, sk).sum(dim=0).view(ctx.bias_shape)
-        return grad, None, None, None, grad_bias
+        return grad, None, None, None, grad_bias, None
 
 
 class ScaledMaskedSoftmax(torch.autograd.Function):
@@ -144,11 +149,11 @@ class FusedScaleMaskSoftmax(nn.Module):
             self.register_buffer("alibi_slopes", alibi_slopes.detach().float().clone(), persistent=False)
 
     # ------------------------------------------------------------------ dispatch
-    def forward(self, input, mask, bias=None):
+    def forward(self, input, mask, bias=None, key_lengths=None):
         assert input.dim() == 4  # [b, np, sq, sk]
         if self.is_kernel_available(mask, *input.size()):
-            return self.forward_fused_softmax(input, mask, bias)
-        return self.forward_torch_softmax(input, mask, bias)
+            return self.forward_fused_softmax(input, mask, bias, key_lengths)
+        return self.forward_torch_softmax(input, mask, bias, key_lengths)
 
     def is_kernel_available(self, mask, b, np, sq, sk):
         """The reference's conditions (fused_softmax.py:148-168) without ``sk <= 2048``."""
@@ -168,10 +173,21 @@ class FusedScaleMaskSoftmax(nn.Module):
         return scaled_masked_softmax_cuda.get_batch_per_block(sq, sk, b, np)
 
     # ------------------------------------------------------------------ branches
-    def forward_fused_softmax(self, input, mask, bias=None):
+    @staticmethod
+    def _mask_with_padding(mask, key_lengths, b, sk):
+        """The mask with the padding keys ``k >= key_lengths[b]`` added: ``[b, 1, sq, sk]``."""
+        if key_lengths is None:
+            return mask
+        assert key_lengths.shape == (b,), "key_lengths must be [b]"
+        keys = torch.arange(sk, device=mask.device)
+        padding = keys.view(1, 1, 1, sk) >= key_lengths.to(mask.device).view(b, 1, 1, 1)
+        return (mask.bool() | padding).contiguous()
+
+    def forward_fused_softmax(self, input, mask, bias=None, key_lengths=None):
         b, np, sq, sk = input.size()
         factor = 1.0 if self.scale is None else self.scale
         if not self.upper_triang_mask_fusion:
+            mask = self._mask_with_padding(mask, key_lengths, b, sk)
             if bias is not None:
                 input = input + bias
             if self.alibi_slopes is not None:
@@ -186,10 +202,14 @@ class FusedScaleMaskSoftmax(nn.Module):
         flat = input.view(b * np, sq, sk)
         if bias is not None:
             assert bias.shape[-3:] == (np, sq, sk) and bias.numel() == np * sq * sk, "bias must be [1, np, sq, sk]"
-        probs = ScaledUpperTriangMaskedSoftmax.apply(flat, factor, self.sliding_window_width, slopes, bias)
+        if key_lengths is not None:
+            assert key_lengths.shape == (b,), "key_lengths must be [b]"
+        probs = ScaledUpperTriangMaskedSoftmax.apply(flat, factor, self.sliding_window_width, slopes, bias, key_lengths)
         return probs.view(b, np, sq, sk)
 
-    def forward_torch_softmax(self, input, mask, bias=None):
+    def forward_torch_softmax(self, input, mask, bias=None, key_lengths=None):
+        if key_lengths is not None and mask is not None:
+            mask = self._mask_with_padding(mask, key_lengths, input.size(0), input.size(3))
         if bias is not None:
             input = input + bias
         if self.alibi_slopes is not None:

@@ -11,14 +11,28 @@ from megatron.fused_kernels import _hotpath as _hp
 _HALF = (torch.float16, torch.bfloat16)
 
 
-def forward(input, scale_factor, window=None, alibi_slopes=None, bias=None):
+def _key_lengths_arg(key_lengths, attn_batches, heads, who):
+    """(tensor kept alive, pointer, heads per batch entry) for an integer [batch] tensor of key counts."""
+    if key_lengths is None:
+        return None, None, heads
+    if key_lengths.dim() != 1 or key_lengths.numel() == 0 or key_lengths.is_floating_point():
+        raise RuntimeError("key_lengths must be a non-empty 1-D integer tensor")
+    _hp.require_gpu(key_lengths, who)
+    batch = key_lengths.numel()
+    if attn_batches % batch != 0 or (heads is not None and attn_batches != batch * heads):
+        raise RuntimeError("attn_batches must equal len(key_lengths) * heads")
+    lengths = key_lengths.to(torch.int32).contiguous()
+    return lengths, lengths.data_ptr(), attn_batches // batch
+
+
+def forward(input, scale_factor, window=None, alibi_slopes=None, bias=None, key_lengths=None):
     """softmax(scale * input) under an upper-triangular mask.
 
     input: [attn_batches, seq_len, seq_len] fp16/bf16 on the GPU. Returns a new
     tensor of the same shape and dtype (requires_grad False). Checks follow
     scaled_upper_triang_masked_softmax.cpp:31-39; seq_len is not limited to 2048.
 
-    Three optional arguments go beyond the reference function:
+    Four optional arguments go beyond the reference function:
     window: sliding-window width; row q attends to keys q-window..q only.
     alibi_slopes: fp32 tensor [heads] on the GPU (attn_batches % heads == 0);
         the AliBi bias -(q-k)*slope is added to the scores in the storage dtype
@@ -26,6 +40,9 @@ def forward(input, scale_factor, window=None, alibi_slopes=None, bias=None):
     bias: [heads, seq_len, seq_len] tensor of the input's dtype (attn_batches %
         heads == 0), added to the scores in the storage dtype first, as
         `scores += bias` would (e.g. a relative-position bias shared by the batch).
+    key_lengths: integer tensor [batch] on the GPU, input being [batch * heads, s, s]:
+        keys at or beyond a batch entry's length are padding and get probability 0
+        (rows without any key left are all zeros).
     """
     if input.dim() != 3:
         raise RuntimeError("expected 3D tensor")
@@ -36,7 +53,7 @@ def forward(input, scale_factor, window=None, alibi_slopes=None, bias=None):
     _hp.require_gpu(input, "scaled_upper_triang_masked_softmax_cuda.forward")
     x = input.contiguous()
     y = torch.empty_like(x)
-    slopes_ptr, heads = None, 1
+    slopes_ptr, heads = None, None
     if alibi_slopes is not None:
         if alibi_slopes.dtype != torch.float32 or alibi_slopes.dim() != 1:
             raise RuntimeError("alibi_slopes must be a 1-D float32 tensor")
@@ -58,17 +75,20 @@ def forward(input, scale_factor, window=None, alibi_slopes=None, bias=None):
         bias_ptr, heads = bias.data_ptr(), bias.size(0)
         if heads == 0 or x.size(0) % heads != 0:
             raise RuntimeError("attn_batches must be a multiple of the number of bias heads")
+    lengths, lengths_ptr, heads = _key_lengths_arg(key_lengths, x.size(0), heads,
+                                                   "scaled_upper_triang_masked_softmax_cuda.forward")
     with _hp.device_guard(x):
         rc = _hp.lib().nhp_causal_softmax_ex_fwd(
             y.data_ptr(), x.data_ptr(), float(scale_factor), x.size(0), x.size(1),
-            -1 if window is None else int(window), slopes_ptr, bias_ptr, heads, _hp.dtype_code(x, "forward"),
-            _hp.stream_of(x))
+            -1 if window is None else int(window), slopes_ptr, bias_ptr, lengths_ptr, heads or 1,
+            _hp.dtype_code(x, "forward"), _hp.stream_of(x))
     _hp.check(rc, "scaled_upper_triang_masked_softmax_cuda.forward")
     return y
 
 
-def backward(output_grads, softmax_results, scale_factor, window=None):
-    """Gradient w.r.t. the input of ``forward`` (pass the same ``window``; AliBi needs nothing here).
+def backward(output_grads, softmax_results, scale_factor, window=None, key_lengths=None):
+    """Gradient w.r.t. the input of ``forward`` (pass the same ``window`` and ``key_lengths``;
+    AliBi and the bias tensor need nothing here).
 
     Works in place: the result is written into (the contiguous version of)
     ``output_grads`` and that tensor is returned, as in
@@ -86,9 +106,12 @@ def backward(output_grads, softmax_results, scale_factor, window=None):
     _hp.require_gpu(softmax_results, "scaled_upper_triang_masked_softmax_cuda.backward")
     g = output_grads.detach().contiguous()
     y = softmax_results.detach().contiguous()
+    lengths, lengths_ptr, heads = _key_lengths_arg(key_lengths, g.size(0), None,
+                                                   "scaled_upper_triang_masked_softmax_cuda.backward")
     with _hp.device_guard(g):
         rc = _hp.lib().nhp_causal_softmax_ex_bwd(
             g.data_ptr(), g.data_ptr(), y.data_ptr(), float(scale_factor), g.size(0), g.size(1),
-            -1 if window is None else int(window), _hp.dtype_code(g, "backward"), _hp.stream_of(g))
+            -1 if window is None else int(window), lengths_ptr, heads or 1, _hp.dtype_code(g, "backward"),
+            _hp.stream_of(g))
     _hp.check(rc, "scaled_upper_triang_masked_softmax_cuda.backward")
     return g

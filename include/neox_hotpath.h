@@ -110,9 +110,18 @@ int nhp_causal_softmax_bwd(void* dx, const void* dy, const void* y, float scale,
  *      megatron/model/transformer.py:580-582 as `attention_scores += rpe`):
  *      the score becomes x (+) bias[hd, q, k], rounded to the storage dtype,
  *      before AliBi (if any) and the softmax. Only the attended band is read.
+ *  key_lengths != NULL: `attn_batches / heads` int32 values on the device, one
+ *      per batch entry (x is a [b, heads, s, s] tensor): the keys
+ *      k >= key_lengths[b] are padding and masked like the keys above the
+ *      diagonal, i.e. the mask `causal | (k >= len)` handed to
+ *      FusedScaleMaskSoftmax.forward (megatron/model/fused_softmax.py:140-146),
+ *      which the reference's causal kernel ignores. Padding keys are never
+ *      read. A row left without any key (length 0) is written as zeros.
+ *      Values below 0 count as 0, values above seq_len as seq_len.
  *
- * The backward of the AliBi variant is the plain (windowed) backward: the bias
- * is constant.
+ * The backward takes the same window and key_lengths (masked positions get
+ * +0, the row sum runs over the attended keys only); AliBi and the bias tensor
+ * are additive constants and do not appear in it.
  *
  * Extends scaled_upper_triang_masked_softmax_cuda.forward / backward
  * (megatron/fused_kernels/scaled_upper_triang_masked_softmax.cpp:31-56), whose
@@ -122,11 +131,11 @@ int nhp_causal_softmax_bwd(void* dx, const void* dy, const void* y, float scale,
 int nhp_causal_softmax_ex_fwd(void* y, const void* x, float scale,
                               int64_t attn_batches, int64_t seq_len,
                               int64_t window, const float* alibi_slopes, const void* bias,
-                              int64_t heads, int dtype, void* stream);
+                              const int32_t* key_lengths, int64_t heads, int dtype, void* stream);
 
 int nhp_causal_softmax_ex_bwd(void* dx, const void* dy, const void* y, float scale,
                               int64_t attn_batches, int64_t seq_len, int64_t window,
-                              int dtype, void* stream);
+                              const int32_t* key_lengths, int64_t heads, int dtype, void* stream);
 
 /* ------------------------------------------------------------------------
  * Scaled padding-masked softmax

@@ -45,8 +45,8 @@ def lib():
         L = ctypes.CDLL(_LIB_PATH)
         i64, vp, f32, ci = ctypes.c_int64, ctypes.c_void_p, ctypes.c_float, ctypes.c_int
         L.oracle_causal_softmax_fwd.argtypes = [vp, vp, f32, i64, i64, ci]
-        L.oracle_causal_softmax_ex_fwd.argtypes = [vp, vp, f32, i64, i64, i64, vp, vp, i64, ci]
-        L.oracle_softmax_ex_bwd.argtypes = [vp, vp, vp, f32, i64, i64, i64, ci, i64, ci]
+        L.oracle_causal_softmax_ex_fwd.argtypes = [vp, vp, f32, i64, i64, i64, vp, vp, vp, i64, ci]
+        L.oracle_softmax_ex_bwd.argtypes = [vp, vp, vp, f32, i64, i64, i64, ci, i64, vp, i64, ci]
         L.oracle_masked_softmax_fwd.argtypes = [vp, vp, vp, f32, i64, i64, i64, i64, i64, ci]
         L.oracle_softmax_bwd.argtypes = [vp, vp, vp, f32, i64, i64, i64, ci, ci]
         L.oracle_batch_per_block.argtypes = [i64, ci]
@@ -75,14 +75,26 @@ def _cpu_contig(t):
     return t.contiguous()
 
 
-def causal_softmax_fwd(x, scale, window=None, alibi_slopes=None, bias=None):
+def _key_lengths(key_lengths, attn_batches, heads):
+    """int32 [batch] tensor and the heads-per-batch-entry divisor for the C side."""
+    if key_lengths is None:
+        return None, None, heads
+    kl = _cpu_contig(key_lengths.to(torch.int32))
+    if heads is None:
+        heads = attn_batches // kl.numel()
+    assert kl.numel() * heads == attn_batches, "key_lengths needs attn_batches == batch * heads"
+    return kl, kl.data_ptr(), heads
+
+
+def causal_softmax_fwd(x, scale, window=None, alibi_slopes=None, bias=None, key_lengths=None):
     """x: [attn_batches, s, s] fp16/bf16 -> probabilities, same shape and dtype.
     window: sliding-window width or None; alibi_slopes: fp32 [heads] or None;
-    bias: [heads, s, s] in x.dtype or None."""
+    bias: [heads, s, s] in x.dtype or None; key_lengths: integer [batch] or None
+    (attn_batches = batch * heads, keys >= the length are padding)."""
     assert x.dim() == 3 and x.size(1) == x.size(2)
     x = _cpu_contig(x)
     y = torch.empty_like(x)
-    sl_ptr, heads = None, 1
+    sl_ptr, heads = None, None
     if alibi_slopes is not None:
         alibi_slopes = _cpu_contig(alibi_slopes.float())
         sl_ptr, heads = alibi_slopes.data_ptr(), alibi_slopes.numel()
@@ -94,9 +106,10 @@ def causal_softmax_fwd(x, scale, window=None, alibi_slopes=None, bias=None):
         assert alibi_slopes is None or bias.size(0) == heads
         b_ptr, heads = bias.data_ptr(), bias.size(0)
         assert x.size(0) % heads == 0
+    kl, kl_ptr, heads = _key_lengths(key_lengths, x.size(0), heads)
     _check(lib().oracle_causal_softmax_ex_fwd(y.data_ptr(), x.data_ptr(), float(scale), x.size(0), x.size(1),
-                                              -1 if window is None else int(window), sl_ptr, b_ptr, heads,
-                                              _DT[x.dtype]), "causal_softmax_fwd")
+                                              -1 if window is None else int(window), sl_ptr, b_ptr, kl_ptr,
+                                              heads or 1, _DT[x.dtype]), "causal_softmax_fwd")
     return y
 
 
@@ -114,17 +127,19 @@ def masked_softmax_fwd(x, mask, scale):
     return y
 
 
-def softmax_bwd(dy, y, scale, causal, window=None):
-    """Returns dx (a new tensor). dy, y: [..., rows_per_matrix, n]."""
+def softmax_bwd(dy, y, scale, causal, window=None, key_lengths=None):
+    """Returns dx (a new tensor). dy, y: [..., rows_per_matrix, n]; key_lengths
+    (causal only): integer [batch] with dy [batch * heads, s, s]."""
     dy = _cpu_contig(dy)
     y = _cpu_contig(y)
     assert dy.shape == y.shape and dy.dtype == y.dtype
     n = dy.size(-1)
     rows = dy.numel() // max(n, 1)
     dx = torch.empty_like(dy)
+    kl, kl_ptr, heads = _key_lengths(key_lengths, rows // max(dy.size(-2), 1), None)
     _check(lib().oracle_softmax_ex_bwd(dx.data_ptr(), dy.data_ptr(), y.data_ptr(), float(scale), rows, n,
                                        dy.size(-2), 1 if causal else 0, -1 if window is None else int(window),
-                                       _DT[dy.dtype]), "softmax_bwd")
+                                       kl_ptr, heads or 1, _DT[dy.dtype]), "softmax_bwd")
     return dx
 
 

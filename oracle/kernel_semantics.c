@@ -178,9 +178,17 @@ static void softmax_row(float* z, int64_t n)
  *     to the [b, np, sq, sk] scores before scale_mask_softmax);
  *   bias != NULL: `attention_scores += rpe` (transformer.py:580-582), a
  *     [heads, s, s] tensor in the storage dtype added (rounded) before AliBi.
+ *   key_lengths != NULL: int32 [batches / heads]; the keys k >= key_lengths[b]
+ *     of batch entry b = matrix / heads are padding and masked like the keys
+ *     above the diagonal (the mask `causal | (k >= len)` given to
+ *     forward_torch_softmax, fused_softmax.py:184-199). A row that keeps no
+ *     key at all is written as zeros (the fallback's softmax over a row of
+ *     equal fill values would give 1/s there; attention to padding only is
+ *     meaningless either way and zeros keep the output finite).
  */
 int oracle_causal_softmax_ex_fwd(void* y, const void* x, float scale, int64_t batches, int64_t s,
-                                 int64_t window, const float* slopes, const void* bias, int64_t heads, int dt)
+                                 int64_t window, const float* slopes, const void* bias,
+                                 const int32_t* key_lengths, int64_t heads, int dt)
 {
     if (dt != DT_F16 && dt != DT_BF16) return -1;
     float* z = (float*)malloc(sizeof(float) * (size_t)(s > 0 ? s : 1));
@@ -190,7 +198,16 @@ int oracle_causal_softmax_ex_fwd(void* y, const void* x, float scale, int64_t ba
         for (int64_t q = 0; q < s; ++q) {
             const int64_t base = (a * s + q) * s;
             const int64_t lo = (window >= 0 && q > window) ? q - window : 0;
-            for (int64_t k = lo; k <= q; ++k) {
+            int64_t hi = q + 1; /* keys [lo, hi) take part */
+            if (key_lengths) {
+                const int64_t len = key_lengths[a / heads] < 0 ? 0 : key_lengths[a / heads];
+                if (len < hi) hi = len;
+            }
+            if (hi <= lo) {
+                for (int64_t k = 0; k < s; ++k) store_elem(y, base + k, dt, 0.0f);
+                continue;
+            }
+            for (int64_t k = lo; k < hi; ++k) {
                 float v = load_elem(x, base + k, dt);
                 /* attention_scores += rpe (transformer.py:580-582): bias [heads, s, s] in the storage dtype */
                 if (bias) v = add_t(v, load_elem(bias, ((a % heads) * s + q) * s + k, dt), dt);
@@ -200,10 +217,10 @@ int oracle_causal_softmax_ex_fwd(void* y, const void* x, float scale, int64_t ba
                 }
                 z[k - lo] = v * scale;
             }
-            softmax_row(z, q + 1 - lo);
+            softmax_row(z, hi - lo);
             for (int64_t k = 0; k < lo; ++k) store_elem(y, base + k, dt, 0.0f);
-            for (int64_t k = lo; k <= q; ++k) store_elem(y, base + k, dt, z[k - lo]);
-            for (int64_t k = q + 1; k < s; ++k) store_elem(y, base + k, dt, 0.0f);
+            for (int64_t k = lo; k < hi; ++k) store_elem(y, base + k, dt, z[k - lo]);
+            for (int64_t k = hi; k < s; ++k) store_elem(y, base + k, dt, 0.0f);
         }
     }
     free(z);
@@ -212,7 +229,7 @@ int oracle_causal_softmax_ex_fwd(void* y, const void* x, float scale, int64_t ba
 
 int oracle_causal_softmax_fwd(void* y, const void* x, float scale, int64_t batches, int64_t s, int dt)
 {
-    return oracle_causal_softmax_ex_fwd(y, x, scale, batches, s, -1, NULL, NULL, 1, dt);
+    return oracle_causal_softmax_ex_fwd(y, x, scale, batches, s, -1, NULL, NULL, NULL, 1, dt);
 }
 
 /*
@@ -249,7 +266,8 @@ int oracle_masked_softmax_fwd(void* y, const void* x, const uint8_t* mask, float
  * causal row index q = row % rows_per_matrix. dx may alias dy.
  */
 int oracle_softmax_ex_bwd(void* dx, const void* dy, const void* y, float scale, int64_t rows, int64_t n,
-                          int64_t rows_per_matrix, int causal, int64_t window, int dt)
+                          int64_t rows_per_matrix, int causal, int64_t window, const int32_t* key_lengths,
+                          int64_t heads, int dt)
 {
     if (dt != DT_F16 && dt != DT_BF16) return -1;
     float* g = (float*)malloc(sizeof(float) * (size_t)(n > 0 ? n : 1));
@@ -261,7 +279,11 @@ int oracle_softmax_ex_bwd(void* dx, const void* dy, const void* y, float scale, 
     }
     for (int64_t r = 0; r < rows; ++r) {
         const int64_t q = r % rows_per_matrix;
-        const int64_t valid = causal ? q + 1 : n;
+        int64_t valid = causal ? q + 1 : n;
+        if (causal && key_lengths) { /* padding keys, as in the forward */
+            const int64_t len = key_lengths[(r / rows_per_matrix) / heads];
+            if (len < valid) valid = len < 0 ? 0 : len;
+        }
         /* sliding window: columns below q - window are masked like those above the diagonal */
         const int64_t lo = (causal && window >= 0 && q > window) ? q - window : 0;
         const int64_t base = r * n;
@@ -289,7 +311,7 @@ int oracle_softmax_ex_bwd(void* dx, const void* dy, const void* y, float scale, 
 int oracle_softmax_bwd(void* dx, const void* dy, const void* y, float scale, int64_t rows, int64_t n,
                        int64_t rows_per_matrix, int causal, int dt)
 {
-    return oracle_softmax_ex_bwd(dx, dy, y, scale, rows, n, rows_per_matrix, causal, -1, dt);
+    return oracle_softmax_ex_bwd(dx, dy, y, scale, rows, n, rows_per_matrix, causal, -1, NULL, 1, dt);
 }
 
 /*

@@ -16,21 +16,27 @@ DEV = "cuda"
 DTYPES = [torch.bfloat16, torch.float16]
 
 
-def abi_ex_fwd(hp, x, scale, window, slopes, bias=None):
+def abi_ex_fwd(hp, x, scale, window, slopes, bias=None, key_lengths=None):
     y = torch.empty_like(x)
     heads = slopes.numel() if slopes is not None else bias.size(0) if bias is not None else 1
+    if key_lengths is not None:
+        assert key_lengths.dtype == torch.int32
+        heads = x.size(0) // key_lengths.numel()
     rc = hp.lib().nhp_causal_softmax_ex_fwd(
         y.data_ptr(), x.data_ptr(), scale, x.size(0), x.size(1), -1 if window is None else window,
-        None if slopes is None else slopes.data_ptr(), None if bias is None else bias.data_ptr(), heads,
-        hp.dtype_code(x, "t"), None)
+        None if slopes is None else slopes.data_ptr(), None if bias is None else bias.data_ptr(),
+        None if key_lengths is None else key_lengths.data_ptr(), heads, hp.dtype_code(x, "t"), None)
     assert rc == 0, hp.lib().nhp_status_string(rc)
     return y
 
 
-def abi_ex_bwd(hp, dy, y, scale, window):
+def abi_ex_bwd(hp, dy, y, scale, window, key_lengths=None):
     dx = torch.empty_like(dy)
+    heads = 1 if key_lengths is None else dy.size(0) // key_lengths.numel()
     rc = hp.lib().nhp_causal_softmax_ex_bwd(dx.data_ptr(), dy.data_ptr(), y.data_ptr(), scale, dy.size(0), dy.size(1),
-                                            -1 if window is None else window, hp.dtype_code(dy, "t"), None)
+                                            -1 if window is None else window,
+                                            None if key_lengths is None else key_lengths.data_ptr(), heads,
+                                            hp.dtype_code(dy, "t"), None)
     assert rc == 0, hp.lib().nhp_status_string(rc)
     return dx
 
@@ -158,3 +164,76 @@ def test_module_with_relative_position_bias_and_its_gradient():
         f, p = out["fused"][i], out["plain"][i]
         assert (f - p).norm().item() <= 4 * eps * p.norm().item(), what
     assert out["fused"][2].shape == (1, np_, s, s)
+
+
+def padded_mask(s, lengths, window=None):
+    """[batch, s, s] bool, True = masked: above the diagonal, outside the window, or a padding key."""
+    causal = fb.causal_mask(s, sliding_window_width=window)[0, 0]
+    keys = torch.arange(s)
+    return causal[None] | (keys[None, None, :] >= lengths.view(-1, 1, 1))
+
+
+# (batch, heads, seq_len, window, lengths)
+LENGTH_CASES = [
+    (4, 2, 64, None, [0, 1, 64, 37]),
+    (3, 2, 512, None, [512, 100, 511]),
+    (2, 3, 2048, None, [1500, 7]),
+    (2, 2, 2048, 300, [2048, 1111]),       # rows 1411.. keep no key: the window starts in the padding
+    (2, 2, 512, 8, [100, 101]),
+    (2, 1, 4096, None, [4000, 513]),
+    (2, 2, 1001, None, [1001, 333]),       # row length not a multiple of 8: scalar kernels
+    (2, 2, 200, 17, [5000, -3]),           # out-of-range lengths clamp to [0, s]
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
+@pytest.mark.parametrize("case", LENGTH_CASES, ids=lambda c: f"b{c[0]}_h{c[1]}_s{c[2]}_w{c[3]}")
+def test_key_lengths_forward_backward_vs_oracle(hotpath, case, dtype):
+    batch, heads, s, window, lengths = case
+    print(f"key-length case {case} {dtype}", flush=True)
+    scale = 1 / math.sqrt(128)
+    lengths = torch.tensor(lengths, dtype=torch.int32)
+    x = util.randn((batch * heads, s, s), dtype, seed=s, std=2.0)
+    dy = util.randn((batch * heads, s, s), dtype, seed=s + 1)
+    masked = padded_mask(s, lengths, window).repeat_interleave(heads, dim=0)
+    want_y = oracle.causal_softmax_fwd(x, scale, window=window, key_lengths=lengths)
+    # the padding keys are never read: poison them (whole 16-byte chunks beyond the length)
+    chunk_start = torch.arange(s) // 8 * 8
+    beyond = (chunk_start[None, None, :] >= lengths.clamp(0, s).view(-1, 1, 1)).repeat_interleave(heads, dim=0)
+    xp = x.clone()
+    xp[beyond.expand_as(xp)] = float("nan")
+    got_y = abi_ex_fwd(hotpath, xp.to(DEV), scale, window, None, None, lengths.to(DEV)).cpu()
+    assert int(util.raw_bits(got_y)[masked].abs().max()) == 0
+    util.assert_ulp_close(got_y, want_y, 2, "fwd")
+    want_dx = oracle.softmax_bwd(dy, want_y, scale, causal=True, window=window, key_lengths=lengths)
+    got_dx = abi_ex_bwd(hotpath, dy.to(DEV), want_y.to(DEV), scale, window, lengths.to(DEV)).cpu()
+    assert int(util.raw_bits(got_dx)[masked].abs().max()) == 0
+    util.assert_softmax_bwd_close(got_dx, want_dx, dy.masked_fill(masked, 0), want_y, scale, "bwd")
+
+
+@pytest.mark.parametrize("fusion", ["upper_triang", "general"])
+def test_module_with_key_lengths_all_branches_agree(fusion):
+    """forward(input, mask, key_lengths=...) on a fused branch against the torch branch given
+    the same arguments, probabilities and score gradients."""
+    from megatron.model.fused_softmax import FusedScaleMaskSoftmax, SoftmaxFusionTypes as T
+
+    dtype, b, np_, s, scale = torch.bfloat16, 4, 4, 512, 0.125
+    lengths = torch.tensor([512, 300, 17, 450], device=DEV)
+    x = util.randn((b, np_, s, s), dtype, seed=1, std=2.0)
+    dy = util.randn((b, np_, s, s), dtype, seed=2)
+    mask = fb.causal_mask(s, DEV)
+    out = {}
+    for name, kind in (("fused", T[fusion]), ("plain", T.none)):
+        m = FusedScaleMaskSoftmax(False, True, kind, fb.fill_masked_with_dtype_min, True, scale)
+        xd = x.to(DEV).requires_grad_(True)
+        y = m(xd, mask, key_lengths=lengths)
+        y.backward(dy.to(DEV).clone())
+        out[name] = (y.detach().cpu(), xd.grad.float().cpu())
+    masked = padded_mask(s, lengths.cpu())[:, None].expand(b, np_, s, s)
+    util.assert_ulp_close(out["fused"][0], out["plain"][0], 2, "fwd fused vs torch branch")
+    assert int(util.raw_bits(out["fused"][0])[masked].abs().max()) == 0
+    f, p = out["fused"][1], out["plain"][1]
+    assert (f - p).norm().item() <= 4 * 2.0**-8 * p.norm().item()
+    if fusion == "upper_triang":
+        want = oracle.causal_softmax_fwd(x.view(-1, s, s), scale, key_lengths=lengths.cpu()).view(b, np_, s, s)
+        util.assert_ulp_close(out["fused"][0], want, 2, "fwd vs oracle")

@@ -159,3 +159,65 @@ def test_additive_bias_equals_eager_add_then_plain_softmax(dtype):
     both = oracle.causal_softmax_fwd(x.view(-1, s, s), scale, window=9, alibi_slopes=slopes, bias=bias[0])
     eager = oracle.causal_softmax_fwd(fb.alibi_add(x + bias, slopes).view(-1, s, s), scale, window=9)
     assert torch.equal(util.raw_bits(both), util.raw_bits(eager))
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("window", [None, 6])
+def test_key_lengths_forward(dtype, window):
+    """Padding keys k >= len[b] masked by index: float64 brute force over the kept band,
+    the torch fallback given the merged mask, rows the padding does not reach unchanged
+    bit for bit, rows without any key all zeros."""
+    batch, heads, s, scale = 4, 2, 40, 0.3
+    lengths = torch.tensor([40, 13, 1, 0], dtype=torch.int32)
+    x = util.randn((batch * heads, s, s), dtype, seed=5, std=2.0)
+    y = oracle.causal_softmax_fwd(x, scale, window=window, key_lengths=lengths)
+    plain = oracle.causal_softmax_fwd(x, scale, window=window)
+    causal = fb.causal_mask(s, sliding_window_width=window)[0, 0]
+    keys = torch.arange(s)
+    masked = (causal[None] | (keys[None, None, :] >= lengths.view(-1, 1, 1))).repeat_interleave(heads, dim=0)
+    assert int(util.raw_bits(y)[masked].abs().max()) == 0
+    empty = masked.all(-1)
+    assert empty[-heads:].all() and not empty[:heads].any()        # length 0 / full length
+    assert int(util.raw_bits(y)[empty].abs().max()) == 0
+    z = (x.double() * float(torch.tensor(scale, dtype=torch.float32))).masked_fill(masked, float("-inf"))
+    live = ~empty
+    util.assert_ulp_close(y[live], f64_softmax_rows(z[live]).to(dtype), 1, "vs float64")
+    ref = fb.torch_softmax_fallback(x.view(batch, heads, s, s), masked.view(batch, heads, s, s)[:, :1], scale)
+    util.assert_ulp_close(y[live], ref.view(-1, s, s)[live], 1, "vs torch fallback with the merged mask")
+    # a row whose causal band ends before the padding starts is the plain row
+    q = torch.arange(s)
+    untouched = (q[None, :] < lengths.view(-1, 1)).repeat_interleave(heads, dim=0)
+    assert torch.equal(util.raw_bits(y)[untouched], util.raw_bits(plain)[untouched])
+    assert not torch.equal(util.raw_bits(y)[live & ~untouched], util.raw_bits(plain)[live & ~untouched])
+    # lengths beyond the row change nothing; negative ones count as zero
+    assert torch.equal(util.raw_bits(oracle.causal_softmax_fwd(x, scale, window=window,
+                                                               key_lengths=torch.tensor([99, 40, 41, 1000]))),
+                       util.raw_bits(plain))
+    assert int(util.raw_bits(oracle.causal_softmax_fwd(x, scale, key_lengths=torch.tensor([-1, -5, 0, -2]))).abs().max()) == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_key_lengths_backward(dtype):
+    """dx = scale * y * (dy - sum_kept(dy * y)) on the kept band, +0 elsewhere: float64
+    evaluation of the Jacobian-vector product from the rounded y, and autograd through
+    the float64 softmax with the merged mask."""
+    batch, heads, s, scale = 3, 2, 24, 0.7
+    lengths = torch.tensor([24, 9, 0], dtype=torch.int32)
+    x = util.randn((batch * heads, s, s), dtype, seed=6, std=1.5)
+    dy = util.randn((batch * heads, s, s), dtype, seed=7)
+    y = oracle.causal_softmax_fwd(x, scale, key_lengths=lengths)
+    dx = oracle.softmax_bwd(dy, y, scale, causal=True, key_lengths=lengths)
+    keys = torch.arange(s)
+    masked = (fb.causal_mask(s)[0, 0][None] | (keys[None, None, :] >= lengths.view(-1, 1, 1))).repeat_interleave(heads, dim=0)
+    assert int(util.raw_bits(dx)[masked].abs().max()) == 0
+    yd, gd = y.double().masked_fill(masked, 0), dy.double().masked_fill(masked, 0)
+    f32scale = float(torch.tensor(scale, dtype=torch.float32))
+    want = f32scale * yd * (gd - (gd * yd).sum(-1, keepdim=True))
+    util.assert_softmax_bwd_close(dx, want.to(dtype), dy.masked_fill(masked, 0), y, scale, "vs float64 formula")
+    # autograd of the float64 softmax (exact y instead of the rounded one: looser)
+    live = ~masked.all(-1)
+    xd = x.double().requires_grad_(True)
+    p = torch.softmax((xd * f32scale).masked_fill(masked, float("-inf"))[live], -1)
+    p.backward(dy.double()[live])
+    err = (dx.double()[live] - xd.grad[live]).abs().max().item()
+    assert err <= 3 * 2.0 ** (-8 if dtype == torch.bfloat16 else -11) * xd.grad.abs().max().item()
