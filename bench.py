@@ -21,6 +21,9 @@ the drop-in extension modules (which call libneox_hotpath.so):
   alibi-1.4b     causal softmax fwd+bwd [128,2048,2048] bf16 with the AliBi bias of 16 heads added in the kernel
   rpe-bias-1.4b  causal softmax fwd+bwd [128,2048,2048] bf16 with a bias tensor [16,2048,2048] added in the kernel
 
+  mlp-gelu-1.4b  bias + tanh-GeLU fwd and bwd (with the bias gradient) on the MLP activation [2048*8, 8192] bf16
+  bias-residual-1.4b  residual + (x + bias) on the hidden state [2048*8, 2048] bf16
+
 `value` is algorithmic bytes per step / wall time per step (inputs resident in
 HBM, K steps bracketed by device synchronisation). Algorithmic bytes: softmax
 forward reads the lower triangle and writes the dense result; backward reads
@@ -226,6 +229,51 @@ def make_workload(name, torch, dev):
 
         cfg = {"workload": name, "qk": [s, b, h, d], "rotary_dim": d2}
         return step, kernel_bytes, {}, "rope_qk_fwd", "bf16", cfg
+
+    if name == "mlp-gelu-1.4b":
+        from megatron.model.activations import bias_gelu, _bias_gelu_backward
+
+        rows, cols = 2048 * 8, 8192
+        sets = []
+        for i in range(2):  # two buffer sets: a 256 MiB tensor alone would sit in the last-level cache
+            y = torch.empty((rows, cols), dtype=torch.bfloat16, device=dev)
+            g = torch.empty_like(y)
+            for r in range(0, rows, 2048):
+                y[r:r + 2048] = randn((2048, cols), 100 * i + r, torch.bfloat16, 2.0)
+                g[r:r + 2048] = randn((2048, cols), 100 * i + r + 1, torch.bfloat16)
+            sets.append((y, g))
+        bias = randn((cols,), 5, torch.bfloat16, 0.5)
+        n = rows * cols
+        kernel_bytes = {"bias_gelu_fwd": 2 * n * 2 + cols * 2, "bias_gelu_bwd": 3 * n * 2 + 2 * cols * 2}
+        state = {"i": 0}
+
+        def step(t):
+            y, g = sets[state["i"] % len(sets)]
+            state["i"] += 1
+            t.run("bias_gelu_fwd", lambda: bias_gelu(bias, y))
+            t.run("bias_gelu_bwd", lambda: _bias_gelu_backward(g, bias, y, True))
+
+        cfg = {"workload": name, "activation": [rows, cols], "bias_gradient": "fused column sums",
+               "bytes_convention": "every tensor element read or written once"}
+        return step, kernel_bytes, {}, "bias_gelu_bwd", "bf16", cfg
+
+    if name == "bias-residual-1.4b":
+        from megatron.model.fused_bias_dropout import bias_dropout_add_fused_inference
+
+        rows, cols = 2048 * 8, 2048
+        sets = [(randn((rows, cols), 10 * i, torch.bfloat16, 2.0), randn((rows, cols), 10 * i + 1, torch.bfloat16, 2.0))
+                for i in range(6)]  # 64 MiB tensors: rotate so that they come from HBM
+        bias = randn((cols,), 7, torch.bfloat16)
+        kernel_bytes = {"bias_add_residual": 3 * rows * cols * 2 + cols * 2}
+        state = {"i": 0}
+
+        def step(t):
+            x, res = sets[state["i"] % len(sets)]
+            state["i"] += 1
+            t.run("bias_add_residual", lambda: bias_dropout_add_fused_inference(x, bias, res, 0.0))
+
+        cfg = {"workload": name, "hidden_state": [rows, cols]}
+        return step, kernel_bytes, {}, "bias_add_residual", "bf16", cfg
 
     if name == "rope-c4-qkv-view":
         s, b, h, d, d2 = 4096, 4, 32, 128, 128

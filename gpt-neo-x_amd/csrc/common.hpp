@@ -1,4 +1,4 @@
-// Device-side helpers shared by the softmax and rotary kernels (gfx950, wave64).
+// Device-side helpers shared by all kernels of the library (gfx950, wave64).
 //
 // Everything here assumes a 64-lane wavefront and is compiled for gfx950 only.
 // The translation units are built with -ffp-contract=off: a fused multiply-add
@@ -105,6 +105,78 @@ __device__ __forceinline__ u32x4 pack8(const float (&f)[8])
 }
 
 // ---------------------------------------------------------------------------
+// Element types (the two 16-bit formats and fp32) behind one interface; a
+// 16-byte chunk holds kVec elements.
+// ---------------------------------------------------------------------------
+template <int DT>
+struct Elt;
+
+template <>
+struct Elt<NHP_BF16> {
+    using storage = uint16_t;
+    static constexpr int kVec = 8;
+    static __device__ __forceinline__ float load(const void* p, int64_t i)
+    {
+        return Half2<NHP_BF16>::from_bits(static_cast<const uint16_t*>(p)[i]);
+    }
+    static __device__ __forceinline__ void store(void* p, int64_t i, float v)
+    {
+        static_cast<uint16_t*>(p)[i] = Half2<NHP_BF16>::to_bits(v);
+    }
+    static __device__ __forceinline__ float round(float v) { return Half2<NHP_BF16>::round(v); }
+};
+template <>
+struct Elt<NHP_F16> {
+    using storage = uint16_t;
+    static constexpr int kVec = 8;
+    static __device__ __forceinline__ float load(const void* p, int64_t i)
+    {
+        return Half2<NHP_F16>::from_bits(static_cast<const uint16_t*>(p)[i]);
+    }
+    static __device__ __forceinline__ void store(void* p, int64_t i, float v)
+    {
+        static_cast<uint16_t*>(p)[i] = Half2<NHP_F16>::to_bits(v);
+    }
+    static __device__ __forceinline__ float round(float v) { return Half2<NHP_F16>::round(v); }
+};
+template <>
+struct Elt<NHP_F32> {
+    using storage = float;
+    static constexpr int kVec = 4;
+    static __device__ __forceinline__ float load(const void* p, int64_t i)
+    {
+        return static_cast<const float*>(p)[i];
+    }
+    static __device__ __forceinline__ void store(void* p, int64_t i, float v)
+    {
+        static_cast<float*>(p)[i] = v;
+    }
+    static __device__ __forceinline__ float round(float v) { return v; }
+};
+
+// A 16-byte chunk as V floats.
+template <int DT>
+__device__ __forceinline__ void chunk_to_float(const u32x4& raw, float (&f)[Elt<DT>::kVec])
+{
+    if constexpr (DT == NHP_F32) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) f[i] = bitcast<float>(raw[i]);
+    } else {
+        unpack8<DT>(raw, f);
+    }
+}
+template <int DT>
+__device__ __forceinline__ u32x4 float_to_chunk(const float (&f)[Elt<DT>::kVec])
+{
+    if constexpr (DT == NHP_F32) {
+        return u32x4{bitcast<uint32_t>(f[0]), bitcast<uint32_t>(f[1]), bitcast<uint32_t>(f[2]),
+                     bitcast<uint32_t>(f[3])};
+    } else {
+        return pack8<DT>(f);
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Streaming global memory access: every byte of these tensors is touched once,
 // so loads and stores carry the non-temporal hint.
 // ---------------------------------------------------------------------------
@@ -185,5 +257,13 @@ __device__ __forceinline__ float block_combine(float v, float* slots, int wave, 
 
 // 2^(x) with the raw v_exp_f32 instruction (about 1 ulp, no denormal results).
 __device__ __forceinline__ float exp2_raw(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// ---------------------------------------------------------------------------
+// Host-side launch checks
+// ---------------------------------------------------------------------------
+static inline bool ptr_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+// A grid of `blocks` workgroups of `threads` work-items must stay below 2^32 work-items.
+static inline bool grid_fits(int64_t blocks, int threads) { return blocks > 0 && blocks * threads < ((int64_t)1 << 32); }
+static inline int launch_result() { return hipGetLastError() == hipSuccess ? NHP_OK : NHP_ERR_LAUNCH; }
 
 }  // namespace nhp

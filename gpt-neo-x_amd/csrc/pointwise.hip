@@ -1,0 +1,387 @@
+// Element-wise kernels of the transformer layer for gfx950: bias + tanh-GeLU
+// (forward, backward with the bias gradient) and bias + residual add.
+//
+// Tensors are [rows, cols] with a [cols] bias. A workgroup of 256 threads
+// covers a tile of TW 16-byte chunks (TW a power of two) by `rows_per_block`
+// rows: thread (tr, tc) keeps the bias values of chunk column tc in registers
+// and walks down the rows tr, tr + 256/TW, ..., U rows in flight at a time.
+// Workgroups that are consecutive in launch order are adjacent along a row,
+// so the memory touched at any moment is a band of whole rows.
+//
+// Arithmetic: operands are widened to fp32, the expression is evaluated in
+// fp32 in the order of the reference's source, and the result is rounded once
+// to the storage type -- what the reference's TorchScript-fused kernels do.
+// tanh(u) is computed as 1 - 2 / (1 + e^(2u)) with the hardware exp2 and
+// reciprocal (absolute error about 1e-7, the same size as the rounding of the
+// `1 + tanh` that follows it in the reference formula).
+
+#include "common.hpp"
+
+#include <cstdlib>
+
+namespace nhp {
+
+constexpr int kPwThreads = 256;
+
+// tanh argument of bias_gelu, in source order (megatron/model/activations.py:81-82)
+__device__ __forceinline__ float gelu_inner(float x)
+{
+    const float a = 0.044715f * x;
+    const float b = a * x;
+    const float c = 1.0f + b;
+    const float d = 0.79788456f * x;
+    return d * c;
+}
+
+__device__ __forceinline__ float tanh_fast(float u)
+{
+    const float e = exp2_raw(u * (2.0f * kLog2e));
+    return 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + e);
+}
+
+__device__ __forceinline__ float gelu_fwd(float x)
+{
+    const float t = tanh_fast(gelu_inner(x));
+    return (x * 0.5f) * (1.0f + t);
+}
+
+// d gelu(x) / dx, the expression of bias_gelu_back (activations.py:88-97)
+__device__ __forceinline__ float gelu_grad(float x)
+{
+    const float t = tanh_fast(gelu_inner(x));
+    const float sech2 = 1.0f - t * t;
+    const float poly = 0.79788456f + (0.1070322243f * x) * x;
+    const float left = (0.5f * x) * (sech2 * poly);
+    const float right = 0.5f * (1.0f + t);
+    return left + right;
+}
+
+enum PointOp {
+    kGeluFwd = 0,        // out = gelu(a + bias)
+    kGeluBwd = 1,        // out = gelu'(b + bias) * a
+    kBiasAddResidual = 2 // out = b + (a + bias), b optional
+};
+
+// One element. `a`, `b`: the two tensor operands (b unused by kGeluFwd), `bv`: bias.
+template <int OP>
+__device__ __forceinline__ float point_op(float a, float b, float bv, bool has_b)
+{
+    if constexpr (OP == kGeluFwd) {
+        return gelu_fwd(bv + a);
+    } else if constexpr (OP == kGeluBwd) {
+        return gelu_grad(bv + b) * a;
+    } else {
+        const float v = a + bv;
+        return has_b ? b + v : v;
+    }
+}
+
+template <int OP>
+constexpr bool kNeedsB = (OP != kGeluFwd);
+
+// ---------------------------------------------------------------------------
+// Tiled kernel. COLSUM: also accumulate, per chunk column, the sum over the
+// tile's rows of the *stored* (rounded) results and write it to
+// partial[blockIdx.y][cols] (fp32); a second kernel adds the tiles up.
+// ---------------------------------------------------------------------------
+template <int DT, int OP, int TW, int U, bool COLSUM>
+__global__ void __launch_bounds__(kPwThreads)
+pointwise_kernel(void* out, const void* a, const void* b, const void* bias, float* partial, uint32_t rows,
+                 uint32_t cpr, uint32_t rows_per_block)
+{
+    constexpr int V = Elt<DT>::kVec;
+    constexpr int TR = kPwThreads / TW;
+    using S = typename Elt<DT>::storage;
+    const uint32_t tc = threadIdx.x % TW;
+    const uint32_t tr = threadIdx.x / TW;
+    const uint32_t cc = blockIdx.x * TW + tc;  // chunk column
+    const bool live = cc < cpr;
+    const uint32_t row0 = blockIdx.y * rows_per_block;
+    const uint32_t row_end = min(rows, row0 + rows_per_block);
+    const size_t row_elems = (size_t)cpr * V;
+    const bool has_b = kNeedsB<OP> && b != nullptr;
+
+    float bv[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) bv[j] = 0.0f;
+    if (live && bias != nullptr) chunk_to_float<DT>(load16(static_cast<const S*>(bias) + (size_t)cc * V), bv);
+
+    float sums[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) sums[j] = 0.0f;
+
+    if (live) {
+        for (uint32_t r = row0 + tr; r < row_end; r += TR * U) {
+            u32x4 ra[U], rb[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const uint32_t row = r + u * TR;
+                const size_t off = (size_t)row * row_elems + (size_t)cc * V;
+                ra[u] = u32x4{0, 0, 0, 0};
+                rb[u] = u32x4{0, 0, 0, 0};
+                if (row < row_end) {
+                    ra[u] = load16_stream(static_cast<const S*>(a) + off);
+                    if (has_b) rb[u] = load16_stream(static_cast<const S*>(b) + off);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const uint32_t row = r + u * TR;
+                if (row < row_end) {
+                    float fa[V], fb[V], fo[V];
+                    chunk_to_float<DT>(ra[u], fa);
+                    chunk_to_float<DT>(rb[u], fb);
+#pragma unroll
+                    for (int j = 0; j < V; ++j) fo[j] = point_op<OP>(fa[j], fb[j], bv[j], has_b);
+                    const u32x4 packed = float_to_chunk<DT>(fo);
+                    store16_stream(static_cast<S*>(out) + (size_t)row * row_elems + (size_t)cc * V, packed);
+                    if constexpr (COLSUM) {
+                        float stored[V];
+                        chunk_to_float<DT>(packed, stored);
+#pragma unroll
+                        for (int j = 0; j < V; ++j) sums[j] += stored[j];
+                    }
+                }
+            }
+        }
+    }
+
+    if constexpr (COLSUM) {
+        // combine the TR row-lanes of a chunk column in a fixed order
+        __shared__ float lds[TR > 1 ? kPwThreads * V : 1];
+        if constexpr (TR > 1) {
+#pragma unroll
+            for (int j = 0; j < V; ++j) lds[(tr * V + j) * TW + tc] = sums[j];
+            __syncthreads();
+            if (tr == 0) {
+#pragma unroll
+                for (int j = 0; j < V; ++j) {
+                    float s = lds[j * TW + tc];
+                    for (int t = 1; t < TR; ++t) s += lds[(t * V + j) * TW + tc];
+                    sums[j] = s;
+                }
+            }
+        }
+        if (tr == 0 && live) {
+            float* dst = partial + (size_t)blockIdx.y * row_elems + (size_t)cc * V;
+#pragma unroll
+            for (int j = 0; j < V; j += 4)
+                *reinterpret_cast<f32x4*>(dst + j) = f32x4{sums[j], sums[j + 1], sums[j + 2], sums[j + 3]};
+        }
+    }
+}
+
+// out[c] = storage(sum over tiles t of partial[t][c]); 64 columns by 4 tile slices per workgroup
+template <int DT>
+__global__ void __launch_bounds__(kPwThreads)
+column_sum_finish_kernel(void* out, const float* partial, uint32_t tiles, uint32_t cols)
+{
+    __shared__ float lds[4][64];
+    const uint32_t tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    const uint32_t c = blockIdx.x * 64 + tx;
+    float s = 0.0f;
+    if (c < cols)
+        for (uint32_t t = ty; t < tiles; t += 4) s += partial[(size_t)t * cols + c];
+    lds[ty][tx] = s;
+    __syncthreads();
+    if (ty == 0 && c < cols) Elt<DT>::store(out, c, (lds[0][tx] + lds[1][tx]) + (lds[2][tx] + lds[3][tx]));
+}
+
+// ---------------------------------------------------------------------------
+// Scalar kernels for shapes the chunked layout cannot take (cols not a
+// multiple of the chunk, unaligned pointers).
+// ---------------------------------------------------------------------------
+template <int DT, int OP>
+__global__ void __launch_bounds__(kPwThreads)
+pointwise_scalar_kernel(void* out, const void* a, const void* b, const void* bias, uint64_t total, uint64_t cols)
+{
+    const uint64_t i = (uint64_t)blockIdx.x * kPwThreads + threadIdx.x;
+    if (i >= total) return;
+    const bool has_b = kNeedsB<OP> && b != nullptr;
+    const float bv = bias != nullptr ? Elt<DT>::load(bias, (int64_t)(i % cols)) : 0.0f;
+    const float fa = Elt<DT>::load(a, (int64_t)i);
+    const float fb = has_b ? Elt<DT>::load(b, (int64_t)i) : 0.0f;
+    Elt<DT>::store(out, (int64_t)i, point_op<OP>(fa, fb, bv, has_b));
+}
+
+// one thread per column, rows in order (used after the scalar kernel has stored dx)
+template <int DT>
+__global__ void __launch_bounds__(kPwThreads)
+column_sum_scalar_kernel(void* out, const void* dx, uint64_t rows, uint64_t cols)
+{
+    const uint64_t c = (uint64_t)blockIdx.x * kPwThreads + threadIdx.x;
+    if (c >= cols) return;
+    float s = 0.0f;
+    for (uint64_t r = 0; r < rows; ++r) s += Elt<DT>::load(dx, (int64_t)(r * cols + c));
+    Elt<DT>::store(out, (int64_t)c, s);
+}
+
+// ---------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------
+#ifdef NHP_TUNING
+static int pw_tune(const char* name, int def)
+{
+    const char* v = getenv(name);
+    return v ? atoi(v) : def;
+}
+#else
+static inline int pw_tune(const char*, int def) { return def; }
+#endif
+
+struct TilePlan {
+    int tw;                  // chunk columns per workgroup (power of two <= 256)
+    uint32_t rows_per_block;
+    uint32_t col_tiles, row_tiles;
+};
+
+static int elem_size(int dt) { return dt == NHP_F32 ? 4 : 2; }
+
+// Tile shape for a [rows, cols] tensor of cpr chunks per row: as wide as the
+// row allows, and rows_per_block so that a thread moves a few hundred bytes.
+static TilePlan plan_tiles(int64_t rows, int64_t cpr)
+{
+    TilePlan p;
+    p.tw = 1;
+    while (p.tw < 256 && p.tw < cpr) p.tw *= 2;
+    const int tr = kPwThreads / p.tw;
+    const int per_thread = pw_tune("NHP_PW_ROWS", 32);  // rows walked by one thread
+    int64_t rpb = (int64_t)tr * per_thread;
+    while ((rows + rpb - 1) / rpb > 65535) rpb *= 2;  // grid.y limit
+    if (rpb > rows) rpb = rows;
+    p.rows_per_block = (uint32_t)rpb;
+    p.col_tiles = (uint32_t)((cpr + p.tw - 1) / p.tw);
+    p.row_tiles = (uint32_t)((rows + rpb - 1) / rpb);
+    return p;
+}
+
+template <int DT, int OP, bool COLSUM>
+static int launch_tiled(void* out, const void* a, const void* b, const void* bias, float* partial, int64_t rows,
+                        int64_t cpr, const TilePlan& p, hipStream_t st)
+{
+    const dim3 grid(p.col_tiles, p.row_tiles);
+    if (p.row_tiles > 65535u || !grid_fits((int64_t)p.col_tiles * p.row_tiles, kPwThreads)) return NHP_ERR_SHAPE;
+    constexpr int U = 4;
+#define CASE(TW_)                                                                                        \
+    case TW_:                                                                                            \
+        pointwise_kernel<DT, OP, TW_, U, COLSUM><<<grid, kPwThreads, 0, st>>>(                           \
+            out, a, b, bias, partial, (uint32_t)rows, (uint32_t)cpr, p.rows_per_block);                  \
+        break;
+    switch (p.tw) {
+        CASE(1) CASE(2) CASE(4) CASE(8) CASE(16) CASE(32) CASE(64) CASE(128) CASE(256)
+    default:
+        return NHP_ERR_SHAPE;
+    }
+#undef CASE
+    return launch_result();
+}
+
+// Runs OP over [rows, cols]; with dbias != nullptr (kGeluBwd only) also the column sums of the result.
+template <int DT, int OP>
+static int run_pointwise(void* out, const void* a, const void* b, const void* bias, void* dbias, float* workspace,
+                         int64_t rows, int64_t cols, hipStream_t st)
+{
+    constexpr int V = Elt<DT>::kVec;
+    const bool chunked = cols % V == 0 && ptr_aligned16(out) && ptr_aligned16(a) && ptr_aligned16(b) &&
+                         ptr_aligned16(bias) && ptr_aligned16(workspace) && rows < ((int64_t)1 << 31) &&
+                         cols / V < ((int64_t)1 << 31);
+    if (chunked) {
+        const int64_t cpr = cols / V;
+        const TilePlan p = plan_tiles(rows, cpr);
+        if (dbias == nullptr) return launch_tiled<DT, OP, false>(out, a, b, bias, nullptr, rows, cpr, p, st);
+        if constexpr (OP == kGeluBwd) {
+            int rc = launch_tiled<DT, OP, true>(out, a, b, bias, workspace, rows, cpr, p, st);
+            if (rc != NHP_OK) return rc;
+            const int64_t blocks = (cols + 63) / 64;
+            if (!grid_fits(blocks, kPwThreads)) return NHP_ERR_SHAPE;
+            column_sum_finish_kernel<DT><<<(uint32_t)blocks, kPwThreads, 0, st>>>(dbias, workspace, p.row_tiles,
+                                                                                (uint32_t)cols);
+            return launch_result();
+        }
+        return NHP_ERR_SHAPE;
+    }
+    const int64_t total = rows * cols;
+    const int64_t blocks = (total + kPwThreads - 1) / kPwThreads;
+    if (!grid_fits(blocks, kPwThreads)) return NHP_ERR_SHAPE;
+    pointwise_scalar_kernel<DT, OP><<<(uint32_t)blocks, kPwThreads, 0, st>>>(out, a, b, bias, (uint64_t)total,
+                                                                             (uint64_t)cols);
+    int rc = launch_result();
+    if (rc != NHP_OK || dbias == nullptr) return rc;
+    column_sum_scalar_kernel<DT><<<(uint32_t)((cols + kPwThreads - 1) / kPwThreads), kPwThreads, 0, st>>>(
+        dbias, out, (uint64_t)rows, (uint64_t)cols);
+    return launch_result();
+}
+
+template <int OP>
+static int dispatch_pointwise(void* out, const void* a, const void* b, const void* bias, void* dbias,
+                              float* workspace, int64_t rows, int64_t cols, int dtype, hipStream_t st)
+{
+    switch (dtype) {
+    case NHP_F16:
+        return run_pointwise<NHP_F16, OP>(out, a, b, bias, dbias, workspace, rows, cols, st);
+    case NHP_BF16:
+        return run_pointwise<NHP_BF16, OP>(out, a, b, bias, dbias, workspace, rows, cols, st);
+    case NHP_F32:
+        return run_pointwise<NHP_F32, OP>(out, a, b, bias, dbias, workspace, rows, cols, st);
+    default:
+        return NHP_ERR_DTYPE;
+    }
+}
+
+static int check_shape(int64_t rows, int64_t cols, int dtype)
+{
+    if (dtype != NHP_F16 && dtype != NHP_BF16 && dtype != NHP_F32) return NHP_ERR_DTYPE;
+    if (rows < 0 || cols < 0) return NHP_ERR_SHAPE;
+    if (rows > 0 && cols > ((int64_t)1 << 62) / rows) return NHP_ERR_SHAPE;
+    return NHP_OK;
+}
+
+}  // namespace nhp
+
+using namespace nhp;
+
+extern "C" {
+
+int nhp_bias_gelu_fwd(void* out, const void* y, const void* bias, int64_t rows, int64_t cols, int dtype,
+                      void* stream)
+{
+    if (int rc = check_shape(rows, cols, dtype)) return rc;
+    if (rows == 0 || cols == 0) return NHP_OK;
+    if (!out || !y) return NHP_ERR_NULL;
+    return dispatch_pointwise<kGeluFwd>(out, y, nullptr, bias, nullptr, nullptr, rows, cols, dtype,
+                                        static_cast<hipStream_t>(stream));
+}
+
+int64_t nhp_bias_gelu_bwd_workspace_bytes(int64_t rows, int64_t cols, int dtype)
+{
+    if (check_shape(rows, cols, dtype) != NHP_OK || rows == 0 || cols == 0) return 0;
+    const int v = 16 / elem_size(dtype);
+    if (cols % v != 0) return 0;  // the scalar path sums the stored result directly
+    const TilePlan p = plan_tiles(rows, cols / v);
+    return (int64_t)p.row_tiles * cols * (int64_t)sizeof(float);
+}
+
+int nhp_bias_gelu_bwd(void* dx, const void* g, const void* y, const void* bias, void* dbias, void* workspace,
+                      int64_t rows, int64_t cols, int dtype, void* stream)
+{
+    if (int rc = check_shape(rows, cols, dtype)) return rc;
+    if (rows == 0 || cols == 0) return NHP_OK;  // dbias of an empty tensor is left untouched
+    if (!dx || !g || !y) return NHP_ERR_NULL;
+    if (dbias != nullptr && workspace == nullptr && nhp_bias_gelu_bwd_workspace_bytes(rows, cols, dtype) > 0)
+        return NHP_ERR_NULL;
+    if (dbias != nullptr && (dbias == dx || dbias == workspace)) return NHP_ERR_ALIAS;
+    return dispatch_pointwise<kGeluBwd>(dx, g, y, bias, dbias, static_cast<float*>(workspace), rows, cols, dtype,
+                                        static_cast<hipStream_t>(stream));
+}
+
+int nhp_bias_add_residual(void* out, const void* x, const void* bias, const void* residual, int64_t rows,
+                          int64_t cols, int dtype, void* stream)
+{
+    if (int rc = check_shape(rows, cols, dtype)) return rc;
+    if (rows == 0 || cols == 0) return NHP_OK;
+    if (!out || !x) return NHP_ERR_NULL;
+    return dispatch_pointwise<kBiasAddResidual>(out, x, residual, bias, nullptr, nullptr, rows, cols, dtype,
+                                                static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -24,77 +24,6 @@
 
 namespace nhp {
 
-// ---------------------------------------------------------------------------
-// element types
-// ---------------------------------------------------------------------------
-template <int DT>
-struct Elt;
-
-template <>
-struct Elt<NHP_BF16> {
-    using storage = uint16_t;
-    static constexpr int kVec = 8;
-    static __device__ __forceinline__ float load(const void* p, int64_t i)
-    {
-        return Half2<NHP_BF16>::from_bits(static_cast<const uint16_t*>(p)[i]);
-    }
-    static __device__ __forceinline__ void store(void* p, int64_t i, float v)
-    {
-        static_cast<uint16_t*>(p)[i] = Half2<NHP_BF16>::to_bits(v);
-    }
-    static __device__ __forceinline__ float round(float v) { return Half2<NHP_BF16>::round(v); }
-};
-template <>
-struct Elt<NHP_F16> {
-    using storage = uint16_t;
-    static constexpr int kVec = 8;
-    static __device__ __forceinline__ float load(const void* p, int64_t i)
-    {
-        return Half2<NHP_F16>::from_bits(static_cast<const uint16_t*>(p)[i]);
-    }
-    static __device__ __forceinline__ void store(void* p, int64_t i, float v)
-    {
-        static_cast<uint16_t*>(p)[i] = Half2<NHP_F16>::to_bits(v);
-    }
-    static __device__ __forceinline__ float round(float v) { return Half2<NHP_F16>::round(v); }
-};
-template <>
-struct Elt<NHP_F32> {
-    using storage = float;
-    static constexpr int kVec = 4;
-    static __device__ __forceinline__ float load(const void* p, int64_t i)
-    {
-        return static_cast<const float*>(p)[i];
-    }
-    static __device__ __forceinline__ void store(void* p, int64_t i, float v)
-    {
-        static_cast<float*>(p)[i] = v;
-    }
-    static __device__ __forceinline__ float round(float v) { return v; }
-};
-
-// A 16-byte chunk as V floats.
-template <int DT>
-__device__ __forceinline__ void chunk_to_float(const u32x4& raw, float (&f)[Elt<DT>::kVec])
-{
-    if constexpr (DT == NHP_F32) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) f[i] = bitcast<float>(raw[i]);
-    } else {
-        unpack8<DT>(raw, f);
-    }
-}
-template <int DT>
-__device__ __forceinline__ u32x4 float_to_chunk(const float (&f)[Elt<DT>::kVec])
-{
-    if constexpr (DT == NHP_F32) {
-        return u32x4{bitcast<uint32_t>(f[0]), bitcast<uint32_t>(f[1]), bitcast<uint32_t>(f[2]),
-                     bitcast<uint32_t>(f[3])};
-    } else {
-        return pack8<DT>(f);
-    }
-}
-
 // out = round(round(x*c) +/- round(r*s)); the three roundings of the scalar types.
 // Negating r or s before the product equals subtracting the rounded product
 // (rounding to nearest is symmetric), so the sign is taken as a flag.

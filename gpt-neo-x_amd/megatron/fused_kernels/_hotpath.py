@@ -51,6 +51,10 @@ def _declare(lib):
         "nhp_rope_cached_qk_bwd": ([vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, p64, p64, p64, p64, ci, ci, vp], ci),
         "nhp_rope_freqs_fwd": ([vp, vp, vp, i64, i64, i64, i64, i64, p64, p64, ci, vp], ci),
         "nhp_rope_freqs_bwd": ([vp, vp, vp, i64, i64, i64, i64, i64, p64, p64, ci, vp], ci),
+        "nhp_bias_gelu_fwd": ([vp, vp, vp, i64, i64, ci, vp], ci),
+        "nhp_bias_gelu_bwd": ([vp, vp, vp, vp, vp, vp, i64, i64, ci, vp], ci),
+        "nhp_bias_gelu_bwd_workspace_bytes": ([i64, i64, ci], i64),
+        "nhp_bias_add_residual": ([vp, vp, vp, vp, i64, i64, ci, vp], ci),
     }
     for name, (args, res) in sigs.items():
         fn = getattr(lib, name)  # AttributeError if the symbol is missing

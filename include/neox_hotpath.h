@@ -267,6 +267,63 @@ int nhp_rope_freqs_bwd(void* out, const void* in, const float* freqs,
                        const int64_t in_stride[4], const int64_t out_stride[4],
                        int dtype, void* stream);
 
+/* ------------------------------------------------------------------------
+ * Element-wise neighbours of attention in the transformer layer
+ *
+ * The reference reaches these through TorchScript functions, not through an
+ * extension module; the entry points below are what a binding for those
+ * functions calls. Tensors are dense [rows, cols] (rows = all leading
+ * dimensions flattened), the bias is [cols]. dtype: NHP_F16, NHP_BF16 or
+ * NHP_F32, the same for every operand. Operands are widened to fp32, the
+ * expression is evaluated in fp32 in the order of the reference's source and
+ * rounded once to the storage type (what a fused TorchScript kernel does;
+ * eager 16-bit torch rounds after every operator). Outputs may alias inputs.
+ * ---------------------------------------------------------------------- */
+
+/*
+ * out = x * 0.5 * (1 + tanh(0.79788456 * x * (1 + 0.044715 * x * x))), x = bias + y.
+ * bias may be NULL.
+ *
+ * Replaces bias_gelu
+ *   megatron/model/activations.py:79-82 (called from GeLUFunction.forward :101-105,
+ *   used by ParallelMLP, megatron/model/transformer.py:176-186)
+ */
+int nhp_bias_gelu_fwd(void* out, const void* y, const void* bias,
+                      int64_t rows, int64_t cols, int dtype, void* stream);
+
+/*
+ * dx = ff * g with x = bias + y, t = tanh(0.79788456 * x * (1 + 0.044715 * x * x)),
+ * ff = 0.5 * x * ((1 - t*t) * (0.79788456 + 0.1070322243 * x * x)) + 0.5 * (1 + t).
+ *
+ * dbias (optional, [cols] in `dtype`): the column sums of the stored dx,
+ * accumulated in fp32 -- the reduction autograd performs on the second tensor
+ * GeLUFunction.backward returns. It needs `workspace`, a device buffer of
+ * nhp_bias_gelu_bwd_workspace_bytes(rows, cols, dtype) bytes, 16-byte aligned,
+ * owned by the caller (0 bytes: none needed, NULL is accepted). The sums are
+ * formed in a fixed order: results are reproducible from run to run.
+ *
+ * Replaces bias_gelu_back
+ *   megatron/model/activations.py:88-97 (GeLUFunction.backward :107-112)
+ */
+int nhp_bias_gelu_bwd(void* dx, const void* g, const void* y, const void* bias,
+                      void* dbias, void* workspace,
+                      int64_t rows, int64_t cols, int dtype, void* stream);
+
+int64_t nhp_bias_gelu_bwd_workspace_bytes(int64_t rows, int64_t cols, int dtype);
+
+/*
+ * out = residual + (x + bias): bias_dropout_add with dropout switched off
+ * (training False or prob 0, when torch's dropout is the identity).
+ * bias and residual may each be NULL.
+ *
+ * Replaces bias_dropout_add / bias_dropout_add_fused_inference (and
+ * bias_dropout_add_fused_train with prob = 0)
+ *   megatron/model/fused_bias_dropout.py:28-60
+ *   (call sites megatron/model/transformer.py:1168-1178,1229-1246,1269-1320)
+ */
+int nhp_bias_add_residual(void* out, const void* x, const void* bias, const void* residual,
+                          int64_t rows, int64_t cols, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

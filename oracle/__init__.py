@@ -50,6 +50,10 @@ def lib():
         L.oracle_masked_softmax_fwd.argtypes = [vp, vp, vp, f32, i64, i64, i64, i64, i64, ci]
         L.oracle_softmax_bwd.argtypes = [vp, vp, vp, f32, i64, i64, i64, ci, ci]
         L.oracle_batch_per_block.argtypes = [i64, ci]
+        L.oracle_bias_gelu_fwd.argtypes = [vp, vp, vp, i64, i64, ci]
+        L.oracle_bias_gelu_bwd.argtypes = [vp, vp, vp, vp, i64, i64, ci]
+        L.oracle_column_sum.argtypes = [vp, vp, i64, i64, ci]
+        L.oracle_bias_add_residual.argtypes = [vp, vp, vp, vp, i64, i64, ci]
         p64 = ctypes.POINTER(i64)
         L.oracle_rope_cached.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, p64, p64, ci, ci, ci]
         L.oracle_rope_freqs.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, p64, p64, ci, ci]
@@ -182,4 +186,64 @@ def rope_freqs(t, freqs, backward=False, transpose_output=False):
     _check(lib().oracle_rope_freqs(out.data_ptr(), t.data_ptr(), freqs.data_ptr(), s, b, h, d, d2,
                                    _strides4(t), _strides4(out), _DT[t.dtype], 1 if backward else 0),
            "rope_freqs")
+    return out
+
+
+# ---------------------------------------------------------------------------
+# element-wise layer functions (layer_semantics.c)
+# ---------------------------------------------------------------------------
+def _rows_cols(t):
+    cols = t.size(-1)
+    return t.numel() // max(cols, 1), cols
+
+
+def _opt_ptr(t, like, what):
+    if t is None:
+        return None, None
+    t = _cpu_contig(t)
+    assert t.dtype == like.dtype, what
+    return t, t.data_ptr()
+
+
+def bias_gelu_fwd(y, bias=None):
+    """gelu_tanh(bias + y); y: [..., cols], bias: [cols] or None."""
+    y = _cpu_contig(y)
+    out = torch.empty_like(y)
+    rows, cols = _rows_cols(y)
+    bias, bp = _opt_ptr(bias, y, "bias dtype")
+    _check(lib().oracle_bias_gelu_fwd(out.data_ptr(), y.data_ptr(), bp, rows, cols, _DT[y.dtype]), "bias_gelu_fwd")
+    return out
+
+
+def bias_gelu_bwd(g, y, bias=None):
+    """gelu_tanh'(bias + y) * g."""
+    y = _cpu_contig(y)
+    g = _cpu_contig(g)
+    assert g.shape == y.shape and g.dtype == y.dtype
+    dx = torch.empty_like(y)
+    rows, cols = _rows_cols(y)
+    bias, bp = _opt_ptr(bias, y, "bias dtype")
+    _check(lib().oracle_bias_gelu_bwd(dx.data_ptr(), g.data_ptr(), y.data_ptr(), bp, rows, cols, _DT[y.dtype]),
+           "bias_gelu_bwd")
+    return dx
+
+
+def column_sum(t):
+    """Sum over all leading dimensions, fp32 accumulation, result [cols] in t.dtype."""
+    t = _cpu_contig(t)
+    rows, cols = _rows_cols(t)
+    out = torch.empty(cols, dtype=t.dtype)
+    _check(lib().oracle_column_sum(out.data_ptr(), t.data_ptr(), rows, cols, _DT[t.dtype]), "column_sum")
+    return out
+
+
+def bias_add_residual(x, bias=None, residual=None):
+    """residual + (x + bias), one rounding."""
+    x = _cpu_contig(x)
+    out = torch.empty_like(x)
+    rows, cols = _rows_cols(x)
+    bias, bp = _opt_ptr(bias, x, "bias dtype")
+    residual, rp = _opt_ptr(residual, x, "residual dtype")
+    _check(lib().oracle_bias_add_residual(out.data_ptr(), x.data_ptr(), bp, rp, rows, cols, _DT[x.dtype]),
+           "bias_add_residual")
     return out

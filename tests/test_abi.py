@@ -39,10 +39,12 @@ def test_every_header_comment_cites_the_reference():
     for name in declared_functions():
         if name in ("nhp_abi_version", "nhp_status_string", "nhp_softmax_max_resident_row"):
             continue
+        if name.endswith("_workspace_bytes"):  # size query, documented with the function it serves
+            continue
         before = text[: text.index(name + "(")]
         comment = before[before.rindex("/*") :]
         # the backward/forward pairs of the rotary functions share one comment
-        assert "megatron/fused_kernels/" in comment or name.startswith("nhp_rope_"), name
+        assert "megatron/fused_kernels/" in comment or "megatron/model/" in comment or name.startswith("nhp_rope_"), name
     assert text.count("Replaces ") >= 7
 
 

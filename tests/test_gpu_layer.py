@@ -1,0 +1,213 @@
+"""GPU parity of the element-wise layer kernels (bias + tanh-GeLU forward/backward
+with the fused bias gradient, bias + residual add) through the C ABI and the
+Python functions, against the CPU oracle.
+
+Tolerances: GeLU results within 2 representable values of the oracle, or within the
+fp32 rounding noise the reference's own expression carries (util.gelu_noise);
+bias + residual add bit-exact; column sums within fp32 summation noise."""
+import ctypes
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle
+import util
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+DTYPES = [torch.bfloat16, torch.float16, torch.float32]
+IDS = ["bf16", "fp16", "fp32"]
+
+
+def ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def abi_gelu_fwd(hp, y, bias, out=None):
+    out = torch.empty_like(y) if out is None else out
+    cols = y.size(-1)
+    rc = hp.lib().nhp_bias_gelu_fwd(out.data_ptr(), y.data_ptr(), ptr(bias), y.numel() // cols, cols,
+                                    hp.dtype_code(y, "t"), None)
+    assert rc == 0, hp.lib().nhp_status_string(rc)
+    return out
+
+
+def abi_gelu_bwd(hp, g, y, bias, with_dbias=True):
+    dx = torch.empty_like(y)
+    cols = y.size(-1)
+    rows = y.numel() // cols
+    code = hp.dtype_code(y, "t")
+    dbias = torch.full((cols,), float("nan"), dtype=y.dtype, device=y.device) if with_dbias else None
+    nbytes = hp.lib().nhp_bias_gelu_bwd_workspace_bytes(rows, cols, code)
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=y.device) if with_dbias else None
+    rc = hp.lib().nhp_bias_gelu_bwd(dx.data_ptr(), g.data_ptr(), y.data_ptr(), ptr(bias), ptr(dbias), ptr(ws),
+                                    rows, cols, code, None)
+    assert rc == 0, hp.lib().nhp_status_string(rc)
+    return dx, dbias
+
+
+# rows, cols: wide and narrow tiles, partial tiles, column counts that are not a multiple of the chunk
+SHAPES = [(1, 8), (3, 16), (37, 96), (5, 1000), (300, 2048), (64, 8192), (1000, 24), (129, 2056), (7, 4100), (2, 5)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: f"{s[0]}x{s[1]}")
+def test_bias_gelu_forward_backward_vs_oracle(hotpath, shape, dtype):
+    rows, cols = shape
+    print(f"bias_gelu case {shape} {dtype}", flush=True)
+    y = util.randn((rows, cols), dtype, seed=rows + cols, std=3.0)
+    bias = util.randn((cols,), dtype, seed=cols, std=0.5)
+    g = util.randn((rows, cols), dtype, seed=rows, std=1.0)
+    x32 = bias.float() + y.float()
+    got = abi_gelu_fwd(hotpath, y.to(DEV), bias.to(DEV)).cpu()
+    util.assert_close_ulp_or_noise(got, oracle.bias_gelu_fwd(y, bias), 2, util.gelu_noise(x32), "fwd")
+    dx, dbias = abi_gelu_bwd(hotpath, g.to(DEV), y.to(DEV), bias.to(DEV))
+    dx, dbias = dx.cpu(), dbias.cpu()
+    util.assert_close_ulp_or_noise(dx, oracle.bias_gelu_bwd(g, y, bias), 2, util.gelu_noise(x32, g), "bwd")
+    # the bias gradient is the column sum of the dx that was stored
+    noise = dx.float().abs().sum(0) * 16 * util.EPS32
+    util.assert_close_ulp_or_noise(dbias, oracle.column_sum(dx), 1, noise, "dbias")
+    dx_only, none = abi_gelu_bwd(hotpath, g.to(DEV), y.to(DEV), bias.to(DEV), with_dbias=False)
+    assert none is None and torch.equal(util.raw_bits(dx_only.cpu()), util.raw_bits(dx))
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_bias_gelu_edge_cases(hotpath, dtype):
+    # no bias, special values, in place, unaligned pointers, empty tensors
+    v = torch.tensor([[0.0, -0.0, 30.0, -30.0, float("inf"), float("-inf"), float("nan"), 1.0]], dtype=dtype)
+    got = abi_gelu_fwd(hotpath, v.to(DEV), None).cpu()
+    want = oracle.bias_gelu_fwd(v, None)
+    util.assert_ulp_close(got, want, 2, "special values")
+    y = util.randn((40, 256), dtype, seed=1, std=3.0)
+    yd = y.to(DEV)
+    inplace = abi_gelu_fwd(hotpath, yd, None, out=yd).cpu()
+    util.assert_close_ulp_or_noise(inplace, oracle.bias_gelu_fwd(y, None), 2, util.gelu_noise(y), "in place")
+    # a view that starts one element into a buffer is not 16-byte aligned
+    buf = torch.zeros(40 * 256 + 8, dtype=dtype, device=DEV)
+    shifted = buf[1:1 + 40 * 256].view(40, 256)
+    shifted.copy_(y)
+    util.assert_close_ulp_or_noise(abi_gelu_fwd(hotpath, shifted, None).cpu(), oracle.bias_gelu_fwd(y, None), 2,
+                                   util.gelu_noise(y), "unaligned")
+    empty = torch.empty((0, 64), dtype=dtype, device=DEV)
+    assert abi_gelu_fwd(hotpath, empty, None).shape == (0, 64)
+
+
+def test_bias_gelu_results_are_reproducible(hotpath):
+    y = util.randn((777, 2048), torch.bfloat16, seed=1, std=3.0).to(DEV)
+    bias = util.randn((2048,), torch.bfloat16, seed=2).to(DEV)
+    g = util.randn((777, 2048), torch.bfloat16, seed=3).to(DEV)
+    first = abi_gelu_bwd(hotpath, g, y, bias)
+    for _ in range(3):
+        again = abi_gelu_bwd(hotpath, g, y, bias)
+        assert torch.equal(util.raw_bits(first[0]), util.raw_bits(again[0]))
+        assert torch.equal(util.raw_bits(first[1]), util.raw_bits(again[1]))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+def test_gelu_function_autograd(dtype):
+    """bias_gelu_impl under autograd: output, input gradient and the reduced bias gradient against
+    torch's own tanh-GeLU evaluated in fp32 on the same device."""
+    from megatron.model.activations import bias_gelu, bias_gelu_back, bias_gelu_impl
+
+    s, b, h = 64, 3, 1024
+    y = util.randn((s, b, h), dtype, seed=1, std=2.0).to(DEV).requires_grad_(True)
+    bias = util.randn((h,), dtype, seed=2, std=0.5).to(DEV).requires_grad_(True)
+    g = util.randn((s, b, h), dtype, seed=3).to(DEV)
+    out = bias_gelu_impl(y, bias)
+    out.backward(g)
+    assert out.shape == (s, b, h) and y.grad.shape == (s, b, h) and bias.grad.shape == (h,)
+    yr = y.detach().float().requires_grad_(True)
+    br = bias.detach().float().requires_grad_(True)
+    ref = F.gelu(yr + br, approximate="tanh")
+    ref.backward(g.float())
+    x32 = (yr + br).detach().cpu()
+    util.assert_close_ulp_or_noise(out.detach().cpu(), ref.detach().to(dtype).cpu(), 2, util.gelu_noise(x32), "out")
+    util.assert_close_ulp_or_noise(y.grad.cpu(), yr.grad.to(dtype).cpu(), 2, util.gelu_noise(x32, g.cpu()), "dx")
+    # the reduced gradient sums rounded values: compare with the fp32 sum within the rounding of s*b terms
+    tol = (yr.grad.abs().sum(dim=(0, 1)) * 2.0 ** (-8 if dtype == torch.bfloat16 else -11)).cpu()
+    assert torch.all((bias.grad.float().cpu() - br.grad.cpu()).abs() <= tol + 1e-6)
+    # the two plain functions
+    assert torch.equal(util.raw_bits(bias_gelu(bias.detach(), y.detach()).cpu()), util.raw_bits(out.detach().cpu()))
+    assert torch.equal(util.raw_bits(bias_gelu_back(g, bias.detach(), y.detach()).cpu()), util.raw_bits(y.grad.cpu()))
+
+
+def test_bias_gelu_rejects_cpu_tensors_and_mismatches():
+    from megatron.model.activations import bias_gelu
+
+    with pytest.raises(RuntimeError):
+        bias_gelu(torch.zeros(8), torch.zeros(4, 8))
+    with pytest.raises(RuntimeError):
+        bias_gelu(torch.zeros(4, device=DEV), torch.zeros(4, 8, device=DEV))
+    with pytest.raises(RuntimeError):
+        bias_gelu(torch.zeros(8, device=DEV, dtype=torch.float16), torch.zeros(4, 8, device=DEV))
+
+
+def test_bias_gelu_full_size(hotpath):
+    """The MLP activation of the 1.4B configuration: [2048*8, 8192] bf16. Sampled rows against the
+    oracle, everything against torch's fp32 tanh-GeLU on the device."""
+    rows, cols = 2048 * 8, 8192
+    gen = torch.Generator(device=DEV).manual_seed(0)
+    y = (torch.randn((rows, cols), generator=gen, device=DEV) * 2).bfloat16()
+    bias = (torch.randn((cols,), generator=gen, device=DEV) * 0.5).bfloat16()
+    g = torch.randn((rows, cols), generator=gen, device=DEV).bfloat16()
+    out = abi_gelu_fwd(hotpath, y, bias)
+    dx, dbias = abi_gelu_bwd(hotpath, g, y, bias)
+    pick = torch.tensor([0, 1, 31, 32, 4095, 9000, rows - 1])
+    yc, gc, bc = y[pick.to(DEV)].cpu(), g[pick.to(DEV)].cpu(), bias.cpu()
+    x32 = bc.float() + yc.float()
+    util.assert_close_ulp_or_noise(out[pick.to(DEV)].cpu(), oracle.bias_gelu_fwd(yc, bc), 2, util.gelu_noise(x32), "fwd")
+    util.assert_close_ulp_or_noise(dx[pick.to(DEV)].cpu(), oracle.bias_gelu_bwd(gc, yc, bc), 2,
+                                   util.gelu_noise(x32, gc), "bwd")
+    ref = F.gelu(y.float() + bias.float(), approximate="tanh")
+    err = (out.float() - ref).abs()
+    assert bool((err <= 2.0**-7 * ref.abs() + 1e-6).all())
+    del ref, err
+    want_dbias = dx.float().sum(0)
+    scale = dx.float().abs().sum(0)
+    assert bool(((dbias.float() - want_dbias).abs() <= 2.0**-8 * want_dbias.abs() + scale * 16 * util.EPS32).all())
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("shape", [(1, 8), (37, 96), (5, 1000), (300, 2048), (1000, 24), (64, 8192)],
+                         ids=lambda s: f"{s[0]}x{s[1]}")
+def test_bias_add_residual_bit_exact(hotpath, shape, dtype):
+    rows, cols = shape
+    x = util.randn((rows, cols), dtype, seed=1, std=2.0)
+    bias = util.randn((cols,), dtype, seed=2)
+    res = util.randn((rows, cols), dtype, seed=3, std=2.0)
+    xd = x.to(DEV)
+    for b, r in ((bias, res), (None, res), (bias, None), (None, None)):
+        out = torch.empty((rows, cols), dtype=dtype, device=DEV)
+        bd = None if b is None else b.to(DEV)  # named, so that the device copies outlive the launch
+        rd = None if r is None else r.to(DEV)
+        rc = hotpath.lib().nhp_bias_add_residual(out.data_ptr(), xd.data_ptr(), ptr(bd), ptr(rd), rows, cols,
+                                                 hotpath.dtype_code(x, "t"), None)
+        assert rc == 0
+        assert torch.equal(util.raw_bits(out.cpu()), util.raw_bits(oracle.bias_add_residual(x, b, r)))
+
+
+def test_bias_dropout_add_functions():
+    from megatron.model.fused_bias_dropout import (bias_dropout_add_fused_inference, bias_dropout_add_fused_train,
+                                                    get_bias_dropout_add)
+
+    dtype = torch.bfloat16
+    x = util.randn((32, 4, 512), dtype, seed=1, std=2.0)
+    bias = util.randn((512,), dtype, seed=2)
+    res = util.randn((32, 4, 512), dtype, seed=3, std=2.0)
+    want = oracle.bias_add_residual(x, bias, res)
+    xd = x.to(DEV).requires_grad_(True)
+    bd = bias.to(DEV).requires_grad_(True)
+    rd = res.to(DEV).requires_grad_(True)
+    out = bias_dropout_add_fused_inference(xd, bd, rd, 0.1)
+    assert torch.equal(util.raw_bits(out.detach().cpu()), util.raw_bits(want))
+    g = util.randn(x.shape, dtype, seed=4).to(DEV)
+    out.backward(g)
+    assert torch.equal(xd.grad, g) and torch.equal(rd.grad, g)
+    assert torch.allclose(bd.grad.float(), g.float().sum(dim=(0, 1)), rtol=2.0**-7, atol=1e-2)
+    same = bias_dropout_add_fused_train(x.to(DEV), bias.to(DEV), res.to(DEV), 0.0)
+    assert torch.equal(util.raw_bits(same.cpu()), util.raw_bits(want))
+    assert torch.equal(util.raw_bits(get_bias_dropout_add(False)(x.to(DEV), bias.to(DEV), res.to(DEV), 0.5).cpu()),
+                       util.raw_bits(want))
+    with pytest.raises(NotImplementedError):
+        bias_dropout_add_fused_train(x.to(DEV), bias.to(DEV), res.to(DEV), 0.1)

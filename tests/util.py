@@ -85,6 +85,35 @@ def assert_softmax_bwd_close(got, want, dy, y, scale, what=""):
     return int(ulp_distance(got, want).max())
 
 
+def assert_close_ulp_or_noise(got, want, max_ulp, noise, what=""):
+    """Every element within max_ulp representable values of `want`, or within the
+    absolute bound `noise` (a tensor: the fp32 rounding noise that the expression
+    being tested carries by construction) plus max_ulp spacings."""
+    got, want = got.cpu(), want.cpu()
+    nan_g, nan_w = torch.isnan(got.float()), torch.isnan(want.float())
+    assert torch.equal(nan_g, nan_w), f"{what}: NaN pattern differs"
+    d = ulp_distance(got, want)
+    diff = (got.float() - want.float()).abs()
+    ok = (d <= max_ulp) | (diff <= noise.float() + max_ulp * ulp_size(want)) | nan_w
+    if not ok.all():
+        idx = int((~ok).flatten().nonzero()[0])
+        raise AssertionError(
+            f"{what}: element {idx}: got {got.flatten()[idx].item()!r} want {want.flatten()[idx].item()!r} "
+            f"({int(d.flatten()[idx])} ulp, allowed noise {noise.float().expand_as(diff).flatten()[idx].item():.3e})")
+    return int(torch.where(nan_w, torch.zeros_like(d), d).max()) if d.numel() else 0
+
+
+def gelu_noise(x, g=None):
+    """fp32 rounding noise of the reference's tanh-GeLU expressions at input x (fp32
+    tensor): `1 + tanh(u)` and `1 - tanh(u)^2` are formed from a tanh that is only
+    known to about 2^-23 absolute, so the forward result carries |x| * 2^-23 of
+    noise and the derivative (1 + |x|^3) * 2^-22, whatever their own size."""
+    x = x.float().abs()
+    if g is None:
+        return x * 2.0**-22
+    return (1 + x**3) * g.float().abs() * 2.0**-21
+
+
 # ---------------------------------------------------------------------------
 # direct C-ABI calls on torch GPU tensors
 # ---------------------------------------------------------------------------
