@@ -2,11 +2,11 @@
 // (forward, backward with the bias gradient) and bias + residual add.
 //
 // Tensors are [rows, cols] with a [cols] bias. A workgroup of 256 threads
-// covers a tile of TW 16-byte chunks (TW a power of two) by `rows_per_block`
-// rows: thread (tr, tc) keeps the bias values of chunk column tc in registers
-// and walks down the rows tr, tr + 256/TW, ..., U rows in flight at a time.
-// Workgroups that are consecutive in launch order are adjacent along a row,
-// so the memory touched at any moment is a band of whole rows.
+// covers TW 16-byte chunk columns (TW a power of two, at most 64: a wave reads
+// 1 KiB of a row) by 256/TW * U rows per step; thread (tr, tc) keeps the bias
+// values of chunk column tc in registers. Workgroups that are consecutive in
+// launch order are adjacent along a row, so the memory touched at any moment
+// is a band of whole rows that moves down the tensor.
 //
 // Arithmetic: operands are widened to fp32, the expression is evaluated in
 // fp32 in the order of the reference's source, and the result is rounded once
@@ -80,14 +80,21 @@ template <int OP>
 constexpr bool kNeedsB = (OP != kGeluFwd);
 
 // ---------------------------------------------------------------------------
-// Tiled kernel. COLSUM: also accumulate, per chunk column, the sum over the
-// tile's rows of the *stored* (rounded) results and write it to
-// partial[blockIdx.y][cols] (fp32); a second kernel adds the tiles up.
+// Tiled kernel. Thread (tr, tc) of a workgroup owns chunk column
+// blockIdx.x * TW + tc; one step of the workgroup covers TR * U consecutive
+// rows (all loads of a step are issued before the first result is computed).
+// Steps are numbered down the tensor and workgroup row y takes the steps
+// y, y + gridDim.y, ...: with gridDim.y = number of steps every workgroup does
+// one step, with fewer the resident workgroups sweep the tensor together,
+// front to back, which is the order HBM likes.
+// COLSUM: also accumulate, per chunk column, the sum of the *stored* (rounded)
+// results over the workgroup's steps and write it to partial[blockIdx.y][cols]
+// (fp32); a second kernel adds these up.
 // ---------------------------------------------------------------------------
 template <int DT, int OP, int TW, int U, bool COLSUM>
 __global__ void __launch_bounds__(kPwThreads)
 pointwise_kernel(void* out, const void* a, const void* b, const void* bias, float* partial, uint32_t rows,
-                 uint32_t cpr, uint32_t rows_per_block)
+                 uint32_t cpr, uint32_t steps)
 {
     constexpr int V = Elt<DT>::kVec;
     constexpr int TR = kPwThreads / TW;
@@ -96,8 +103,6 @@ pointwise_kernel(void* out, const void* a, const void* b, const void* bias, floa
     const uint32_t tr = threadIdx.x / TW;
     const uint32_t cc = blockIdx.x * TW + tc;  // chunk column
     const bool live = cc < cpr;
-    const uint32_t row0 = blockIdx.y * rows_per_block;
-    const uint32_t row_end = min(rows, row0 + rows_per_block);
     const size_t row_elems = (size_t)cpr * V;
     const bool has_b = kNeedsB<OP> && b != nullptr;
 
@@ -110,24 +115,35 @@ pointwise_kernel(void* out, const void* a, const void* b, const void* bias, floa
 #pragma unroll
     for (int j = 0; j < V; ++j) sums[j] = 0.0f;
 
-    if (live) {
-        for (uint32_t r = row0 + tr; r < row_end; r += TR * U) {
-            u32x4 ra[U], rb[U];
+    // loads of one step; rows beyond the tensor leave zeros
+    auto fetch = [&](uint32_t step, u32x4 (&ra)[U], u32x4 (&rb)[U]) {
+        const uint32_t r = step * (TR * U) + tr;
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const uint32_t row = r + u * TR;
-                const size_t off = (size_t)row * row_elems + (size_t)cc * V;
-                ra[u] = u32x4{0, 0, 0, 0};
-                rb[u] = u32x4{0, 0, 0, 0};
-                if (row < row_end) {
-                    ra[u] = load16_stream(static_cast<const S*>(a) + off);
-                    if (has_b) rb[u] = load16_stream(static_cast<const S*>(b) + off);
-                }
+        for (int u = 0; u < U; ++u) {
+            const uint32_t row = r + u * TR;
+            const size_t off = (size_t)row * row_elems + (size_t)cc * V;
+            ra[u] = u32x4{0, 0, 0, 0};
+            rb[u] = u32x4{0, 0, 0, 0};
+            if (row < rows) {
+                ra[u] = load16_stream(static_cast<const S*>(a) + off);
+                if (has_b) rb[u] = load16_stream(static_cast<const S*>(b) + off);
             }
+        }
+    };
+
+    if (live && blockIdx.y < steps) {
+        u32x4 ra[U], rb[U];
+        fetch(blockIdx.y, ra, rb);
+        for (uint32_t step = blockIdx.y; step < steps; step += gridDim.y) {
+            // the next step's loads are in flight while this one is computed and stored
+            u32x4 na[U], nb[U];
+            const uint32_t next = step + gridDim.y;
+            if (next < steps) fetch(next, na, nb);
+            const uint32_t r = step * (TR * U) + tr;
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const uint32_t row = r + u * TR;
-                if (row < row_end) {
+                if (row < rows) {
                     float fa[V], fb[V], fo[V];
                     chunk_to_float<DT>(ra[u], fa);
                     chunk_to_float<DT>(rb[u], fb);
@@ -141,6 +157,13 @@ pointwise_kernel(void* out, const void* a, const void* b, const void* bias, floa
 #pragma unroll
                         for (int j = 0; j < V; ++j) sums[j] += stored[j];
                     }
+                }
+            }
+            if (next < steps) {
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    ra[u] = na[u];
+                    rb[u] = nb[u];
                 }
             }
         }
@@ -171,7 +194,10 @@ pointwise_kernel(void* out, const void* a, const void* b, const void* bias, floa
     }
 }
 
-// out[c] = storage(sum over tiles t of partial[t][c]); 64 columns by 4 tile slices per workgroup
+// out[c] = storage(sum over t of partial[t][c]); 64 columns by 4 slices of t per
+// workgroup. The loads of a thread are independent: they are issued eight at a
+// time, since with one in flight the kernel would take `tiles / 4` memory
+// latencies.
 template <int DT>
 __global__ void __launch_bounds__(kPwThreads)
 column_sum_finish_kernel(void* out, const float* partial, uint32_t tiles, uint32_t cols)
@@ -180,8 +206,17 @@ column_sum_finish_kernel(void* out, const float* partial, uint32_t tiles, uint32
     const uint32_t tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
     const uint32_t c = blockIdx.x * 64 + tx;
     float s = 0.0f;
-    if (c < cols)
-        for (uint32_t t = ty; t < tiles; t += 4) s += partial[(size_t)t * cols + c];
+    if (c < cols) {
+        uint32_t t = ty;
+        for (; t + 28 < tiles; t += 32) {
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = partial[(size_t)(t + 4 * i) * cols + c];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) s += v[i];
+        }
+        for (; t < tiles; t += 4) s += partial[(size_t)t * cols + c];
+    }
     lds[ty][tx] = s;
     __syncthreads();
     if (ty == 0 && c < cols) Elt<DT>::store(out, c, (lds[0][tx] + lds[1][tx]) + (lds[2][tx] + lds[3][tx]));
@@ -230,28 +265,34 @@ static inline int pw_tune(const char*, int def) { return def; }
 #endif
 
 struct TilePlan {
-    int tw;                  // chunk columns per workgroup (power of two <= 256)
-    uint32_t rows_per_block;
-    uint32_t col_tiles, row_tiles;
+    int tw;          // chunk columns per workgroup (power of two <= 64)
+    uint32_t steps;  // row steps of TR * U rows
+    uint32_t col_tiles, grid_y;
 };
 
 static int elem_size(int dt) { return dt == NHP_F32 ? 4 : 2; }
 
-// Tile shape for a [rows, cols] tensor of cpr chunks per row: as wide as the
-// row allows, and rows_per_block so that a thread moves a few hundred bytes.
-static TilePlan plan_tiles(int64_t rows, int64_t cpr)
+constexpr int kPwU = 2;       // rows in flight per thread
+constexpr int kPwMaxTw = 64;  // a wave reads 1 KiB of a row
+// Dynamic LDS asked for only to bound the resident workgroups per CU: with two
+// input tensors six workgroups per CU stream better than eight (measured).
+constexpr uint32_t kPwLdsTwoInputs = 24576;
+// With column sums the grid is bounded, so that few partial rows are written.
+constexpr uint32_t kPwColsumGridY = 128;
+
+// Tile shape for a [rows, cols] tensor of cpr chunks per row.
+static TilePlan plan_tiles(int64_t rows, int64_t cpr, bool colsum)
 {
     TilePlan p;
     p.tw = 1;
-    while (p.tw < 256 && p.tw < cpr) p.tw *= 2;
-    const int tr = kPwThreads / p.tw;
-    const int per_thread = pw_tune("NHP_PW_ROWS", 32);  // rows walked by one thread
-    int64_t rpb = (int64_t)tr * per_thread;
-    while ((rows + rpb - 1) / rpb > 65535) rpb *= 2;  // grid.y limit
-    if (rpb > rows) rpb = rows;
-    p.rows_per_block = (uint32_t)rpb;
+    const int max_tw = pw_tune("NHP_PW_TW", kPwMaxTw);
+    while (p.tw < max_tw && p.tw < cpr) p.tw *= 2;
+    const int64_t step_rows = (int64_t)(kPwThreads / p.tw) * pw_tune("NHP_PW_U", kPwU);
+    p.steps = (uint32_t)((rows + step_rows - 1) / step_rows);
     p.col_tiles = (uint32_t)((cpr + p.tw - 1) / p.tw);
-    p.row_tiles = (uint32_t)((rows + rpb - 1) / rpb);
+    uint32_t cap = colsum ? (uint32_t)pw_tune("NHP_PW_GY", kPwColsumGridY) : 65535u;
+    if (cap == 0 || cap > 65535u) cap = 65535u;
+    p.grid_y = p.steps < cap ? p.steps : cap;
     return p;
 }
 
@@ -259,20 +300,38 @@ template <int DT, int OP, bool COLSUM>
 static int launch_tiled(void* out, const void* a, const void* b, const void* bias, float* partial, int64_t rows,
                         int64_t cpr, const TilePlan& p, hipStream_t st)
 {
-    const dim3 grid(p.col_tiles, p.row_tiles);
-    if (p.row_tiles > 65535u || !grid_fits((int64_t)p.col_tiles * p.row_tiles, kPwThreads)) return NHP_ERR_SHAPE;
-    constexpr int U = 4;
+    const dim3 grid(p.col_tiles, p.grid_y);
+    if (!grid_fits((int64_t)p.col_tiles * p.grid_y, kPwThreads)) return NHP_ERR_SHAPE;
+    const uint32_t lds = (uint32_t)pw_tune("NHP_PW_LDS", (kNeedsB<OP> && b != nullptr) ? kPwLdsTwoInputs : 0);
+#define CASE_U(TW_, U_)                                                                                  \
+        pointwise_kernel<DT, OP, TW_, U_, COLSUM><<<grid, kPwThreads, lds, st>>>(                        \
+            out, a, b, bias, partial, (uint32_t)rows, (uint32_t)cpr, p.steps);
+#ifdef NHP_TUNING
 #define CASE(TW_)                                                                                        \
     case TW_:                                                                                            \
-        pointwise_kernel<DT, OP, TW_, U, COLSUM><<<grid, kPwThreads, 0, st>>>(                           \
-            out, a, b, bias, partial, (uint32_t)rows, (uint32_t)cpr, p.rows_per_block);                  \
+        switch (pw_tune("NHP_PW_U", kPwU)) {                                                             \
+        case 1: CASE_U(TW_, 1) break;                                                                    \
+        case 2: CASE_U(TW_, 2) break;                                                                    \
+        case 8: CASE_U(TW_, 8) break;                                                                    \
+        default: CASE_U(TW_, kPwU) break;                                                                \
+        }                                                                                                \
         break;
+#else
+#define CASE(TW_)                                                                                        \
+    case TW_:                                                                                            \
+        CASE_U(TW_, kPwU)                                                                                \
+        break;
+#endif
     switch (p.tw) {
-        CASE(1) CASE(2) CASE(4) CASE(8) CASE(16) CASE(32) CASE(64) CASE(128) CASE(256)
+        CASE(1) CASE(2) CASE(4) CASE(8) CASE(16) CASE(32) CASE(64)
+#ifdef NHP_TUNING
+        CASE(128) CASE(256)
+#endif
     default:
         return NHP_ERR_SHAPE;
     }
 #undef CASE
+#undef CASE_U
     return launch_result();
 }
 
@@ -287,14 +346,15 @@ static int run_pointwise(void* out, const void* a, const void* b, const void* bi
                          cols / V < ((int64_t)1 << 31);
     if (chunked) {
         const int64_t cpr = cols / V;
-        const TilePlan p = plan_tiles(rows, cpr);
-        if (dbias == nullptr) return launch_tiled<DT, OP, false>(out, a, b, bias, nullptr, rows, cpr, p, st);
+        if (dbias == nullptr)
+            return launch_tiled<DT, OP, false>(out, a, b, bias, nullptr, rows, cpr, plan_tiles(rows, cpr, false), st);
         if constexpr (OP == kGeluBwd) {
+            const TilePlan p = plan_tiles(rows, cpr, true);
             int rc = launch_tiled<DT, OP, true>(out, a, b, bias, workspace, rows, cpr, p, st);
             if (rc != NHP_OK) return rc;
             const int64_t blocks = (cols + 63) / 64;
             if (!grid_fits(blocks, kPwThreads)) return NHP_ERR_SHAPE;
-            column_sum_finish_kernel<DT><<<(uint32_t)blocks, kPwThreads, 0, st>>>(dbias, workspace, p.row_tiles,
+            column_sum_finish_kernel<DT><<<(uint32_t)blocks, kPwThreads, 0, st>>>(dbias, workspace, p.grid_y,
                                                                                 (uint32_t)cols);
             return launch_result();
         }
@@ -357,8 +417,8 @@ int64_t nhp_bias_gelu_bwd_workspace_bytes(int64_t rows, int64_t cols, int dtype)
     if (check_shape(rows, cols, dtype) != NHP_OK || rows == 0 || cols == 0) return 0;
     const int v = 16 / elem_size(dtype);
     if (cols % v != 0) return 0;  // the scalar path sums the stored result directly
-    const TilePlan p = plan_tiles(rows, cols / v);
-    return (int64_t)p.row_tiles * cols * (int64_t)sizeof(float);
+    const TilePlan p = plan_tiles(rows, cols / v, true);
+    return (int64_t)p.grid_y * cols * (int64_t)sizeof(float);
 }
 
 int nhp_bias_gelu_bwd(void* dx, const void* g, const void* y, const void* bias, void* dbias, void* workspace,
