@@ -23,6 +23,8 @@ the drop-in extension modules (which call libneox_hotpath.so):
 
   mlp-gelu-1.4b  bias + tanh-GeLU fwd and bwd (with the bias gradient) on the MLP activation [2048*8, 8192] bf16
   bias-residual-1.4b  residual + (x + bias) on the hidden state [2048*8, 2048] bf16
+  layernorm-1.4b  LayerNorm fwd and bwd (with the parameter gradients) on the hidden state [2048*8, 2048] bf16
+  rmsnorm-7b     RMSNorm fwd and bwd on [4096*4, 4096] bf16 (the Llama-2 7B hidden size)
 
 `value` is algorithmic bytes per step / wall time per step (inputs resident in
 HBM, K steps bracketed by device synchronisation). Algorithmic bytes: softmax
@@ -256,6 +258,32 @@ def make_workload(name, torch, dev):
         cfg = {"workload": name, "activation": [rows, cols], "bias_gradient": "fused column sums",
                "bytes_convention": "every tensor element read or written once"}
         return step, kernel_bytes, {}, "bias_gelu_bwd", "bf16", cfg
+
+    if name in ("layernorm-1.4b", "rmsnorm-7b"):
+        from megatron.model.norms import LayerNorm, RMSNorm
+
+        rows, cols = (2048 * 8, 2048) if name == "layernorm-1.4b" else (4096 * 4, 4096)
+        module = (LayerNorm(cols, eps=1e-5) if name == "layernorm-1.4b" else RMSNorm(cols, eps=1e-8)).to(dev).bfloat16()
+        nsets = 6 if name == "layernorm-1.4b" else 3  # rotate buffers so that they come from HBM
+        sets = [(randn((rows, cols), 10 * i, torch.bfloat16, 2.0).requires_grad_(True),
+                 randn((rows, cols), 10 * i + 1, torch.bfloat16)) for i in range(nsets)]
+        n = rows * cols
+        stats = rows * 4 * (2 if name == "layernorm-1.4b" else 1)
+        nparam = 2 if name == "layernorm-1.4b" else 1
+        kernel_bytes = {"norm_fwd": 2 * n * 2 + nparam * cols * 2 + stats,
+                        "norm_bwd": 3 * n * 2 + stats + (1 + nparam) * cols * 2}
+        state = {"i": 0}
+
+        def step(t):
+            x, g = sets[state["i"] % len(sets)]
+            state["i"] += 1
+            x.grad = None
+            y = t.run("norm_fwd", lambda: module(x))
+            t.run("norm_bwd", lambda: y.backward(g))
+
+        cfg = {"workload": name, "hidden_state": [rows, cols], "parameters": "bf16",
+               "bytes_convention": "every tensor element read or written once, plus the fp32 row statistics"}
+        return step, kernel_bytes, {}, "norm_bwd", "bf16", cfg
 
     if name == "bias-residual-1.4b":
         from megatron.model.fused_bias_dropout import bias_dropout_add_fused_inference

@@ -1,0 +1,764 @@
+// LayerNorm and RMSNorm, forward and backward, for gfx950.
+//
+// x: [rows, cols]; every row is normalised on its own. A row is cut into
+// 16-byte chunks; chunk c = (k * W + w) * L + l belongs to lane l of a group
+// of L lanes (a power of two up to 64; several rows share a wave when the
+// row is short), register slot k < K and wave w < W of the row's workgroup.
+// The row stays in registers (packed, as loaded) between the statistics and
+// the output pass, so every element is read from memory once.
+//
+// Statistics and arithmetic are fp32 whatever the storage type; the mean is
+// subtracted before the squares are summed (two passes over registers).
+// Results are rounded once to the storage type. gamma / beta (scale /
+// offset) are fp32 or of the storage type.
+//
+// The backward kernel walks over row blocks with a bounded grid, keeps the
+// per-column sums for the parameter gradients in registers and writes one
+// partial row per workgroup; a second kernel adds the partial rows in a fixed
+// order, so results are reproducible from run to run.
+
+#include "common.hpp"
+
+#include <cstdlib>
+
+namespace nhp {
+
+constexpr int kNormBlockWaves = 4;  // waves per workgroup when a wave holds whole rows
+constexpr int kNormScalarThreads = 256;
+
+// Sum over groups of L consecutive lanes (L a power of two, uniform over the wave).
+__device__ __forceinline__ float lanes_sum(float v, uint32_t L)
+{
+    if (L >= 2) v += dpp_move<0xB1>(v);
+    if (L >= 4) v += dpp_move<0x4E>(v);
+    if (L >= 8) v += dpp_move<0x141>(v);
+    if (L >= 16) v += dpp_move<0x140>(v);
+    if (L >= 32) v += bitcast<float>(__builtin_amdgcn_ds_swizzle(bitcast<int>(v), 0x401F));
+    if (L >= 64) {
+        const float a = bitcast<float>(__builtin_amdgcn_readlane(bitcast<int>(v), 0));
+        const float b = bitcast<float>(__builtin_amdgcn_readlane(bitcast<int>(v), 32));
+        v = a + b;
+    }
+    return v;
+}
+
+// Sum over the W waves of a workgroup (one row per workgroup). `slots`: 16 floats of LDS
+// not used by another reduction that could still be in flight.
+template <int W>
+__device__ __forceinline__ float waves_sum(float v, float* slots, int wave, int lane)
+{
+    if constexpr (W == 1) {
+        return v;
+    } else {
+        if (lane == 0) slots[wave] = v;
+        __syncthreads();
+        float r = slots[0];
+#pragma unroll
+        for (int i = 1; i < W; ++i) r += slots[i];
+        return r;
+    }
+}
+
+// V consecutive parameter values starting at element e (a multiple of V).
+template <int DT>
+__device__ __forceinline__ void load_params(const void* p, bool f32, size_t e, float (&out)[Elt<DT>::kVec])
+{
+    constexpr int V = Elt<DT>::kVec;
+    if (f32 || DT == NHP_F32) {
+        const float* src = static_cast<const float*>(p) + e;
+#pragma unroll
+        for (int j = 0; j < V; j += 4) {
+            const u32x4 r = load16(src + j);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) out[j + i] = bitcast<float>(r[i]);
+        }
+    } else {
+        chunk_to_float<DT>(load16(static_cast<const typename Elt<DT>::storage*>(p) + e), out);
+    }
+}
+
+// 1 / (rms + eps) (eps_mode 1, the Python RMSNorm class) or rsqrt(mean(x^2) + eps) (eps_mode 0)
+__device__ __forceinline__ float rms_inverse(float sumsq, float n, float eps, int eps_mode)
+{
+    if (eps_mode == 1) return 1.0f / (sqrtf(sumsq) * (1.0f / sqrtf(n)) + eps);
+    return 1.0f / sqrtf(sumsq / n + eps);
+}
+
+struct RowSlot {
+    uint32_t row;
+    int w;
+    uint32_t l;
+    bool ok;
+};
+
+// Which row (and which part of it) this thread works on in row block `rb`.
+template <int W>
+__device__ __forceinline__ RowSlot locate(uint32_t rb, uint32_t rows, uint32_t L, uint32_t logL, int wave, int lane)
+{
+    RowSlot s;
+    s.l = (uint32_t)lane & (L - 1);
+    if constexpr (W > 1) {
+        s.row = rb;
+        s.w = wave;
+    } else {
+        const uint32_t rows_per_wave = 64u >> logL;
+        s.row = (rb * kNormBlockWaves + (uint32_t)wave) * rows_per_wave + ((uint32_t)lane >> logL);
+        s.w = 0;
+    }
+    s.ok = s.row < rows;
+    return s;
+}
+
+// ---------------------------------------------------------------------------
+// Forward
+// ---------------------------------------------------------------------------
+struct NormFwdArgs {
+    void* y;
+    float* mean;  // LayerNorm only, may be null
+    float* rstd;  // LayerNorm: 1/sqrt(var + eps); RMSNorm: the factor x is multiplied by; may be null
+    const void* x;
+    const void* gamma;
+    const void* beta;
+    float eps;
+    int eps_mode;
+    uint32_t rows, cpr, L, logL;
+    int params_f32;
+};
+
+template <int DT, int K, int W, bool RMS>
+__global__ void __launch_bounds__(((W > 1) ? W : kNormBlockWaves) * kWave)
+norm_fwd_kernel(NormFwdArgs a)
+{
+    constexpr int V = Elt<DT>::kVec;
+    using S = typename Elt<DT>::storage;
+    __shared__ float slots[2][16];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const RowSlot rs = locate<W>(blockIdx.x, a.rows, a.L, a.logL, wave, lane);
+    const size_t cols = (size_t)a.cpr * V;
+    const float n = (float)cols;
+    const S* xr = static_cast<const S*>(a.x) + (size_t)rs.row * cols;
+    S* yr = static_cast<S*>(a.y) + (size_t)rs.row * cols;
+
+    u32x4 raw[K];
+    bool live[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const uint32_t cc = (uint32_t)(k * W + rs.w) * a.L + rs.l;
+        live[k] = rs.ok && cc < a.cpr;
+        raw[k] = u32x4{0, 0, 0, 0};
+        if (live[k]) raw[k] = load16_stream(xr + (size_t)cc * V);
+    }
+
+    float mean = 0.0f, scale;
+    if constexpr (!RMS) {
+        float s = 0.0f;
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            float f[V];
+            chunk_to_float<DT>(raw[k], f);
+#pragma unroll
+            for (int j = 0; j < V; ++j) s += f[j];
+        }
+        s = waves_sum<W>(lanes_sum(s, a.L), slots[0], wave, lane);
+        mean = s / n;
+    }
+    {
+        float q = 0.0f;
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            if (live[k]) {
+                float f[V];
+                chunk_to_float<DT>(raw[k], f);
+#pragma unroll
+                for (int j = 0; j < V; ++j) {
+                    const float d = f[j] - mean;
+                    q += d * d;
+                }
+            }
+        }
+        q = waves_sum<W>(lanes_sum(q, a.L), slots[1], wave, lane);
+        scale = RMS ? rms_inverse(q, n, a.eps, a.eps_mode) : 1.0f / sqrtf(q / n + a.eps);
+    }
+
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        if (live[k]) {
+            const uint32_t cc = (uint32_t)(k * W + rs.w) * a.L + rs.l;
+            float f[V], g[V], b[V];
+            chunk_to_float<DT>(raw[k], f);
+#pragma unroll
+            for (int j = 0; j < V; ++j) f[j] = (f[j] - mean) * scale;
+            if (a.gamma != nullptr) {
+                load_params<DT>(a.gamma, a.params_f32 != 0, (size_t)cc * V, g);
+#pragma unroll
+                for (int j = 0; j < V; ++j) f[j] = RMS ? g[j] * f[j] : f[j] * g[j];
+            }
+            if (a.beta != nullptr) {
+                load_params<DT>(a.beta, a.params_f32 != 0, (size_t)cc * V, b);
+#pragma unroll
+                for (int j = 0; j < V; ++j) f[j] = f[j] + b[j];
+            }
+            store16_stream(yr + (size_t)cc * V, float_to_chunk<DT>(f));
+        }
+    }
+    if (rs.ok && rs.l == 0 && rs.w == 0) {
+        if (!RMS && a.mean != nullptr) a.mean[rs.row] = mean;
+        if (a.rstd != nullptr) a.rstd[rs.row] = scale;
+    }
+}
+
+// One workgroup per row, elements strided over the threads, the row re-read for every pass.
+__device__ __forceinline__ float block_sum_256(float v, float* slots)
+{
+    v = lanes_sum(v, 64);
+    __syncthreads();  // slots may still be read from the previous reduction
+    if ((threadIdx.x & 63) == 0) slots[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return (slots[0] + slots[1]) + (slots[2] + slots[3]);
+}
+
+template <int DT, bool RMS>
+__global__ void __launch_bounds__(kNormScalarThreads)
+norm_fwd_scalar_kernel(void* y, float* mean_out, float* rstd_out, const void* x, const void* gamma,
+                       const void* beta, float eps, int eps_mode, uint64_t cols, int pdt)
+{
+    __shared__ float slots[4];
+    const uint64_t row = blockIdx.x;
+    const int64_t base = (int64_t)(row * cols);
+    const float n = (float)cols;
+    float mean = 0.0f;
+    if (!RMS) {
+        float s = 0.0f;
+        for (uint64_t c = threadIdx.x; c < cols; c += kNormScalarThreads) s += Elt<DT>::load(x, base + (int64_t)c);
+        mean = block_sum_256(s, slots) / n;
+    }
+    float q = 0.0f;
+    for (uint64_t c = threadIdx.x; c < cols; c += kNormScalarThreads) {
+        const float d = Elt<DT>::load(x, base + (int64_t)c) - mean;
+        q += d * d;
+    }
+    q = block_sum_256(q, slots);
+    const float scale = RMS ? rms_inverse(q, n, eps, eps_mode) : 1.0f / sqrtf(q / n + eps);
+    auto param = [&](const void* p, uint64_t c) {
+        return pdt == NHP_F32 ? static_cast<const float*>(p)[c] : Elt<DT>::load(p, (int64_t)c);
+    };
+    for (uint64_t c = threadIdx.x; c < cols; c += kNormScalarThreads) {
+        float f = (Elt<DT>::load(x, base + (int64_t)c) - mean) * scale;
+        if (gamma != nullptr) f = RMS ? param(gamma, c) * f : f * param(gamma, c);
+        if (beta != nullptr) f = f + param(beta, c);
+        Elt<DT>::store(y, base + (int64_t)c, f);
+    }
+    if (threadIdx.x == 0) {
+        if (!RMS && mean_out != nullptr) mean_out[row] = mean;
+        if (rstd_out != nullptr) rstd_out[row] = scale;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Backward
+//   xhat = (x - mean) * rstd (RMSNorm: x * inv), g = dy * gamma
+//   LayerNorm: dx = rstd * (g - (sum(g) + xhat * sum(g * xhat)) / cols)
+//   RMSNorm:   dx = inv * (g - xhat * sum(g * xhat) / (cols * rho)), rho = 1 for eps_mode 0 and
+//              1 - eps * inv for eps_mode 1 (rho <= 0: the second term is dropped)
+//   dgamma[c] = sum over rows of dy * xhat, dbeta[c] = sum over rows of dy
+// ---------------------------------------------------------------------------
+struct NormBwdArgs {
+    void* dx;
+    float* part_g;  // [gridDim.x, cols] partial sums for dgamma, or null (no parameter gradients)
+    float* part_b;  // same for dbeta
+    const void* dy;
+    const void* x;
+    const float* mean;
+    const float* rstd;
+    const void* gamma;
+    float eps;
+    int eps_mode;
+    uint32_t rows, cpr, L, logL, row_blocks;
+    int params_f32;
+};
+
+template <int DT, int K, int W, bool RMS>
+__global__ void __launch_bounds__(((W > 1) ? W : kNormBlockWaves) * kWave)
+norm_bwd_kernel(NormBwdArgs a)
+{
+    constexpr int V = Elt<DT>::kVec;
+    constexpr int T = ((W > 1) ? W : kNormBlockWaves) * kWave;
+    using S = typename Elt<DT>::storage;
+    __shared__ float slots[2][16];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const size_t cols = (size_t)a.cpr * V;
+    const float n = (float)cols;
+    const bool param_grads = a.part_g != nullptr;
+
+    // this thread's chunk columns do not depend on the row block
+    const RowSlot first = locate<W>(0, a.rows, a.L, a.logL, wave, lane);
+    uint32_t cc[K];
+    bool col_live[K];
+    float gam[K][V];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        cc[k] = (uint32_t)(k * W + first.w) * a.L + first.l;
+        col_live[k] = cc[k] < a.cpr;
+#pragma unroll
+        for (int j = 0; j < V; ++j) gam[k][j] = 1.0f;
+        if (col_live[k] && a.gamma != nullptr) load_params<DT>(a.gamma, a.params_f32 != 0, (size_t)cc[k] * V, gam[k]);
+    }
+
+    float acc_g[K][V], acc_b[K][V];
+#pragma unroll
+    for (int k = 0; k < K; ++k)
+#pragma unroll
+        for (int j = 0; j < V; ++j) acc_g[k][j] = acc_b[k][j] = 0.0f;
+
+    for (uint32_t rb = blockIdx.x; rb < a.row_blocks; rb += gridDim.x) {
+        const RowSlot rs = locate<W>(rb, a.rows, a.L, a.logL, wave, lane);
+        const S* gr = static_cast<const S*>(a.dy) + (size_t)rs.row * cols;
+        const S* xr = static_cast<const S*>(a.x) + (size_t)rs.row * cols;
+        u32x4 rg[K], rx[K];
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            rg[k] = u32x4{0, 0, 0, 0};
+            rx[k] = u32x4{0, 0, 0, 0};
+            if (rs.ok && col_live[k]) {
+                rg[k] = load16_stream(gr + (size_t)cc[k] * V);
+                rx[k] = load16_stream(xr + (size_t)cc[k] * V);
+            }
+        }
+        float mean = 0.0f, scale = 0.0f;
+        if (rs.ok) {
+            if (!RMS) mean = a.mean[rs.row];
+            scale = a.rstd[rs.row];
+        }
+
+        float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            if (rs.ok && col_live[k]) {
+                float fg[V], fx[V];
+                chunk_to_float<DT>(rg[k], fg);
+                chunk_to_float<DT>(rx[k], fx);
+#pragma unroll
+                for (int j = 0; j < V; ++j) {
+                    const float xh = (fx[j] - mean) * scale;
+                    const float g = fg[j] * gam[k][j];
+                    s1 += g;
+                    s2 += g * xh;
+                    acc_g[k][j] += fg[j] * xh;
+                    acc_b[k][j] += fg[j];
+                }
+            }
+        }
+        if (W > 1) __syncthreads();  // the slots of the previous row block have been read by every wave
+        if constexpr (!RMS) s1 = waves_sum<W>(lanes_sum(s1, a.L), slots[0], wave, lane);
+        s2 = waves_sum<W>(lanes_sum(s2, a.L), slots[1], wave, lane);
+
+        float k2 = s2 / n;
+        if (RMS && a.eps_mode == 1) {
+            const float rho = 1.0f - a.eps * scale;
+            k2 = rho > 0.0f ? k2 / rho : 0.0f;
+        }
+        S* dr = static_cast<S*>(a.dx) + (size_t)rs.row * cols;
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            if (rs.ok && col_live[k]) {
+                float fg[V], fx[V], o[V];
+                chunk_to_float<DT>(rg[k], fg);
+                chunk_to_float<DT>(rx[k], fx);
+#pragma unroll
+                for (int j = 0; j < V; ++j) {
+                    const float xh = (fx[j] - mean) * scale;
+                    const float g = fg[j] * gam[k][j];
+                    const float t = RMS ? xh * k2 : (s1 + xh * s2) / n;
+                    o[j] = scale * (g - t);
+                }
+                store16_stream(dr + (size_t)cc[k] * V, float_to_chunk<DT>(o));
+            }
+        }
+    }
+
+    if (!param_grads) return;
+    if constexpr (W > 1) {
+        // one row per workgroup: every thread owns its columns alone
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            if (col_live[k]) {
+                float* pg = a.part_g + (size_t)blockIdx.x * cols + (size_t)cc[k] * V;
+                float* pb = a.part_b + (size_t)blockIdx.x * cols + (size_t)cc[k] * V;
+#pragma unroll
+                for (int j = 0; j < V; ++j) {
+                    pg[j] = acc_g[k][j];
+                    pb[j] = acc_b[k][j];
+                }
+            }
+        }
+    } else {
+        // the T / L threads that hold the same columns (other rows) are added up by the first of them
+        __shared__ float red[K * V * T];
+        for (int pass = 0; pass < 2; ++pass) {
+            __syncthreads();
+#pragma unroll
+            for (int k = 0; k < K; ++k)
+#pragma unroll
+                for (int j = 0; j < V; ++j) red[(k * V + j) * T + threadIdx.x] = pass == 0 ? acc_g[k][j] : acc_b[k][j];
+            __syncthreads();
+            if (threadIdx.x < a.L) {
+                float* dst = (pass == 0 ? a.part_g : a.part_b) + (size_t)blockIdx.x * cols;
+#pragma unroll
+                for (int k = 0; k < K; ++k) {
+                    if (col_live[k]) {
+#pragma unroll
+                        for (int j = 0; j < V; ++j) {
+                            float s = red[(k * V + j) * T + threadIdx.x];
+                            for (uint32_t t = threadIdx.x + a.L; t < (uint32_t)T; t += a.L) s += red[(k * V + j) * T + t];
+                            dst[(size_t)cc[k] * V + j] = s;
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+// out[c] = sum over t of partial[t][c], stored as fp32 or as DT; 64 columns by 4 slices of t
+// per workgroup, loads issued eight at a time. blockIdx.y selects the (partial, out) pair.
+template <int DT>
+__global__ void __launch_bounds__(256)
+param_grad_finish_kernel(void* out0, void* out1, const float* part0, const float* part1, uint32_t tiles,
+                         uint32_t cols, int out_f32)
+{
+    __shared__ float lds[4][64];
+    void* out = blockIdx.y == 0 ? out0 : out1;
+    const float* partial = blockIdx.y == 0 ? part0 : part1;
+    if (out == nullptr) return;
+    const uint32_t tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    const uint32_t c = blockIdx.x * 64 + tx;
+    float s = 0.0f;
+    if (c < cols) {
+        uint32_t t = ty;
+        for (; t + 28 < tiles; t += 32) {
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = partial[(size_t)(t + 4 * i) * cols + c];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) s += v[i];
+        }
+        for (; t < tiles; t += 4) s += partial[(size_t)t * cols + c];
+    }
+    lds[ty][tx] = s;
+    __syncthreads();
+    if (ty == 0 && c < cols) {
+        const float r = (lds[0][tx] + lds[1][tx]) + (lds[2][tx] + lds[3][tx]);
+        if (out_f32)
+            static_cast<float*>(out)[c] = r;
+        else
+            Elt<DT>::store(out, c, r);
+    }
+}
+
+template <int DT, bool RMS>
+__global__ void __launch_bounds__(kNormScalarThreads)
+norm_bwd_scalar_kernel(void* dx, const void* dy, const void* x, const float* mean_in, const float* rstd_in,
+                       const void* gamma, float eps, int eps_mode, uint64_t cols, int pdt)
+{
+    __shared__ float slots[4];
+    const uint64_t row = blockIdx.x;
+    const int64_t base = (int64_t)(row * cols);
+    const float n = (float)cols;
+    const float mean = RMS ? 0.0f : mean_in[row];
+    const float scale = rstd_in[row];
+    auto gval = [&](uint64_t c) {
+        if (gamma == nullptr) return 1.0f;
+        return pdt == NHP_F32 ? static_cast<const float*>(gamma)[c] : Elt<DT>::load(gamma, (int64_t)c);
+    };
+    float s1 = 0.0f, s2 = 0.0f;
+    for (uint64_t c = threadIdx.x; c < cols; c += kNormScalarThreads) {
+        const float xh = (Elt<DT>::load(x, base + (int64_t)c) - mean) * scale;
+        const float g = Elt<DT>::load(dy, base + (int64_t)c) * gval(c);
+        s1 += g;
+        s2 += g * xh;
+    }
+    s1 = block_sum_256(s1, slots);
+    s2 = block_sum_256(s2, slots);
+    float k2 = s2 / n;
+    if (RMS && eps_mode == 1) {
+        const float rho = 1.0f - eps * scale;
+        k2 = rho > 0.0f ? k2 / rho : 0.0f;
+    }
+    for (uint64_t c = threadIdx.x; c < cols; c += kNormScalarThreads) {
+        const float xh = (Elt<DT>::load(x, base + (int64_t)c) - mean) * scale;
+        const float g = Elt<DT>::load(dy, base + (int64_t)c) * gval(c);
+        const float t = RMS ? xh * k2 : (s1 + xh * s2) / n;
+        Elt<DT>::store(dx, base + (int64_t)c, scale * (g - t));
+    }
+}
+
+// parameter gradients for the scalar path: one thread per column, rows in order
+template <int DT, bool RMS>
+__global__ void __launch_bounds__(kNormScalarThreads)
+norm_param_grad_scalar_kernel(void* dgamma, void* dbeta, const void* dy, const void* x, const float* mean_in,
+                              const float* rstd_in, uint64_t rows, uint64_t cols, int pdt)
+{
+    const uint64_t c = (uint64_t)blockIdx.x * kNormScalarThreads + threadIdx.x;
+    if (c >= cols) return;
+    float sg = 0.0f, sb = 0.0f;
+    for (uint64_t r = 0; r < rows; ++r) {
+        const float m = RMS ? 0.0f : mean_in[r];
+        const float g = Elt<DT>::load(dy, (int64_t)(r * cols + c));
+        sg += g * ((Elt<DT>::load(x, (int64_t)(r * cols + c)) - m) * rstd_in[r]);
+        sb += g;
+    }
+    auto put = [&](void* p, float v) {
+        if (p == nullptr) return;
+        if (pdt == NHP_F32)
+            static_cast<float*>(p)[c] = v;
+        else
+            Elt<DT>::store(p, (int64_t)c, v);
+    };
+    put(dgamma, sg);
+    put(dbeta, sb);
+}
+
+// ---------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------
+#ifdef NHP_TUNING
+static int norm_tune(const char* name, int def)
+{
+    const char* v = getenv(name);
+    return v ? atoi(v) : def;
+}
+#else
+static inline int norm_tune(const char*, int def) { return def; }
+#endif
+
+struct NormPlan {
+    uint32_t L, logL;
+    int K, W;
+};
+
+// (K, W) pairs that are compiled
+#define NHP_NORM_GEOMETRIES(X) X(1, 1) X(2, 1) X(4, 1) X(2, 2) X(2, 4) X(2, 8) X(4, 8) X(4, 16)
+
+// Geometry for rows of cpr chunks: a wave reads 1-2 KiB of a row; returns false when the row does not fit.
+static bool plan_norm(int64_t cpr, NormPlan& p)
+{
+    if (cpr < 1) return false;
+    p.L = 1;
+    p.logL = 0;
+    while (p.L < 64 && (int64_t)p.L < cpr) {
+        p.L *= 2;
+        ++p.logL;
+    }
+    const int64_t segs = (cpr + p.L - 1) / p.L;  // 16-byte chunks per lane over the whole row
+    static const int table[][2] = {{1, 1}, {2, 1}, {2, 2}, {2, 4}, {2, 8}, {4, 8}, {4, 16}};
+    p.K = p.W = 0;
+    for (const auto& kw : table) {
+        if ((int64_t)kw[0] * kw[1] >= segs) {
+            p.K = kw[0];
+            p.W = kw[1];
+            break;
+        }
+    }
+    const int tk = norm_tune("NHP_NORM_K", 0), tw = norm_tune("NHP_NORM_W", 0);
+    if (tk > 0 && tw > 0 && (int64_t)tk * tw >= segs) {
+        p.K = tk;
+        p.W = tw;
+    }
+    return p.K != 0;
+}
+
+static uint32_t norm_row_blocks(int64_t rows, const NormPlan& p)
+{
+    const int64_t rows_per_block = p.W > 1 ? 1 : (int64_t)kNormBlockWaves * (64 / p.L);
+    return (uint32_t)((rows + rows_per_block - 1) / rows_per_block);
+}
+
+constexpr uint32_t kNormBwdGrid = 1024;  // workgroups of the backward kernel when parameter gradients are wanted
+
+static uint32_t norm_bwd_grid(uint32_t row_blocks, bool param_grads)
+{
+    if (!param_grads) return row_blocks;
+    const uint32_t cap = (uint32_t)norm_tune("NHP_NORM_GRID", kNormBwdGrid);
+    return row_blocks < cap ? row_blocks : cap;
+}
+
+static bool param_dtype_ok(int dtype, int pdt) { return pdt == dtype || pdt == NHP_F32; }
+
+template <int DT, bool RMS>
+static int norm_fwd(void* y, float* mean, float* rstd, const void* x, const void* gamma, const void* beta, float eps,
+                    int eps_mode, int64_t rows, int64_t cols, int pdt, hipStream_t st)
+{
+    constexpr int V = Elt<DT>::kVec;
+    NormPlan p;
+    const bool params_aligned = ptr_aligned16(gamma) && ptr_aligned16(beta);
+    if (cols % V == 0 && ptr_aligned16(x) && ptr_aligned16(y) && params_aligned && plan_norm(cols / V, p)) {
+        NormFwdArgs a{y, mean, rstd, x, gamma, beta, eps, eps_mode, (uint32_t)rows, (uint32_t)(cols / V),
+                      p.L, p.logL, pdt == NHP_F32 ? 1 : 0};
+        const uint32_t blocks = norm_row_blocks(rows, p);
+        const int threads = (p.W > 1 ? p.W : kNormBlockWaves) * kWave;
+        if (!grid_fits(blocks, threads)) return NHP_ERR_SHAPE;
+#define X(K_, W_)                                                                      \
+    if (p.K == K_ && p.W == W_) {                                                      \
+        norm_fwd_kernel<DT, K_, W_, RMS><<<blocks, threads, 0, st>>>(a);               \
+        return launch_result();                                                        \
+    }
+        NHP_NORM_GEOMETRIES(X)
+#undef X
+        return NHP_ERR_SHAPE;
+    }
+    if (!grid_fits(rows, kNormScalarThreads)) return NHP_ERR_SHAPE;
+    norm_fwd_scalar_kernel<DT, RMS><<<(uint32_t)rows, kNormScalarThreads, 0, st>>>(
+        y, mean, rstd, x, gamma, beta, eps, eps_mode, (uint64_t)cols, pdt);
+    return launch_result();
+}
+
+static int64_t norm_workspace_bytes(int64_t rows, int64_t cols, int dtype)
+{
+    const int v = dtype == NHP_F32 ? 4 : 8;
+    NormPlan p;
+    if (rows <= 0 || cols <= 0 || cols % v != 0 || !plan_norm(cols / v, p)) return 0;
+    return 2 * (int64_t)norm_bwd_grid(norm_row_blocks(rows, p), true) * cols * (int64_t)sizeof(float);
+}
+
+template <int DT, bool RMS>
+static int norm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, const void* x, const float* mean,
+                    const float* rstd, const void* gamma, void* workspace, float eps, int eps_mode, int64_t rows,
+                    int64_t cols, int pdt, hipStream_t st)
+{
+    constexpr int V = Elt<DT>::kVec;
+    NormPlan p;
+    const bool want_params = dgamma != nullptr || dbeta != nullptr;
+    if (cols % V == 0 && ptr_aligned16(dx) && ptr_aligned16(dy) && ptr_aligned16(x) && ptr_aligned16(gamma) &&
+        ptr_aligned16(workspace) && plan_norm(cols / V, p)) {
+        const uint32_t row_blocks = norm_row_blocks(rows, p);
+        const uint32_t grid = norm_bwd_grid(row_blocks, want_params);
+        float* part_g = want_params ? static_cast<float*>(workspace) : nullptr;
+        float* part_b = want_params ? part_g + (size_t)grid * cols : nullptr;
+        NormBwdArgs a{dx, part_g, part_b, dy, x, mean, rstd, gamma, eps, eps_mode, (uint32_t)rows,
+                      (uint32_t)(cols / V), p.L, p.logL, row_blocks, pdt == NHP_F32 ? 1 : 0};
+        const int threads = (p.W > 1 ? p.W : kNormBlockWaves) * kWave;
+        if (!grid_fits(grid, threads)) return NHP_ERR_SHAPE;
+        bool launched = false;
+#define X(K_, W_)                                                                      \
+    if (!launched && p.K == K_ && p.W == W_) {                                         \
+        norm_bwd_kernel<DT, K_, W_, RMS><<<grid, threads, 0, st>>>(a);                 \
+        launched = true;                                                               \
+    }
+        NHP_NORM_GEOMETRIES(X)
+#undef X
+        if (!launched) return NHP_ERR_SHAPE;
+        int rc = launch_result();
+        if (rc != NHP_OK || !want_params) return rc;
+        const dim3 fgrid((uint32_t)((cols + 63) / 64), 2);
+        param_grad_finish_kernel<DT><<<fgrid, 256, 0, st>>>(dgamma, dbeta, part_g, part_b, grid, (uint32_t)cols,
+                                                            pdt == NHP_F32 ? 1 : 0);
+        return launch_result();
+    }
+    if (!grid_fits(rows, kNormScalarThreads)) return NHP_ERR_SHAPE;
+    norm_bwd_scalar_kernel<DT, RMS><<<(uint32_t)rows, kNormScalarThreads, 0, st>>>(dx, dy, x, mean, rstd, gamma, eps,
+                                                                                    eps_mode, (uint64_t)cols, pdt);
+    int rc = launch_result();
+    if (rc != NHP_OK || !want_params) return rc;
+    norm_param_grad_scalar_kernel<DT, RMS>
+        <<<(uint32_t)((cols + kNormScalarThreads - 1) / kNormScalarThreads), kNormScalarThreads, 0, st>>>(
+            dgamma, dbeta, dy, x, mean, rstd, (uint64_t)rows, (uint64_t)cols, pdt);
+    return launch_result();
+}
+
+static int norm_check(int64_t rows, int64_t cols, int dtype, int pdt)
+{
+    if (dtype != NHP_F16 && dtype != NHP_BF16 && dtype != NHP_F32) return NHP_ERR_DTYPE;
+    if (!param_dtype_ok(dtype, pdt)) return NHP_ERR_DTYPE;
+    if (rows < 0 || cols < 0 || rows >= ((int64_t)1 << 31)) return NHP_ERR_SHAPE;
+    if (rows > 0 && cols > ((int64_t)1 << 62) / rows) return NHP_ERR_SHAPE;
+    return NHP_OK;
+}
+
+template <bool RMS>
+static int norm_fwd_dispatch(void* y, float* mean, float* rstd, const void* x, const void* gamma, const void* beta,
+                             float eps, int eps_mode, int64_t rows, int64_t cols, int dtype, int pdt, void* stream)
+{
+    if (int rc = norm_check(rows, cols, dtype, pdt)) return rc;
+    if (rows == 0 || cols == 0) return NHP_OK;
+    if (!y || !x) return NHP_ERR_NULL;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+    case NHP_F16:
+        return norm_fwd<NHP_F16, RMS>(y, mean, rstd, x, gamma, beta, eps, eps_mode, rows, cols, pdt, st);
+    case NHP_BF16:
+        return norm_fwd<NHP_BF16, RMS>(y, mean, rstd, x, gamma, beta, eps, eps_mode, rows, cols, pdt, st);
+    default:
+        return norm_fwd<NHP_F32, RMS>(y, mean, rstd, x, gamma, beta, eps, eps_mode, rows, cols, pdt, st);
+    }
+}
+
+template <bool RMS>
+static int norm_bwd_dispatch(void* dx, void* dgamma, void* dbeta, const void* dy, const void* x, const float* mean,
+                             const float* rstd, const void* gamma, void* workspace, float eps, int eps_mode,
+                             int64_t rows, int64_t cols, int dtype, int pdt, void* stream)
+{
+    if (int rc = norm_check(rows, cols, dtype, pdt)) return rc;
+    if (rows == 0 || cols == 0) return NHP_OK;
+    if (!dx || !dy || !x || !rstd || (!RMS && !mean)) return NHP_ERR_NULL;
+    if ((dgamma != nullptr || dbeta != nullptr) && workspace == nullptr && norm_workspace_bytes(rows, cols, dtype) > 0)
+        return NHP_ERR_NULL;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+    case NHP_F16:
+        return norm_bwd<NHP_F16, RMS>(dx, dgamma, dbeta, dy, x, mean, rstd, gamma, workspace, eps, eps_mode, rows,
+                                      cols, pdt, st);
+    case NHP_BF16:
+        return norm_bwd<NHP_BF16, RMS>(dx, dgamma, dbeta, dy, x, mean, rstd, gamma, workspace, eps, eps_mode, rows,
+                                       cols, pdt, st);
+    default:
+        return norm_bwd<NHP_F32, RMS>(dx, dgamma, dbeta, dy, x, mean, rstd, gamma, workspace, eps, eps_mode, rows,
+                                      cols, pdt, st);
+    }
+}
+
+}  // namespace nhp
+
+using namespace nhp;
+
+extern "C" {
+
+int nhp_layernorm_fwd(void* y, float* mean, float* rstd, const void* x, const void* gamma, const void* beta,
+                      float eps, int64_t rows, int64_t cols, int dtype, int param_dtype, void* stream)
+{
+    return norm_fwd_dispatch<false>(y, mean, rstd, x, gamma, beta, eps, 0, rows, cols, dtype, param_dtype, stream);
+}
+
+int nhp_layernorm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, const void* x, const float* mean,
+                      const float* rstd, const void* gamma, void* workspace, int64_t rows, int64_t cols, int dtype,
+                      int param_dtype, void* stream)
+{
+    return norm_bwd_dispatch<false>(dx, dgamma, dbeta, dy, x, mean, rstd, gamma, workspace, 0.0f, 0, rows, cols,
+                                    dtype, param_dtype, stream);
+}
+
+int nhp_rmsnorm_fwd(void* y, float* inv, const void* x, const void* scale, const void* offset, float eps,
+                    int eps_mode, int64_t rows, int64_t cols, int dtype, int param_dtype, void* stream)
+{
+    if (eps_mode != 0 && eps_mode != 1) return NHP_ERR_SHAPE;
+    return norm_fwd_dispatch<true>(y, nullptr, inv, x, scale, offset, eps, eps_mode, rows, cols, dtype, param_dtype,
+                                   stream);
+}
+
+int nhp_rmsnorm_bwd(void* dx, void* dscale, void* doffset, const void* dy, const void* x, const float* inv,
+                    const void* scale, void* workspace, float eps, int eps_mode, int64_t rows, int64_t cols,
+                    int dtype, int param_dtype, void* stream)
+{
+    if (eps_mode != 0 && eps_mode != 1) return NHP_ERR_SHAPE;
+    return norm_bwd_dispatch<true>(dx, dscale, doffset, dy, x, nullptr, inv, scale, workspace, eps, eps_mode, rows,
+                                   cols, dtype, param_dtype, stream);
+}
+
+int64_t nhp_norm_bwd_workspace_bytes(int64_t rows, int64_t cols, int dtype)
+{
+    if (dtype != NHP_F16 && dtype != NHP_BF16 && dtype != NHP_F32) return 0;
+    return norm_workspace_bytes(rows, cols, dtype);
+}
+
+}  // extern "C"

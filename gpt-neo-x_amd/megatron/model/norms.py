@@ -1,0 +1,223 @@
+"""LayerNorm and RMSNorm on MI355X.
+
+Surface of GPT-NeoX's ``megatron/model/norms.py``: ``get_norm`` (:19-51),
+``LayerNorm`` (:16, torch's class there) and ``RMSNorm`` (:54-107), with the same
+constructor arguments and parameter names (``weight`` / ``bias``, ``scale`` /
+``offset``). Forward and backward are hand-written gfx950 kernels
+(libneox_hotpath.so): one pass over the row for the forward, one for the
+backward including the parameter gradients. Statistics and arithmetic are fp32
+and the result is rounded once, which is what torch's LayerNorm kernel and the
+fused RMSNorm variants do; the Python ``RMSNorm`` of the reference, run eagerly
+on 16-bit tensors, rounds after every operator and so differs by a few units in
+the last place.
+
+Not provided: partial RMSNorm (``p`` in [0, 1]) and ``ScaleNorm``.
+"""
+import numbers
+
+import torch
+
+from ..fused_kernels import _hotpath as _hp
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _param_code(x, *params):
+    dtypes = {p.dtype for p in params if p is not None}
+    if not dtypes:
+        return _hp.dtype_code(x, "norm")
+    if len(dtypes) > 1:
+        raise RuntimeError("norm: the parameters must share one dtype")
+    dt = dtypes.pop()
+    if dt not in (x.dtype, torch.float32):
+        raise RuntimeError(f"norm: parameters must be float32 or {x.dtype}, got {dt}")
+    return _hp._DTYPE[dt]
+
+
+def _check_param(p, cols, x, what):
+    if p is None:
+        return None
+    if p.numel() != cols:
+        raise RuntimeError(f"{what}: parameter of {p.numel()} elements for rows of {cols}")
+    _hp.require_gpu(p, what)
+    return p.contiguous()
+
+
+def _workspace(rows, cols, code, device):
+    nbytes = _hp.lib().nhp_norm_bwd_workspace_bytes(rows, cols, code)
+    return torch.empty(nbytes, dtype=torch.uint8, device=device) if nbytes else None
+
+
+class _LayerNormFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, weight, bias, eps):
+        what = "LayerNorm"
+        _hp.require_gpu(x, what)
+        cols = x.size(-1)
+        src = x.contiguous()
+        weight = _check_param(weight, cols, x, what)
+        bias = _check_param(bias, cols, x, what)
+        rows = src.numel() // max(cols, 1)
+        y = torch.empty_like(src)
+        mean = torch.empty(rows, dtype=torch.float32, device=src.device)
+        rstd = torch.empty(rows, dtype=torch.float32, device=src.device)
+        code, pcode = _hp.dtype_code(src, what), _param_code(src, weight, bias)
+        with _hp.device_guard(src):
+            rc = _hp.lib().nhp_layernorm_fwd(y.data_ptr(), mean.data_ptr(), rstd.data_ptr(), src.data_ptr(),
+                                             _ptr(weight), _ptr(bias), float(eps), rows, cols, code, pcode,
+                                             _hp.stream_of(src))
+        _hp.check(rc, what)
+        ctx.save_for_backward(src, weight, mean, rstd)
+        ctx.has_bias = bias is not None
+        ctx.codes = (code, pcode)
+        return y
+
+    @staticmethod
+    def backward(ctx, grad):
+        what = "LayerNorm backward"
+        src, weight, mean, rstd = ctx.saved_tensors
+        g = grad.contiguous()
+        cols = src.size(-1)
+        rows = src.numel() // max(cols, 1)
+        code, pcode = ctx.codes
+        want_w = weight is not None and ctx.needs_input_grad[1]
+        want_b = ctx.has_bias and ctx.needs_input_grad[2]
+        pdtype = weight.dtype if weight is not None else (torch.float32 if pcode == _hp.F32 else src.dtype)
+        dx = torch.empty_like(src)
+        dw = torch.empty(cols, dtype=pdtype, device=src.device) if want_w else None
+        db = torch.empty(cols, dtype=pdtype, device=src.device) if want_b else None
+        ws = _workspace(rows, cols, code, src.device) if (want_w or want_b) else None
+        with _hp.device_guard(src):
+            rc = _hp.lib().nhp_layernorm_bwd(dx.data_ptr(), _ptr(dw), _ptr(db), g.data_ptr(), src.data_ptr(),
+                                             mean.data_ptr(), rstd.data_ptr(), _ptr(weight), _ptr(ws), rows, cols,
+                                             code, pcode, _hp.stream_of(src))
+        _hp.check(rc, what)
+        if rows == 0:
+            dw = None if dw is None else dw.zero_()
+            db = None if db is None else db.zero_()
+        return dx, dw, db, None
+
+
+class LayerNorm(torch.nn.Module):
+    """``torch.nn.LayerNorm`` over the last dimension (what ``get_norm`` returns for ``norm: layernorm``)."""
+
+    def __init__(self, normalized_shape, eps=1e-5, elementwise_affine=True, bias=True, device=None, dtype=None):
+        super().__init__()
+        if isinstance(normalized_shape, numbers.Integral):
+            normalized_shape = (int(normalized_shape),)
+        if len(normalized_shape) != 1:
+            raise NotImplementedError("only normalisation over the last dimension is provided")
+        self.normalized_shape = tuple(normalized_shape)
+        self.eps = eps
+        self.elementwise_affine = elementwise_affine
+        if elementwise_affine:
+            self.weight = torch.nn.Parameter(torch.ones(self.normalized_shape, device=device, dtype=dtype))
+            if bias:
+                self.bias = torch.nn.Parameter(torch.zeros(self.normalized_shape, device=device, dtype=dtype))
+            else:
+                self.register_parameter("bias", None)
+        else:
+            self.register_parameter("weight", None)
+            self.register_parameter("bias", None)
+
+    def forward(self, input):
+        if input.size(-1) != self.normalized_shape[0]:
+            raise RuntimeError(f"LayerNorm: expected last dimension {self.normalized_shape[0]}, got {input.size(-1)}")
+        return _LayerNormFunction.apply(input, self.weight, self.bias, self.eps)
+
+    def extra_repr(self):
+        return f"{self.normalized_shape}, eps={self.eps}, elementwise_affine={self.elementwise_affine}"
+
+
+class _RMSNormFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, scale, offset, eps, eps_mode):
+        what = "RMSNorm"
+        _hp.require_gpu(x, what)
+        cols = x.size(-1)
+        src = x.contiguous()
+        scale = _check_param(scale, cols, x, what)
+        offset = _check_param(offset, cols, x, what)
+        rows = src.numel() // max(cols, 1)
+        y = torch.empty_like(src)
+        inv = torch.empty(rows, dtype=torch.float32, device=src.device)
+        code, pcode = _hp.dtype_code(src, what), _param_code(src, scale, offset)
+        with _hp.device_guard(src):
+            rc = _hp.lib().nhp_rmsnorm_fwd(y.data_ptr(), inv.data_ptr(), src.data_ptr(), _ptr(scale), _ptr(offset),
+                                           float(eps), int(eps_mode), rows, cols, code, pcode, _hp.stream_of(src))
+        _hp.check(rc, what)
+        ctx.save_for_backward(src, scale, inv)
+        ctx.has_offset = offset is not None
+        ctx.conf = (code, pcode, float(eps), int(eps_mode))
+        return y
+
+    @staticmethod
+    def backward(ctx, grad):
+        what = "RMSNorm backward"
+        src, scale, inv = ctx.saved_tensors
+        g = grad.contiguous()
+        cols = src.size(-1)
+        rows = src.numel() // max(cols, 1)
+        code, pcode, eps, eps_mode = ctx.conf
+        want_s = scale is not None and ctx.needs_input_grad[1]
+        want_o = ctx.has_offset and ctx.needs_input_grad[2]
+        pdtype = scale.dtype if scale is not None else (torch.float32 if pcode == _hp.F32 else src.dtype)
+        dx = torch.empty_like(src)
+        ds = torch.empty(cols, dtype=pdtype, device=src.device) if want_s else None
+        do = torch.empty(cols, dtype=pdtype, device=src.device) if want_o else None
+        ws = _workspace(rows, cols, code, src.device) if (want_s or want_o) else None
+        with _hp.device_guard(src):
+            rc = _hp.lib().nhp_rmsnorm_bwd(dx.data_ptr(), _ptr(ds), _ptr(do), g.data_ptr(), src.data_ptr(),
+                                           inv.data_ptr(), _ptr(scale), _ptr(ws), eps, eps_mode, rows, cols, code,
+                                           pcode, _hp.stream_of(src))
+        _hp.check(rc, what)
+        if rows == 0:
+            ds = None if ds is None else ds.zero_()
+            do = None if do is None else do.zero_()
+        return dx, ds, do, None, None
+
+
+class RMSNorm(torch.nn.Module):
+    """Root-mean-square normalisation, ``scale * x / (rms(x) + eps) [+ offset]``
+    (the reference's Python class, megatron/model/norms.py:54-107).
+
+    ``fused_eps=True`` selects the other definition the reference knows,
+    ``scale * x * rsqrt(mean(x^2) + eps)`` (MixedFusedRMSNorm)."""
+
+    def __init__(self, dim, p=-1.0, eps=1e-8, bias=False, fused_eps=False):
+        super().__init__()
+        if 0.0 <= p <= 1.0:
+            raise NotImplementedError("partial RMSNorm (p in [0, 1]) is not provided by the MI355X kernels")
+        self.eps = eps
+        self.d = dim
+        self.p = p
+        self.bias = bias
+        self.fused_eps = fused_eps
+        self.scale = torch.nn.Parameter(torch.ones(dim))
+        if self.bias:
+            self.offset = torch.nn.Parameter(torch.zeros(dim))
+        else:
+            self.register_parameter("offset", None)
+
+    def forward(self, x):
+        if x.size(-1) != self.d:
+            raise RuntimeError(f"RMSNorm: expected last dimension {self.d}, got {x.size(-1)}")
+        return _RMSNormFunction.apply(x, self.scale, self.offset, self.eps, 0 if self.fused_eps else 1)
+
+
+class _FusedRMSNorm(RMSNorm):
+    def __init__(self, dim, eps=1e-5, **_):
+        super().__init__(dim, eps=eps, fused_eps=True)
+
+
+def get_norm(neox_args):
+    """(norm class, eps) for ``neox_args.norm`` in {"layernorm", "rmsnorm"}; the ``*_fusion`` flags pick
+    the fused definition of the epsilon for RMSNorm and change nothing for LayerNorm."""
+    if neox_args.norm == "rmsnorm":
+        norm = _FusedRMSNorm if getattr(neox_args, "rmsnorm_fusion", False) else RMSNorm
+        return norm, neox_args.rms_norm_epsilon
+    if neox_args.norm == "layernorm":
+        return LayerNorm, neox_args.layernorm_epsilon
+    raise ValueError(f"norm {neox_args.norm} not provided by the MI355X kernels")

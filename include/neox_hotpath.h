@@ -324,6 +324,71 @@ int64_t nhp_bias_gelu_bwd_workspace_bytes(int64_t rows, int64_t cols, int dtype)
 int nhp_bias_add_residual(void* out, const void* x, const void* bias, const void* residual,
                           int64_t rows, int64_t cols, int dtype, void* stream);
 
+/* ------------------------------------------------------------------------
+ * LayerNorm and RMSNorm
+ *
+ * x, y, dy, dx: dense [rows, cols] in `dtype` (NHP_F16, NHP_BF16, NHP_F32);
+ * every row is normalised over its `cols` elements. gamma / beta (scale /
+ * offset) and their gradients: [cols] in `param_dtype`, which is `dtype` or
+ * NHP_F32; each may be NULL. Statistics and arithmetic are fp32, results are
+ * rounded once. mean / rstd / inv: fp32 [rows], written by the forward (NULL:
+ * not wanted) and read by the backward.
+ *
+ * The backward needs `workspace` when a parameter gradient is asked for: a
+ * 16-byte aligned device buffer of nhp_norm_bwd_workspace_bytes(rows, cols,
+ * dtype) bytes owned by the caller (0: none needed). Parameter gradients are
+ * summed in a fixed order: results are reproducible from run to run.
+ * ---------------------------------------------------------------------- */
+
+/*
+ * y = ((x - mean) * rstd) * gamma + beta, mean and biased variance per row,
+ * rstd = 1 / sqrt(var + eps).
+ *
+ * Replaces torch.nn.LayerNorm as handed out by get_norm
+ *   megatron/model/norms.py:16,19-51 (norm = "layernorm"), used as input_layernorm,
+ *   post_attention_layernorm and final norm, megatron/model/transformer.py:985-1040,1362
+ * and the apex-backed MixedFusedLayerNorm, megatron/model/fused_layer_norm.py:34-153.
+ */
+int nhp_layernorm_fwd(void* y, float* mean, float* rstd, const void* x,
+                      const void* gamma, const void* beta, float eps,
+                      int64_t rows, int64_t cols, int dtype, int param_dtype, void* stream);
+
+/*
+ * xhat = (x - mean) * rstd, g = dy * gamma:
+ *   dx = rstd * (g - (sum(g) + xhat * sum(g * xhat)) / cols)
+ *   dgamma = column sums of dy * xhat, dbeta = column sums of dy (each optional).
+ * The adjoint of nhp_layernorm_fwd, i.e. what autograd runs for torch.nn.LayerNorm
+ *   (megatron/model/norms.py:16).
+ */
+int nhp_layernorm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, const void* x,
+                      const float* mean, const float* rstd, const void* gamma, void* workspace,
+                      int64_t rows, int64_t cols, int dtype, int param_dtype, void* stream);
+
+/*
+ * y = scale * (x * inv) + offset with
+ *   eps_mode 1: inv = 1 / (||x||_2 * cols^(-1/2) + eps), the Python class
+ *               RMSNorm.forward, megatron/model/norms.py:54-107 (p disabled);
+ *   eps_mode 0: inv = 1 / sqrt(mean(x^2) + eps), the fused variants
+ *               MixedFusedRMSNorm, megatron/model/fused_layer_norm.py:156-252.
+ */
+int nhp_rmsnorm_fwd(void* y, float* inv, const void* x, const void* scale, const void* offset,
+                    float eps, int eps_mode,
+                    int64_t rows, int64_t cols, int dtype, int param_dtype, void* stream);
+
+/*
+ * xhat = x * inv, g = dy * scale, s = sum(g * xhat):
+ *   dx = inv * (g - xhat * s / (cols * rho)), rho = 1 (eps_mode 0) or 1 - eps * inv (eps_mode 1;
+ *   rho <= 0, an all-zero row, drops the second term);
+ *   dscale = column sums of dy * xhat, doffset = column sums of dy (each optional).
+ * The adjoint of nhp_rmsnorm_fwd, i.e. what autograd runs for RMSNorm.forward
+ *   (megatron/model/norms.py:85-107).
+ */
+int nhp_rmsnorm_bwd(void* dx, void* dscale, void* doffset, const void* dy, const void* x,
+                    const float* inv, const void* scale, void* workspace, float eps, int eps_mode,
+                    int64_t rows, int64_t cols, int dtype, int param_dtype, void* stream);
+
+int64_t nhp_norm_bwd_workspace_bytes(int64_t rows, int64_t cols, int dtype);
+
 #ifdef __cplusplus
 }
 #endif

@@ -54,6 +54,10 @@ def lib():
         L.oracle_bias_gelu_bwd.argtypes = [vp, vp, vp, vp, i64, i64, ci]
         L.oracle_column_sum.argtypes = [vp, vp, i64, i64, ci]
         L.oracle_bias_add_residual.argtypes = [vp, vp, vp, vp, i64, i64, ci]
+        L.oracle_layernorm_fwd.argtypes = [vp, vp, vp, vp, vp, vp, f32, i64, i64, ci, ci]
+        L.oracle_layernorm_bwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, ci, ci]
+        L.oracle_rmsnorm_fwd.argtypes = [vp, vp, vp, vp, vp, f32, ci, i64, i64, ci, ci]
+        L.oracle_rmsnorm_bwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, f32, ci, i64, i64, ci, ci]
         p64 = ctypes.POINTER(i64)
         L.oracle_rope_cached.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, p64, p64, ci, ci, ci]
         L.oracle_rope_freqs.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, p64, p64, ci, ci]
@@ -247,3 +251,82 @@ def bias_add_residual(x, bias=None, residual=None):
     _check(lib().oracle_bias_add_residual(out.data_ptr(), x.data_ptr(), bp, rp, rows, cols, _DT[x.dtype]),
            "bias_add_residual")
     return out
+
+
+# ---------------------------------------------------------------------------
+# LayerNorm / RMSNorm (layer_semantics.c)
+# ---------------------------------------------------------------------------
+def _param(t, x):
+    """(tensor kept alive, pointer, dtype code) of an optional [cols] parameter: fp32 or x.dtype."""
+    if t is None:
+        return None, None, None
+    t = _cpu_contig(t)
+    assert t.dtype in (x.dtype, torch.float32) and t.numel() == x.size(-1)
+    return t, t.data_ptr(), _DT[t.dtype]
+
+
+def _param_code(x, *codes):
+    codes = {c for c in codes if c is not None}
+    assert len(codes) <= 1, "all parameters must share one dtype"
+    return codes.pop() if codes else _DT[x.dtype]
+
+
+def layernorm_fwd(x, gamma=None, beta=None, eps=1e-5):
+    """Returns (y, mean, rstd); x: [..., cols]."""
+    x = _cpu_contig(x)
+    rows, cols = _rows_cols(x)
+    y = torch.empty_like(x)
+    mean = torch.empty(rows, dtype=torch.float32)
+    rstd = torch.empty(rows, dtype=torch.float32)
+    gamma, gp, gc = _param(gamma, x)
+    beta, bp, bc = _param(beta, x)
+    _check(lib().oracle_layernorm_fwd(y.data_ptr(), mean.data_ptr(), rstd.data_ptr(), x.data_ptr(), gp, bp,
+                                      float(eps), rows, cols, _DT[x.dtype], _param_code(x, gc, bc)), "layernorm_fwd")
+    return y, mean, rstd
+
+
+def layernorm_bwd(dy, x, mean, rstd, gamma=None, param_dtype=None):
+    """Returns (dx, dgamma, dbeta); the parameter gradients come in param_dtype (default: gamma's, else x's)."""
+    x = _cpu_contig(x)
+    dy = _cpu_contig(dy)
+    rows, cols = _rows_cols(x)
+    gamma, gp, gc = _param(gamma, x)
+    pdt = param_dtype or (gamma.dtype if gamma is not None else x.dtype)
+    dx = torch.empty_like(x)
+    dg = torch.empty(cols, dtype=pdt)
+    db = torch.empty(cols, dtype=pdt)
+    mean, rstd = _cpu_contig(mean.float()), _cpu_contig(rstd.float())
+    _check(lib().oracle_layernorm_bwd(dx.data_ptr(), dg.data_ptr(), db.data_ptr(), dy.data_ptr(), x.data_ptr(),
+                                      mean.data_ptr(), rstd.data_ptr(), gp, rows, cols, _DT[x.dtype], _DT[pdt]),
+           "layernorm_bwd")
+    return dx, dg, db
+
+
+def rmsnorm_fwd(x, scale=None, offset=None, eps=1e-8, eps_mode=1):
+    """Returns (y, inv). eps_mode 1: x / (rms + eps) (the Python RMSNorm class); 0: x * rsqrt(mean(x^2) + eps)."""
+    x = _cpu_contig(x)
+    rows, cols = _rows_cols(x)
+    y = torch.empty_like(x)
+    inv = torch.empty(rows, dtype=torch.float32)
+    scale, sp, sc = _param(scale, x)
+    offset, op, oc = _param(offset, x)
+    _check(lib().oracle_rmsnorm_fwd(y.data_ptr(), inv.data_ptr(), x.data_ptr(), sp, op, float(eps), int(eps_mode),
+                                    rows, cols, _DT[x.dtype], _param_code(x, sc, oc)), "rmsnorm_fwd")
+    return y, inv
+
+
+def rmsnorm_bwd(dy, x, inv, scale=None, eps=1e-8, eps_mode=1, param_dtype=None):
+    """Returns (dx, dscale, doffset)."""
+    x = _cpu_contig(x)
+    dy = _cpu_contig(dy)
+    rows, cols = _rows_cols(x)
+    scale, sp, sc = _param(scale, x)
+    pdt = param_dtype or (scale.dtype if scale is not None else x.dtype)
+    dx = torch.empty_like(x)
+    ds = torch.empty(cols, dtype=pdt)
+    do = torch.empty(cols, dtype=pdt)
+    inv = _cpu_contig(inv.float())
+    _check(lib().oracle_rmsnorm_bwd(dx.data_ptr(), ds.data_ptr(), do.data_ptr(), dy.data_ptr(), x.data_ptr(),
+                                    inv.data_ptr(), sp, float(eps), int(eps_mode), rows, cols, _DT[x.dtype],
+                                    _DT[pdt]), "rmsnorm_bwd")
+    return dx, ds, do

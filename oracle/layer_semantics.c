@@ -124,3 +124,192 @@ int oracle_bias_add_residual(void* out, const void* x, const void* bias, const v
         }
     return 0;
 }
+
+/* ------------------------------------------------------------------------ */
+/* LayerNorm and RMSNorm                                                      */
+/* ------------------------------------------------------------------------ */
+
+static float load_param(const void* p, int64_t i, int pdt) { return p ? load_elem(p, i, pdt) : 0.0f; }
+
+/*
+ * torch.nn.LayerNorm, which megatron/model/norms.py:16,32 hands out for
+ * norm = "layernorm" (used as input_layernorm / post_attention_layernorm,
+ * megatron/model/transformer.py:985-1040): per row of `cols` elements
+ *   mean = sum(x) / cols, var = sum((x - mean)^2) / cols (biased),
+ *   rstd = 1 / sqrt(var + eps), y = ((x - mean) * rstd) * gamma + beta,
+ * statistics and arithmetic in fp32 whatever the storage type, y rounded once.
+ * gamma / beta: [cols] in storage type pdt (fp32 or the type of x), or NULL
+ * (no affine term). mean, rstd: fp32 [rows], what the backward needs.
+ */
+int oracle_layernorm_fwd(void* y, float* mean, float* rstd, const void* x, const void* gamma, const void* beta,
+                         float eps, int64_t rows, int64_t cols, int dt, int pdt)
+{
+    float* v = (float*)malloc(sizeof(float) * (size_t)(cols > 0 ? cols : 1));
+    if (!v) return -2;
+    for (int64_t r = 0; r < rows; ++r) {
+        for (int64_t c = 0; c < cols; ++c) v[c] = load_elem(x, r * cols + c, dt);
+        const float m = pairwise_sum(v, cols) / (float)cols;
+        for (int64_t c = 0; c < cols; ++c) {
+            const float d = v[c] - m;
+            v[c] = d * d;
+        }
+        const float var = pairwise_sum(v, cols) / (float)cols;
+        const float rs = 1.0f / sqrtf(var + eps);
+        for (int64_t c = 0; c < cols; ++c) {
+            float o = (load_elem(x, r * cols + c, dt) - m) * rs;
+            if (gamma) o = o * load_param(gamma, c, pdt);
+            if (beta) o = o + load_param(beta, c, pdt);
+            store_elem(y, r * cols + c, dt, o);
+        }
+        if (mean) mean[r] = m;
+        if (rstd) rstd[r] = rs;
+    }
+    free(v);
+    return 0;
+}
+
+/*
+ * Backward of the above (the textbook adjoint, as torch's layer_norm backward):
+ *   xhat = (x - mean) * rstd, g = dy * gamma,
+ *   dx = rstd * (g - (sum(g) + xhat * sum(g * xhat)) / cols),
+ *   dgamma[c] = sum over rows of dy * xhat, dbeta[c] = sum over rows of dy,
+ * fp32 throughout, outputs rounded once (dgamma, dbeta to pdt). Any of dx,
+ * dgamma, dbeta may be NULL.
+ */
+int oracle_layernorm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, const void* x, const float* mean,
+                         const float* rstd, const void* gamma, int64_t rows, int64_t cols, int dt, int pdt)
+{
+    const size_t n = (size_t)(cols > 0 ? cols : 1);
+    float* g = (float*)malloc(sizeof(float) * n);
+    float* gx = (float*)malloc(sizeof(float) * n);
+    float* col = (float*)malloc(sizeof(float) * (size_t)(rows > 0 ? rows : 1));
+    if (!g || !gx || !col) {
+        free(g);
+        free(gx);
+        free(col);
+        return -2;
+    }
+    if (dx)
+        for (int64_t r = 0; r < rows; ++r) {
+            for (int64_t c = 0; c < cols; ++c) {
+                const float xh = (load_elem(x, r * cols + c, dt) - mean[r]) * rstd[r];
+                g[c] = load_elem(dy, r * cols + c, dt) * (gamma ? load_param(gamma, c, pdt) : 1.0f);
+                gx[c] = g[c] * xh;
+            }
+            const float s1 = pairwise_sum(g, cols), s2 = pairwise_sum(gx, cols);
+            for (int64_t c = 0; c < cols; ++c) {
+                const float xh = (load_elem(x, r * cols + c, dt) - mean[r]) * rstd[r];
+                const float t = (s1 + xh * s2) / (float)cols;
+                store_elem(dx, r * cols + c, dt, rstd[r] * (g[c] - t));
+            }
+        }
+    for (int64_t c = 0; c < cols; ++c) {
+        if (dgamma) {
+            for (int64_t r = 0; r < rows; ++r)
+                col[r] = load_elem(dy, r * cols + c, dt) * ((load_elem(x, r * cols + c, dt) - mean[r]) * rstd[r]);
+            store_elem(dgamma, c, pdt, pairwise_sum(col, rows));
+        }
+        if (dbeta) {
+            for (int64_t r = 0; r < rows; ++r) col[r] = load_elem(dy, r * cols + c, dt);
+            store_elem(dbeta, c, pdt, pairwise_sum(col, rows));
+        }
+    }
+    free(g);
+    free(gx);
+    free(col);
+    return 0;
+}
+
+/*
+ * RMSNorm. Two definitions live in the reference, selected here by eps_mode:
+ *   1: the Python class megatron/model/norms.py:54-107 (p disabled):
+ *        rms = ||x||_2 * cols^(-1/2);  y = scale * (x / (rms + eps)) [+ offset]
+ *   0: the fused variants (MixedFusedRMSNorm, megatron/model/fused_layer_norm.py:156-252,
+ *      backed by apex, and TERMSNorm): y = scale * (x * rsqrt(mean(x^2) + eps))
+ * fp32 arithmetic, one rounding of y. inv: fp32 [rows], the factor x is
+ * multiplied by (1 / (rms + eps) or rsqrt(mean(x^2) + eps)).
+ */
+static float rms_inverse(float sumsq, int64_t cols, float eps, int eps_mode)
+{
+    if (eps_mode == 1) return 1.0f / (sqrtf(sumsq) * (1.0f / sqrtf((float)cols)) + eps);
+    return 1.0f / sqrtf(sumsq / (float)cols + eps);
+}
+
+int oracle_rmsnorm_fwd(void* y, float* inv, const void* x, const void* scale, const void* offset, float eps,
+                       int eps_mode, int64_t rows, int64_t cols, int dt, int pdt)
+{
+    float* v = (float*)malloc(sizeof(float) * (size_t)(cols > 0 ? cols : 1));
+    if (!v) return -2;
+    for (int64_t r = 0; r < rows; ++r) {
+        for (int64_t c = 0; c < cols; ++c) {
+            const float f = load_elem(x, r * cols + c, dt);
+            v[c] = f * f;
+        }
+        const float iv = rms_inverse(pairwise_sum(v, cols), cols, eps, eps_mode);
+        for (int64_t c = 0; c < cols; ++c) {
+            float o = load_elem(x, r * cols + c, dt) * iv;
+            if (scale) o = load_param(scale, c, pdt) * o;
+            if (offset) o = o + load_param(offset, c, pdt);
+            store_elem(y, r * cols + c, dt, o);
+        }
+        if (inv) inv[r] = iv;
+    }
+    free(v);
+    return 0;
+}
+
+/*
+ * Backward of RMSNorm: with xhat = x * inv, g = dy * scale, s = sum(g * xhat),
+ *   eps_mode 0: dx = inv * (g - xhat * s / cols)
+ *   eps_mode 1: dx = inv * (g - xhat * s / (cols * rho)), rho = rms / (rms + eps) = 1 - eps * inv
+ *               (rho = 0, an all-zero row with eps > 0: the second term is 0, as
+ *               torch's norm backward defines it)
+ *   dscale[c] = sum over rows of dy * xhat, doffset[c] = sum over rows of dy.
+ */
+int oracle_rmsnorm_bwd(void* dx, void* dscale, void* doffset, const void* dy, const void* x, const float* inv,
+                       const void* scale, float eps, int eps_mode, int64_t rows, int64_t cols, int dt, int pdt)
+{
+    const size_t n = (size_t)(cols > 0 ? cols : 1);
+    float* g = (float*)malloc(sizeof(float) * n);
+    float* gx = (float*)malloc(sizeof(float) * n);
+    float* col = (float*)malloc(sizeof(float) * (size_t)(rows > 0 ? rows : 1));
+    if (!g || !gx || !col) {
+        free(g);
+        free(gx);
+        free(col);
+        return -2;
+    }
+    if (dx)
+        for (int64_t r = 0; r < rows; ++r) {
+            for (int64_t c = 0; c < cols; ++c) {
+                const float xh = load_elem(x, r * cols + c, dt) * inv[r];
+                g[c] = load_elem(dy, r * cols + c, dt) * (scale ? load_param(scale, c, pdt) : 1.0f);
+                gx[c] = g[c] * xh;
+            }
+            const float s = pairwise_sum(gx, cols);
+            float k = s / (float)cols;
+            if (eps_mode == 1) {
+                const float rho = 1.0f - eps * inv[r];
+                k = rho > 0.0f ? k / rho : 0.0f;
+            }
+            for (int64_t c = 0; c < cols; ++c) {
+                const float xh = load_elem(x, r * cols + c, dt) * inv[r];
+                store_elem(dx, r * cols + c, dt, inv[r] * (g[c] - xh * k));
+            }
+        }
+    for (int64_t c = 0; c < cols; ++c) {
+        if (dscale) {
+            for (int64_t r = 0; r < rows; ++r)
+                col[r] = load_elem(dy, r * cols + c, dt) * (load_elem(x, r * cols + c, dt) * inv[r]);
+            store_elem(dscale, c, pdt, pairwise_sum(col, rows));
+        }
+        if (doffset) {
+            for (int64_t r = 0; r < rows; ++r) col[r] = load_elem(dy, r * cols + c, dt);
+            store_elem(doffset, c, pdt, pairwise_sum(col, rows));
+        }
+    }
+    free(g);
+    free(gx);
+    free(col);
+    return 0;
+}

@@ -1,0 +1,276 @@
+"""GPU parity of LayerNorm and RMSNorm (forward, backward with parameter gradients)
+through the C ABI and the modules, against the CPU oracle.
+
+Tolerances: outputs and dx within 2 representable values of the oracle, or within a few
+fp32 roundings of the terms that are added up (the sums over a row are formed in a
+different order); parameter gradients within the fp32 noise of a sum over all rows."""
+import types
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle
+import util
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+DTYPES = [torch.bfloat16, torch.float16, torch.float32]
+IDS = ["bf16", "fp16", "fp32"]
+
+
+def ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def make(dtype, rows, cols, seed, pdtype):
+    g = torch.Generator().manual_seed(seed)
+    x = (torch.randn((rows, cols), generator=g) * 2 + 0.5).to(dtype)
+    dy = torch.randn((rows, cols), generator=g).to(dtype)
+    gamma = (1 + 0.3 * torch.randn(cols, generator=g)).to(pdtype)
+    beta = (0.2 * torch.randn(cols, generator=g)).to(pdtype)
+    return x, dy, gamma, beta
+
+
+def abi_layernorm(hp, x, dy, gamma, beta, eps, want_params=True):
+    rows, cols = x.shape
+    code, pcode = hp.dtype_code(x, "t"), hp._DTYPE[(gamma if gamma is not None else x).dtype]
+    y = torch.empty_like(x)
+    mean = torch.empty(rows, dtype=torch.float32, device=x.device)
+    rstd = torch.empty_like(mean)
+    L = hp.lib()
+    rc = L.nhp_layernorm_fwd(y.data_ptr(), mean.data_ptr(), rstd.data_ptr(), x.data_ptr(), ptr(gamma), ptr(beta), eps,
+                             rows, cols, code, pcode, None)
+    assert rc == 0, L.nhp_status_string(rc)
+    dx = torch.empty_like(x)
+    pd = gamma.dtype if gamma is not None else x.dtype
+    dg = torch.full((cols,), float("nan"), dtype=pd, device=x.device) if want_params else None
+    db = torch.full((cols,), float("nan"), dtype=pd, device=x.device) if want_params else None
+    ws = torch.empty(max(L.nhp_norm_bwd_workspace_bytes(rows, cols, code), 1), dtype=torch.uint8, device=x.device)
+    rc = L.nhp_layernorm_bwd(dx.data_ptr(), ptr(dg), ptr(db), dy.data_ptr(), x.data_ptr(), mean.data_ptr(),
+                             rstd.data_ptr(), ptr(gamma), ws.data_ptr(), rows, cols, code, pcode, None)
+    assert rc == 0, L.nhp_status_string(rc)
+    return y, mean, rstd, dx, dg, db
+
+
+def abi_rmsnorm(hp, x, dy, scale, offset, eps, mode):
+    rows, cols = x.shape
+    code, pcode = hp.dtype_code(x, "t"), hp._DTYPE[(scale if scale is not None else x).dtype]
+    y = torch.empty_like(x)
+    inv = torch.empty(rows, dtype=torch.float32, device=x.device)
+    L = hp.lib()
+    rc = L.nhp_rmsnorm_fwd(y.data_ptr(), inv.data_ptr(), x.data_ptr(), ptr(scale), ptr(offset), eps, mode, rows, cols,
+                           code, pcode, None)
+    assert rc == 0, L.nhp_status_string(rc)
+    dx = torch.empty_like(x)
+    pd = scale.dtype if scale is not None else x.dtype
+    ds = torch.full((cols,), float("nan"), dtype=pd, device=x.device)
+    do = torch.full((cols,), float("nan"), dtype=pd, device=x.device)
+    ws = torch.empty(max(L.nhp_norm_bwd_workspace_bytes(rows, cols, code), 1), dtype=torch.uint8, device=x.device)
+    rc = L.nhp_rmsnorm_bwd(dx.data_ptr(), ds.data_ptr(), do.data_ptr(), dy.data_ptr(), x.data_ptr(), inv.data_ptr(),
+                           ptr(scale), ws.data_ptr(), eps, mode, rows, cols, code, pcode, None)
+    assert rc == 0, L.nhp_status_string(rc)
+    return y, inv, dx, ds, do
+
+
+def out_noise(gamma, like):
+    g = gamma.float().abs() if gamma is not None else torch.ones(like.size(-1))
+    return (g * 64 * util.EPS32).expand_as(like.float())
+
+
+def dx_noise(dy, gamma, factor):
+    g = gamma.float().abs() if gamma is not None else 1.0
+    return ((dy.float().abs() * g).sum(-1, keepdim=True) * factor[:, None] * 64 * util.EPS32).expand_as(dy.float())
+
+
+# rows, cols: every geometry (lanes per row 1..64, 1..16 waves per row), partial row blocks, scalar fallbacks
+SHAPES = [(5, 8), (9, 16), (33, 64), (70, 128), (300, 512), (37, 1024), (129, 2048), (21, 4096), (19, 8192),
+          (7, 16384), (3, 32768), (11, 1000), (4, 65536), (13, 2056), (1, 24)]
+
+
+@pytest.mark.parametrize("pd", ["same", "fp32"])
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: f"{s[0]}x{s[1]}")
+def test_layernorm_vs_oracle(hotpath, shape, dtype, pd):
+    rows, cols = shape
+    if pd == "fp32" and dtype == torch.float32:
+        pytest.skip("same case")
+    pdtype = dtype if pd == "same" else torch.float32
+    print(f"layernorm case {shape} {dtype} params {pdtype}", flush=True)
+    x, dy, gamma, beta = make(dtype, rows, cols, rows + cols, pdtype)
+    eps = 1e-5
+    want_y, want_mean, want_rstd = oracle.layernorm_fwd(x, gamma, beta, eps)
+    y, mean, rstd, dx, dg, db = [t.cpu() for t in abi_layernorm(hotpath, x.to(DEV), dy.to(DEV), gamma.to(DEV),
+                                                                  beta.to(DEV), eps)]
+    util.assert_close_ulp_or_noise(y, want_y, 2, out_noise(gamma, x), "y")
+    assert torch.allclose(mean, want_mean, rtol=0, atol=2e-6 * (1 + x.float().abs().max().item()))
+    assert torch.allclose(rstd, want_rstd, rtol=1e-5, atol=0)
+    # backward from the statistics the GPU produced, against the oracle fed with the same statistics
+    want_dx, want_dg, want_db = oracle.layernorm_bwd(dy, x, mean, rstd, gamma)
+    util.assert_close_ulp_or_noise(dx, want_dx, 2, dx_noise(dy, gamma, rstd), "dx")
+    col = (dy.float().abs() * ((x.float() - mean[:, None]) * rstd[:, None]).abs()).sum(0) * 32 * util.EPS32
+    util.assert_close_ulp_or_noise(dg, want_dg, 2, col, "dgamma")
+    util.assert_close_ulp_or_noise(db, want_db, 2, dy.float().abs().sum(0) * 32 * util.EPS32, "dbeta")
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("shape", [(5, 8), (70, 128), (129, 2048), (21, 4096), (19, 8192), (3, 32768), (11, 1000)],
+                         ids=lambda s: f"{s[0]}x{s[1]}")
+def test_rmsnorm_vs_oracle(hotpath, shape, dtype, mode):
+    rows, cols = shape
+    print(f"rmsnorm case {shape} {dtype} mode {mode}", flush=True)
+    x, dy, scale, offset = make(dtype, rows, cols, rows + cols + 1, dtype)
+    eps = 1e-5 if mode == 0 else 1e-2
+    want_y, want_inv = oracle.rmsnorm_fwd(x, scale, offset, eps, mode)
+    y, inv, dx, ds, do = [t.cpu() for t in abi_rmsnorm(hotpath, x.to(DEV), dy.to(DEV), scale.to(DEV), offset.to(DEV),
+                                                      eps, mode)]
+    util.assert_close_ulp_or_noise(y, want_y, 2, out_noise(scale, x), "y")
+    assert torch.allclose(inv, want_inv, rtol=1e-5, atol=0)
+    want_dx, want_ds, want_do = oracle.rmsnorm_bwd(dy, x, inv, scale, eps, mode)
+    util.assert_close_ulp_or_noise(dx, want_dx, 2, dx_noise(dy, scale, inv), "dx")
+    col = (dy.float().abs() * (x.float() * inv[:, None]).abs()).sum(0) * 32 * util.EPS32
+    util.assert_close_ulp_or_noise(ds, want_ds, 2, col, "dscale")
+    util.assert_close_ulp_or_noise(do, want_do, 2, dy.float().abs().sum(0) * 32 * util.EPS32, "doffset")
+
+
+def test_norm_edge_cases(hotpath):
+    L = hotpath.lib()
+    # no affine terms, no statistics wanted, no parameter gradients, unaligned input, empty tensors
+    x, dy, _, _ = make(torch.bfloat16, 50, 256, 3, torch.bfloat16)
+    xd, dyd = x.to(DEV), dy.to(DEV)
+    y = torch.empty_like(xd)
+    rc = L.nhp_layernorm_fwd(y.data_ptr(), None, None, xd.data_ptr(), None, None, 1e-5, 50, 256, 1, 1, None)
+    assert rc == 0
+    want, mean, rstd = oracle.layernorm_fwd(x, None, None, 1e-5)
+    util.assert_close_ulp_or_noise(y.cpu(), want, 2, out_noise(None, x), "plain")
+    dx = torch.empty_like(xd)
+    mean_d, rstd_d = mean.to(DEV), rstd.to(DEV)  # named, so that the device copies outlive the launch
+    rc = L.nhp_layernorm_bwd(dx.data_ptr(), None, None, dyd.data_ptr(), xd.data_ptr(), mean_d.data_ptr(),
+                             rstd_d.data_ptr(), None, None, 50, 256, 1, 1, None)
+    assert rc == 0
+    util.assert_close_ulp_or_noise(dx.cpu(), oracle.layernorm_bwd(dy, x, mean, rstd, None)[0], 2,
+                                   dx_noise(dy, None, rstd), "dx without parameters")
+    buf = torch.zeros(50 * 256 + 8, dtype=torch.bfloat16, device=DEV)
+    shifted = buf[1:1 + 50 * 256].view(50, 256)
+    shifted.copy_(xd)
+    rc = L.nhp_layernorm_fwd(y.data_ptr(), None, None, shifted.data_ptr(), None, None, 1e-5, 50, 256, 1, 1, None)
+    assert rc == 0
+    util.assert_close_ulp_or_noise(y.cpu(), want, 2, out_noise(None, x), "unaligned")
+    assert L.nhp_layernorm_fwd(None, None, None, None, None, None, 1e-5, 0, 256, 1, 1, None) == 0
+    assert L.nhp_layernorm_fwd(y.data_ptr(), None, None, xd.data_ptr(), None, None, 1e-5, 50, 256, 1, 0, None) == -1
+    assert L.nhp_rmsnorm_fwd(y.data_ptr(), None, xd.data_ptr(), None, None, 1e-5, 2, 50, 256, 1, 1, None) == -2
+    # a constant row (zero variance) and an all-zero row
+    const = torch.full((4, 512), 3.0, dtype=torch.bfloat16, device=DEV)
+    out = torch.empty_like(const)
+    assert L.nhp_layernorm_fwd(out.data_ptr(), None, None, const.data_ptr(), None, None, 1e-5, 4, 512, 1, 1, None) == 0
+    assert out.abs().max().item() == 0
+    zero = torch.zeros((4, 512), dtype=torch.bfloat16, device=DEV)
+    inv = torch.empty(4, dtype=torch.float32, device=DEV)
+    for mode in (0, 1):
+        assert L.nhp_rmsnorm_fwd(out.data_ptr(), inv.data_ptr(), zero.data_ptr(), None, None, 1e-3, mode, 4, 512, 1, 1, None) == 0
+        assert out.abs().max().item() == 0 and torch.isfinite(inv).all()
+        ones = torch.ones_like(zero)
+        assert L.nhp_rmsnorm_bwd(out.data_ptr(), None, None, ones.data_ptr(), zero.data_ptr(), inv.data_ptr(), None, None,
+                                 1e-3, mode, 4, 512, 1, 1, None) == 0
+        assert torch.isfinite(out.float()).all()
+
+
+def test_norm_parameter_gradients_are_reproducible(hotpath):
+    x, dy, gamma, beta = [t.to(DEV) for t in make(torch.bfloat16, 5000, 2048, 1, torch.float32)]
+    first = abi_layernorm(hotpath, x, dy, gamma, beta, 1e-5)
+    for _ in range(3):
+        again = abi_layernorm(hotpath, x, dy, gamma, beta, 1e-5)
+        for a, b in zip(first, again):
+            assert torch.equal(util.raw_bits(a), util.raw_bits(b))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+def test_layernorm_module_matches_torch_module(dtype):
+    from megatron.model.norms import LayerNorm
+
+    s, b, h = 96, 4, 2048
+    mine = LayerNorm(h, eps=1e-5).to(DEV).to(dtype)
+    ref = torch.nn.LayerNorm(h, eps=1e-5).to(DEV).to(dtype)
+    with torch.no_grad():
+        w = (1 + 0.3 * torch.randn(h, generator=torch.Generator().manual_seed(1))).to(dtype).to(DEV)
+        bb = (0.2 * torch.randn(h, generator=torch.Generator().manual_seed(2))).to(dtype).to(DEV)
+        for m in (mine, ref):
+            m.weight.copy_(w)
+            m.bias.copy_(bb)
+    x = util.randn((s, b, h), dtype, seed=3, std=2.0).to(DEV)
+    g = util.randn((s, b, h), dtype, seed=4).to(DEV)
+    xa = x.clone().requires_grad_(True)
+    xb = x.clone().requires_grad_(True)
+    ya = mine(xa)
+    yb = ref(xb)
+    ya.backward(g)
+    yb.backward(g)
+    assert sorted(n for n, _ in mine.named_parameters()) == ["bias", "weight"]
+    util.assert_close_ulp_or_noise(ya.detach().cpu(), yb.detach().cpu(), 2, out_noise(w.cpu(), x.cpu()), "y")
+    lim = 2.0 ** (-7 if dtype == torch.bfloat16 else -10)
+    assert (xa.grad.float() - xb.grad.float()).norm() <= lim * xb.grad.float().norm()
+    assert (mine.weight.grad.float() - ref.weight.grad.float()).norm() <= lim * ref.weight.grad.float().norm()
+    assert (mine.bias.grad.float() - ref.bias.grad.float()).norm() <= lim * ref.bias.grad.float().norm()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "fp32"])
+def test_rmsnorm_module_against_the_reference_expression(dtype):
+    """The module against the eager expression of the reference's Python class (autograd through
+    torch ops in fp32), and get_norm's choices."""
+    from megatron.model.norms import LayerNorm, RMSNorm, get_norm
+
+    s, b, h = 64, 2, 1024
+    m = RMSNorm(h, eps=1e-8, bias=True).to(DEV)
+    with torch.no_grad():
+        m.scale.copy_(1 + 0.3 * torch.randn(h, generator=torch.Generator().manual_seed(1)))
+        m.offset.copy_(0.2 * torch.randn(h, generator=torch.Generator().manual_seed(2)))
+    assert sorted(n for n, _ in m.named_parameters()) == ["offset", "scale"]
+    x = util.randn((s, b, h), dtype, seed=3, std=2.0).to(DEV)
+    g = util.randn((s, b, h), dtype, seed=4).to(DEV)
+    xa = x.clone().requires_grad_(True)
+    y = m(xa)
+    y.backward(g)
+    xr = x.float().requires_grad_(True)
+    sr = m.scale.detach().clone().requires_grad_(True)
+    orf = m.offset.detach().clone().requires_grad_(True)
+    norm_x = xr.norm(2, dim=-1, keepdim=True)
+    rms_x = norm_x * h ** (-1.0 / 2)
+    ref = sr * (xr / (rms_x + 1e-8)) + orf
+    ref.backward(g.float())
+    util.assert_close_ulp_or_noise(y.detach().cpu(), ref.detach().to(dtype).cpu(), 2, out_noise(sr.detach().cpu(), x.cpu()), "y")
+    lim = 2.0 ** (-7 if dtype == torch.bfloat16 else -18)
+    assert (xa.grad.float() - xr.grad).norm() <= lim * xr.grad.norm()
+    assert (m.scale.grad - sr.grad).norm() <= lim * sr.grad.norm()
+    assert (m.offset.grad - orf.grad).norm() <= lim * orf.grad.norm()
+    args = types.SimpleNamespace(norm="rmsnorm", rms_norm_epsilon=1e-6, rmsnorm_fusion=False, layernorm_epsilon=1e-5)
+    cls, eps = get_norm(args)
+    assert cls is RMSNorm and eps == 1e-6
+    args.norm = "layernorm"
+    assert get_norm(args) == (LayerNorm, 1e-5)
+    with pytest.raises(NotImplementedError):
+        RMSNorm(h, p=0.5)
+
+
+def test_layernorm_full_size(hotpath):
+    """The hidden state of the 1.4B configuration, [2048*8, 2048] bf16 with fp32 parameters."""
+    rows, cols = 2048 * 8, 2048
+    gen = torch.Generator(device=DEV).manual_seed(0)
+    x = (torch.randn((rows, cols), generator=gen, device=DEV) * 2 + 0.5).bfloat16()
+    dy = torch.randn((rows, cols), generator=gen, device=DEV).bfloat16()
+    gamma = 1 + 0.3 * torch.randn(cols, generator=gen, device=DEV)
+    beta = 0.2 * torch.randn(cols, generator=gen, device=DEV)
+    y, mean, rstd, dx, dg, db = abi_layernorm(hotpath, x, dy, gamma, beta, 1e-5)
+    pick = torch.tensor([0, 1, 3, 4, 4095, 9001, rows - 1], device=DEV)
+    xc, dyc = x[pick].cpu(), dy[pick].cpu()
+    want_y, _, _ = oracle.layernorm_fwd(xc, gamma.cpu(), beta.cpu(), 1e-5)
+    util.assert_close_ulp_or_noise(y[pick].cpu(), want_y, 2, out_noise(gamma.cpu(), xc), "y rows")
+    want_dx, _, _ = oracle.layernorm_bwd(dyc, xc, mean[pick].cpu(), rstd[pick].cpu(), gamma.cpu())
+    util.assert_close_ulp_or_noise(dx[pick].cpu(), want_dx, 2, dx_noise(dyc, gamma.cpu(), rstd[pick].cpu()), "dx rows")
+    xr = x.float().requires_grad_(True)
+    gr = gamma.clone().requires_grad_(True)
+    br = beta.clone().requires_grad_(True)
+    F.layer_norm(xr, (cols,), gr, br, 1e-5).backward(dy.float())
+    assert (dg - gr.grad).abs().max().item() <= 1e-3 * gr.grad.abs().max().item()
+    assert (db - br.grad).abs().max().item() <= 1e-3 * br.grad.abs().max().item()
+    assert (dx.float() - xr.grad).norm().item() <= 2.0**-8 * xr.grad.norm().item()

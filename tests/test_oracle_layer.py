@@ -142,3 +142,136 @@ def test_bias_add_residual(dtype):
                        util.raw_bits((x.float() + bias.float()).to(dtype)))
     assert torch.equal(util.raw_bits(oracle.bias_add_residual(x, None, res)),
                        util.raw_bits((res.float() + x.float()).to(dtype)))
+
+
+# ---------------------------------------------------------------------------
+# LayerNorm / RMSNorm
+# ---------------------------------------------------------------------------
+def norm_inputs(dtype, rows=23, cols=80, seed=0, pdtype=None):
+    pdtype = pdtype or dtype
+    x = util.randn((rows, cols), dtype, seed=seed, std=2.0) + 0.5
+    gamma = (1 + 0.3 * torch.randn(cols, generator=torch.Generator().manual_seed(seed + 1))).to(pdtype)
+    beta = (0.2 * torch.randn(cols, generator=torch.Generator().manual_seed(seed + 2))).to(pdtype)
+    dy = util.randn((rows, cols), dtype, seed=seed + 3)
+    return x, gamma, beta, dy
+
+
+def norm_noise(x, gamma, eps_like=util.EPS32):
+    """fp32 rounding noise of a normalised, scaled value: a few fp32 spacings of |gamma| * |xhat| ~ |gamma| * 8."""
+    g = 1.0 if gamma is None else gamma.float().abs()
+    return (g * 64 * eps_like).expand_as(x.float()) if gamma is not None else torch.full_like(x.float(), 64 * eps_like)
+
+
+@pytest.mark.parametrize("pd", ["same", "fp32"])
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_layernorm_forward(dtype, pd):
+    pdtype = dtype if pd == "same" else torch.float32
+    x, gamma, beta, _ = norm_inputs(dtype, pdtype=pdtype)
+    eps = 1e-5
+    y, mean, rstd = oracle.layernorm_fwd(x, gamma, beta, eps)
+    # float64 closed form
+    xd = x.double()
+    m = xd.mean(-1, keepdim=True)
+    v = ((xd - m) ** 2).mean(-1, keepdim=True)
+    want = (xd - m) / torch.sqrt(v + eps) * gamma.double() + beta.double()
+    util.assert_close_ulp_or_noise(y, want.to(dtype), 1, norm_noise(x, gamma), "vs float64")
+    assert torch.allclose(mean.double(), m[:, 0], rtol=0, atol=1e-6)
+    assert torch.allclose(rstd.double(), (1 / torch.sqrt(v + eps))[:, 0], rtol=1e-6)
+    # torch's library routine on fp32 operands
+    lib = F.layer_norm(x.float(), (x.size(-1),), gamma.float(), beta.float(), eps).to(dtype)
+    util.assert_close_ulp_or_noise(y, lib, 1, norm_noise(x, gamma), "vs torch layer_norm")
+    # without affine terms the rows have zero mean and unit mean square (up to eps and rounding)
+    plain, _, _ = oracle.layernorm_fwd(x.float(), None, None, eps)
+    assert plain.mean(-1).abs().max() < 1e-6
+    assert ((plain ** 2).mean(-1) - 1).abs().max() < 1e-4
+    # special cases: a constant row has zero variance -> output beta; biased (not Bessel) variance
+    const = torch.full((1, 16), 3.0, dtype=dtype)
+    yc, mc, rc = oracle.layernorm_fwd(const, None, None, eps)
+    assert yc.abs().max() == 0 and mc[0] == 3.0 and abs(rc[0].item() - eps ** -0.5) < 1e-2
+    two = torch.tensor([[1.0, 3.0]], dtype=torch.float32)
+    y2, _, r2 = oracle.layernorm_fwd(two, None, None, 0.0)
+    assert torch.equal(y2, torch.tensor([[-1.0, 1.0]])) and r2[0] == 1.0
+
+
+@pytest.mark.parametrize("pd", ["same", "fp32"])
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_layernorm_backward_is_the_adjoint(dtype, pd):
+    pdtype = dtype if pd == "same" else torch.float32
+    x, gamma, beta, dy = norm_inputs(dtype, seed=4, pdtype=pdtype)
+    eps = 1e-5
+    _, mean, rstd = oracle.layernorm_fwd(x, gamma, beta, eps)
+    dx, dg, db = oracle.layernorm_bwd(dy, x, mean, rstd, gamma)
+    xd = x.double().requires_grad_(True)
+    gd = gamma.double().requires_grad_(True)
+    bd = beta.double().requires_grad_(True)
+    F.layer_norm(xd, (x.size(-1),), gd, bd, eps).backward(dy.double())
+    scale = (dy.float().abs() * gamma.float().abs()).sum(-1, keepdim=True) * rstd[:, None] * 16 * util.EPS32
+    util.assert_close_ulp_or_noise(dx, xd.grad.to(dtype), 1, scale.expand_as(dx.float()) * 8, "dx vs float64 autograd")
+    col_noise = dy.float().abs().sum(0) * 64 * util.EPS32 * 8
+    util.assert_close_ulp_or_noise(dg, gd.grad.to(pdtype), 1, col_noise, "dgamma")
+    util.assert_close_ulp_or_noise(db, bd.grad.to(pdtype), 1, col_noise, "dbeta")
+    # the gradient is orthogonal to the two directions LayerNorm removes: constants and xhat
+    x32, g32, b32, dy32 = norm_inputs(torch.float32, seed=4)
+    _, m32, r32 = oracle.layernorm_fwd(x32, g32, b32, eps)
+    dx32, _, _ = oracle.layernorm_bwd(dy32, x32, m32, r32, g32)
+    xhat = (x32 - m32[:, None]) * r32[:, None]
+    assert dx32.sum(-1).abs().max() < 1e-4
+    assert (dx32 * xhat).sum(-1).abs().max() < 1e-3
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_rmsnorm_forward(dtype, mode):
+    x, scale, offset, _ = norm_inputs(dtype, seed=8)
+    eps = 1e-6 if mode == 0 else 1e-3  # an eps large enough to tell the two placements apart
+    y, inv = oracle.rmsnorm_fwd(x, scale, offset, eps, mode)
+    xd = x.double()
+    ms = (xd ** 2).mean(-1, keepdim=True)
+    inv64 = 1 / (torch.sqrt(ms) + eps) if mode == 1 else 1 / torch.sqrt(ms + eps)
+    want = scale.double() * (xd * inv64) + offset.double()
+    util.assert_close_ulp_or_noise(y, want.to(dtype), 1, norm_noise(x, scale), "vs float64")
+    assert torch.allclose(inv.double(), inv64[:, 0], rtol=1e-6)
+    other, _ = oracle.rmsnorm_fwd(x.float(), scale.float(), offset.float(), eps, 1 - mode)
+    mine, _ = oracle.rmsnorm_fwd(x.float(), scale.float(), offset.float(), eps, mode)
+    assert not torch.equal(other, mine)
+    if mode == 1:
+        # the reference's Python class, spelled with the same torch calls in fp32
+        x32 = x.float()
+        norm_x = x32.norm(2, dim=-1, keepdim=True)
+        rms_x = norm_x * x.size(-1) ** (-1.0 / 2)
+        ref = scale.float() * (x32 / (rms_x + eps)) + offset.float()
+        util.assert_close_ulp_or_noise(y, ref.to(dtype), 1, norm_noise(x, scale), "vs the class's expression in fp32")
+    else:
+        ref = F.rms_norm(x.float(), (x.size(-1),), scale.float(), eps) + offset.float()
+        util.assert_close_ulp_or_noise(y, ref.to(dtype), 1, norm_noise(x, scale), "vs torch rms_norm")
+    # unit scale, no offset, eps 0: rows of unit mean square; an all-zero row stays zero with eps > 0
+    plain, _ = oracle.rmsnorm_fwd(x.float(), None, None, 0.0, mode)
+    assert ((plain ** 2).mean(-1) - 1).abs().max() < 1e-5
+    zero, zinv = oracle.rmsnorm_fwd(torch.zeros((1, 8), dtype=dtype), None, None, 1e-3, mode)
+    assert zero.abs().max() == 0 and torch.isfinite(zinv).all()
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_rmsnorm_backward_is_the_adjoint(dtype, mode):
+    x, scale, offset, dy = norm_inputs(dtype, seed=12)
+    eps = 1e-6 if mode == 0 else 1e-2
+    _, inv = oracle.rmsnorm_fwd(x, scale, offset, eps, mode)
+    dx, ds, do = oracle.rmsnorm_bwd(dy, x, inv, scale, eps, mode)
+    xd = x.double().requires_grad_(True)
+    sd = scale.double().requires_grad_(True)
+    od = offset.double().requires_grad_(True)
+    ms = (xd ** 2).mean(-1, keepdim=True)
+    inv64 = 1 / (torch.sqrt(ms) + eps) if mode == 1 else 1 / torch.sqrt(ms + eps)
+    (sd * (xd * inv64) + od).backward(dy.double())
+    noise = (dy.float().abs() * scale.float().abs()).sum(-1, keepdim=True) * inv[:, None] * 128 * util.EPS32
+    util.assert_close_ulp_or_noise(dx, xd.grad.to(dtype), 1, noise.expand_as(dx.float()), "dx vs float64 autograd")
+    col_noise = dy.float().abs().sum(0) * 512 * util.EPS32
+    util.assert_close_ulp_or_noise(ds, sd.grad.to(dtype), 1, col_noise, "dscale")
+    util.assert_close_ulp_or_noise(do, od.grad.to(dtype), 1, col_noise, "doffset")
+    # an all-zero row: finite gradient, the projection term vanishes
+    z = torch.zeros((1, 8), dtype=torch.float32)
+    g = torch.ones((1, 8), dtype=torch.float32)
+    _, zi = oracle.rmsnorm_fwd(z, None, None, 1e-3, mode)
+    dz, _, _ = oracle.rmsnorm_bwd(g, z, zi, None, 1e-3, mode)
+    assert torch.isfinite(dz).all() and torch.allclose(dz, g * zi[0])
