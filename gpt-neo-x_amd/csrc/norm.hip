@@ -42,15 +42,15 @@ __device__ __forceinline__ float lanes_sum(float v, uint32_t L)
     return v;
 }
 
-// Sum over the W waves of a workgroup (one row per workgroup). `slots`: 16 floats of LDS
-// not used by another reduction that could still be in flight.
+// Sum over the W waves of a row group. `slots`: W floats of LDS per row group (the caller
+// passes the group's own), not used by another reduction that could still be in flight.
 template <int W>
-__device__ __forceinline__ float waves_sum(float v, float* slots, int wave, int lane)
+__device__ __forceinline__ float waves_sum(float v, float* slots, int w, int lane)
 {
     if constexpr (W == 1) {
         return v;
     } else {
-        if (lane == 0) slots[wave] = v;
+        if (lane == 0) slots[w] = v;
         __syncthreads();
         float r = slots[0];
 #pragma unroll
@@ -86,23 +86,28 @@ __device__ __forceinline__ float rms_inverse(float sumsq, float n, float eps, in
 
 struct RowSlot {
     uint32_t row;
-    int w;
+    int w;      // which of the row's W waves
+    int group;  // row group inside the workgroup
     uint32_t l;
     bool ok;
 };
 
-// Which row (and which part of it) this thread works on in row block `rb`.
-template <int W>
+// Which row (and which part of it) this thread works on in row block `rb`. A workgroup of G
+// waves holds G / W row groups; with W = 1 a wave holds 64 / L rows of its own.
+template <int W, int G>
 __device__ __forceinline__ RowSlot locate(uint32_t rb, uint32_t rows, uint32_t L, uint32_t logL, int wave, int lane)
 {
+    static_assert(G % W == 0, "whole row groups");
     RowSlot s;
     s.l = (uint32_t)lane & (L - 1);
     if constexpr (W > 1) {
-        s.row = rb;
-        s.w = wave;
+        s.group = wave / W;
+        s.row = rb * (G / W) + (uint32_t)s.group;
+        s.w = wave % W;
     } else {
         const uint32_t rows_per_wave = 64u >> logL;
-        s.row = (rb * kNormBlockWaves + (uint32_t)wave) * rows_per_wave + ((uint32_t)lane >> logL);
+        s.group = wave;
+        s.row = (rb * G + (uint32_t)wave) * rows_per_wave + ((uint32_t)lane >> logL);
         s.w = 0;
     }
     s.ok = s.row < rows;
@@ -131,10 +136,11 @@ norm_fwd_kernel(NormFwdArgs a)
 {
     constexpr int V = Elt<DT>::kVec;
     using S = typename Elt<DT>::storage;
+    constexpr int G = (W > 1) ? W : kNormBlockWaves;
     __shared__ float slots[2][16];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const RowSlot rs = locate<W>(blockIdx.x, a.rows, a.L, a.logL, wave, lane);
+    const RowSlot rs = locate<W, G>(blockIdx.x, a.rows, a.L, a.logL, wave, lane);
     const size_t cols = (size_t)a.cpr * V;
     const float n = (float)cols;
     const S* xr = static_cast<const S*>(a.x) + (size_t)rs.row * cols;
@@ -160,7 +166,7 @@ norm_fwd_kernel(NormFwdArgs a)
 #pragma unroll
             for (int j = 0; j < V; ++j) s += f[j];
         }
-        s = waves_sum<W>(lanes_sum(s, a.L), slots[0], wave, lane);
+        s = waves_sum<W>(lanes_sum(s, a.L), slots[0], rs.w, lane);
         mean = s / n;
     }
     {
@@ -177,7 +183,7 @@ norm_fwd_kernel(NormFwdArgs a)
                 }
             }
         }
-        q = waves_sum<W>(lanes_sum(q, a.L), slots[1], wave, lane);
+        q = waves_sum<W>(lanes_sum(q, a.L), slots[1], rs.w, lane);
         scale = RMS ? rms_inverse(q, n, a.eps, a.eps_mode) : 1.0f / sqrtf(q / n + a.eps);
     }
 
@@ -278,14 +284,27 @@ struct NormBwdArgs {
     int params_f32;
 };
 
+// Waves per workgroup of the backward kernel: as many row groups as the LDS buffer of the final
+// accumulator reduction (K * V floats per thread, at most 32 KiB) and 1024 threads allow.
+template <int K, int W, int V>
+constexpr int bwd_waves()
+{
+    int g = 8192 / (K * V) / kWave;  // threads by the LDS bound, in waves
+    if (g > 16) g = 16;
+    g = g / W * W;                    // whole row groups
+    return g < W ? W : g;
+}
+
 template <int DT, int K, int W, bool RMS>
-__global__ void __launch_bounds__(((W > 1) ? W : kNormBlockWaves) * kWave)
+__global__ void __launch_bounds__((bwd_waves<K, W, Elt<DT>::kVec>() * kWave))
 norm_bwd_kernel(NormBwdArgs a)
 {
     constexpr int V = Elt<DT>::kVec;
-    constexpr int T = ((W > 1) ? W : kNormBlockWaves) * kWave;
+    constexpr int G = bwd_waves<K, W, V>();
+    constexpr int T = G * kWave;
+    constexpr int GROUPS = G / W;
     using S = typename Elt<DT>::storage;
-    __shared__ float slots[2][16];
+    __shared__ float slots[2][GROUPS > 1 ? GROUPS : 1][16];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const size_t cols = (size_t)a.cpr * V;
@@ -293,7 +312,7 @@ norm_bwd_kernel(NormBwdArgs a)
     const bool param_grads = a.part_g != nullptr;
 
     // this thread's chunk columns do not depend on the row block
-    const RowSlot first = locate<W>(0, a.rows, a.L, a.logL, wave, lane);
+    const RowSlot first = locate<W, G>(0, a.rows, a.L, a.logL, wave, lane);
     uint32_t cc[K];
     bool col_live[K];
     float gam[K][V];
@@ -313,7 +332,7 @@ norm_bwd_kernel(NormBwdArgs a)
         for (int j = 0; j < V; ++j) acc_g[k][j] = acc_b[k][j] = 0.0f;
 
     for (uint32_t rb = blockIdx.x; rb < a.row_blocks; rb += gridDim.x) {
-        const RowSlot rs = locate<W>(rb, a.rows, a.L, a.logL, wave, lane);
+        const RowSlot rs = locate<W, G>(rb, a.rows, a.L, a.logL, wave, lane);
         const S* gr = static_cast<const S*>(a.dy) + (size_t)rs.row * cols;
         const S* xr = static_cast<const S*>(a.x) + (size_t)rs.row * cols;
         u32x4 rg[K], rx[K];
@@ -351,8 +370,9 @@ norm_bwd_kernel(NormBwdArgs a)
             }
         }
         if (W > 1) __syncthreads();  // the slots of the previous row block have been read by every wave
-        if constexpr (!RMS) s1 = waves_sum<W>(lanes_sum(s1, a.L), slots[0], wave, lane);
-        s2 = waves_sum<W>(lanes_sum(s2, a.L), slots[1], wave, lane);
+        const int grp = (W > 1) ? rs.group : 0;
+        if constexpr (!RMS) s1 = waves_sum<W>(lanes_sum(s1, a.L), slots[0][grp], rs.w, lane);
+        s2 = waves_sum<W>(lanes_sum(s2, a.L), slots[1][grp], rs.w, lane);
 
         float k2 = s2 / n;
         if (RMS && a.eps_mode == 1) {
@@ -379,8 +399,8 @@ norm_bwd_kernel(NormBwdArgs a)
     }
 
     if (!param_grads) return;
-    if constexpr (W > 1) {
-        // one row per workgroup: every thread owns its columns alone
+    if constexpr (W > 1 && GROUPS == 1) {
+        // one row group: every thread owns its columns alone
 #pragma unroll
         for (int k = 0; k < K; ++k) {
             if (col_live[k]) {
@@ -394,7 +414,9 @@ norm_bwd_kernel(NormBwdArgs a)
             }
         }
     } else {
-        // the T / L threads that hold the same columns (other rows) are added up by the first of them
+        // the threads that hold the same columns for other rows are `stride` apart; the first of
+        // them adds the others up, in a fixed order
+        const uint32_t stride = (W > 1) ? (uint32_t)(W * kWave) : a.L;
         __shared__ float red[K * V * T];
         for (int pass = 0; pass < 2; ++pass) {
             __syncthreads();
@@ -403,17 +425,22 @@ norm_bwd_kernel(NormBwdArgs a)
 #pragma unroll
                 for (int j = 0; j < V; ++j) red[(k * V + j) * T + threadIdx.x] = pass == 0 ? acc_g[k][j] : acc_b[k][j];
             __syncthreads();
-            if (threadIdx.x < a.L) {
+            if (threadIdx.x < stride) {
                 float* dst = (pass == 0 ? a.part_g : a.part_b) + (size_t)blockIdx.x * cols;
 #pragma unroll
                 for (int k = 0; k < K; ++k) {
                     if (col_live[k]) {
+                        float o[V];
 #pragma unroll
                         for (int j = 0; j < V; ++j) {
                             float s = red[(k * V + j) * T + threadIdx.x];
-                            for (uint32_t t = threadIdx.x + a.L; t < (uint32_t)T; t += a.L) s += red[(k * V + j) * T + t];
-                            dst[(size_t)cc[k] * V + j] = s;
+                            for (uint32_t t = threadIdx.x + stride; t < (uint32_t)T; t += stride)
+                                s += red[(k * V + j) * T + t];
+                            o[j] = s;
                         }
+#pragma unroll
+                        for (int j = 0; j < V; j += 4)
+                            *reinterpret_cast<f32x4*>(dst + (size_t)cc[k] * V + j) = f32x4{o[j], o[j + 1], o[j + 2], o[j + 3]};
                     }
                 }
             }
@@ -421,35 +448,41 @@ norm_bwd_kernel(NormBwdArgs a)
     }
 }
 
-// out[c] = sum over t of partial[t][c], stored as fp32 or as DT; 64 columns by 4 slices of t
-// per workgroup, loads issued eight at a time. blockIdx.y selects the (partial, out) pair.
+// out[c] = sum over t of partial[t][c], stored as fp32 or as DT. A workgroup of 1024 threads
+// takes 32 columns by 32 slices of t (a thread adds the rows t = slice, slice + 32, ...,
+// eight loads in flight), then the slices are added in a fixed order through LDS.
+// blockIdx.y selects the (partial, out) pair.
+constexpr int kFinishCols = 32, kFinishSlices = 32;
+
 template <int DT>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(kFinishCols* kFinishSlices)
 param_grad_finish_kernel(void* out0, void* out1, const float* part0, const float* part1, uint32_t tiles,
                          uint32_t cols, int out_f32)
 {
-    __shared__ float lds[4][64];
+    __shared__ float lds[kFinishSlices][kFinishCols + 1];
     void* out = blockIdx.y == 0 ? out0 : out1;
     const float* partial = blockIdx.y == 0 ? part0 : part1;
     if (out == nullptr) return;
-    const uint32_t tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-    const uint32_t c = blockIdx.x * 64 + tx;
+    const uint32_t tx = threadIdx.x % kFinishCols, ty = threadIdx.x / kFinishCols;
+    const uint32_t c = blockIdx.x * kFinishCols + tx;
     float s = 0.0f;
     if (c < cols) {
         uint32_t t = ty;
-        for (; t + 28 < tiles; t += 32) {
+        for (; t + 7 * kFinishSlices < tiles; t += 8 * kFinishSlices) {
             float v[8];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) v[i] = partial[(size_t)(t + 4 * i) * cols + c];
+            for (int i = 0; i < 8; ++i) v[i] = partial[(size_t)(t + i * kFinishSlices) * cols + c];
 #pragma unroll
             for (int i = 0; i < 8; ++i) s += v[i];
         }
-        for (; t < tiles; t += 4) s += partial[(size_t)t * cols + c];
+        for (; t < tiles; t += kFinishSlices) s += partial[(size_t)t * cols + c];
     }
     lds[ty][tx] = s;
     __syncthreads();
     if (ty == 0 && c < cols) {
-        const float r = (lds[0][tx] + lds[1][tx]) + (lds[2][tx] + lds[3][tx]);
+        float r = lds[0][tx];
+#pragma unroll
+        for (int i = 1; i < kFinishSlices; ++i) r += lds[i][tx];
         if (out_f32)
             static_cast<float*>(out)[c] = r;
         else
@@ -539,10 +572,11 @@ struct NormPlan {
 };
 
 // (K, W) pairs that are compiled
-#define NHP_NORM_GEOMETRIES(X) X(1, 1) X(2, 1) X(4, 1) X(2, 2) X(2, 4) X(2, 8) X(4, 8) X(4, 16)
+#define NHP_NORM_GEOMETRIES(X) X(1, 1) X(2, 1) X(4, 1) X(1, 2) X(2, 2) X(1, 4) X(2, 4) X(2, 8) X(4, 8) X(4, 16)
 
-// Geometry for rows of cpr chunks: a wave reads 1-2 KiB of a row; returns false when the row does not fit.
-static bool plan_norm(int64_t cpr, NormPlan& p)
+// Geometry for rows of cpr chunks: a wave reads 1-2 KiB of a row (1 KiB of each of its two
+// inputs in the backward); returns false when the row does not fit.
+static bool plan_norm(int64_t cpr, bool backward, NormPlan& p)
 {
     if (cpr < 1) return false;
     p.L = 1;
@@ -552,9 +586,10 @@ static bool plan_norm(int64_t cpr, NormPlan& p)
         ++p.logL;
     }
     const int64_t segs = (cpr + p.L - 1) / p.L;  // 16-byte chunks per lane over the whole row
-    static const int table[][2] = {{1, 1}, {2, 1}, {2, 2}, {2, 4}, {2, 8}, {4, 8}, {4, 16}};
+    static const int fwd_table[][2] = {{1, 1}, {2, 1}, {2, 2}, {2, 4}, {2, 8}, {4, 8}, {4, 16}};
+    static const int bwd_table[][2] = {{1, 1}, {1, 2}, {1, 4}, {2, 4}, {2, 8}, {4, 8}, {4, 16}};
     p.K = p.W = 0;
-    for (const auto& kw : table) {
+    for (const auto& kw : (backward ? bwd_table : fwd_table)) {
         if ((int64_t)kw[0] * kw[1] >= segs) {
             p.K = kw[0];
             p.W = kw[1];
@@ -569,18 +604,29 @@ static bool plan_norm(int64_t cpr, NormPlan& p)
     return p.K != 0;
 }
 
-static uint32_t norm_row_blocks(int64_t rows, const NormPlan& p)
+// Row blocks when a workgroup has `waves` waves.
+static uint32_t norm_row_blocks(int64_t rows, const NormPlan& p, int waves)
 {
-    const int64_t rows_per_block = p.W > 1 ? 1 : (int64_t)kNormBlockWaves * (64 / p.L);
+    const int64_t rows_per_block = p.W > 1 ? waves / p.W : (int64_t)waves * (64 / p.L);
     return (uint32_t)((rows + rows_per_block - 1) / rows_per_block);
 }
 
-constexpr uint32_t kNormBwdGrid = 1024;  // workgroups of the backward kernel when parameter gradients are wanted
+static int bwd_waves_of(const NormPlan& p, int v)
+{
+    int g = 8192 / (p.K * v) / kWave;
+    if (g > 16) g = 16;
+    g = g / p.W * p.W;
+    return g < p.W ? p.W : g;
+}
 
-static uint32_t norm_bwd_grid(uint32_t row_blocks, bool param_grads)
+// With parameter gradients the backward grid is bounded (every workgroup writes a partial row
+// that the second kernel has to read): 4096 waves in all, 16 per CU.
+constexpr uint32_t kNormBwdWaves = 4096;
+
+static uint32_t norm_bwd_grid(uint32_t row_blocks, bool param_grads, int waves_per_block)
 {
     if (!param_grads) return row_blocks;
-    const uint32_t cap = (uint32_t)norm_tune("NHP_NORM_GRID", kNormBwdGrid);
+    const uint32_t cap = (uint32_t)norm_tune("NHP_NORM_GRID", (int)(kNormBwdWaves / (uint32_t)waves_per_block));
     return row_blocks < cap ? row_blocks : cap;
 }
 
@@ -593,11 +639,12 @@ static int norm_fwd(void* y, float* mean, float* rstd, const void* x, const void
     constexpr int V = Elt<DT>::kVec;
     NormPlan p;
     const bool params_aligned = ptr_aligned16(gamma) && ptr_aligned16(beta);
-    if (cols % V == 0 && ptr_aligned16(x) && ptr_aligned16(y) && params_aligned && plan_norm(cols / V, p)) {
+    if (cols % V == 0 && ptr_aligned16(x) && ptr_aligned16(y) && params_aligned && plan_norm(cols / V, false, p)) {
         NormFwdArgs a{y, mean, rstd, x, gamma, beta, eps, eps_mode, (uint32_t)rows, (uint32_t)(cols / V),
                       p.L, p.logL, pdt == NHP_F32 ? 1 : 0};
-        const uint32_t blocks = norm_row_blocks(rows, p);
-        const int threads = (p.W > 1 ? p.W : kNormBlockWaves) * kWave;
+        const int waves = p.W > 1 ? p.W : kNormBlockWaves;
+        const uint32_t blocks = norm_row_blocks(rows, p, waves);
+        const int threads = waves * kWave;
         if (!grid_fits(blocks, threads)) return NHP_ERR_SHAPE;
 #define X(K_, W_)                                                                      \
     if (p.K == K_ && p.W == W_) {                                                      \
@@ -618,8 +665,9 @@ static int64_t norm_workspace_bytes(int64_t rows, int64_t cols, int dtype)
 {
     const int v = dtype == NHP_F32 ? 4 : 8;
     NormPlan p;
-    if (rows <= 0 || cols <= 0 || cols % v != 0 || !plan_norm(cols / v, p)) return 0;
-    return 2 * (int64_t)norm_bwd_grid(norm_row_blocks(rows, p), true) * cols * (int64_t)sizeof(float);
+    if (rows <= 0 || cols <= 0 || cols % v != 0 || !plan_norm(cols / v, true, p)) return 0;
+    const int waves = bwd_waves_of(p, v);
+    return 2 * (int64_t)norm_bwd_grid(norm_row_blocks(rows, p, waves), true, waves) * cols * (int64_t)sizeof(float);
 }
 
 template <int DT, bool RMS>
@@ -631,14 +679,15 @@ static int norm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, const v
     NormPlan p;
     const bool want_params = dgamma != nullptr || dbeta != nullptr;
     if (cols % V == 0 && ptr_aligned16(dx) && ptr_aligned16(dy) && ptr_aligned16(x) && ptr_aligned16(gamma) &&
-        ptr_aligned16(workspace) && plan_norm(cols / V, p)) {
-        const uint32_t row_blocks = norm_row_blocks(rows, p);
-        const uint32_t grid = norm_bwd_grid(row_blocks, want_params);
+        ptr_aligned16(workspace) && plan_norm(cols / V, true, p)) {
+        const int waves = bwd_waves_of(p, V);
+        const uint32_t row_blocks = norm_row_blocks(rows, p, waves);
+        const uint32_t grid = norm_bwd_grid(row_blocks, want_params, waves);
         float* part_g = want_params ? static_cast<float*>(workspace) : nullptr;
         float* part_b = want_params ? part_g + (size_t)grid * cols : nullptr;
         NormBwdArgs a{dx, part_g, part_b, dy, x, mean, rstd, gamma, eps, eps_mode, (uint32_t)rows,
                       (uint32_t)(cols / V), p.L, p.logL, row_blocks, pdt == NHP_F32 ? 1 : 0};
-        const int threads = (p.W > 1 ? p.W : kNormBlockWaves) * kWave;
+        const int threads = waves * kWave;
         if (!grid_fits(grid, threads)) return NHP_ERR_SHAPE;
         bool launched = false;
 #define X(K_, W_)                                                                      \
@@ -651,8 +700,8 @@ static int norm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, const v
         if (!launched) return NHP_ERR_SHAPE;
         int rc = launch_result();
         if (rc != NHP_OK || !want_params) return rc;
-        const dim3 fgrid((uint32_t)((cols + 63) / 64), 2);
-        param_grad_finish_kernel<DT><<<fgrid, 256, 0, st>>>(dgamma, dbeta, part_g, part_b, grid, (uint32_t)cols,
+        const dim3 fgrid((uint32_t)((cols + kFinishCols - 1) / kFinishCols), 2);
+        param_grad_finish_kernel<DT><<<fgrid, kFinishCols * kFinishSlices, 0, st>>>(dgamma, dbeta, part_g, part_b, grid, (uint32_t)cols,
                                                             pdt == NHP_F32 ? 1 : 0);
         return launch_result();
     }
