@@ -1,7 +1,9 @@
 #!/usr/bin/env python3
-"""Writes tests/golden/hotpath_golden.npz: small seeded inputs and the outputs
-of the CPU oracle (oracle/kernel_semantics.c) for every entry point, stored as
-raw bit patterns. The oracle itself is pinned by tests/test_oracle_*.py; these
+"""Writes tests/golden/hotpath_golden.npz (softmax and rotary entry points) and
+tests/golden/layer_golden.npz (the window / AliBi / bias / key-length variants of
+the causal softmax, bias + GeLU, bias + residual add, LayerNorm, RMSNorm): small
+seeded inputs and the outputs of the CPU oracle (oracle/*.c), stored as raw bit
+patterns. The oracle itself is pinned by tests/test_oracle_*.py; these
 vectors freeze its answers so that the GPU path (and any later change to the
 oracle) is compared against fixed data.
 
@@ -69,6 +71,50 @@ def main():
             fwd_freqs=oracle.rope_freqs(t, ang), bwd_freqs=oracle.rope_freqs(t, ang, backward=True))
 
     path = os.path.join(HERE, "hotpath_golden.npz")
+    np.savez_compressed(path, **out)
+    print(path, os.path.getsize(path), "bytes,", len(out), "arrays")
+
+    out.clear()
+    for name, dtype, seed in (("ex_bf16", torch.bfloat16, 11), ("ex_fp16", torch.float16, 12)):
+        batch, heads, s, window, scale = 2, 2, 24, 5, 0.25
+        x = util.randn((batch * heads, s, s), dtype, seed, std=2.0)
+        dy = util.randn((batch * heads, s, s), dtype, seed + 100)
+        bias = util.randn((heads, s, s), dtype, seed + 200)
+        slopes = torch.tensor([0.5, 0.0625], dtype=torch.float32)
+        lengths = torch.tensor([24, 9], dtype=torch.int32)
+        y = oracle.causal_softmax_fwd(x, scale, window=window, alibi_slopes=slopes, bias=bias, key_lengths=lengths)
+        dx = oracle.softmax_bwd(dy, y, scale, True, window=window, key_lengths=lengths)
+        put(name, x=x, dy=dy, bias=bias, slopes=slopes, lengths=lengths, y=y, dx=dx, window=np.int64(window),
+            scale=np.float32(scale))
+
+    for name, dtype, seed in (("gelu_bf16", torch.bfloat16, 21), ("gelu_fp16", torch.float16, 22),
+                              ("gelu_fp32", torch.float32, 23)):
+        y = util.randn((6, 16), dtype, seed, std=3.0)
+        bias = util.randn((16,), dtype, seed + 1, std=0.5)
+        g = util.randn((6, 16), dtype, seed + 2)
+        res = util.randn((6, 16), dtype, seed + 3, std=2.0)
+        dx = oracle.bias_gelu_bwd(g, y, bias)
+        put(name, y=y, bias=bias, g=g, res=res, out=oracle.bias_gelu_fwd(y, bias), dx=dx, dbias=oracle.column_sum(dx),
+            added=oracle.bias_add_residual(y, bias, res))
+
+    for name, dtype, seed in (("norm_bf16", torch.bfloat16, 31), ("norm_fp16", torch.float16, 32),
+                              ("norm_fp32", torch.float32, 33)):
+        x = util.randn((5, 24), dtype, seed, std=2.0) + 0.5
+        dy = util.randn((5, 24), dtype, seed + 1)
+        g = torch.Generator().manual_seed(seed)
+        gamma = (1 + 0.3 * torch.randn(24, generator=g)).to(dtype)
+        beta = (0.2 * torch.randn(24, generator=g)).to(dtype)
+        y, mean, rstd = oracle.layernorm_fwd(x, gamma, beta, 1e-5)
+        dx, dg, db = oracle.layernorm_bwd(dy, x, mean, rstd, gamma)
+        put(name, x=x, dy=dy, gamma=gamma, beta=beta, ln_y=y, ln_mean=mean, ln_rstd=rstd, ln_dx=dx, ln_dgamma=dg,
+            ln_dbeta=db)
+        for mode, eps in ((0, 1e-5), (1, 1e-2)):
+            ry, inv = oracle.rmsnorm_fwd(x, gamma, beta, eps, mode)
+            rdx, rds, rdo = oracle.rmsnorm_bwd(dy, x, inv, gamma, eps, mode)
+            put(name, **{f"rms{mode}_y": ry, f"rms{mode}_inv": inv, f"rms{mode}_dx": rdx, f"rms{mode}_dscale": rds,
+                         f"rms{mode}_doffset": rdo, f"rms{mode}_eps": np.float32(eps)})
+
+    path = os.path.join(HERE, "layer_golden.npz")
     np.savez_compressed(path, **out)
     print(path, os.path.getsize(path), "bytes,", len(out), "arrays")
 

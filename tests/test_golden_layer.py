@@ -1,0 +1,155 @@
+"""Committed golden vectors of the causal-softmax variants and the layer kernels
+(tests/golden/layer_golden.npz, written by tests/golden/make_golden.py from the CPU
+oracle). Without a GPU: the oracle reproduces them bit for bit. With a GPU: the HIP
+path, called through the C ABI, matches them to the tolerance of the parity tests."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import util
+
+GOLDEN = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "layer_golden.npz"))
+DT = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}
+FP32_KEYS = ("slopes", "ln_mean", "ln_rstd", "rms0_inv", "rms1_inv")
+
+
+def get(prefix, key):
+    arr = GOLDEN[f"{prefix}.{key}"]
+    if arr.ndim == 0:
+        return arr.item()
+    t = torch.from_numpy(np.ascontiguousarray(arr))
+    if key == "lengths":
+        return t
+    if key in FP32_KEYS:
+        return t.view(torch.float32)
+    return t.view(DT[prefix.split("_")[-1]])
+
+
+def same(a, b):
+    return torch.equal(util.raw_bits(a), util.raw_bits(b))
+
+
+EX = ["ex_bf16", "ex_fp16"]
+GELU = ["gelu_bf16", "gelu_fp16", "gelu_fp32"]
+NORM = ["norm_bf16", "norm_fp16", "norm_fp32"]
+
+
+@pytest.mark.parametrize("name", EX)
+def test_oracle_reproduces_softmax_variant_golden(name):
+    x, dy, bias, slopes, lengths = (get(name, k) for k in ("x", "dy", "bias", "slopes", "lengths"))
+    window, scale = get(name, "window"), get(name, "scale")
+    y = oracle.causal_softmax_fwd(x, scale, window=window, alibi_slopes=slopes, bias=bias, key_lengths=lengths)
+    assert same(y, get(name, "y"))
+    assert same(oracle.softmax_bwd(dy, y, scale, True, window=window, key_lengths=lengths), get(name, "dx"))
+
+
+@pytest.mark.parametrize("name", GELU)
+def test_oracle_reproduces_gelu_golden(name):
+    y, bias, g, res = (get(name, k) for k in ("y", "bias", "g", "res"))
+    assert same(oracle.bias_gelu_fwd(y, bias), get(name, "out"))
+    dx = oracle.bias_gelu_bwd(g, y, bias)
+    assert same(dx, get(name, "dx")) and same(oracle.column_sum(dx), get(name, "dbias"))
+    assert same(oracle.bias_add_residual(y, bias, res), get(name, "added"))
+
+
+@pytest.mark.parametrize("name", NORM)
+def test_oracle_reproduces_norm_golden(name):
+    x, dy, gamma, beta = (get(name, k) for k in ("x", "dy", "gamma", "beta"))
+    y, mean, rstd = oracle.layernorm_fwd(x, gamma, beta, 1e-5)
+    assert same(y, get(name, "ln_y")) and same(mean, get(name, "ln_mean")) and same(rstd, get(name, "ln_rstd"))
+    dx, dg, db = oracle.layernorm_bwd(dy, x, mean, rstd, gamma)
+    assert same(dx, get(name, "ln_dx")) and same(dg, get(name, "ln_dgamma")) and same(db, get(name, "ln_dbeta"))
+    for mode in (0, 1):
+        eps = get(name, f"rms{mode}_eps")
+        ry, inv = oracle.rmsnorm_fwd(x, gamma, beta, eps, mode)
+        assert same(ry, get(name, f"rms{mode}_y")) and same(inv, get(name, f"rms{mode}_inv"))
+        rdx, rds, rdo = oracle.rmsnorm_bwd(dy, x, inv, gamma, eps, mode)
+        assert same(rdx, get(name, f"rms{mode}_dx")) and same(rds, get(name, f"rms{mode}_dscale"))
+        assert same(rdo, get(name, f"rms{mode}_doffset"))
+
+
+def ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", EX)
+def test_gpu_matches_softmax_variant_golden(hotpath, name):
+    x, dy, bias, slopes, lengths, y, dx = (get(name, k).cuda() for k in ("x", "dy", "bias", "slopes", "lengths", "y", "dx"))
+    window, scale = get(name, "window"), get(name, "scale")
+    L, code = hotpath.lib(), hotpath.dtype_code(x, "t")
+    got = torch.empty_like(x)
+    assert L.nhp_causal_softmax_ex_fwd(got.data_ptr(), x.data_ptr(), scale, x.size(0), x.size(1), window, slopes.data_ptr(),
+                                       bias.data_ptr(), lengths.data_ptr(), 2, code, None) == 0
+    zeros = util.raw_bits(y.cpu()) == 0
+    assert int(util.raw_bits(got.cpu())[zeros & (y.cpu().float() == 0)].abs().max()) == 0
+    util.assert_ulp_close(got.cpu(), y.cpu(), 2, name)
+    gdx = torch.empty_like(x)
+    assert L.nhp_causal_softmax_ex_bwd(gdx.data_ptr(), dy.data_ptr(), y.data_ptr(), scale, x.size(0), x.size(1), window,
+                                       lengths.data_ptr(), 2, code, None) == 0
+    util.assert_softmax_bwd_close(gdx.cpu(), dx.cpu(), dy.cpu() * (y.cpu() != 0), y.cpu(), scale, name)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", GELU)
+def test_gpu_matches_gelu_golden(hotpath, name):
+    y, bias, g, res = (get(name, k).cuda() for k in ("y", "bias", "g", "res"))
+    L, code = hotpath.lib(), hotpath.dtype_code(y, "t")
+    rows, cols = y.shape
+    x32 = (bias.float() + y.float()).cpu()
+    out = torch.empty_like(y)
+    assert L.nhp_bias_gelu_fwd(out.data_ptr(), y.data_ptr(), bias.data_ptr(), rows, cols, code, None) == 0
+    util.assert_close_ulp_or_noise(out.cpu(), get(name, "out"), 2, util.gelu_noise(x32), name)
+    dx, dbias = torch.empty_like(y), torch.empty_like(bias)
+    ws = torch.empty(max(L.nhp_bias_gelu_bwd_workspace_bytes(rows, cols, code), 16), dtype=torch.uint8, device="cuda")
+    assert L.nhp_bias_gelu_bwd(dx.data_ptr(), g.data_ptr(), y.data_ptr(), bias.data_ptr(), dbias.data_ptr(), ws.data_ptr(),
+                               rows, cols, code, None) == 0
+    util.assert_close_ulp_or_noise(dx.cpu(), get(name, "dx"), 2, util.gelu_noise(x32, g.cpu()), name)
+    util.assert_close_ulp_or_noise(dbias.cpu(), oracle.column_sum(dx.cpu()), 1, dx.float().abs().sum(0).cpu() * 16 * util.EPS32, name)
+    added = torch.empty_like(y)
+    assert L.nhp_bias_add_residual(added.data_ptr(), y.data_ptr(), bias.data_ptr(), res.data_ptr(), rows, cols, code, None) == 0
+    assert same(added.cpu(), get(name, "added"))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", NORM)
+def test_gpu_matches_norm_golden(hotpath, name):
+    x, dy, gamma, beta = (get(name, k).cuda() for k in ("x", "dy", "gamma", "beta"))
+    L, code = hotpath.lib(), hotpath.dtype_code(x, "t")
+    rows, cols = x.shape
+    noise_y = (gamma.float().abs().cpu() * 64 * util.EPS32).expand(rows, cols)
+    ws = torch.empty(max(L.nhp_norm_bwd_workspace_bytes(rows, cols, code), 16), dtype=torch.uint8, device="cuda")
+
+    def dx_noise(inv):
+        return ((dy.float().abs() * gamma.float().abs()).sum(-1, keepdim=True).cpu() * inv[:, None] * 64 * util.EPS32).expand(rows, cols)
+
+    col = dy.float().abs().sum(0).cpu() * 8 * 64 * util.EPS32
+    y, mean, rstd = torch.empty_like(x), torch.empty(rows, device="cuda"), torch.empty(rows, device="cuda")
+    assert L.nhp_layernorm_fwd(y.data_ptr(), mean.data_ptr(), rstd.data_ptr(), x.data_ptr(), gamma.data_ptr(), beta.data_ptr(),
+                               1e-5, rows, cols, code, code, None) == 0
+    util.assert_close_ulp_or_noise(y.cpu(), get(name, "ln_y"), 2, noise_y, name)
+    assert torch.allclose(mean.cpu(), get(name, "ln_mean"), rtol=0, atol=1e-5)
+    assert torch.allclose(rstd.cpu(), get(name, "ln_rstd"), rtol=1e-5, atol=0)
+    gm, gr = get(name, "ln_mean").cuda(), get(name, "ln_rstd").cuda()
+    dx, dg, db = torch.empty_like(x), torch.empty_like(gamma), torch.empty_like(beta)
+    assert L.nhp_layernorm_bwd(dx.data_ptr(), dg.data_ptr(), db.data_ptr(), dy.data_ptr(), x.data_ptr(), gm.data_ptr(),
+                               gr.data_ptr(), gamma.data_ptr(), ws.data_ptr(), rows, cols, code, code, None) == 0
+    util.assert_close_ulp_or_noise(dx.cpu(), get(name, "ln_dx"), 2, dx_noise(gr.cpu()), name)
+    util.assert_close_ulp_or_noise(dg.cpu(), get(name, "ln_dgamma"), 2, col, name)
+    util.assert_close_ulp_or_noise(db.cpu(), get(name, "ln_dbeta"), 2, col, name)
+    for mode in (0, 1):
+        eps = get(name, f"rms{mode}_eps")
+        inv = torch.empty(rows, device="cuda")
+        assert L.nhp_rmsnorm_fwd(y.data_ptr(), inv.data_ptr(), x.data_ptr(), gamma.data_ptr(), beta.data_ptr(), eps, mode,
+                                 rows, cols, code, code, None) == 0
+        util.assert_close_ulp_or_noise(y.cpu(), get(name, f"rms{mode}_y"), 2, noise_y, name)
+        gi = get(name, f"rms{mode}_inv").cuda()
+        assert torch.allclose(inv.cpu(), gi.cpu(), rtol=1e-5, atol=0)
+        assert L.nhp_rmsnorm_bwd(dx.data_ptr(), dg.data_ptr(), db.data_ptr(), dy.data_ptr(), x.data_ptr(), gi.data_ptr(),
+                                 gamma.data_ptr(), ws.data_ptr(), eps, mode, rows, cols, code, code, None) == 0
+        util.assert_close_ulp_or_noise(dx.cpu(), get(name, f"rms{mode}_dx"), 2, dx_noise(gi.cpu()), name)
+        util.assert_close_ulp_or_noise(dg.cpu(), get(name, f"rms{mode}_dscale"), 2, col, name)
+        util.assert_close_ulp_or_noise(db.cpu(), get(name, f"rms{mode}_doffset"), 2, col, name)
