@@ -233,8 +233,10 @@ def make_workload(name, torch, dev):
         return step, kernel_bytes, {}, "rope_qk_fwd", "bf16", cfg
 
     if name == "mlp-gelu-1.4b":
-        from megatron.model.activations import bias_gelu, _bias_gelu_backward
+        # through the C ABI with preallocated outputs and workspace
+        from megatron.fused_kernels import _hotpath as hp
 
+        lib = hp.lib()
         rows, cols = 2048 * 8, 8192
         sets = []
         for i in range(2):  # two buffer sets: a 256 MiB tensor alone would sit in the last-level cache
@@ -245,15 +247,27 @@ def make_workload(name, torch, dev):
                 g[r:r + 2048] = randn((2048, cols), 100 * i + r + 1, torch.bfloat16)
             sets.append((y, g))
         bias = randn((cols,), 5, torch.bfloat16, 0.5)
+        out = torch.empty_like(sets[0][0])
+        dbias = torch.empty_like(bias)
+        ws = torch.empty(max(lib.nhp_bias_gelu_bwd_workspace_bytes(rows, cols, hp.BF16), 16), dtype=torch.uint8, device=dev)
         n = rows * cols
         kernel_bytes = {"bias_gelu_fwd": 2 * n * 2 + cols * 2, "bias_gelu_bwd": 3 * n * 2 + 2 * cols * 2}
         state = {"i": 0}
+        stream = hp.stream_of(out)
+
+        def fwd(y):
+            hp.check(lib.nhp_bias_gelu_fwd(out.data_ptr(), y.data_ptr(), bias.data_ptr(), rows, cols, hp.BF16, stream),
+                     "bias_gelu forward")
+
+        def bwd(y, g):
+            hp.check(lib.nhp_bias_gelu_bwd(out.data_ptr(), g.data_ptr(), y.data_ptr(), bias.data_ptr(), dbias.data_ptr(),
+                                           ws.data_ptr(), rows, cols, hp.BF16, stream), "bias_gelu backward")
 
         def step(t):
             y, g = sets[state["i"] % len(sets)]
             state["i"] += 1
-            t.run("bias_gelu_fwd", lambda: bias_gelu(bias, y))
-            t.run("bias_gelu_bwd", lambda: _bias_gelu_backward(g, bias, y, True))
+            t.run("bias_gelu_fwd", lambda: fwd(y))
+            t.run("bias_gelu_bwd", lambda: bwd(y, g))
 
         cfg = {"workload": name, "activation": [rows, cols], "bias_gradient": "fused column sums",
                "bytes_convention": "every tensor element read or written once"}

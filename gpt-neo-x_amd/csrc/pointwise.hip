@@ -16,6 +16,7 @@
 // `1 + tanh` that follows it in the reference formula).
 
 #include "common.hpp"
+#include "colsum.hpp"
 
 #include <cstdlib>
 
@@ -194,34 +195,6 @@ pointwise_kernel(void* out, const void* a, const void* b, const void* bias, floa
     }
 }
 
-// out[c] = storage(sum over t of partial[t][c]); 64 columns by 4 slices of t per
-// workgroup. The loads of a thread are independent: they are issued eight at a
-// time, since with one in flight the kernel would take `tiles / 4` memory
-// latencies.
-template <int DT>
-__global__ void __launch_bounds__(kPwThreads)
-column_sum_finish_kernel(void* out, const float* partial, uint32_t tiles, uint32_t cols)
-{
-    __shared__ float lds[4][64];
-    const uint32_t tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-    const uint32_t c = blockIdx.x * 64 + tx;
-    float s = 0.0f;
-    if (c < cols) {
-        uint32_t t = ty;
-        for (; t + 28 < tiles; t += 32) {
-            float v[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) v[i] = partial[(size_t)(t + 4 * i) * cols + c];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) s += v[i];
-        }
-        for (; t < tiles; t += 4) s += partial[(size_t)t * cols + c];
-    }
-    lds[ty][tx] = s;
-    __syncthreads();
-    if (ty == 0 && c < cols) Elt<DT>::store(out, c, (lds[0][tx] + lds[1][tx]) + (lds[2][tx] + lds[3][tx]));
-}
-
 // ---------------------------------------------------------------------------
 // Scalar kernels for shapes the chunked layout cannot take (cols not a
 // multiple of the chunk, unaligned pointers).
@@ -277,8 +250,8 @@ constexpr int kPwMaxTw = 64;  // a wave reads 1 KiB of a row
 // Dynamic LDS asked for only to bound the resident workgroups per CU: with two
 // input tensors six workgroups per CU stream better than eight (measured).
 constexpr uint32_t kPwLdsTwoInputs = 24576;
-// With column sums the grid is bounded, so that few partial rows are written.
-constexpr uint32_t kPwColsumGridY = 128;
+// With column sums the grid is bounded, so that the partial rows stay a few per cent of the traffic.
+constexpr uint32_t kPwColsumGridY = 512;
 
 // Tile shape for a [rows, cols] tensor of cpr chunks per row.
 static TilePlan plan_tiles(int64_t rows, int64_t cpr, bool colsum)
@@ -312,8 +285,9 @@ static int launch_tiled(void* out, const void* a, const void* b, const void* bia
         switch (pw_tune("NHP_PW_U", kPwU)) {                                                             \
         case 1: CASE_U(TW_, 1) break;                                                                    \
         case 2: CASE_U(TW_, 2) break;                                                                    \
+        case 4: CASE_U(TW_, 4) break;                                                                    \
         case 8: CASE_U(TW_, 8) break;                                                                    \
-        default: CASE_U(TW_, kPwU) break;                                                                \
+        default: return NHP_ERR_SHAPE;                                                                   \
         }                                                                                                \
         break;
 #else
@@ -352,10 +326,10 @@ static int run_pointwise(void* out, const void* a, const void* b, const void* bi
             const TilePlan p = plan_tiles(rows, cpr, true);
             int rc = launch_tiled<DT, OP, true>(out, a, b, bias, workspace, rows, cpr, p, st);
             if (rc != NHP_OK) return rc;
-            const int64_t blocks = (cols + 63) / 64;
-            if (!grid_fits(blocks, kPwThreads)) return NHP_ERR_SHAPE;
-            column_sum_finish_kernel<DT><<<(uint32_t)blocks, kPwThreads, 0, st>>>(dbias, workspace, p.grid_y,
-                                                                                (uint32_t)cols);
+            const int64_t blocks = (cols + kFinishCols - 1) / kFinishCols;
+            if (!grid_fits(blocks, kFinishCols * kFinishSlices)) return NHP_ERR_SHAPE;
+            partial_rows_sum_kernel<DT><<<dim3((uint32_t)blocks, 1), kFinishCols * kFinishSlices, 0, st>>>(
+                dbias, nullptr, workspace, nullptr, p.grid_y, (uint32_t)cols, DT == NHP_F32 ? 1 : 0);
             return launch_result();
         }
         return NHP_ERR_SHAPE;
