@@ -305,7 +305,9 @@ norm_bwd_kernel(NormBwdArgs a)
     constexpr int T = G * kWave;
     constexpr int GROUPS = G / W;
     using S = typename Elt<DT>::storage;
-    __shared__ float slots[2][GROUPS > 1 ? GROUPS : 1][16];
+    // [parity of the loop iteration][sum][row group][wave]: one barrier per iteration is enough when
+    // consecutive iterations use different slots
+    __shared__ float slots[2][2][GROUPS > 1 ? GROUPS : 1][16];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const size_t cols = (size_t)a.cpr * V;
@@ -332,11 +334,11 @@ norm_bwd_kernel(NormBwdArgs a)
 #pragma unroll
         for (int j = 0; j < V; ++j) acc_g[k][j] = acc_b[k][j] = 0.0f;
 
-    for (uint32_t rb = blockIdx.x; rb < a.row_blocks; rb += gridDim.x) {
+    // loads of one row block (this thread's chunks of dy and x, the row's statistics)
+    auto fetch = [&](uint32_t rb, u32x4 (&rg)[K], u32x4 (&rx)[K], float& mean, float& scale) {
         const RowSlot rs = locate<W, G>(rb, a.rows, a.L, a.logL, wave, lane);
         const S* gr = static_cast<const S*>(a.dy) + (size_t)rs.row * cols;
         const S* xr = static_cast<const S*>(a.x) + (size_t)rs.row * cols;
-        u32x4 rg[K], rx[K];
 #pragma unroll
         for (int k = 0; k < K; ++k) {
             rg[k] = u32x4{0, 0, 0, 0};
@@ -346,11 +348,25 @@ norm_bwd_kernel(NormBwdArgs a)
                 rx[k] = load16_stream(xr + (size_t)cc[k] * V);
             }
         }
-        float mean = 0.0f, scale = 0.0f;
+        mean = 0.0f;
+        scale = 0.0f;
         if (rs.ok) {
             if (!RMS) mean = a.mean[rs.row];
             scale = a.rstd[rs.row];
         }
+    };
+
+    u32x4 rg[K], rx[K];
+    float mean = 0.0f, scale = 0.0f;
+    int parity = 0;
+    if (blockIdx.x < a.row_blocks) fetch(blockIdx.x, rg, rx, mean, scale);
+    for (uint32_t rb = blockIdx.x; rb < a.row_blocks; rb += gridDim.x) {
+        const RowSlot rs = locate<W, G>(rb, a.rows, a.L, a.logL, wave, lane);
+        // the next row block's loads are in flight while this one is reduced and stored
+        u32x4 ng[K], nx[K];
+        float nmean = 0.0f, nscale = 0.0f;
+        const uint32_t next = rb + gridDim.x;
+        if (next < a.row_blocks) fetch(next, ng, nx, nmean, nscale);
 
         float s1 = 0.0f, s2 = 0.0f;
 #pragma unroll
@@ -370,11 +386,29 @@ norm_bwd_kernel(NormBwdArgs a)
                 }
             }
         }
-        if (W > 1) __syncthreads();  // the slots of the previous row block have been read by every wave
-        const int grp = (W > 1) ? rs.group : 0;
-        if constexpr (!RMS) s1 = waves_sum<W>(lanes_sum(s1, a.L), slots[0][grp], rs.w, lane);
-        s2 = waves_sum<W>(lanes_sum(s2, a.L), slots[1][grp], rs.w, lane);
+        s1 = lanes_sum(s1, a.L);
+        s2 = lanes_sum(s2, a.L);
+        if constexpr (W > 1) {
+            // both sums cross the row's waves behind one barrier
+            float* mine1 = slots[parity][0][rs.group];
+            float* mine2 = slots[parity][1][rs.group];
+            if (lane == 0) {
+                mine1[rs.w] = s1;
+                mine2[rs.w] = s2;
+            }
+            __syncthreads();
+            s1 = mine1[0];
+            s2 = mine2[0];
+#pragma unroll
+            for (int i = 1; i < W; ++i) {
+                s1 += mine1[i];
+                s2 += mine2[i];
+            }
+            parity ^= 1;
+        }
 
+        // LayerNorm: t = (s1 + xhat * s2) / n as c1 + xhat * c2 (no division per element)
+        const float c1 = s1 / n;
         float k2 = s2 / n;
         if (RMS && a.eps_mode == 1) {
             const float rho = 1.0f - a.eps * scale;
@@ -391,11 +425,20 @@ norm_bwd_kernel(NormBwdArgs a)
                 for (int j = 0; j < V; ++j) {
                     const float xh = (fx[j] - mean) * scale;
                     const float g = fg[j] * gam[k][j];
-                    const float t = RMS ? xh * k2 : (s1 + xh * s2) / n;
+                    const float t = RMS ? xh * k2 : c1 + xh * k2;
                     o[j] = scale * (g - t);
                 }
                 store16_stream(dr + (size_t)cc[k] * V, float_to_chunk<DT>(o));
             }
+        }
+        if (next < a.row_blocks) {
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+                rg[k] = ng[k];
+                rx[k] = nx[k];
+            }
+            mean = nmean;
+            scale = nscale;
         }
     }
 
