@@ -112,6 +112,51 @@ def test_argument_validation_needs_no_gpu(hotpath):
     assert lib.nhp_rope_cached_fwd(p, p, p, p, 1, 1, 1, 8, 8, st, st, BF16, BF16, None) == -6
 
 
+def test_argument_validation_of_the_layer_entry_points(hotpath):
+    lib = hotpath.lib()
+    F16, BF16, F32 = hotpath.F16, hotpath.BF16, hotpath.F32
+    p = ctypes.c_void_p(0x1000)  # never dereferenced
+    q = ctypes.c_void_p(0x2000)
+    null = ctypes.c_void_p(0)
+    # causal softmax variants: heads must divide attn_batches when a per-head operand is given
+    assert lib.nhp_causal_softmax_ex_fwd(q, p, 1.0, 6, 8, -1, p, null, null, 4, BF16, None) == -2
+    assert lib.nhp_causal_softmax_ex_fwd(q, p, 1.0, 6, 8, -1, null, p, null, 0, BF16, None) == -2
+    assert lib.nhp_causal_softmax_ex_fwd(q, p, 1.0, 6, 8, -1, null, null, p, 5, BF16, None) == -2
+    assert lib.nhp_causal_softmax_ex_fwd(q, p, 1.0, 6, 8, -1, null, q, null, 3, BF16, None) == -6   # bias over the output
+    assert lib.nhp_causal_softmax_ex_bwd(q, p, p, 1.0, 6, 8, -1, p, 4, BF16, None) == -2
+    assert lib.nhp_causal_softmax_ex_fwd(null, null, 1.0, 0, 8, 3, null, null, null, 1, F16, None) == 0
+    # bias + GeLU, bias + residual
+    assert lib.nhp_bias_gelu_fwd(q, p, p, 4, 8, 9, None) == -1
+    assert lib.nhp_bias_gelu_fwd(q, p, p, -1, 8, BF16, None) == -2
+    assert lib.nhp_bias_gelu_fwd(null, null, null, 0, 8, BF16, None) == 0
+    assert lib.nhp_bias_gelu_fwd(null, p, p, 4, 8, BF16, None) == -3
+    assert lib.nhp_bias_gelu_bwd(q, p, null, p, null, null, 4, 8, F32, None) == -3
+    assert lib.nhp_bias_gelu_bwd(q, p, p, p, q, p, 4, 8, BF16, None) == -6        # dbias over dx
+    assert lib.nhp_bias_gelu_bwd(q, p, p, p, ctypes.c_void_p(0x3000), null, 4, 8, BF16, None) == -3  # workspace missing
+    assert lib.nhp_bias_gelu_bwd_workspace_bytes(4, 8, BF16) > 0
+    assert lib.nhp_bias_gelu_bwd_workspace_bytes(4, 7, BF16) == 0                 # scalar path needs none
+    assert lib.nhp_bias_gelu_bwd_workspace_bytes(0, 8, BF16) == 0
+    big = lib.nhp_bias_gelu_bwd_workspace_bytes(1 << 20, 8192, BF16)
+    assert 0 < big <= 512 * 8192 * 4                                               # bounded, whatever the row count
+    assert lib.nhp_bias_add_residual(q, null, p, p, 4, 8, F16, None) == -3
+    assert lib.nhp_bias_add_residual(q, p, null, null, 4, 8, 3, None) == -1
+    # norms: parameter dtype is the data dtype or fp32
+    assert lib.nhp_layernorm_fwd(q, null, null, p, p, p, 1e-5, 4, 8, BF16, F16, None) == -1
+    assert lib.nhp_layernorm_fwd(q, null, null, p, p, p, 1e-5, 4, 8, 4, F32, None) == -1
+    assert lib.nhp_layernorm_fwd(q, null, null, p, p, p, 1e-5, -4, 8, BF16, F32, None) == -2
+    assert lib.nhp_layernorm_fwd(q, null, null, null, p, p, 1e-5, 4, 8, BF16, F32, None) == -3
+    assert lib.nhp_layernorm_fwd(null, null, null, null, null, null, 1e-5, 4, 0, BF16, BF16, None) == 0
+    assert lib.nhp_layernorm_bwd(q, null, null, p, p, null, p, p, null, 4, 8, BF16, BF16, None) == -3   # mean missing
+    assert lib.nhp_layernorm_bwd(q, p, null, p, p, p, p, p, null, 4, 8, BF16, BF16, None) == -3          # workspace missing
+    assert lib.nhp_rmsnorm_fwd(q, null, p, p, null, 1e-5, 2, 4, 8, BF16, BF16, None) == -2               # eps_mode
+    assert lib.nhp_rmsnorm_bwd(q, null, null, p, p, null, p, null, 1e-5, 1, 4, 8, BF16, BF16, None) == -3  # inv missing
+    assert lib.nhp_rmsnorm_bwd(q, null, null, p, p, p, p, null, 1e-5, 3, 4, 8, BF16, BF16, None) == -2
+    assert lib.nhp_norm_bwd_workspace_bytes(4, 8, BF16) > 0
+    assert lib.nhp_norm_bwd_workspace_bytes(4, 7, BF16) == 0
+    assert lib.nhp_norm_bwd_workspace_bytes(4, 8, 11) == 0
+    assert 0 < lib.nhp_norm_bwd_workspace_bytes(1 << 22, 2048, BF16) <= 2 * 4096 * 2048 * 4
+
+
 def test_missing_library_fails_loudly(hotpath, monkeypatch, tmp_path):
     """No fallback: without the built library the binding raises ImportError."""
     monkeypatch.setattr(hotpath, "_lib", None)

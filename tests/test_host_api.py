@@ -209,3 +209,46 @@ def test_load_fused_kernels_exits_when_not_installed(hotpath, monkeypatch, tmp_p
     with pytest.raises(SystemExit):
         fk.load_fused_kernels()
     assert "Fused kernels configured but not properly installed" in capsys.readouterr().out
+
+
+# ---------------------------------------------------------------------------
+# element-wise and normalisation modules: names, parameters, errors (no GPU needed)
+# ---------------------------------------------------------------------------
+def test_layer_modules_surface_and_errors():
+    import types
+
+    from megatron.model import activations, fused_bias_dropout, norms
+
+    for name in ("bias_gelu", "bias_gelu_back", "GeLUFunction", "bias_gelu_impl"):
+        assert hasattr(activations, name)
+    for name in ("bias_dropout_add", "get_bias_dropout_add", "bias_dropout_add_fused_train",
+                 "bias_dropout_add_fused_inference"):
+        assert hasattr(fused_bias_dropout, name)
+    # the kernels are the only implementation: CPU tensors are refused, not silently computed elsewhere
+    with pytest.raises(RuntimeError, match="GPU"):
+        activations.bias_gelu(torch.zeros(8), torch.zeros(2, 8))
+    with pytest.raises(RuntimeError, match="GPU"):
+        fused_bias_dropout.bias_dropout_add_fused_inference(torch.zeros(2, 8), torch.zeros(8), torch.zeros(2, 8), 0.0)
+    with pytest.raises(NotImplementedError):
+        fused_bias_dropout.bias_dropout_add(torch.zeros(2, 8), torch.zeros(8), None, 0.1, True)
+    ln = norms.LayerNorm(16, eps=1e-5)
+    assert sorted(n for n, _ in ln.named_parameters()) == ["bias", "weight"]
+    assert ln.weight.shape == (16,) and float(ln.weight.sum()) == 16 and float(ln.bias.abs().sum()) == 0
+    assert norms.LayerNorm((16,), elementwise_affine=False).weight is None
+    with pytest.raises(NotImplementedError):
+        norms.LayerNorm((4, 16))
+    with pytest.raises(RuntimeError, match="GPU"):
+        ln(torch.zeros(2, 16))
+    rms = norms.RMSNorm(16, eps=1e-8)
+    assert [n for n, _ in rms.named_parameters()] == ["scale"] and rms.offset is None
+    assert sorted(n for n, _ in norms.RMSNorm(16, bias=True).named_parameters()) == ["offset", "scale"]
+    with pytest.raises(NotImplementedError):
+        norms.RMSNorm(16, p=0.25)
+    args = types.SimpleNamespace(norm="rmsnorm", rms_norm_epsilon=1e-6, rmsnorm_fusion=True, layernorm_epsilon=1e-5)
+    cls, eps = norms.get_norm(args)
+    assert issubclass(cls, norms.RMSNorm) and cls(8, eps=eps).fused_eps and eps == 1e-6
+    args.rmsnorm_fusion = False
+    assert norms.get_norm(args)[0] is norms.RMSNorm
+    args.norm = "scalenorm"
+    with pytest.raises(ValueError):
+        norms.get_norm(args)
