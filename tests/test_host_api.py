@@ -233,7 +233,7 @@ def test_layer_modules_surface_and_errors():
         fused_bias_dropout.bias_dropout_add(torch.zeros(2, 8), torch.zeros(8), None, 0.1, True)
     ln = norms.LayerNorm(16, eps=1e-5)
     assert sorted(n for n, _ in ln.named_parameters()) == ["bias", "weight"]
-    assert ln.weight.shape == (16,) and float(ln.weight.sum()) == 16 and float(ln.bias.abs().sum()) == 0
+    assert ln.weight.shape == (16,) and float(ln.weight.detach().sum()) == 16 and float(ln.bias.detach().abs().sum()) == 0
     assert norms.LayerNorm((16,), elementwise_affine=False).weight is None
     with pytest.raises(NotImplementedError):
         norms.LayerNorm((4, 16))
