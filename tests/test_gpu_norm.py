@@ -274,3 +274,60 @@ def test_layernorm_full_size(hotpath):
     assert (dg - gr.grad).abs().max().item() <= 1e-3 * gr.grad.abs().max().item()
     assert (db - br.grad).abs().max().item() <= 1e-3 * br.grad.abs().max().item()
     assert (dx.float() - xr.grad).norm().item() <= 2.0**-8 * xr.grad.norm().item()
+
+
+def test_layer_kernels_in_a_hip_graph_and_on_a_side_stream(hotpath):
+    """LayerNorm forward + backward and bias+GeLU backward (each backward is two kernels that hand
+    partial sums over through the caller's workspace) captured in one HIP graph: every replay, with
+    eager work and synchronisation in between, gives the eager result bit for bit. The same calls
+    on a non-default stream give the same bits as well."""
+    L = hotpath.lib()
+    rows, cols, BF16 = 777, 2048, hotpath.BF16
+    x = torch.empty((rows, cols), dtype=torch.bfloat16, device=DEV)
+    dy = util.randn((rows, cols), torch.bfloat16, seed=2).to(DEV)
+    gamma = (1 + 0.3 * util.randn((cols,), torch.float32, seed=3)).bfloat16().to(DEV)
+    beta = util.randn((cols,), torch.bfloat16, seed=4).to(DEV)
+
+    def buffers():
+        return dict(y=torch.empty_like(x), mean=torch.empty(rows, device=DEV), rstd=torch.empty(rows, device=DEV),
+                    dx=torch.empty_like(x), dg=torch.empty_like(gamma), db=torch.empty_like(beta),
+                    gx=torch.empty_like(x), gb=torch.empty_like(beta),
+                    ws1=torch.empty(max(L.nhp_norm_bwd_workspace_bytes(rows, cols, BF16), 16), dtype=torch.uint8, device=DEV),
+                    ws2=torch.empty(max(L.nhp_bias_gelu_bwd_workspace_bytes(rows, cols, BF16), 16), dtype=torch.uint8, device=DEV))
+
+    def enqueue(b, st):
+        assert L.nhp_layernorm_fwd(b["y"].data_ptr(), b["mean"].data_ptr(), b["rstd"].data_ptr(), x.data_ptr(), gamma.data_ptr(),
+                                   beta.data_ptr(), 1e-5, rows, cols, BF16, BF16, st) == 0
+        assert L.nhp_layernorm_bwd(b["dx"].data_ptr(), b["dg"].data_ptr(), b["db"].data_ptr(), dy.data_ptr(), x.data_ptr(),
+                                   b["mean"].data_ptr(), b["rstd"].data_ptr(), gamma.data_ptr(), b["ws1"].data_ptr(), rows, cols,
+                                   BF16, BF16, st) == 0
+        assert L.nhp_bias_gelu_bwd(b["gx"].data_ptr(), dy.data_ptr(), x.data_ptr(), beta.data_ptr(), b["gb"].data_ptr(),
+                                   b["ws2"].data_ptr(), rows, cols, BF16, st) == 0
+
+    keys = ("y", "mean", "rstd", "dx", "dg", "db", "gx", "gb")
+    captured, eager, aside = buffers(), buffers(), buffers()
+    side = torch.cuda.Stream()
+    x.copy_(util.randn((rows, cols), torch.bfloat16, seed=1, std=2.0).to(DEV))
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm-up on a side stream, as capture needs
+        enqueue(aside, side.cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        enqueue(captured, torch.cuda.current_stream().cuda_stream)
+    for rep in range(3):
+        x.copy_(util.randn((rows, cols), torch.bfloat16, seed=10 + rep, std=2.0).to(DEV))
+        for k in keys:
+            captured[k].fill_(7)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        enqueue(eager, None)
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            enqueue(aside, side.cuda_stream)
+        torch.cuda.synchronize()
+        for k in keys:
+            assert torch.equal(util.raw_bits(captured[k]), util.raw_bits(eager[k])), (rep, k)
+            assert torch.equal(util.raw_bits(aside[k]), util.raw_bits(eager[k])), (rep, k)
