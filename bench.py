@@ -22,6 +22,7 @@ the drop-in extension modules (which call libneox_hotpath.so):
   rpe-bias-1.4b  causal softmax fwd+bwd [128,2048,2048] bf16 with a bias tensor [16,2048,2048] added in the kernel
 
   mlp-gelu-1.4b  bias + tanh-GeLU fwd and bwd (with the bias gradient) on the MLP activation [2048*8, 8192] bf16
+  swiglu-7b      SwiGLU forward and backward on the Llama-2 7B MLP activation [4096*4, 2*11008] -> [4096*4, 11008] bf16
   bias-residual-1.4b  residual + (x + bias) on the hidden state [2048*8, 2048] bf16
   layernorm-1.4b  LayerNorm fwd and bwd (with the parameter gradients) on the hidden state [2048*8, 2048] bf16
   rmsnorm-7b     RMSNorm fwd and bwd on [4096*4, 4096] bf16 (the Llama-2 7B hidden size)
@@ -272,6 +273,31 @@ def make_workload(name, torch, dev):
         cfg = {"workload": name, "activation": [rows, cols], "bias_gradient": "fused column sums",
                "bytes_convention": "every tensor element read or written once"}
         return step, kernel_bytes, {}, "bias_gelu_bwd", "bf16", cfg
+
+    if name == "swiglu-7b":
+        from megatron.fused_kernels import _hotpath as hp
+
+        lib = hp.lib()
+        rows, f = 4096 * 4, 11008
+        inp = torch.empty((rows, 2 * f), dtype=torch.bfloat16, device=dev)   # 688 MiB: larger than the last-level cache
+        for r in range(0, rows, 2048):
+            inp[r:r + 2048] = randn((2048, 2 * f), r, torch.bfloat16, 2.0)
+        dy = randn((rows, f), 3, torch.bfloat16)
+        out = torch.empty((rows, f), dtype=torch.bfloat16, device=dev)
+        din = torch.empty_like(inp)
+        n = rows * f
+        kernel_bytes = {"swiglu_fwd": 3 * n * 2, "swiglu_bwd": 5 * n * 2}
+        stream = hp.stream_of(out)
+
+        def step(t):
+            t.run("swiglu_fwd", lambda: hp.check(lib.nhp_gated_act_fwd(out.data_ptr(), inp.data_ptr(), None, rows, f, 0,
+                                                                       hp.BF16, stream), "swiglu forward"))
+            t.run("swiglu_bwd", lambda: hp.check(lib.nhp_gated_act_bwd(din.data_ptr(), dy.data_ptr(), inp.data_ptr(), None,
+                                                                       rows, f, 0, hp.BF16, stream), "swiglu backward"))
+
+        cfg = {"workload": name, "input": [rows, 2 * f], "output": [rows, f],
+               "bytes_convention": "every tensor element read or written once"}
+        return step, kernel_bytes, {}, "swiglu_bwd", "bf16", cfg
 
     if name in ("layernorm-1.4b", "rmsnorm-7b"):
         # through the C ABI with preallocated outputs: these kernels run for a few tens of

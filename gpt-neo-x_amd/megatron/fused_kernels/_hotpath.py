@@ -55,6 +55,8 @@ def _declare(lib):
         "nhp_bias_gelu_bwd": ([vp, vp, vp, vp, vp, vp, i64, i64, ci, vp], ci),
         "nhp_bias_gelu_bwd_workspace_bytes": ([i64, i64, ci], i64),
         "nhp_bias_add_residual": ([vp, vp, vp, vp, i64, i64, ci, vp], ci),
+        "nhp_gated_act_fwd": ([vp, vp, vp, i64, i64, ci, ci, vp], ci),
+        "nhp_gated_act_bwd": ([vp, vp, vp, vp, i64, i64, ci, ci, vp], ci),
         "nhp_layernorm_fwd": ([vp, vp, vp, vp, vp, vp, f32, i64, i64, ci, ci, vp], ci),
         "nhp_layernorm_bwd": ([vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, ci, ci, vp], ci),
         "nhp_rmsnorm_fwd": ([vp, vp, vp, vp, vp, f32, ci, i64, i64, ci, ci, vp], ci),

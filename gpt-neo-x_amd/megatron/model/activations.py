@@ -1,10 +1,14 @@
-"""bias + GeLU (tanh form) on MI355X.
+"""bias + GeLU (tanh form) and the gated MLP activations on MI355X.
 
 The fused part of GPT-NeoX's ``megatron/model/activations.py``: ``bias_gelu``
 (:79-82), ``bias_gelu_back`` (:88-97), ``GeLUFunction`` (:100-112) and
 ``bias_gelu_impl`` (:115), with the same arguments. The reference compiles the
 two expressions with TorchScript; here each is one hand-written gfx950 kernel
 (libneox_hotpath.so), evaluated in fp32 with one rounding to the storage dtype.
+
+``Gated_Activation`` (the class of megatron/model/transformer.py:186-206) with the
+activations ``get_activation`` (:30-66) pairs with a gate -- geglu, reglu,
+bilinear, swiglu, glu -- is one kernel forward and one backward.
 
 One difference, to the caller's advantage: ``GeLUFunction.backward`` returns
 the bias gradient already reduced to the bias shape (the column sums are formed
@@ -97,3 +101,97 @@ class GeLUFunction(torch.autograd.Function):
 
 
 bias_gelu_impl = GeLUFunction.apply
+
+
+# ---------------------------------------------------------------------------
+# gated activations
+# ---------------------------------------------------------------------------
+def swish(x, beta: float = 1.0):
+    """``x * sigmoid(beta * x)`` (megatron/model/activations.py:128-130); as a gate only beta = 1 is fused."""
+    return x * torch.sigmoid(beta * x)
+
+
+def _identity(x):
+    return x
+
+
+# what get_activation hands to Gated_Activation for each gated `activation` setting
+_GATES = {"swiglu": swish, "geglu": torch.nn.functional.gelu, "reglu": torch.nn.functional.relu,
+          "glu": torch.nn.functional.sigmoid, "bilinear": _identity}
+_GATE_CODE = {swish: 0, torch.nn.functional.gelu: 1, torch.nn.functional.relu: 2, torch.nn.functional.sigmoid: 3,
+              torch.sigmoid: 3, _identity: 4}
+
+
+def get_activation(neox_args):
+    """(activation function, is_gated) for the settings served by the kernels here: the gated ones and
+    ``gelu`` with ``bias_gelu_fusion``; other settings are left to the reference's function."""
+    name = neox_args.activation
+    if name in _GATES:
+        return _GATES[name], True
+    if name == "gelu" and getattr(neox_args, "bias_gelu_fusion", False) and not getattr(neox_args, "onnx_safe", False):
+        return bias_gelu_impl, False
+    raise ValueError(f"Activation function {name} is not provided by the MI355X kernels")
+
+
+class _GatedActivationFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, inp, bias, code):
+        what = "Gated_Activation"
+        _hp.require_gpu(inp, what)
+        if inp.size(-1) % 2:
+            raise RuntimeError(f"{what}: the last dimension must be even")
+        features = inp.size(-1) // 2
+        src = inp.contiguous()
+        b = None
+        if bias is not None:
+            if bias.numel() != 2 * features or bias.dtype != inp.dtype:
+                raise RuntimeError(f"{what}: bias must hold 2 * features values in the dtype of the input")
+            _hp.require_gpu(bias, what)
+            b = bias.contiguous().view(-1)
+        out = torch.empty(src.shape[:-1] + (features,), dtype=src.dtype, device=src.device)
+        rows = src.numel() // max(2 * features, 1)
+        with _hp.device_guard(src):
+            rc = _hp.lib().nhp_gated_act_fwd(out.data_ptr(), src.data_ptr(), None if b is None else b.data_ptr(), rows,
+                                             features, code, _hp.dtype_code(src, what), _hp.stream_of(src))
+        _hp.check(rc, what)
+        ctx.save_for_backward(src, b)
+        ctx.code = code
+        ctx.bias_shape = None if bias is None else bias.shape
+        return out
+
+    @staticmethod
+    def backward(ctx, grad):
+        what = "Gated_Activation backward"
+        src, b = ctx.saved_tensors
+        g = grad.contiguous()
+        features = src.size(-1) // 2
+        rows = src.numel() // max(2 * features, 1)
+        din = torch.empty_like(src)
+        with _hp.device_guard(src):
+            rc = _hp.lib().nhp_gated_act_bwd(din.data_ptr(), g.data_ptr(), src.data_ptr(), None if b is None else b.data_ptr(),
+                                             rows, features, ctx.code, _hp.dtype_code(src, what), _hp.stream_of(src))
+        _hp.check(rc, what)
+        dbias = None
+        if b is not None and ctx.needs_input_grad[1]:
+            dbias = din.reshape(-1, 2 * features).sum(dim=0).view(ctx.bias_shape)
+        return din, dbias, None
+
+
+class Gated_Activation(torch.nn.Module):
+    """``x, gate = x.chunk(2, dim=-1); activation_func(gate + bias_2) * (x + bias_1)``
+    (megatron/model/transformer.py:186-206). ``activation_func`` is one of the functions ``get_activation``
+    returns for a gated setting (or its name); ``use_swiglu`` is accepted and changes nothing, the fused
+    SwiGLU it selects in the reference computes the same expression."""
+
+    def __init__(self, activation_func, use_swiglu=False):
+        super().__init__()
+        if isinstance(activation_func, str):
+            activation_func = _GATES[activation_func]
+        if activation_func not in _GATE_CODE:
+            raise ValueError("Gated_Activation: activation function not provided by the MI355X kernels")
+        self.activation_func = activation_func
+        self.use_swiglu = use_swiglu
+        self._code = _GATE_CODE[activation_func]
+
+    def forward(self, x, bias=None):
+        return _GatedActivationFunction.apply(x, bias, self._code)

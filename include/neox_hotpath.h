@@ -324,6 +324,35 @@ int64_t nhp_bias_gelu_bwd_workspace_bytes(int64_t rows, int64_t cols, int dtype)
 int nhp_bias_add_residual(void* out, const void* x, const void* bias, const void* residual,
                           int64_t rows, int64_t cols, int dtype, void* stream);
 
+/*
+ * Gated MLP activations. in: [rows, 2 * features]; the first `features` values
+ * of a row are x, the last `features` the gates g (x, gate = in.chunk(2, dim=-1));
+ * bias: [2 * features] or NULL, each half added to its half of the row.
+ *   forward:  out[rows, features] = act(g) * x
+ *   backward: din[rows, 2 * features] = (dy * act(g), dy * x * act'(g))
+ * act (enum nhp_gate_act): swish g * sigmoid(g) (SwiGLU), exact erf GeLU
+ * (GeGLU), relu (ReGLU), sigmoid (GLU), identity (bilinear). `out` / `din`
+ * must not alias `in`.
+ *
+ * Replaces Gated_Activation.forward
+ *   megatron/model/transformer.py:186-206 with the activations get_activation selects
+ *   for geglu / reglu / bilinear / swiglu / glu, megatron/model/activations.py:30-49,
+ *   swish :128-130 (the reference differentiates it with autograd).
+ */
+enum nhp_gate_act {
+    NHP_GATE_SWISH = 0,
+    NHP_GATE_GELU = 1,
+    NHP_GATE_RELU = 2,
+    NHP_GATE_SIGMOID = 3,
+    NHP_GATE_IDENTITY = 4
+};
+
+int nhp_gated_act_fwd(void* out, const void* in, const void* bias,
+                      int64_t rows, int64_t features, int act, int dtype, void* stream);
+
+int nhp_gated_act_bwd(void* din, const void* dy, const void* in, const void* bias,
+                      int64_t rows, int64_t features, int act, int dtype, void* stream);
+
 /* ------------------------------------------------------------------------
  * LayerNorm and RMSNorm
  *

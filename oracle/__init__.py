@@ -54,6 +54,8 @@ def lib():
         L.oracle_bias_gelu_bwd.argtypes = [vp, vp, vp, vp, i64, i64, ci]
         L.oracle_column_sum.argtypes = [vp, vp, i64, i64, ci]
         L.oracle_bias_add_residual.argtypes = [vp, vp, vp, vp, i64, i64, ci]
+        L.oracle_gated_act_fwd.argtypes = [vp, vp, vp, i64, i64, ci, ci]
+        L.oracle_gated_act_bwd.argtypes = [vp, vp, vp, vp, i64, i64, ci, ci]
         L.oracle_layernorm_fwd.argtypes = [vp, vp, vp, vp, vp, vp, f32, i64, i64, ci, ci]
         L.oracle_layernorm_bwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, ci, ci]
         L.oracle_rmsnorm_fwd.argtypes = [vp, vp, vp, vp, vp, f32, ci, i64, i64, ci, ci]
@@ -330,3 +332,36 @@ def rmsnorm_bwd(dy, x, inv, scale=None, eps=1e-8, eps_mode=1, param_dtype=None):
                                     inv.data_ptr(), sp, float(eps), int(eps_mode), rows, cols, _DT[x.dtype],
                                     _DT[pdt]), "rmsnorm_bwd")
     return dx, ds, do
+
+
+# ---------------------------------------------------------------------------
+# gated activations (layer_semantics.c)
+# ---------------------------------------------------------------------------
+GATE_ACTS = {"swiglu": 0, "geglu": 1, "reglu": 2, "glu": 3, "bilinear": 4}
+
+
+def gated_act_fwd(inp, act, bias=None):
+    """act(gate) * x with x, gate = inp.chunk(2, -1) (+ the halves of bias); act: a key of GATE_ACTS."""
+    inp = _cpu_contig(inp)
+    assert inp.size(-1) % 2 == 0
+    f = inp.size(-1) // 2
+    rows = inp.numel() // max(2 * f, 1)
+    out = torch.empty(inp.shape[:-1] + (f,), dtype=inp.dtype)
+    bias, bp = _opt_ptr(bias, inp, "bias dtype")
+    _check(lib().oracle_gated_act_fwd(out.data_ptr(), inp.data_ptr(), bp, rows, f, GATE_ACTS[act], _DT[inp.dtype]),
+           "gated_act_fwd")
+    return out
+
+
+def gated_act_bwd(dy, inp, act, bias=None):
+    """Gradient with respect to inp (the bias gradient is its column sum)."""
+    inp = _cpu_contig(inp)
+    dy = _cpu_contig(dy)
+    f = inp.size(-1) // 2
+    rows = inp.numel() // max(2 * f, 1)
+    assert dy.shape == inp.shape[:-1] + (f,) and dy.dtype == inp.dtype
+    din = torch.empty_like(inp)
+    bias, bp = _opt_ptr(bias, inp, "bias dtype")
+    _check(lib().oracle_gated_act_bwd(din.data_ptr(), dy.data_ptr(), inp.data_ptr(), bp, rows, f, GATE_ACTS[act],
+                                      _DT[inp.dtype]), "gated_act_bwd")
+    return din

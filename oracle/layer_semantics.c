@@ -313,3 +313,90 @@ int oracle_rmsnorm_bwd(void* dx, void* dscale, void* doffset, const void* dy, co
     free(col);
     return 0;
 }
+
+/* ------------------------------------------------------------------------ */
+/* gated MLP activations                                                      */
+/* ------------------------------------------------------------------------ */
+
+enum { GATE_SWISH = 0, GATE_GELU = 1, GATE_RELU = 2, GATE_SIGMOID = 3, GATE_IDENTITY = 4 };
+
+static float sigmoid_f(float v) { return 1.0f / (1.0f + expf(-v)); }
+
+/* act(g) for the activation functions get_activation pairs with a gate
+ * (megatron/model/activations.py:30-49): swish = x * sigmoid(x) (:128-130),
+ * F.gelu (erf form), F.relu, F.sigmoid, identity; and its derivative. */
+static void gate_eval(int act, float g, float* a, float* da)
+{
+    switch (act) {
+    case GATE_SWISH: {
+        const float s = sigmoid_f(g);
+        *a = g * s;
+        *da = s * (1.0f + g * (1.0f - s));
+        break;
+    }
+    case GATE_GELU: {
+        const float cdf = 0.5f * (1.0f + erff(g * 0.70710678118654752f));
+        const float pdf = 0.3989422804014327f * expf(-0.5f * g * g);
+        *a = g * cdf;
+        *da = cdf + g * pdf;
+        break;
+    }
+    case GATE_RELU:
+        *a = g > 0.0f ? g : 0.0f;
+        *da = g > 0.0f ? 1.0f : 0.0f;
+        break;
+    case GATE_SIGMOID: {
+        const float s = sigmoid_f(g);
+        *a = s;
+        *da = s * (1.0f - s);
+        break;
+    }
+    default:
+        *a = g;
+        *da = 1.0f;
+    }
+}
+
+/*
+ * Gated_Activation.forward (megatron/model/transformer.py:192-206):
+ *   x, gate = in.chunk(2, dim=-1); with a bias, x += bias_1, gate += bias_2;
+ *   out = activation_func(gate) * x
+ * in: [rows, 2f], bias: [2f] or NULL, out: [rows, f].
+ */
+int oracle_gated_act_fwd(void* out, const void* in, const void* bias, int64_t rows, int64_t f, int act, int dt)
+{
+    for (int64_t r = 0; r < rows; ++r)
+        for (int64_t c = 0; c < f; ++c) {
+            float x = load_elem(in, r * 2 * f + c, dt);
+            float g = load_elem(in, r * 2 * f + f + c, dt);
+            if (bias) {
+                x = x + load_elem(bias, c, dt);
+                g = g + load_elem(bias, f + c, dt);
+            }
+            float a, da;
+            gate_eval(act, g, &a, &da);
+            store_elem(out, r * f + c, dt, a * x);
+        }
+    return 0;
+}
+
+/* Its adjoint (the reference leaves it to autograd): din = (dy * act(g), dy * x * act'(g)). */
+int oracle_gated_act_bwd(void* din, const void* dy, const void* in, const void* bias, int64_t rows, int64_t f,
+                         int act, int dt)
+{
+    for (int64_t r = 0; r < rows; ++r)
+        for (int64_t c = 0; c < f; ++c) {
+            float x = load_elem(in, r * 2 * f + c, dt);
+            float g = load_elem(in, r * 2 * f + f + c, dt);
+            if (bias) {
+                x = x + load_elem(bias, c, dt);
+                g = g + load_elem(bias, f + c, dt);
+            }
+            float a, da;
+            gate_eval(act, g, &a, &da);
+            const float d = load_elem(dy, r * f + c, dt);
+            store_elem(din, r * 2 * f + c, dt, d * a);
+            store_elem(din, r * 2 * f + f + c, dt, (d * x) * da);
+        }
+    return 0;
+}

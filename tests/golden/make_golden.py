@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Writes tests/golden/hotpath_golden.npz (softmax and rotary entry points) and
 tests/golden/layer_golden.npz (the window / AliBi / bias / key-length variants of
-the causal softmax, bias + GeLU, bias + residual add, LayerNorm, RMSNorm): small
+the causal softmax, bias + GeLU, bias + residual add, gated activations, LayerNorm, RMSNorm): small
 seeded inputs and the outputs of the CPU oracle (oracle/*.c), stored as raw bit
 patterns. The oracle itself is pinned by tests/test_oracle_*.py; these
 vectors freeze its answers so that the GPU path (and any later change to the
@@ -113,6 +113,15 @@ def main():
             rdx, rds, rdo = oracle.rmsnorm_bwd(dy, x, inv, gamma, eps, mode)
             put(name, **{f"rms{mode}_y": ry, f"rms{mode}_inv": inv, f"rms{mode}_dx": rdx, f"rms{mode}_dscale": rds,
                          f"rms{mode}_doffset": rdo, f"rms{mode}_eps": np.float32(eps)})
+
+    for name, dtype, seed in (("gated_bf16", torch.bfloat16, 41), ("gated_fp16", torch.float16, 42),
+                              ("gated_fp32", torch.float32, 43)):
+        inp = util.randn((5, 32), dtype, seed, std=2.5)
+        bias = util.randn((32,), dtype, seed + 1, std=0.5)
+        dy = util.randn((5, 16), dtype, seed + 2)
+        put(name, inp=inp, bias=bias, dy=dy)
+        for act in sorted(oracle.GATE_ACTS):
+            put(name, **{f"{act}_out": oracle.gated_act_fwd(inp, act, bias), f"{act}_din": oracle.gated_act_bwd(dy, inp, act, bias)})
 
     path = os.path.join(HERE, "layer_golden.npz")
     np.savez_compressed(path, **out)

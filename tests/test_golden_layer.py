@@ -71,8 +71,35 @@ def test_oracle_reproduces_norm_golden(name):
         assert same(rdo, get(name, f"rms{mode}_doffset"))
 
 
+GATED = ["gated_bf16", "gated_fp16", "gated_fp32"]
+
+
+@pytest.mark.parametrize("name", GATED)
+def test_oracle_reproduces_gated_golden(name):
+    inp, bias, dy = (get(name, k) for k in ("inp", "bias", "dy"))
+    for act in sorted(oracle.GATE_ACTS):
+        assert same(oracle.gated_act_fwd(inp, act, bias), get(name, f"{act}_out")), act
+        assert same(oracle.gated_act_bwd(dy, inp, act, bias), get(name, f"{act}_din")), act
+
+
 def ptr(t):
     return None if t is None else t.data_ptr()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", GATED)
+def test_gpu_matches_gated_golden(hotpath, name):
+    inp, bias, dy = (get(name, k) for k in ("inp", "bias", "dy"))
+    L, code = hotpath.lib(), hotpath.dtype_code(inp, "t")
+    di, db, dd = inp.cuda(), bias.cuda(), dy.cuda()
+    rows, f = dy.shape
+    for act, num in sorted(oracle.GATE_ACTS.items()):
+        out, din = torch.empty_like(dd), torch.empty_like(di)
+        assert L.nhp_gated_act_fwd(out.data_ptr(), di.data_ptr(), db.data_ptr(), rows, f, num, code, None) == 0
+        assert L.nhp_gated_act_bwd(din.data_ptr(), dd.data_ptr(), di.data_ptr(), db.data_ptr(), rows, f, num, code, None) == 0
+        want, want_d = get(name, f"{act}_out"), get(name, f"{act}_din")
+        util.assert_close_ulp_or_noise(out.cpu(), want, 2, util.gated_noise(inp, bias, act, want), f"{name} {act}")
+        util.assert_close_ulp_or_noise(din.cpu(), want_d, 2, util.gated_noise(inp, bias, act, want_d, dy), f"{name} {act}")
 
 
 @pytest.mark.gpu

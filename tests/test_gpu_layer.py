@@ -211,3 +211,75 @@ def test_bias_dropout_add_functions():
                        util.raw_bits(want))
     with pytest.raises(NotImplementedError):
         bias_dropout_add_fused_train(x.to(DEV), bias.to(DEV), res.to(DEV), 0.1)
+
+
+# ---------------------------------------------------------------------------
+# gated activations
+# ---------------------------------------------------------------------------
+GATES = ["swiglu", "geglu", "reglu", "glu", "bilinear"]
+
+
+def abi_gated(hp, inp, dy, bias, act):
+    rows, f2 = inp.shape
+    f = f2 // 2
+    code = hp.dtype_code(inp, "t")
+    out = torch.empty((rows, f), dtype=inp.dtype, device=inp.device)
+    din = torch.empty_like(inp)
+    L = hp.lib()
+    rc = L.nhp_gated_act_fwd(out.data_ptr(), inp.data_ptr(), ptr(bias), rows, f, oracle.GATE_ACTS[act], code, None)
+    assert rc == 0, L.nhp_status_string(rc)
+    rc = L.nhp_gated_act_bwd(din.data_ptr(), dy.data_ptr(), inp.data_ptr(), ptr(bias), rows, f, oracle.GATE_ACTS[act], code, None)
+    assert rc == 0, L.nhp_status_string(rc)
+    return out, din
+
+
+@pytest.mark.parametrize("act", GATES)
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("shape", [(1, 8), (37, 96), (5, 1000), (300, 2048), (19, 5504), (1000, 24), (2, 5)],
+                         ids=lambda s: f"{s[0]}x{s[1]}")
+def test_gated_activation_vs_oracle(hotpath, shape, dtype, act):
+    rows, f = shape
+    print(f"gated case {shape} {dtype} {act}", flush=True)
+    inp = util.randn((rows, 2 * f), dtype, seed=rows + f, std=2.5)
+    dy = util.randn((rows, f), dtype, seed=rows)
+    bias = util.randn((2 * f,), dtype, seed=f, std=0.5)
+    for b in (None, bias):
+        out, din = abi_gated(hotpath, inp.to(DEV), dy.to(DEV), None if b is None else b.to(DEV), act)
+        want = oracle.gated_act_fwd(inp, act, b)
+        util.assert_close_ulp_or_noise(out.cpu(), want, 2, util.gated_noise(inp, b, act, want), "fwd")
+        want_d = oracle.gated_act_bwd(dy, inp, act, b)
+        util.assert_close_ulp_or_noise(din.cpu(), want_d, 2, util.gated_noise(inp, b, act, want_d, dy), "bwd")
+
+
+@pytest.mark.parametrize("act", ["swiglu", "geglu"])
+def test_gated_activation_module_autograd(act):
+    """Gated_Activation under autograd against the reference's expression in fp32 on the device."""
+    import types
+
+    from megatron.model.activations import Gated_Activation, get_activation
+
+    func, gated = get_activation(types.SimpleNamespace(activation=act))
+    assert gated
+    m = Gated_Activation(func, use_swiglu=(act == "swiglu"))
+    dtype, s, b, f = torch.bfloat16, 48, 2, 1376
+    x = util.randn((s, b, 2 * f), dtype, seed=1, std=2.0).to(DEV).requires_grad_(True)
+    bias = util.randn((2 * f,), dtype, seed=2, std=0.5).to(DEV).requires_grad_(True)
+    g = util.randn((s, b, f), dtype, seed=3).to(DEV)
+    out = m(x, bias)
+    out.backward(g)
+    xr = x.detach().float().requires_grad_(True)
+    br = bias.detach().float().requires_grad_(True)
+    xx, gate = xr.chunk(2, dim=-1)
+    b1, b2 = br.chunk(2, dim=-1)
+    ref = func(gate + b2) * (xx + b1)
+    ref.backward(g.float())
+    assert out.shape == (s, b, f) and x.grad.shape == x.shape and bias.grad.shape == bias.shape
+    lim = 2.0**-7
+    assert (out.float() - ref).norm() <= lim * ref.norm()
+    assert (x.grad.float() - xr.grad).norm() <= lim * xr.grad.norm()
+    assert (bias.grad.float() - br.grad).norm() <= 2 * lim * br.grad.norm()
+    plain = m(x.detach())
+    util.assert_close_ulp_or_noise(plain.cpu(), oracle.gated_act_fwd(x.detach().cpu(), act), 2,
+                                   util.gated_noise(x.detach().cpu(), None, act, plain.cpu()), "no bias")
+    with pytest.raises(ValueError):
+        Gated_Activation(torch.tanh)

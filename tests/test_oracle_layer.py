@@ -275,3 +275,62 @@ def test_rmsnorm_backward_is_the_adjoint(dtype, mode):
     _, zi = oracle.rmsnorm_fwd(z, None, None, 1e-3, mode)
     dz, _, _ = oracle.rmsnorm_bwd(g, z, zi, None, 1e-3, mode)
     assert torch.isfinite(dz).all() and torch.allclose(dz, g * zi[0])
+
+
+# ---------------------------------------------------------------------------
+# gated activations
+# ---------------------------------------------------------------------------
+def swish(x):
+    return x * torch.sigmoid(1.0 * x)  # megatron/model/activations.py:128-130 with beta = 1
+
+
+GATE_FUNCS = {"swiglu": swish, "geglu": F.gelu, "reglu": F.relu, "glu": torch.sigmoid, "bilinear": lambda x: x}
+
+
+def reference_gated(inp, bias, act):
+    """Gated_Activation.forward (megatron/model/transformer.py:192-206) with torch calls."""
+    x, gate = inp.chunk(2, dim=-1)
+    if bias is not None:
+        b1, b2 = bias.chunk(2, dim=-1)
+        x = x + b1
+        gate = gate + b2
+    return GATE_FUNCS[act](gate) * x
+
+
+@pytest.mark.parametrize("act", sorted(GATE_FUNCS))
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_gated_activation_forward(dtype, act):
+    inp = util.randn((9, 2 * 40), dtype, seed=3, std=2.5)
+    bias = util.randn((2 * 40,), dtype, seed=4, std=0.5)
+    for b in (None, bias):
+        out = oracle.gated_act_fwd(inp, act, b)
+        want64 = reference_gated(inp.double(), None if b is None else b.double(), act)
+        noise = util.gated_noise(inp, b, act, want64)
+        util.assert_close_ulp_or_noise(out, want64.to(dtype), 1, noise, f"{act} vs float64")
+        want32 = reference_gated(inp.float(), None if b is None else b.float(), act)
+        util.assert_close_ulp_or_noise(out, want32.to(dtype), 1, noise, f"{act} vs torch fp32")
+    # which half gates which: swapping the halves changes the result (except for the symmetric bilinear case)
+    swapped = torch.cat(inp.chunk(2, -1)[::-1], -1)
+    same = torch.equal(util.raw_bits(oracle.gated_act_fwd(swapped, act)), util.raw_bits(oracle.gated_act_fwd(inp, act)))
+    assert same == (act == "bilinear")
+    # known values: act(0) * x, and a closed form per activation at gate = 1, x = 2
+    one = torch.tensor([[2.0, 1.0]], dtype=torch.float32)
+    expect = {"swiglu": 2 / (1 + math.exp(-1.0)), "geglu": 2 * 0.5 * (1 + math.erf(2 ** -0.5)), "reglu": 2.0,
+              "glu": 2 / (1 + math.exp(-1.0)), "bilinear": 2.0}[act]
+    assert abs(oracle.gated_act_fwd(one, act).item() - expect) < 1e-6
+
+
+@pytest.mark.parametrize("act", sorted(GATE_FUNCS))
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_gated_activation_backward_is_the_adjoint(dtype, act):
+    inp = util.randn((7, 2 * 24), dtype, seed=5, std=2.0)
+    bias = util.randn((2 * 24,), dtype, seed=6, std=0.5)
+    dy = util.randn((7, 24), dtype, seed=7)
+    din = oracle.gated_act_bwd(dy, inp, act, bias)
+    x64 = inp.double().requires_grad_(True)
+    reference_gated(x64, bias.double(), act).backward(dy.double())
+    noise = util.gated_noise(inp, bias, act, x64.grad, dy)
+    util.assert_close_ulp_or_noise(din, x64.grad.to(dtype), 1, noise, f"{act} vs float64 autograd")
+    x32 = inp.float().requires_grad_(True)
+    reference_gated(x32, bias.float(), act).backward(dy.float())
+    util.assert_close_ulp_or_noise(din, x32.grad.to(dtype), 1, noise, f"{act} vs fp32 autograd")

@@ -114,6 +114,30 @@ def gelu_noise(x, g=None):
     return (1 + x**3) * g.float().abs() * 2.0**-21
 
 
+def gated_noise(inp, bias, act, want, dy=None):
+    """fp32 rounding noise of the expression: a few roundings of the result and, for the erf GeLU,
+    the cancellation in 1 + erf(g / sqrt 2) for negative gates (absolute 2^-24 on a factor that
+    multiplies g * x), as for the tanh form."""
+    x, g = inp.float().chunk(2, -1)
+    if bias is not None:
+        b1, b2 = bias.float().chunk(2, -1)
+        x, g = x + b1, g + b2
+    noise = want.abs().float() * 16 * EPS32 + 1e-30
+    if dy is not None:
+        # 1 - sigmoid(g) in the derivatives cancels for large g: absolute 2^-24 on a factor of dy * x * (1 + |g|)
+        d = dy.float().abs()
+        noise = noise + torch.cat([torch.zeros_like(d), d * x.abs() * (1 + g.abs())], -1) * 4 * EPS32
+    if act == "geglu":
+        tail = (x * g).abs() * 4 * EPS32
+        if dy is None:
+            noise = noise + tail
+        else:
+            d = dy.float().abs()
+            noise = noise + torch.cat([d * g.abs(), d * x.abs() * (1 + g * g)], -1) * 4 * EPS32
+    return noise
+
+
+
 # ---------------------------------------------------------------------------
 # direct C-ABI calls on torch GPU tensors
 # ---------------------------------------------------------------------------
