@@ -54,8 +54,9 @@ METRIC = "achieved HBM GB/s (% of MI355X peak), causal softmax+rotary fwd/bwd, 1
 HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch of the dominant kernel of the default workload measured
-# with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE; profiles/pythia-1.4b_step_hbm_traffic.txt).
-MEASURED_TRAFFIC_BYTES = {"pythia-1.4b": 2181026543}
+# with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE; profiles/pythia-1.4b_step_hbm_traffic.txt,
+# profiles/layer_neighbours_hbm_traffic.txt).
+MEASURED_TRAFFIC_BYTES = {"pythia-1.4b": 2181026543, "mlp-gelu-1.4b": 838974329, "swiglu-7b": 1803563138, "layernorm-1.4b": 210897047}
 
 
 def tri(n):
