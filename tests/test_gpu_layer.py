@@ -283,3 +283,37 @@ def test_gated_activation_module_autograd(act):
                                    util.gated_noise(x.detach().cpu(), None, act, plain.cpu()), "no bias")
     with pytest.raises(ValueError):
         Gated_Activation(torch.tanh)
+
+
+def test_element_offsets_beyond_32_bits(hotpath):
+    """[65544, 65536] bf16 holds more than 2^32 elements: rows near the end must come out like rows near
+    the start for bias+GeLU (in place), SwiGLU and LayerNorm."""
+    rows, cols = 65544, 65536
+    L, BF16 = hotpath.lib(), hotpath.BF16
+    gen = torch.Generator(device=DEV).manual_seed(0)
+    block = (torch.randn((8, cols), generator=gen, device=DEV) * 2).bfloat16()
+    x = torch.empty((rows, cols), dtype=torch.bfloat16, device=DEV)
+    x.view(-1, 8, cols)[:] = block                       # every group of 8 rows holds the same data
+    bias = (torch.randn((cols,), generator=gen, device=DEV) * 0.5).bfloat16()
+    want = oracle.bias_gelu_fwd(block.cpu(), bias.cpu())
+    noise = util.gelu_noise(bias.float().cpu() + block.float().cpu())
+    # SwiGLU first (x is still intact): [rows, 2 * 32768] -> [rows, 32768]
+    sw = torch.empty((rows, cols // 2), dtype=torch.bfloat16, device=DEV)
+    assert L.nhp_gated_act_fwd(sw.data_ptr(), x.data_ptr(), None, rows, cols // 2, 0, BF16, None) == 0
+    want_sw = oracle.gated_act_fwd(block.cpu(), "swiglu")
+    for r0 in (0, rows - 8):
+        util.assert_close_ulp_or_noise(sw[r0:r0 + 8].cpu(), want_sw, 2, util.gated_noise(block.cpu(), None, "swiglu", want_sw),
+                                       f"swiglu rows {r0}")
+    del sw
+    # LayerNorm into a second tensor
+    y = torch.empty_like(x)
+    assert L.nhp_layernorm_fwd(y.data_ptr(), None, None, x.data_ptr(), None, None, 1e-5, rows, cols, BF16, BF16, None) == 0
+    want_ln, _, _ = oracle.layernorm_fwd(block.cpu(), None, None, 1e-5)
+    for r0 in (0, 32768, rows - 8):
+        util.assert_close_ulp_or_noise(y[r0:r0 + 8].cpu(), want_ln, 2, torch.full((8, cols), 64 * util.EPS32), f"layernorm rows {r0}")
+    del y
+    # bias + GeLU in place
+    assert L.nhp_bias_gelu_fwd(x.data_ptr(), x.data_ptr(), bias.data_ptr(), rows, cols, BF16, None) == 0
+    for r0 in (0, 32768, rows - 8):
+        util.assert_close_ulp_or_noise(x[r0:r0 + 8].cpu(), want, 2, noise, f"gelu rows {r0}")
+    assert torch.equal(x[:8], x[rows - 8:])
