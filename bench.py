@@ -24,6 +24,7 @@ the drop-in extension modules (which call libneox_hotpath.so):
   mlp-gelu-1.4b  bias + tanh-GeLU fwd and bwd (with the bias gradient) on the MLP activation [2048*8, 8192] bf16
   swiglu-7b      SwiGLU forward and backward on the Llama-2 7B MLP activation [4096*4, 2*11008] -> [4096*4, 11008] bf16
   bias-residual-1.4b  residual + (x + bias) on the hidden state [2048*8, 2048] bf16
+  bias-dropout-add-1.4b  residual + dropout(x + bias) with p = 0.1, and the dropout backward, same shape
   layernorm-1.4b  LayerNorm fwd and bwd (with the parameter gradients) on the hidden state [2048*8, 2048] bf16
   rmsnorm-7b     RMSNorm fwd and bwd on [4096*4, 4096] bf16 (the Llama-2 7B hidden size)
 
@@ -355,6 +356,33 @@ def make_workload(name, torch, dev):
         cfg = {"workload": name, "hidden_state": [rows, cols], "parameters": "bf16", "parameter_gradients": True,
                "bytes_convention": "every tensor element read or written once, plus the fp32 row statistics"}
         return step, kernel_bytes, {}, "norm_bwd", "bf16", cfg
+
+    if name == "bias-dropout-add-1.4b":
+        from megatron.fused_kernels import _hotpath as hp
+
+        lib = hp.lib()
+        rows, cols = 2048 * 8, 2048
+        sets = [(randn((rows, cols), 10 * i, torch.bfloat16, 2.0), randn((rows, cols), 10 * i + 1, torch.bfloat16, 2.0))
+                for i in range(6)]
+        bias = randn((cols,), 7, torch.bfloat16)
+        out = torch.empty_like(sets[0][0])
+        n = rows * cols
+        kernel_bytes = {"bias_dropout_add": 3 * n * 2 + cols * 2, "dropout_bwd": 2 * n * 2}
+        state = {"i": 0}
+        stream = hp.stream_of(out)
+
+        def step(t):
+            x, res = sets[state["i"] % len(sets)]
+            state["i"] += 1
+            seed = 1000 + state["i"]
+            t.run("bias_dropout_add", lambda: hp.check(lib.nhp_bias_dropout_add(
+                out.data_ptr(), x.data_ptr(), bias.data_ptr(), res.data_ptr(), rows, cols, 0.1, seed, 0, hp.BF16, stream),
+                "bias_dropout_add"))
+            t.run("dropout_bwd", lambda: hp.check(lib.nhp_dropout_bwd(out.data_ptr(), res.data_ptr(), rows, cols, 0.1, seed,
+                                                                      0, hp.BF16, stream), "dropout_bwd"))
+
+        cfg = {"workload": name, "hidden_state": [rows, cols], "dropout": 0.1, "mask": "regenerated (Philox4x32-10), not stored"}
+        return step, kernel_bytes, {}, "bias_dropout_add", "bf16", cfg
 
     if name == "bias-residual-1.4b":
         from megatron.model.fused_bias_dropout import bias_dropout_add_fused_inference

@@ -34,6 +34,7 @@ def build(force=False, verbose=False):
 def _declare(lib):
     i64, vp, f32, ci = ctypes.c_int64, ctypes.c_void_p, ctypes.c_float, ctypes.c_int
     p64 = ctypes.POINTER(i64)
+    u64, pu32 = ctypes.c_uint64, ctypes.POINTER(ctypes.c_uint32)
     sigs = {
         "nhp_abi_version": ([], ci),
         "nhp_status_string": ([ci], ctypes.c_char_p),
@@ -55,6 +56,9 @@ def _declare(lib):
         "nhp_bias_gelu_bwd": ([vp, vp, vp, vp, vp, vp, i64, i64, ci, vp], ci),
         "nhp_bias_gelu_bwd_workspace_bytes": ([i64, i64, ci], i64),
         "nhp_bias_add_residual": ([vp, vp, vp, vp, i64, i64, ci, vp], ci),
+        "nhp_bias_dropout_add": ([vp, vp, vp, vp, i64, i64, f32, u64, u64, ci, vp], ci),
+        "nhp_dropout_bwd": ([vp, vp, i64, i64, f32, u64, u64, ci, vp], ci),
+        "nhp_philox4x32_10": ([pu32, pu32, pu32], None),
         "nhp_gated_act_fwd": ([vp, vp, vp, i64, i64, ci, ci, vp], ci),
         "nhp_gated_act_bwd": ([vp, vp, vp, vp, i64, i64, ci, ci, vp], ci),
         "nhp_layernorm_fwd": ([vp, vp, vp, vp, vp, vp, f32, i64, i64, ci, ci, vp], ci),

@@ -3,9 +3,12 @@
 Surface of GPT-NeoX's ``megatron/model/fused_bias_dropout.py``:
 ``bias_dropout_add`` (:28-35), ``get_bias_dropout_add`` (:38-42),
 ``bias_dropout_add_fused_train`` (:45-50), ``bias_dropout_add_fused_inference``
-(:53-58). With dropout off (``training`` False or ``prob`` 0, the default
-``hidden_dropout``) the whole expression ``residual + (x + bias)`` is one
-gfx950 kernel, evaluated in fp32 and rounded once.
+(:53-58). The whole expression ``residual + dropout(x + bias)`` is one gfx950
+kernel, evaluated in fp32 and rounded once. With dropout active the keep mask
+comes from the library's own counter-based generator (Philox4x32-10, seeded
+per call from torch's CPU generator, so ``torch.manual_seed`` makes runs
+repeatable); it is regenerated in the backward instead of being stored. Which
+elements are dropped therefore differs from what torch's dropout would pick.
 """
 from typing import Optional
 
@@ -59,12 +62,69 @@ class _BiasAddResidual(torch.autograd.Function):
         return grad, gb, grad if ctx.needs_input_grad[2] else None
 
 
+def _prepare(x, bias, residual, what):
+    _hp.require_gpu(x, what)
+    cols = x.size(-1)
+    src = x.contiguous()
+    b = None
+    if bias is not None:
+        if bias.numel() != cols or bias.dtype != x.dtype:
+            raise RuntimeError(f"{what}: bias must hold one value per feature, in the dtype of x")
+        _hp.require_gpu(bias, what)
+        b = bias.contiguous().view(-1)
+    res = None
+    if residual is not None:
+        if residual.shape != x.shape or residual.dtype != x.dtype:
+            raise RuntimeError(f"{what}: residual and x must have the same shape and dtype")
+        _hp.require_gpu(residual, what)
+        res = residual.contiguous()
+    return src, b, res, src.numel() // max(cols, 1), cols
+
+
+class _BiasDropoutAdd(torch.autograd.Function):
+    """``residual + dropout(x + bias)`` with the mask regenerated from (seed, prob) in the backward."""
+
+    @staticmethod
+    def forward(ctx, x, bias, residual, prob, seed):
+        what = "bias_dropout_add"
+        src, b, res, rows, cols = _prepare(x, bias, residual, what)
+        out = torch.empty_like(src)
+        with _hp.device_guard(src):
+            rc = _hp.lib().nhp_bias_dropout_add(out.data_ptr(), src.data_ptr(), None if b is None else b.data_ptr(),
+                                                None if res is None else res.data_ptr(), rows, cols, float(prob), seed,
+                                                0, _hp.dtype_code(src, what), _hp.stream_of(src))
+        _hp.check(rc, what)
+        ctx.conf = (float(prob), seed, None if bias is None else bias.shape)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad):
+        what = "bias_dropout_add backward"
+        prob, seed, bias_shape = ctx.conf
+        g = grad.contiguous()
+        cols = g.size(-1)
+        rows = g.numel() // max(cols, 1)
+        dx = torch.empty_like(g)
+        with _hp.device_guard(g):
+            rc = _hp.lib().nhp_dropout_bwd(dx.data_ptr(), g.data_ptr(), rows, cols, prob, seed, 0,
+                                           _hp.dtype_code(g, what), _hp.stream_of(g))
+        _hp.check(rc, what)
+        gb = None
+        if bias_shape is not None and ctx.needs_input_grad[1]:
+            gb = dx.reshape(-1, cols).sum(dim=0).view(bias_shape)
+        return dx, gb, grad if ctx.needs_input_grad[2] else None, None, None
+
+
+def _fresh_seed():
+    # from torch's CPU generator: no device synchronisation, repeatable under torch.manual_seed
+    return int(torch.empty((), dtype=torch.int64).random_().item())
+
+
 def bias_dropout_add(x: Tensor, bias: Tensor, residual: Optional[Tensor], prob: float, training: bool) -> Tensor:
     if training and prob > 0.0:
-        raise NotImplementedError(
-            "bias_dropout_add with dropout active (training and prob > 0) is not provided by the MI355X kernels; "
-            "set hidden_dropout to 0 or keep the reference's function for this call"
-        )
+        if not prob < 1.0:
+            raise ValueError(f"dropout probability has to be between 0 and 1, but got {prob}")
+        return _BiasDropoutAdd.apply(x, bias, residual, prob, _fresh_seed())
     return _BiasAddResidual.apply(x, bias, residual)
 
 

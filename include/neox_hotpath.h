@@ -325,6 +325,32 @@ int nhp_bias_add_residual(void* out, const void* x, const void* bias, const void
                           int64_t rows, int64_t cols, int dtype, void* stream);
 
 /*
+ * bias_dropout_add with dropout active (training and 0 < p < 1):
+ *   out = residual + keep * (x + bias) / (1 - p),  dx = keep * g / (1 - p)
+ * evaluated in fp32 and rounded once. The keep mask is not stored: element e
+ * (flat index) is kept when 16 bits of Philox4x32-10(counter = (e / 8, offset),
+ * key = seed) -- bits 16 * (e % 8) of the 128-bit output -- are below
+ * round((1 - p) * 65536); forward and backward regenerate it from (seed, offset).
+ * The generator is this library's own: which elements are dropped differs
+ * from what torch's generator would drop for the same seed, the distribution
+ * (independent Bernoulli(1 - p) per element) is the same. bias and residual
+ * may be NULL; p = 0 keeps everything.
+ *
+ * Replaces bias_dropout_add / bias_dropout_add_fused_train
+ *   megatron/model/fused_bias_dropout.py:28-50 (torch.nn.functional.dropout, differentiated by autograd)
+ */
+int nhp_bias_dropout_add(void* out, const void* x, const void* bias, const void* residual,
+                         int64_t rows, int64_t cols, float p, uint64_t seed, uint64_t offset,
+                         int dtype, void* stream);
+
+int nhp_dropout_bwd(void* dx, const void* g, int64_t rows, int64_t cols,
+                    float p, uint64_t seed, uint64_t offset, int dtype, void* stream);
+
+/* Philox4x32-10 on the host, the generator of the dropout mask above (for known-answer tests);
+ * megatron/model/fused_bias_dropout.py:31 is where the reference draws its mask. */
+void nhp_philox4x32_10(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4]);
+
+/*
  * Gated MLP activations. in: [rows, 2 * features]; the first `features` values
  * of a row are x, the last `features` the gates g (x, gate = in.chunk(2, dim=-1));
  * bias: [2 * features] or NULL, each half added to its half of the row.

@@ -54,6 +54,12 @@ def lib():
         L.oracle_bias_gelu_bwd.argtypes = [vp, vp, vp, vp, i64, i64, ci]
         L.oracle_column_sum.argtypes = [vp, vp, i64, i64, ci]
         L.oracle_bias_add_residual.argtypes = [vp, vp, vp, vp, i64, i64, ci]
+        u64 = ctypes.c_uint64
+        pu32 = ctypes.POINTER(ctypes.c_uint32)
+        L.oracle_philox4x32_10.argtypes = [pu32, pu32, pu32]
+        L.oracle_philox4x32_10.restype = None
+        L.oracle_dropout_mask.argtypes = [vp, i64, f32, u64, u64]
+        L.oracle_bias_dropout_add.argtypes = [vp, vp, vp, vp, i64, i64, f32, u64, u64, ci]
         L.oracle_gated_act_fwd.argtypes = [vp, vp, vp, i64, i64, ci, ci]
         L.oracle_gated_act_bwd.argtypes = [vp, vp, vp, vp, i64, i64, ci, ci]
         L.oracle_layernorm_fwd.argtypes = [vp, vp, vp, vp, vp, vp, f32, i64, i64, ci, ci]
@@ -365,3 +371,34 @@ def gated_act_bwd(dy, inp, act, bias=None):
     _check(lib().oracle_gated_act_bwd(din.data_ptr(), dy.data_ptr(), inp.data_ptr(), bp, rows, f, GATE_ACTS[act],
                                       _DT[inp.dtype]), "gated_act_bwd")
     return din
+
+
+# ---------------------------------------------------------------------------
+# dropout (layer_semantics.c)
+# ---------------------------------------------------------------------------
+def philox4x32_10(counter, key):
+    """The four 32-bit output words for a 4-word counter and a 2-word key."""
+    c = (ctypes.c_uint32 * 4)(*counter)
+    k = (ctypes.c_uint32 * 2)(*key)
+    out = (ctypes.c_uint32 * 4)()
+    lib().oracle_philox4x32_10(c, k, out)
+    return list(out)
+
+
+def dropout_mask(n, p, seed, offset=0):
+    """bool [n]: which elements (by flat index) are kept."""
+    keep = torch.empty(max(n, 1), dtype=torch.uint8)
+    _check(lib().oracle_dropout_mask(keep.data_ptr(), n, float(p), int(seed), int(offset)), "dropout_mask")
+    return keep[:n].bool()
+
+
+def bias_dropout_add(x, bias, residual, p, seed, offset=0):
+    """residual + keep * (x + bias) / (1 - p) with the mask of dropout_mask."""
+    x = _cpu_contig(x)
+    out = torch.empty_like(x)
+    rows, cols = _rows_cols(x)
+    bias, bp = _opt_ptr(bias, x, "bias dtype")
+    residual, rp = _opt_ptr(residual, x, "residual dtype")
+    _check(lib().oracle_bias_dropout_add(out.data_ptr(), x.data_ptr(), bp, rp, rows, cols, float(p), int(seed),
+                                         int(offset), _DT[x.dtype]), "bias_dropout_add")
+    return out

@@ -4,8 +4,8 @@
  * Plain-C, single-threaded restatement of the bandwidth-bound element-wise and
  * normalisation functions that sit next to attention in a GPT-NeoX transformer
  * layer: bias + tanh-GeLU (forward, backward), bias + dropout + residual add in
- * its deterministic form (dropout off), LayerNorm and RMSNorm (forward,
- * backward). Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline
+ * both forms (dropout off; dropout active with a counter-based mask), gated
+ * MLP activations, LayerNorm and RMSNorm (forward, backward). Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline
  * leg may load this library, and only as the checker.
  *
  * Arithmetic: what the reference's fused (TorchScript) kernels and torch's
@@ -19,7 +19,11 @@
  * evaluation of the closed forms, torch's own library routines
  * (gelu(approximate="tanh"), layer_norm, autograd in float64), invariants
  * (normalised rows have zero mean / unit mean square, gradients are orthogonal
- * to the directions the normalisation removes), special values.
+ * to the directions the normalisation removes), special values. The dropout
+ * mask is this build's own definition (Philox4x32-10, pinned by its published
+ * known-answer vectors and statistically); which elements torch's generator
+ * would drop for the same seed is a different set: that part is PARITY
+ * UNPINNED against the reference by construction.
  */
 #include <math.h>
 #include <stdint.h>
@@ -398,5 +402,79 @@ int oracle_gated_act_bwd(void* din, const void* dy, const void* in, const void* 
             store_elem(din, r * 2 * f + c, dt, d * a);
             store_elem(din, r * 2 * f + f + c, dt, (d * x) * da);
         }
+    return 0;
+}
+
+/* ------------------------------------------------------------------------ */
+/* bias + dropout + residual add with dropout active                         */
+/* ------------------------------------------------------------------------ */
+
+/* Philox4x32-10 (Salmon, Moraes, Dror, Shaw: "Parallel random numbers: as easy
+ * as 1, 2, 3", SC'11; the generator family torch's CUDA dropout draws from). */
+void oracle_philox4x32_10(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4])
+{
+    uint32_t c0 = counter[0], c1 = counter[1], c2 = counter[2], c3 = counter[3], k0 = key[0], k1 = key[1];
+    for (int r = 0; r < 10; ++r) {
+        const uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+        const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+        c0 = n0;
+        c1 = (uint32_t)p1;
+        c2 = n2;
+        c3 = (uint32_t)p0;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+    out[0] = c0;
+    out[1] = c1;
+    out[2] = c2;
+    out[3] = c3;
+}
+
+/* keep[e] for e in [0, n): 16 bits per element, eight elements per Philox call
+ * with counter (e / 8, offset) and key seed; kept when below round((1 - p) * 65536). */
+int oracle_dropout_mask(uint8_t* keep, int64_t n, float p, uint64_t seed, uint64_t offset)
+{
+    const double kp = 1.0 - (double)p;
+    uint32_t threshold = (uint32_t)(kp * 65536.0 + 0.5);
+    if (threshold > 65536u) threshold = 65536u;
+    const uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+    for (int64_t g = 0; g * 8 < n; ++g) {
+        const uint32_t ctr[4] = {(uint32_t)g, (uint32_t)((uint64_t)g >> 32), (uint32_t)offset, (uint32_t)(offset >> 32)};
+        uint32_t r[4];
+        oracle_philox4x32_10(ctr, key, r);
+        for (int j = 0; j < 8 && g * 8 + j < n; ++j) {
+            const uint32_t v = (r[j >> 1] >> ((j & 1) * 16)) & 0xffffu;
+            keep[g * 8 + j] = v < threshold;
+        }
+    }
+    return 0;
+}
+
+/*
+ * bias_dropout_add (megatron/model/fused_bias_dropout.py:28-35) with training
+ * True and 0 < prob < 1: out = residual + dropout(x + bias), dropout(v) = keep ?
+ * v / (1 - p) : 0 (torch.nn.functional.dropout), here with the mask above,
+ * fp32 arithmetic and one rounding. x == NULL is not allowed; bias, residual
+ * may be NULL. With residual == NULL and bias == NULL this is the backward of
+ * the dropout applied to x = grad.
+ */
+int oracle_bias_dropout_add(void* out, const void* x, const void* bias, const void* residual, int64_t rows,
+                            int64_t cols, float p, uint64_t seed, uint64_t offset, int dt)
+{
+    const int64_t n = rows * cols;
+    uint8_t* keep = (uint8_t*)malloc((size_t)(n > 0 ? n : 1));
+    if (!keep) return -2;
+    oracle_dropout_mask(keep, n, p, seed, offset);
+    const float scale = (float)(1.0 / (1.0 - (double)p));
+    for (int64_t r = 0; r < rows; ++r)
+        for (int64_t c = 0; c < cols; ++c) {
+            const int64_t e = r * cols + c;
+            float v = load_elem(x, e, dt);
+            if (bias) v = v + load_elem(bias, c, dt);
+            v = keep[e] ? v * scale : 0.0f;
+            if (residual) v = load_elem(residual, e, dt) + v;
+            store_elem(out, e, dt, v);
+        }
+    free(keep);
     return 0;
 }

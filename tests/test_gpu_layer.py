@@ -209,8 +209,65 @@ def test_bias_dropout_add_functions():
     assert torch.equal(util.raw_bits(same.cpu()), util.raw_bits(want))
     assert torch.equal(util.raw_bits(get_bias_dropout_add(False)(x.to(DEV), bias.to(DEV), res.to(DEV), 0.5).cpu()),
                        util.raw_bits(want))
-    with pytest.raises(NotImplementedError):
-        bias_dropout_add_fused_train(x.to(DEV), bias.to(DEV), res.to(DEV), 0.1)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("shape", [(1, 8), (37, 96), (5, 1000), (300, 2048), (1000, 24), (64, 8192), (3, 7)],
+                         ids=lambda s: f"{s[0]}x{s[1]}")
+def test_bias_dropout_add_with_dropout_bit_exact(hotpath, shape, dtype):
+    """The mask comes from the library's generator, which the oracle restates: same seed, same bits."""
+    rows, cols = shape
+    x = util.randn((rows, cols), dtype, seed=1, std=2.0)
+    bias = util.randn((cols,), dtype, seed=2)
+    res = util.randn((rows, cols), dtype, seed=3, std=2.0)
+    L, code = hotpath.lib(), hotpath.dtype_code(x, "t")
+    xd, bd, rd = x.to(DEV), bias.to(DEV), res.to(DEV)
+    for p, seed, offset in ((0.1, 7, 0), (0.5, (1 << 40) + 3, 5), (0.0, 1, 0)):
+        out = torch.empty_like(xd)
+        assert L.nhp_bias_dropout_add(out.data_ptr(), xd.data_ptr(), bd.data_ptr(), rd.data_ptr(), rows, cols, p, seed, offset,
+                                      code, None) == 0
+        want = oracle.bias_dropout_add(x, bias, res, p, seed, offset)
+        assert torch.equal(util.raw_bits(out.cpu()), util.raw_bits(want)), (p, seed)
+        dx = torch.empty_like(xd)
+        assert L.nhp_dropout_bwd(dx.data_ptr(), xd.data_ptr(), rows, cols, p, seed, offset, code, None) == 0
+        assert torch.equal(util.raw_bits(dx.cpu()), util.raw_bits(oracle.bias_dropout_add(x, None, None, p, seed, offset)))
+    assert L.nhp_bias_dropout_add(out.data_ptr(), xd.data_ptr(), None, None, rows, cols, 1.0, 1, 0, code, None) == -2
+    assert L.nhp_bias_dropout_add(out.data_ptr(), xd.data_ptr(), None, None, rows, cols, -0.1, 1, 0, code, None) == -2
+
+
+def test_bias_dropout_add_training_functions():
+    from megatron.model.fused_bias_dropout import bias_dropout_add_fused_train, get_bias_dropout_add
+
+    dtype, p = torch.bfloat16, 0.2
+    x = util.randn((64, 4, 1024), dtype, seed=1, std=2.0).to(DEV).requires_grad_(True)
+    bias = util.randn((1024,), dtype, seed=2).to(DEV).requires_grad_(True)
+    res = util.randn((64, 4, 1024), dtype, seed=3, std=2.0).to(DEV).requires_grad_(True)
+    torch.manual_seed(5)
+    seed = int(torch.empty((), dtype=torch.int64).random_().item())  # what the function will draw
+    torch.manual_seed(5)
+    out = bias_dropout_add_fused_train(x, bias, res, p)
+    dropped = ~oracle.dropout_mask(x.numel(), p, seed).view(x.shape).to(DEV)
+    rate = dropped.float().mean().item()
+    assert abs(rate - p) < 0.01
+    assert torch.equal(out.detach()[dropped], res.detach()[dropped])
+    full = (res.detach().float() + (x.detach().float() + bias.detach().float()) / (1 - p)).to(dtype)
+    assert torch.equal(out.detach()[~dropped], full[~dropped])
+    g = util.randn(x.shape, dtype, seed=4).to(DEV)
+    out.backward(g)
+    assert torch.equal(res.grad, g)
+    assert (x.grad[dropped] == 0).all()
+    assert torch.equal(x.grad[~dropped], (g.float() / (1 - p)).to(dtype)[~dropped])
+    assert torch.allclose(bias.grad.float(), x.grad.float().sum(dim=(0, 1)), rtol=2.0**-7, atol=1e-2)
+    # repeatable under torch.manual_seed, different from call to call otherwise
+    torch.manual_seed(5)
+    again = bias_dropout_add_fused_train(x.detach(), bias.detach(), res.detach(), p)
+    other = bias_dropout_add_fused_train(x.detach(), bias.detach(), res.detach(), p)
+    assert torch.equal(again, out.detach()) and not torch.equal(other, again)
+    evaluated = get_bias_dropout_add(False)(x.detach(), bias.detach(), res.detach(), p)
+    assert torch.equal(util.raw_bits(evaluated.cpu()),
+                       util.raw_bits(oracle.bias_add_residual(x.detach().cpu(), bias.detach().cpu(), res.detach().cpu())))
+    with pytest.raises(ValueError):
+        bias_dropout_add_fused_train(x.detach(), bias.detach(), res.detach(), 1.0)
 
 
 # ---------------------------------------------------------------------------

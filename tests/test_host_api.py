@@ -229,7 +229,7 @@ def test_layer_modules_surface_and_errors():
         activations.bias_gelu(torch.zeros(8), torch.zeros(2, 8))
     with pytest.raises(RuntimeError, match="GPU"):
         fused_bias_dropout.bias_dropout_add_fused_inference(torch.zeros(2, 8), torch.zeros(8), torch.zeros(2, 8), 0.0)
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(RuntimeError, match="GPU"):
         fused_bias_dropout.bias_dropout_add(torch.zeros(2, 8), torch.zeros(8), None, 0.1, True)
     ln = norms.LayerNorm(16, eps=1e-5)
     assert sorted(n for n, _ in ln.named_parameters()) == ["bias", "weight"]

@@ -334,3 +334,72 @@ def test_gated_activation_backward_is_the_adjoint(dtype, act):
     x32 = inp.float().requires_grad_(True)
     reference_gated(x32, bias.float(), act).backward(dy.float())
     util.assert_close_ulp_or_noise(din, x32.grad.to(dtype), 1, noise, f"{act} vs fp32 autograd")
+
+
+# ---------------------------------------------------------------------------
+# dropout
+# ---------------------------------------------------------------------------
+PHILOX_KAT = [  # known-answer vectors published with Random123 (philox4x32, 10 rounds)
+    ([0, 0, 0, 0], [0, 0], [0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8]),
+    ([0xFFFFFFFF] * 4, [0xFFFFFFFF] * 2, [0x408F276D, 0x41C83B0E, 0xA20BC7C6, 0x6D5451FD]),
+    ([0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344], [0xA4093822, 0x299F31D0],
+     [0xD16CFE09, 0x94FDCCEB, 0x5001E420, 0x24126EA1]),
+]
+
+
+def test_philox_known_answers(hotpath):
+    import ctypes
+
+    for counter, key, want in PHILOX_KAT:
+        assert oracle.philox4x32_10(counter, key) == want
+        out = (ctypes.c_uint32 * 4)()
+        hotpath.lib().nhp_philox4x32_10((ctypes.c_uint32 * 4)(*counter), (ctypes.c_uint32 * 2)(*key), out)
+        assert list(out) == want
+
+
+def test_dropout_mask_is_bernoulli_and_keyed():
+    n = 1 << 20
+    for p in (0.1, 0.5, 0.9):
+        keep = oracle.dropout_mask(n, p, seed=1234)
+        rate = keep.float().mean().item()
+        sigma = math.sqrt(p * (1 - p) / n)
+        assert abs(rate - (1 - p)) < 5 * sigma + 2.0**-16, (p, rate)
+        # every one of the eight 16-bit lanes of a Philox call has that rate
+        lanes = keep.view(-1, 8).float().mean(0)
+        assert (lanes - (1 - p)).abs().max().item() < 5 * sigma * math.sqrt(8) + 2.0**-16
+        # neighbours are uncorrelated
+        k = keep.float() - (1 - p)
+        assert abs((k[:-1] * k[1:]).mean().item()) < 5 * p * (1 - p) / math.sqrt(n)
+    base = oracle.dropout_mask(4096, 0.5, seed=1)
+    assert not torch.equal(base, oracle.dropout_mask(4096, 0.5, seed=2))
+    assert not torch.equal(base, oracle.dropout_mask(4096, 0.5, seed=1, offset=1))
+    assert not torch.equal(base, oracle.dropout_mask(4096, 0.5, seed=1 << 32))
+    assert torch.equal(base, oracle.dropout_mask(4096, 0.5, seed=1))
+    assert torch.equal(base[:1000], oracle.dropout_mask(1000, 0.5, seed=1))          # a prefix, whatever the length
+    assert oracle.dropout_mask(4096, 0.0, seed=7).all()
+    # the mask is monotone in p: what is dropped at p stays dropped at p' > p
+    assert not (oracle.dropout_mask(4096, 0.7, seed=1) & ~oracle.dropout_mask(4096, 0.3, seed=1)).any()
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_bias_dropout_add_with_dropout(dtype):
+    x, bias = inputs(dtype, rows=33, cols=40, seed=21)
+    res = util.randn(x.shape, dtype, seed=22, std=2.0)
+    p, seed = 0.25, 99
+    keep = oracle.dropout_mask(x.numel(), p, seed).view_as(x)
+    out = oracle.bias_dropout_add(x, bias, res, p, seed)
+    # torch's definition of dropout applied with this mask, in fp32
+    scale = torch.tensor(1.0 / (1.0 - p), dtype=torch.float64).float()
+    want = (res.float() + torch.where(keep, (x.float() + bias.float()) * scale, torch.zeros(()))).to(dtype)
+    assert torch.equal(util.raw_bits(out), util.raw_bits(want))
+    assert torch.equal(util.raw_bits(out)[~keep], util.raw_bits(res)[~keep])
+    # p = 0 is the deterministic function; without bias and residual it is the backward of the dropout
+    assert torch.equal(util.raw_bits(oracle.bias_dropout_add(x, bias, res, 0.0, seed)),
+                       util.raw_bits(oracle.bias_add_residual(x, bias, res)))
+    g = oracle.bias_dropout_add(x, None, None, p, seed)
+    assert torch.equal(util.raw_bits(g), util.raw_bits(torch.where(keep, x.float() * scale, torch.zeros(())).to(dtype)))
+    # the expectation is preserved: mean over many seeds of dropout(v) approaches v
+    v = torch.ones((1, 64), dtype=torch.float32)
+    mean = sum(oracle.bias_dropout_add(v, None, None, 0.5, s) for s in range(400)) / 400
+    assert (mean - 1).abs().max().item() < 0.5
+    assert abs(mean.mean().item() - 1) < 0.05
