@@ -19,6 +19,7 @@ the drop-in extension modules (which call libneox_hotpath.so):
   rope-qk-1.4b   rotary fwd+bwd on q,k [2048,8,16,128] bf16, rotary_pct 0.25, q and k in one launch
   mistral-window causal softmax fwd+bwd [64,8192,8192] bf16 with a 4096-key sliding window applied by index
   alibi-1.4b     causal softmax fwd+bwd [128,2048,2048] bf16 with the AliBi bias of 16 heads added in the kernel
+  attn-dropout-1.4b  causal softmax + attention dropout (p = 0.1) in one kernel, fwd+bwd [128,2048,2048] bf16
   rpe-bias-1.4b  causal softmax fwd+bwd [128,2048,2048] bf16 with a bias tensor [16,2048,2048] added in the kernel
 
   mlp-gelu-1.4b  bias + tanh-GeLU fwd and bwd (with the bias gradient) on the MLP activation [2048*8, 8192] bf16
@@ -156,6 +157,30 @@ def make_workload(name, torch, dev):
         cfg = {"workload": name, "scores": [a, s, s], "qk": [s, b, h, d], "rotary_dim": d2,
                "scale": "1/sqrt(%d)" % d, "bytes_convention": "causal-min (reads of the lower triangle, dense writes)"}
         return step, kernel_bytes, dense, "causal_softmax_bwd", "bf16", cfg
+
+    if name == "attn-dropout-1.4b":
+        a, s = 128, 2048
+        scale = 1.0 / math.sqrt(128)
+        x = torch.empty((a, s, s), dtype=torch.bfloat16, device=dev)
+        dy = torch.empty_like(x)
+        for i in range(0, a, 8):
+            x[i:i + 8] = randn((8, s, s), i, torch.bfloat16, 2.0)
+            dy[i:i + 8] = randn((8, s, s), 1000 + i, torch.bfloat16)
+        n = a * s * s
+        fwd_b = a * tri(s) * 2 + 2 * n * 2          # triangle read, probabilities and dropped probabilities written
+        bwd_b = 2 * a * tri(s) * 2 + n * 2
+        kernel_bytes = {"softmax_dropout_fwd": fwd_b, "softmax_dropout_bwd": bwd_b}
+        state = {"i": 0}
+
+        def step(t):
+            state["i"] += 1
+            seed = state["i"]
+            dropped, y = t.run("softmax_dropout_fwd", lambda: causal_ext.forward_dropout(x, scale, 0.1, seed))
+            t.run("softmax_dropout_bwd", lambda: causal_ext.backward_dropout(dy, y, scale, 0.1, seed))
+
+        cfg = {"workload": name, "scores": [a, s, s], "dropout": 0.1, "mask": "regenerated (Philox4x32-10), not stored",
+               "bytes_convention": "lower-triangle reads, dense writes (two dense outputs in the forward)"}
+        return step, kernel_bytes, {}, "softmax_dropout_fwd", "bf16", cfg
 
     if name in ("mistral-window", "alibi-1.4b", "rpe-bias-1.4b"):
         from megatron.model.positional_embeddings import AliBi

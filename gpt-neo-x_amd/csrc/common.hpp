@@ -259,6 +259,68 @@ __device__ __forceinline__ float block_combine(float v, float* slots, int wave, 
 __device__ __forceinline__ float exp2_raw(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // ---------------------------------------------------------------------------
+// Counter-based random bits for dropout masks
+// ---------------------------------------------------------------------------
+// Philox4x32-10 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3", SC'11)
+struct Philox {
+    uint32_t v[4];
+};
+
+__device__ __forceinline__ Philox philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0,
+                                                uint32_t k1)
+{
+    constexpr uint32_t M0 = 0xD2511F53u, M1 = 0xCD9E8D57u, W0 = 0x9E3779B9u, W1 = 0xBB67AE85u;
+#pragma unroll
+    for (int r = 0; r < 10; ++r) {
+        const uint32_t hi0 = __umulhi(M0, c0), lo0 = M0 * c0;
+        const uint32_t hi1 = __umulhi(M1, c2), lo1 = M1 * c2;
+        const uint32_t n0 = hi1 ^ c1 ^ k0, n2 = hi0 ^ c3 ^ k1;
+        c0 = n0;
+        c1 = lo1;
+        c2 = n2;
+        c3 = lo0;
+        k0 += W0;
+        k1 += W1;
+    }
+    return Philox{{c0, c1, c2, c3}};
+}
+
+// 16-bit random value of element `lane8` (0..7) of the group of eight elements `group`
+__device__ __forceinline__ uint32_t random16(const Philox& r, int lane8)
+{
+    return (r.v[lane8 >> 1] >> ((lane8 & 1) * 16)) & 0xffffu;
+}
+
+// Dropout parameters as the kernels take them: keep when random16 < threshold, kept values are
+// multiplied by scale = 1 / (1 - p); counter = (element index / 8, offset), key = seed.
+struct DropoutKey {
+    uint32_t threshold;
+    float scale;
+    uint32_t seed_lo, seed_hi, off_lo, off_hi;
+};
+
+// Random bits for the group of eight consecutive elements that starts at flat index e0 (a multiple of 8).
+__device__ __forceinline__ Philox dropout_bits(const DropoutKey& k, uint64_t e0)
+{
+    const uint64_t group = e0 >> 3;
+    return philox4x32_10((uint32_t)group, (uint32_t)(group >> 32), k.off_lo, k.off_hi, k.seed_lo, k.seed_hi);
+}
+
+static inline DropoutKey make_dropout_key(float p, uint64_t seed, uint64_t offset)
+{
+    DropoutKey k;
+    const double keep = 1.0 - (double)p;
+    const uint32_t threshold = (uint32_t)(keep * 65536.0 + 0.5);
+    k.threshold = threshold > 65536u ? 65536u : threshold;
+    k.scale = (float)(1.0 / keep);
+    k.seed_lo = (uint32_t)seed;
+    k.seed_hi = (uint32_t)(seed >> 32);
+    k.off_lo = (uint32_t)offset;
+    k.off_hi = (uint32_t)(offset >> 32);
+    return k;
+}
+
+// ---------------------------------------------------------------------------
 // Host-side launch checks
 // ---------------------------------------------------------------------------
 static inline bool ptr_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

@@ -22,36 +22,6 @@ constexpr int kDropThreads = 256;
 constexpr int kDropU = 2;
 constexpr int kDropMaxTw = 64;
 
-// Philox4x32-10 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3", SC'11)
-struct Philox {
-    uint32_t v[4];
-};
-
-__device__ __forceinline__ Philox philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0,
-                                                uint32_t k1)
-{
-    constexpr uint32_t M0 = 0xD2511F53u, M1 = 0xCD9E8D57u, W0 = 0x9E3779B9u, W1 = 0xBB67AE85u;
-#pragma unroll
-    for (int r = 0; r < 10; ++r) {
-        const uint32_t hi0 = __umulhi(M0, c0), lo0 = M0 * c0;
-        const uint32_t hi1 = __umulhi(M1, c2), lo1 = M1 * c2;
-        const uint32_t n0 = hi1 ^ c1 ^ k0, n2 = hi0 ^ c3 ^ k1;
-        c0 = n0;
-        c1 = lo1;
-        c2 = n2;
-        c3 = lo0;
-        k0 += W0;
-        k1 += W1;
-    }
-    return Philox{{c0, c1, c2, c3}};
-}
-
-// 16-bit random value of element `lane8` (0..7) of the group of eight elements `group`
-__device__ __forceinline__ uint32_t random16(const Philox& r, int lane8)
-{
-    return (r.v[lane8 >> 1] >> ((lane8 & 1) * 16)) & 0xffffu;
-}
-
 struct DropArgs {
     void* out;
     const void* a;         // x (forward) or g (backward)

@@ -184,14 +184,20 @@ __device__ __forceinline__ uint32_t active_slots(const Band& band, int w)
 // ---------------------------------------------------------------------------
 // Causal forward
 // ---------------------------------------------------------------------------
-// PER_HEAD = false compiles the per-head extras (bias tensor, AliBi, key
-// lengths) out of the plain kernel, which then keeps its registers for loads in flight.
-template <int DT, int L, int K, int W, int BW, bool PER_HEAD>
+// EXTRA selects what is compiled in besides the plain kernel (which keeps its
+// registers for loads in flight): kPerHead = bias tensor, AliBi, key lengths;
+// kDropout = a second output `dropped` = dropout(y) (y, the probabilities, is
+// still written: the backward needs it).
+enum CausalExtra { kPlain = 0, kPerHead = 1, kDropout = 2 };
+
+template <int DT, int L, int K, int W, int BW, int EXTRA>
 __global__ void __launch_bounds__((Geo<L, K, W, BW>::kThreads))
 causal_fwd_kernel(uint16_t* y, const uint16_t* x, float scale, uint32_t total_rows, uint32_t n, uint32_t window,
-                  const float* slopes, const uint16_t* bias, const int32_t* key_lengths, uint32_t heads)
+                  const float* slopes, const uint16_t* bias, const int32_t* key_lengths, uint32_t heads,
+                  uint16_t* dropped, DropoutKey dk)
 {
     using G = Geo<L, K, W, BW>;
+    constexpr bool PER_HEAD = EXTRA == kPerHead;
     __shared__ float lds[32];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -286,9 +292,20 @@ causal_fwd_kernel(uint16_t* y, const uint16_t* x, float scale, uint32_t total_ro
         const uint32_t col = chunk_col<L, W>(k, w, l);
         if (ok && col < n) {
             if ((act >> k & 1u) && col < band.hi && col + 8 > band.lo) {
-                store16_stream(yr + col, pack8<DT>(z[k]));
+                const u32x4 py = pack8<DT>(z[k]);
+                store16_stream(yr + col, py);
+                if constexpr (EXTRA == kDropout) {
+                    // dropout of the stored (rounded) probabilities, as the separate dropout kernel would see them
+                    float f[8];
+                    unpack8<DT>(py, f);
+                    const Philox rnd = dropout_bits(dk, (uint64_t)row * n + col);
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) f[j] = random16(rnd, j) < dk.threshold ? f[j] * dk.scale : 0.0f;
+                    store16_stream(dropped + (size_t)row * n + col, pack8<DT>(f));
+                }
             } else {
                 store16_stream(yr + col, u32x4{0, 0, 0, 0});
+                if constexpr (EXTRA == kDropout) store16_stream(dropped + (size_t)row * n + col, u32x4{0, 0, 0, 0});
             }
         }
     }
@@ -434,11 +451,14 @@ masked_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
 // Backward (causal and unmasked). dx = scale * (dy*y - y * sum(dy*y)).
 // dy and y stay packed in registers between the two passes.
 // ---------------------------------------------------------------------------
-template <int DT, int L, int K, int W, int BW, bool CAUSAL, bool LENGTHS>
+// EXTRA: kPlain, kPerHead (key lengths; causal only) or kDropout (dy is the gradient of
+// dropout(y): the kernel first forms keep * dy / (1 - p), rounded to the storage type as the
+// separate dropout backward would store it; causal only).
+template <int DT, int L, int K, int W, int BW, bool CAUSAL, int EXTRA>
 __global__ void __launch_bounds__((Geo<L, K, W, BW>::kThreads))
 softmax_bwd_kernel(uint16_t* dx, const uint16_t* dy, const uint16_t* y, float scale,
                    uint32_t total_rows, uint32_t n, uint32_t rows_per_matrix, uint32_t window,
-                   const int32_t* key_lengths, uint32_t heads)
+                   const int32_t* key_lengths, uint32_t heads, DropoutKey dk)
 {
     using G = Geo<L, K, W, BW>;
     __shared__ float lds[32];
@@ -453,7 +473,8 @@ softmax_bwd_kernel(uint16_t* dx, const uint16_t* dy, const uint16_t* y, float sc
     const bool ok = row < total_rows;
     Band band;
     if constexpr (CAUSAL) {
-        band = causal_band(q, window, ok, (LENGTHS && ok) ? key_limit(key_lengths, mat, heads) : 0xffffffffu);
+        band = causal_band(q, window, ok,
+                           (EXTRA == kPerHead && ok) ? key_limit(key_lengths, mat, heads) : 0xffffffffu);
     } else {
         band.lo = 0;
         band.hi = ok ? n : 0;
@@ -471,6 +492,14 @@ softmax_bwd_kernel(uint16_t* dx, const uint16_t* dy, const uint16_t* y, float sc
         if ((act >> k & 1u) && col < band.hi && col + 8 > band.lo) {
             rg[k] = load16_stream(dy + base + col);
             ry[k] = load16_stream(y + base + col);
+            if constexpr (EXTRA == kDropout) {
+                float f[8];
+                unpack8<DT>(rg[k], f);
+                const Philox rnd = dropout_bits(dk, (uint64_t)base + col);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) f[j] = random16(rnd, j) < dk.threshold ? f[j] * dk.scale : 0.0f;
+                rg[k] = pack8<DT>(f);
+            }
             if (CAUSAL && (col + 8 > band.hi || col < band.lo)) {
                 // zero the elements outside the band (both operands): keep [a, b) of the chunk
                 const uint32_t b_end = (band.hi - col < 8u) ? band.hi - col : 8u;
@@ -552,7 +581,8 @@ template <int DT, int MODE>
 __global__ void __launch_bounds__(kScalarThreads)
 scalar_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float scale,
                   uint64_t n, uint64_t sq, uint64_t np, int mask_per_batch, uint32_t window,
-                  const float* slopes, const uint16_t* bias, const int32_t* key_lengths, uint32_t heads)
+                  const float* slopes, const uint16_t* bias, const int32_t* key_lengths, uint32_t heads,
+                  uint16_t* dropped, DropoutKey dk)
 {
     __shared__ float slots[4];
     const uint64_t row = blockIdx.x;
@@ -601,13 +631,20 @@ scalar_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
         float p = 0.0f;
         if (c >= lo && c < hi) p = exp2_raw(fmaf(logit(c) - m, kLog2e, kExpBias)) * inv;
         yr[c] = Half2<DT>::to_bits(p);
+        if (MODE == 0 && dropped != nullptr) {
+            const uint64_t e = row * n + c;
+            const Philox rnd = dropout_bits(dk, e & ~(uint64_t)7);
+            const float kept = random16(rnd, (int)(e & 7u)) < dk.threshold ? Half2<DT>::round(p) * dk.scale : 0.0f;
+            dropped[e] = Half2<DT>::to_bits(kept);
+        }
     }
 }
 
 template <int DT, bool CAUSAL>
 __global__ void __launch_bounds__(kScalarThreads)
 scalar_bwd_kernel(uint16_t* dx, const uint16_t* dy, const uint16_t* y, float scale,
-                  uint64_t n, uint64_t rows_per_matrix, uint32_t window, const int32_t* key_lengths, uint32_t heads)
+                  uint64_t n, uint64_t rows_per_matrix, uint32_t window, const int32_t* key_lengths, uint32_t heads,
+                  int with_dropout, DropoutKey dk)
 {
     __shared__ float slots[4];
     const uint64_t row = blockIdx.x;
@@ -619,15 +656,26 @@ scalar_bwd_kernel(uint16_t* dx, const uint16_t* dy, const uint16_t* y, float sca
     const uint16_t* yr = y + row * n;
     uint16_t* dr = dx + row * n;
 
+    // the incoming gradient of column c: with dropout, keep * dy / (1 - p) rounded to the storage type
+    auto grad = [&](uint64_t c) {
+        float g = Half2<DT>::from_bits(gr[c]);
+        if (with_dropout) {
+            const uint64_t e = row * n + c;
+            const Philox rnd = dropout_bits(dk, e & ~(uint64_t)7);
+            g = random16(rnd, (int)(e & 7u)) < dk.threshold ? Half2<DT>::round(g * dk.scale) : 0.0f;
+        }
+        return g;
+    };
+
     float s = 0.0f;
-    for (uint64_t c = lo + threadIdx.x; c < hi; c += kScalarThreads)
-        s = fmaf(Half2<DT>::from_bits(gr[c]), Half2<DT>::from_bits(yr[c]), s);
+    for (uint64_t c = lo + threadIdx.x; c < hi; c += kScalarThreads) s = fmaf(grad(c), Half2<DT>::from_bits(yr[c]), s);
     s = block_reduce_256<OpSum>(s, slots);
 
+    // each thread reads its columns of dy before it overwrites them: dx may alias dy
     for (uint64_t c = threadIdx.x; c < n; c += kScalarThreads) {
         float g = 0.0f, p = 0.0f;
         if (c >= lo && c < hi) {
-            g = Half2<DT>::from_bits(gr[c]);
+            g = grad(c);
             p = Half2<DT>::from_bits(yr[c]);
         }
         dr[c] = Half2<DT>::to_bits(scale * fmaf(-p, s, g * p));
@@ -743,41 +791,50 @@ constexpr uint32_t kNoWindow = 0xffffffffu;
 
 template <int DT>
 static int causal_fwd(void* y, const void* x, float scale, int64_t batches, int64_t n, uint32_t window,
-                      const float* slopes, const void* bias, const int32_t* kl, uint32_t heads, hipStream_t st)
+                      const float* slopes, const void* bias, const int32_t* kl, uint32_t heads, hipStream_t st,
+                      void* dropped = nullptr, const DropoutKey* drop = nullptr)
 {
     const int64_t rows = batches * n;
     RowPlan p;
     uint16_t* yp = static_cast<uint16_t*>(y);
+    uint16_t* dp = static_cast<uint16_t*>(dropped);
     const uint16_t* xp = static_cast<const uint16_t*>(x);
     const uint16_t* bp = static_cast<const uint16_t*>(bias);
-    if (plan_row(n, kCausalFwd, p) && aligned16(x) && aligned16(y) && aligned16(bias)) {
+    const DropoutKey dk = drop != nullptr ? *drop : DropoutKey{};
+    if (plan_row(n, kCausalFwd, p) && aligned16(x) && aligned16(y) && aligned16(bias) && aligned16(dropped)) {
 #define CALL(L_, K_, W_)                                                                   \
     {                                                                                      \
         using G = Geo<L_, K_, W_, kBlockWaves>;                                            \
         const uint32_t blocks = (uint32_t)((rows + G::kRowsPerBlock - 1) / G::kRowsPerBlock); \
         if (!launch_fits(blocks, G::kThreads)) return NHP_ERR_SHAPE;                       \
-        if (slopes != nullptr || bp != nullptr || kl != nullptr)                           \
-            causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves, true><<<blocks, G::kThreads, p.lds, st>>>(  \
-                yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, slopes, bp, kl, heads); \
+        if (dp != nullptr)                                                                 \
+            causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves, kDropout><<<blocks, G::kThreads, p.lds, st>>>( \
+                yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, nullptr, nullptr, nullptr, 1, dp, dk); \
+        else if (slopes != nullptr || bp != nullptr || kl != nullptr)                      \
+            causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves, kPerHead><<<blocks, G::kThreads, p.lds, st>>>( \
+                yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, slopes, bp, kl, heads, nullptr, dk); \
         else                                                                               \
-            causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves, false><<<blocks, G::kThreads, p.lds, st>>>( \
-                yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, nullptr, nullptr, nullptr, 1); \
+            causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves, kPlain><<<blocks, G::kThreads, p.lds, st>>>( \
+                yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, nullptr, nullptr, nullptr, 1, nullptr, dk); \
     }
         NHP_FOR_PLAN(p);
 #undef CALL
     } else {
         if (!launch_fits(rows, kScalarThreads)) return NHP_ERR_SHAPE;
         scalar_fwd_kernel<DT, 0><<<(uint32_t)rows, kScalarThreads, 0, st>>>(
-            yp, xp, nullptr, scale, (uint64_t)n, (uint64_t)n, 1, 0, window, slopes, bp, kl, heads);
+            yp, xp, nullptr, scale, (uint64_t)n, (uint64_t)n, 1, 0, window, slopes, bp, kl, heads, dp, dk);
     }
     return launch_status();
 }
 
 template <int DT, bool CAUSAL>
 static int softmax_bwd(void* dx, const void* dy, const void* y, float scale, int64_t rows, int64_t n,
-                       int64_t rows_per_matrix, uint32_t window, const int32_t* kl, uint32_t heads, hipStream_t st)
+                       int64_t rows_per_matrix, uint32_t window, const int32_t* kl, uint32_t heads, hipStream_t st,
+                       const DropoutKey* drop = nullptr)
 {
     RowPlan p;
+    const DropoutKey dk = drop != nullptr ? *drop : DropoutKey{};
+    const bool dropout = CAUSAL && drop != nullptr;
     uint16_t* dxp = static_cast<uint16_t*>(dx);
     const uint16_t* dyp = static_cast<const uint16_t*>(dy);
     const uint16_t* yp = static_cast<const uint16_t*>(y);
@@ -787,19 +844,25 @@ static int softmax_bwd(void* dx, const void* dy, const void* y, float scale, int
         using G = Geo<L_, K_, W_, kBlockWaves>;                                            \
         const uint32_t blocks = (uint32_t)((rows + G::kRowsPerBlock - 1) / G::kRowsPerBlock); \
         if (!launch_fits(blocks, G::kThreads)) return NHP_ERR_SHAPE;                       \
-        if (CAUSAL && kl != nullptr)                                                       \
-            softmax_bwd_kernel<DT, L_, K_, W_, kBlockWaves, CAUSAL, CAUSAL><<<blocks, G::kThreads, p.lds, st>>>( \
-                dxp, dyp, yp, scale, (uint32_t)rows, (uint32_t)n, (uint32_t)rows_per_matrix, window, kl, heads); \
+        if (dropout)                                                                       \
+            softmax_bwd_kernel<DT, L_, K_, W_, kBlockWaves, CAUSAL, CAUSAL ? kDropout : kPlain>    \
+                <<<blocks, G::kThreads, p.lds, st>>>(dxp, dyp, yp, scale, (uint32_t)rows, (uint32_t)n, \
+                                                     (uint32_t)rows_per_matrix, window, nullptr, 1, dk); \
+        else if (CAUSAL && kl != nullptr)                                                  \
+            softmax_bwd_kernel<DT, L_, K_, W_, kBlockWaves, CAUSAL, CAUSAL ? kPerHead : kPlain>    \
+                <<<blocks, G::kThreads, p.lds, st>>>(dxp, dyp, yp, scale, (uint32_t)rows, (uint32_t)n, \
+                                                     (uint32_t)rows_per_matrix, window, kl, heads, dk); \
         else                                                                               \
-            softmax_bwd_kernel<DT, L_, K_, W_, kBlockWaves, CAUSAL, false><<<blocks, G::kThreads, p.lds, st>>>( \
-                dxp, dyp, yp, scale, (uint32_t)rows, (uint32_t)n, (uint32_t)rows_per_matrix, window, nullptr, 1); \
+            softmax_bwd_kernel<DT, L_, K_, W_, kBlockWaves, CAUSAL, kPlain><<<blocks, G::kThreads, p.lds, st>>>( \
+                dxp, dyp, yp, scale, (uint32_t)rows, (uint32_t)n, (uint32_t)rows_per_matrix, window, nullptr, 1, dk); \
     }
         NHP_FOR_PLAN(p);
 #undef CALL
     } else {
         if (!launch_fits(rows, kScalarThreads)) return NHP_ERR_SHAPE;
         scalar_bwd_kernel<DT, CAUSAL><<<(uint32_t)rows, kScalarThreads, 0, st>>>(
-            dxp, dyp, yp, scale, (uint64_t)n, (uint64_t)rows_per_matrix, window, CAUSAL ? kl : nullptr, heads);
+            dxp, dyp, yp, scale, (uint64_t)n, (uint64_t)rows_per_matrix, window, CAUSAL ? kl : nullptr, heads,
+            dropout ? 1 : 0, dk);
     }
     return launch_status();
 }
@@ -838,7 +901,7 @@ static int masked_fwd(void* y, const void* x, const uint8_t* mask, float scale, 
     } else {
         if (!launch_fits(b * np * sq, kScalarThreads)) return NHP_ERR_SHAPE;
         scalar_fwd_kernel<DT, 1><<<(uint32_t)(b * np * sq), kScalarThreads, 0, st>>>(
-            yp, xp, mask, scale, (uint64_t)n, (uint64_t)sq, (uint64_t)np, per_batch, kNoWindow, nullptr, nullptr, nullptr, 1);
+            yp, xp, mask, scale, (uint64_t)n, (uint64_t)sq, (uint64_t)np, per_batch, kNoWindow, nullptr, nullptr, nullptr, 1, nullptr, DropoutKey{});
     }
     return launch_status();
 }
@@ -902,6 +965,43 @@ int nhp_causal_softmax_bwd(void* dx, const void* dy, const void* y, float scale,
                            int64_t seq_len, int dtype, void* stream)
 {
     return nhp_causal_softmax_ex_bwd(dx, dy, y, scale, attn_batches, seq_len, -1, nullptr, 1, dtype, stream);
+}
+
+int nhp_causal_softmax_dropout_fwd(void* dropped, void* y, const void* x, float scale, int64_t attn_batches,
+                                   int64_t seq_len, int64_t window, float p, uint64_t seed, uint64_t offset, int dtype,
+                                   void* stream)
+{
+    if (dtype != NHP_F16 && dtype != NHP_BF16) return NHP_ERR_DTYPE;
+    if (attn_batches < 0 || seq_len < 0 || !(p >= 0.0f && p < 1.0f)) return NHP_ERR_SHAPE;
+    if (attn_batches == 0 || seq_len == 0) return NHP_OK;
+    if (attn_batches > kMaxRows / seq_len - 1) return NHP_ERR_SHAPE;
+    if (!x || !y || !dropped) return NHP_ERR_NULL;
+    if (dropped == y || dropped == x) return NHP_ERR_ALIAS;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const uint32_t win = (window < 0 || window >= seq_len) ? kNoWindow : (uint32_t)window;
+    const DropoutKey dk = make_dropout_key(p, seed, offset);
+    return dtype == NHP_BF16
+               ? causal_fwd<NHP_BF16>(y, x, scale, attn_batches, seq_len, win, nullptr, nullptr, nullptr, 1, st, dropped, &dk)
+               : causal_fwd<NHP_F16>(y, x, scale, attn_batches, seq_len, win, nullptr, nullptr, nullptr, 1, st, dropped, &dk);
+}
+
+int nhp_causal_softmax_dropout_bwd(void* dx, const void* dy, const void* y, float scale, int64_t attn_batches,
+                                   int64_t seq_len, int64_t window, float p, uint64_t seed, uint64_t offset, int dtype,
+                                   void* stream)
+{
+    if (dtype != NHP_F16 && dtype != NHP_BF16) return NHP_ERR_DTYPE;
+    if (attn_batches < 0 || seq_len < 0 || !(p >= 0.0f && p < 1.0f)) return NHP_ERR_SHAPE;
+    if (attn_batches == 0 || seq_len == 0) return NHP_OK;
+    if (attn_batches > kMaxRows / seq_len - 1) return NHP_ERR_SHAPE;
+    if (!dx || !dy || !y) return NHP_ERR_NULL;
+    if (dx == y) return NHP_ERR_ALIAS;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int64_t rows = attn_batches * seq_len;
+    const uint32_t win = (window < 0 || window >= seq_len) ? kNoWindow : (uint32_t)window;
+    const DropoutKey dk = make_dropout_key(p, seed, offset);
+    return dtype == NHP_BF16
+               ? softmax_bwd<NHP_BF16, true>(dx, dy, y, scale, rows, seq_len, seq_len, win, nullptr, 1, st, &dk)
+               : softmax_bwd<NHP_F16, true>(dx, dy, y, scale, rows, seq_len, seq_len, win, nullptr, 1, st, &dk);
 }
 
 int nhp_masked_softmax_fwd(void* y, const void* x, const uint8_t* mask, float scale, int64_t b,

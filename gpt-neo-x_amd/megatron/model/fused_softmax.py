@@ -26,7 +26,11 @@ all of it widening:
 * ``forward(..., key_lengths=None)``: an integer tensor ``[b]`` of real key counts for
   right-padded batches. The causal kernel masks the padding keys by index (the
   reference's ignores the mask, so padding is attended to on its fused branch); the
-  other branches merge ``k >= key_lengths[b]`` into the mask they are given.
+  other branches merge ``k >= key_lengths[b]`` into the mask they are given;
+* constructor argument ``attention_dropout`` (default 0): in training mode the module returns
+  ``dropout(probabilities)``; on the causal fused branch softmax and dropout are one kernel and
+  the keep mask (the library's counter-based generator, seeded from torch's CPU generator) is
+  regenerated in the backward instead of being stored. The caller must then not apply its own dropout.
 """
 import enum
 
@@ -82,6 +86,29 @@ class ScaledUpperTriangMaskedSoftmax(torch.autograd.Function):
         return grad, None, None, None, grad_bias, None
 
 
+class ScaledUpperTriangMaskedSoftmaxDropout(torch.autograd.Function):
+    """``dropout(softmax(scale * x))`` under the causal mask in one kernel forward and one backward.
+    No counterpart in the reference, which runs ``torch.nn.Dropout`` on the probabilities."""
+
+    @staticmethod
+    def forward(ctx, inputs, scale, prob, seed, window=None):
+        import scaled_upper_triang_masked_softmax_cuda as kernels
+
+        factor = _scale_tensor(scale)
+        dropped, probs = kernels.forward_dropout(inputs, factor[0], prob, seed, window)
+        ctx.conf = (float(prob), int(seed), window)
+        ctx.save_for_backward(probs, factor)
+        return dropped
+
+    @staticmethod
+    def backward(ctx, output_grads):
+        import scaled_upper_triang_masked_softmax_cuda as kernels
+
+        probs, factor = ctx.saved_tensors
+        prob, seed, window = ctx.conf
+        return kernels.backward_dropout(output_grads, probs, factor[0], prob, seed, window), None, None, None, None
+
+
 class ScaledMaskedSoftmax(torch.autograd.Function):
     """``softmax(where(mask, -10000, scale * x))`` over the last dimension of
     ``[b, np, sq, sk]`` scores with a ``[1 or b, 1, sq, sk]`` mask."""
@@ -121,10 +148,13 @@ class FusedScaleMaskSoftmax(nn.Module):
         alibi_slopes: (extension) fp32 tensor ``[np]``; the AliBi bias is added
             inside the causal kernel, and by the other branches with the same
             roundings, so the caller must not add it.
+        attention_dropout: (extension) dropout probability applied to the
+            probabilities in training mode; fused with the softmax on the
+            causal branch. The caller must not apply its own dropout.
     """
 
     def __init__(self, input_in_fp16, input_in_bf16, fusion_type, mask_func, softmax_in_fp32, scale,
-                 sliding_window_width=None, alibi_slopes=None):
+                 sliding_window_width=None, alibi_slopes=None, attention_dropout=0.0):
         super().__init__()
         assert isinstance(fusion_type, SoftmaxFusionTypes), f"Invalid fusion type {fusion_type}"
         assert scale is None or softmax_in_fp32, "softmax should be in fp32 when scaled"
@@ -142,6 +172,8 @@ class FusedScaleMaskSoftmax(nn.Module):
         self.mask_func = mask_func
         self.scale = scale
 
+        assert 0.0 <= attention_dropout < 1.0, "attention_dropout must be in [0, 1)"
+        self.attention_dropout = float(attention_dropout)
         self.sliding_window_width = sliding_window_width
         if alibi_slopes is None:
             self.alibi_slopes = None
@@ -151,9 +183,24 @@ class FusedScaleMaskSoftmax(nn.Module):
     # ------------------------------------------------------------------ dispatch
     def forward(self, input, mask, bias=None, key_lengths=None):
         assert input.dim() == 4  # [b, np, sq, sk]
+        dropout = self.attention_dropout if self.training else 0.0
         if self.is_kernel_available(mask, *input.size()):
-            return self.forward_fused_softmax(input, mask, bias, key_lengths)
-        return self.forward_torch_softmax(input, mask, bias, key_lengths)
+            plain_causal = (self.upper_triang_mask_fusion and bias is None and key_lengths is None
+                            and self.alibi_slopes is None)
+            if dropout > 0.0 and plain_causal:
+                b, np, sq, sk = input.size()
+                assert sq == sk, "causal mask is only for self attention"
+                factor = 1.0 if self.scale is None else self.scale
+                seed = int(torch.empty((), dtype=torch.int64).random_().item())  # CPU generator: no device sync
+                probs = ScaledUpperTriangMaskedSoftmaxDropout.apply(input.view(b * np, sq, sk), factor, dropout, seed,
+                                                                    self.sliding_window_width)
+                return probs.view(b, np, sq, sk)
+            probs = self.forward_fused_softmax(input, mask, bias, key_lengths)
+        else:
+            probs = self.forward_torch_softmax(input, mask, bias, key_lengths)
+        if dropout > 0.0:
+            probs = torch.nn.functional.dropout(probs, p=dropout, training=True)
+        return probs
 
     def is_kernel_available(self, mask, b, np, sq, sk):
         """The reference's conditions (fused_softmax.py:148-168) without ``sk <= 2048``."""

@@ -115,3 +115,50 @@ def backward(output_grads, softmax_results, scale_factor, window=None, key_lengt
             _hp.stream_of(g))
     _hp.check(rc, "scaled_upper_triang_masked_softmax_cuda.backward")
     return g
+
+
+def forward_dropout(input, scale_factor, p, seed, window=None):
+    """``forward`` and attention dropout in one kernel: returns ``(dropped, probabilities)``.
+
+    ``dropped = keep * probabilities / (1 - p)`` with the library's counter-based keep mask for
+    ``seed`` (see ``nhp_causal_softmax_dropout_fwd``); ``probabilities`` is what ``forward`` returns
+    and what ``backward_dropout`` needs. Not part of the reference's extension module."""
+    if input.dim() != 3:
+        raise RuntimeError("expected 3D tensor")
+    if input.dtype not in _HALF:
+        raise RuntimeError("Only fp16 and bf16 are supported")
+    if input.size(1) != input.size(2):
+        raise RuntimeError("expected a square [attn_batches, seq_len, seq_len] tensor")
+    _hp.require_gpu(input, "scaled_upper_triang_masked_softmax_cuda.forward_dropout")
+    x = input.contiguous()
+    y = torch.empty_like(x)
+    dropped = torch.empty_like(x)
+    with _hp.device_guard(x):
+        rc = _hp.lib().nhp_causal_softmax_dropout_fwd(
+            dropped.data_ptr(), y.data_ptr(), x.data_ptr(), float(scale_factor), x.size(0), x.size(1),
+            -1 if window is None else int(window), float(p), int(seed), 0, _hp.dtype_code(x, "forward_dropout"),
+            _hp.stream_of(x))
+    _hp.check(rc, "scaled_upper_triang_masked_softmax_cuda.forward_dropout")
+    return dropped, y
+
+
+def backward_dropout(output_grads, softmax_results, scale_factor, p, seed, window=None):
+    """Gradient of ``forward_dropout`` with respect to its input, given the gradient of ``dropped``;
+    in place on ``output_grads`` like ``backward``."""
+    if output_grads.dim() != 3 or softmax_results.dim() != 3:
+        raise RuntimeError("expected 3D tensor")
+    if output_grads.dtype not in _HALF or softmax_results.dtype not in _HALF:
+        raise RuntimeError("Only fp16 and bf16 are supported")
+    if output_grads.shape != softmax_results.shape or output_grads.dtype != softmax_results.dtype:
+        raise RuntimeError("output_grads and softmax_results must have the same shape and dtype")
+    _hp.require_gpu(output_grads, "scaled_upper_triang_masked_softmax_cuda.backward_dropout")
+    _hp.require_gpu(softmax_results, "scaled_upper_triang_masked_softmax_cuda.backward_dropout")
+    g = output_grads.detach().contiguous()
+    y = softmax_results.detach().contiguous()
+    with _hp.device_guard(g):
+        rc = _hp.lib().nhp_causal_softmax_dropout_bwd(
+            g.data_ptr(), g.data_ptr(), y.data_ptr(), float(scale_factor), g.size(0), g.size(1),
+            -1 if window is None else int(window), float(p), int(seed), 0, _hp.dtype_code(g, "backward_dropout"),
+            _hp.stream_of(g))
+    _hp.check(rc, "scaled_upper_triang_masked_softmax_cuda.backward_dropout")
+    return g

@@ -137,6 +137,30 @@ int nhp_causal_softmax_ex_bwd(void* dx, const void* dy, const void* y, float sca
                               int64_t attn_batches, int64_t seq_len, int64_t window,
                               const int32_t* key_lengths, int64_t heads, int dtype, void* stream);
 
+/*
+ * Causal softmax and attention dropout in one pass:
+ *   y       = the probabilities of nhp_causal_softmax_ex_fwd (window as there; needed by the backward),
+ *   dropped = keep ? y / (1 - p) : 0, formed from the stored y and rounded to the storage type,
+ * i.e. what attention_probs = attention_dropout(scale_mask_softmax(...)) leaves in memory
+ * (megatron/model/transformer.py:588-593), without the pass that re-reads y and without a stored mask.
+ * The keep mask is the counter-based one of nhp_bias_dropout_add over the flat element index of the
+ * [attn_batches, seq_len, seq_len] tensor, regenerated by the backward from (seed, offset):
+ *   dx = softmax backward of g = keep ? dy / (1 - p) : 0 (g rounded to the storage type).
+ * dx may alias dy; dropped must not alias y or x. Which elements are dropped differs from what
+ * torch's generator would pick (see nhp_bias_dropout_add).
+ *
+ * Replaces scaled_upper_triang_masked_softmax_cuda.forward / backward
+ * (megatron/fused_kernels/scaled_upper_triang_masked_softmax.cpp:31-56) followed / preceded by
+ * torch.nn.Dropout (self.attention_dropout, megatron/model/transformer.py:509,592-593).
+ */
+int nhp_causal_softmax_dropout_fwd(void* dropped, void* y, const void* x, float scale,
+                                   int64_t attn_batches, int64_t seq_len, int64_t window,
+                                   float p, uint64_t seed, uint64_t offset, int dtype, void* stream);
+
+int nhp_causal_softmax_dropout_bwd(void* dx, const void* dy, const void* y, float scale,
+                                   int64_t attn_batches, int64_t seq_len, int64_t window,
+                                   float p, uint64_t seed, uint64_t offset, int dtype, void* stream);
+
 /* ------------------------------------------------------------------------
  * Scaled padding-masked softmax
  * ---------------------------------------------------------------------- */

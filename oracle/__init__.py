@@ -60,6 +60,8 @@ def lib():
         L.oracle_philox4x32_10.restype = None
         L.oracle_dropout_mask.argtypes = [vp, i64, f32, u64, u64]
         L.oracle_bias_dropout_add.argtypes = [vp, vp, vp, vp, i64, i64, f32, u64, u64, ci]
+        L.oracle_causal_softmax_dropout_fwd.argtypes = [vp, vp, vp, f32, i64, i64, i64, f32, u64, u64, ci]
+        L.oracle_causal_softmax_dropout_bwd.argtypes = [vp, vp, vp, f32, i64, i64, i64, f32, u64, u64, ci]
         L.oracle_gated_act_fwd.argtypes = [vp, vp, vp, i64, i64, ci, ci]
         L.oracle_gated_act_bwd.argtypes = [vp, vp, vp, vp, i64, i64, ci, ci]
         L.oracle_layernorm_fwd.argtypes = [vp, vp, vp, vp, vp, vp, f32, i64, i64, ci, ci]
@@ -402,3 +404,24 @@ def bias_dropout_add(x, bias, residual, p, seed, offset=0):
     _check(lib().oracle_bias_dropout_add(out.data_ptr(), x.data_ptr(), bp, rp, rows, cols, float(p), int(seed),
                                          int(offset), _DT[x.dtype]), "bias_dropout_add")
     return out
+
+
+def causal_softmax_dropout_fwd(x, scale, p, seed, offset=0, window=None):
+    """Returns (dropped, y): the probabilities y and dropout(y) with the mask of dropout_mask over x's flat index."""
+    assert x.dim() == 3 and x.size(1) == x.size(2)
+    x = _cpu_contig(x)
+    y, dropped = torch.empty_like(x), torch.empty_like(x)
+    _check(lib().oracle_causal_softmax_dropout_fwd(dropped.data_ptr(), y.data_ptr(), x.data_ptr(), float(scale), x.size(0),
+                                                   x.size(1), -1 if window is None else int(window), float(p), int(seed),
+                                                   int(offset), _DT[x.dtype]), "causal_softmax_dropout_fwd")
+    return dropped, y
+
+
+def causal_softmax_dropout_bwd(dy, y, scale, p, seed, offset=0, window=None):
+    """Gradient with respect to the scores, given the gradient of dropout(y)."""
+    dy, y = _cpu_contig(dy), _cpu_contig(y)
+    dx = torch.empty_like(dy)
+    _check(lib().oracle_causal_softmax_dropout_bwd(dx.data_ptr(), dy.data_ptr(), y.data_ptr(), float(scale), dy.size(0),
+                                                   dy.size(1), -1 if window is None else int(window), float(p), int(seed),
+                                                   int(offset), _DT[dy.dtype]), "causal_softmax_dropout_bwd")
+    return dx

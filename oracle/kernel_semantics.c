@@ -199,6 +199,54 @@ int oracle_softmax_ex_bwd(void* dx, const void* dy, const void* y, float scale, 
     return 0;
 }
 
+/*
+ * Causal softmax followed by attention dropout, as the attention layer applies them
+ * (megatron/model/transformer.py:588-593: attention_probs = scale_mask_softmax(...), then
+ * attention_probs = attention_dropout(attention_probs)): y as above, and
+ * dropped = keep ? y_stored / (1 - p) : 0 computed from the stored (rounded) y and rounded again,
+ * which is what a separate dropout kernel reading y produces. The mask is oracle_dropout_mask
+ * (layer_semantics.c) over the flat element index of the [batches, s, s] tensor.
+ */
+int oracle_dropout_mask(uint8_t* keep, int64_t n, float p, uint64_t seed, uint64_t offset);
+
+int oracle_causal_softmax_dropout_fwd(void* dropped, void* y, const void* x, float scale, int64_t batches, int64_t s,
+                                      int64_t window, float p, uint64_t seed, uint64_t offset, int dt)
+{
+    int rc = oracle_causal_softmax_ex_fwd(y, x, scale, batches, s, window, NULL, NULL, NULL, 1, dt);
+    if (rc) return rc;
+    const int64_t n = batches * s * s;
+    uint8_t* keep = (uint8_t*)malloc((size_t)(n > 0 ? n : 1));
+    if (!keep) return -2;
+    oracle_dropout_mask(keep, n, p, seed, offset);
+    const float ds = (float)(1.0 / (1.0 - (double)p));
+    for (int64_t e = 0; e < n; ++e) store_elem(dropped, e, dt, keep[e] ? load_elem(y, e, dt) * ds : 0.0f);
+    free(keep);
+    return 0;
+}
+
+/* Backward of the pair: first the dropout backward, g = keep ? dy / (1 - p) : 0 stored in the
+ * storage type, then the softmax backward on g. dx may alias dy. */
+int oracle_causal_softmax_dropout_bwd(void* dx, const void* dy, const void* y, float scale, int64_t batches, int64_t s,
+                                      int64_t window, float p, uint64_t seed, uint64_t offset, int dt)
+{
+    if (dt != DT_F16 && dt != DT_BF16) return -1;
+    const int64_t n = batches * s * s;
+    uint8_t* keep = (uint8_t*)malloc((size_t)(n > 0 ? n : 1));
+    uint16_t* g = (uint16_t*)malloc(sizeof(uint16_t) * (size_t)(n > 0 ? n : 1));
+    if (!keep || !g) {
+        free(keep);
+        free(g);
+        return -2;
+    }
+    oracle_dropout_mask(keep, n, p, seed, offset);
+    const float ds = (float)(1.0 / (1.0 - (double)p));
+    for (int64_t e = 0; e < n; ++e) store_elem(g, e, dt, keep[e] ? load_elem(dy, e, dt) * ds : 0.0f);
+    int rc = oracle_softmax_ex_bwd(dx, g, y, scale, batches * s, s, s, 1, window, NULL, 1, dt);
+    free(keep);
+    free(g);
+    return rc;
+}
+
 int oracle_softmax_bwd(void* dx, const void* dy, const void* y, float scale, int64_t rows, int64_t n,
                        int64_t rows_per_matrix, int causal, int dt)
 {

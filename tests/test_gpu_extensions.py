@@ -237,3 +237,65 @@ def test_module_with_key_lengths_all_branches_agree(fusion):
     if fusion == "upper_triang":
         want = oracle.causal_softmax_fwd(x.view(-1, s, s), scale, key_lengths=lengths.cpu()).view(b, np_, s, s)
         util.assert_ulp_close(out["fused"][0], want, 2, "fwd vs oracle")
+
+
+# (attn_batches, seq_len, window)
+DROPOUT_CASES = [(4, 64, None), (3, 200, 63), (2, 512, None), (2, 1024, 100), (6, 2048, None), (1, 4096, 1000),
+                 (1, 8192, None), (2, 1001, None), (2, 33, 7)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
+@pytest.mark.parametrize("case", DROPOUT_CASES, ids=lambda c: f"a{c[0]}_s{c[1]}_w{c[2]}")
+def test_softmax_with_attention_dropout_vs_oracle(hotpath, case, dtype):
+    """Probabilities within 2 ulp of the oracle; the dropped tensor is exactly dropout (oracle mask) of the
+    probabilities the GPU stored; the backward against the oracle given the same y."""
+    import scaled_upper_triang_masked_softmax_cuda as ext
+
+    a, s, window = case
+    print(f"softmax+dropout case {case} {dtype}", flush=True)
+    scale, p, seed = 1 / math.sqrt(128), 0.1, 1234 + s
+    x = util.randn((a, s, s), dtype, seed=s, std=2.0)
+    dy = util.randn((a, s, s), dtype, seed=s + 1)
+    want_y = oracle.causal_softmax_fwd(x, scale, window=window)
+    dropped, y = [t.cpu() for t in ext.forward_dropout(x.to(DEV), scale, p, seed, window)]
+    util.assert_ulp_close(y, want_y, 2, "y")
+    masked = fb.causal_mask(s, sliding_window_width=window)[0, 0]
+    assert int(util.raw_bits(y)[:, masked].abs().max()) == 0 and int(util.raw_bits(dropped)[:, masked].abs().max()) == 0
+    assert torch.equal(util.raw_bits(dropped), util.raw_bits(oracle.bias_dropout_add(y, None, None, p, seed)))
+    want_dx = oracle.causal_softmax_dropout_bwd(dy, want_y, scale, p, seed, window=window)
+    got_dx = ext.backward_dropout(dy.to(DEV).clone(), want_y.to(DEV), scale, p, seed, window).cpu()
+    assert int(util.raw_bits(got_dx)[:, masked].abs().max()) == 0
+    g = oracle.bias_dropout_add(dy, None, None, p, seed)
+    util.assert_softmax_bwd_close(got_dx, want_dx, g.masked_fill(masked, 0), want_y, scale, "bwd")
+
+
+def test_module_with_attention_dropout():
+    from megatron.model.fused_softmax import FusedScaleMaskSoftmax, SoftmaxFusionTypes as T
+
+    dtype, b, np_, s, scale, p = torch.bfloat16, 2, 4, 512, 0.125, 0.2
+    x = util.randn((b, np_, s, s), dtype, seed=1, std=2.0)
+    dy = util.randn((b, np_, s, s), dtype, seed=2)
+    mask = fb.causal_mask(s, DEV)
+    m = FusedScaleMaskSoftmax(False, True, T.upper_triang, fb.fill_masked_with_dtype_min, True, scale, attention_dropout=p)
+    torch.manual_seed(3)
+    seed = int(torch.empty((), dtype=torch.int64).random_().item())
+    torch.manual_seed(3)
+    xd = x.to(DEV).requires_grad_(True)
+    out = m(xd, mask)
+    out.backward(dy.to(DEV).clone())
+    want_d, want_y = oracle.causal_softmax_dropout_fwd(x.view(-1, s, s), scale, p, seed)
+    keep = oracle.dropout_mask(x.numel(), p, seed).view(-1, s, s)
+    got = out.detach().cpu().view(-1, s, s)
+    assert int(util.raw_bits(got)[~keep].abs().max()) == 0
+    assert (got.float() - want_d.float()).abs().max().item() <= 2.0**-7 * want_d.float().abs().max().item()
+    want_dx = oracle.causal_softmax_dropout_bwd(dy.view(-1, s, s), want_y, scale, p, seed)
+    gx = xd.grad.cpu().view(-1, s, s).float()
+    assert (gx - want_dx.float()).norm().item() <= 2.0**-6 * want_dx.float().norm().item()
+    # evaluation mode: no dropout, the plain kernel
+    m.eval()
+    util.assert_ulp_close(m(x.to(DEV), mask).cpu().view(-1, s, s), oracle.causal_softmax_fwd(x.view(-1, s, s), scale), 2, "eval")
+    # the general-mask branch applies torch's dropout after the kernel: same rate, rows still normalised on average
+    g = FusedScaleMaskSoftmax(False, True, T.general, fb.fill_masked_with_dtype_min, True, scale, attention_dropout=p)
+    yg = g(x.to(DEV), mask)
+    zero_rate = ((yg == 0) & ~mask).float().sum().item() / (~mask).expand_as(yg).float().sum().item()
+    assert abs(zero_rate - p) < 0.02

@@ -221,3 +221,36 @@ def test_key_lengths_backward(dtype):
     p.backward(dy.double()[live])
     err = (dx.double()[live] - xd.grad[live]).abs().max().item()
     assert err <= 3 * 2.0 ** (-8 if dtype == torch.bfloat16 else -11) * xd.grad.abs().max().item()
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("window", [None, 5])
+def test_softmax_with_attention_dropout_is_the_composition(dtype, window):
+    """softmax + dropout in one function == the softmax oracle followed by torch's definition of
+    dropout (keep ? v / (1 - p) : 0 on the stored probabilities) with the oracle's mask; the backward
+    == the dropout backward followed by the softmax backward, and matches float64 autograd."""
+    a, s, scale, p, seed = 3, 24, 0.4, 0.3, 77
+    x = util.randn((a, s, s), dtype, seed=1, std=2.0)
+    dy = util.randn((a, s, s), dtype, seed=2)
+    dropped, y = oracle.causal_softmax_dropout_fwd(x, scale, p, seed, window=window)
+    plain = oracle.causal_softmax_fwd(x, scale, window=window)
+    assert torch.equal(util.raw_bits(y), util.raw_bits(plain))
+    keep = oracle.dropout_mask(x.numel(), p, seed).view_as(x)
+    ds = torch.tensor(1.0 / (1.0 - p), dtype=torch.float64).float()
+    want = torch.where(keep, plain.float() * ds, torch.zeros(())).to(dtype)
+    assert torch.equal(util.raw_bits(dropped), util.raw_bits(want))
+    assert torch.equal(util.raw_bits(dropped), util.raw_bits(oracle.bias_dropout_add(plain, None, None, p, seed)))
+    dx = oracle.causal_softmax_dropout_bwd(dy, y, scale, p, seed, window=window)
+    g = oracle.bias_dropout_add(dy, None, None, p, seed)       # the dropout backward, stored in the dtype
+    assert torch.equal(util.raw_bits(dx), util.raw_bits(oracle.softmax_bwd(g, y, scale, True, window=window)))
+    # float64 autograd through softmax and the same mask (exact y instead of the rounded one: looser)
+    masked = fb.causal_mask(s, sliding_window_width=window)[0, 0]
+    xd = x.double().requires_grad_(True)
+    f32scale = float(torch.tensor(scale, dtype=torch.float32))
+    probs = torch.softmax((xd * f32scale).masked_fill(masked, float("-inf")), -1)
+    (probs * keep / (1 - p)).backward(dy.double())
+    err = (dx.double() - xd.grad).abs().max().item()
+    assert err <= 4 * 2.0 ** (-8 if dtype == torch.bfloat16 else -11) * xd.grad.abs().max().item()
+    # p = 0 is the plain pair
+    d0, y0 = oracle.causal_softmax_dropout_fwd(x, scale, 0.0, seed, window=window)
+    assert torch.equal(util.raw_bits(d0), util.raw_bits(plain)) and torch.equal(util.raw_bits(y0), util.raw_bits(plain))
