@@ -286,15 +286,18 @@ struct NormBwdArgs {
 };
 
 // Waves per workgroup of the backward kernel: as many row groups as the LDS buffer of the final
-// accumulator reduction (K * V floats per thread, at most 32 KiB) and 1024 threads allow.
+// accumulator reduction (K * V floats per thread, at most 32 KiB) and 512 threads allow (workgroups
+// of 1024 threads measured slower), or the W waves of one row if that is more.
 template <int K, int W, int V>
 constexpr int bwd_waves()
 {
     int g = 8192 / (K * V) / kWave;  // threads by the LDS bound, in waves
-    if (g > 16) g = 16;
+    if (g > 8) g = 8;
     g = g / W * W;                    // whole row groups
     return g < W ? W : g;
 }
+
+constexpr int kBwdU = 2;  // row blocks in flight per iteration of the backward loop
 
 template <int DT, int K, int W, bool RMS>
 __global__ void __launch_bounds__((bwd_waves<K, W, Elt<DT>::kVec>() * kWave))
@@ -307,7 +310,7 @@ norm_bwd_kernel(NormBwdArgs a)
     using S = typename Elt<DT>::storage;
     // [parity of the loop iteration][sum][row group][wave]: one barrier per iteration is enough when
     // consecutive iterations use different slots
-    __shared__ float slots[2][2][GROUPS > 1 ? GROUPS : 1][16];
+    __shared__ float slots[2][2 * kBwdU][GROUPS > 1 ? GROUPS : 1][16];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const size_t cols = (size_t)a.cpr * V;
@@ -334,111 +337,112 @@ norm_bwd_kernel(NormBwdArgs a)
 #pragma unroll
         for (int j = 0; j < V; ++j) acc_g[k][j] = acc_b[k][j] = 0.0f;
 
-    // loads of one row block (this thread's chunks of dy and x, the row's statistics)
-    auto fetch = [&](uint32_t rb, u32x4 (&rg)[K], u32x4 (&rx)[K], float& mean, float& scale) {
-        const RowSlot rs = locate<W, G>(rb, a.rows, a.L, a.logL, wave, lane);
-        const S* gr = static_cast<const S*>(a.dy) + (size_t)rs.row * cols;
-        const S* xr = static_cast<const S*>(a.x) + (size_t)rs.row * cols;
-#pragma unroll
-        for (int k = 0; k < K; ++k) {
-            rg[k] = u32x4{0, 0, 0, 0};
-            rx[k] = u32x4{0, 0, 0, 0};
-            if (rs.ok && col_live[k]) {
-                rg[k] = load16_stream(gr + (size_t)cc[k] * V);
-                rx[k] = load16_stream(xr + (size_t)cc[k] * V);
-            }
-        }
-        mean = 0.0f;
-        scale = 0.0f;
-        if (rs.ok) {
-            if (!RMS) mean = a.mean[rs.row];
-            scale = a.rstd[rs.row];
-        }
-    };
-
-    u32x4 rg[K], rx[K];
-    float mean = 0.0f, scale = 0.0f;
+    // Every iteration takes kBwdU consecutive row blocks; all their loads are issued before the
+    // first value is used (several rows in flight per thread without relying on a prefetch that
+    // the compiler would have to track across the loop's back edge).
     int parity = 0;
-    if (blockIdx.x < a.row_blocks) fetch(blockIdx.x, rg, rx, mean, scale);
-    for (uint32_t rb = blockIdx.x; rb < a.row_blocks; rb += gridDim.x) {
-        const RowSlot rs = locate<W, G>(rb, a.rows, a.L, a.logL, wave, lane);
-        // the next row block's loads are in flight while this one is reduced and stored
-        u32x4 ng[K], nx[K];
-        float nmean = 0.0f, nscale = 0.0f;
-        const uint32_t next = rb + gridDim.x;
-        if (next < a.row_blocks) fetch(next, ng, nx, nmean, nscale);
-
-        float s1 = 0.0f, s2 = 0.0f;
+    for (uint32_t rb0 = blockIdx.x * kBwdU; rb0 < a.row_blocks; rb0 += gridDim.x * kBwdU) {
+        RowSlot rs[kBwdU];
+        u32x4 rg[kBwdU][K], rx[kBwdU][K];
+        float mean[kBwdU], scale[kBwdU];
 #pragma unroll
-        for (int k = 0; k < K; ++k) {
-            if (rs.ok && col_live[k]) {
-                float fg[V], fx[V];
-                chunk_to_float<DT>(rg[k], fg);
-                chunk_to_float<DT>(rx[k], fx);
+        for (int u = 0; u < kBwdU; ++u) {
+            rs[u] = locate<W, G>(rb0 + u, a.rows, a.L, a.logL, wave, lane);
+            rs[u].ok = rs[u].ok && rb0 + u < a.row_blocks;
+            const S* gr = static_cast<const S*>(a.dy) + (size_t)rs[u].row * cols;
+            const S* xr = static_cast<const S*>(a.x) + (size_t)rs[u].row * cols;
 #pragma unroll
-                for (int j = 0; j < V; ++j) {
-                    const float xh = (fx[j] - mean) * scale;
-                    const float g = fg[j] * gam[k][j];
-                    s1 += g;
-                    s2 += g * xh;
-                    acc_g[k][j] += fg[j] * xh;
-                    acc_b[k][j] += fg[j];
+            for (int k = 0; k < K; ++k) {
+                rg[u][k] = u32x4{0, 0, 0, 0};
+                rx[u][k] = u32x4{0, 0, 0, 0};
+                if (rs[u].ok && col_live[k]) {
+                    rg[u][k] = load16_stream(gr + (size_t)cc[k] * V);
+                    rx[u][k] = load16_stream(xr + (size_t)cc[k] * V);
                 }
             }
+            mean[u] = 0.0f;
+            scale[u] = 0.0f;
+            if (rs[u].ok) {
+                if (!RMS) mean[u] = a.mean[rs[u].row];
+                scale[u] = a.rstd[rs[u].row];
+            }
         }
-        s1 = lanes_sum(s1, a.L);
-        s2 = lanes_sum(s2, a.L);
+
+        float s1[kBwdU], s2[kBwdU];
+#pragma unroll
+        for (int u = 0; u < kBwdU; ++u) {
+            s1[u] = s2[u] = 0.0f;
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+                if (rs[u].ok && col_live[k]) {
+                    float fg[V], fx[V];
+                    chunk_to_float<DT>(rg[u][k], fg);
+                    chunk_to_float<DT>(rx[u][k], fx);
+#pragma unroll
+                    for (int j = 0; j < V; ++j) {
+                        const float xh = (fx[j] - mean[u]) * scale[u];
+                        const float g = fg[j] * gam[k][j];
+                        s1[u] += g;
+                        s2[u] += g * xh;
+                        acc_g[k][j] += fg[j] * xh;
+                        acc_b[k][j] += fg[j];
+                    }
+                }
+            }
+            s1[u] = lanes_sum(s1[u], a.L);
+            s2[u] = lanes_sum(s2[u], a.L);
+        }
         if constexpr (W > 1) {
-            // both sums cross the row's waves behind one barrier
-            float* mine1 = slots[parity][0][rs.group];
-            float* mine2 = slots[parity][1][rs.group];
+            // all sums of the iteration cross the rows' waves behind one barrier
+            float(*mine)[GROUPS > 1 ? GROUPS : 1][16] = slots[parity];
+            const int grp = rs[0].group, w = rs[0].w;
             if (lane == 0) {
-                mine1[rs.w] = s1;
-                mine2[rs.w] = s2;
+#pragma unroll
+                for (int u = 0; u < kBwdU; ++u) {
+                    mine[2 * u][grp][w] = s1[u];
+                    mine[2 * u + 1][grp][w] = s2[u];
+                }
             }
             __syncthreads();
-            s1 = mine1[0];
-            s2 = mine2[0];
 #pragma unroll
-            for (int i = 1; i < W; ++i) {
-                s1 += mine1[i];
-                s2 += mine2[i];
+            for (int u = 0; u < kBwdU; ++u) {
+                s1[u] = mine[2 * u][grp][0];
+                s2[u] = mine[2 * u + 1][grp][0];
+#pragma unroll
+                for (int i = 1; i < W; ++i) {
+                    s1[u] += mine[2 * u][grp][i];
+                    s2[u] += mine[2 * u + 1][grp][i];
+                }
             }
             parity ^= 1;
         }
 
-        // LayerNorm: t = (s1 + xhat * s2) / n as c1 + xhat * c2 (no division per element)
-        const float c1 = s1 / n;
-        float k2 = s2 / n;
-        if (RMS && a.eps_mode == 1) {
-            const float rho = 1.0f - a.eps * scale;
-            k2 = rho > 0.0f ? k2 / rho : 0.0f;
-        }
-        S* dr = static_cast<S*>(a.dx) + (size_t)rs.row * cols;
 #pragma unroll
-        for (int k = 0; k < K; ++k) {
-            if (rs.ok && col_live[k]) {
-                float fg[V], fx[V], o[V];
-                chunk_to_float<DT>(rg[k], fg);
-                chunk_to_float<DT>(rx[k], fx);
-#pragma unroll
-                for (int j = 0; j < V; ++j) {
-                    const float xh = (fx[j] - mean) * scale;
-                    const float g = fg[j] * gam[k][j];
-                    const float t = RMS ? xh * k2 : c1 + xh * k2;
-                    o[j] = scale * (g - t);
-                }
-                store16_stream(dr + (size_t)cc[k] * V, float_to_chunk<DT>(o));
+        for (int u = 0; u < kBwdU; ++u) {
+            // LayerNorm: t = (s1 + xhat * s2) / n as c1 + xhat * c2 (no division per element)
+            const float c1 = s1[u] / n;
+            float k2 = s2[u] / n;
+            if (RMS && a.eps_mode == 1) {
+                const float rho = 1.0f - a.eps * scale[u];
+                k2 = rho > 0.0f ? k2 / rho : 0.0f;
             }
-        }
-        if (next < a.row_blocks) {
+            S* dr = static_cast<S*>(a.dx) + (size_t)rs[u].row * cols;
 #pragma unroll
             for (int k = 0; k < K; ++k) {
-                rg[k] = ng[k];
-                rx[k] = nx[k];
+                if (rs[u].ok && col_live[k]) {
+                    float fg[V], fx[V], o[V];
+                    chunk_to_float<DT>(rg[u][k], fg);
+                    chunk_to_float<DT>(rx[u][k], fx);
+#pragma unroll
+                    for (int j = 0; j < V; ++j) {
+                        const float xh = (fx[j] - mean[u]) * scale[u];
+                        const float g = fg[j] * gam[k][j];
+                        const float t = RMS ? xh * k2 : c1 + xh * k2;
+                        o[j] = scale[u] * (g - t);
+                    }
+                    store16_stream(dr + (size_t)cc[k] * V, float_to_chunk<DT>(o));
+                }
             }
-            mean = nmean;
-            scale = nscale;
         }
     }
 
@@ -616,7 +620,7 @@ static uint32_t norm_row_blocks(int64_t rows, const NormPlan& p, int waves)
 static int bwd_waves_of(const NormPlan& p, int v)
 {
     int g = 8192 / (p.K * v) / kWave;
-    if (g > 16) g = 16;
+    if (g > 8) g = 8;
     g = g / p.W * p.W;
     return g < p.W ? p.W : g;
 }
@@ -627,6 +631,7 @@ constexpr uint32_t kNormBwdWaves = 4096;
 
 static uint32_t norm_bwd_grid(uint32_t row_blocks, bool param_grads, int waves_per_block)
 {
+    row_blocks = (row_blocks + kBwdU - 1) / kBwdU;  // a workgroup takes kBwdU row blocks per iteration
     if (!param_grads) return row_blocks;
     const uint32_t cap = (uint32_t)norm_tune("NHP_NORM_GRID", (int)(kNormBwdWaves / (uint32_t)waves_per_block));
     return row_blocks < cap ? row_blocks : cap;

@@ -132,14 +132,11 @@ pointwise_kernel(void* out, const void* a, const void* b, const void* bias, floa
         }
     };
 
-    if (live && blockIdx.y < steps) {
-        u32x4 ra[U], rb[U];
-        fetch(blockIdx.y, ra, rb);
+    if (live) {
         for (uint32_t step = blockIdx.y; step < steps; step += gridDim.y) {
-            // the next step's loads are in flight while this one is computed and stored
-            u32x4 na[U], nb[U];
-            const uint32_t next = step + gridDim.y;
-            if (next < steps) fetch(next, na, nb);
+            // all loads of the step are issued before the first value is used
+            u32x4 ra[U], rb[U];
+            fetch(step, ra, rb);
             const uint32_t r = step * (TR * U) + tr;
 #pragma unroll
             for (int u = 0; u < U; ++u) {
@@ -158,13 +155,6 @@ pointwise_kernel(void* out, const void* a, const void* b, const void* bias, floa
 #pragma unroll
                         for (int j = 0; j < V; ++j) sums[j] += stored[j];
                     }
-                }
-            }
-            if (next < steps) {
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    ra[u] = na[u];
-                    rb[u] = nb[u];
                 }
             }
         }
@@ -245,7 +235,8 @@ struct TilePlan {
 
 static int elem_size(int dt) { return dt == NHP_F32 ? 4 : 2; }
 
-constexpr int kPwU = 2;       // rows in flight per thread
+constexpr int kPwU = 2;       // rows in flight per thread, one step per workgroup
+constexpr int kPwColsumU = 4; // ... when a workgroup loops over steps (column sums)
 constexpr int kPwMaxTw = 64;  // a wave reads 1 KiB of a row
 // Dynamic LDS asked for only to bound the resident workgroups per CU: with two
 // input tensors six workgroups per CU stream better than eight (measured).
@@ -260,7 +251,7 @@ static TilePlan plan_tiles(int64_t rows, int64_t cpr, bool colsum)
     p.tw = 1;
     const int max_tw = pw_tune("NHP_PW_TW", kPwMaxTw);
     while (p.tw < max_tw && p.tw < cpr) p.tw *= 2;
-    const int64_t step_rows = (int64_t)(kPwThreads / p.tw) * pw_tune("NHP_PW_U", kPwU);
+    const int64_t step_rows = (int64_t)(kPwThreads / p.tw) * pw_tune("NHP_PW_U", colsum ? kPwColsumU : kPwU);
     p.steps = (uint32_t)((rows + step_rows - 1) / step_rows);
     p.col_tiles = (uint32_t)((cpr + p.tw - 1) / p.tw);
     uint32_t cap = colsum ? (uint32_t)pw_tune("NHP_PW_GY", kPwColsumGridY) : 65535u;
@@ -282,7 +273,7 @@ static int launch_tiled(void* out, const void* a, const void* b, const void* bia
 #ifdef NHP_TUNING
 #define CASE(TW_)                                                                                        \
     case TW_:                                                                                            \
-        switch (pw_tune("NHP_PW_U", kPwU)) {                                                             \
+        switch (pw_tune("NHP_PW_U", COLSUM ? kPwColsumU : kPwU)) {                                                             \
         case 1: CASE_U(TW_, 1) break;                                                                    \
         case 2: CASE_U(TW_, 2) break;                                                                    \
         case 4: CASE_U(TW_, 4) break;                                                                    \
@@ -293,7 +284,7 @@ static int launch_tiled(void* out, const void* a, const void* b, const void* bia
 #else
 #define CASE(TW_)                                                                                        \
     case TW_:                                                                                            \
-        CASE_U(TW_, kPwU)                                                                                \
+        CASE_U(TW_, (COLSUM ? kPwColsumU : kPwU))                                                                             \
         break;
 #endif
     switch (p.tw) {
