@@ -1,0 +1,160 @@
+"""Randomised differential test: every kernel family against the CPU oracle on shapes drawn
+around the boundaries of the launch geometries (multiples of the 16-byte chunk +-1, powers
+of two +-8, one row, one column, rows that end in the middle of a workgroup). Seeds are fixed:
+the cases are the same on every run. Tolerances as in the per-kernel parity tests."""
+import math
+import random
+
+import pytest
+import torch
+
+import oracle
+import util
+from oracle import fallback_semantics as fb
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+HALF = [torch.bfloat16, torch.float16]
+ALL = HALF + [torch.float32]
+
+
+def boundary_int(rng, lo, hi):
+    """An integer in [lo, hi], biased towards chunk and power-of-two boundaries."""
+    kind = rng.random()
+    if kind < 0.35:
+        v = (1 << rng.randint(0, max(0, hi.bit_length() - 1))) + rng.choice((-8, -1, 0, 1, 8))
+    elif kind < 0.7:
+        v = 8 * rng.randint(1, max(1, hi // 8)) + rng.choice((-1, 0, 0, 1))
+    else:
+        v = rng.randint(lo, hi)
+    return max(lo, min(hi, v))
+
+
+def ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_causal_softmax_random_shapes(hotpath, seed):
+    import scaled_upper_triang_masked_softmax_cuda as ext
+
+    rng = random.Random(1000 + seed)
+    dtype = rng.choice(HALF)
+    a, s = rng.randint(1, 5), boundary_int(rng, 1, 1500)
+    window = rng.choice((None, None, rng.randint(0, s)))
+    scale = rng.choice((1.0, 0.125, 1 / math.sqrt(128), 0.3))
+    print(f"causal a={a} s={s} window={window} {dtype} scale={scale}", flush=True)
+    x = util.randn((a, s, s), dtype, seed=seed, std=2.0)
+    dy = util.randn((a, s, s), dtype, seed=seed + 1)
+    masked = fb.causal_mask(s, sliding_window_width=window)[0, 0]
+    want = oracle.causal_softmax_fwd(x, scale, window=window)
+    got = ext.forward(x.to(DEV), scale, window).cpu()
+    if masked.any():
+        assert int(util.raw_bits(got)[:, masked].abs().max()) == 0
+    util.assert_ulp_close(got, want, 2, "fwd")
+    want_dx = oracle.softmax_bwd(dy, want, scale, True, window=window)
+    got_dx = ext.backward(dy.to(DEV).clone(), want.to(DEV), scale, window).cpu()
+    util.assert_softmax_bwd_close(got_dx, want_dx, dy.masked_fill(masked, 0), want, scale, "bwd")
+    if rng.random() < 0.5:
+        p, sd = rng.choice((0.1, 0.5)), rng.randint(0, 1 << 40)
+        dropped, y = [t.cpu() for t in ext.forward_dropout(x.to(DEV), scale, p, sd, window)]
+        util.assert_ulp_close(y, want, 2, "dropout y")
+        assert torch.equal(util.raw_bits(dropped), util.raw_bits(oracle.bias_dropout_add(y, None, None, p, sd)))
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_masked_softmax_random_shapes(hotpath, seed):
+    rng = random.Random(2000 + seed)
+    dtype = rng.choice(HALF)
+    b, np_, sq, sk = rng.randint(1, 3), rng.randint(1, 5), rng.randint(2, 9), boundary_int(rng, 1, 3000)
+    pb = rng.choice((1, b))
+    scale = rng.choice((1.0, 0.125, 1 / math.sqrt(128)))
+    print(f"masked b={b} np={np_} sq={sq} sk={sk} pb={pb} {dtype}", flush=True)
+    x = util.randn((b, np_, sq, sk), dtype, seed=seed, std=3.0)
+    dy = util.randn((b, np_, sq, sk), dtype, seed=seed + 1)
+    mask = util.padding_mask(pb, sq, sk, seed, full_batch=0 if rng.random() < 0.3 else None)
+    want = oracle.masked_softmax_fwd(x, mask, scale)
+    got = util.abi_masked_fwd(hotpath, x.to(DEV), mask.to(DEV), scale).cpu()
+    util.assert_ulp_close(got, want, 2, "fwd")
+    want_dx = oracle.softmax_bwd(dy, want, scale, False)
+    got_dx = util.abi_masked_bwd(hotpath, dy.to(DEV), want.to(DEV), scale).cpu()
+    util.assert_softmax_bwd_close(got_dx, want_dx, dy, want, scale, "bwd")
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_rope_random_shapes(hotpath, seed):
+    rng = random.Random(3000 + seed)
+    dtype = rng.choice(ALL)
+    s, b, h = rng.randint(1, 40), rng.randint(1, 3), rng.randint(1, 5)
+    d = rng.choice((8, 16, 24, 32, 64, 96, 128, 256, 20, 6))
+    d2 = rng.choice([v for v in (d, d // 2, d // 4, 2, 4, 8) if 2 <= v <= d and v % 2 == 0])
+    print(f"rope s={s} b={b} h={h} d={d} d2={d2} {dtype}", flush=True)
+    t = util.randn((s, b, h, d), dtype, seed=seed)
+    g = torch.Generator().manual_seed(seed)
+    ang = (torch.rand((s, 1, 1, d2), generator=g) * 20 - 10).contiguous()
+    cos, sin = ang.cos().to(dtype), ang.sin().to(dtype)
+    for backward in (False, True):
+        want = oracle.rope_cached(t, cos, sin, backward=backward)
+        got = util.abi_rope_cached(hotpath, t.to(DEV), cos.to(DEV), sin.to(DEV), backward=backward).cpu()
+        assert torch.equal(util.raw_bits(got), util.raw_bits(want)), backward
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_layer_kernels_random_shapes(hotpath, seed):
+    rng = random.Random(4000 + seed)
+    dtype = rng.choice(ALL)
+    rows, cols = boundary_int(rng, 1, 600), boundary_int(rng, 1, 5000)
+    L, code = hotpath.lib(), hotpath._DTYPE[dtype]
+    print(f"layer rows={rows} cols={cols} {dtype}", flush=True)
+    x = util.randn((rows, cols), dtype, seed=seed, std=2.5) + 0.25
+    g = util.randn((rows, cols), dtype, seed=seed + 1)
+    bias = util.randn((cols,), dtype, seed=seed + 2, std=0.5)
+    gamma = (1 + 0.3 * util.randn((cols,), torch.float32, seed=seed + 3)).to(dtype)
+    xd, gd, bd, gmd = x.to(DEV), g.to(DEV), bias.to(DEV), gamma.to(DEV)
+    # bias + GeLU forward / backward with the bias gradient
+    x32 = bias.float() + x.float()
+    out, dx, dbias = torch.empty_like(xd), torch.empty_like(xd), torch.empty_like(bd)
+    ws = torch.empty(max(L.nhp_bias_gelu_bwd_workspace_bytes(rows, cols, code), 16), dtype=torch.uint8, device=DEV)
+    assert L.nhp_bias_gelu_fwd(out.data_ptr(), xd.data_ptr(), bd.data_ptr(), rows, cols, code, None) == 0
+    util.assert_close_ulp_or_noise(out.cpu(), oracle.bias_gelu_fwd(x, bias), 2, util.gelu_noise(x32), "gelu fwd")
+    assert L.nhp_bias_gelu_bwd(dx.data_ptr(), gd.data_ptr(), xd.data_ptr(), bd.data_ptr(), dbias.data_ptr(), ws.data_ptr(), rows,
+                               cols, code, None) == 0
+    util.assert_close_ulp_or_noise(dx.cpu(), oracle.bias_gelu_bwd(g, x, bias), 2, util.gelu_noise(x32, g), "gelu bwd")
+    util.assert_close_ulp_or_noise(dbias.cpu(), oracle.column_sum(dx.cpu()), 1, dx.float().abs().sum(0).cpu() * 16 * util.EPS32, "dbias")
+    # bias + residual add, with and without dropout: bit-exact
+    assert L.nhp_bias_add_residual(out.data_ptr(), xd.data_ptr(), bd.data_ptr(), gd.data_ptr(), rows, cols, code, None) == 0
+    assert torch.equal(util.raw_bits(out.cpu()), util.raw_bits(oracle.bias_add_residual(x, bias, g)))
+    p, sd = rng.choice((0.1, 0.5)), rng.randint(0, 1 << 50)
+    assert L.nhp_bias_dropout_add(out.data_ptr(), xd.data_ptr(), bd.data_ptr(), gd.data_ptr(), rows, cols, p, sd, 3, code, None) == 0
+    assert torch.equal(util.raw_bits(out.cpu()), util.raw_bits(oracle.bias_dropout_add(x, bias, g, p, sd, 3)))
+    # LayerNorm and RMSNorm forward / backward
+    nws = torch.empty(max(L.nhp_norm_bwd_workspace_bytes(rows, cols, code), 16), dtype=torch.uint8, device=DEV)
+    y, mean, rstd = torch.empty_like(xd), torch.empty(rows, device=DEV), torch.empty(rows, device=DEV)
+    dg, db = torch.empty_like(gmd), torch.empty_like(gmd)
+    noise_y = (gamma.float().abs() * 64 * util.EPS32).expand(rows, cols)
+    assert L.nhp_layernorm_fwd(y.data_ptr(), mean.data_ptr(), rstd.data_ptr(), xd.data_ptr(), gmd.data_ptr(), bd.data_ptr(), 1e-5,
+                               rows, cols, code, code, None) == 0
+    want_y, _, _ = oracle.layernorm_fwd(x, gamma, bias, 1e-5)
+    util.assert_close_ulp_or_noise(y.cpu(), want_y, 2, noise_y, "layernorm fwd")
+    assert L.nhp_layernorm_bwd(dx.data_ptr(), dg.data_ptr(), db.data_ptr(), gd.data_ptr(), xd.data_ptr(), mean.data_ptr(),
+                               rstd.data_ptr(), gmd.data_ptr(), nws.data_ptr(), rows, cols, code, code, None) == 0
+    want_dx, want_dg, want_db = oracle.layernorm_bwd(g, x, mean.cpu(), rstd.cpu(), gamma)
+    dxn = ((g.float().abs() * gamma.float().abs()).sum(-1, keepdim=True) * rstd.cpu()[:, None] * 64 * util.EPS32).expand(rows, cols)
+    util.assert_close_ulp_or_noise(dx.cpu(), want_dx, 2, dxn, "layernorm dx")
+    xhat = ((x.float() - mean.cpu()[:, None]) * rstd.cpu()[:, None]).abs()
+    util.assert_close_ulp_or_noise(dg.cpu(), want_dg, 2, (g.float().abs() * xhat).sum(0) * 32 * util.EPS32, "dgamma")
+    util.assert_close_ulp_or_noise(db.cpu(), want_db, 2, g.float().abs().sum(0) * 32 * util.EPS32, "dbeta")
+    mode = rng.choice((0, 1))
+    inv = torch.empty(rows, device=DEV)
+    assert L.nhp_rmsnorm_fwd(y.data_ptr(), inv.data_ptr(), xd.data_ptr(), gmd.data_ptr(), None, 1e-5, mode, rows, cols, code, code,
+                             None) == 0
+    want_r, _ = oracle.rmsnorm_fwd(x, gamma, None, 1e-5, mode)
+    util.assert_close_ulp_or_noise(y.cpu(), want_r, 2, noise_y, "rmsnorm fwd")
+    # gated activation on the same data when the width is even
+    if cols % 2 == 0:
+        act = rng.choice(sorted(oracle.GATE_ACTS))
+        f = cols // 2
+        go = torch.empty((rows, f), dtype=dtype, device=DEV)
+        assert L.nhp_gated_act_fwd(go.data_ptr(), xd.data_ptr(), bd.data_ptr(), rows, f, oracle.GATE_ACTS[act], code, None) == 0
+        want_g = oracle.gated_act_fwd(x, act, bias)
+        util.assert_close_ulp_or_noise(go.cpu(), want_g, 2, util.gated_noise(x, bias, act, want_g), f"gated {act}")
