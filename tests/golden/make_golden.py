@@ -123,6 +123,17 @@ def main():
         for act in sorted(oracle.GATE_ACTS):
             put(name, **{f"{act}_out": oracle.gated_act_fwd(inp, act, bias), f"{act}_din": oracle.gated_act_bwd(dy, inp, act, bias)})
 
+    for name, dtype, seed in (("drop_bf16", torch.bfloat16, 51), ("drop_fp16", torch.float16, 52)):
+        x = util.randn((3, 24, 24), dtype, seed, std=2.0)
+        dy = util.randn((3, 24, 24), dtype, seed + 1)
+        bias = util.randn((24,), dtype, seed + 2)
+        p, sd, scale = 0.25, 1234567890123 + seed, 0.25
+        dropped, y = oracle.causal_softmax_dropout_fwd(x, scale, p, sd)
+        put(name, x=x, dy=dy, bias=bias, p=np.float32(p), seed=np.int64(sd), scale=np.float32(scale),
+            keep=oracle.dropout_mask(x.numel(), p, sd).to(torch.uint8), y=y, dropped=dropped,
+            dx=oracle.causal_softmax_dropout_bwd(dy, y, scale, p, sd),
+            bda=oracle.bias_dropout_add(x.view(-1, 24), bias, dy.view(-1, 24), p, sd))
+
     path = os.path.join(HERE, "layer_golden.npz")
     np.savez_compressed(path, **out)
     print(path, os.path.getsize(path), "bytes,", len(out), "arrays")

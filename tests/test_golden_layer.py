@@ -21,7 +21,7 @@ def get(prefix, key):
     if arr.ndim == 0:
         return arr.item()
     t = torch.from_numpy(np.ascontiguousarray(arr))
-    if key == "lengths":
+    if key in ("lengths", "keep"):
         return t
     if key in FP32_KEYS:
         return t.view(torch.float32)
@@ -82,8 +82,45 @@ def test_oracle_reproduces_gated_golden(name):
         assert same(oracle.gated_act_bwd(dy, inp, act, bias), get(name, f"{act}_din")), act
 
 
+DROP = ["drop_bf16", "drop_fp16"]
+
+
+@pytest.mark.parametrize("name", DROP)
+def test_oracle_reproduces_dropout_golden(name):
+    x, dy, bias = (get(name, k) for k in ("x", "dy", "bias"))
+    p, seed, scale = get(name, "p"), get(name, "seed"), get(name, "scale")
+    assert torch.equal(oracle.dropout_mask(x.numel(), p, seed).to(torch.uint8), get(name, "keep"))
+    dropped, y = oracle.causal_softmax_dropout_fwd(x, scale, p, seed)
+    assert same(y, get(name, "y")) and same(dropped, get(name, "dropped"))
+    assert same(oracle.causal_softmax_dropout_bwd(dy, y, scale, p, seed), get(name, "dx"))
+    assert same(oracle.bias_dropout_add(x.view(-1, 24), bias, dy.view(-1, 24), p, seed), get(name, "bda"))
+
+
 def ptr(t):
     return None if t is None else t.data_ptr()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", DROP)
+def test_gpu_matches_dropout_golden(hotpath, name):
+    x, dy, bias, y = (get(name, k).cuda() for k in ("x", "dy", "bias", "y"))
+    p, seed, scale = get(name, "p"), get(name, "seed"), get(name, "scale")
+    L, code = hotpath.lib(), hotpath.dtype_code(x, "t")
+    a, s = x.size(0), x.size(1)
+    gy, gd = torch.empty_like(x), torch.empty_like(x)
+    assert L.nhp_causal_softmax_dropout_fwd(gd.data_ptr(), gy.data_ptr(), x.data_ptr(), scale, a, s, -1, p, seed, 0, code, None) == 0
+    util.assert_ulp_close(gy.cpu(), y.cpu(), 2, name)
+    keep = get(name, "keep").view(a, s, s).bool()
+    assert int(util.raw_bits(gd.cpu())[~keep].abs().max()) == 0                       # the golden mask, bit for bit
+    assert same(gd.cpu(), oracle.bias_dropout_add(gy.cpu(), None, None, p, seed))     # dropout of the GPU's own y
+    gdx = torch.empty_like(x)
+    assert L.nhp_causal_softmax_dropout_bwd(gdx.data_ptr(), dy.data_ptr(), y.data_ptr(), scale, a, s, -1, p, seed, 0, code, None) == 0
+    g = oracle.bias_dropout_add(dy.cpu(), None, None, p, seed)
+    upper = torch.triu(torch.ones(s, s, dtype=torch.bool), diagonal=1)
+    util.assert_softmax_bwd_close(gdx.cpu(), get(name, "dx"), g.masked_fill(upper, 0), y.cpu(), scale, name)
+    out = torch.empty((a * s, s), dtype=x.dtype, device="cuda")
+    assert L.nhp_bias_dropout_add(out.data_ptr(), x.data_ptr(), bias.data_ptr(), dy.data_ptr(), a * s, s, p, seed, 0, code, None) == 0
+    assert same(out.cpu(), get(name, "bda"))
 
 
 @pytest.mark.gpu
