@@ -23,9 +23,15 @@
 //
 // Masks are applied by index: in the causal kernels only the columns of the
 // band max(0, q - window) <= k <= q are loaded (window = none: 0 <= k <= q),
-// everything else is written as zeros; an AliBi bias is computed from (q - k)
-// and the head's slope; in the padding-mask kernel a chunk whose 8 mask bytes
-// are all 1 is not loaded.
+// everything else is written as zeros; the band also ends at the number of
+// real keys of the row's batch entry when key lengths are given; an AliBi bias
+// is computed from (q - k) and the head's slope, an additive bias tensor is
+// read beside the scores; in the padding-mask kernel a chunk whose 8 mask
+// bytes are all 1 is not loaded.
+//
+// Attention dropout (causal kernels): the forward also writes dropout(y), the
+// backward first applies the dropout backward to dy; the keep mask is
+// regenerated from a counter-based generator, never stored.
 
 #include "common.hpp"
 
