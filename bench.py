@@ -527,7 +527,14 @@ def cpu_baseline(torch):
     med = times[len(times) // 2]
     fwd_b, bwd_b = causal_bytes(h, s)
     nbytes = fwd_b + bwd_b + 4 * rope_bytes(s, 1, h, d, d2)
+    model = "unknown CPU"
+    try:
+        with open("/proc/cpuinfo") as f:
+            model = next((line.split(":", 1)[1].strip() for line in f if line.startswith("model name")), model)
+    except OSError:
+        pass
     return {"value": round(nbytes / med / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "cpu": f"{model} ({os.cpu_count()} logical cores visible)",
             "sample": "reference torch fallback (fp32 softmax via autograd, eager rotary) on 1/8 of the default "
                       f"workload: scores [1,16,2048,2048], q,k [2048,1,16,128] bf16; median of {len(times)} runs, "
                       f"{med * 1e3:.1f} ms each, same algorithmic-byte convention"}
