@@ -19,6 +19,12 @@
  *     dispatcher narrows it to the input dtype first
  *     (scaled_upper_triang_masked_softmax.h:368, scaled_masked_softmax.h:358);
  *     pass an already narrowed value to reproduce that.
+ * Two definitions that are this build's own, for variants the reference's kernels do not have:
+ *   - with key lengths, a row that keeps no key at all is written as zeros (the torch
+ *     fallback given the merged mask yields 1/s there; see oracle_causal_softmax_ex_fwd);
+ *   - the attention-dropout mask is the counter-based one of layer_semantics.c: which
+ *     elements torch's generator would drop is PARITY UNPINNED by construction, everything
+ *     else about oracle_causal_softmax_dropout_fwd/bwd is the composition of pinned parts.
  *
  * How this oracle is pinned (tests/test_oracle_*.py): closed forms (row 0 of a
  * causal softmax is [1,0,...], constant rows give 1/(q+1), fully masked rows
