@@ -374,3 +374,30 @@ def test_element_offsets_beyond_32_bits(hotpath):
     for r0 in (0, 32768, rows - 8):
         util.assert_close_ulp_or_noise(x[r0:r0 + 8].cpu(), want, 2, noise, f"gelu rows {r0}")
     assert torch.equal(x[:8], x[rows - 8:])
+
+
+def test_python_functions_accept_non_contiguous_inputs():
+    """The Python functions make their inputs contiguous themselves (the reference's TorchScript functions take
+    any strides): a transposed view gives the same bits as its contiguous copy."""
+    from megatron.model.activations import Gated_Activation, bias_gelu_impl
+    from megatron.model.fused_bias_dropout import bias_dropout_add_fused_inference
+    from megatron.model.norms import LayerNorm, RMSNorm
+
+    dtype = torch.bfloat16
+    base = util.randn((6, 40, 512), dtype, seed=1, std=2.0).to(DEV)
+    view = base.transpose(0, 1)                      # [40, 6, 512], not contiguous
+    assert not view.is_contiguous()
+    bias = util.randn((512,), dtype, seed=2).to(DEV)
+    res = util.randn((40, 6, 512), dtype, seed=3).to(DEV)
+    ln = LayerNorm(512).to(DEV).to(dtype)
+    rms = RMSNorm(512).to(DEV)
+    gate = Gated_Activation("swiglu")
+    for fn in (lambda t: bias_gelu_impl(t, bias), lambda t: bias_dropout_add_fused_inference(t, bias, res, 0.0), ln, rms,
+               lambda t: gate(t, bias)):
+        a, b = fn(view), fn(view.contiguous())
+        assert a.shape == b.shape and a.shape[:2] == (40, 6)
+        assert torch.equal(util.raw_bits(a), util.raw_bits(b))
+    # and gradients flow back to a non-contiguous leaf
+    leaf = base.clone().requires_grad_(True)
+    ln(leaf.transpose(0, 1)).sum().backward()
+    assert leaf.grad.shape == leaf.shape and torch.isfinite(leaf.grad.float()).all()
