@@ -710,7 +710,7 @@ static int tune(const char* name, int def)
 static inline int tune(const char*, int def) { return def; }
 #endif
 
-enum RowKind { kCausalFwd, kCausalBwd, kMaskedFwd, kMaskedBwd };
+enum RowKind { kCausalFwd, kCausalFwdExtra, kCausalBwd, kMaskedFwd, kMaskedBwd };
 
 // Geometry for rows of n elements, from measurements on MI355X. HBM efficiency
 // drops when too many different rows are in flight per CU, and a row should be
@@ -739,14 +739,17 @@ static bool plan_row(int64_t n, RowKind kind, RowPlan& p)
     p.L = 64;
     const int64_t segs = (chunks + 63) / 64;  // 1 KiB segments per row
     int W, K;
-    if (kind == kMaskedFwd && segs <= 4) {
+    if ((kind == kMaskedFwd || kind == kCausalFwdExtra) && segs <= 4) {
+        // masked forward: see above. Causal forward with per-element extra work (AliBi, bias tensor):
+        // without a barrier in the row the extra instructions of one wave overlap the loads of the
+        // others (measured at 2048: the extras cost 30-45 us with two waves per row, 15-20 us with one)
         W = 1;
         K = (int)segs;
     } else if (segs > 64) {
         W = 16;
         K = 8;
     } else {
-        K = (kind == kCausalFwd || kind == kMaskedFwd) ? 2 : 1;
+        K = (kind == kCausalFwd || kind == kCausalFwdExtra || kind == kMaskedFwd) ? 2 : 1;
         while (8 * K < segs) K *= 2;
         static const int kWaves[] = {1, 2, 3, 4, 6, 8};
         W = 8;
@@ -807,7 +810,9 @@ static int causal_fwd(void* y, const void* x, float scale, int64_t batches, int6
     const uint16_t* xp = static_cast<const uint16_t*>(x);
     const uint16_t* bp = static_cast<const uint16_t*>(bias);
     const DropoutKey dk = drop != nullptr ? *drop : DropoutKey{};
-    if (plan_row(n, kCausalFwd, p) && aligned16(x) && aligned16(y) && aligned16(bias) && aligned16(dropped)) {
+    const bool extras = slopes != nullptr || bp != nullptr;  // not dropout: its second output wants the two-wave shape
+    if (plan_row(n, extras ? kCausalFwdExtra : kCausalFwd, p) && aligned16(x) && aligned16(y) && aligned16(bias) &&
+        aligned16(dropped)) {
 #define CALL(L_, K_, W_)                                                                   \
     {                                                                                      \
         using G = Geo<L_, K_, W_, kBlockWaves>;                                            \
