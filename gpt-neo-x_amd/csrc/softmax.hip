@@ -720,9 +720,10 @@ enum RowKind { kCausalFwd, kCausalFwdExtra, kCausalBwd, kMaskedFwd, kMaskedBwd }
 //   backward (two input tensors): K = 1;
 //   at most 8 waves per row (workgroups of 1024 threads measured slower), so K
 //   doubles for rows beyond 8 * K KiB; rows beyond 32768 elements use 16 waves;
-//   padding-mask forward: one wave per row up to 2048 elements (K <= 4), since
-//   its waves walk over heads and a multi-wave row would synchronise twice
-//   per head.
+//   padding-mask forward: as the causal forward, its waves walking over two
+//   heads with one decoded mask row (measured at [16,32,1024,2048] fp16: 582 us
+//   with two waves per row and two heads, 615 with four heads, 633 with one,
+//   619 with one wave per row and two heads).
 static bool plan_row(int64_t n, RowKind kind, RowPlan& p)
 {
     if (n < 8 || n % 8 != 0 || n > kMaxResidentRow) return false;
@@ -739,8 +740,8 @@ static bool plan_row(int64_t n, RowKind kind, RowPlan& p)
     p.L = 64;
     const int64_t segs = (chunks + 63) / 64;  // 1 KiB segments per row
     int W, K;
-    if ((kind == kMaskedFwd || kind == kCausalFwdExtra) && segs <= 4) {
-        // masked forward: see above. Causal forward with per-element extra work (AliBi, bias tensor):
+    if (kind == kCausalFwdExtra && segs <= 4) {
+        // Causal forward with per-element extra work (AliBi, bias tensor):
         // without a barrier in the row the extra instructions of one wave overlap the loads of the
         // others (measured at 2048: the extras cost 30-45 us with two waves per row, 15-20 us with one)
         W = 1;
@@ -878,9 +879,9 @@ static int softmax_bwd(void* dx, const void* dy, const void* y, float scale, int
     return launch_status();
 }
 
-// Heads a wave walks over with one decoded mask row. A few are enough to
-// amortise the decoding; more would only make the access order less sequential.
-static uint32_t pick_heads_per_wave(int64_t np) { return (uint32_t)(np < 4 ? np : 4); }
+// Heads a wave walks over with one decoded mask row. Two amortise the decoding;
+// more make the access order less sequential and measured slower.
+static uint32_t pick_heads_per_wave(int64_t np) { return (uint32_t)(np < 2 ? np : 2); }
 
 template <int DT>
 static int masked_fwd(void* y, const void* x, const uint8_t* mask, float scale, int64_t b, int64_t np,
