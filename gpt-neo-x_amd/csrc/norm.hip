@@ -78,11 +78,26 @@ __device__ __forceinline__ void load_params(const void* p, bool f32, size_t e, f
     }
 }
 
-// 1 / (rms + eps) (eps_mode 1, the Python RMSNorm class) or rsqrt(mean(x^2) + eps) (eps_mode 0)
+// The factor a row is multiplied by, from the sum of squares over its n statistic columns:
+// 1 / (rms + eps) (eps_mode 1, the Python RMSNorm class), rsqrt(mean(x^2) + eps) (eps_mode 0) or
+// 1 / max(||x||, eps) (eps_mode 2, ScaleNorm).
 __device__ __forceinline__ float rms_inverse(float sumsq, float n, float eps, int eps_mode)
 {
+    if (eps_mode == 2) return 1.0f / fmaxf(sqrtf(sumsq), eps);
     if (eps_mode == 1) return 1.0f / (sqrtf(sumsq) * (1.0f / sqrtf(n)) + eps);
     return 1.0f / sqrtf(sumsq / n + eps);
+}
+
+// Factor of xhat * sum(g * xhat) in the RMSNorm backward (see norm_bwd_kernel).
+__device__ __forceinline__ float rms_bwd_factor(float s2, float n, float inv, float eps, int eps_mode)
+{
+    if (eps_mode == 2) return inv < 1.0f / eps ? s2 : 0.0f;  // clamped norm: the factor does not depend on x
+    float k2 = s2 / n;
+    if (eps_mode == 1) {
+        const float rho = 1.0f - eps * inv;
+        k2 = rho > 0.0f ? k2 / rho : 0.0f;
+    }
+    return k2;
 }
 
 struct RowSlot {
@@ -129,6 +144,7 @@ struct NormFwdArgs {
     int eps_mode;
     uint32_t rows, cpr, L, logL;
     int params_f32;
+    uint32_t stat;  // RMSNorm: the statistic is taken over the first `stat` columns
 };
 
 template <int DT, int K, int W, bool RMS>
@@ -143,7 +159,7 @@ norm_fwd_kernel(NormFwdArgs a)
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const RowSlot rs = locate<W, G>(blockIdx.x, a.rows, a.L, a.logL, wave, lane);
     const size_t cols = (size_t)a.cpr * V;
-    const float n = (float)cols;
+    const float n = RMS ? (float)a.stat : (float)cols;
     const S* xr = static_cast<const S*>(a.x) + (size_t)rs.row * cols;
     S* yr = static_cast<S*>(a.y) + (size_t)rs.row * cols;
 
@@ -177,10 +193,16 @@ norm_fwd_kernel(NormFwdArgs a)
             if (live[k]) {
                 float f[V];
                 chunk_to_float<DT>(raw[k], f);
+                const uint32_t e0 = ((uint32_t)(k * W + rs.w) * a.L + rs.l) * V;
+                if (!RMS || e0 + V <= a.stat) {
 #pragma unroll
-                for (int j = 0; j < V; ++j) {
-                    const float d = f[j] - mean;
-                    q += d * d;
+                    for (int j = 0; j < V; ++j) {
+                        const float d = f[j] - mean;
+                        q += d * d;
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < V; ++j) q += (e0 + j < a.stat) ? f[j] * f[j] : 0.0f;
                 }
             }
         }
@@ -228,12 +250,12 @@ __device__ __forceinline__ float block_sum_256(float v, float* slots)
 template <int DT, bool RMS>
 __global__ void __launch_bounds__(kNormScalarThreads)
 norm_fwd_scalar_kernel(void* y, float* mean_out, float* rstd_out, const void* x, const void* gamma,
-                       const void* beta, float eps, int eps_mode, uint64_t cols, int pdt)
+                       const void* beta, float eps, int eps_mode, uint64_t cols, uint64_t stat, int pdt)
 {
     __shared__ float slots[4];
     const uint64_t row = blockIdx.x;
     const int64_t base = (int64_t)(row * cols);
-    const float n = (float)cols;
+    const float n = RMS ? (float)stat : (float)cols;
     float mean = 0.0f;
     if (!RMS) {
         float s = 0.0f;
@@ -241,7 +263,7 @@ norm_fwd_scalar_kernel(void* y, float* mean_out, float* rstd_out, const void* x,
         mean = block_sum_256(s, slots) / n;
     }
     float q = 0.0f;
-    for (uint64_t c = threadIdx.x; c < cols; c += kNormScalarThreads) {
+    for (uint64_t c = threadIdx.x; c < (RMS ? stat : cols); c += kNormScalarThreads) {
         const float d = Elt<DT>::load(x, base + (int64_t)c) - mean;
         q += d * d;
     }
@@ -266,8 +288,9 @@ norm_fwd_scalar_kernel(void* y, float* mean_out, float* rstd_out, const void* x,
 // Backward
 //   xhat = (x - mean) * rstd (RMSNorm: x * inv), g = dy * gamma
 //   LayerNorm: dx = rstd * (g - (sum(g) + xhat * sum(g * xhat)) / cols)
-//   RMSNorm:   dx = inv * (g - xhat * sum(g * xhat) / (cols * rho)), rho = 1 for eps_mode 0 and
-//              1 - eps * inv for eps_mode 1 (rho <= 0: the second term is dropped)
+//   RMSNorm:   dx = inv * (g - [c < stat] * xhat * sum(g * xhat) / (stat * rho)), rho = 1 for eps_mode 0
+//              and 1 - eps * inv for eps_mode 1 (rho <= 0: the second term is dropped); eps_mode 2:
+//              dx = inv * (g - xhat * sum(g * xhat)) while the norm is above eps, inv * g below
 //   dgamma[c] = sum over rows of dy * xhat, dbeta[c] = sum over rows of dy
 // ---------------------------------------------------------------------------
 struct NormBwdArgs {
@@ -283,6 +306,7 @@ struct NormBwdArgs {
     int eps_mode;
     uint32_t rows, cpr, L, logL, row_blocks;
     int params_f32;
+    uint32_t stat;  // RMSNorm: number of leading columns the statistic was taken over
 };
 
 // Waves per workgroup of the backward kernel: as many row groups as the LDS buffer of the final
@@ -314,18 +338,20 @@ norm_bwd_kernel(NormBwdArgs a)
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const size_t cols = (size_t)a.cpr * V;
-    const float n = (float)cols;
+    const float n = RMS ? (float)a.stat : (float)cols;
     const bool param_grads = a.part_g != nullptr;
 
     // this thread's chunk columns do not depend on the row block
     const RowSlot first = locate<W, G>(0, a.rows, a.L, a.logL, wave, lane);
     uint32_t cc[K];
     bool col_live[K];
+    bool stat_full[K];  // every column of the chunk took part in the statistic
     float gam[K][V];
 #pragma unroll
     for (int k = 0; k < K; ++k) {
         cc[k] = (uint32_t)(k * W + first.w) * a.L + first.l;
         col_live[k] = cc[k] < a.cpr;
+        stat_full[k] = !RMS || (cc[k] + 1) * V <= a.stat;
 #pragma unroll
         for (int j = 0; j < V; ++j) gam[k][j] = 1.0f;
         if (col_live[k] && a.gamma != nullptr) load_params<DT>(a.gamma, a.params_f32 != 0, (size_t)cc[k] * V, gam[k]);
@@ -421,11 +447,7 @@ norm_bwd_kernel(NormBwdArgs a)
         for (int u = 0; u < kBwdU; ++u) {
             // LayerNorm: t = (s1 + xhat * s2) / n as c1 + xhat * c2 (no division per element)
             const float c1 = s1[u] / n;
-            float k2 = s2[u] / n;
-            if (RMS && a.eps_mode == 1) {
-                const float rho = 1.0f - a.eps * scale[u];
-                k2 = rho > 0.0f ? k2 / rho : 0.0f;
-            }
+            const float k2 = RMS ? rms_bwd_factor(s2[u], n, scale[u], a.eps, a.eps_mode) : s2[u] / n;
             S* dr = static_cast<S*>(a.dx) + (size_t)rs[u].row * cols;
 #pragma unroll
             for (int k = 0; k < K; ++k) {
@@ -437,7 +459,8 @@ norm_bwd_kernel(NormBwdArgs a)
                     for (int j = 0; j < V; ++j) {
                         const float xh = (fx[j] - mean[u]) * scale[u];
                         const float g = fg[j] * gam[k][j];
-                        const float t = RMS ? xh * k2 : c1 + xh * k2;
+                        float t = RMS ? xh * k2 : c1 + xh * k2;
+                        if (RMS && !stat_full[k]) t = (cc[k] * V + j < a.stat) ? t : 0.0f;
                         o[j] = scale[u] * (g - t);
                     }
                     store16_stream(dr + (size_t)cc[k] * V, float_to_chunk<DT>(o));
@@ -499,12 +522,12 @@ norm_bwd_kernel(NormBwdArgs a)
 template <int DT, bool RMS>
 __global__ void __launch_bounds__(kNormScalarThreads)
 norm_bwd_scalar_kernel(void* dx, const void* dy, const void* x, const float* mean_in, const float* rstd_in,
-                       const void* gamma, float eps, int eps_mode, uint64_t cols, int pdt)
+                       const void* gamma, float eps, int eps_mode, uint64_t cols, uint64_t stat, int pdt)
 {
     __shared__ float slots[4];
     const uint64_t row = blockIdx.x;
     const int64_t base = (int64_t)(row * cols);
-    const float n = (float)cols;
+    const float n = RMS ? (float)stat : (float)cols;
     const float mean = RMS ? 0.0f : mean_in[row];
     const float scale = rstd_in[row];
     auto gval = [&](uint64_t c) {
@@ -520,15 +543,11 @@ norm_bwd_scalar_kernel(void* dx, const void* dy, const void* x, const float* mea
     }
     s1 = block_sum_256(s1, slots);
     s2 = block_sum_256(s2, slots);
-    float k2 = s2 / n;
-    if (RMS && eps_mode == 1) {
-        const float rho = 1.0f - eps * scale;
-        k2 = rho > 0.0f ? k2 / rho : 0.0f;
-    }
+    const float k2 = RMS ? rms_bwd_factor(s2, n, scale, eps, eps_mode) : 0.0f;
     for (uint64_t c = threadIdx.x; c < cols; c += kNormScalarThreads) {
         const float xh = (Elt<DT>::load(x, base + (int64_t)c) - mean) * scale;
         const float g = Elt<DT>::load(dy, base + (int64_t)c) * gval(c);
-        const float t = RMS ? xh * k2 : (s1 + xh * s2) / n;
+        const float t = RMS ? (c < stat ? xh * k2 : 0.0f) : (s1 + xh * s2) / n;
         Elt<DT>::store(dx, base + (int64_t)c, scale * (g - t));
     }
 }
@@ -641,14 +660,14 @@ static bool param_dtype_ok(int dtype, int pdt) { return pdt == dtype || pdt == N
 
 template <int DT, bool RMS>
 static int norm_fwd(void* y, float* mean, float* rstd, const void* x, const void* gamma, const void* beta, float eps,
-                    int eps_mode, int64_t rows, int64_t cols, int pdt, hipStream_t st)
+                    int eps_mode, int64_t rows, int64_t cols, int64_t stat, int pdt, hipStream_t st)
 {
     constexpr int V = Elt<DT>::kVec;
     NormPlan p;
     const bool params_aligned = ptr_aligned16(gamma) && ptr_aligned16(beta);
     if (cols % V == 0 && ptr_aligned16(x) && ptr_aligned16(y) && params_aligned && plan_norm(cols / V, false, p)) {
         NormFwdArgs a{y, mean, rstd, x, gamma, beta, eps, eps_mode, (uint32_t)rows, (uint32_t)(cols / V),
-                      p.L, p.logL, pdt == NHP_F32 ? 1 : 0};
+                      p.L, p.logL, pdt == NHP_F32 ? 1 : 0, (uint32_t)stat};
         const int waves = p.W > 1 ? p.W : kNormBlockWaves;
         const uint32_t blocks = norm_row_blocks(rows, p, waves);
         const int threads = waves * kWave;
@@ -664,7 +683,7 @@ static int norm_fwd(void* y, float* mean, float* rstd, const void* x, const void
     }
     if (!grid_fits(rows, kNormScalarThreads)) return NHP_ERR_SHAPE;
     norm_fwd_scalar_kernel<DT, RMS><<<(uint32_t)rows, kNormScalarThreads, 0, st>>>(
-        y, mean, rstd, x, gamma, beta, eps, eps_mode, (uint64_t)cols, pdt);
+        y, mean, rstd, x, gamma, beta, eps, eps_mode, (uint64_t)cols, (uint64_t)stat, pdt);
     return launch_result();
 }
 
@@ -680,7 +699,7 @@ static int64_t norm_workspace_bytes(int64_t rows, int64_t cols, int dtype)
 template <int DT, bool RMS>
 static int norm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, const void* x, const float* mean,
                     const float* rstd, const void* gamma, void* workspace, float eps, int eps_mode, int64_t rows,
-                    int64_t cols, int pdt, hipStream_t st)
+                    int64_t cols, int64_t stat, int pdt, hipStream_t st)
 {
     constexpr int V = Elt<DT>::kVec;
     NormPlan p;
@@ -693,7 +712,7 @@ static int norm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, const v
         float* part_g = want_params ? static_cast<float*>(workspace) : nullptr;
         float* part_b = want_params ? part_g + (size_t)grid * cols : nullptr;
         NormBwdArgs a{dx, part_g, part_b, dy, x, mean, rstd, gamma, eps, eps_mode, (uint32_t)rows,
-                      (uint32_t)(cols / V), p.L, p.logL, row_blocks, pdt == NHP_F32 ? 1 : 0};
+                      (uint32_t)(cols / V), p.L, p.logL, row_blocks, pdt == NHP_F32 ? 1 : 0, (uint32_t)stat};
         const int threads = waves * kWave;
         if (!grid_fits(grid, threads)) return NHP_ERR_SHAPE;
         bool launched = false;
@@ -713,8 +732,8 @@ static int norm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, const v
         return launch_result();
     }
     if (!grid_fits(rows, kNormScalarThreads)) return NHP_ERR_SHAPE;
-    norm_bwd_scalar_kernel<DT, RMS><<<(uint32_t)rows, kNormScalarThreads, 0, st>>>(dx, dy, x, mean, rstd, gamma, eps,
-                                                                                    eps_mode, (uint64_t)cols, pdt);
+    norm_bwd_scalar_kernel<DT, RMS><<<(uint32_t)rows, kNormScalarThreads, 0, st>>>(
+        dx, dy, x, mean, rstd, gamma, eps, eps_mode, (uint64_t)cols, (uint64_t)stat, pdt);
     int rc = launch_result();
     if (rc != NHP_OK || !want_params) return rc;
     norm_param_grad_scalar_kernel<DT, RMS>
@@ -734,29 +753,34 @@ static int norm_check(int64_t rows, int64_t cols, int dtype, int pdt)
 
 template <bool RMS>
 static int norm_fwd_dispatch(void* y, float* mean, float* rstd, const void* x, const void* gamma, const void* beta,
-                             float eps, int eps_mode, int64_t rows, int64_t cols, int dtype, int pdt, void* stream)
+                             float eps, int eps_mode, int64_t rows, int64_t cols, int64_t stat, int dtype, int pdt,
+                             void* stream)
 {
     if (int rc = norm_check(rows, cols, dtype, pdt)) return rc;
+    if (RMS && (eps_mode < 0 || eps_mode > 2)) return NHP_ERR_SHAPE;
     if (rows == 0 || cols == 0) return NHP_OK;
+    if (RMS && (stat < 1 || stat > cols)) return NHP_ERR_SHAPE;
     if (!y || !x) return NHP_ERR_NULL;
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (dtype) {
     case NHP_F16:
-        return norm_fwd<NHP_F16, RMS>(y, mean, rstd, x, gamma, beta, eps, eps_mode, rows, cols, pdt, st);
+        return norm_fwd<NHP_F16, RMS>(y, mean, rstd, x, gamma, beta, eps, eps_mode, rows, cols, stat, pdt, st);
     case NHP_BF16:
-        return norm_fwd<NHP_BF16, RMS>(y, mean, rstd, x, gamma, beta, eps, eps_mode, rows, cols, pdt, st);
+        return norm_fwd<NHP_BF16, RMS>(y, mean, rstd, x, gamma, beta, eps, eps_mode, rows, cols, stat, pdt, st);
     default:
-        return norm_fwd<NHP_F32, RMS>(y, mean, rstd, x, gamma, beta, eps, eps_mode, rows, cols, pdt, st);
+        return norm_fwd<NHP_F32, RMS>(y, mean, rstd, x, gamma, beta, eps, eps_mode, rows, cols, stat, pdt, st);
     }
 }
 
 template <bool RMS>
 static int norm_bwd_dispatch(void* dx, void* dgamma, void* dbeta, const void* dy, const void* x, const float* mean,
                              const float* rstd, const void* gamma, void* workspace, float eps, int eps_mode,
-                             int64_t rows, int64_t cols, int dtype, int pdt, void* stream)
+                             int64_t rows, int64_t cols, int64_t stat, int dtype, int pdt, void* stream)
 {
     if (int rc = norm_check(rows, cols, dtype, pdt)) return rc;
+    if (RMS && (eps_mode < 0 || eps_mode > 2)) return NHP_ERR_SHAPE;
     if (rows == 0 || cols == 0) return NHP_OK;
+    if (RMS && (stat < 1 || stat > cols)) return NHP_ERR_SHAPE;
     if (!dx || !dy || !x || !rstd || (!RMS && !mean)) return NHP_ERR_NULL;
     if ((dgamma != nullptr || dbeta != nullptr) && workspace == nullptr && norm_workspace_bytes(rows, cols, dtype) > 0)
         return NHP_ERR_NULL;
@@ -764,13 +788,13 @@ static int norm_bwd_dispatch(void* dx, void* dgamma, void* dbeta, const void* dy
     switch (dtype) {
     case NHP_F16:
         return norm_bwd<NHP_F16, RMS>(dx, dgamma, dbeta, dy, x, mean, rstd, gamma, workspace, eps, eps_mode, rows,
-                                      cols, pdt, st);
+                                      cols, stat, pdt, st);
     case NHP_BF16:
         return norm_bwd<NHP_BF16, RMS>(dx, dgamma, dbeta, dy, x, mean, rstd, gamma, workspace, eps, eps_mode, rows,
-                                       cols, pdt, st);
+                                       cols, stat, pdt, st);
     default:
         return norm_bwd<NHP_F32, RMS>(dx, dgamma, dbeta, dy, x, mean, rstd, gamma, workspace, eps, eps_mode, rows,
-                                      cols, pdt, st);
+                                      cols, stat, pdt, st);
     }
 }
 
@@ -783,7 +807,8 @@ extern "C" {
 int nhp_layernorm_fwd(void* y, float* mean, float* rstd, const void* x, const void* gamma, const void* beta,
                       float eps, int64_t rows, int64_t cols, int dtype, int param_dtype, void* stream)
 {
-    return norm_fwd_dispatch<false>(y, mean, rstd, x, gamma, beta, eps, 0, rows, cols, dtype, param_dtype, stream);
+    return norm_fwd_dispatch<false>(y, mean, rstd, x, gamma, beta, eps, 0, rows, cols, cols, dtype, param_dtype,
+                                    stream);
 }
 
 int nhp_layernorm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, const void* x, const float* mean,
@@ -791,24 +816,38 @@ int nhp_layernorm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, const
                       int param_dtype, void* stream)
 {
     return norm_bwd_dispatch<false>(dx, dgamma, dbeta, dy, x, mean, rstd, gamma, workspace, 0.0f, 0, rows, cols,
-                                    dtype, param_dtype, stream);
+                                    cols, dtype, param_dtype, stream);
 }
 
 int nhp_rmsnorm_fwd(void* y, float* inv, const void* x, const void* scale, const void* offset, float eps,
                     int eps_mode, int64_t rows, int64_t cols, int dtype, int param_dtype, void* stream)
 {
-    if (eps_mode != 0 && eps_mode != 1) return NHP_ERR_SHAPE;
-    return norm_fwd_dispatch<true>(y, nullptr, inv, x, scale, offset, eps, eps_mode, rows, cols, dtype, param_dtype,
-                                   stream);
+    return norm_fwd_dispatch<true>(y, nullptr, inv, x, scale, offset, eps, eps_mode, rows, cols, cols, dtype,
+                                   param_dtype, stream);
+}
+
+int nhp_rmsnorm_partial_fwd(void* y, float* inv, const void* x, const void* scale, const void* offset, float eps,
+                            int eps_mode, int64_t rows, int64_t cols, int64_t stat_cols, int dtype, int param_dtype,
+                            void* stream)
+{
+    return norm_fwd_dispatch<true>(y, nullptr, inv, x, scale, offset, eps, eps_mode, rows, cols, stat_cols, dtype,
+                                   param_dtype, stream);
 }
 
 int nhp_rmsnorm_bwd(void* dx, void* dscale, void* doffset, const void* dy, const void* x, const float* inv,
                     const void* scale, void* workspace, float eps, int eps_mode, int64_t rows, int64_t cols,
                     int dtype, int param_dtype, void* stream)
 {
-    if (eps_mode != 0 && eps_mode != 1) return NHP_ERR_SHAPE;
     return norm_bwd_dispatch<true>(dx, dscale, doffset, dy, x, nullptr, inv, scale, workspace, eps, eps_mode, rows,
-                                   cols, dtype, param_dtype, stream);
+                                   cols, cols, dtype, param_dtype, stream);
+}
+
+int nhp_rmsnorm_partial_bwd(void* dx, void* dscale, void* doffset, const void* dy, const void* x, const float* inv,
+                            const void* scale, void* workspace, float eps, int eps_mode, int64_t rows, int64_t cols,
+                            int64_t stat_cols, int dtype, int param_dtype, void* stream)
+{
+    return norm_bwd_dispatch<true>(dx, dscale, doffset, dy, x, nullptr, inv, scale, workspace, eps, eps_mode, rows,
+                                   cols, stat_cols, dtype, param_dtype, stream);
 }
 
 int64_t nhp_norm_bwd_workspace_bytes(int64_t rows, int64_t cols, int dtype)

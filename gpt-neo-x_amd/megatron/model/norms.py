@@ -1,9 +1,9 @@
 """LayerNorm and RMSNorm on MI355X.
 
 Surface of GPT-NeoX's ``megatron/model/norms.py``: ``get_norm`` (:19-51),
-``LayerNorm`` (:16, torch's class there) and ``RMSNorm`` (:54-107), with the same
-constructor arguments and parameter names (``weight`` / ``bias``, ``scale`` /
-``offset``). Forward and backward are hand-written gfx950 kernels
+``LayerNorm`` (:16, torch's class there), ``RMSNorm`` (:54-107, partial variant
+included) and ``ScaleNorm`` (:110-119), with the same constructor arguments and
+parameter names (``weight`` / ``bias``, ``scale`` / ``offset``, ``g``). Forward and backward are hand-written gfx950 kernels
 (libneox_hotpath.so): one pass over the row for the forward, one for the
 backward including the parameter gradients. Statistics and arithmetic are fp32
 and the result is rounded once, which is what torch's LayerNorm kernel and the
@@ -11,7 +11,7 @@ fused RMSNorm variants do; the Python ``RMSNorm`` of the reference, run eagerly
 on 16-bit tensors, rounds after every operator and so differs by a few units in
 the last place.
 
-Not provided: partial RMSNorm (``p`` in [0, 1]) and ``ScaleNorm``.
+Not provided: the Transformer Engine classes (``te_rmsnorm``, ``te_layernorm``).
 """
 import numbers
 
@@ -133,7 +133,7 @@ class LayerNorm(torch.nn.Module):
 
 class _RMSNormFunction(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, scale, offset, eps, eps_mode):
+    def forward(ctx, x, scale, offset, eps, eps_mode, stat_cols=None):
         what = "RMSNorm"
         _hp.require_gpu(x, what)
         cols = x.size(-1)
@@ -144,13 +144,15 @@ class _RMSNormFunction(torch.autograd.Function):
         y = torch.empty_like(src)
         inv = torch.empty(rows, dtype=torch.float32, device=src.device)
         code, pcode = _hp.dtype_code(src, what), _param_code(src, scale, offset)
+        stat = cols if stat_cols is None else int(stat_cols)
         with _hp.device_guard(src):
-            rc = _hp.lib().nhp_rmsnorm_fwd(y.data_ptr(), inv.data_ptr(), src.data_ptr(), _ptr(scale), _ptr(offset),
-                                           float(eps), int(eps_mode), rows, cols, code, pcode, _hp.stream_of(src))
+            rc = _hp.lib().nhp_rmsnorm_partial_fwd(y.data_ptr(), inv.data_ptr(), src.data_ptr(), _ptr(scale),
+                                                   _ptr(offset), float(eps), int(eps_mode), rows, cols, stat, code,
+                                                   pcode, _hp.stream_of(src))
         _hp.check(rc, what)
         ctx.save_for_backward(src, scale, inv)
         ctx.has_offset = offset is not None
-        ctx.conf = (code, pcode, float(eps), int(eps_mode))
+        ctx.conf = (code, pcode, float(eps), int(eps_mode), stat)
         return y
 
     @staticmethod
@@ -160,7 +162,7 @@ class _RMSNormFunction(torch.autograd.Function):
         g = grad.contiguous()
         cols = src.size(-1)
         rows = src.numel() // max(cols, 1)
-        code, pcode, eps, eps_mode = ctx.conf
+        code, pcode, eps, eps_mode, stat = ctx.conf
         want_s = scale is not None and ctx.needs_input_grad[1]
         want_o = ctx.has_offset and ctx.needs_input_grad[2]
         pdtype = scale.dtype if scale is not None else (torch.float32 if pcode == _hp.F32 else src.dtype)
@@ -169,27 +171,33 @@ class _RMSNormFunction(torch.autograd.Function):
         do = torch.empty(cols, dtype=pdtype, device=src.device) if want_o else None
         ws = _workspace(rows, cols, code, src.device) if (want_s or want_o) else None
         with _hp.device_guard(src):
-            rc = _hp.lib().nhp_rmsnorm_bwd(dx.data_ptr(), _ptr(ds), _ptr(do), g.data_ptr(), src.data_ptr(),
-                                           inv.data_ptr(), _ptr(scale), _ptr(ws), eps, eps_mode, rows, cols, code,
-                                           pcode, _hp.stream_of(src))
+            rc = _hp.lib().nhp_rmsnorm_partial_bwd(dx.data_ptr(), _ptr(ds), _ptr(do), g.data_ptr(), src.data_ptr(),
+                                                   inv.data_ptr(), _ptr(scale), _ptr(ws), eps, eps_mode, rows, cols,
+                                                   stat, code, pcode, _hp.stream_of(src))
         _hp.check(rc, what)
         if rows == 0:
             ds = None if ds is None else ds.zero_()
             do = None if do is None else do.zero_()
-        return dx, ds, do, None, None
+        return dx, ds, do, None, None, None
 
 
 class RMSNorm(torch.nn.Module):
     """Root-mean-square normalisation, ``scale * x / (rms(x) + eps) [+ offset]``
-    (the reference's Python class, megatron/model/norms.py:54-107).
+    (the reference's Python class, megatron/model/norms.py:54-107). With
+    ``0 <= p <= 1`` the rms is taken over the first ``int(dim * p)`` features only
+    (partial RMSNorm, :87-94).
 
     ``fused_eps=True`` selects the other definition the reference knows,
     ``scale * x * rsqrt(mean(x^2) + eps)`` (MixedFusedRMSNorm)."""
 
     def __init__(self, dim, p=-1.0, eps=1e-8, bias=False, fused_eps=False):
         super().__init__()
+        self.partial_size = None
         if 0.0 <= p <= 1.0:
-            raise NotImplementedError("partial RMSNorm (p in [0, 1]) is not provided by the MI355X kernels")
+            self.partial_size = int(dim * p)
+            if self.partial_size < 1:
+                # the reference divides by zero here (0 ** -0.5)
+                raise ZeroDivisionError(f"partial RMSNorm: int({dim} * {p}) = 0 features to take the rms of")
         self.eps = eps
         self.d = dim
         self.p = p
@@ -204,20 +212,42 @@ class RMSNorm(torch.nn.Module):
     def forward(self, x):
         if x.size(-1) != self.d:
             raise RuntimeError(f"RMSNorm: expected last dimension {self.d}, got {x.size(-1)}")
-        return _RMSNormFunction.apply(x, self.scale, self.offset, self.eps, 0 if self.fused_eps else 1)
+        return _RMSNormFunction.apply(x, self.scale, self.offset, self.eps, 0 if self.fused_eps else 1,
+                                      self.partial_size)
 
 
-class _FusedRMSNorm(RMSNorm):
-    def __init__(self, dim, eps=1e-5, **_):
-        super().__init__(dim, eps=eps, fused_eps=True)
+class ScaleNorm(torch.nn.Module):
+    """``x / clamp(||x||_2, min=eps) * g`` with one learned scalar ``g``
+    (megatron/model/norms.py:110-119). Runs on the RMSNorm kernels: the scalar is
+    handed over as a vector of equal values, and its gradient is the sum of that
+    vector's gradient (autograd does both through ``expand``)."""
+
+    def __init__(self, dim, eps=1e-5):
+        super().__init__()
+        self.g = torch.nn.Parameter(torch.ones(1))
+        self.eps = eps
+
+    def forward(self, x):
+        g = self.g if self.g.dtype in (x.dtype, torch.float32) else self.g.to(x.dtype)
+        return _RMSNormFunction.apply(x, g.expand(x.size(-1)), None, self.eps, 2, None)
 
 
 def get_norm(neox_args):
-    """(norm class, eps) for ``neox_args.norm`` in {"layernorm", "rmsnorm"}; the ``*_fusion`` flags pick
-    the fused definition of the epsilon for RMSNorm and change nothing for LayerNorm."""
+    """(norm class, eps) for ``neox_args.norm`` in {"layernorm", "rmsnorm", "scalenorm"}
+    (megatron/model/norms.py:19-51); the ``*_fusion`` flags select the classes of
+    ``fused_layer_norm``, which run on the same kernels."""
     if neox_args.norm == "rmsnorm":
-        norm = _FusedRMSNorm if getattr(neox_args, "rmsnorm_fusion", False) else RMSNorm
-        return norm, neox_args.rms_norm_epsilon
+        if getattr(neox_args, "rmsnorm_fusion", False):
+            from .fused_layer_norm import MixedFusedRMSNorm
+
+            return MixedFusedRMSNorm, neox_args.rms_norm_epsilon
+        return RMSNorm, neox_args.rms_norm_epsilon
     if neox_args.norm == "layernorm":
+        if getattr(neox_args, "layernorm_fusion", False):
+            from .fused_layer_norm import MixedFusedLayerNorm
+
+            return MixedFusedLayerNorm, neox_args.layernorm_epsilon
         return LayerNorm, neox_args.layernorm_epsilon
+    if neox_args.norm == "scalenorm":
+        return ScaleNorm, neox_args.scalenorm_epsilon
     raise ValueError(f"norm {neox_args.norm} not provided by the MI355X kernels")

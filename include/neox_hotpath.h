@@ -448,7 +448,10 @@ int nhp_layernorm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, const
  *   eps_mode 1: inv = 1 / (||x||_2 * cols^(-1/2) + eps), the Python class
  *               RMSNorm.forward, megatron/model/norms.py:54-107 (p disabled);
  *   eps_mode 0: inv = 1 / sqrt(mean(x^2) + eps), the fused variants
- *               MixedFusedRMSNorm, megatron/model/fused_layer_norm.py:156-252.
+ *               MixedFusedRMSNorm, megatron/model/fused_layer_norm.py:156-252;
+ *   eps_mode 2: inv = 1 / max(||x||_2, eps), ScaleNorm.forward,
+ *               megatron/model/norms.py:110-119 (its scalar g is passed as a
+ *               `scale` vector of cols equal values).
  */
 int nhp_rmsnorm_fwd(void* y, float* inv, const void* x, const void* scale, const void* offset,
                     float eps, int eps_mode,
@@ -457,14 +460,30 @@ int nhp_rmsnorm_fwd(void* y, float* inv, const void* x, const void* scale, const
 /*
  * xhat = x * inv, g = dy * scale, s = sum(g * xhat):
  *   dx = inv * (g - xhat * s / (cols * rho)), rho = 1 (eps_mode 0) or 1 - eps * inv (eps_mode 1;
- *   rho <= 0, an all-zero row, drops the second term);
+ *   rho <= 0, an all-zero row, drops the second term); eps_mode 2: dx = inv * (g - xhat * s)
+ *   while ||x|| > eps (inv < 1 / eps), dx = inv * g for a clamped norm;
  *   dscale = column sums of dy * xhat, doffset = column sums of dy (each optional).
  * The adjoint of nhp_rmsnorm_fwd, i.e. what autograd runs for RMSNorm.forward
- *   (megatron/model/norms.py:85-107).
+ *   (megatron/model/norms.py:85-107) and ScaleNorm.forward (:117-119).
  */
 int nhp_rmsnorm_bwd(void* dx, void* dscale, void* doffset, const void* dy, const void* x,
                     const float* inv, const void* scale, void* workspace, float eps, int eps_mode,
                     int64_t rows, int64_t cols, int dtype, int param_dtype, void* stream);
+
+/*
+ * Partial RMSNorm (the `p` argument of RMSNorm, megatron/model/norms.py:87-94):
+ * the statistic is taken over the first stat_cols columns of a row
+ * (1 <= stat_cols <= cols; `cols` in the formulas above becomes stat_cols),
+ * every column is scaled by it. In the backward the xhat * s term reaches
+ * only the columns that took part in the statistic.
+ */
+int nhp_rmsnorm_partial_fwd(void* y, float* inv, const void* x, const void* scale,
+                            const void* offset, float eps, int eps_mode, int64_t rows, int64_t cols,
+                            int64_t stat_cols, int dtype, int param_dtype, void* stream);
+int nhp_rmsnorm_partial_bwd(void* dx, void* dscale, void* doffset, const void* dy, const void* x,
+                            const float* inv, const void* scale, void* workspace, float eps,
+                            int eps_mode, int64_t rows, int64_t cols, int64_t stat_cols, int dtype,
+                            int param_dtype, void* stream);
 
 int64_t nhp_norm_bwd_workspace_bytes(int64_t rows, int64_t cols, int dtype);
 

@@ -66,8 +66,8 @@ def lib():
         L.oracle_gated_act_bwd.argtypes = [vp, vp, vp, vp, i64, i64, ci, ci]
         L.oracle_layernorm_fwd.argtypes = [vp, vp, vp, vp, vp, vp, f32, i64, i64, ci, ci]
         L.oracle_layernorm_bwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, ci, ci]
-        L.oracle_rmsnorm_fwd.argtypes = [vp, vp, vp, vp, vp, f32, ci, i64, i64, ci, ci]
-        L.oracle_rmsnorm_bwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, f32, ci, i64, i64, ci, ci]
+        L.oracle_rmsnorm_fwd.argtypes = [vp, vp, vp, vp, vp, f32, ci, i64, i64, i64, ci, ci]
+        L.oracle_rmsnorm_bwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, f32, ci, i64, i64, i64, ci, ci]
         p64 = ctypes.POINTER(i64)
         L.oracle_rope_cached.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, p64, p64, ci, ci, ci]
         L.oracle_rope_freqs.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, p64, p64, ci, ci]
@@ -312,8 +312,9 @@ def layernorm_bwd(dy, x, mean, rstd, gamma=None, param_dtype=None):
     return dx, dg, db
 
 
-def rmsnorm_fwd(x, scale=None, offset=None, eps=1e-8, eps_mode=1):
-    """Returns (y, inv). eps_mode 1: x / (rms + eps) (the Python RMSNorm class); 0: x * rsqrt(mean(x^2) + eps)."""
+def rmsnorm_fwd(x, scale=None, offset=None, eps=1e-8, eps_mode=1, stat_cols=None):
+    """Returns (y, inv). eps_mode 1: x / (rms + eps) (the Python RMSNorm class); 0: x * rsqrt(mean(x^2) + eps);
+    2: x / max(||x||, eps) (ScaleNorm). stat_cols: leading columns the statistic is taken over (default: all)."""
     x = _cpu_contig(x)
     rows, cols = _rows_cols(x)
     y = torch.empty_like(x)
@@ -321,11 +322,12 @@ def rmsnorm_fwd(x, scale=None, offset=None, eps=1e-8, eps_mode=1):
     scale, sp, sc = _param(scale, x)
     offset, op, oc = _param(offset, x)
     _check(lib().oracle_rmsnorm_fwd(y.data_ptr(), inv.data_ptr(), x.data_ptr(), sp, op, float(eps), int(eps_mode),
-                                    rows, cols, _DT[x.dtype], _param_code(x, sc, oc)), "rmsnorm_fwd")
+                                    rows, cols, cols if stat_cols is None else int(stat_cols), _DT[x.dtype],
+                                    _param_code(x, sc, oc)), "rmsnorm_fwd")
     return y, inv
 
 
-def rmsnorm_bwd(dy, x, inv, scale=None, eps=1e-8, eps_mode=1, param_dtype=None):
+def rmsnorm_bwd(dy, x, inv, scale=None, eps=1e-8, eps_mode=1, param_dtype=None, stat_cols=None):
     """Returns (dx, dscale, doffset)."""
     x = _cpu_contig(x)
     dy = _cpu_contig(dy)
@@ -337,8 +339,9 @@ def rmsnorm_bwd(dy, x, inv, scale=None, eps=1e-8, eps_mode=1, param_dtype=None):
     do = torch.empty(cols, dtype=pdt)
     inv = _cpu_contig(inv.float())
     _check(lib().oracle_rmsnorm_bwd(dx.data_ptr(), ds.data_ptr(), do.data_ptr(), dy.data_ptr(), x.data_ptr(),
-                                    inv.data_ptr(), sp, float(eps), int(eps_mode), rows, cols, _DT[x.dtype],
-                                    _DT[pdt]), "rmsnorm_bwd")
+                                    inv.data_ptr(), sp, float(eps), int(eps_mode), rows, cols,
+                                    cols if stat_cols is None else int(stat_cols), _DT[x.dtype], _DT[pdt]),
+           "rmsnorm_bwd")
     return dx, ds, do
 
 

@@ -225,31 +225,42 @@ int oracle_layernorm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, co
 }
 
 /*
- * RMSNorm. Two definitions live in the reference, selected here by eps_mode:
- *   1: the Python class megatron/model/norms.py:54-107 (p disabled):
- *        rms = ||x||_2 * cols^(-1/2);  y = scale * (x / (rms + eps)) [+ offset]
+ * RMSNorm and ScaleNorm. Three definitions live in the reference, selected here by eps_mode:
+ *   1: the Python class RMSNorm, megatron/model/norms.py:54-107:
+ *        rms = ||x[:stat]||_2 * stat^(-1/2);  y = scale * (x / (rms + eps)) [+ offset]
+ *      stat = cols, or int(cols * p) leading columns for the partial variant (:87-94)
  *   0: the fused variants (MixedFusedRMSNorm, megatron/model/fused_layer_norm.py:156-252,
  *      backed by apex, and TERMSNorm): y = scale * (x * rsqrt(mean(x^2) + eps))
+ *   2: ScaleNorm, megatron/model/norms.py:110-119: y = x / max(||x||_2, eps) * g; the
+ *      scalar g arrives as a scale vector of equal values
  * fp32 arithmetic, one rounding of y. inv: fp32 [rows], the factor x is
- * multiplied by (1 / (rms + eps) or rsqrt(mean(x^2) + eps)).
+ * multiplied by.
  */
-static float rms_inverse(float sumsq, int64_t cols, float eps, int eps_mode)
+static float rms_inverse(float sumsq, int64_t stat, float eps, int eps_mode)
 {
-    if (eps_mode == 1) return 1.0f / (sqrtf(sumsq) * (1.0f / sqrtf((float)cols)) + eps);
-    return 1.0f / sqrtf(sumsq / (float)cols + eps);
+    if (eps_mode == 2) {
+        const float nrm = sqrtf(sumsq);
+        return 1.0f / (nrm > eps ? nrm : eps);
+    }
+    if (eps_mode == 1) return 1.0f / (sqrtf(sumsq) * (1.0f / sqrtf((float)stat)) + eps);
+    return 1.0f / sqrtf(sumsq / (float)stat + eps);
 }
 
 int oracle_rmsnorm_fwd(void* y, float* inv, const void* x, const void* scale, const void* offset, float eps,
-                       int eps_mode, int64_t rows, int64_t cols, int dt, int pdt)
+                       int eps_mode, int64_t rows, int64_t cols, int64_t stat, int dt, int pdt)
 {
     float* v = (float*)malloc(sizeof(float) * (size_t)(cols > 0 ? cols : 1));
     if (!v) return -2;
+    if (stat < 1 || stat > cols) {
+        free(v);
+        return -1;
+    }
     for (int64_t r = 0; r < rows; ++r) {
-        for (int64_t c = 0; c < cols; ++c) {
+        for (int64_t c = 0; c < stat; ++c) {
             const float f = load_elem(x, r * cols + c, dt);
             v[c] = f * f;
         }
-        const float iv = rms_inverse(pairwise_sum(v, cols), cols, eps, eps_mode);
+        const float iv = rms_inverse(pairwise_sum(v, stat), stat, eps, eps_mode);
         for (int64_t c = 0; c < cols; ++c) {
             float o = load_elem(x, r * cols + c, dt) * iv;
             if (scale) o = load_param(scale, c, pdt) * o;
@@ -263,16 +274,21 @@ int oracle_rmsnorm_fwd(void* y, float* inv, const void* x, const void* scale, co
 }
 
 /*
- * Backward of RMSNorm: with xhat = x * inv, g = dy * scale, s = sum(g * xhat),
- *   eps_mode 0: dx = inv * (g - xhat * s / cols)
- *   eps_mode 1: dx = inv * (g - xhat * s / (cols * rho)), rho = rms / (rms + eps) = 1 - eps * inv
+ * Backward of RMSNorm: with xhat = x * inv, g = dy * scale, s = sum over all columns of g * xhat,
+ * and m[c] = 1 for the columns c < stat the statistic was taken over, else 0:
+ *   eps_mode 0: dx = inv * (g - m * xhat * s / stat)
+ *   eps_mode 1: dx = inv * (g - m * xhat * s / (stat * rho)), rho = rms / (rms + eps) = 1 - eps * inv
  *               (rho = 0, an all-zero row with eps > 0: the second term is 0, as
  *               torch's norm backward defines it)
+ *   eps_mode 2: dx = inv * (g - xhat * s) while ||x|| > eps (inv < 1 / eps); a clamped norm
+ *               is a constant: dx = inv * g
  *   dscale[c] = sum over rows of dy * xhat, doffset[c] = sum over rows of dy.
  */
 int oracle_rmsnorm_bwd(void* dx, void* dscale, void* doffset, const void* dy, const void* x, const float* inv,
-                       const void* scale, float eps, int eps_mode, int64_t rows, int64_t cols, int dt, int pdt)
+                       const void* scale, float eps, int eps_mode, int64_t rows, int64_t cols, int64_t stat, int dt,
+                       int pdt)
 {
+    if (stat < 1 || stat > cols) return -1;
     const size_t n = (size_t)(cols > 0 ? cols : 1);
     float* g = (float*)malloc(sizeof(float) * n);
     float* gx = (float*)malloc(sizeof(float) * n);
@@ -291,14 +307,17 @@ int oracle_rmsnorm_bwd(void* dx, void* dscale, void* doffset, const void* dy, co
                 gx[c] = g[c] * xh;
             }
             const float s = pairwise_sum(gx, cols);
-            float k = s / (float)cols;
+            float k = s / (float)stat;
             if (eps_mode == 1) {
                 const float rho = 1.0f - eps * inv[r];
                 k = rho > 0.0f ? k / rho : 0.0f;
+            } else if (eps_mode == 2) {
+                k = inv[r] < 1.0f / eps ? s : 0.0f;
             }
             for (int64_t c = 0; c < cols; ++c) {
                 const float xh = load_elem(x, r * cols + c, dt) * inv[r];
-                store_elem(dx, r * cols + c, dt, inv[r] * (g[c] - xh * k));
+                const float t = c < stat ? xh * k : 0.0f;
+                store_elem(dx, r * cols + c, dt, inv[r] * (g[c] - t));
             }
         }
     for (int64_t c = 0; c < cols; ++c) {

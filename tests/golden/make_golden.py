@@ -113,6 +113,14 @@ def main():
             rdx, rds, rdo = oracle.rmsnorm_bwd(dy, x, inv, gamma, eps, mode)
             put(name, **{f"rms{mode}_y": ry, f"rms{mode}_inv": inv, f"rms{mode}_dx": rdx, f"rms{mode}_dscale": rds,
                          f"rms{mode}_doffset": rdo, f"rms{mode}_eps": np.float32(eps)})
+        # partial RMSNorm (statistic over the first 7 of 24 columns) and ScaleNorm (g = 1.25)
+        py, pinv = oracle.rmsnorm_fwd(x, gamma, beta, 1e-2, 1, stat_cols=7)
+        pdx, pds, pdo = oracle.rmsnorm_bwd(dy, x, pinv, gamma, 1e-2, 1, stat_cols=7)
+        gvec = torch.full((24,), 1.25, dtype=dtype)
+        sy, sinv = oracle.rmsnorm_fwd(x, gvec, None, 1e-2, 2)
+        sdx, sds, _ = oracle.rmsnorm_bwd(dy, x, sinv, gvec, 1e-2, 2)
+        put(name, part_y=py, part_inv=pinv, part_dx=pdx, part_dscale=pds, part_doffset=pdo, sn_y=sy, sn_inv=sinv,
+            sn_dx=sdx, sn_dscale=sds)
 
     for name, dtype, seed in (("gated_bf16", torch.bfloat16, 41), ("gated_fp16", torch.float16, 42),
                               ("gated_fp32", torch.float32, 43)):

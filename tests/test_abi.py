@@ -148,7 +148,11 @@ def test_argument_validation_of_the_layer_entry_points(hotpath):
     assert lib.nhp_layernorm_fwd(null, null, null, null, null, null, 1e-5, 4, 0, BF16, BF16, None) == 0
     assert lib.nhp_layernorm_bwd(q, null, null, p, p, null, p, p, null, 4, 8, BF16, BF16, None) == -3   # mean missing
     assert lib.nhp_layernorm_bwd(q, p, null, p, p, p, p, p, null, 4, 8, BF16, BF16, None) == -3          # workspace missing
-    assert lib.nhp_rmsnorm_fwd(q, null, p, p, null, 1e-5, 2, 4, 8, BF16, BF16, None) == -2               # eps_mode
+    assert lib.nhp_rmsnorm_fwd(q, null, p, p, null, 1e-5, 3, 4, 8, BF16, BF16, None) == -2               # eps_mode
+    assert lib.nhp_rmsnorm_partial_fwd(q, null, p, p, null, 1e-5, 1, 4, 8, 0, BF16, BF16, None) == -2    # no statistic columns
+    assert lib.nhp_rmsnorm_partial_fwd(q, null, p, p, null, 1e-5, 1, 4, 8, 9, BF16, BF16, None) == -2    # more than the row has
+    assert lib.nhp_rmsnorm_partial_fwd(q, null, null, p, null, 1e-5, 1, 4, 8, 3, BF16, BF16, None) == -3
+    assert lib.nhp_rmsnorm_partial_bwd(q, null, null, p, p, p, p, null, 1e-5, 1, 4, 8, 9, BF16, BF16, None) == -2
     assert lib.nhp_rmsnorm_bwd(q, null, null, p, p, null, p, null, 1e-5, 1, 4, 8, BF16, BF16, None) == -3  # inv missing
     assert lib.nhp_rmsnorm_bwd(q, null, null, p, p, p, p, null, 1e-5, 3, 4, 8, BF16, BF16, None) == -2
     assert lib.nhp_norm_bwd_workspace_bytes(4, 8, BF16) > 0

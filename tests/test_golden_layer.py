@@ -13,7 +13,7 @@ import util
 
 GOLDEN = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "layer_golden.npz"))
 DT = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}
-FP32_KEYS = ("slopes", "ln_mean", "ln_rstd", "rms0_inv", "rms1_inv")
+FP32_KEYS = ("slopes", "ln_mean", "ln_rstd", "rms0_inv", "rms1_inv", "part_inv", "sn_inv")
 
 
 def get(prefix, key):
@@ -69,6 +69,15 @@ def test_oracle_reproduces_norm_golden(name):
         rdx, rds, rdo = oracle.rmsnorm_bwd(dy, x, inv, gamma, eps, mode)
         assert same(rdx, get(name, f"rms{mode}_dx")) and same(rds, get(name, f"rms{mode}_dscale"))
         assert same(rdo, get(name, f"rms{mode}_doffset"))
+    py, pinv = oracle.rmsnorm_fwd(x, gamma, beta, 1e-2, 1, stat_cols=7)
+    assert same(py, get(name, "part_y")) and same(pinv, get(name, "part_inv"))
+    pdx, pds, pdo = oracle.rmsnorm_bwd(dy, x, pinv, gamma, 1e-2, 1, stat_cols=7)
+    assert same(pdx, get(name, "part_dx")) and same(pds, get(name, "part_dscale")) and same(pdo, get(name, "part_doffset"))
+    gvec = torch.full((24,), 1.25, dtype=x.dtype)
+    sy, sinv = oracle.rmsnorm_fwd(x, gvec, None, 1e-2, 2)
+    assert same(sy, get(name, "sn_y")) and same(sinv, get(name, "sn_inv"))
+    sdx, sds, _ = oracle.rmsnorm_bwd(dy, x, sinv, gvec, 1e-2, 2)
+    assert same(sdx, get(name, "sn_dx")) and same(sds, get(name, "sn_dscale"))
 
 
 GATED = ["gated_bf16", "gated_fp16", "gated_fp32"]
@@ -217,3 +226,26 @@ def test_gpu_matches_norm_golden(hotpath, name):
         util.assert_close_ulp_or_noise(dx.cpu(), get(name, f"rms{mode}_dx"), 2, dx_noise(gi.cpu()), name)
         util.assert_close_ulp_or_noise(dg.cpu(), get(name, f"rms{mode}_dscale"), 2, col, name)
         util.assert_close_ulp_or_noise(db.cpu(), get(name, f"rms{mode}_doffset"), 2, col, name)
+    # partial RMSNorm and ScaleNorm
+    inv = torch.empty(rows, device="cuda")
+    assert L.nhp_rmsnorm_partial_fwd(y.data_ptr(), inv.data_ptr(), x.data_ptr(), gamma.data_ptr(), beta.data_ptr(), 1e-2, 1,
+                                     rows, cols, 7, code, code, None) == 0
+    grow = (get(name, "x").float().abs() * get(name, "part_inv")[:, None]).clamp(min=1.0)
+    util.assert_close_ulp_or_noise(y.cpu(), get(name, "part_y"), 2, noise_y * grow, name)
+    gi = get(name, "part_inv").cuda()
+    assert torch.allclose(inv.cpu(), gi.cpu(), rtol=1e-5, atol=0)
+    assert L.nhp_rmsnorm_partial_bwd(dx.data_ptr(), dg.data_ptr(), db.data_ptr(), dy.data_ptr(), x.data_ptr(), gi.data_ptr(),
+                                     gamma.data_ptr(), ws.data_ptr(), 1e-2, 1, rows, cols, 7, code, code, None) == 0
+    util.assert_close_ulp_or_noise(dx.cpu(), get(name, "part_dx"), 2, dx_noise(gi.cpu()) * grow * cols / 7, name)
+    util.assert_close_ulp_or_noise(dg.cpu(), get(name, "part_dscale"), 2, col * grow.amax(0), name)
+    util.assert_close_ulp_or_noise(db.cpu(), get(name, "part_doffset"), 2, col, name)
+    gvec = torch.full((cols,), 1.25, dtype=x.dtype, device="cuda")
+    assert L.nhp_rmsnorm_fwd(y.data_ptr(), inv.data_ptr(), x.data_ptr(), gvec.data_ptr(), None, 1e-2, 2, rows, cols, code,
+                             code, None) == 0
+    util.assert_close_ulp_or_noise(y.cpu(), get(name, "sn_y"), 2, noise_y, name)
+    gi = get(name, "sn_inv").cuda()
+    assert torch.allclose(inv.cpu(), gi.cpu(), rtol=1e-5, atol=0)
+    assert L.nhp_rmsnorm_bwd(dx.data_ptr(), dg.data_ptr(), None, dy.data_ptr(), x.data_ptr(), gi.data_ptr(), gvec.data_ptr(),
+                             ws.data_ptr(), 1e-2, 2, rows, cols, code, code, None) == 0
+    util.assert_close_ulp_or_noise(dx.cpu(), get(name, "sn_dx"), 2, dx_noise(gi.cpu()) * 2, name)
+    util.assert_close_ulp_or_noise(dg.cpu(), get(name, "sn_dscale"), 2, col, name)

@@ -53,7 +53,9 @@ def abi_layernorm(hp, x, dy, gamma, beta, eps, want_params=True):
     return y, mean, rstd, dx, dg, db
 
 
-def abi_rmsnorm(hp, x, dy, scale, offset, eps, mode):
+def abi_rmsnorm(hp, x, dy, scale, offset, eps, mode, stat=None):
+    if stat is not None:
+        return abi_rmsnorm_partial(hp, x, dy, scale, offset, eps, mode, stat)
     rows, cols = x.shape
     code, pcode = hp.dtype_code(x, "t"), hp._DTYPE[(scale if scale is not None else x).dtype]
     y = torch.empty_like(x)
@@ -69,6 +71,27 @@ def abi_rmsnorm(hp, x, dy, scale, offset, eps, mode):
     ws = torch.empty(max(L.nhp_norm_bwd_workspace_bytes(rows, cols, code), 1), dtype=torch.uint8, device=x.device)
     rc = L.nhp_rmsnorm_bwd(dx.data_ptr(), ds.data_ptr(), do.data_ptr(), dy.data_ptr(), x.data_ptr(), inv.data_ptr(),
                            ptr(scale), ws.data_ptr(), eps, mode, rows, cols, code, pcode, None)
+    assert rc == 0, L.nhp_status_string(rc)
+    return y, inv, dx, ds, do
+
+
+def abi_rmsnorm_partial(hp, x, dy, scale, offset, eps, mode, stat):
+    rows, cols = x.shape
+    code, pcode = hp.dtype_code(x, "t"), hp._DTYPE[(scale if scale is not None else x).dtype]
+    y = torch.empty_like(x)
+    inv = torch.empty(rows, dtype=torch.float32, device=x.device)
+    L = hp.lib()
+    rc = L.nhp_rmsnorm_partial_fwd(y.data_ptr(), inv.data_ptr(), x.data_ptr(), ptr(scale), ptr(offset), eps, mode, rows,
+                                   cols, stat, code, pcode, None)
+    assert rc == 0, L.nhp_status_string(rc)
+    dx = torch.empty_like(x)
+    pd = scale.dtype if scale is not None else x.dtype
+    ds = torch.full((cols,), float("nan"), dtype=pd, device=x.device)
+    do = torch.full((cols,), float("nan"), dtype=pd, device=x.device)
+    ws = torch.empty(max(L.nhp_norm_bwd_workspace_bytes(rows, cols, code), 1), dtype=torch.uint8, device=x.device)
+    rc = L.nhp_rmsnorm_partial_bwd(dx.data_ptr(), ds.data_ptr(), do.data_ptr(), dy.data_ptr(), x.data_ptr(),
+                                   inv.data_ptr(), ptr(scale), ws.data_ptr(), eps, mode, rows, cols, stat, code, pcode,
+                                   None)
     assert rc == 0, L.nhp_status_string(rc)
     return y, inv, dx, ds, do
 
@@ -134,6 +157,61 @@ def test_rmsnorm_vs_oracle(hotpath, shape, dtype, mode):
     util.assert_close_ulp_or_noise(do, want_do, 2, dy.float().abs().sum(0) * 32 * util.EPS32, "doffset")
 
 
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("shape_stat", [((5, 8), 3), ((70, 128), 32), ((70, 128), 1), ((129, 2048), 512), ((129, 2048), 1023),
+                                        ((21, 4096), 4096), ((19, 8192), 2457), ((3, 32768), 16385), ((11, 1000), 333),
+                                        ((13, 2056), 2049)],
+                         ids=lambda v: f"{v[0][0]}x{v[0][1]}-{v[1]}")
+def test_partial_rmsnorm_vs_oracle(hotpath, shape_stat, dtype, mode):
+    """Partial RMSNorm: the statistic over the first `stat` columns (chunk-aligned or not, one
+    column, all columns), through nhp_rmsnorm_partial_fwd / _bwd."""
+    (rows, cols), stat = shape_stat
+    print(f"partial rmsnorm case {rows}x{cols} stat {stat} {dtype} mode {mode}", flush=True)
+    x, dy, scale, offset = make(dtype, rows, cols, rows + cols + stat, dtype)
+    eps = 1e-5 if mode == 0 else 1e-2
+    want_y, want_inv = oracle.rmsnorm_fwd(x, scale, offset, eps, mode, stat_cols=stat)
+    y, inv, dx, ds, do = [t.cpu() for t in abi_rmsnorm(hotpath, x.to(DEV), dy.to(DEV), scale.to(DEV), offset.to(DEV),
+                                                      eps, mode, stat)]
+    grow = (x.float().abs() * want_inv[:, None]).clamp(min=1.0)   # columns outside the statistic are not bounded by it
+    util.assert_close_ulp_or_noise(y, want_y, 2, out_noise(scale, x) * grow, "y")
+    assert torch.allclose(inv, want_inv, rtol=1e-5, atol=0)
+    want_dx, want_ds, want_do = oracle.rmsnorm_bwd(dy, x, inv, scale, eps, mode, stat_cols=stat)
+    xh = (x.float() * inv[:, None]).abs()
+    noise = ((dy.float().abs() * scale.float().abs() * xh).sum(-1, keepdim=True) * xh * inv[:, None] / stat * 256 * util.EPS32
+             + dx_noise(dy, scale, inv) / cols)
+    util.assert_close_ulp_or_noise(dx, want_dx, 2, noise, "dx")
+    col = (dy.float().abs() * xh).sum(0) * 32 * util.EPS32
+    util.assert_close_ulp_or_noise(ds, want_ds, 2, col, "dscale")
+    util.assert_close_ulp_or_noise(do, want_do, 2, dy.float().abs().sum(0) * 32 * util.EPS32, "doffset")
+    if stat == cols:
+        full = [t.cpu() for t in abi_rmsnorm(hotpath, x.to(DEV), dy.to(DEV), scale.to(DEV), offset.to(DEV), eps, mode)]
+        for a, b in zip((y, inv, dx, ds, do), full):
+            assert torch.equal(util.raw_bits(a), util.raw_bits(b))
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("shape", [(9, 16), (70, 128), (129, 2048), (19, 8192), (11, 1000)], ids=lambda s: f"{s[0]}x{s[1]}")
+def test_scalenorm_vs_oracle(hotpath, shape, dtype):
+    """eps_mode 2: x / max(||x||, eps) * g, with rows whose norm is below eps and an all-zero row."""
+    rows, cols = shape
+    print(f"scalenorm case {shape} {dtype}", flush=True)
+    x, dy, _, _ = make(dtype, rows, cols, rows + cols + 5, dtype)
+    x[1] = x[1] * 1e-5          # norm below eps: clamped
+    x[2] = 0
+    eps = 1e-2
+    gvec = torch.full((cols,), 1.7, dtype=dtype)
+    want_y, want_inv = oracle.rmsnorm_fwd(x, gvec, None, eps, 2)
+    y, inv, dx, ds, _ = [t.cpu() for t in abi_rmsnorm(hotpath, x.to(DEV), dy.to(DEV), gvec.to(DEV), None, eps, 2)]
+    util.assert_close_ulp_or_noise(y, want_y, 2, out_noise(gvec, x), "y")
+    assert torch.allclose(inv, want_inv, rtol=1e-5, atol=0)
+    assert inv[1].item() == pytest.approx(1 / eps) and inv[2].item() == pytest.approx(1 / eps)
+    want_dx, want_ds, _ = oracle.rmsnorm_bwd(dy, x, inv, gvec, eps, 2)
+    util.assert_close_ulp_or_noise(dx, want_dx, 2, dx_noise(dy, gvec, inv), "dx")
+    col = (dy.float().abs() * (x.float() * inv[:, None]).abs()).sum(0) * 32 * util.EPS32
+    util.assert_close_ulp_or_noise(ds, want_ds, 2, col, "dscale")
+
+
 def test_norm_edge_cases(hotpath):
     L = hotpath.lib()
     # no affine terms, no statistics wanted, no parameter gradients, unaligned input, empty tensors
@@ -159,7 +237,8 @@ def test_norm_edge_cases(hotpath):
     util.assert_close_ulp_or_noise(y.cpu(), want, 2, out_noise(None, x), "unaligned")
     assert L.nhp_layernorm_fwd(None, None, None, None, None, None, 1e-5, 0, 256, 1, 1, None) == 0
     assert L.nhp_layernorm_fwd(y.data_ptr(), None, None, xd.data_ptr(), None, None, 1e-5, 50, 256, 1, 0, None) == -1
-    assert L.nhp_rmsnorm_fwd(y.data_ptr(), None, xd.data_ptr(), None, None, 1e-5, 2, 50, 256, 1, 1, None) == -2
+    assert L.nhp_rmsnorm_fwd(y.data_ptr(), None, xd.data_ptr(), None, None, 1e-5, 3, 50, 256, 1, 1, None) == -2
+    assert L.nhp_rmsnorm_partial_fwd(y.data_ptr(), None, xd.data_ptr(), None, None, 1e-5, 1, 50, 256, 257, 1, 1, None) == -2
     # a constant row (zero variance) and an all-zero row
     const = torch.full((4, 512), 3.0, dtype=torch.bfloat16, device=DEV)
     out = torch.empty_like(const)
@@ -248,8 +327,102 @@ def test_rmsnorm_module_against_the_reference_expression(dtype):
     assert cls is RMSNorm and eps == 1e-6
     args.norm = "layernorm"
     assert get_norm(args) == (LayerNorm, 1e-5)
-    with pytest.raises(NotImplementedError):
-        RMSNorm(h, p=0.5)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "fp32"])
+def test_partial_rmsnorm_and_scalenorm_modules_against_the_reference_expressions(dtype):
+    """RMSNorm(p=0.3) and ScaleNorm against the eager expressions of the reference's classes
+    (megatron/model/norms.py:85-107, :117-119) with autograd through torch ops in fp32."""
+    from megatron.model.norms import RMSNorm, ScaleNorm
+
+    s, b, h = 64, 2, 1024
+    x = util.randn((s, b, h), dtype, seed=3, std=2.0).to(DEV)
+    g = util.randn((s, b, h), dtype, seed=4).to(DEV)
+    lim = 2.0 ** (-7 if dtype == torch.bfloat16 else -18)
+
+    m = RMSNorm(h, p=0.3, eps=1e-8).to(DEV)
+    with torch.no_grad():
+        m.scale.copy_(1 + 0.3 * torch.randn(h, generator=torch.Generator().manual_seed(1)))
+    part = int(h * 0.3)
+    assert m.partial_size == part
+    xa = x.clone().requires_grad_(True)
+    y = m(xa)
+    y.backward(g)
+    xr = x.detach().clone().float().requires_grad_(True)
+    sr = m.scale.detach().clone().requires_grad_(True)
+    partial_x, _ = torch.split(xr, [part, h - part], dim=-1)
+    rms_x = partial_x.norm(2, dim=-1, keepdim=True) * part ** (-1.0 / 2)
+    ref = sr * (xr / (rms_x + 1e-8))
+    ref.backward(g.float())
+    grow = (ref.detach().abs() / sr.detach().abs()).clamp(min=1.0).cpu()
+    util.assert_close_ulp_or_noise(y.detach().cpu(), ref.detach().to(dtype).cpu(), 2,
+                                   out_noise(sr.detach().cpu(), x.cpu()) * grow, "partial y")
+    assert (xa.grad.float() - xr.grad).norm() <= lim * xr.grad.norm()
+    assert (m.scale.grad - sr.grad).norm() <= lim * sr.grad.norm()
+
+    sn = ScaleNorm(h, eps=1e-5).to(DEV)
+    with torch.no_grad():
+        sn.g.fill_(1.3)
+    xa = x.clone().requires_grad_(True)
+    y = sn(xa)
+    y.backward(g)
+    xr = x.detach().clone().float().requires_grad_(True)
+    gr = sn.g.detach().clone().requires_grad_(True)
+    n = torch.norm(xr, dim=-1, keepdim=True).clamp(min=1e-5)
+    ref = xr / n * gr
+    ref.backward(g.float())
+    assert y.dtype == dtype and sn.g.grad.shape == (1,)
+    util.assert_close_ulp_or_noise(y.detach().cpu(), ref.detach().to(dtype).cpu(), 2,
+                                   out_noise(torch.full((h,), 1.3), x.cpu()), "scalenorm y")
+    assert (xa.grad.float() - xr.grad).norm() <= lim * xr.grad.norm()
+    assert abs(sn.g.grad.item() - gr.grad.item()) <= max(lim, 1e-3) * (g.float() * (xr.detach() / n.detach())).abs().sum().item() / h ** 0.5
+
+
+@pytest.mark.parametrize("one_p", [False, True], ids=["plain", "1p"])
+def test_mixed_fused_classes_match_torch(one_p):
+    """MixedFusedLayerNorm / MixedFusedRMSNorm (megatron/model/fused_layer_norm.py:34-262) against torch's
+    layer_norm / rms_norm on the same weights, including the zero-centred (`1p`) parameter storage."""
+    from megatron.model.fused_layer_norm import MixedFusedLayerNorm, MixedFusedRMSNorm
+
+    dtype, h = torch.bfloat16, 2048
+    x = util.randn((48, 4, h), dtype, seed=5, std=2.0).to(DEV)
+    g = util.randn((48, 4, h), dtype, seed=6).to(DEV)
+    w = (1 + 0.3 * torch.randn(h, generator=torch.Generator().manual_seed(1))).to(dtype).to(DEV)
+    bb = (0.2 * torch.randn(h, generator=torch.Generator().manual_seed(2))).to(dtype).to(DEV)
+    lim = 2.0 ** -7
+
+    ln = MixedFusedLayerNorm(h, eps=1e-5, apply_layernorm_1p=one_p).to(DEV).to(dtype)
+    with torch.no_grad():
+        ln.weight.copy_(w - 1 if one_p else w)
+        ln.bias.copy_(bb)
+    eff_w = (ln.weight.detach() + 1) if one_p else ln.weight.detach()
+    xa = x.clone().requires_grad_(True)
+    y = ln(xa)
+    y.backward(g)
+    xr = x.clone().requires_grad_(True)
+    wr = eff_w.clone().requires_grad_(True)
+    br = bb.clone().requires_grad_(True)
+    ref = F.layer_norm(xr, (h,), wr, br, 1e-5)
+    ref.backward(g)
+    util.assert_close_ulp_or_noise(y.detach().cpu(), ref.detach().cpu(), 2, out_noise(eff_w.cpu(), x.cpu()), "layernorm y")
+    assert (xa.grad.float() - xr.grad.float()).norm() <= lim * xr.grad.float().norm()
+    assert (ln.weight.grad.float() - wr.grad.float()).norm() <= lim * wr.grad.float().norm()
+    assert (ln.bias.grad.float() - br.grad.float()).norm() <= lim * br.grad.float().norm()
+
+    rms = MixedFusedRMSNorm(h, eps=1e-5, apply_rmsnorm_1p=one_p).to(DEV).to(dtype)
+    with torch.no_grad():
+        rms.scale.copy_(w - 1 if one_p else w)
+    eff_s = (rms.scale.detach() + 1) if one_p else rms.scale.detach()
+    xa = x.clone().requires_grad_(True)
+    y = rms(xa)
+    y.backward(g)
+    xr = x.float().requires_grad_(True)
+    sr = eff_s.float().clone().requires_grad_(True)
+    ref = F.rms_norm(xr, (h,), sr, 1e-5)
+    ref.backward(g.float())
+    util.assert_close_ulp_or_noise(y.detach().cpu(), ref.detach().to(dtype).cpu(), 2, out_noise(eff_s.cpu(), x.cpu()), "rmsnorm y")
+    assert (xa.grad.float() - xr.grad).norm() <= lim * xr.grad.norm()
+    assert (rms.scale.grad.float() - sr.grad).norm() <= lim * sr.grad.norm()
 
 
 def test_layernorm_full_size(hotpath):

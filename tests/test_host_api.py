@@ -242,13 +242,31 @@ def test_layer_modules_surface_and_errors():
     rms = norms.RMSNorm(16, eps=1e-8)
     assert [n for n, _ in rms.named_parameters()] == ["scale"] and rms.offset is None
     assert sorted(n for n, _ in norms.RMSNorm(16, bias=True).named_parameters()) == ["offset", "scale"]
-    with pytest.raises(NotImplementedError):
-        norms.RMSNorm(16, p=0.25)
-    args = types.SimpleNamespace(norm="rmsnorm", rms_norm_epsilon=1e-6, rmsnorm_fusion=True, layernorm_epsilon=1e-5)
+    assert norms.RMSNorm(16, p=0.25).partial_size == 4 and norms.RMSNorm(16).partial_size is None
+    with pytest.raises(ZeroDivisionError):
+        norms.RMSNorm(16, p=0.01)   # int(16 * 0.01) = 0 features: the reference raises the same on its first forward
+    sn = norms.ScaleNorm(16, eps=1e-5)
+    assert [(n, tuple(p.shape)) for n, p in sn.named_parameters()] == [("g", (1,))] and float(sn.g.detach()) == 1.0
+    from megatron.model import fused_layer_norm as fln
+    args = types.SimpleNamespace(norm="rmsnorm", rms_norm_epsilon=1e-6, rmsnorm_fusion=True, layernorm_epsilon=1e-5,
+                                 layernorm_fusion=True, scalenorm_epsilon=1e-8)
     cls, eps = norms.get_norm(args)
-    assert issubclass(cls, norms.RMSNorm) and cls(8, eps=eps).fused_eps and eps == 1e-6
+    assert cls is fln.MixedFusedRMSNorm and eps == 1e-6
+    fused = cls(8, eps=eps, sequence_parallel=True, apply_rmsnorm_1p=True)
+    assert [n for n, _ in fused.named_parameters()] == ["scale"] and fused.scale.sequence_parallel
+    assert float(fused.scale.detach().abs().sum()) == 0          # stored as weight - 1
     args.rmsnorm_fusion = False
     assert norms.get_norm(args)[0] is norms.RMSNorm
+    args.norm = "layernorm"
+    cls, eps = norms.get_norm(args)
+    assert cls is fln.MixedFusedLayerNorm and eps == 1e-5
+    fl = cls(16, eps=eps)
+    assert sorted(n for n, _ in fl.named_parameters()) == ["bias", "weight"] and float(fl.weight.detach().sum()) == 16
+    assert fl.normalized_shape == torch.Size([16]) and not fl.weight.sequence_parallel
+    args.layernorm_fusion = False
+    assert norms.get_norm(args)[0] is norms.LayerNorm
     args.norm = "scalenorm"
+    assert norms.get_norm(args) == (norms.ScaleNorm, 1e-8)
+    args.norm = "te_rmsnorm"
     with pytest.raises(ValueError):
         norms.get_norm(args)

@@ -277,6 +277,96 @@ def test_rmsnorm_backward_is_the_adjoint(dtype, mode):
     assert torch.isfinite(dz).all() and torch.allclose(dz, g * zi[0])
 
 
+@pytest.mark.parametrize("frac", [0.5, 0.3, 1.0, 0.01])
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_partial_rmsnorm_is_the_class_expression(dtype, frac):
+    """RMSNorm with 0 <= p <= 1 (megatron/model/norms.py:87-94): the statistic comes from the first
+    int(dim * p) columns, every column is divided by it. Spelled here with the class's own torch
+    calls in fp32 and in float64; the backward against float64 autograd of the same expression."""
+    x, scale, offset, dy = norm_inputs(dtype, seed=21)
+    d = x.size(-1)
+    part = max(int(d * frac), 1)
+    eps = 1e-3
+    y, inv = oracle.rmsnorm_fwd(x, scale, offset, eps, 1, stat_cols=part)
+
+    def class_forward(xx, sc, of):
+        partial_x, _ = torch.split(xx, [part, d - part], dim=-1)
+        norm_x = partial_x.norm(2, dim=-1, keepdim=True)
+        rms_x = norm_x * part ** (-1.0 / 2)
+        return sc * (xx / (rms_x + eps)) + of
+
+    util.assert_close_ulp_or_noise(y, class_forward(x.float(), scale.float(), offset.float()).to(dtype), 1,
+                                   norm_noise(x, scale) * (d / part) ** 0.5, "vs the class's expression in fp32")
+    xd = x.double().requires_grad_(True)
+    sd = scale.double().requires_grad_(True)
+    od = offset.double().requires_grad_(True)
+    out = class_forward(xd, sd, od)
+    util.assert_close_ulp_or_noise(y, out.detach().to(dtype), 1, norm_noise(x, scale) * (d / part) ** 0.5, "vs float64")
+    out.backward(dy.double())
+    dx, ds, do = oracle.rmsnorm_bwd(dy, x, inv, scale, eps, 1, stat_cols=part)
+    noise = (dy.float().abs() * scale.float().abs() * x.float().abs()).sum(-1, keepdim=True) * inv[:, None] ** 2 \
+        * x.float().abs().amax(-1, keepdim=True) * 256 * util.EPS32 * (d / part) \
+        + (dy.float().abs() * scale.float().abs()).amax(-1, keepdim=True) * inv[:, None] * 16 * util.EPS32
+    util.assert_close_ulp_or_noise(dx, xd.grad.to(dtype), 1, noise.expand_as(dx.float()), "dx vs float64 autograd")
+    col_noise = (dy.float().abs() * x.float().abs() * inv[:, None]).sum(0) * 64 * util.EPS32 + dy.float().abs().sum(0) * 64 * util.EPS32
+    util.assert_close_ulp_or_noise(ds, sd.grad.to(dtype), 1, col_noise, "dscale")
+    util.assert_close_ulp_or_noise(do, od.grad.to(dtype), 1, col_noise, "doffset")
+    if part == d:
+        full, finv = oracle.rmsnorm_fwd(x, scale, offset, eps, 1)
+        assert torch.equal(full, y) and torch.equal(finv, inv)
+    else:
+        # columns outside the statistic only see the first term of the gradient
+        x32, s32, o32, dy32 = norm_inputs(torch.float32, seed=21)
+        _, i32 = oracle.rmsnorm_fwd(x32, s32, o32, eps, 1, stat_cols=part)
+        dx32, _, _ = oracle.rmsnorm_bwd(dy32, x32, i32, s32, eps, 1, stat_cols=part)
+        assert torch.equal(dx32[:, part:], i32[:, None] * (dy32 * s32)[:, part:])
+    # the other epsilon placement takes the same statistic columns
+    y0, inv0 = oracle.rmsnorm_fwd(x.float(), None, None, 1e-6, 0, stat_cols=part)
+    want0 = x.double() / torch.sqrt((x.double()[:, :part] ** 2).mean(-1, keepdim=True) + 1e-6)
+    assert torch.allclose(y0.double(), want0, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_scalenorm_is_the_class_expression(dtype):
+    """ScaleNorm.forward (megatron/model/norms.py:117-119): x / clamp(||x||, min=eps) * g with a scalar g;
+    a row whose norm is below eps is divided by eps and its norm has no gradient."""
+    x, _, _, dy = norm_inputs(dtype, seed=31)
+    x = x.clone()
+    x[3] = x[3] * 1e-4          # clamped row (norm below eps)
+    x[5] = 0                    # all-zero row
+    eps = 1e-2
+    g = torch.tensor([1.7], dtype=torch.float32)
+    cols = x.size(-1)
+    gvec = g.to(dtype).expand(cols).contiguous()
+    y, inv = oracle.rmsnorm_fwd(x, gvec, None, eps, 2)
+
+    def class_forward(xx, gg):
+        n = torch.norm(xx, dim=-1, keepdim=True).clamp(min=eps)
+        return xx / n * gg
+
+    ref32 = class_forward(x.float(), g.to(dtype).float())
+    noise = x.float().abs() * inv[:, None] * 1.7 * 8 * util.EPS32
+    util.assert_close_ulp_or_noise(y, ref32.to(dtype), 1, noise, "vs the class's expression in fp32")
+    assert torch.allclose(inv[3], torch.tensor(1 / eps)) and torch.allclose(inv[5], torch.tensor(1 / eps))
+    assert y[5].abs().max() == 0
+    xd = x.double().requires_grad_(True)
+    gd = g.to(dtype).double().requires_grad_(True)
+    class_forward(xd, gd).backward(dy.double())
+    dx, ds, _ = oracle.rmsnorm_bwd(dy, x, inv, gvec, eps, 2)
+    bnoise = (dy.float().abs() * 1.7).sum(-1, keepdim=True) * inv[:, None] * 128 * util.EPS32
+    util.assert_close_ulp_or_noise(dx, xd.grad.to(dtype), 1, bnoise.expand_as(dx.float()), "dx vs float64 autograd")
+    # the scalar's gradient is the sum of the per-column gradients
+    dg = ds.double().sum()
+    tol = {torch.float32: 1e-5, torch.float16: 2e-3, torch.bfloat16: 1e-2}[dtype]  # per-column sums are rounded to dtype
+    assert abs(dg - gd.grad[0]) <= tol * (dy.double().abs() * (x.double() * inv[:, None].double()).abs()).sum()
+    # unclamped rows come out with unit norm times g
+    y32, _ = oracle.rmsnorm_fwd(x.float(), g.expand(cols).contiguous(), None, eps, 2)
+    norms = y32.norm(dim=-1)
+    keep = torch.ones(x.size(0), dtype=torch.bool)
+    keep[3] = keep[5] = False
+    assert (norms[keep] - 1.7).abs().max() < 1e-5
+
+
 # ---------------------------------------------------------------------------
 # gated activations
 # ---------------------------------------------------------------------------
