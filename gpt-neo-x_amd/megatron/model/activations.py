@@ -122,15 +122,40 @@ _GATE_CODE = {swish: 0, torch.nn.functional.gelu: 1, torch.nn.functional.relu: 2
               torch.sigmoid: 3, _identity: 4}
 
 
+def erf_gelu(x):
+    """GeLU through erf with the reference's rounded constant, ``x * 0.5 * (erf(x / 1.41421) + 1)``
+    (megatron/model/activations.py:117-126)."""
+    return x * 0.5 * (torch.erf(x / 1.41421).to(dtype=x.dtype) + torch.ones_like(x).to(dtype=x.dtype))
+
+
+def mish(x):
+    """``x * tanh(softplus(x))`` (megatron/model/activations.py:134-135)."""
+    return x * torch.tanh(torch.nn.functional.softplus(x))
+
+
+# Settings that are one torch call on one tensor in the reference as well (no fused kernel on either side).
+_PLAIN = {"relu": torch.nn.functional.relu, "softsign": torch.nn.functional.softsign, "swish": swish, "mish": mish,
+          "silu": torch.nn.functional.silu}
+
+
 def get_activation(neox_args):
-    """(activation function, is_gated) for the settings served by the kernels here: the gated ones and
-    ``gelu`` with ``bias_gelu_fusion``; other settings are left to the reference's function."""
+    """(activation function, is_gated), as megatron/model/activations.py:27-66. The gated settings and
+    ``gelu`` with ``bias_gelu_fusion`` are served by the kernels of this library; the remaining settings
+    return the same torch functions as the reference."""
     name = neox_args.activation
     if name in _GATES:
         return _GATES[name], True
-    if name == "gelu" and getattr(neox_args, "bias_gelu_fusion", False) and not getattr(neox_args, "onnx_safe", False):
-        return bias_gelu_impl, False
-    raise ValueError(f"Activation function {name} is not provided by the MI355X kernels")
+    if name == "gelu":
+        onnx_safe = getattr(neox_args, "onnx_safe", False)
+        fusion = getattr(neox_args, "bias_gelu_fusion", False)
+        if onnx_safe and fusion:
+            raise ValueError("onnx_safe + bias_gelu_fusion not compatible")
+        if onnx_safe:
+            return erf_gelu, False
+        return (bias_gelu_impl if fusion else torch.nn.functional.gelu), False
+    if name in _PLAIN:
+        return _PLAIN[name], False
+    raise ValueError(f"Activation function {name} not recognized")
 
 
 class _GatedActivationFunction(torch.autograd.Function):

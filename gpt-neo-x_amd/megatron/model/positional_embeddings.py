@@ -1,6 +1,7 @@
-"""Rotary cache, the eager (unfused) rotary functions and the AliBi slopes, with
-the public surface of GPT-NeoX's ``megatron/model/positional_embeddings.py``
-(RotaryEmbedding :38-97, rotate_half :103-107, apply_rotary_pos_emb :110-116,
+"""Rotary cache, the eager (unfused) rotary functions, the AliBi slopes and the
+sinusoidal table, with the public surface of GPT-NeoX's
+``megatron/model/positional_embeddings.py`` (SinusoidalPositionalEmbedding :19-35,
+RotaryEmbedding :38-97, rotate_half :103-107, apply_rotary_pos_emb :110-116,
 apply_rotary_pos_emb_torch :119-126, AliBi :129-257).
 """
 import math
@@ -14,6 +15,26 @@ def _rotary_angles(dim, seq_len, base):
     positions = torch.arange(seq_len).type_as(inv_freq)
     half = torch.einsum("i,j->ij", positions, inv_freq)
     return inv_freq, torch.cat((half, half), dim=-1)
+
+
+class SinusoidalPositionalEmbedding(torch.nn.Module):
+    """``[1, seq, dim]`` table ``cat(sin(p * f_j), cos(p * f_j))`` with ``f_j = base^(-2j/dim)``, added to the
+    token embeddings once per forward pass (not a per-layer operation, so plain torch here as in the reference)."""
+
+    def __init__(self, dim, base=10000, precision=torch.half):
+        super().__init__()
+        self.register_buffer("inv_freq", 1.0 / (base ** (torch.arange(0, dim, 2).float() / dim)))
+        self.precision = precision
+
+    def forward(self, x, seq_dim=1):
+        positions = torch.arange(x.shape[seq_dim], device=x.device).type_as(self.inv_freq)
+        angles = torch.einsum("i,j->ij", positions, self.inv_freq)
+        if self.precision == torch.bfloat16:
+            angles = angles.float()
+        sin, cos = angles.sin(), angles.cos()
+        if self.precision == torch.bfloat16:
+            sin, cos = sin.bfloat16(), cos.bfloat16()
+        return torch.cat((sin, cos), dim=-1)[None, :, :]
 
 
 class RotaryEmbedding(torch.nn.Module):

@@ -2,9 +2,11 @@
 fused_rope, positional_embeddings, megatron.fused_kernels): names, argument
 meaning, gating logic and error behaviour. Runs without a GPU."""
 import math
+import types
 
 import pytest
 import torch
+import torch.nn.functional as F
 
 import util
 from oracle import fallback_semantics as fb
@@ -270,3 +272,46 @@ def test_layer_modules_surface_and_errors():
     args.norm = "te_rmsnorm"
     with pytest.raises(ValueError):
         norms.get_norm(args)
+
+
+def test_get_activation_covers_the_reference_settings():
+    """get_activation (megatron/model/activations.py:27-66): every setting the reference recognises, the
+    gating flag, the onnx_safe / bias_gelu_fusion conflict; the unfused ones against their closed forms."""
+    from megatron.model import activations as A
+
+    def pick(name, **kw):
+        return A.get_activation(types.SimpleNamespace(activation=name, **kw))
+
+    for name in ("geglu", "reglu", "bilinear", "swiglu", "glu"):
+        assert pick(name)[1] is True
+    assert pick("gelu", bias_gelu_fusion=True, onnx_safe=False) == (A.bias_gelu_impl, False)
+    assert pick("gelu", bias_gelu_fusion=False, onnx_safe=False) == (F.gelu, False)
+    assert pick("gelu", bias_gelu_fusion=False, onnx_safe=True) == (A.erf_gelu, False)
+    with pytest.raises(ValueError, match="not compatible"):
+        pick("gelu", bias_gelu_fusion=True, onnx_safe=True)
+    with pytest.raises(ValueError, match="not recognized"):
+        pick("tanh")
+    x = torch.linspace(-6, 6, 49, dtype=torch.float64)
+    for name, want in (("relu", x.clamp(min=0)), ("softsign", x / (1 + x.abs())), ("swish", x / (1 + torch.exp(-x))),
+                       ("silu", x / (1 + torch.exp(-x))), ("mish", x * torch.tanh(torch.log1p(torch.exp(x))))):
+        func, gated = pick(name)
+        assert gated is False and torch.allclose(func(x), want, atol=1e-12), name
+    assert torch.allclose(A.erf_gelu(x), x * 0.5 * (1 + torch.erf(x / 1.41421)), atol=1e-12)
+    assert torch.allclose(A.erf_gelu(x), F.gelu(x), atol=1e-5)       # 1.41421 is sqrt(2) to 6 digits
+
+
+def test_sinusoidal_positional_embedding():
+    """SinusoidalPositionalEmbedding (megatron/model/positional_embeddings.py:19-35): [1, seq, dim], sines then cosines of
+    position * base^(-2j/dim)."""
+    from megatron.model.positional_embeddings import SinusoidalPositionalEmbedding
+
+    for precision in (torch.half, torch.bfloat16):
+        emb = SinusoidalPositionalEmbedding(16, base=10000, precision=precision)
+        out = emb(torch.zeros(2, 7, 16))
+        assert out.shape == (1, 7, 16) and emb.inv_freq.shape == (8,)
+        assert out.dtype == (torch.bfloat16 if precision == torch.bfloat16 else torch.float32)
+        pos = torch.arange(7, dtype=torch.float64)[:, None]
+        freq = 10000.0 ** (-torch.arange(0, 16, 2, dtype=torch.float64) / 16)[None, :]
+        want = torch.cat((torch.sin(pos * freq), torch.cos(pos * freq)), dim=-1)
+        assert torch.allclose(out[0].double(), want, atol=1e-2 if precision == torch.bfloat16 else 1e-6)
+        assert emb(torch.zeros(5, 3, 16), seq_dim=0).shape == (1, 5, 16)
