@@ -15,7 +15,8 @@ the drop-in extension modules (which call libneox_hotpath.so):
   rope-c4        rotary fwd+bwd on q,k [4096,4,32,128] bf16, rotary_pct 1.0 and 0.25
   llama2-7b-c5   rotary on q,k [8192,2,32,128] + causal softmax fwd+bwd [64,8192,8192] bf16
   rope-c4-qkv-view  rotary fwd+bwd on q,k given as views of one fused [4096,4,32,3*128] bf16 buffer (the layout
-                 the attention layer slices q and k from), rotary_pct 1.0
+                 the attention layer slices q and k from), rotary_pct 1.0; one launch per tensor, then q and k
+                 in one launch
   rope-qk-1.4b   rotary fwd+bwd on q,k [2048,8,16,128] bf16, rotary_pct 0.25, q and k in one launch
   mistral-window causal softmax fwd+bwd [64,8192,8192] bf16 with a 4096-key sliding window applied by index
   alibi-1.4b     causal softmax fwd+bwd [128,2048,2048] bf16 with the AliBi bias of 16 heads added in the kernel
@@ -441,7 +442,9 @@ def make_workload(name, torch, dev):
             cos, sin = RotaryEmbedding(d2, s, base=10000, precision=torch.bfloat16)(qkv, seq_len=s)
             sets.append((qkv[..., :d], qkv[..., d:2 * d], dqkv[..., :d], dqkv[..., d:2 * d], cos.contiguous(), sin.contiguous()))
         rb = rope_bytes(s, b, h, d, d2)
-        kernel_bytes = {"rope_fwd_view": 2 * rb, "rope_bwd_view": 2 * rb}
+        one_launch = 2 * rb - 2 * s * d2 * 2   # the tables are read once for q and k
+        kernel_bytes = {"rope_fwd_view": 2 * rb, "rope_bwd_view": 2 * rb, "rope_qk_fwd_view": one_launch,
+                        "rope_qk_bwd_view": one_launch}
         state = {"i": 0}
 
         def step(t):
@@ -458,6 +461,9 @@ def make_workload(name, torch, dev):
 
             t.run("rope_fwd_view", f)
             t.run("rope_bwd_view", bw)
+            # the same through the two-tensor entry point: q and k in one launch
+            t.run("rope_qk_fwd_view", lambda: rope_ext.forward_cached_qk(q, k, cos, sin, False))
+            t.run("rope_qk_bwd_view", lambda: rope_ext.backward_cached_qk(dq, dk, cos, sin, False))
 
         cfg = {"workload": name, "qk": [s, b, h, d], "qk_strides": list(sets[0][0].stride()), "rotary_dim": d2}
         return step, kernel_bytes, {}, "rope_fwd_view", "bf16", cfg
