@@ -1,0 +1,94 @@
+"""The caller of the fused softmax: scores -> probabilities -> context.
+
+What ``ParallelSelfAttention.attention`` does in GPT-NeoX
+(megatron/model/transformer.py:526-625) with the pieces of its constructor that
+set the scaling (:417-424, :499-511), as a module of its own without the model
+parallel layers around it:
+
+    scores  = baddbmm(q, k^T) * (1 / norm_factor)          library GEMM (rocBLAS / hipBLASLt)
+    probs   = softmax(scores * coeff + masks and biases)     one kernel of libneox_hotpath.so
+    probs   = dropout(probs)                                 same kernel on the causal branch
+    context = bmm(probs, v)                                  library GEMM
+
+``norm_factor = sqrt(head_dim) * coeff`` and ``coeff = max(1, layer_number)`` with
+``apply_query_key_layer_scaling``, otherwise ``coeff`` is None and the softmax does not
+scale: the two factors cancel in exact arithmetic and only keep fp16 scores in range.
+
+Everything between the two GEMMs that the reference runs as separate passes over
+``[b, np, sq, sk]`` -- the relative-position bias add (:580-582), the AliBi add (:584-585),
+the dropout (:592-593) -- is handed to ``FusedScaleMaskSoftmax`` and happens inside its
+kernel. Tensors are laid out as in the reference: q ``[sq, b, np, hn]``, k and v
+``[sk, b, np, hn]``, result ``[b, np, sq, hn]``.
+"""
+import math
+
+import torch
+
+from .fused_softmax import FusedScaleMaskSoftmax, SoftmaxFusionTypes
+
+
+def get_fusion_type(neox_args):
+    """``SoftmaxFusionTypes`` member for the two fusion flags (megatron/model/utils.py:356-362)."""
+    if neox_args.scaled_upper_triang_masked_softmax_fusion:
+        return SoftmaxFusionTypes.upper_triang
+    if neox_args.scaled_masked_softmax_fusion:
+        return SoftmaxFusionTypes.general
+    return SoftmaxFusionTypes.none
+
+
+class CoreAttention(torch.nn.Module):
+    """Unfused ("global") attention on top of the fused softmax.
+
+    Arguments:
+        head_dim: features per head (``hidden_size_per_attention_head``).
+        layer_number: 1-based layer index, used by ``apply_query_key_layer_scaling``.
+        fp16, bf16: the precision flags of the model (both False: fp32, torch softmax).
+        fusion_type: a ``SoftmaxFusionTypes`` member.
+        mask_func: ``mask_func(scores, mask)`` for the softmax's torch branch.
+        attention_softmax_in_fp32, apply_query_key_layer_scaling: as in the reference's arguments;
+            layer scaling forces the fp32 softmax (transformer.py:350-352).
+        use_mup: divide by ``head_dim`` instead of its square root (transformer.py:423-424).
+        attention_dropout, sliding_window_width, alibi_slopes: handed to the softmax module.
+        rpe: optional module ``rpe(sq, sk) -> [1, np, sq, sk]`` (relative position bias).
+        use_cache: crop the mask to the current key length (inference with a KV cache).
+    """
+
+    def __init__(self, head_dim, layer_number, fp16, bf16, fusion_type, mask_func, attention_softmax_in_fp32=False,
+                 apply_query_key_layer_scaling=False, use_mup=False, attention_dropout=0.0,
+                 sliding_window_width=None, alibi_slopes=None, rpe=None, use_cache=False):
+        super().__init__()
+        self.layer_number = max(1, int(layer_number))
+        if apply_query_key_layer_scaling:
+            attention_softmax_in_fp32 = True
+        coeff = None
+        self.norm_factor = math.sqrt(head_dim)
+        if apply_query_key_layer_scaling:
+            coeff = max(1, self.layer_number)
+            self.norm_factor *= coeff
+        if use_mup:
+            self.norm_factor = head_dim
+        self.rpe = rpe
+        self.use_cache = use_cache
+        self.scale_mask_softmax = FusedScaleMaskSoftmax(
+            input_in_fp16=fp16, input_in_bf16=bf16, fusion_type=fusion_type, mask_func=mask_func,
+            softmax_in_fp32=attention_softmax_in_fp32, scale=coeff, sliding_window_width=sliding_window_width,
+            alibi_slopes=alibi_slopes, attention_dropout=attention_dropout)
+
+    def forward(self, query_layer, key_layer, value_layer, attention_mask, key_lengths=None):
+        b, np_, sq, sk = query_layer.size(1), query_layer.size(2), query_layer.size(0), key_layer.size(0)
+        hn = query_layer.size(3)
+        # [sq, b, np, hn] -> [sq, b * np, hn]
+        q = query_layer.reshape(sq, b * np_, hn)
+        k = key_layer.reshape(sk, b * np_, hn)
+        scores = torch.empty((b * np_, sq, sk), dtype=q.dtype, device=q.device)
+        scores = torch.baddbmm(scores, q.transpose(0, 1), k.transpose(0, 1).transpose(1, 2), beta=0.0,
+                               alpha=1.0 / self.norm_factor).view(b, np_, sq, sk)
+        if self.use_cache and attention_mask is not None:
+            with torch.no_grad():
+                attention_mask = attention_mask[..., :sk, :sk]
+        bias = self.rpe(sq, sk) if self.rpe is not None else None
+        probs = self.scale_mask_softmax(scores, attention_mask, bias=bias, key_lengths=key_lengths)
+        # [sk, b, np, hn] -> [sk, b * np, hn]; context [b * np, sq, hn]
+        v = value_layer.reshape(sk, b * np_, value_layer.size(3))
+        context = torch.bmm(probs.view(b * np_, sq, sk), v.transpose(0, 1))
+        return context.view(b, np_, sq, value_layer.size(3))

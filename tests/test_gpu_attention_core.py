@@ -1,0 +1,138 @@
+"""The caller of the fused softmax on the GPU: CoreAttention (the score -> probability ->
+context part of ParallelSelfAttention.attention, megatron/model/transformer.py:526-625) against
+textbook attention evaluated in fp32 with torch ops, forward and backward.
+
+Tolerance: the two GEMMs run in the 16-bit storage type, so results are compared by relative
+Frobenius error (2^-7 for bf16, 2^-9 for fp16), not by units in the last place; the softmax
+kernel itself is held to 2 ulp in the other GPU tests."""
+import math
+
+import pytest
+import torch
+
+import util
+from oracle import fallback_semantics as fb
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def mask_func(scores, mask):
+    return fb.fill_masked_with_dtype_min(scores, mask)
+
+
+def textbook(q, k, v, mask, extra=None):
+    """softmax(q k^T / sqrt(hn) + extra, masked) v in fp32; q [sq,b,np,hn] -> [b,np,sq,hn]."""
+    q, k, v = (t.float().permute(1, 2, 0, 3) for t in (q, k, v))
+    scores = q @ k.transpose(-1, -2) / math.sqrt(q.size(-1))
+    if extra is not None:
+        scores = scores + extra
+    scores = scores.masked_fill(mask, float("-inf"))
+    return torch.softmax(scores, dim=-1) @ v
+
+
+def rel_err(a, b):
+    return ((a.float() - b.float()).norm() / b.float().norm()).item()
+
+
+def qkv(dtype, sq, b, np_, hn, seed):
+    return [util.randn((sq, b, np_, hn), dtype, seed=seed + i).to(DEV).requires_grad_(True) for i in range(3)]
+
+
+@pytest.mark.parametrize("layer_scaling", [False, True], ids=["plain", "qk-layer-scaling"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+def test_causal_attention_matches_textbook(dtype, layer_scaling):
+    from megatron.model.attention_core import CoreAttention
+    from megatron.model.fused_softmax import SoftmaxFusionTypes as T
+
+    sq, b, np_, hn = 512, 2, 4, 64
+    lim = 2.0 ** (-7 if dtype == torch.bfloat16 else -9)
+    core = CoreAttention(hn, 7, dtype == torch.float16, dtype == torch.bfloat16, T.upper_triang, mask_func,
+                         attention_softmax_in_fp32=True, apply_query_key_layer_scaling=layer_scaling)
+    assert core.norm_factor == math.sqrt(hn) * (7 if layer_scaling else 1)
+    assert core.scale_mask_softmax.scale == (7 if layer_scaling else None)
+    q, k, v = qkv(dtype, sq, b, np_, hn, 1)
+    mask = fb.causal_mask(sq, DEV)
+    assert core.scale_mask_softmax.is_kernel_available(mask, b, np_, sq, sq)
+    out = core(q, k, v, mask)
+    assert out.shape == (b, np_, sq, hn) and out.dtype == dtype
+    g = util.randn((b, np_, sq, hn), dtype, seed=9).to(DEV)
+    out.backward(g)
+    qr, kr, vr = (t.detach().clone().requires_grad_(True) for t in (q, k, v))
+    ref = textbook(qr, kr, vr, mask)
+    ref.backward(g.float())
+    assert rel_err(out, ref) <= lim
+    for got, want in ((q.grad, qr.grad), (k.grad, kr.grad), (v.grad, vr.grad)):
+        assert rel_err(got, want) <= 2 * lim
+    # the fused and the torch branch of the softmax module agree inside the caller
+    plain = CoreAttention(hn, 7, dtype == torch.float16, dtype == torch.bfloat16, T.none, mask_func,
+                          attention_softmax_in_fp32=True, apply_query_key_layer_scaling=layer_scaling)
+    assert rel_err(plain(q.detach(), k.detach(), v.detach(), mask), out) <= lim
+
+
+def test_padding_mask_alibi_window_and_rpe_inside_the_caller():
+    from megatron.model.attention_core import CoreAttention
+    from megatron.model.fused_softmax import SoftmaxFusionTypes as T
+    from megatron.model.positional_embeddings import AliBi
+
+    dtype, sq, b, np_, hn = torch.bfloat16, 256, 4, 4, 64
+    lim = 2.0 ** -7
+    q, k, v = qkv(dtype, sq, b, np_, hn, 11)
+    pos = torch.arange(sq, device=DEV)
+    causal = fb.causal_mask(sq, DEV)
+
+    # padding mask through the general kernel
+    lengths = torch.tensor([256, 200, 64, 1], device=DEV)
+    pad = (pos.view(1, 1, 1, sq) >= lengths.view(b, 1, 1, 1)).expand(b, 1, sq, sq).contiguous()
+    core = CoreAttention(hn, 1, False, True, T.general, mask_func, attention_softmax_in_fp32=True)
+    assert rel_err(core(q, k, v, pad), textbook(q, k, v, pad)) <= lim
+
+    # the same padding by key lengths on the causal kernel
+    core = CoreAttention(hn, 1, False, True, T.upper_triang, mask_func, attention_softmax_in_fp32=True)
+    both = causal | pad
+    assert rel_err(core(q, k, v, causal, key_lengths=lengths.int()), textbook(q, k, v, both)) <= lim
+
+    # AliBi inside the kernel
+    slopes = AliBi(np_, 1, 0).slopes
+    core = CoreAttention(hn, 1, False, True, T.upper_triang, mask_func, attention_softmax_in_fp32=True, alibi_slopes=slopes)
+    dist = -(pos.view(sq, 1) - pos.view(1, sq)).clamp(min=0).float()
+    extra = dist.view(1, 1, sq, sq) * slopes.to(DEV).float().view(1, np_, 1, 1)
+    assert rel_err(core(q, k, v, causal), textbook(q, k, v, causal, extra)) <= lim
+
+    # sliding window of 32 keys
+    window = causal | (pos.view(1, sq) < pos.view(sq, 1) - 32).view(1, 1, sq, sq)
+    core = CoreAttention(hn, 1, False, True, T.upper_triang, mask_func, attention_softmax_in_fp32=True, sliding_window_width=32)
+    assert rel_err(core(q, k, v, window), textbook(q, k, v, window)) <= lim
+
+    # relative position bias handed to the kernel as a tensor
+    table = util.randn((1, np_, sq, sq), dtype, seed=3, std=0.5).to(DEV)
+    core = CoreAttention(hn, 1, False, True, T.upper_triang, mask_func, attention_softmax_in_fp32=True,
+                         rpe=lambda a, c: table[..., :a, :c])
+    assert rel_err(core(q, k, v, causal), textbook(q, k, v, causal, table.float())) <= lim
+
+
+def test_attention_dropout_inside_the_caller():
+    from megatron.model.attention_core import CoreAttention
+    from megatron.model.fused_softmax import SoftmaxFusionTypes as T
+
+    dtype, sq, b, np_, hn = torch.bfloat16, 256, 2, 4, 64
+    q, k, v = (t.detach() for t in qkv(dtype, sq, b, np_, hn, 21))
+    mask = fb.causal_mask(sq, DEV)
+    core = CoreAttention(hn, 1, False, True, T.upper_triang, mask_func, attention_softmax_in_fp32=True, attention_dropout=0.2)
+    core.eval()
+    quiet = core(q, k, v, mask)
+    assert rel_err(quiet, textbook(q, k, v, mask)) <= 2.0 ** -7
+    core.train()
+    torch.manual_seed(5)
+    a = core(q, k, v, mask)
+    torch.manual_seed(5)
+    again = core(q, k, v, mask)
+    torch.manual_seed(6)
+    other = core(q, k, v, mask)
+    assert torch.equal(a, again) and not torch.equal(a, other) and not torch.equal(a, quiet)
+    # dropout keeps the expectation: averaged over many masks the result approaches the plain one
+    acc = torch.zeros_like(quiet, dtype=torch.float32)
+    for i in range(64):
+        torch.manual_seed(100 + i)
+        acc += core(q, k, v, mask).float()
+    assert rel_err(acc / 64, quiet) <= 0.12

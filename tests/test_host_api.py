@@ -315,3 +315,36 @@ def test_sinusoidal_positional_embedding():
         want = torch.cat((torch.sin(pos * freq), torch.cos(pos * freq)), dim=-1)
         assert torch.allclose(out[0].double(), want, atol=1e-2 if precision == torch.bfloat16 else 1e-6)
         assert emb(torch.zeros(5, 3, 16), seq_dim=0).shape == (1, 5, 16)
+
+
+def test_core_attention_scaling_and_torch_branch_on_cpu():
+    """CoreAttention (the caller of the softmax, megatron/model/transformer.py:417-424, :526-625): the two scaling
+    factors, get_fusion_type, and the unfused branch in fp32 against textbook attention in float64."""
+    from megatron.model.attention_core import CoreAttention, get_fusion_type
+    from megatron.model.fused_softmax import SoftmaxFusionTypes as T
+
+    ns = types.SimpleNamespace
+    assert get_fusion_type(ns(scaled_upper_triang_masked_softmax_fusion=True, scaled_masked_softmax_fusion=True)) is T.upper_triang
+    assert get_fusion_type(ns(scaled_upper_triang_masked_softmax_fusion=False, scaled_masked_softmax_fusion=True)) is T.general
+    assert get_fusion_type(ns(scaled_upper_triang_masked_softmax_fusion=False, scaled_masked_softmax_fusion=False)) is T.none
+
+    def mask_func(scores, mask):
+        return fb.fill_masked_with_dtype_min(scores, mask)
+
+    core = CoreAttention(64, 5, False, False, T.none, mask_func, apply_query_key_layer_scaling=True)
+    assert core.norm_factor == 8 * 5 and core.scale_mask_softmax.scale == 5 and core.scale_mask_softmax.softmax_in_fp32
+    assert CoreAttention(64, 0, False, False, T.none, mask_func, apply_query_key_layer_scaling=True).norm_factor == 8
+    assert CoreAttention(64, 5, False, False, T.none, mask_func, use_mup=True).norm_factor == 64
+    sq, b, np_, hn = 24, 2, 3, 16
+    core = CoreAttention(hn, 3, False, False, T.none, mask_func, apply_query_key_layer_scaling=True)
+    q, k, v = (util.randn((sq, b, np_, hn), torch.float32, seed=i) for i in range(3))
+    mask = fb.causal_mask(sq, "cpu")
+    out = core(q, k, v, mask)
+    qd, kd, vd = (t.double().permute(1, 2, 0, 3) for t in (q, k, v))
+    scores = (qd @ kd.transpose(-1, -2) / math.sqrt(hn)).masked_fill(mask, float("-inf"))
+    want = torch.softmax(scores, -1) @ vd
+    assert out.shape == (b, np_, sq, hn) and torch.allclose(out.double(), want, atol=1e-5)
+    # with a KV cache the mask is cropped to the keys present
+    cached = CoreAttention(hn, 1, False, False, T.none, mask_func, use_cache=True)
+    big = fb.causal_mask(sq + 8, "cpu")
+    assert torch.allclose(cached(q, k, v, big).double(), want, atol=1e-5)
