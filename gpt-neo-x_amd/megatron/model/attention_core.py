@@ -92,3 +92,47 @@ class CoreAttention(torch.nn.Module):
         v = value_layer.reshape(sk, b * np_, value_layer.size(3))
         context = torch.bmm(probs.view(b * np_, sq, sk), v.transpose(0, 1))
         return context.view(b, np_, sq, value_layer.size(3))
+
+
+def apply_rotary_to_query_key(query_layer, key_layer, rotary_emb, rotary_ndims=None, rope_fusion=True, bf16=False,
+                              layer_past=None, one_launch=True):
+    """The rotary block of ``ParallelSelfAttention.forward`` (megatron/model/transformer.py:877-914).
+
+    ``query_layer`` ``[sq, b, np, hn]`` and ``key_layer`` ``[sq, b, nkv, hn]`` (possibly views of one fused
+    projection output); ``rotary_emb`` a ``RotaryEmbedding`` over ``rotary_ndims`` features (None: all
+    ``hn``); ``layer_past`` the cached ``(keys, values)`` of earlier positions when decoding.
+
+    ``one_launch=True`` (fused path only): a single kernel launch rotates q and k, copies the features
+    beyond ``rotary_ndims`` and starts at the position after the cache, so the slices, the two launches and
+    the two concatenations of the reference disappear -- and the cached positions are honoured, which the
+    reference's fused branch does not do (it passes no offset). ``one_launch=False`` follows the reference
+    statement by statement.
+    """
+    from .fused_rope import fused_apply_rotary_pos_emb_cached, fused_apply_rotary_pos_emb_qk_cached
+    from .positional_embeddings import apply_rotary_pos_emb, apply_rotary_pos_emb_torch
+
+    seq_len = key_layer.shape[0]
+    offset = 0
+    if layer_past is not None and layer_past.numel() > 0:
+        offset = layer_past[0].shape[0]
+        seq_len += offset
+    cos, sin = rotary_emb(key_layer, seq_len=seq_len)
+    if rope_fusion and one_launch:
+        return fused_apply_rotary_pos_emb_qk_cached(query_layer, key_layer, cos, sin, offset=offset)
+
+    if rotary_ndims is not None:
+        query_rot, query_pass = query_layer[..., :rotary_ndims], query_layer[..., rotary_ndims:]
+        key_rot, key_pass = key_layer[..., :rotary_ndims], key_layer[..., rotary_ndims:]
+    else:
+        query_rot, key_rot = query_layer, key_layer
+    if rope_fusion:
+        # as the reference: positions 0..sq-1 whatever the cache holds
+        rows = slice(0, query_rot.shape[0])
+        query_layer, key_layer = (fused_apply_rotary_pos_emb_cached(rot, cos[rows], sin[rows]) for rot in (query_rot, key_rot))
+    else:
+        eager = apply_rotary_pos_emb_torch if bf16 else apply_rotary_pos_emb
+        query_layer, key_layer = eager(query_rot, key_rot, cos, sin, offset=offset)
+    if rotary_ndims is not None:
+        query_layer = torch.cat((query_layer, query_pass), dim=-1)
+        key_layer = torch.cat((key_layer, key_pass), dim=-1)
+    return query_layer, key_layer

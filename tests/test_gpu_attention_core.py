@@ -136,3 +136,51 @@ def test_attention_dropout_inside_the_caller():
         torch.manual_seed(100 + i)
         acc += core(q, k, v, mask).float()
     assert rel_err(acc / 64, quiet) <= 0.12
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("rotary_ndims", [None, 32], ids=["full", "partial"])
+def test_rotary_call_site(dtype, rotary_ndims):
+    """apply_rotary_to_query_key (the rotary block of ParallelSelfAttention.forward, transformer.py:877-914) on q and k
+    sliced from one fused projection output: the single-launch path, the reference's statement-by-statement fused
+    path and the eager path agree bit for bit; with cached keys the single launch follows the eager path (which
+    honours the offset), the reference's fused branch does not."""
+    from megatron.model.attention_core import apply_rotary_to_query_key
+    from megatron.model.positional_embeddings import RotaryEmbedding
+
+    sq, b, np_, hn = 96, 2, 4, 128
+    qkv_out = util.randn((sq, b, np_, 3 * hn), dtype, seed=4).to(DEV)
+    q, k = qkv_out[..., :hn], qkv_out[..., hn:2 * hn]
+    emb = RotaryEmbedding(rotary_ndims or hn, 256, base=10000, precision=dtype)
+    bf16 = dtype == torch.bfloat16
+
+    def run(**kw):
+        return apply_rotary_to_query_key(q, k, emb, rotary_ndims=rotary_ndims, bf16=bf16, **kw)
+
+    one = run(rope_fusion=True, one_launch=True)
+    two = run(rope_fusion=True, one_launch=False)
+    eager = run(rope_fusion=False)
+    for got in (one, two):
+        for a, e in zip(got, eager):
+            assert a.shape == (sq, b, np_, hn) and a.is_contiguous()
+            assert torch.equal(util.raw_bits(a), util.raw_bits(e))
+    # decoding: 40 cached positions
+    past = torch.zeros((2, 40, b, np_, hn), dtype=dtype, device=DEV)
+    one = run(rope_fusion=True, one_launch=True, layer_past=past)
+    eager = run(rope_fusion=False, layer_past=past)
+    ref_style = run(rope_fusion=True, one_launch=False, layer_past=past)
+    for a, e, r, plain in zip(one, eager, ref_style, two):
+        assert torch.equal(util.raw_bits(a), util.raw_bits(e))
+        assert torch.equal(util.raw_bits(r), util.raw_bits(plain))     # positions 0..sq-1 whatever the cache holds
+        assert not torch.equal(util.raw_bits(a), util.raw_bits(r))
+    # gradients flow through both fused paths and agree
+    qa = q.detach().clone().requires_grad_(True)
+    ka = k.detach().clone().requires_grad_(True)
+    outs = apply_rotary_to_query_key(qa, ka, emb, rotary_ndims=rotary_ndims, rope_fusion=True, one_launch=True)
+    gq, gk = util.randn((sq, b, np_, hn), dtype, seed=7).to(DEV), util.randn((sq, b, np_, hn), dtype, seed=8).to(DEV)
+    torch.autograd.backward(outs, (gq, gk))
+    qb = q.detach().clone().requires_grad_(True)
+    kb = k.detach().clone().requires_grad_(True)
+    outs = apply_rotary_to_query_key(qb, kb, emb, rotary_ndims=rotary_ndims, rope_fusion=True, one_launch=False)
+    torch.autograd.backward(outs, (gq, gk))
+    assert torch.equal(util.raw_bits(qa.grad), util.raw_bits(qb.grad)) and torch.equal(util.raw_bits(ka.grad), util.raw_bits(kb.grad))
