@@ -150,6 +150,25 @@ def test_layer_kernels_random_shapes(hotpath, seed):
                              None) == 0
     want_r, _ = oracle.rmsnorm_fwd(x, gamma, None, 1e-5, mode)
     util.assert_close_ulp_or_noise(y.cpu(), want_r, 2, noise_y, "rmsnorm fwd")
+    # partial statistic (any number of leading columns) and the clamped-norm definition, forward and backward
+    stat = rng.randint(1, cols)
+    pmode = rng.choice((0, 1, 2))
+    assert L.nhp_rmsnorm_partial_fwd(y.data_ptr(), inv.data_ptr(), xd.data_ptr(), gmd.data_ptr(), None, 1e-3, pmode, rows, cols,
+                                     stat, code, code, None) == 0
+    want_p, want_inv = oracle.rmsnorm_fwd(x, gamma, None, 1e-3, pmode, stat_cols=stat)
+    grow = (x.float().abs() * want_inv[:, None]).clamp(min=1.0)
+    util.assert_close_ulp_or_noise(y.cpu(), want_p, 2, noise_y * grow, f"partial rmsnorm fwd, stat {stat} mode {pmode}")
+    assert torch.allclose(inv.cpu(), want_inv, rtol=1e-5, atol=0)
+    assert L.nhp_rmsnorm_partial_bwd(dx.data_ptr(), dg.data_ptr(), None, gd.data_ptr(), xd.data_ptr(), inv.data_ptr(),
+                                     gmd.data_ptr(), nws.data_ptr(), 1e-3, pmode, rows, cols, stat, code, code, None) == 0
+    icpu = inv.cpu()
+    want_pdx, want_pds, _ = oracle.rmsnorm_bwd(g, x, icpu, gamma, 1e-3, pmode, stat_cols=stat)
+    xh = (x.float() * icpu[:, None]).abs()
+    denom = 1.0 if pmode == 2 else float(stat)
+    pnoise = ((g.float().abs() * gamma.float().abs() * xh).sum(-1, keepdim=True) * xh * icpu[:, None] / denom * 256 * util.EPS32
+              + (g.float().abs() * gamma.float().abs()) * icpu[:, None] * 16 * util.EPS32)
+    util.assert_close_ulp_or_noise(dx.cpu(), want_pdx, 2, pnoise, f"partial rmsnorm dx, stat {stat} mode {pmode}")
+    util.assert_close_ulp_or_noise(dg.cpu(), want_pds, 2, (g.float().abs() * xh).sum(0) * 32 * util.EPS32, "partial rmsnorm dscale")
     # gated activation on the same data when the width is even
     if cols % 2 == 0:
         act = rng.choice(sorted(oracle.GATE_ACTS))
