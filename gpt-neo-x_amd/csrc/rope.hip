@@ -211,6 +211,98 @@ rope_vec_kernel(RopePair pair, Tables tab, int cpr, int rot_chunks, int rpw)
 }
 
 // ---------------------------------------------------------------------------
+// Transposing kernel: the input is contiguous along the sequence (stride_s == 1,
+// features stride_d apart), the output along the features. This is the layout in
+// which the gradient of the keys arrives from the backward of the score GEMM
+// (q k^T hands its second operand's gradient over as [b, h, d, s]).
+//   grid  = (b * h rows, ceil(s / 64)), block = 256 threads
+//   phase 1: 16-byte loads along s (8 lanes cover the 64 positions of one
+//            feature), written to LDS transposed, one 16-bit element at a time;
+//            the chunk slot of a feature is XOR-ed with the load chunk index so
+//            that the 8 lanes of a feature hit 8 different bank groups
+//   phase 2: one lane per (position, feature chunk) reads its chunk and the
+//            partner chunk from LDS, rotates, and stores 16 bytes
+// 16-bit data only; P = ceil(d / 32) load passes, all in flight together.
+// Requires: s % 8 == 0, stride_d and the batch / head strides multiples of 8,
+// output stride_d == 1, aligned pointers and tables, d % 8 == 0, d2 % 16 == 0.
+// ---------------------------------------------------------------------------
+constexpr int kTrTile = 64;  // positions per workgroup
+
+template <int DT, bool BWD, int P, typename Tables>
+__global__ void __launch_bounds__(256)
+rope_tr_kernel(RopeTensor T, Tables tab, int s, int cpr, int rot_chunks, int row_chunks, int64_t is_d)
+{
+    static_assert(DT != NHP_F32, "16-bit data");
+    constexpr int V = 8;
+    extern __shared__ u32x4 tile[];  // [kTrTile][row_chunks] chunks of 8 elements
+    uint16_t* tile16 = reinterpret_cast<uint16_t*>(tile);
+    const int tid = threadIdx.x;
+    const int r = blockIdx.x;
+    const int s0 = blockIdx.y * kTrTile;
+    const int bi = r / T.h;
+    const int hi = r - bi * T.h;
+    const int d = cpr * V;
+    const uint16_t* in = static_cast<const uint16_t*>(T.in) + bi * T.is_b + hi * T.is_h;
+    uint16_t* out = static_cast<uint16_t*>(T.out) + bi * T.os_b + hi * T.os_h;
+
+    const int sc = tid & 7;   // which 8 positions of the tile
+    const int dr = tid >> 3;  // feature within a pass of 32
+    const int pos8 = s0 + sc * 8;
+    u32x4 raw[P];
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+        const int di = p * 32 + dr;
+        raw[p] = u32x4{0, 0, 0, 0};
+        if (di < d && pos8 < s) raw[p] = load16_stream(in + (int64_t)di * is_d + pos8);
+    }
+    const int row_elems = row_chunks * V;
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+        const int di = p * 32 + dr;
+        if (di < d) {
+            const int slot = ((di >> 3) ^ sc) * V + (di & 7);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint32_t word = raw[p][j >> 1];
+                tile16[(sc * 8 + j) * row_elems + slot] = (uint16_t)((j & 1) ? (word >> 16) : (word & 0xffffu));
+            }
+        }
+    }
+    __syncthreads();
+
+    const int half = rot_chunks / 2;
+    for (int idx = tid; idx < kTrTile * cpr; idx += 256) {
+        const int row = idx / cpr;
+        const int c = idx - row * cpr;
+        const int pos = s0 + row;
+        if (pos >= s) continue;
+        const int swz = row >> 3;
+        const u32x4 x = tile[row * row_chunks + (c ^ swz)];
+        u32x4 res = x;
+        if (c < rot_chunks) {
+            const bool first = c < half;
+            const int pc = first ? c + half : c - half;
+            const u32x4 px = tile[row * row_chunks + (pc ^ swz)];
+            float cv[V], sv[V], unused[V], xf[V], pf[V], y[V];
+            if (!BWD) {
+                tab.get_vec(pos, (int64_t)c * V, cv, sv);
+            } else {
+                tab.get_vec(pos, (int64_t)c * V, cv, unused);
+                tab.get_vec(pos, (int64_t)pc * V, unused, sv);
+            }
+            const bool negate = BWD ? !first : first;
+            chunk_to_float<DT>(x, xf);
+            chunk_to_float<DT>(px, pf);
+#pragma unroll
+            for (int v = 0; v < V; ++v)
+                y[v] = negate ? rot<DT, true>(xf[v], cv[v], pf[v], sv[v]) : rot<DT>(xf[v], cv[v], pf[v], sv[v]);
+            res = float_to_chunk<DT>(y);
+        }
+        store16_stream(out + (int64_t)pos * T.os_s + (int64_t)c * V, res);
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Scalar kernel: one thread per element, any strides, any d2.
 // Index arithmetic follows fused_rotary_positional_embedding.h:27-225 of the
 // reference, including odd d2 (h2 = d2/2 rounded down).
@@ -343,10 +435,62 @@ static int rope_launch_vec(const RopeArgs& a, const RopeArgs* b, const Tables& t
     return hipGetLastError() == hipSuccess ? NHP_OK : NHP_ERR_LAUNCH;
 }
 
+// LDS row length (in chunks) of the transposing kernel: the XOR with the load chunk index needs a
+// power-of-two number of slots (at least 8), one more chunk staggers the rows over the banks.
+static int tr_row_chunks(int64_t cpr)
+{
+    int n = 8;
+    while (n < cpr) n *= 2;
+    return n + 1;
+}
+
+template <int DT>
+static bool transposed_ok(const RopeArgs& a, bool tables_ok)
+{
+    if (DT == NHP_F32 || !tables_ok) return false;
+    if (a.is[0] != 1 || a.os[3] != 1 || a.is[3] % 8 != 0) return false;
+    if (a.s % 8 != 0 || a.d % 8 != 0 || a.d2 % 16 != 0 || a.d > 256) return false;
+    const int64_t passes = (a.d + 31) / 32;
+    if (passes != 2 && passes != 3 && passes != 4 && passes != 8) return false;
+    if (a.is[1] % 8 != 0 || a.is[2] % 8 != 0) return false;
+    for (int i = 0; i < 3; ++i)
+        if (a.os[i] % 8 != 0) return false;
+    if (!is_aligned16(a.in) || !is_aligned16(a.out)) return false;
+    if (a.b * a.h >= ((int64_t)1 << 31) || (a.s + kTrTile - 1) / kTrTile > 65535) return false;
+    return true;
+}
+
+template <int DT, bool BWD, typename Tables>
+static int rope_launch_transposed(const RopeArgs& a, const Tables& tab)
+{
+    if constexpr (DT == NHP_F32) {
+        return NHP_ERR_SHAPE;
+    } else {
+        const int cpr = (int)(a.d / 8);
+        const int row_chunks = tr_row_chunks(cpr);
+        const uint32_t lds = (uint32_t)(kTrTile * row_chunks * 16);
+        const dim3 grid((uint32_t)(a.b * a.h), (uint32_t)((a.s + kTrTile - 1) / kTrTile));
+        const RopeTensor t = rope_tensor(a);
+#define CASE(P_)                                                                                              \
+    case P_:                                                                                                  \
+        rope_tr_kernel<DT, BWD, P_, Tables><<<grid, 256, lds, a.st>>>(t, tab, (int)a.s, cpr, (int)(a.d2 / 8),   \
+                                                                      row_chunks, a.is[3]);                   \
+        break;
+        switch ((int)((a.d + 31) / 32)) {
+            CASE(2) CASE(3) CASE(4) CASE(8)
+        default:
+            return NHP_ERR_SHAPE;
+        }
+#undef CASE
+        return hipGetLastError() == hipSuccess ? NHP_OK : NHP_ERR_LAUNCH;
+    }
+}
+
 template <int DT, bool BWD, typename Tables>
 static int rope_launch(const RopeArgs& a, const Tables& tab, bool tables_ok)
 {
     if (vector_ok<DT>(a, tables_ok)) return rope_launch_vec<DT, BWD>(a, nullptr, tab);
+    if (transposed_ok<DT>(a, tables_ok)) return rope_launch_transposed<DT, BWD>(a, tab);
     return rope_launch_scalar<DT, BWD>(a, tab);
 }
 

@@ -18,31 +18,43 @@ from torch import Tensor
 from ..fused_kernels import _hotpath as _hp
 
 
-def _launch(x, bias, residual):
-    what = "bias_dropout_add"
+def _bias_vector(bias, x, what):
+    """The bias as a contiguous ``[cols]`` vector, and whether it came expanded to the shape of ``x``
+    (the reference's call sites pass ``bias.expand_as(residual)``, megatron/model/transformer.py:1229,1271)."""
+    if bias is None:
+        return None, False
+    cols = x.size(-1)
+    _hp.require_gpu(bias, what)
+    if bias.dtype != x.dtype:
+        raise RuntimeError(f"{what}: bias must hold one value per feature, in the dtype of x")
+    if bias.numel() == cols:
+        return bias.contiguous().view(-1), False
+    if bias.shape == x.shape and all(st == 0 or sz == 1 for st, sz in zip(bias.stride()[:-1], bias.shape[:-1])):
+        row = bias.detach().as_strided((cols,), (bias.stride(-1),), bias.storage_offset())
+        return row.contiguous(), True
+    raise RuntimeError(f"{what}: bias must hold one value per feature (a vector, or one expanded to the shape of x)")
+
+
+def _prepare(x, bias, residual, what):
     _hp.require_gpu(x, what)
     cols = x.size(-1)
     src = x.contiguous()
-    b = None
-    if bias is not None:
-        if bias.numel() != cols or bias.dtype != x.dtype:
-            raise RuntimeError(f"{what}: bias must hold one value per feature, in the dtype of x")
-        _hp.require_gpu(bias, what)
-        b = bias.contiguous().view(-1)
+    b, expanded = _bias_vector(bias, x, what)
     res = None
     if residual is not None:
         if residual.shape != x.shape or residual.dtype != x.dtype:
             raise RuntimeError(f"{what}: residual and x must have the same shape and dtype")
         _hp.require_gpu(residual, what)
         res = residual.contiguous()
-    out = torch.empty_like(src)
-    rows = src.numel() // max(cols, 1)
-    with _hp.device_guard(src):
-        rc = _hp.lib().nhp_bias_add_residual(out.data_ptr(), src.data_ptr(), None if b is None else b.data_ptr(),
-                                             None if res is None else res.data_ptr(), rows, cols,
-                                             _hp.dtype_code(src, what), _hp.stream_of(src))
-    _hp.check(rc, what)
-    return out
+    return src, b, res, src.numel() // max(cols, 1), cols, expanded
+
+
+def _bias_grad(per_element, bias_shape, expanded):
+    """Gradient for the bias argument: of an expanded bias every element has its own gradient (autograd
+    sums them when it undoes the expansion); for a vector the rows are summed here."""
+    if expanded:
+        return per_element
+    return per_element.reshape(-1, per_element.size(-1)).sum(dim=0).view(bias_shape)
 
 
 class _BiasAddResidual(torch.autograd.Function):
@@ -51,34 +63,24 @@ class _BiasAddResidual(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, bias, residual):
-        ctx.bias_shape = None if bias is None else bias.shape
-        return _launch(x, bias, residual)
+        what = "bias_dropout_add"
+        src, b, res, rows, cols, expanded = _prepare(x, bias, residual, what)
+        out = torch.empty_like(src)
+        with _hp.device_guard(src):
+            rc = _hp.lib().nhp_bias_add_residual(out.data_ptr(), src.data_ptr(), None if b is None else b.data_ptr(),
+                                                 None if res is None else res.data_ptr(), rows, cols,
+                                                 _hp.dtype_code(src, what), _hp.stream_of(src))
+        _hp.check(rc, what)
+        ctx.conf = (None if bias is None else bias.shape, expanded)
+        return out
 
     @staticmethod
     def backward(ctx, grad):
+        bias_shape, expanded = ctx.conf
         gb = None
-        if ctx.bias_shape is not None and ctx.needs_input_grad[1]:
-            gb = grad.reshape(-1, grad.size(-1)).sum(dim=0).view(ctx.bias_shape)
+        if bias_shape is not None and ctx.needs_input_grad[1]:
+            gb = _bias_grad(grad, bias_shape, expanded)
         return grad, gb, grad if ctx.needs_input_grad[2] else None
-
-
-def _prepare(x, bias, residual, what):
-    _hp.require_gpu(x, what)
-    cols = x.size(-1)
-    src = x.contiguous()
-    b = None
-    if bias is not None:
-        if bias.numel() != cols or bias.dtype != x.dtype:
-            raise RuntimeError(f"{what}: bias must hold one value per feature, in the dtype of x")
-        _hp.require_gpu(bias, what)
-        b = bias.contiguous().view(-1)
-    res = None
-    if residual is not None:
-        if residual.shape != x.shape or residual.dtype != x.dtype:
-            raise RuntimeError(f"{what}: residual and x must have the same shape and dtype")
-        _hp.require_gpu(residual, what)
-        res = residual.contiguous()
-    return src, b, res, src.numel() // max(cols, 1), cols
 
 
 class _BiasDropoutAdd(torch.autograd.Function):
@@ -87,20 +89,20 @@ class _BiasDropoutAdd(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, bias, residual, prob, seed):
         what = "bias_dropout_add"
-        src, b, res, rows, cols = _prepare(x, bias, residual, what)
+        src, b, res, rows, cols, expanded = _prepare(x, bias, residual, what)
         out = torch.empty_like(src)
         with _hp.device_guard(src):
             rc = _hp.lib().nhp_bias_dropout_add(out.data_ptr(), src.data_ptr(), None if b is None else b.data_ptr(),
                                                 None if res is None else res.data_ptr(), rows, cols, float(prob), seed,
                                                 0, _hp.dtype_code(src, what), _hp.stream_of(src))
         _hp.check(rc, what)
-        ctx.conf = (float(prob), seed, None if bias is None else bias.shape)
+        ctx.conf = (float(prob), seed, None if bias is None else bias.shape, expanded)
         return out
 
     @staticmethod
     def backward(ctx, grad):
         what = "bias_dropout_add backward"
-        prob, seed, bias_shape = ctx.conf
+        prob, seed, bias_shape, expanded = ctx.conf
         g = grad.contiguous()
         cols = g.size(-1)
         rows = g.numel() // max(cols, 1)
@@ -111,7 +113,7 @@ class _BiasDropoutAdd(torch.autograd.Function):
         _hp.check(rc, what)
         gb = None
         if bias_shape is not None and ctx.needs_input_grad[1]:
-            gb = dx.reshape(-1, cols).sum(dim=0).view(bias_shape)
+            gb = _bias_grad(dx, bias_shape, expanded)
         return dx, gb, grad if ctx.needs_input_grad[2] else None, None, None
 
 

@@ -401,3 +401,31 @@ def test_python_functions_accept_non_contiguous_inputs():
     leaf = base.clone().requires_grad_(True)
     ln(leaf.transpose(0, 1)).sum().backward()
     assert leaf.grad.shape == leaf.shape and torch.isfinite(leaf.grad.float()).all()
+
+
+@pytest.mark.parametrize("prob", [0.0, 0.3], ids=["no-dropout", "dropout"])
+def test_bias_dropout_add_takes_the_expanded_bias_of_the_reference_call_sites(prob):
+    """The reference's layer passes ``bias.expand_as(residual)`` (megatron/model/transformer.py:1229, 1271): same
+    result as the vector, and the gradient reaches the vector through autograd's sum over the expansion."""
+    from megatron.model.fused_bias_dropout import bias_dropout_add_fused_train
+
+    dtype = torch.bfloat16
+    x = util.randn((24, 3, 256), dtype, seed=1).to(DEV).requires_grad_(True)
+    res = util.randn((24, 3, 256), dtype, seed=2).to(DEV).requires_grad_(True)
+    g = util.randn((24, 3, 256), dtype, seed=3).to(DEV)
+    va = util.randn((256,), dtype, seed=4).to(DEV).requires_grad_(True)
+    vb = va.detach().clone().requires_grad_(True)
+    torch.manual_seed(11)
+    a = bias_dropout_add_fused_train(x, va.expand_as(res), res, prob)
+    a.backward(g)
+    ga, gx, gr = va.grad.clone(), x.grad.clone(), res.grad.clone()
+    x.grad = res.grad = None
+    torch.manual_seed(11)
+    b = bias_dropout_add_fused_train(x, vb, res, prob)
+    b.backward(g)
+    assert torch.equal(a, b) and torch.equal(gx, x.grad) and torch.equal(gr, res.grad)
+    assert ga.shape == (256,)
+    # both are sums of the same 72 bf16 values per column, formed in different orders and widths
+    assert torch.allclose(ga.float(), vb.grad.float(), rtol=2.0 ** -6, atol=2.0 ** -6)
+    with pytest.raises(RuntimeError, match="one value per feature"):
+        bias_dropout_add_fused_train(x, torch.zeros_like(res), res, prob)   # a genuinely full-size "bias"

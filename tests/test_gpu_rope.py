@@ -236,3 +236,37 @@ def test_fused_qk_function_matches_eager_apply_with_offset(dtype, offset):
     assert torch.equal(util.raw_bits(fk.detach().cpu()), util.raw_bits(ok.detach()))
     assert torch.equal(util.raw_bits(qd.grad.cpu()), util.raw_bits(qe.grad))
     assert torch.equal(util.raw_bits(kd.grad.cpu()), util.raw_bits(ke.grad))
+
+
+# (s, b, h, d, d2): tile boundaries (s around 64), every number of load passes, partial rotary, shapes the
+# transposing kernel refuses (s not a multiple of 8, d beyond 256) and that fall back to the scalar kernel
+SEQ_MAJOR = [(64, 2, 3, 128, 128), (200, 2, 4, 128, 32), (72, 1, 5, 64, 64), (136, 2, 2, 96, 48), (8, 2, 2, 80, 16),
+             (256, 1, 2, 256, 256), (120, 3, 2, 128, 64), (30, 2, 2, 128, 32), (16, 1, 2, 512, 64)]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("shape", SEQ_MAJOR, ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("cs_fp32", [False, True], ids=["cs_same", "cs_fp32"])
+def test_rope_input_contiguous_along_the_sequence(hotpath, shape, dtype, cs_fp32):
+    """The layout in which the key gradient reaches the rotary backward in the attention layer: the backward of
+    the score GEMM leaves it as [b, h, d, s], seen as [s, b, h, d] with element strides (1, h*d*s, d*s, s)
+    (megatron/model/transformer.py:556-562 and autograd's baddbmm formula). Bit-exact like every other layout."""
+    s, b, h, d, d2 = shape
+    say(f"rope sequence-major {shape} {dtype} cs_fp32={cs_fp32}")
+    base = util.randn((b, h, d, s), dtype, seed=s + d)
+    t = base.permute(3, 0, 1, 2)
+    t_d = base.to(DEV).permute(3, 0, 1, 2)
+    assert t_d.stride() == (1, h * d * s, d * s, s)
+    cos, sin, _ = generic_tables(d2, s, dtype, cs_fp32, seed=d2)
+    for backward in (False, True):
+        for transpose in (False, True):
+            want = oracle.rope_cached(t.contiguous(), cos, sin, backward=backward, transpose_output=transpose)
+            got = util.abi_rope_cached(hotpath, t_d, cos.to(DEV), sin.to(DEV), backward, transpose)
+            assert got.stride() == want.stride()
+            assert torch.equal(util.raw_bits(got.cpu()), util.raw_bits(want)), (backward, transpose)
+    # a window of a longer sequence: the feature stride exceeds the number of positions
+    if s >= 16:
+        w = t_d[8:s - 0]
+        want = oracle.rope_cached(t[8:].contiguous(), cos[: s - 8].contiguous(), sin[: s - 8].contiguous(), backward=True)
+        got = util.abi_rope_cached(hotpath, w, cos[: s - 8].contiguous().to(DEV), sin[: s - 8].contiguous().to(DEV), True)
+        assert torch.equal(util.raw_bits(got.cpu()), util.raw_bits(want))
