@@ -14,6 +14,10 @@
 // workgroup stays on one sequence position and walks over the (batch, head)
 // rows, re-using the cos/sin values it loaded (or computed) once.
 //
+// Transposing kernel, for 16-bit inputs that are contiguous along the sequence
+// instead of along the features (see rope_tr_kernel). Everything else (odd
+// sizes, unaligned pointers, other strides) takes the scalar kernel.
+//
 // Arithmetic: out = (x (*) c) (+) (r (*) s) where every product and the sum
 // are rounded to the data dtype, which is what the scalar types of the
 // reference kernels and eager torch do.

@@ -103,7 +103,7 @@ def backward_cached(output_grads, cos, sin, transpose_output):
                        output_grads, cos, sin, transpose_output, "output_grads")
 
 
-def _run_cached_qk(name, fn, q, k, cos, sin, transpose_output):
+def _run_cached_qk(name, fn, q, k, cos, sin, transpose_output, out=None):
     for t, what in ((q, "q"), (k, "k")):
         _check(t.dim() == 4, "expected 4D tensor")
         _check(t.size(0) == cos.size(0), f"expected {what} and cos tensor have the same sequence length")
@@ -124,8 +124,15 @@ def _run_cached_qk(name, fn, q, k, cos, sin, transpose_output):
     _hp.require_gpu(sin, name)
     c = cos.contiguous()
     sn = sin.contiguous()
-    q_out = _new_output(q, transpose_output)
-    k_out = _new_output(k, transpose_output)
+    if out is None:
+        q_out = _new_output(q, transpose_output)
+        k_out = _new_output(k, transpose_output)
+    else:
+        # caller-provided results with any strides, e.g. two slices of one buffer
+        q_out, k_out = out
+        for o, t, what in ((q_out, q, "q"), (k_out, k, "k")):
+            _check(o.shape == t.shape and o.dtype == t.dtype and o.device == t.device,
+                   f"{name}: the result tensor for {what} must match it in shape, dtype and device")
     s, b, hq, d = q.shape
     with _hp.device_guard(q):
         rc = fn(q_out.data_ptr(), k_out.data_ptr(), q.data_ptr(), k.data_ptr(), c.data_ptr(), sn.data_ptr(), s, b, hq,
@@ -135,13 +142,15 @@ def _run_cached_qk(name, fn, q, k, cos, sin, transpose_output):
     return q_out, k_out
 
 
-def forward_cached_qk(q, k, cos, sin, transpose_output):
-    """(not in the reference module) ``forward_cached`` for q and k in one launch; k may have fewer heads."""
+def forward_cached_qk(q, k, cos, sin, transpose_output, out=None):
+    """(not in the reference module) ``forward_cached`` for q and k in one launch; k may have fewer heads.
+    ``out``: optional ``(q_result, k_result)`` tensors to write into (any strides) instead of new ones."""
     return _run_cached_qk("fused_rotary_positional_embedding.forward_cached_qk", _hp.lib().nhp_rope_cached_qk_fwd, q, k,
-                          cos, sin, transpose_output)
+                          cos, sin, transpose_output, out)
 
 
-def backward_cached_qk(grad_q, grad_k, cos, sin, transpose_output):
-    """(not in the reference module) ``backward_cached`` for the gradients of q and k in one launch."""
+def backward_cached_qk(grad_q, grad_k, cos, sin, transpose_output, out=None):
+    """(not in the reference module) ``backward_cached`` for the gradients of q and k in one launch.
+    ``out``: optional ``(q_result, k_result)`` tensors to write into (any strides) instead of new ones."""
     return _run_cached_qk("fused_rotary_positional_embedding.backward_cached_qk", _hp.lib().nhp_rope_cached_qk_bwd,
-                          grad_q, grad_k, cos, sin, transpose_output)
+                          grad_q, grad_k, cos, sin, transpose_output, out)

@@ -136,3 +136,58 @@ def apply_rotary_to_query_key(query_layer, key_layer, rotary_emb, rotary_ndims=N
         query_layer = torch.cat((query_layer, query_pass), dim=-1)
         key_layer = torch.cat((key_layer, key_pass), dim=-1)
     return query_layer, key_layer
+
+
+class _SplitRotaryQKV(torch.autograd.Function):
+    """``[sq, b, np, 3 * hn]`` -> rotated q, rotated k (new contiguous tensors) and v (a view).
+
+    Forward: one rotary launch reads q and k straight from the projection output. Backward: the two rotary
+    backward kernels write into their slices of one gradient buffer for the projection output and the
+    gradient of v is copied into the third slice, which replaces the concatenation that undoes
+    ``torch.split`` (a pass over all three tensors) by a copy of one."""
+
+    @staticmethod
+    def forward(ctx, mixed, cos, sin):
+        import fused_rotary_positional_embedding as ext
+
+        hn = mixed.size(-1) // 3
+        ctx.save_for_backward(cos, sin)
+        q_rot, k_rot = ext.forward_cached_qk(mixed[..., :hn], mixed[..., hn:2 * hn], cos, sin, False)
+        return q_rot, k_rot, mixed[..., 2 * hn:]
+
+    @staticmethod
+    def backward(ctx, grad_q, grad_k, grad_v):
+        import fused_rotary_positional_embedding as ext
+
+        cos, sin = ctx.saved_tensors
+        like = next(g for g in (grad_q, grad_k, grad_v) if g is not None)
+        sq, b, np_, hn = like.shape
+        grad = torch.empty((sq, b, np_, 3 * hn), dtype=like.dtype, device=like.device)
+        gq, gk, gv = grad[..., :hn], grad[..., hn:2 * hn], grad[..., 2 * hn:]
+        if grad_q is not None and grad_k is not None:
+            ext.backward_cached_qk(grad_q, grad_k, cos, sin, False, out=(gq, gk))
+        else:
+            for dst, g in ((gq, grad_q), (gk, grad_k)):
+                if g is None:
+                    dst.zero_()
+                else:
+                    dst.copy_(ext.backward_cached(g, cos, sin, False))
+        if grad_v is None:
+            gv.zero_()
+        else:
+            gv.copy_(grad_v)
+        return grad, None, None
+
+
+def split_qkv_and_rotate(mixed_x_layer, rotary_emb, layer_past=None):
+    """The split of the fused projection output and the rotary block of ``ParallelSelfAttention.forward``
+    (megatron/model/transformer.py:852-914) as one differentiable step: ``mixed_x_layer`` is
+    ``[sq, b, np, 3 * hn]``; returns ``(query, key, value)``, each ``[sq, b, np, hn]``, query and key rotated
+    over the first ``rotary_emb.dim`` features starting at the position after the cached keys."""
+    seq_len = mixed_x_layer.shape[0]
+    offset = 0
+    if layer_past is not None and layer_past.numel() > 0:
+        offset = layer_past[0].shape[0]
+    cos, sin = rotary_emb(mixed_x_layer, seq_len=seq_len + offset)
+    rows = slice(offset, offset + seq_len)
+    return _SplitRotaryQKV.apply(mixed_x_layer, cos[rows], sin[rows])

@@ -8,7 +8,8 @@ the GEMMs is one of the fused kernels:
 
     norm                      nhp_layernorm / nhp_rmsnorm
     qkv projection            GEMM (bias added by the GEMM, as ColumnParallelLinear does for qkv)
-    rotary on q and k         nhp_rope_cached_qk on the two views of the projection output
+    rotary on q and k         nhp_rope_cached_qk on the two views of the projection output; its backward writes
+                              into the gradient of the projection output (no concatenation)
     scores / probs / context  CoreAttention: GEMM, fused softmax (+ dropout), GEMM
     output projection         GEMM, bias handed on
     bias + dropout + residual nhp_bias_add_residual / nhp_bias_dropout_add
@@ -24,7 +25,7 @@ import torch
 import torch.nn.functional as F
 
 from .activations import Gated_Activation, get_activation
-from .attention_core import CoreAttention, apply_rotary_to_query_key, get_fusion_type
+from .attention_core import CoreAttention, apply_rotary_to_query_key, get_fusion_type, split_qkv_and_rotate
 from .fused_bias_dropout import bias_dropout_add_fused_inference, bias_dropout_add_fused_train, get_bias_dropout_add
 from .norms import get_norm
 from .positional_embeddings import AliBi, RotaryEmbedding
@@ -122,10 +123,13 @@ class SelfAttention(torch.nn.Module):
         mixed, _ = self.query_key_value(hidden_states)
         # [sq, b, np * 3 * hn] -> [sq, b, np, 3 * hn] -> three views [sq, b, np, hn]
         mixed = mixed.view(sq, b, self.num_heads, 3 * self.head_dim)
-        query, key, value = torch.split(mixed, self.head_dim, dim=-1)
-        if self.rotary_emb is not None:
-            query, key = apply_rotary_to_query_key(query, key, self.rotary_emb, rotary_ndims=self.rotary_ndims,
-                                                   rope_fusion=self.rope_fusion, bf16=self.bf16)
+        if self.rotary_emb is not None and self.rope_fusion:
+            query, key, value = split_qkv_and_rotate(mixed, self.rotary_emb)
+        else:
+            query, key, value = torch.split(mixed, self.head_dim, dim=-1)
+            if self.rotary_emb is not None:
+                query, key = apply_rotary_to_query_key(query, key, self.rotary_emb, rotary_ndims=self.rotary_ndims,
+                                                       rope_fusion=False, bf16=self.bf16)
         context = self.core(query, key, value, attention_mask)
         # [b, np, sq, hn] -> [sq, b, np * hn]
         context = context.permute(2, 0, 1, 3).contiguous().view(sq, b, self.num_heads * self.head_dim)

@@ -184,3 +184,41 @@ def test_rotary_call_site(dtype, rotary_ndims):
     outs = apply_rotary_to_query_key(qb, kb, emb, rotary_ndims=rotary_ndims, rope_fusion=True, one_launch=False)
     torch.autograd.backward(outs, (gq, gk))
     assert torch.equal(util.raw_bits(qa.grad), util.raw_bits(qb.grad)) and torch.equal(util.raw_bits(ka.grad), util.raw_bits(kb.grad))
+
+
+@pytest.mark.parametrize("rotary_ndims", [None, 32], ids=["full", "partial"])
+def test_split_and_rotate_matches_split_then_rotate(rotary_ndims):
+    """split_qkv_and_rotate against torch.split followed by apply_rotary_to_query_key: same results, and the same
+    gradient for the projection output although it is assembled without a concatenation. The key gradient is fed
+    in the layout the score GEMM's backward produces (contiguous along the sequence)."""
+    from megatron.model.attention_core import apply_rotary_to_query_key, split_qkv_and_rotate
+    from megatron.model.positional_embeddings import RotaryEmbedding
+
+    dtype, sq, b, np_, hn = torch.bfloat16, 128, 2, 4, 128
+    emb = RotaryEmbedding(rotary_ndims or hn, 256, base=10000, precision=dtype)
+    base = util.randn((sq, b, np_, 3 * hn), dtype, seed=4).to(DEV)
+    ma = base.clone().requires_grad_(True)
+    mb = base.clone().requires_grad_(True)
+    qa, ka, va = split_qkv_and_rotate(ma, emb)
+    q0, k0, vb = torch.split(mb, hn, dim=-1)
+    qb, kb = apply_rotary_to_query_key(q0, k0, emb, rotary_ndims=rotary_ndims, rope_fusion=True, one_launch=True)
+    for a, e in ((qa, qb), (ka, kb), (va, vb)):
+        assert a.shape == e.shape and torch.equal(util.raw_bits(a), util.raw_bits(e))
+    gq = util.randn((sq, b, np_, hn), dtype, seed=5).to(DEV)
+    gk = util.randn((b, np_, hn, sq), dtype, seed=6).to(DEV).permute(3, 0, 1, 2)   # [sq, b, np, hn], sequence-major
+    gv = util.randn((sq, b, np_, hn), dtype, seed=7).to(DEV)
+    torch.autograd.backward((qa, ka, va), (gq, gk, gv))
+    torch.autograd.backward((qb, kb, vb), (gq, gk, gv))
+    assert torch.equal(util.raw_bits(ma.grad), util.raw_bits(mb.grad))
+    # only part of the outputs used
+    mc = base.clone().requires_grad_(True)
+    qc, kc, vc = split_qkv_and_rotate(mc, emb)
+    qc.backward(gq)
+    assert torch.equal(util.raw_bits(mc.grad[..., :hn]), util.raw_bits(ma.grad[..., :hn]))
+    assert mc.grad[..., hn:].abs().max().item() == 0
+    # with cached keys the rotation starts at the position after them
+    past = torch.zeros((2, 40, b, np_, hn), dtype=dtype, device=DEV)
+    qd, kd, _ = split_qkv_and_rotate(base, emb, layer_past=past)
+    qe, ke = apply_rotary_to_query_key(base[..., :hn], base[..., hn:2 * hn], emb, rotary_ndims=rotary_ndims,
+                                       rope_fusion=False, bf16=True, layer_past=past)
+    assert torch.equal(util.raw_bits(qd), util.raw_bits(qe)) and torch.equal(util.raw_bits(kd), util.raw_bits(ke))
