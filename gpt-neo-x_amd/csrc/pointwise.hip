@@ -60,7 +60,8 @@ __device__ __forceinline__ float gelu_grad(float x)
 enum PointOp {
     kGeluFwd = 0,        // out = gelu(a + bias)
     kGeluBwd = 1,        // out = gelu'(b + bias) * a
-    kBiasAddResidual = 2 // out = b + (a + bias), b optional
+    kBiasAddResidual = 2, // out = b + (a + bias), b optional
+    kColumnSum = 3        // nothing stored: only the column sums of a (with COLSUM)
 };
 
 // One element. `a`, `b`: the two tensor operands (b unused by kGeluFwd), `bv`: bias.
@@ -78,7 +79,7 @@ __device__ __forceinline__ float point_op(float a, float b, float bv, bool has_b
 }
 
 template <int OP>
-constexpr bool kNeedsB = (OP != kGeluFwd);
+constexpr bool kNeedsB = (OP != kGeluFwd && OP != kColumnSum);
 
 // ---------------------------------------------------------------------------
 // Tiled kernel. Thread (tr, tc) of a workgroup owns chunk column
@@ -144,6 +145,11 @@ pointwise_kernel(void* out, const void* a, const void* b, const void* bias, floa
                 if (row < rows) {
                     float fa[V], fb[V], fo[V];
                     chunk_to_float<DT>(ra[u], fa);
+                    if constexpr (OP == kColumnSum) {
+#pragma unroll
+                        for (int j = 0; j < V; ++j) sums[j] += fa[j];
+                        continue;
+                    }
                     chunk_to_float<DT>(rb[u], fb);
 #pragma unroll
                     for (int j = 0; j < V; ++j) fo[j] = point_op<OP>(fa[j], fb[j], bv[j], has_b);
@@ -313,7 +319,7 @@ static int run_pointwise(void* out, const void* a, const void* b, const void* bi
         const int64_t cpr = cols / V;
         if (dbias == nullptr)
             return launch_tiled<DT, OP, false>(out, a, b, bias, nullptr, rows, cpr, plan_tiles(rows, cpr, false), st);
-        if constexpr (OP == kGeluBwd) {
+        if constexpr (OP == kGeluBwd || OP == kColumnSum) {
             const TilePlan p = plan_tiles(rows, cpr, true);
             int rc = launch_tiled<DT, OP, true>(out, a, b, bias, workspace, rows, cpr, p, st);
             if (rc != NHP_OK) return rc;
@@ -324,6 +330,12 @@ static int run_pointwise(void* out, const void* a, const void* b, const void* bi
             return launch_result();
         }
         return NHP_ERR_SHAPE;
+    }
+    if constexpr (OP == kColumnSum) {
+        if (!grid_fits((cols + kPwThreads - 1) / kPwThreads, kPwThreads)) return NHP_ERR_SHAPE;
+        column_sum_scalar_kernel<DT><<<(uint32_t)((cols + kPwThreads - 1) / kPwThreads), kPwThreads, 0, st>>>(
+            dbias, a, (uint64_t)rows, (uint64_t)cols);
+        return launch_result();
     }
     const int64_t total = rows * cols;
     const int64_t blocks = (total + kPwThreads - 1) / kPwThreads;
@@ -397,6 +409,22 @@ int nhp_bias_gelu_bwd(void* dx, const void* g, const void* y, const void* bias, 
     if (dbias != nullptr && (dbias == dx || dbias == workspace)) return NHP_ERR_ALIAS;
     return dispatch_pointwise<kGeluBwd>(dx, g, y, bias, dbias, static_cast<float*>(workspace), rows, cols, dtype,
                                         static_cast<hipStream_t>(stream));
+}
+
+int64_t nhp_column_sum_workspace_bytes(int64_t rows, int64_t cols, int dtype)
+{
+    return nhp_bias_gelu_bwd_workspace_bytes(rows, cols, dtype);
+}
+
+int nhp_column_sum(void* out, const void* x, void* workspace, int64_t rows, int64_t cols, int dtype, void* stream)
+{
+    if (int rc = check_shape(rows, cols, dtype)) return rc;
+    if (rows == 0 || cols == 0) return NHP_OK;  // the sums of an empty tensor are left untouched
+    if (!out || !x) return NHP_ERR_NULL;
+    if (workspace == nullptr && nhp_column_sum_workspace_bytes(rows, cols, dtype) > 0) return NHP_ERR_NULL;
+    if (out == x || out == workspace) return NHP_ERR_ALIAS;
+    return dispatch_pointwise<kColumnSum>(nullptr, x, nullptr, nullptr, out, static_cast<float*>(workspace), rows,
+                                          cols, dtype, static_cast<hipStream_t>(stream));
 }
 
 int nhp_bias_add_residual(void* out, const void* x, const void* bias, const void* residual, int64_t rows,

@@ -54,7 +54,25 @@ def _bias_grad(per_element, bias_shape, expanded):
     sums them when it undoes the expansion); for a vector the rows are summed here."""
     if expanded:
         return per_element
-    return per_element.reshape(-1, per_element.size(-1)).sum(dim=0).view(bias_shape)
+    return _column_sum(per_element).view(bias_shape)
+
+
+def _column_sum(t):
+    """Sum over all but the last dimension, fp32 accumulation in a fixed order, one rounding."""
+    what = "bias_dropout_add backward"
+    cols = t.size(-1)
+    src = t.contiguous()
+    rows = src.numel() // max(cols, 1)
+    out = torch.zeros(cols, dtype=src.dtype, device=src.device) if rows == 0 else \
+        torch.empty(cols, dtype=src.dtype, device=src.device)
+    code = _hp.dtype_code(src, what)
+    nbytes = _hp.lib().nhp_column_sum_workspace_bytes(rows, cols, code)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=src.device) if nbytes else None
+    with _hp.device_guard(src):
+        rc = _hp.lib().nhp_column_sum(out.data_ptr(), src.data_ptr(), None if ws is None else ws.data_ptr(), rows, cols,
+                                      code, _hp.stream_of(src))
+    _hp.check(rc, what)
+    return out
 
 
 class _BiasAddResidual(torch.autograd.Function):

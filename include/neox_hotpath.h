@@ -336,6 +336,20 @@ int nhp_bias_gelu_bwd(void* dx, const void* g, const void* y, const void* bias,
 int64_t nhp_bias_gelu_bwd_workspace_bytes(int64_t rows, int64_t cols, int dtype);
 
 /*
+ * out[c] = sum over rows of x[r, c], accumulated in fp32 in a fixed order
+ * (reproducible from run to run) and rounded once: the reduction autograd
+ * performs for a bias that was expanded over the rows, i.e. the bias gradient
+ * of bias_dropout_add at the reference's call sites
+ * (megatron/model/transformer.py:1229, 1271: bias.expand_as(residual);
+ * megatron/model/fused_bias_dropout.py:28-35). `workspace`: fp32 partial rows,
+ * nhp_column_sum_workspace_bytes() bytes (a few MiB, bounded whatever the
+ * row count; 0 for shapes that take the scalar path).
+ */
+int nhp_column_sum(void* out, const void* x, void* workspace, int64_t rows, int64_t cols,
+                   int dtype, void* stream);
+int64_t nhp_column_sum_workspace_bytes(int64_t rows, int64_t cols, int dtype);
+
+/*
  * out = residual + (x + bias): bias_dropout_add with dropout switched off
  * (training False or prob 0, when torch's dropout is the identity).
  * bias and residual may each be NULL.

@@ -138,6 +138,13 @@ def test_argument_validation_of_the_layer_entry_points(hotpath):
     assert lib.nhp_bias_gelu_bwd_workspace_bytes(0, 8, BF16) == 0
     big = lib.nhp_bias_gelu_bwd_workspace_bytes(1 << 20, 8192, BF16)
     assert 0 < big <= 512 * 8192 * 4                                               # bounded, whatever the row count
+    assert lib.nhp_column_sum(null, p, p, 4, 8, BF16, None) == -3
+    assert lib.nhp_column_sum(q, p, null, 4, 8, BF16, None) == -3                  # workspace missing
+    assert lib.nhp_column_sum(p, p, q, 4, 8, BF16, None) == -6                     # sums over their own input
+    assert lib.nhp_column_sum(q, p, p, 4, 8, 7, None) == -1
+    assert lib.nhp_column_sum(null, null, null, 0, 8, BF16, None) == 0
+    assert lib.nhp_column_sum_workspace_bytes(4, 8, BF16) == lib.nhp_bias_gelu_bwd_workspace_bytes(4, 8, BF16) > 0
+    assert lib.nhp_column_sum_workspace_bytes(4, 7, BF16) == 0
     assert lib.nhp_bias_add_residual(q, null, p, p, 4, 8, F16, None) == -3
     assert lib.nhp_bias_add_residual(q, p, null, null, 4, 8, 3, None) == -1
     # norms: parameter dtype is the data dtype or fp32

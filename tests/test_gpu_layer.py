@@ -429,3 +429,24 @@ def test_bias_dropout_add_takes_the_expanded_bias_of_the_reference_call_sites(pr
     assert torch.allclose(ga.float(), vb.grad.float(), rtol=2.0 ** -6, atol=2.0 ** -6)
     with pytest.raises(RuntimeError, match="one value per feature"):
         bias_dropout_add_fused_train(x, torch.zeros_like(res), res, prob)   # a genuinely full-size "bias"
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32], ids=["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("shape", [(1, 8), (37, 64), (1000, 512), (4097, 2048), (16, 8192), (33, 1000), (5, 20)],
+                         ids=lambda s: f"{s[0]}x{s[1]}")
+def test_column_sum_vs_oracle(hotpath, shape, dtype):
+    """nhp_column_sum: fp32 accumulation, one rounding; against the oracle's pairwise sum, within the fp32
+    noise of a sum of `rows` terms formed in another order. Reproducible from run to run."""
+    rows, cols = shape
+    print(f"column sum {shape} {dtype}", flush=True)
+    x = util.randn((rows, cols), dtype, seed=rows + cols, std=2.0)
+    xd = x.to(DEV)
+    L, code = hotpath.lib(), hotpath.dtype_code(xd, "t")
+    ws = torch.empty(max(L.nhp_column_sum_workspace_bytes(rows, cols, code), 16), dtype=torch.uint8, device=DEV)
+    out = torch.full((cols,), float("nan"), dtype=dtype, device=DEV)
+    assert L.nhp_column_sum(out.data_ptr(), xd.data_ptr(), ws.data_ptr(), rows, cols, code, None) == 0
+    want = oracle.column_sum(x)
+    util.assert_close_ulp_or_noise(out.cpu(), want, 1, x.float().abs().sum(0) * 16 * util.EPS32, "column sums")
+    again = torch.empty_like(out)
+    assert L.nhp_column_sum(again.data_ptr(), xd.data_ptr(), ws.data_ptr(), rows, cols, code, None) == 0
+    assert torch.equal(util.raw_bits(out), util.raw_bits(again))
