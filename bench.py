@@ -18,6 +18,8 @@ the drop-in extension modules (which call libneox_hotpath.so):
                  the attention layer slices q and k from), rotary_pct 1.0; one launch per tensor, then q and k
                  in one launch
   rope-qk-1.4b   rotary fwd+bwd on q,k [2048,8,16,128] bf16, rotary_pct 0.25, q and k in one launch
+  rope-kgrad-1.4b  rotary bwd on a gradient [2048,8,16,128] bf16 that is contiguous along the sequence (strides
+                 (1, h*d*s, d*s, s)): the layout of the key gradient behind the score GEMM's backward
   mistral-window causal softmax fwd+bwd [64,8192,8192] bf16 with a 4096-key sliding window applied by index
   alibi-1.4b     causal softmax fwd+bwd [128,2048,2048] bf16 with the AliBi bias of 16 heads added in the kernel
   attn-dropout-1.4b  causal softmax + attention dropout (p = 0.1) in one kernel, fwd+bwd [128,2048,2048] bf16
@@ -467,6 +469,24 @@ def make_workload(name, torch, dev):
 
         cfg = {"workload": name, "qk": [s, b, h, d], "qk_strides": list(sets[0][0].stride()), "rotary_dim": d2}
         return step, kernel_bytes, {}, "rope_fwd_view", "bf16", cfg
+
+    if name == "rope-kgrad-1.4b":
+        s, b, h, d, d2 = 2048, 8, 16, 128, 32
+        sets = []
+        for i in range(4):  # rotate buffers: 64 MiB tensors fit the cache
+            g = randn((b, h, d, s), 120 + i, torch.bfloat16).permute(3, 0, 1, 2)   # [s, b, h, d], contiguous along s
+            cos, sin = RotaryEmbedding(d2, s, base=10000, precision=torch.bfloat16)(g, seq_len=s)
+            sets.append((g, cos.contiguous(), sin.contiguous()))
+        kernel_bytes = {"rope_bwd_seq_major": rope_bytes(s, b, h, d, d2)}
+        state = {"i": 0}
+
+        def step(t):
+            g, cos, sin = sets[state["i"] % len(sets)]
+            state["i"] += 1
+            t.run("rope_bwd_seq_major", lambda: rope_ext.backward_cached(g, cos, sin, False))
+
+        cfg = {"workload": name, "grad": [s, b, h, d], "grad_strides": list(sets[0][0].stride()), "rotary_dim": d2}
+        return step, kernel_bytes, {}, "rope_bwd_seq_major", "bf16", cfg
 
     if name == "rope-c4":
         s, b, h, d = 4096, 4, 32, 128
