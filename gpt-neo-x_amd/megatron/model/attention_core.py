@@ -36,6 +36,29 @@ def get_fusion_type(neox_args):
     return SoftmaxFusionTypes.none
 
 
+class _ContextGemm(torch.autograd.Function):
+    """``probs [B, sq, sk] x v [sk, B, hn] -> [sq, B, hn]``: the context GEMM writing the layout the output
+    projection wants, which saves the ``permute(2, 0, 1, 3).contiguous()`` copy of
+    megatron/model/transformer.py:941 and its counterpart in the backward (the library GEMM takes the
+    strides; nothing is computed differently)."""
+
+    @staticmethod
+    def forward(ctx, probs, value):
+        sk, batches, hn = value.shape
+        out = torch.empty((probs.size(1), batches, hn), dtype=probs.dtype, device=probs.device)
+        torch.bmm(probs, value.transpose(0, 1), out=out.transpose(0, 1))
+        ctx.save_for_backward(probs, value)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad):
+        probs, value = ctx.saved_tensors
+        g = grad.transpose(0, 1)  # [B, sq, hn], a view
+        grad_probs = torch.bmm(g, value.transpose(0, 1).transpose(1, 2)) if ctx.needs_input_grad[0] else None
+        grad_value = torch.bmm(probs.transpose(1, 2), g).transpose(0, 1) if ctx.needs_input_grad[1] else None
+        return grad_probs, grad_value
+
+
 class CoreAttention(torch.nn.Module):
     """Unfused ("global") attention on top of the fused softmax.
 
@@ -74,7 +97,10 @@ class CoreAttention(torch.nn.Module):
             softmax_in_fp32=attention_softmax_in_fp32, scale=coeff, sliding_window_width=sliding_window_width,
             alibi_slopes=alibi_slopes, attention_dropout=attention_dropout)
 
-    def forward(self, query_layer, key_layer, value_layer, attention_mask, key_lengths=None):
+    def forward(self, query_layer, key_layer, value_layer, attention_mask, key_lengths=None, merged_heads=False):
+        """Returns the context as ``[b, np, sq, hn]`` (what ``ParallelSelfAttention.attention`` returns), or with
+        ``merged_heads`` as ``[sq, b, np * hn]``, the layout its caller brings it into before the output
+        projection, written by the context GEMM itself."""
         b, np_, sq, sk = query_layer.size(1), query_layer.size(2), query_layer.size(0), key_layer.size(0)
         hn = query_layer.size(3)
         # [sq, b, np, hn] -> [sq, b * np, hn]
@@ -90,6 +116,8 @@ class CoreAttention(torch.nn.Module):
         probs = self.scale_mask_softmax(scores, attention_mask, bias=bias, key_lengths=key_lengths)
         # [sk, b, np, hn] -> [sk, b * np, hn]; context [b * np, sq, hn]
         v = value_layer.reshape(sk, b * np_, value_layer.size(3))
+        if merged_heads:
+            return _ContextGemm.apply(probs.view(b * np_, sq, sk), v).view(sq, b, np_ * value_layer.size(3))
         context = torch.bmm(probs.view(b * np_, sq, sk), v.transpose(0, 1))
         return context.view(b, np_, sq, value_layer.size(3))
 

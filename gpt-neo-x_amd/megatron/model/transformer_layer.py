@@ -130,9 +130,8 @@ class SelfAttention(torch.nn.Module):
             if self.rotary_emb is not None:
                 query, key = apply_rotary_to_query_key(query, key, self.rotary_emb, rotary_ndims=self.rotary_ndims,
                                                        rope_fusion=False, bf16=self.bf16)
-        context = self.core(query, key, value, attention_mask)
-        # [b, np, sq, hn] -> [sq, b, np * hn]
-        context = context.permute(2, 0, 1, 3).contiguous().view(sq, b, self.num_heads * self.head_dim)
+        # [sq, b, np * hn], written in that layout by the context GEMM
+        context = self.core(query, key, value, attention_mask, merged_heads=True)
         return self.dense(context)
 
 

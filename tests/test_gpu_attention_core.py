@@ -222,3 +222,25 @@ def test_split_and_rotate_matches_split_then_rotate(rotary_ndims):
     qe, ke = apply_rotary_to_query_key(base[..., :hn], base[..., hn:2 * hn], emb, rotary_ndims=rotary_ndims,
                                        rope_fusion=False, bf16=True, layer_past=past)
     assert torch.equal(util.raw_bits(qd), util.raw_bits(qe)) and torch.equal(util.raw_bits(kd), util.raw_bits(ke))
+
+
+def test_merged_heads_output_equals_the_permuted_context():
+    """CoreAttention(..., merged_heads=True) returns permute(2, 0, 1, 3) of the default result, reshaped to
+    [sq, b, np * hn] (megatron/model/transformer.py:941-947), bit for bit, with the same gradients."""
+    from megatron.model.attention_core import CoreAttention
+    from megatron.model.fused_softmax import SoftmaxFusionTypes as T
+
+    dtype, sq, b, np_, hn = torch.bfloat16, 256, 2, 4, 64
+    core = CoreAttention(hn, 1, False, True, T.upper_triang, mask_func, attention_softmax_in_fp32=True)
+    mask = fb.causal_mask(sq, DEV)
+    qa, ka, va = qkv(dtype, sq, b, np_, hn, 31)
+    qb, kb, vb = (t.detach().clone().requires_grad_(True) for t in (qa, ka, va))
+    merged = core(qa, ka, va, mask, merged_heads=True)
+    plain = core(qb, kb, vb, mask).permute(2, 0, 1, 3).contiguous().view(sq, b, np_ * hn)
+    assert merged.shape == (sq, b, np_ * hn) and merged.is_contiguous()
+    assert torch.equal(util.raw_bits(merged), util.raw_bits(plain))
+    g = util.randn((sq, b, np_ * hn), dtype, seed=5).to(DEV)
+    merged.backward(g)
+    plain.backward(g)
+    for a, e in ((qa, qb), (ka, kb), (va, vb)):
+        assert torch.equal(util.raw_bits(a.grad), util.raw_bits(e.grad))
