@@ -74,11 +74,15 @@ class CoreAttention(torch.nn.Module):
         attention_dropout, sliding_window_width, alibi_slopes: handed to the softmax module.
         rpe: optional module ``rpe(sq, sk) -> [1, np, sq, sk]`` (relative position bias).
         use_cache: crop the mask to the current key length (inference with a KV cache).
+        fold_scale: apply ``1 / norm_factor`` inside the softmax kernel (as part of its fp32 scale) instead of
+            as the ``alpha`` of the score GEMM, whose backward pays for ``alpha`` with an extra pass over the
+            gradients of q and k. None (default): fold unless the scores are fp16 (there the scaled GEMM is
+            what keeps them in range, the reason the reference scales twice) or the softmax is not in fp32.
     """
 
     def __init__(self, head_dim, layer_number, fp16, bf16, fusion_type, mask_func, attention_softmax_in_fp32=False,
                  apply_query_key_layer_scaling=False, use_mup=False, attention_dropout=0.0,
-                 sliding_window_width=None, alibi_slopes=None, rpe=None, use_cache=False):
+                 sliding_window_width=None, alibi_slopes=None, rpe=None, use_cache=False, fold_scale=None):
         super().__init__()
         self.layer_number = max(1, int(layer_number))
         if apply_query_key_layer_scaling:
@@ -92,9 +96,17 @@ class CoreAttention(torch.nn.Module):
             self.norm_factor = head_dim
         self.rpe = rpe
         self.use_cache = use_cache
+        if fold_scale is None:
+            fold_scale = not fp16 and attention_softmax_in_fp32
+        assert not fold_scale or attention_softmax_in_fp32, "a folded scale needs the softmax in fp32"
+        # additive terms (rpe bias, AliBi) are added to the scores before the softmax scales them, so the
+        # factor can only move behind the GEMM when there are none
+        self.fold_scale = bool(fold_scale) and rpe is None and alibi_slopes is None
+        self.gemm_alpha = 1.0 if self.fold_scale else 1.0 / self.norm_factor
+        softmax_scale = (coeff or 1.0) / self.norm_factor if self.fold_scale else coeff
         self.scale_mask_softmax = FusedScaleMaskSoftmax(
             input_in_fp16=fp16, input_in_bf16=bf16, fusion_type=fusion_type, mask_func=mask_func,
-            softmax_in_fp32=attention_softmax_in_fp32, scale=coeff, sliding_window_width=sliding_window_width,
+            softmax_in_fp32=attention_softmax_in_fp32, scale=softmax_scale, sliding_window_width=sliding_window_width,
             alibi_slopes=alibi_slopes, attention_dropout=attention_dropout)
 
     def forward(self, query_layer, key_layer, value_layer, attention_mask, key_lengths=None, merged_heads=False):
@@ -106,9 +118,12 @@ class CoreAttention(torch.nn.Module):
         # [sq, b, np, hn] -> [sq, b * np, hn]
         q = query_layer.reshape(sq, b * np_, hn)
         k = key_layer.reshape(sk, b * np_, hn)
-        scores = torch.empty((b * np_, sq, sk), dtype=q.dtype, device=q.device)
-        scores = torch.baddbmm(scores, q.transpose(0, 1), k.transpose(0, 1).transpose(1, 2), beta=0.0,
-                               alpha=1.0 / self.norm_factor).view(b, np_, sq, sk)
+        if self.fold_scale:
+            scores = torch.bmm(q.transpose(0, 1), k.transpose(0, 1).transpose(1, 2)).view(b, np_, sq, sk)
+        else:
+            scores = torch.empty((b * np_, sq, sk), dtype=q.dtype, device=q.device)
+            scores = torch.baddbmm(scores, q.transpose(0, 1), k.transpose(0, 1).transpose(1, 2), beta=0.0,
+                                   alpha=self.gemm_alpha).view(b, np_, sq, sk)
         if self.use_cache and attention_mask is not None:
             with torch.no_grad():
                 attention_mask = attention_mask[..., :sk, :sk]

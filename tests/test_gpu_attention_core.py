@@ -50,7 +50,12 @@ def test_causal_attention_matches_textbook(dtype, layer_scaling):
     core = CoreAttention(hn, 7, dtype == torch.float16, dtype == torch.bfloat16, T.upper_triang, mask_func,
                          attention_softmax_in_fp32=True, apply_query_key_layer_scaling=layer_scaling)
     assert core.norm_factor == math.sqrt(hn) * (7 if layer_scaling else 1)
-    assert core.scale_mask_softmax.scale == (7 if layer_scaling else None)
+    if dtype == torch.float16:   # the reference's split: 1 / norm_factor in the GEMM, coeff in the softmax
+        assert not core.fold_scale and core.gemm_alpha == 1 / core.norm_factor
+        assert core.scale_mask_softmax.scale == (7 if layer_scaling else None)
+    else:                        # both factors in the softmax kernel's fp32 scale
+        assert core.fold_scale and core.gemm_alpha == 1.0
+        assert core.scale_mask_softmax.scale == pytest.approx(1 / math.sqrt(hn))
     q, k, v = qkv(dtype, sq, b, np_, hn, 1)
     mask = fb.causal_mask(sq, DEV)
     assert core.scale_mask_softmax.is_kernel_available(mask, b, np_, sq, sq)
@@ -64,6 +69,12 @@ def test_causal_attention_matches_textbook(dtype, layer_scaling):
     assert rel_err(out, ref) <= lim
     for got, want in ((q.grad, qr.grad), (k.grad, kr.grad), (v.grad, vr.grad)):
         assert rel_err(got, want) <= 2 * lim
+    # folding the GEMM's factor into the softmax scale changes nothing beyond bf16 rounding of the scores
+    if dtype == torch.bfloat16:
+        split = CoreAttention(hn, 7, False, True, T.upper_triang, mask_func, attention_softmax_in_fp32=True,
+                              apply_query_key_layer_scaling=layer_scaling, fold_scale=False)
+        assert not split.fold_scale and split.scale_mask_softmax.scale == (7 if layer_scaling else None)
+        assert rel_err(split(q.detach(), k.detach(), v.detach(), mask), ref) <= lim
     # the fused and the torch branch of the softmax module agree inside the caller
     plain = CoreAttention(hn, 7, dtype == torch.float16, dtype == torch.bfloat16, T.none, mask_func,
                           attention_softmax_in_fp32=True, apply_query_key_layer_scaling=layer_scaling)

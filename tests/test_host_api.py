@@ -331,8 +331,15 @@ def test_core_attention_scaling_and_torch_branch_on_cpu():
     def mask_func(scores, mask):
         return fb.fill_masked_with_dtype_min(scores, mask)
 
-    core = CoreAttention(64, 5, False, False, T.none, mask_func, apply_query_key_layer_scaling=True)
+    core = CoreAttention(64, 5, False, False, T.none, mask_func, apply_query_key_layer_scaling=True, fold_scale=False)
     assert core.norm_factor == 8 * 5 and core.scale_mask_softmax.scale == 5 and core.scale_mask_softmax.softmax_in_fp32
+    assert core.gemm_alpha == 1 / 40
+    folded = CoreAttention(64, 5, False, False, T.none, mask_func, apply_query_key_layer_scaling=True)
+    assert folded.fold_scale and folded.gemm_alpha == 1.0 and folded.scale_mask_softmax.scale == 5 / 40
+    half = CoreAttention(64, 5, True, False, T.none, mask_func, apply_query_key_layer_scaling=True)
+    assert not half.fold_scale and half.scale_mask_softmax.scale == 5          # fp16 scores keep the scaled GEMM
+    biased = CoreAttention(64, 5, False, True, T.none, mask_func, attention_softmax_in_fp32=True, rpe=lambda a, c: None)
+    assert not biased.fold_scale                                               # additive terms come before the scale
     assert CoreAttention(64, 0, False, False, T.none, mask_func, apply_query_key_layer_scaling=True).norm_factor == 8
     assert CoreAttention(64, 5, False, False, T.none, mask_func, use_mup=True).norm_factor == 64
     sq, b, np_, hn = 24, 2, 3, 16
