@@ -103,6 +103,11 @@ class Timer:
     def averages_ms(self):
         return {k: sum(a.elapsed_time(b) for a, b in v) / len(v) for k, v in self.pairs.items()}
 
+    def spread_ms(self, name):
+        """(min, median, max) of the bracketed launches of `name`."""
+        t = sorted(a.elapsed_time(b) for a, b in self.pairs[name])
+        return t[0], t[len(t) // 2], t[-1]
+
     def reset(self):
         self.pairs = {}
 
@@ -617,6 +622,7 @@ def main():
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     dominant_ms = timer.averages_ms()[dominant]
+    dominant_spread = timer.spread_ms(dominant)
 
     # Untimed extra pass for the per-kernel breakdown.
     full = Timer(torch)
@@ -658,7 +664,9 @@ def main():
         "kernels": kernels,
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": dom["GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": dom["frac_of_peak"], "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-                     "algorithmic_bytes": kernel_bytes[dominant], "avg_launch_ms": dom["ms"]},
+                     "algorithmic_bytes": kernel_bytes[dominant], "avg_launch_ms": dom["ms"],
+                     "min_launch_ms": round(dominant_spread[0], 4), "median_launch_ms": round(dominant_spread[1], 4),
+                     "max_launch_ms": round(dominant_spread[2], 4)},
     }
     if args.workload == "pythia-1.4b" and not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch)
