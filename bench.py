@@ -23,6 +23,7 @@ the drop-in extension modules (which call libneox_hotpath.so):
   mistral-window causal softmax fwd+bwd [64,8192,8192] bf16 with a 4096-key sliding window applied by index
   alibi-1.4b     causal softmax fwd+bwd [128,2048,2048] bf16 with the AliBi bias of 16 heads added in the kernel
   attn-dropout-1.4b  causal softmax + attention dropout (p = 0.1) in one kernel, fwd+bwd [128,2048,2048] bf16
+  masked-dropout-c3  padding-masked softmax + attention dropout (p = 0.1) in one kernel, fwd+bwd on the masked-c3 tensors
   rpe-bias-1.4b  causal softmax fwd+bwd [128,2048,2048] bf16 with a bias tensor [16,2048,2048] added in the kernel
 
   mlp-gelu-1.4b  bias + tanh-GeLU fwd and bwd (with the bias gradient) on the MLP activation [2048*8, 8192] bf16
@@ -227,7 +228,7 @@ def make_workload(name, torch, dev):
                "bytes_convention": "reads of the attended band, dense writes"}
         return step, kernel_bytes, {}, "causal_softmax_bwd", "bf16", cfg
 
-    if name == "masked-c3":
+    if name in ("masked-c3", "masked-dropout-c3"):
         b, np_, sq, sk = 16, 32, 1024, 2048
         scale = 1.0 / math.sqrt(128)
         x = randn((b, np_, sq, sk), 0, torch.float16, 3.0)
@@ -253,6 +254,20 @@ def make_workload(name, torch, dev):
             y = t.run("masked_softmax_fwd", lambda: masked_ext.forward(x, mask, scale))
             t.run("masked_softmax_bwd", lambda: masked_ext.backward(dy, y, scale))
 
+        if name == "masked-dropout-c3":
+            kernel_bytes = {"masked_softmax_dropout_fwd": 3 * n * 2 + mask.numel(), "masked_softmax_dropout_bwd": 3 * n * 2}
+            state = {"i": 0}
+
+            def step_dropout(t):
+                state["i"] += 1
+                seed = 1000 + state["i"]
+                _, y = t.run("masked_softmax_dropout_fwd", lambda: masked_ext.forward_dropout(x, mask, scale, 0.1, seed))
+                t.run("masked_softmax_dropout_bwd", lambda: masked_ext.backward_dropout(dy, y, scale, 0.1, seed))
+
+            cfg = {"workload": name, "scores": [b, np_, sq, sk], "mask": [b, 1, sq, sk], "dropout": 0.1,
+                   "bytes_convention": "dense (tensor read + mask once + probabilities and dropped probabilities written; "
+                                       "3x tensor backward)"}
+            return step_dropout, kernel_bytes, {}, "masked_softmax_dropout_bwd", "f16", cfg
         cfg = {"workload": name, "scores": [b, np_, sq, sk], "mask": [b, 1, sq, sk],
                "bytes_convention": "dense (2x tensor forward + mask once, 3x tensor backward)"}
         return step, kernel_bytes, needed, "masked_softmax_bwd", "f16", cfg

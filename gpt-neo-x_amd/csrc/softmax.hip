@@ -29,7 +29,7 @@
 // read beside the scores; in the padding-mask kernel a chunk whose 8 mask
 // bytes are all 1 is not loaded.
 //
-// Attention dropout (causal kernels): the forward also writes dropout(y), the
+// Attention dropout: the forward also writes dropout(y), the
 // backward first applies the dropout backward to dy; the keep mask is
 // regenerated from a counter-based generator, never stored.
 
@@ -322,12 +322,13 @@ causal_fwd_kernel(uint16_t* y, const uint16_t* x, float scale, uint32_t total_ro
 // over `heads_per_wave` heads with them, so the mask bytes of a row are
 // fetched and decoded once per head group.
 // ---------------------------------------------------------------------------
-template <int DT, int L, int K, int W, int BW>
+// DROP: also write dropped = dropout(y), as the causal kernel does.
+template <int DT, int L, int K, int W, int BW, bool DROP>
 __global__ void __launch_bounds__((Geo<L, K, W, BW>::kThreads))
 masked_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float scale,
                   uint32_t bq_rows, uint32_t sq, uint32_t np, uint32_t n,
                   uint32_t heads_per_wave, uint32_t head_groups, int mask_per_batch, uint32_t row_blocks,
-                  uint32_t tile)
+                  uint32_t tile, uint16_t* dropped, DropoutKey dk)
 {
     using G = Geo<L, K, W, BW>;
     __shared__ float lds[2][32];
@@ -445,9 +446,27 @@ masked_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
                 float o[8];
 #pragma unroll
                 for (int j = 0; j < 8; ++j) o[j] = z[k][j] * inv;
-                store16_stream(yr + col, pack8<DT>(o));
+                const u32x4 py = pack8<DT>(o);
+                store16_stream(yr + col, py);
+                if constexpr (DROP) {
+                    // dropout of the stored (rounded) probabilities
+                    float f[8];
+                    unpack8<DT>(py, f);
+                    const Philox rnd = dropout_bits(dk, (uint64_t)base + col);
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) f[j] = random16(rnd, j) < dk.threshold ? f[j] * dk.scale : 0.0f;
+                    store16_stream(dropped + base + col, pack8<DT>(f));
+                }
             } else if (dead[k]) {
                 store16_stream(yr + col, u32x4{pd, pd, pd, pd});
+                if constexpr (DROP) {
+                    const float v = Half2<DT>::lo(pd);
+                    float f[8];
+                    const Philox rnd = dropout_bits(dk, (uint64_t)base + col);
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) f[j] = random16(rnd, j) < dk.threshold ? v * dk.scale : 0.0f;
+                    store16_stream(dropped + base + col, pack8<DT>(f));
+                }
             }
         }
     }
@@ -459,7 +478,7 @@ masked_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
 // ---------------------------------------------------------------------------
 // EXTRA: kPlain, kPerHead (key lengths; causal only) or kDropout (dy is the gradient of
 // dropout(y): the kernel first forms keep * dy / (1 - p), rounded to the storage type as the
-// separate dropout backward would store it; causal only).
+// separate dropout backward would store it).
 template <int DT, int L, int K, int W, int BW, bool CAUSAL, int EXTRA>
 __global__ void __launch_bounds__((Geo<L, K, W, BW>::kThreads))
 softmax_bwd_kernel(uint16_t* dx, const uint16_t* dy, const uint16_t* y, float scale,
@@ -637,7 +656,7 @@ scalar_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
         float p = 0.0f;
         if (c >= lo && c < hi) p = exp2_raw(fmaf(logit(c) - m, kLog2e, kExpBias)) * inv;
         yr[c] = Half2<DT>::to_bits(p);
-        if (MODE == 0 && dropped != nullptr) {
+        if (dropped != nullptr) {
             const uint64_t e = row * n + c;
             const Philox rnd = dropout_bits(dk, e & ~(uint64_t)7);
             const float kept = random16(rnd, (int)(e & 7u)) < dk.threshold ? Half2<DT>::round(p) * dk.scale : 0.0f;
@@ -846,7 +865,7 @@ static int softmax_bwd(void* dx, const void* dy, const void* y, float scale, int
 {
     RowPlan p;
     const DropoutKey dk = drop != nullptr ? *drop : DropoutKey{};
-    const bool dropout = CAUSAL && drop != nullptr;
+    const bool dropout = drop != nullptr;
     uint16_t* dxp = static_cast<uint16_t*>(dx);
     const uint16_t* dyp = static_cast<const uint16_t*>(dy);
     const uint16_t* yp = static_cast<const uint16_t*>(y);
@@ -857,7 +876,7 @@ static int softmax_bwd(void* dx, const void* dy, const void* y, float scale, int
         const uint32_t blocks = (uint32_t)((rows + G::kRowsPerBlock - 1) / G::kRowsPerBlock); \
         if (!launch_fits(blocks, G::kThreads)) return NHP_ERR_SHAPE;                       \
         if (dropout)                                                                       \
-            softmax_bwd_kernel<DT, L_, K_, W_, kBlockWaves, CAUSAL, CAUSAL ? kDropout : kPlain>    \
+            softmax_bwd_kernel<DT, L_, K_, W_, kBlockWaves, CAUSAL, kDropout>                      \
                 <<<blocks, G::kThreads, p.lds, st>>>(dxp, dyp, yp, scale, (uint32_t)rows, (uint32_t)n, \
                                                      (uint32_t)rows_per_matrix, window, nullptr, 1, dk); \
         else if (CAUSAL && kl != nullptr)                                                  \
@@ -885,15 +904,18 @@ static uint32_t pick_heads_per_wave(int64_t np) { return (uint32_t)(np < 2 ? np 
 
 template <int DT>
 static int masked_fwd(void* y, const void* x, const uint8_t* mask, float scale, int64_t b, int64_t np,
-                      int64_t sq, int64_t n, int64_t pad_batches, hipStream_t st)
+                      int64_t sq, int64_t n, int64_t pad_batches, hipStream_t st, void* dropped = nullptr,
+                      const DropoutKey* drop = nullptr)
 {
+    uint16_t* dp = static_cast<uint16_t*>(dropped);
+    const DropoutKey dk = drop != nullptr ? *drop : DropoutKey{};
     const int64_t bq_rows = b * sq;
     const int per_batch = (pad_batches != 1) ? 1 : 0;
     RowPlan p;
     uint16_t* yp = static_cast<uint16_t*>(y);
     const uint16_t* xp = static_cast<const uint16_t*>(x);
     const bool mask_ok = (reinterpret_cast<uintptr_t>(mask) & 7u) == 0;
-    if (plan_row(n, kMaskedFwd, p) && aligned16(x) && aligned16(y) && mask_ok) {
+    if (plan_row(n, kMaskedFwd, p) && aligned16(x) && aligned16(y) && aligned16(dropped) && mask_ok) {
 #define CALL(L_, K_, W_)                                                                   \
     {                                                                                      \
         using G = Geo<L_, K_, W_, kBlockWaves>;                                            \
@@ -904,16 +926,21 @@ static int masked_fwd(void* y, const void* x, const uint8_t* mask, float scale, 
         int64_t tile = tune("NHP_MASK_TILE", (int)((sq + G::kRowsPerBlock - 1) / G::kRowsPerBlock)); \
         if (tile < 1) tile = 1;                                                            \
         if (tile > rb) tile = rb;                                                          \
-        masked_fwd_kernel<DT, L_, K_, W_, kBlockWaves><<<(uint32_t)(rb * hgs), G::kThreads, p.lds, st>>>( \
-            yp, xp, mask, scale, (uint32_t)bq_rows, (uint32_t)sq, (uint32_t)np, (uint32_t)n, hpw, hgs, \
-            per_batch, (uint32_t)rb, (uint32_t)tile);                                      \
+        if (dp != nullptr)                                                                 \
+            masked_fwd_kernel<DT, L_, K_, W_, kBlockWaves, true><<<(uint32_t)(rb * hgs), G::kThreads, p.lds, st>>>( \
+                yp, xp, mask, scale, (uint32_t)bq_rows, (uint32_t)sq, (uint32_t)np, (uint32_t)n, hpw, hgs, \
+                per_batch, (uint32_t)rb, (uint32_t)tile, dp, dk);                          \
+        else                                                                               \
+            masked_fwd_kernel<DT, L_, K_, W_, kBlockWaves, false><<<(uint32_t)(rb * hgs), G::kThreads, p.lds, st>>>( \
+                yp, xp, mask, scale, (uint32_t)bq_rows, (uint32_t)sq, (uint32_t)np, (uint32_t)n, hpw, hgs, \
+                per_batch, (uint32_t)rb, (uint32_t)tile, nullptr, dk);                     \
     }
         NHP_FOR_PLAN(p);
 #undef CALL
     } else {
         if (!launch_fits(b * np * sq, kScalarThreads)) return NHP_ERR_SHAPE;
         scalar_fwd_kernel<DT, 1><<<(uint32_t)(b * np * sq), kScalarThreads, 0, st>>>(
-            yp, xp, mask, scale, (uint64_t)n, (uint64_t)sq, (uint64_t)np, per_batch, kNoWindow, nullptr, nullptr, nullptr, 1, nullptr, DropoutKey{});
+            yp, xp, mask, scale, (uint64_t)n, (uint64_t)sq, (uint64_t)np, per_batch, kNoWindow, nullptr, nullptr, nullptr, 1, dp, dk);
     }
     return launch_status();
 }
@@ -1044,6 +1071,39 @@ int nhp_masked_softmax_bwd(void* dx, const void* dy, const void* y, float scale,
     // rows_per_matrix only matters for the causal variant; any non-zero value works here
     return dtype == NHP_BF16 ? softmax_bwd<NHP_BF16, false>(dx, dy, y, scale, rows, sk, rows, kNoWindow, nullptr, 1, st)
                              : softmax_bwd<NHP_F16, false>(dx, dy, y, scale, rows, sk, rows, kNoWindow, nullptr, 1, st);
+}
+
+int nhp_masked_softmax_dropout_fwd(void* dropped, void* y, const void* x, const uint8_t* mask, float scale,
+                                   int64_t b, int64_t np, int64_t sq, int64_t sk, int64_t pad_batches, float p,
+                                   uint64_t seed, uint64_t offset, int dtype, void* stream)
+{
+    if (dtype != NHP_F16 && dtype != NHP_BF16) return NHP_ERR_DTYPE;
+    if (b < 0 || np < 0 || sq < 0 || sk < 0 || !(p >= 0.0f && p < 1.0f)) return NHP_ERR_SHAPE;
+    if (b == 0 || np == 0 || sq == 0 || sk == 0) return NHP_OK;
+    if (pad_batches != 1 && pad_batches != b) return NHP_ERR_PAD_BATCHES;
+    if (b > kMaxRows / np - 1 || b * np > kMaxRows / sq - 1) return NHP_ERR_SHAPE;
+    if (!x || !y || !mask || !dropped) return NHP_ERR_NULL;
+    if (dropped == y || dropped == x) return NHP_ERR_ALIAS;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const DropoutKey dk = make_dropout_key(p, seed, offset);
+    return dtype == NHP_BF16 ? masked_fwd<NHP_BF16>(y, x, mask, scale, b, np, sq, sk, pad_batches, st, dropped, &dk)
+                             : masked_fwd<NHP_F16>(y, x, mask, scale, b, np, sq, sk, pad_batches, st, dropped, &dk);
+}
+
+int nhp_masked_softmax_dropout_bwd(void* dx, const void* dy, const void* y, float scale, int64_t rows, int64_t sk,
+                                   float p, uint64_t seed, uint64_t offset, int dtype, void* stream)
+{
+    if (dtype != NHP_F16 && dtype != NHP_BF16) return NHP_ERR_DTYPE;
+    if (rows < 0 || sk < 0 || !(p >= 0.0f && p < 1.0f)) return NHP_ERR_SHAPE;
+    if (rows == 0 || sk == 0) return NHP_OK;
+    if (rows >= kMaxRows) return NHP_ERR_SHAPE;
+    if (!dx || !dy || !y) return NHP_ERR_NULL;
+    if (dx == y) return NHP_ERR_ALIAS;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const DropoutKey dk = make_dropout_key(p, seed, offset);
+    return dtype == NHP_BF16
+               ? softmax_bwd<NHP_BF16, false>(dx, dy, y, scale, rows, sk, rows, kNoWindow, nullptr, 1, st, &dk)
+               : softmax_bwd<NHP_F16, false>(dx, dy, y, scale, rows, sk, rows, kNoWindow, nullptr, 1, st, &dk);
 }
 
 int nhp_softmax_batch_per_block(int64_t query_seq_len, int64_t key_seq_len, int64_t batches,

@@ -130,6 +130,29 @@ class ScaledMaskedSoftmax(torch.autograd.Function):
         return kernels.backward(output_grads, out, factor[0]), None, None
 
 
+class ScaledMaskedSoftmaxDropout(torch.autograd.Function):
+    """``dropout(softmax(where(mask, -10000, scale * x)))`` in one kernel forward and one backward.
+    No counterpart in the reference, which runs ``torch.nn.Dropout`` on the probabilities."""
+
+    @staticmethod
+    def forward(ctx, inputs, mask, scale, prob, seed):
+        import scaled_masked_softmax_cuda as kernels
+
+        factor = _scale_tensor(scale)
+        dropped, probs = kernels.forward_dropout(inputs, mask, factor[0], prob, seed)
+        ctx.conf = (float(prob), int(seed))
+        ctx.save_for_backward(probs, factor)
+        return dropped
+
+    @staticmethod
+    def backward(ctx, output_grads):
+        import scaled_masked_softmax_cuda as kernels
+
+        probs, factor = ctx.saved_tensors
+        prob, seed = ctx.conf
+        return kernels.backward_dropout(output_grads, probs, factor[0], prob, seed), None, None, None, None
+
+
 class FusedScaleMaskSoftmax(nn.Module):
     """Scaling, masking and softmax of attention scores ``[b, np, sq, sk]``.
 
@@ -149,8 +172,9 @@ class FusedScaleMaskSoftmax(nn.Module):
             inside the causal kernel, and by the other branches with the same
             roundings, so the caller must not add it.
         attention_dropout: (extension) dropout probability applied to the
-            probabilities in training mode; fused with the softmax on the
-            causal branch. The caller must not apply its own dropout.
+            probabilities in training mode; fused with the softmax on both
+            kernel branches (unless a bias, AliBi or key lengths are in play).
+            The caller must not apply its own dropout.
     """
 
     def __init__(self, input_in_fp16, input_in_bf16, fusion_type, mask_func, softmax_in_fp32, scale,
@@ -195,6 +219,11 @@ class FusedScaleMaskSoftmax(nn.Module):
                 probs = ScaledUpperTriangMaskedSoftmaxDropout.apply(input.view(b * np, sq, sk), factor, dropout, seed,
                                                                     self.sliding_window_width)
                 return probs.view(b, np, sq, sk)
+            if (dropout > 0.0 and self.general_mask_fusion and bias is None and key_lengths is None
+                    and self.alibi_slopes is None):
+                factor = 1.0 if self.scale is None else self.scale
+                seed = int(torch.empty((), dtype=torch.int64).random_().item())
+                return ScaledMaskedSoftmaxDropout.apply(input, mask, factor, dropout, seed)
             probs = self.forward_fused_softmax(input, mask, bias, key_lengths)
         else:
             probs = self.forward_torch_softmax(input, mask, bias, key_lengths)

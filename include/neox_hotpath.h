@@ -161,6 +161,24 @@ int nhp_causal_softmax_dropout_bwd(void* dx, const void* dy, const void* y, floa
                                    int64_t attn_batches, int64_t seq_len, int64_t window,
                                    float p, uint64_t seed, uint64_t offset, int dtype, void* stream);
 
+/*
+ * The same for the padding-mask softmax: y as nhp_masked_softmax_fwd, dropped = keep ? y / (1 - p) : 0
+ * over the flat element index of the [b, np, sq, sk] tensor; the backward is nhp_masked_softmax_bwd of
+ * g = keep ? dy / (1 - p) : 0 (rows = b * np * sq).
+ *
+ * Replaces scaled_masked_softmax_cuda.forward / backward
+ * (megatron/fused_kernels/scaled_masked_softmax.cpp:33-59) followed / preceded by torch.nn.Dropout
+ * (self.attention_dropout, megatron/model/transformer.py:509,592-593).
+ */
+int nhp_masked_softmax_dropout_fwd(void* dropped, void* y, const void* x, const uint8_t* mask,
+                                   float scale, int64_t b, int64_t np, int64_t sq, int64_t sk,
+                                   int64_t pad_batches, float p, uint64_t seed, uint64_t offset,
+                                   int dtype, void* stream);
+
+int nhp_masked_softmax_dropout_bwd(void* dx, const void* dy, const void* y, float scale,
+                                   int64_t rows, int64_t sk, float p, uint64_t seed, uint64_t offset,
+                                   int dtype, void* stream);
+
 /* ------------------------------------------------------------------------
  * Scaled padding-masked softmax
  * ---------------------------------------------------------------------- */

@@ -428,3 +428,29 @@ def causal_softmax_dropout_bwd(dy, y, scale, p, seed, offset=0, window=None):
                                                    dy.size(1), -1 if window is None else int(window), float(p), int(seed),
                                                    int(offset), _DT[dy.dtype]), "causal_softmax_dropout_bwd")
     return dx
+
+
+def _dropout_of_stored(t, p, seed, offset):
+    """keep ? t / (1 - p) : 0 on the stored values of t, rounded to t's dtype (fp32 product, as in
+    oracle_causal_softmax_dropout_fwd), with the mask of dropout_mask over t's flat index."""
+    import numpy as np
+
+    keep = dropout_mask(t.numel(), p, seed, offset).view(t.shape)
+    ds = torch.tensor(np.float32(1.0 / (1.0 - float(np.float32(p)))))
+    scaled = (t.float() * ds).to(t.dtype)
+    return torch.where(keep, scaled, torch.zeros_like(scaled))
+
+
+def masked_softmax_dropout_fwd(x, mask, scale, p, seed, offset=0):
+    """Returns (dropped, y) for the padding-mask softmax followed by attention dropout
+    (megatron/model/transformer.py:588-593): the composition of masked_softmax_fwd and the dropout of its
+    stored result, the mask taken over the flat index of the [b, np, sq, sk] tensor."""
+    y = masked_softmax_fwd(x, mask, scale)
+    return _dropout_of_stored(y, p, seed, offset), y
+
+
+def masked_softmax_dropout_bwd(dy, y, scale, p, seed, offset=0):
+    """Gradient with respect to the scores, given the gradient of dropout(y): the dropout backward stored in
+    the storage type, then the (unmasked) softmax backward."""
+    dy, y = _cpu_contig(dy), _cpu_contig(y)
+    return softmax_bwd(_dropout_of_stored(dy, p, seed, offset), y, scale, False)

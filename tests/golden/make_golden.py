@@ -141,6 +141,11 @@ def main():
             keep=oracle.dropout_mask(x.numel(), p, sd).to(torch.uint8), y=y, dropped=dropped,
             dx=oracle.causal_softmax_dropout_bwd(dy, y, scale, p, sd),
             bda=oracle.bias_dropout_add(x.view(-1, 24), bias, dy.view(-1, 24), p, sd))
+        # the same through the padding-mask softmax: x as [b = 3, np = 1, sq = 24, sk = 24], the last entry fully masked
+        pad = util.padding_mask(3, 24, 24, seed=seed, full_batch=2, lo=6)
+        mdropped, my = oracle.masked_softmax_dropout_fwd(x.view(3, 1, 24, 24), pad, scale, p, sd)
+        put(name, pad=pad.to(torch.uint8), m_y=my, m_dropped=mdropped,
+            m_dx=oracle.masked_softmax_dropout_bwd(dy.view(3, 1, 24, 24), my, scale, p, sd))
 
     path = os.path.join(HERE, "layer_golden.npz")
     np.savez_compressed(path, **out)

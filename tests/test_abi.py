@@ -138,6 +138,18 @@ def test_argument_validation_of_the_layer_entry_points(hotpath):
     assert lib.nhp_bias_gelu_bwd_workspace_bytes(0, 8, BF16) == 0
     big = lib.nhp_bias_gelu_bwd_workspace_bytes(1 << 20, 8192, BF16)
     assert 0 < big <= 512 * 8192 * 4                                               # bounded, whatever the row count
+    # softmax + dropout: probability range, missing or aliased second output, mask layout
+    assert lib.nhp_causal_softmax_dropout_fwd(q, p, p, 1.0, 2, 8, -1, 1.0, 1, 0, BF16, None) == -2
+    assert lib.nhp_causal_softmax_dropout_fwd(null, p, p, 1.0, 2, 8, -1, 0.1, 1, 0, BF16, None) == -3
+    assert lib.nhp_causal_softmax_dropout_fwd(p, p, q, 1.0, 2, 8, -1, 0.1, 1, 0, BF16, None) == -6
+    assert lib.nhp_masked_softmax_dropout_fwd(q, p, p, p, 1.0, 2, 2, 4, 8, 2, -0.5, 1, 0, BF16, None) == -2
+    assert lib.nhp_masked_softmax_dropout_fwd(q, p, p, p, 1.0, 2, 2, 4, 8, 3, 0.1, 1, 0, BF16, None) == -4   # pad_batches
+    assert lib.nhp_masked_softmax_dropout_fwd(q, p, p, null, 1.0, 2, 2, 4, 8, 2, 0.1, 1, 0, BF16, None) == -3
+    assert lib.nhp_masked_softmax_dropout_fwd(p, p, q, p, 1.0, 2, 2, 4, 8, 2, 0.1, 1, 0, BF16, None) == -6
+    assert lib.nhp_masked_softmax_dropout_fwd(q, p, p, p, 1.0, 2, 2, 4, 8, 2, 0.1, 1, 0, F32, None) == -1
+    assert lib.nhp_masked_softmax_dropout_bwd(p, q, p, 1.0, 16, 8, 0.1, 1, 0, BF16, None) == -6              # dx == y
+    assert lib.nhp_masked_softmax_dropout_bwd(q, q, p, 1.0, 16, 8, 1.5, 1, 0, BF16, None) == -2
+    assert lib.nhp_masked_softmax_dropout_bwd(null, null, null, 1.0, 0, 8, 0.1, 1, 0, BF16, None) == 0
     assert lib.nhp_column_sum(null, p, p, 4, 8, BF16, None) == -3
     assert lib.nhp_column_sum(q, p, null, 4, 8, BF16, None) == -3                  # workspace missing
     assert lib.nhp_column_sum(p, p, q, 4, 8, BF16, None) == -6                     # sums over their own input

@@ -21,7 +21,7 @@ def get(prefix, key):
     if arr.ndim == 0:
         return arr.item()
     t = torch.from_numpy(np.ascontiguousarray(arr))
-    if key in ("lengths", "keep"):
+    if key in ("lengths", "keep", "pad"):
         return t
     if key in FP32_KEYS:
         return t.view(torch.float32)
@@ -103,6 +103,10 @@ def test_oracle_reproduces_dropout_golden(name):
     assert same(y, get(name, "y")) and same(dropped, get(name, "dropped"))
     assert same(oracle.causal_softmax_dropout_bwd(dy, y, scale, p, seed), get(name, "dx"))
     assert same(oracle.bias_dropout_add(x.view(-1, 24), bias, dy.view(-1, 24), p, seed), get(name, "bda"))
+    pad = get(name, "pad").bool()
+    mdropped, my = oracle.masked_softmax_dropout_fwd(x.view(3, 1, 24, 24), pad, scale, p, seed)
+    assert same(my, get(name, "m_y")) and same(mdropped, get(name, "m_dropped"))
+    assert same(oracle.masked_softmax_dropout_bwd(dy.view(3, 1, 24, 24), my, scale, p, seed), get(name, "m_dx"))
 
 
 def ptr(t):
@@ -130,6 +134,15 @@ def test_gpu_matches_dropout_golden(hotpath, name):
     out = torch.empty((a * s, s), dtype=x.dtype, device="cuda")
     assert L.nhp_bias_dropout_add(out.data_ptr(), x.data_ptr(), bias.data_ptr(), dy.data_ptr(), a * s, s, p, seed, 0, code, None) == 0
     assert same(out.cpu(), get(name, "bda"))
+    # the padding-mask softmax with dropout
+    pad = get(name, "pad").cuda()
+    my, x4, dy4 = get(name, "m_y").cuda(), x.view(3, 1, s, s), dy.view(3, 1, s, s)
+    assert L.nhp_masked_softmax_dropout_fwd(gd.data_ptr(), gy.data_ptr(), x4.data_ptr(), pad.data_ptr(), scale, 3, 1, s, s, 3, p, seed,
+                                            0, code, None) == 0
+    util.assert_ulp_close(gy.cpu().view(3, 1, s, s), my.cpu(), 2, name)
+    assert same(gd.cpu(), oracle.bias_dropout_add(gy.cpu(), None, None, p, seed))
+    assert L.nhp_masked_softmax_dropout_bwd(gdx.data_ptr(), dy4.data_ptr(), my.data_ptr(), scale, 3 * s, s, p, seed, 0, code, None) == 0
+    util.assert_softmax_bwd_close(gdx.cpu(), get(name, "m_dx").view(3, s, s), g, my.cpu().view(3, s, s), scale, name)
 
 
 @pytest.mark.gpu

@@ -294,8 +294,55 @@ def test_module_with_attention_dropout():
     # evaluation mode: no dropout, the plain kernel
     m.eval()
     util.assert_ulp_close(m(x.to(DEV), mask).cpu().view(-1, s, s), oracle.causal_softmax_fwd(x.view(-1, s, s), scale), 2, "eval")
-    # the general-mask branch applies torch's dropout after the kernel: same rate, rows still normalised on average
+    # the general-mask branch has its own fused kernel: same mask definition over the [b, np, sq, sk] tensor
     g = FusedScaleMaskSoftmax(False, True, T.general, fb.fill_masked_with_dtype_min, True, scale, attention_dropout=p)
-    yg = g(x.to(DEV), mask)
-    zero_rate = ((yg == 0) & ~mask).float().sum().item() / (~mask).expand_as(yg).float().sum().item()
+    torch.manual_seed(3)
+    xg = x.to(DEV).requires_grad_(True)
+    yg = g(xg, mask)
+    yg.backward(dy.to(DEV).clone())
+    want_gd, want_gy = oracle.masked_softmax_dropout_fwd(x, mask.cpu(), scale, p, seed)
+    keep4 = keep.view(b, np_, s, s)
+    assert int(util.raw_bits(yg.detach().cpu())[~keep4].abs().max()) == 0
+    assert (yg.detach().cpu().float() - want_gd.float()).abs().max().item() <= 2.0**-7 * want_gd.float().abs().max().item()
+    want_gdx = oracle.masked_softmax_dropout_bwd(dy, want_gy, scale, p, seed)
+    assert (xg.grad.cpu().float() - want_gdx.float()).norm().item() <= 2.0**-6 * want_gdx.float().norm().item()
+    # with a bias the module falls back to torch's dropout after the kernel: same rate
+    yb = g(x.to(DEV), mask, bias=torch.zeros((1, np_, s, s), dtype=dtype, device=DEV))
+    zero_rate = ((yb == 0) & ~mask).float().sum().item() / (~mask).expand_as(yb).float().sum().item()
     assert abs(zero_rate - p) < 0.02
+
+
+# (b, np, sq, sk): every forward geometry of the padding-mask kernel incl. the scalar fallback, both mask layouts
+MASKED_DROPOUT_CASES = [(2, 3, 8, 64), (3, 2, 5, 200), (2, 2, 12, 512), (4, 2, 4, 1024), (2, 4, 16, 2048), (1, 2, 4, 4096),
+                        (1, 2, 2, 8192), (2, 2, 6, 1001), (2, 1, 3, 24)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
+@pytest.mark.parametrize("pad_batches", ["one", "each"])
+@pytest.mark.parametrize("case", MASKED_DROPOUT_CASES, ids=lambda c: "x".join(map(str, c)))
+def test_masked_softmax_with_attention_dropout_vs_oracle(hotpath, case, pad_batches, dtype):
+    """As the causal test above, for the padding-mask kernel: probabilities within 2 ulp, the dropped tensor exactly
+    the oracle's dropout of the stored probabilities, the backward against the oracle given the same y."""
+    import scaled_masked_softmax_cuda as ext
+
+    b, np_, sq, sk = case
+    print(f"masked softmax+dropout case {case} {pad_batches} {dtype}", flush=True)
+    scale, p, seed = 1 / math.sqrt(128), 0.15, 4321 + sk
+    x = util.randn((b, np_, sq, sk), dtype, seed=sk, std=2.0)
+    dy = util.randn((b, np_, sq, sk), dtype, seed=sk + 1)
+    mask = util.padding_mask(b, sq, sk, seed=sk, full_batch=b - 1, lo=sk // 4)
+    if pad_batches == "one":
+        mask = mask[:1].contiguous()
+    want_y = oracle.masked_softmax_fwd(x, mask, scale)
+    dropped, y = [t.cpu() for t in ext.forward_dropout(x.to(DEV), mask.to(DEV), scale, p, seed)]
+    util.assert_ulp_close(y, want_y, 2, "y")
+    assert torch.equal(util.raw_bits(dropped), util.raw_bits(oracle.bias_dropout_add(y, None, None, p, seed)))
+    want_dx = oracle.masked_softmax_dropout_bwd(dy, want_y, scale, p, seed)
+    got_dx = ext.backward_dropout(dy.to(DEV).clone(), want_y.to(DEV), scale, p, seed).cpu()
+    g = oracle.bias_dropout_add(dy, None, None, p, seed)
+    util.assert_softmax_bwd_close(got_dx.view(-1, sq, sk), want_dx.view(-1, sq, sk), g.view(-1, sq, sk), want_y.view(-1, sq, sk),
+                                  scale, "bwd")
+    # p = 0 degenerates to the plain pair
+    d0, y0 = ext.forward_dropout(x.to(DEV), mask.to(DEV), scale, 0.0, seed)
+    plain = ext.forward(x.to(DEV), mask.to(DEV), scale)
+    assert torch.equal(d0, y0) and torch.equal(y0, plain)

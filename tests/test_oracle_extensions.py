@@ -254,3 +254,34 @@ def test_softmax_with_attention_dropout_is_the_composition(dtype, window):
     # p = 0 is the plain pair
     d0, y0 = oracle.causal_softmax_dropout_fwd(x, scale, 0.0, seed, window=window)
     assert torch.equal(util.raw_bits(d0), util.raw_bits(plain)) and torch.equal(util.raw_bits(y0), util.raw_bits(plain))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+def test_masked_softmax_with_attention_dropout_is_the_composition(dtype):
+    """The padding-mask softmax followed by dropout: the probabilities are those of masked_softmax_fwd, the
+    dropped tensor equals the C oracle's dropout of them (one shared mask definition over the flat index), the
+    backward is the dropout backward followed by the unmasked softmax backward and matches float64 autograd
+    on the rows that are not fully masked."""
+    b, np_, sq, sk, scale, p, seed = 3, 2, 5, 24, 0.4, 0.3, 91
+    x = util.randn((b, np_, sq, sk), dtype, seed=1, std=2.0)
+    dy = util.randn((b, np_, sq, sk), dtype, seed=2)
+    mask = util.padding_mask(b, sq, sk, seed=3, full_batch=1, lo=4)
+    dropped, y = oracle.masked_softmax_dropout_fwd(x, mask, scale, p, seed)
+    plain = oracle.masked_softmax_fwd(x, mask, scale)
+    assert torch.equal(util.raw_bits(y), util.raw_bits(plain))
+    assert torch.equal(util.raw_bits(dropped), util.raw_bits(oracle.bias_dropout_add(plain, None, None, p, seed)))
+    keep = oracle.dropout_mask(x.numel(), p, seed).view_as(x)
+    assert dropped[~keep].abs().max().item() == 0
+    dx = oracle.masked_softmax_dropout_bwd(dy, y, scale, p, seed)
+    g = oracle.bias_dropout_add(dy, None, None, p, seed)
+    assert torch.equal(util.raw_bits(dx), util.raw_bits(oracle.softmax_bwd(g, y, scale, False)))
+    xd = x.double().requires_grad_(True)
+    f32scale = float(torch.tensor(scale, dtype=torch.float32))
+    full = mask.expand(b, np_, sq, sk)
+    probs = torch.softmax((xd * f32scale).masked_fill(full, -10000.0), -1)
+    (probs * keep / (1 - p)).backward(dy.double())
+    live = ~mask.all(dim=-1, keepdim=True).expand_as(x)       # fully masked rows: the kernel backward has no mask
+    err = ((dx.double() - xd.grad).abs() * live).max().item()
+    assert err <= 4 * 2.0 ** (-8 if dtype == torch.bfloat16 else -11) * xd.grad.abs().max().item()
+    d0, y0 = oracle.masked_softmax_dropout_fwd(x, mask, scale, 0.0, seed)
+    assert torch.equal(util.raw_bits(d0), util.raw_bits(plain)) and torch.equal(util.raw_bits(y0), util.raw_bits(plain))
