@@ -79,6 +79,18 @@ def test_masked_softmax_random_shapes(hotpath, seed):
     want_dx = oracle.softmax_bwd(dy, want, scale, False)
     got_dx = util.abi_masked_bwd(hotpath, dy.to(DEV), want.to(DEV), scale).cpu()
     util.assert_softmax_bwd_close(got_dx, want_dx, dy, want, scale, "bwd")
+    if rng.random() < 0.6:   # the same with attention dropout in the kernel
+        import scaled_masked_softmax_cuda as ext
+
+        p, sd = rng.choice((0.1, 0.5)), rng.randint(0, 1 << 40)
+        if sq > 1:
+            dropped, y = [t.cpu() for t in ext.forward_dropout(x.to(DEV), mask.to(DEV), scale, p, sd)]
+            util.assert_ulp_close(y, want, 2, "fwd with dropout")
+            assert torch.equal(util.raw_bits(dropped), util.raw_bits(oracle.bias_dropout_add(y, None, None, p, sd)))
+            got_ddx = ext.backward_dropout(dy.to(DEV).clone(), want.to(DEV), scale, p, sd).cpu()
+            g = oracle.bias_dropout_add(dy, None, None, p, sd)
+            util.assert_softmax_bwd_close(got_ddx, oracle.masked_softmax_dropout_bwd(dy, want, scale, p, sd), g, want, scale,
+                                          "bwd with dropout")
 
 
 @pytest.mark.parametrize("seed", range(16))
@@ -96,6 +108,39 @@ def test_rope_random_shapes(hotpath, seed):
     for backward in (False, True):
         want = oracle.rope_cached(t, cos, sin, backward=backward)
         got = util.abi_rope_cached(hotpath, t.to(DEV), cos.to(DEV), sin.to(DEV), backward=backward).cpu()
+        assert torch.equal(util.raw_bits(got), util.raw_bits(want)), backward
+    # the same values laid out contiguously along the sequence (the layout of the key gradient)
+    seq_major = t.permute(1, 2, 3, 0).contiguous().to(DEV).permute(3, 0, 1, 2)
+    assert seq_major.stride(0) == 1 or s == 1
+    for backward in (False, True):
+        want = oracle.rope_cached(t, cos, sin, backward=backward)
+        got = util.abi_rope_cached(hotpath, seq_major, cos.to(DEV), sin.to(DEV), backward=backward).cpu()
+        assert torch.equal(util.raw_bits(got), util.raw_bits(want)), ("sequence-major", backward)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_rope_sequence_major_random_shapes(hotpath, seed):
+    """Shapes inside and around the conditions of the transposing kernel (s a multiple of 8 or not, every head
+    size it takes and some it does not, windows of a longer sequence)."""
+    rng = random.Random(3500 + seed)
+    dtype = rng.choice(HALF)
+    s_total = rng.choice((8, 64, 72, 200, 256, 1000, 1001, 130))
+    b, h = rng.randint(1, 3), rng.randint(1, 5)
+    d = rng.choice((32, 64, 80, 96, 128, 160, 256, 512, 24))
+    d2 = rng.choice([v for v in (d, d // 2, d // 4, 16, 32) if 2 <= v <= d and v % 2 == 0])
+    first = rng.choice((0, 0, 8, 3))
+    s = s_total - first
+    print(f"rope sequence-major s={s} of {s_total} b={b} h={h} d={d} d2={d2} {dtype}", flush=True)
+    base = util.randn((b, h, d, s_total), dtype, seed=seed)
+    t = base.permute(3, 0, 1, 2)[first:]
+    t_d = base.to(DEV).permute(3, 0, 1, 2)[first:]
+    g = torch.Generator().manual_seed(seed)
+    ang = (torch.rand((s, 1, 1, d2), generator=g) * 20 - 10).contiguous()
+    cs = torch.float32 if rng.random() < 0.3 else dtype
+    cos, sin = ang.cos().to(cs), ang.sin().to(cs)
+    for backward in (False, True):
+        want = oracle.rope_cached(t.contiguous(), cos, sin, backward=backward)
+        got = util.abi_rope_cached(hotpath, t_d, cos.to(DEV), sin.to(DEV), backward=backward).cpu()
         assert torch.equal(util.raw_bits(got), util.raw_bits(want)), backward
 
 
