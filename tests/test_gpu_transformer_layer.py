@@ -154,3 +154,34 @@ def test_layer_with_dropout_trains_and_is_repeatable():
     xg = x.clone().requires_grad_(True)
     layer(xg, mask).float().square().mean().backward()
     assert torch.isfinite(xg.grad.float()).all() and all(torch.isfinite(p.grad.float()).all() for p in layer.parameters())
+
+
+def test_layer_under_activation_checkpointing_reproduces_its_dropout_masks():
+    """With activation checkpointing (GPT-NeoX's `checkpoint-activations`) the forward runs a second time in the
+    backward; the dropout seeds come from torch's CPU generator, whose state checkpointing restores, so the recomputed
+    masks are the ones of the first pass and the gradients equal those of a run without checkpointing."""
+    from torch.utils.checkpoint import checkpoint
+
+    from megatron.model.transformer_layer import TransformerLayer
+
+    cfg = args_for(gpt_j_residual=True, attention_dropout=0.1, hidden_dropout=0.1)
+    torch.manual_seed(0)
+    layer = TransformerLayer(cfg, mask_func, layer_number=1, rotary=True).to(DEV).to(torch.bfloat16).train()
+    s, b, h = 256, 2, cfg.hidden_size
+    x = util.randn((s, b, h), torch.bfloat16, seed=1).to(DEV)
+    g = util.randn((s, b, h), torch.bfloat16, seed=2).to(DEV)
+    mask = fb.causal_mask(s, DEV)
+
+    def run(use_checkpoint):
+        layer.zero_grad(set_to_none=True)
+        xg = x.clone().requires_grad_(True)
+        torch.manual_seed(21)
+        out = checkpoint(layer, xg, mask, use_reentrant=False) if use_checkpoint else layer(xg, mask)
+        out.backward(g)
+        return out.detach(), xg.grad, {n: p.grad.clone() for n, p in layer.named_parameters()}
+
+    out_a, dx_a, grads_a = run(False)
+    out_b, dx_b, grads_b = run(True)
+    assert torch.equal(out_a, out_b) and torch.equal(dx_a, dx_b)
+    for n in grads_a:
+        assert torch.equal(grads_a[n], grads_b[n]), n
