@@ -31,6 +31,7 @@ the drop-in extension modules (which call libneox_hotpath.so):
   bias-residual-1.4b  residual + (x + bias) on the hidden state [2048*8, 2048] bf16
   bias-dropout-add-1.4b  residual + dropout(x + bias) with p = 0.1, and the dropout backward, same shape
   layernorm-1.4b  LayerNorm fwd and bwd (with the parameter gradients) on the hidden state [2048*8, 2048] bf16
+  layernorm-pair-1.4b  the two LayerNorms of the parallel-residual layer in one launch each way, same hidden state
   rmsnorm-7b     RMSNorm fwd and bwd on [4096*4, 4096] bf16 (the Llama-2 7B hidden size)
 
 `value` is algorithmic bytes per step / wall time per step (inputs resident in
@@ -409,6 +410,43 @@ def make_workload(name, torch, dev):
         cfg = {"workload": name, "hidden_state": [rows, cols], "parameters": "bf16", "parameter_gradients": True,
                "bytes_convention": "every tensor element read or written once, plus the fp32 row statistics"}
         return step, kernel_bytes, {}, "norm_bwd", "bf16", cfg
+
+    if name == "layernorm-pair-1.4b":
+        from megatron.fused_kernels import _hotpath as hp
+
+        lib = hp.lib()
+        rows, cols = 2048 * 8, 2048
+        sets = [(randn((rows, cols), 10 * i, torch.bfloat16, 2.0), randn((rows, cols), 10 * i + 1, torch.bfloat16),
+                 randn((rows, cols), 10 * i + 2, torch.bfloat16)) for i in range(5)]
+        gammas = [randn((cols,), 91 + i, torch.float32) + 1 for i in range(2)]
+        betas = [randn((cols,), 95 + i, torch.float32) for i in range(2)]
+        y1, y2, dx = (torch.empty_like(sets[0][0]) for _ in range(3))
+        mean = torch.empty(rows, dtype=torch.float32, device=dev)
+        rstd = torch.empty_like(mean)
+        grads = [torch.empty_like(gammas[0]) for _ in range(4)]
+        ws = torch.empty(max(lib.nhp_layernorm_pair_bwd_workspace_bytes(rows, cols, hp.BF16), 16), dtype=torch.uint8,
+                         device=dev)
+        n = rows * cols
+        kernel_bytes = {"norm_pair_fwd": 3 * n * 2 + 4 * cols * 4 + rows * 8,
+                        "norm_pair_bwd": 4 * n * 2 + rows * 8 + 6 * cols * 4}
+        state = {"i": 0}
+        stream = hp.stream_of(y1)
+
+        def step(t):
+            x, g1, g2 = sets[state["i"] % len(sets)]
+            state["i"] += 1
+            t.run("norm_pair_fwd", lambda: hp.check(lib.nhp_layernorm_pair_fwd(
+                y1.data_ptr(), y2.data_ptr(), mean.data_ptr(), rstd.data_ptr(), x.data_ptr(), gammas[0].data_ptr(),
+                betas[0].data_ptr(), gammas[1].data_ptr(), betas[1].data_ptr(), 1e-5, rows, cols, hp.BF16, hp.F32, stream),
+                "LayerNorm pair forward"))
+            t.run("norm_pair_bwd", lambda: hp.check(lib.nhp_layernorm_pair_bwd(
+                dx.data_ptr(), grads[0].data_ptr(), grads[1].data_ptr(), grads[2].data_ptr(), grads[3].data_ptr(),
+                g1.data_ptr(), g2.data_ptr(), x.data_ptr(), mean.data_ptr(), rstd.data_ptr(), gammas[0].data_ptr(),
+                gammas[1].data_ptr(), ws.data_ptr(), rows, cols, hp.BF16, hp.F32, stream), "LayerNorm pair backward"))
+
+        cfg = {"workload": name, "hidden_state": [rows, cols], "parameters": "fp32", "parameter_gradients": True,
+               "bytes_convention": "every tensor element read or written once, plus the fp32 row statistics"}
+        return step, kernel_bytes, {}, "norm_pair_bwd", "bf16", cfg
 
     if name == "bias-dropout-add-1.4b":
         from megatron.fused_kernels import _hotpath as hp

@@ -145,6 +145,11 @@ struct NormFwdArgs {
     uint32_t rows, cpr, L, logL;
     int params_f32;
     uint32_t stat;  // RMSNorm: the statistic is taken over the first `stat` columns
+    // LayerNorm only, all null for a single norm: a second affine transform of the same normalised
+    // row (two LayerNorms applied to one input share their statistics)
+    void* y2;
+    const void* gamma2;
+    const void* beta2;
 };
 
 template <int DT, int K, int W, bool RMS>
@@ -218,6 +223,22 @@ norm_fwd_kernel(NormFwdArgs a)
             chunk_to_float<DT>(raw[k], f);
 #pragma unroll
             for (int j = 0; j < V; ++j) f[j] = (f[j] - mean) * scale;
+            if (!RMS && a.y2 != nullptr) {
+                float f2[V];
+#pragma unroll
+                for (int j = 0; j < V; ++j) f2[j] = f[j];
+                if (a.gamma2 != nullptr) {
+                    load_params<DT>(a.gamma2, a.params_f32 != 0, (size_t)cc * V, g);
+#pragma unroll
+                    for (int j = 0; j < V; ++j) f2[j] = f2[j] * g[j];
+                }
+                if (a.beta2 != nullptr) {
+                    load_params<DT>(a.beta2, a.params_f32 != 0, (size_t)cc * V, b);
+#pragma unroll
+                    for (int j = 0; j < V; ++j) f2[j] = f2[j] + b[j];
+                }
+                store16_stream(static_cast<S*>(a.y2) + (size_t)rs.row * cols + (size_t)cc * V, float_to_chunk<DT>(f2));
+            }
             if (a.gamma != nullptr) {
                 load_params<DT>(a.gamma, a.params_f32 != 0, (size_t)cc * V, g);
 #pragma unroll
@@ -250,7 +271,8 @@ __device__ __forceinline__ float block_sum_256(float v, float* slots)
 template <int DT, bool RMS>
 __global__ void __launch_bounds__(kNormScalarThreads)
 norm_fwd_scalar_kernel(void* y, float* mean_out, float* rstd_out, const void* x, const void* gamma,
-                       const void* beta, float eps, int eps_mode, uint64_t cols, uint64_t stat, int pdt)
+                       const void* beta, float eps, int eps_mode, uint64_t cols, uint64_t stat, int pdt,
+                       void* y2, const void* gamma2, const void* beta2)
 {
     __shared__ float slots[4];
     const uint64_t row = blockIdx.x;
@@ -274,6 +296,12 @@ norm_fwd_scalar_kernel(void* y, float* mean_out, float* rstd_out, const void* x,
     };
     for (uint64_t c = threadIdx.x; c < cols; c += kNormScalarThreads) {
         float f = (Elt<DT>::load(x, base + (int64_t)c) - mean) * scale;
+        if (!RMS && y2 != nullptr) {
+            float f2 = f;
+            if (gamma2 != nullptr) f2 = f2 * param(gamma2, c);
+            if (beta2 != nullptr) f2 = f2 + param(beta2, c);
+            Elt<DT>::store(y2, base + (int64_t)c, f2);
+        }
         if (gamma != nullptr) f = RMS ? param(gamma, c) * f : f * param(gamma, c);
         if (beta != nullptr) f = f + param(beta, c);
         Elt<DT>::store(y, base + (int64_t)c, f);
@@ -307,6 +335,11 @@ struct NormBwdArgs {
     uint32_t rows, cpr, L, logL, row_blocks;
     int params_f32;
     uint32_t stat;  // RMSNorm: number of leading columns the statistic was taken over
+    // PAIR kernels (two LayerNorms of one input): the second incoming gradient, its gamma and partial sums
+    const void* dy2;
+    const void* gamma2;
+    float* part_g2;
+    float* part_b2;
 };
 
 // Waves per workgroup of the backward kernel: as many row groups as the LDS buffer of the final
@@ -321,12 +354,16 @@ constexpr int bwd_waves()
     return g < W ? W : g;
 }
 
-constexpr int kBwdU = 2;  // row blocks in flight per iteration of the backward loop
+constexpr int kBwdU = 2;      // row blocks in flight per iteration of the backward loop
+constexpr int kBwdUPair = 1;  // the same with two incoming gradients
 
-template <int DT, int K, int W, bool RMS>
+// PAIR (LayerNorm only): g = dy * gamma + dy2 * gamma2, one dx for both norms, and the parameter
+// gradients of the second norm beside those of the first.
+template <int DT, int K, int W, bool RMS, bool PAIR = false, int U = (PAIR ? kBwdUPair : kBwdU)>
 __global__ void __launch_bounds__((bwd_waves<K, W, Elt<DT>::kVec>() * kWave))
 norm_bwd_kernel(NormBwdArgs a)
 {
+    static_assert(!PAIR || !RMS, "pairs of LayerNorms only");
     constexpr int V = Elt<DT>::kVec;
     constexpr int G = bwd_waves<K, W, V>();
     constexpr int T = G * kWave;
@@ -334,7 +371,7 @@ norm_bwd_kernel(NormBwdArgs a)
     using S = typename Elt<DT>::storage;
     // [parity of the loop iteration][sum][row group][wave]: one barrier per iteration is enough when
     // consecutive iterations use different slots
-    __shared__ float slots[2][2 * kBwdU][GROUPS > 1 ? GROUPS : 1][16];
+    __shared__ float slots[2][2 * U][GROUPS > 1 ? GROUPS : 1][16];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const size_t cols = (size_t)a.cpr * V;
@@ -346,7 +383,8 @@ norm_bwd_kernel(NormBwdArgs a)
     uint32_t cc[K];
     bool col_live[K];
     bool stat_full[K];  // every column of the chunk took part in the statistic
-    float gam[K][V];
+    constexpr int K2 = PAIR ? K : 1;  // extent of the arrays only a pair uses
+    float gam[K][V], gam2[K2][V];
 #pragma unroll
     for (int k = 0; k < K; ++k) {
         cc[k] = (uint32_t)(k * W + first.w) * a.L + first.l;
@@ -355,24 +393,34 @@ norm_bwd_kernel(NormBwdArgs a)
 #pragma unroll
         for (int j = 0; j < V; ++j) gam[k][j] = 1.0f;
         if (col_live[k] && a.gamma != nullptr) load_params<DT>(a.gamma, a.params_f32 != 0, (size_t)cc[k] * V, gam[k]);
+        if constexpr (PAIR) {
+#pragma unroll
+            for (int j = 0; j < V; ++j) gam2[k][j] = 1.0f;
+            if (col_live[k] && a.gamma2 != nullptr)
+                load_params<DT>(a.gamma2, a.params_f32 != 0, (size_t)cc[k] * V, gam2[k]);
+        }
     }
 
-    float acc_g[K][V], acc_b[K][V];
+    float acc_g[K][V], acc_b[K][V], acc_g2[K2][V], acc_b2[K2][V];
 #pragma unroll
     for (int k = 0; k < K; ++k)
 #pragma unroll
         for (int j = 0; j < V; ++j) acc_g[k][j] = acc_b[k][j] = 0.0f;
+#pragma unroll
+    for (int k = 0; k < K2; ++k)
+#pragma unroll
+        for (int j = 0; j < V; ++j) acc_g2[k][j] = acc_b2[k][j] = 0.0f;
 
-    // Every iteration takes kBwdU consecutive row blocks; all their loads are issued before the
+    // Every iteration takes U consecutive row blocks; all their loads are issued before the
     // first value is used (several rows in flight per thread without relying on a prefetch that
     // the compiler would have to track across the loop's back edge).
     int parity = 0;
-    for (uint32_t rb0 = blockIdx.x * kBwdU; rb0 < a.row_blocks; rb0 += gridDim.x * kBwdU) {
-        RowSlot rs[kBwdU];
-        u32x4 rg[kBwdU][K], rx[kBwdU][K];
-        float mean[kBwdU], scale[kBwdU];
+    for (uint32_t rb0 = blockIdx.x * U; rb0 < a.row_blocks; rb0 += gridDim.x * U) {
+        RowSlot rs[U];
+        u32x4 rg[U][K], rx[U][K], rg2[U][K2];
+        float mean[U], scale[U];
 #pragma unroll
-        for (int u = 0; u < kBwdU; ++u) {
+        for (int u = 0; u < U; ++u) {
             rs[u] = locate<W, G>(rb0 + u, a.rows, a.L, a.logL, wave, lane);
             rs[u].ok = rs[u].ok && rb0 + u < a.row_blocks;
             const S* gr = static_cast<const S*>(a.dy) + (size_t)rs[u].row * cols;
@@ -381,9 +429,12 @@ norm_bwd_kernel(NormBwdArgs a)
             for (int k = 0; k < K; ++k) {
                 rg[u][k] = u32x4{0, 0, 0, 0};
                 rx[u][k] = u32x4{0, 0, 0, 0};
+                if constexpr (PAIR) rg2[u][k] = u32x4{0, 0, 0, 0};
                 if (rs[u].ok && col_live[k]) {
                     rg[u][k] = load16_stream(gr + (size_t)cc[k] * V);
                     rx[u][k] = load16_stream(xr + (size_t)cc[k] * V);
+                    if constexpr (PAIR)
+                        rg2[u][k] = load16_stream(static_cast<const S*>(a.dy2) + (size_t)rs[u].row * cols + (size_t)cc[k] * V);
                 }
             }
             mean[u] = 0.0f;
@@ -394,20 +445,26 @@ norm_bwd_kernel(NormBwdArgs a)
             }
         }
 
-        float s1[kBwdU], s2[kBwdU];
+        float s1[U], s2[U];
 #pragma unroll
-        for (int u = 0; u < kBwdU; ++u) {
+        for (int u = 0; u < U; ++u) {
             s1[u] = s2[u] = 0.0f;
 #pragma unroll
             for (int k = 0; k < K; ++k) {
                 if (rs[u].ok && col_live[k]) {
-                    float fg[V], fx[V];
+                    float fg[V], fx[V], fg2[V];
                     chunk_to_float<DT>(rg[u][k], fg);
                     chunk_to_float<DT>(rx[u][k], fx);
+                    if constexpr (PAIR) chunk_to_float<DT>(rg2[u][k], fg2);
 #pragma unroll
                     for (int j = 0; j < V; ++j) {
                         const float xh = (fx[j] - mean[u]) * scale[u];
-                        const float g = fg[j] * gam[k][j];
+                        float g = fg[j] * gam[k][j];
+                        if constexpr (PAIR) {
+                            g = g + fg2[j] * gam2[k][j];
+                            acc_g2[k][j] += fg2[j] * xh;
+                            acc_b2[k][j] += fg2[j];
+                        }
                         s1[u] += g;
                         s2[u] += g * xh;
                         acc_g[k][j] += fg[j] * xh;
@@ -424,14 +481,14 @@ norm_bwd_kernel(NormBwdArgs a)
             const int grp = rs[0].group, w = rs[0].w;
             if (lane == 0) {
 #pragma unroll
-                for (int u = 0; u < kBwdU; ++u) {
+                for (int u = 0; u < U; ++u) {
                     mine[2 * u][grp][w] = s1[u];
                     mine[2 * u + 1][grp][w] = s2[u];
                 }
             }
             __syncthreads();
 #pragma unroll
-            for (int u = 0; u < kBwdU; ++u) {
+            for (int u = 0; u < U; ++u) {
                 s1[u] = mine[2 * u][grp][0];
                 s2[u] = mine[2 * u + 1][grp][0];
 #pragma unroll
@@ -444,7 +501,7 @@ norm_bwd_kernel(NormBwdArgs a)
         }
 
 #pragma unroll
-        for (int u = 0; u < kBwdU; ++u) {
+        for (int u = 0; u < U; ++u) {
             // LayerNorm: t = (s1 + xhat * s2) / n as c1 + xhat * c2 (no division per element)
             const float c1 = s1[u] / n;
             const float k2 = RMS ? rms_bwd_factor(s2[u], n, scale[u], a.eps, a.eps_mode) : s2[u] / n;
@@ -452,13 +509,15 @@ norm_bwd_kernel(NormBwdArgs a)
 #pragma unroll
             for (int k = 0; k < K; ++k) {
                 if (rs[u].ok && col_live[k]) {
-                    float fg[V], fx[V], o[V];
+                    float fg[V], fx[V], o[V], fg2[V];
                     chunk_to_float<DT>(rg[u][k], fg);
                     chunk_to_float<DT>(rx[u][k], fx);
+                    if constexpr (PAIR) chunk_to_float<DT>(rg2[u][k], fg2);
 #pragma unroll
                     for (int j = 0; j < V; ++j) {
                         const float xh = (fx[j] - mean[u]) * scale[u];
-                        const float g = fg[j] * gam[k][j];
+                        float g = fg[j] * gam[k][j];
+                        if constexpr (PAIR) g = g + fg2[j] * gam2[k][j];
                         float t = RMS ? xh * k2 : c1 + xh * k2;
                         if (RMS && !stat_full[k]) t = (cc[k] * V + j < a.stat) ? t : 0.0f;
                         o[j] = scale[u] * (g - t);
@@ -482,6 +541,15 @@ norm_bwd_kernel(NormBwdArgs a)
                     pg[j] = acc_g[k][j];
                     pb[j] = acc_b[k][j];
                 }
+                if constexpr (PAIR) {
+                    float* pg2 = a.part_g2 + (size_t)blockIdx.x * cols + (size_t)cc[k] * V;
+                    float* pb2 = a.part_b2 + (size_t)blockIdx.x * cols + (size_t)cc[k] * V;
+#pragma unroll
+                    for (int j = 0; j < V; ++j) {
+                        pg2[j] = acc_g2[k][j];
+                        pb2[j] = acc_b2[k][j];
+                    }
+                }
             }
         }
     } else {
@@ -489,15 +557,23 @@ norm_bwd_kernel(NormBwdArgs a)
         // them adds the others up, in a fixed order
         const uint32_t stride = (W > 1) ? (uint32_t)(W * kWave) : a.L;
         __shared__ float red[K * V * T];
-        for (int pass = 0; pass < 2; ++pass) {
+        for (int pass = 0; pass < (PAIR ? 4 : 2); ++pass) {
             __syncthreads();
 #pragma unroll
             for (int k = 0; k < K; ++k)
 #pragma unroll
-                for (int j = 0; j < V; ++j) red[(k * V + j) * T + threadIdx.x] = pass == 0 ? acc_g[k][j] : acc_b[k][j];
+                for (int j = 0; j < V; ++j) {
+                    float v = pass == 0 ? acc_g[k][j] : acc_b[k][j];
+                    if constexpr (PAIR) {
+                        if (pass == 2) v = acc_g2[k][j];
+                        if (pass == 3) v = acc_b2[k][j];
+                    }
+                    red[(k * V + j) * T + threadIdx.x] = v;
+                }
             __syncthreads();
             if (threadIdx.x < stride) {
-                float* dst = (pass == 0 ? a.part_g : a.part_b) + (size_t)blockIdx.x * cols;
+                float* part = pass == 0 ? a.part_g : pass == 1 ? a.part_b : pass == 2 ? a.part_g2 : a.part_b2;
+                float* dst = part + (size_t)blockIdx.x * cols;
 #pragma unroll
                 for (int k = 0; k < K; ++k) {
                     if (col_live[k]) {
@@ -522,7 +598,8 @@ norm_bwd_kernel(NormBwdArgs a)
 template <int DT, bool RMS>
 __global__ void __launch_bounds__(kNormScalarThreads)
 norm_bwd_scalar_kernel(void* dx, const void* dy, const void* x, const float* mean_in, const float* rstd_in,
-                       const void* gamma, float eps, int eps_mode, uint64_t cols, uint64_t stat, int pdt)
+                       const void* gamma, float eps, int eps_mode, uint64_t cols, uint64_t stat, int pdt,
+                       const void* dy2, const void* gamma2)
 {
     __shared__ float slots[4];
     const uint64_t row = blockIdx.x;
@@ -530,14 +607,20 @@ norm_bwd_scalar_kernel(void* dx, const void* dy, const void* x, const float* mea
     const float n = RMS ? (float)stat : (float)cols;
     const float mean = RMS ? 0.0f : mean_in[row];
     const float scale = rstd_in[row];
+    auto pval = [&](const void* p, uint64_t c) {
+        if (p == nullptr) return 1.0f;
+        return pdt == NHP_F32 ? static_cast<const float*>(p)[c] : Elt<DT>::load(p, (int64_t)c);
+    };
+    // the incoming gradient times gamma; with a second LayerNorm of the same input the sum of both
     auto gval = [&](uint64_t c) {
-        if (gamma == nullptr) return 1.0f;
-        return pdt == NHP_F32 ? static_cast<const float*>(gamma)[c] : Elt<DT>::load(gamma, (int64_t)c);
+        float g = Elt<DT>::load(dy, base + (int64_t)c) * pval(gamma, c);
+        if (!RMS && dy2 != nullptr) g = g + Elt<DT>::load(dy2, base + (int64_t)c) * pval(gamma2, c);
+        return g;
     };
     float s1 = 0.0f, s2 = 0.0f;
     for (uint64_t c = threadIdx.x; c < cols; c += kNormScalarThreads) {
         const float xh = (Elt<DT>::load(x, base + (int64_t)c) - mean) * scale;
-        const float g = Elt<DT>::load(dy, base + (int64_t)c) * gval(c);
+        const float g = gval(c);
         s1 += g;
         s2 += g * xh;
     }
@@ -546,7 +629,7 @@ norm_bwd_scalar_kernel(void* dx, const void* dy, const void* x, const float* mea
     const float k2 = RMS ? rms_bwd_factor(s2, n, scale, eps, eps_mode) : 0.0f;
     for (uint64_t c = threadIdx.x; c < cols; c += kNormScalarThreads) {
         const float xh = (Elt<DT>::load(x, base + (int64_t)c) - mean) * scale;
-        const float g = Elt<DT>::load(dy, base + (int64_t)c) * gval(c);
+        const float g = gval(c);
         const float t = RMS ? (c < stat ? xh * k2 : 0.0f) : (s1 + xh * s2) / n;
         Elt<DT>::store(dx, base + (int64_t)c, scale * (g - t));
     }
@@ -601,7 +684,7 @@ struct NormPlan {
 
 // Geometry for rows of cpr chunks: a wave reads 1-2 KiB of a row (1 KiB of each of its two
 // inputs in the backward); returns false when the row does not fit.
-static bool plan_norm(int64_t cpr, bool backward, NormPlan& p)
+static bool plan_norm(int64_t cpr, bool backward, NormPlan& p, bool pair_fwd = false)
 {
     if (cpr < 1) return false;
     p.L = 1;
@@ -613,8 +696,10 @@ static bool plan_norm(int64_t cpr, bool backward, NormPlan& p)
     const int64_t segs = (cpr + p.L - 1) / p.L;  // 16-byte chunks per lane over the whole row
     static const int fwd_table[][2] = {{1, 1}, {2, 1}, {2, 2}, {2, 4}, {2, 8}, {4, 8}, {4, 16}};
     static const int bwd_table[][2] = {{1, 1}, {1, 2}, {1, 4}, {2, 4}, {2, 8}, {4, 8}, {4, 16}};
+    // a forward that writes two results: a whole row of up to 4 chunks per lane in one wave measured faster
+    static const int pair_fwd_table[][2] = {{1, 1}, {2, 1}, {4, 1}, {2, 4}, {2, 8}, {4, 8}, {4, 16}};
     p.K = p.W = 0;
-    for (const auto& kw : (backward ? bwd_table : fwd_table)) {
+    for (const auto& kw : (backward ? bwd_table : pair_fwd ? pair_fwd_table : fwd_table)) {
         if ((int64_t)kw[0] * kw[1] >= segs) {
             p.K = kw[0];
             p.W = kw[1];
@@ -650,7 +735,7 @@ constexpr uint32_t kNormBwdWaves = 4096;
 
 static uint32_t norm_bwd_grid(uint32_t row_blocks, bool param_grads, int waves_per_block)
 {
-    row_blocks = (row_blocks + kBwdU - 1) / kBwdU;  // a workgroup takes kBwdU row blocks per iteration
+    row_blocks = (row_blocks + kBwdU - 1) / kBwdU;  // a workgroup takes up to kBwdU row blocks per iteration
     if (!param_grads) return row_blocks;
     const uint32_t cap = (uint32_t)norm_tune("NHP_NORM_GRID", (int)(kNormBwdWaves / (uint32_t)waves_per_block));
     return row_blocks < cap ? row_blocks : cap;
@@ -658,16 +743,28 @@ static uint32_t norm_bwd_grid(uint32_t row_blocks, bool param_grads, int waves_p
 
 static bool param_dtype_ok(int dtype, int pdt) { return pdt == dtype || pdt == NHP_F32; }
 
+// The second LayerNorm of a pair applied to one input (all null for a single norm).
+struct NormSecond {
+    void* y2 = nullptr;            // forward
+    const void* gamma2 = nullptr;  // forward and backward
+    const void* beta2 = nullptr;   // forward
+    const void* dy2 = nullptr;     // backward
+    void* dgamma2 = nullptr;       // backward
+    void* dbeta2 = nullptr;        // backward
+};
+
 template <int DT, bool RMS>
 static int norm_fwd(void* y, float* mean, float* rstd, const void* x, const void* gamma, const void* beta, float eps,
-                    int eps_mode, int64_t rows, int64_t cols, int64_t stat, int pdt, hipStream_t st)
+                    int eps_mode, int64_t rows, int64_t cols, int64_t stat, int pdt, hipStream_t st,
+                    const NormSecond& second = NormSecond{})
 {
     constexpr int V = Elt<DT>::kVec;
     NormPlan p;
-    const bool params_aligned = ptr_aligned16(gamma) && ptr_aligned16(beta);
-    if (cols % V == 0 && ptr_aligned16(x) && ptr_aligned16(y) && params_aligned && plan_norm(cols / V, false, p)) {
+    const bool params_aligned = ptr_aligned16(gamma) && ptr_aligned16(beta) && ptr_aligned16(second.gamma2) &&
+                                ptr_aligned16(second.beta2) && ptr_aligned16(second.y2);
+    if (cols % V == 0 && ptr_aligned16(x) && ptr_aligned16(y) && params_aligned && plan_norm(cols / V, false, p, second.y2 != nullptr)) {
         NormFwdArgs a{y, mean, rstd, x, gamma, beta, eps, eps_mode, (uint32_t)rows, (uint32_t)(cols / V),
-                      p.L, p.logL, pdt == NHP_F32 ? 1 : 0, (uint32_t)stat};
+                      p.L, p.logL, pdt == NHP_F32 ? 1 : 0, (uint32_t)stat, second.y2, second.gamma2, second.beta2};
         const int waves = p.W > 1 ? p.W : kNormBlockWaves;
         const uint32_t blocks = norm_row_blocks(rows, p, waves);
         const int threads = waves * kWave;
@@ -683,7 +780,8 @@ static int norm_fwd(void* y, float* mean, float* rstd, const void* x, const void
     }
     if (!grid_fits(rows, kNormScalarThreads)) return NHP_ERR_SHAPE;
     norm_fwd_scalar_kernel<DT, RMS><<<(uint32_t)rows, kNormScalarThreads, 0, st>>>(
-        y, mean, rstd, x, gamma, beta, eps, eps_mode, (uint64_t)cols, (uint64_t)stat, pdt);
+        y, mean, rstd, x, gamma, beta, eps, eps_mode, (uint64_t)cols, (uint64_t)stat, pdt, second.y2, second.gamma2,
+        second.beta2);
     return launch_result();
 }
 
@@ -699,26 +797,39 @@ static int64_t norm_workspace_bytes(int64_t rows, int64_t cols, int dtype)
 template <int DT, bool RMS>
 static int norm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, const void* x, const float* mean,
                     const float* rstd, const void* gamma, void* workspace, float eps, int eps_mode, int64_t rows,
-                    int64_t cols, int64_t stat, int pdt, hipStream_t st)
+                    int64_t cols, int64_t stat, int pdt, hipStream_t st, const NormSecond& second = NormSecond{})
 {
     constexpr int V = Elt<DT>::kVec;
     NormPlan p;
-    const bool want_params = dgamma != nullptr || dbeta != nullptr;
+    const bool pair = !RMS && second.dy2 != nullptr;
+    const bool want_params = dgamma != nullptr || dbeta != nullptr || second.dgamma2 != nullptr || second.dbeta2 != nullptr;
     if (cols % V == 0 && ptr_aligned16(dx) && ptr_aligned16(dy) && ptr_aligned16(x) && ptr_aligned16(gamma) &&
-        ptr_aligned16(workspace) && plan_norm(cols / V, true, p)) {
+        ptr_aligned16(second.dy2) && ptr_aligned16(second.gamma2) && ptr_aligned16(workspace) &&
+        plan_norm(cols / V, true, p)) {
         const int waves = bwd_waves_of(p, V);
         const uint32_t row_blocks = norm_row_blocks(rows, p, waves);
         const uint32_t grid = norm_bwd_grid(row_blocks, want_params, waves);
+        const size_t part = (size_t)grid * cols;
         float* part_g = want_params ? static_cast<float*>(workspace) : nullptr;
-        float* part_b = want_params ? part_g + (size_t)grid * cols : nullptr;
+        float* part_b = want_params ? part_g + part : nullptr;
+        float* part_g2 = (want_params && pair) ? part_g + 2 * part : nullptr;
+        float* part_b2 = (want_params && pair) ? part_g + 3 * part : nullptr;
         NormBwdArgs a{dx, part_g, part_b, dy, x, mean, rstd, gamma, eps, eps_mode, (uint32_t)rows,
-                      (uint32_t)(cols / V), p.L, p.logL, row_blocks, pdt == NHP_F32 ? 1 : 0, (uint32_t)stat};
+                      (uint32_t)(cols / V), p.L, p.logL, row_blocks, pdt == NHP_F32 ? 1 : 0, (uint32_t)stat,
+                      second.dy2, second.gamma2, part_g2, part_b2};
         const int threads = waves * kWave;
         if (!grid_fits(grid, threads)) return NHP_ERR_SHAPE;
         bool launched = false;
 #define X(K_, W_)                                                                      \
     if (!launched && p.K == K_ && p.W == W_) {                                         \
-        norm_bwd_kernel<DT, K_, W_, RMS><<<grid, threads, 0, st>>>(a);                 \
+        if constexpr (!RMS) {                                                          \
+            if (pair)                                                                  \
+                norm_bwd_kernel<DT, K_, W_, false, true><<<grid, threads, 0, st>>>(a); \
+            else                                                                       \
+                norm_bwd_kernel<DT, K_, W_, false, false><<<grid, threads, 0, st>>>(a); \
+        } else {                                                                       \
+            norm_bwd_kernel<DT, K_, W_, RMS><<<grid, threads, 0, st>>>(a);             \
+        }                                                                              \
         launched = true;                                                               \
     }
         NHP_NORM_GEOMETRIES(X)
@@ -729,17 +840,30 @@ static int norm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, const v
         const dim3 fgrid((uint32_t)((cols + kFinishCols - 1) / kFinishCols), 2);
         partial_rows_sum_kernel<DT><<<fgrid, kFinishCols * kFinishSlices, 0, st>>>(dgamma, dbeta, part_g, part_b, grid, (uint32_t)cols,
                                                             pdt == NHP_F32 ? 1 : 0);
+        rc = launch_result();
+        if (rc != NHP_OK || !pair) return rc;
+        partial_rows_sum_kernel<DT><<<fgrid, kFinishCols * kFinishSlices, 0, st>>>(
+            second.dgamma2, second.dbeta2, part_g2, part_b2, grid, (uint32_t)cols, pdt == NHP_F32 ? 1 : 0);
         return launch_result();
     }
     if (!grid_fits(rows, kNormScalarThreads)) return NHP_ERR_SHAPE;
     norm_bwd_scalar_kernel<DT, RMS><<<(uint32_t)rows, kNormScalarThreads, 0, st>>>(
-        dx, dy, x, mean, rstd, gamma, eps, eps_mode, (uint64_t)cols, (uint64_t)stat, pdt);
+        dx, dy, x, mean, rstd, gamma, eps, eps_mode, (uint64_t)cols, (uint64_t)stat, pdt, second.dy2, second.gamma2);
     int rc = launch_result();
     if (rc != NHP_OK || !want_params) return rc;
-    norm_param_grad_scalar_kernel<DT, RMS>
-        <<<(uint32_t)((cols + kNormScalarThreads - 1) / kNormScalarThreads), kNormScalarThreads, 0, st>>>(
+    const uint32_t pblocks = (uint32_t)((cols + kNormScalarThreads - 1) / kNormScalarThreads);
+    if (dgamma != nullptr || dbeta != nullptr) {
+        norm_param_grad_scalar_kernel<DT, RMS><<<pblocks, kNormScalarThreads, 0, st>>>(
             dgamma, dbeta, dy, x, mean, rstd, (uint64_t)rows, (uint64_t)cols, pdt);
-    return launch_result();
+        rc = launch_result();
+        if (rc != NHP_OK) return rc;
+    }
+    if (pair && (second.dgamma2 != nullptr || second.dbeta2 != nullptr)) {
+        norm_param_grad_scalar_kernel<DT, RMS><<<pblocks, kNormScalarThreads, 0, st>>>(
+            second.dgamma2, second.dbeta2, second.dy2, x, mean, rstd, (uint64_t)rows, (uint64_t)cols, pdt);
+        rc = launch_result();
+    }
+    return rc;
 }
 
 static int norm_check(int64_t rows, int64_t cols, int dtype, int pdt)
@@ -754,7 +878,7 @@ static int norm_check(int64_t rows, int64_t cols, int dtype, int pdt)
 template <bool RMS>
 static int norm_fwd_dispatch(void* y, float* mean, float* rstd, const void* x, const void* gamma, const void* beta,
                              float eps, int eps_mode, int64_t rows, int64_t cols, int64_t stat, int dtype, int pdt,
-                             void* stream)
+                             void* stream, const NormSecond& second = NormSecond{})
 {
     if (int rc = norm_check(rows, cols, dtype, pdt)) return rc;
     if (RMS && (eps_mode < 0 || eps_mode > 2)) return NHP_ERR_SHAPE;
@@ -764,37 +888,38 @@ static int norm_fwd_dispatch(void* y, float* mean, float* rstd, const void* x, c
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (dtype) {
     case NHP_F16:
-        return norm_fwd<NHP_F16, RMS>(y, mean, rstd, x, gamma, beta, eps, eps_mode, rows, cols, stat, pdt, st);
+        return norm_fwd<NHP_F16, RMS>(y, mean, rstd, x, gamma, beta, eps, eps_mode, rows, cols, stat, pdt, st, second);
     case NHP_BF16:
-        return norm_fwd<NHP_BF16, RMS>(y, mean, rstd, x, gamma, beta, eps, eps_mode, rows, cols, stat, pdt, st);
+        return norm_fwd<NHP_BF16, RMS>(y, mean, rstd, x, gamma, beta, eps, eps_mode, rows, cols, stat, pdt, st, second);
     default:
-        return norm_fwd<NHP_F32, RMS>(y, mean, rstd, x, gamma, beta, eps, eps_mode, rows, cols, stat, pdt, st);
+        return norm_fwd<NHP_F32, RMS>(y, mean, rstd, x, gamma, beta, eps, eps_mode, rows, cols, stat, pdt, st, second);
     }
 }
 
 template <bool RMS>
 static int norm_bwd_dispatch(void* dx, void* dgamma, void* dbeta, const void* dy, const void* x, const float* mean,
                              const float* rstd, const void* gamma, void* workspace, float eps, int eps_mode,
-                             int64_t rows, int64_t cols, int64_t stat, int dtype, int pdt, void* stream)
+                             int64_t rows, int64_t cols, int64_t stat, int dtype, int pdt, void* stream,
+                             const NormSecond& second = NormSecond{})
 {
     if (int rc = norm_check(rows, cols, dtype, pdt)) return rc;
     if (RMS && (eps_mode < 0 || eps_mode > 2)) return NHP_ERR_SHAPE;
     if (rows == 0 || cols == 0) return NHP_OK;
     if (RMS && (stat < 1 || stat > cols)) return NHP_ERR_SHAPE;
     if (!dx || !dy || !x || !rstd || (!RMS && !mean)) return NHP_ERR_NULL;
-    if ((dgamma != nullptr || dbeta != nullptr) && workspace == nullptr && norm_workspace_bytes(rows, cols, dtype) > 0)
-        return NHP_ERR_NULL;
+    const bool want_params = dgamma != nullptr || dbeta != nullptr || second.dgamma2 != nullptr || second.dbeta2 != nullptr;
+    if (want_params && workspace == nullptr && norm_workspace_bytes(rows, cols, dtype) > 0) return NHP_ERR_NULL;
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (dtype) {
     case NHP_F16:
         return norm_bwd<NHP_F16, RMS>(dx, dgamma, dbeta, dy, x, mean, rstd, gamma, workspace, eps, eps_mode, rows,
-                                      cols, stat, pdt, st);
+                                      cols, stat, pdt, st, second);
     case NHP_BF16:
         return norm_bwd<NHP_BF16, RMS>(dx, dgamma, dbeta, dy, x, mean, rstd, gamma, workspace, eps, eps_mode, rows,
-                                       cols, stat, pdt, st);
+                                       cols, stat, pdt, st, second);
     default:
         return norm_bwd<NHP_F32, RMS>(dx, dgamma, dbeta, dy, x, mean, rstd, gamma, workspace, eps, eps_mode, rows,
-                                      cols, stat, pdt, st);
+                                      cols, stat, pdt, st, second);
     }
 }
 
@@ -817,6 +942,41 @@ int nhp_layernorm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, const
 {
     return norm_bwd_dispatch<false>(dx, dgamma, dbeta, dy, x, mean, rstd, gamma, workspace, 0.0f, 0, rows, cols,
                                     cols, dtype, param_dtype, stream);
+}
+
+int nhp_layernorm_pair_fwd(void* y1, void* y2, float* mean, float* rstd, const void* x, const void* gamma1,
+                           const void* beta1, const void* gamma2, const void* beta2, float eps, int64_t rows,
+                           int64_t cols, int dtype, int param_dtype, void* stream)
+{
+    if (rows > 0 && cols > 0 && !y2) return NHP_ERR_NULL;
+    if (y1 != nullptr && y1 == y2) return NHP_ERR_ALIAS;
+    NormSecond second;
+    second.y2 = y2;
+    second.gamma2 = gamma2;
+    second.beta2 = beta2;
+    return norm_fwd_dispatch<false>(y1, mean, rstd, x, gamma1, beta1, eps, 0, rows, cols, cols, dtype, param_dtype,
+                                    stream, second);
+}
+
+int nhp_layernorm_pair_bwd(void* dx, void* dgamma1, void* dbeta1, void* dgamma2, void* dbeta2, const void* dy1,
+                           const void* dy2, const void* x, const float* mean, const float* rstd, const void* gamma1,
+                           const void* gamma2, void* workspace, int64_t rows, int64_t cols, int dtype,
+                           int param_dtype, void* stream)
+{
+    if (rows > 0 && cols > 0 && !dy2) return NHP_ERR_NULL;
+    NormSecond second;
+    second.dy2 = dy2;
+    second.gamma2 = gamma2;
+    second.dgamma2 = dgamma2;
+    second.dbeta2 = dbeta2;
+    return norm_bwd_dispatch<false>(dx, dgamma1, dbeta1, dy1, x, mean, rstd, gamma1, workspace, 0.0f, 0, rows, cols,
+                                    cols, dtype, param_dtype, stream, second);
+}
+
+int64_t nhp_layernorm_pair_bwd_workspace_bytes(int64_t rows, int64_t cols, int dtype)
+{
+    if (dtype != NHP_F16 && dtype != NHP_BF16 && dtype != NHP_F32) return 0;
+    return 2 * norm_workspace_bytes(rows, cols, dtype);
 }
 
 int nhp_rmsnorm_fwd(void* y, float* inv, const void* x, const void* scale, const void* offset, float eps,

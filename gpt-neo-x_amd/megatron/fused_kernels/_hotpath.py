@@ -69,6 +69,9 @@ def _declare(lib):
         "nhp_layernorm_bwd": ([vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, ci, ci, vp], ci),
         "nhp_rmsnorm_fwd": ([vp, vp, vp, vp, vp, f32, ci, i64, i64, ci, ci, vp], ci),
         "nhp_rmsnorm_bwd": ([vp, vp, vp, vp, vp, vp, vp, vp, f32, ci, i64, i64, ci, ci, vp], ci),
+        "nhp_layernorm_pair_fwd": ([vp, vp, vp, vp, vp, vp, vp, vp, vp, f32, i64, i64, ci, ci, vp], ci),
+        "nhp_layernorm_pair_bwd": ([vp] * 13 + [i64, i64, ci, ci, vp], ci),
+        "nhp_layernorm_pair_bwd_workspace_bytes": ([i64, i64, ci], i64),
         "nhp_column_sum": ([vp, vp, vp, i64, i64, ci, vp], ci),
         "nhp_column_sum_workspace_bytes": ([i64, i64, ci], i64),
         "nhp_rmsnorm_partial_fwd": ([vp, vp, vp, vp, vp, f32, ci, i64, i64, i64, ci, ci, vp], ci),

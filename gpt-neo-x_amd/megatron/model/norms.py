@@ -100,6 +100,81 @@ class _LayerNormFunction(torch.autograd.Function):
         return dx, dw, db, None
 
 
+class _LayerNormPairFunction(torch.autograd.Function):
+    """Two LayerNorms of one input: one pass forward (shared statistics, two results) and one pass backward
+    (one gradient for the input, the parameter gradients of both)."""
+
+    @staticmethod
+    def forward(ctx, x, weight1, bias1, weight2, bias2, eps):
+        what = "LayerNorm pair"
+        _hp.require_gpu(x, what)
+        cols = x.size(-1)
+        src = x.contiguous()
+        weight1, bias1 = _check_param(weight1, cols, x, what), _check_param(bias1, cols, x, what)
+        weight2, bias2 = _check_param(weight2, cols, x, what), _check_param(bias2, cols, x, what)
+        rows = src.numel() // max(cols, 1)
+        y1, y2 = torch.empty_like(src), torch.empty_like(src)
+        mean = torch.empty(rows, dtype=torch.float32, device=src.device)
+        rstd = torch.empty(rows, dtype=torch.float32, device=src.device)
+        code, pcode = _hp.dtype_code(src, what), _param_code(src, weight1, bias1, weight2, bias2)
+        with _hp.device_guard(src):
+            rc = _hp.lib().nhp_layernorm_pair_fwd(y1.data_ptr(), y2.data_ptr(), mean.data_ptr(), rstd.data_ptr(),
+                                                  src.data_ptr(), _ptr(weight1), _ptr(bias1), _ptr(weight2), _ptr(bias2),
+                                                  float(eps), rows, cols, code, pcode, _hp.stream_of(src))
+        _hp.check(rc, what)
+        ctx.save_for_backward(src, weight1, weight2, mean, rstd)
+        ctx.has_bias = (bias1 is not None, bias2 is not None)
+        ctx.codes = (code, pcode)
+        return y1, y2
+
+    @staticmethod
+    def backward(ctx, grad1, grad2):
+        what = "LayerNorm pair backward"
+        src, weight1, weight2, mean, rstd = ctx.saved_tensors
+        cols = src.size(-1)
+        rows = src.numel() // max(cols, 1)
+        code, pcode = ctx.codes
+        g1 = torch.zeros_like(src) if grad1 is None else grad1.contiguous()
+        g2 = torch.zeros_like(src) if grad2 is None else grad2.contiguous()
+        needs = ctx.needs_input_grad
+        pdtype = torch.float32 if pcode == _hp.F32 else src.dtype
+
+        def new(wanted):
+            return torch.empty(cols, dtype=pdtype, device=src.device) if wanted else None
+
+        dw1, db1 = new(weight1 is not None and needs[1]), new(ctx.has_bias[0] and needs[2])
+        dw2, db2 = new(weight2 is not None and needs[3]), new(ctx.has_bias[1] and needs[4])
+        dx = torch.empty_like(src)
+        ws = None
+        if any(t is not None for t in (dw1, db1, dw2, db2)):
+            nbytes = _hp.lib().nhp_layernorm_pair_bwd_workspace_bytes(rows, cols, code)
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=src.device) if nbytes else None
+        with _hp.device_guard(src):
+            rc = _hp.lib().nhp_layernorm_pair_bwd(dx.data_ptr(), _ptr(dw1), _ptr(db1), _ptr(dw2), _ptr(db2), g1.data_ptr(),
+                                                  g2.data_ptr(), src.data_ptr(), mean.data_ptr(), rstd.data_ptr(),
+                                                  _ptr(weight1), _ptr(weight2), _ptr(ws), rows, cols, code, pcode,
+                                                  _hp.stream_of(src))
+        _hp.check(rc, what)
+        if rows == 0:
+            for t in (dw1, db1, dw2, db2):
+                if t is not None:
+                    t.zero_()
+        return dx, dw1, db1, dw2, db2, None
+
+
+def layer_norm_pair(x, norm_a, norm_b):
+    """``(norm_a(x), norm_b(x))`` for two ``LayerNorm`` modules of this file applied to the same input, in one
+    kernel each way when their settings allow it (same epsilon, rows of at most 16 KiB), otherwise as two
+    separate calls. The parallel-residual transformer layer does this with its input and post-attention
+    norms (megatron/model/transformer.py:1195-1213)."""
+    same = (isinstance(norm_a, LayerNorm) and isinstance(norm_b, LayerNorm) and norm_a.eps == norm_b.eps
+            and norm_a.normalized_shape == norm_b.normalized_shape and x.size(-1) == norm_a.normalized_shape[0]
+            and x.size(-1) * x.element_size() <= 16384)
+    if not same:
+        return norm_a(x), norm_b(x)
+    return _LayerNormPairFunction.apply(x, norm_a.weight, norm_a.bias, norm_b.weight, norm_b.bias, norm_a.eps)
+
+
 class LayerNorm(torch.nn.Module):
     """``torch.nn.LayerNorm`` over the last dimension (what ``get_norm`` returns for ``norm: layernorm``)."""
 

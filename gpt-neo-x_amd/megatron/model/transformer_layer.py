@@ -6,7 +6,7 @@ model-parallel layers: every linear layer is a plain ``torch.nn.functional.linea
 GEMM) that hands its bias on instead of adding it (``skip_bias_add``), and everything between
 the GEMMs is one of the fused kernels:
 
-    norm                      nhp_layernorm / nhp_rmsnorm
+    norm                      nhp_layernorm / nhp_rmsnorm (the two norms of the parallel-residual layout: nhp_layernorm_pair)
     qkv projection            GEMM (bias added by the GEMM, as ColumnParallelLinear does for qkv)
     rotary on q and k         nhp_rope_cached_qk on the two views of the projection output; its backward writes
                               into the gradient of the projection output (no concatenation)
@@ -27,7 +27,7 @@ import torch.nn.functional as F
 from .activations import Gated_Activation, get_activation
 from .attention_core import CoreAttention, apply_rotary_to_query_key, get_fusion_type, split_qkv_and_rotate
 from .fused_bias_dropout import bias_dropout_add_fused_inference, bias_dropout_add_fused_train, get_bias_dropout_add
-from .norms import get_norm
+from .norms import get_norm, layer_norm_pair
 from .positional_embeddings import AliBi, RotaryEmbedding
 
 
@@ -164,7 +164,7 @@ class TransformerLayer(torch.nn.Module):
             if self.gpt_j_tied:
                 x1 = x2 = self.input_layernorm(x)
             else:
-                x1, x2 = self.input_layernorm(x), self.post_attention_layernorm(x)
+                x1, x2 = layer_norm_pair(x, self.input_layernorm, self.post_attention_layernorm)
             attention_output, attention_bias = self.attention(x1, attention_mask)
             if attention_bias is not None:
                 attention_output = bias_dropout_fn(attention_output, bias=attention_bias, residual=None,

@@ -476,6 +476,27 @@ int nhp_layernorm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, const
                       int64_t rows, int64_t cols, int dtype, int param_dtype, void* stream);
 
 /*
+ * Two LayerNorms of one input in one pass each way: y1 = xhat * gamma1 + beta1, y2 = xhat * gamma2 + beta2
+ * with shared mean / rstd, and in the backward one dx for both,
+ *   g = dy1 * gamma1 + dy2 * gamma2,  dx = rstd * (g - (sum(g) + xhat * sum(g * xhat)) / cols)
+ * (fp32, one rounding; autograd would round the two dx and add them), beside the parameter gradients of
+ * both norms. The parallel-residual layer applies input_layernorm and post_attention_layernorm to the
+ * same x (megatron/model/transformer.py:1195-1213, ParallelTransformerLayer.forward with gpt_j_residual).
+ * `workspace`: nhp_layernorm_pair_bwd_workspace_bytes() bytes when any parameter gradient is wanted.
+ * Rows of more than 16 KiB are accepted but run slower than two single calls would.
+ */
+int nhp_layernorm_pair_fwd(void* y1, void* y2, float* mean, float* rstd, const void* x,
+                           const void* gamma1, const void* beta1, const void* gamma2,
+                           const void* beta2, float eps, int64_t rows, int64_t cols, int dtype,
+                           int param_dtype, void* stream);
+int nhp_layernorm_pair_bwd(void* dx, void* dgamma1, void* dbeta1, void* dgamma2, void* dbeta2,
+                           const void* dy1, const void* dy2, const void* x, const float* mean,
+                           const float* rstd, const void* gamma1, const void* gamma2,
+                           void* workspace, int64_t rows, int64_t cols, int dtype, int param_dtype,
+                           void* stream);
+int64_t nhp_layernorm_pair_bwd_workspace_bytes(int64_t rows, int64_t cols, int dtype);
+
+/*
  * y = scale * (x * inv) + offset with
  *   eps_mode 1: inv = 1 / (||x||_2 * cols^(-1/2) + eps), the Python class
  *               RMSNorm.forward, megatron/model/norms.py:54-107 (p disabled);

@@ -66,6 +66,7 @@ def lib():
         L.oracle_gated_act_bwd.argtypes = [vp, vp, vp, vp, i64, i64, ci, ci]
         L.oracle_layernorm_fwd.argtypes = [vp, vp, vp, vp, vp, vp, f32, i64, i64, ci, ci]
         L.oracle_layernorm_bwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, ci, ci]
+        L.oracle_layernorm_pair_dx.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, ci, ci]
         L.oracle_rmsnorm_fwd.argtypes = [vp, vp, vp, vp, vp, f32, ci, i64, i64, i64, ci, ci]
         L.oracle_rmsnorm_bwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, f32, ci, i64, i64, i64, ci, ci]
         p64 = ctypes.POINTER(i64)
@@ -454,3 +455,30 @@ def masked_softmax_dropout_bwd(dy, y, scale, p, seed, offset=0):
     the storage type, then the (unmasked) softmax backward."""
     dy, y = _cpu_contig(dy), _cpu_contig(y)
     return softmax_bwd(_dropout_of_stored(dy, p, seed, offset), y, scale, False)
+
+
+def layernorm_pair_fwd(x, gamma1, beta1, gamma2, beta2, eps=1e-5):
+    """Two LayerNorms of one input: (y1, y2, mean, rstd), the statistics shared."""
+    y1, mean, rstd = layernorm_fwd(x, gamma1, beta1, eps)
+    y2, _, _ = layernorm_fwd(x, gamma2, beta2, eps)
+    return y1, y2, mean, rstd
+
+
+def layernorm_pair_bwd(dy1, dy2, x, mean, rstd, gamma1, gamma2):
+    """(dx, dgamma1, dbeta1, dgamma2, dbeta2): dx from g = dy1 * gamma1 + dy2 * gamma2 with one rounding, the
+    parameter gradients of the two single LayerNorms."""
+    x, dy1, dy2 = _cpu_contig(x), _cpu_contig(dy1), _cpu_contig(dy2)
+    rows, cols = _rows_cols(x)
+    gamma1, g1p, _ = _param(gamma1, x)
+    gamma2, g2p, _ = _param(gamma2, x)
+    pdt = gamma1.dtype if gamma1 is not None else (gamma2.dtype if gamma2 is not None else x.dtype)
+    if gamma1 is not None and gamma2 is not None:
+        assert gamma1.dtype == gamma2.dtype
+    mean, rstd = _cpu_contig(mean.float()), _cpu_contig(rstd.float())
+    dx = torch.empty_like(x)
+    _check(lib().oracle_layernorm_pair_dx(dx.data_ptr(), dy1.data_ptr(), dy2.data_ptr(), x.data_ptr(), mean.data_ptr(),
+                                          rstd.data_ptr(), g1p, g2p, rows, cols, _DT[x.dtype], _DT[pdt]),
+           "layernorm_pair_dx")
+    _, dg1, db1 = layernorm_bwd(dy1, x, mean, rstd, gamma1, param_dtype=pdt)
+    _, dg2, db2 = layernorm_bwd(dy2, x, mean, rstd, gamma2, param_dtype=pdt)
+    return dx, dg1, db1, dg2, db2

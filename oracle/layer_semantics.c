@@ -180,6 +180,10 @@ int oracle_layernorm_fwd(void* y, float* mean, float* rstd, const void* x, const
  * fp32 throughout, outputs rounded once (dgamma, dbeta to pdt). Any of dx,
  * dgamma, dbeta may be NULL.
  */
+static int layernorm_dx(void* dx, const void* dy, const void* dy2, const void* x, const float* mean,
+                        const float* rstd, const void* gamma, const void* gamma2, int64_t rows, int64_t cols, int dt,
+                        int pdt);
+
 int oracle_layernorm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, const void* x, const float* mean,
                          const float* rstd, const void* gamma, int64_t rows, int64_t cols, int dt, int pdt)
 {
@@ -496,4 +500,50 @@ int oracle_bias_dropout_add(void* out, const void* x, const void* bias, const vo
         }
     free(keep);
     return 0;
+}
+
+/*
+ * Two LayerNorms of one input (the parallel-residual layer applies input_layernorm and
+ * post_attention_layernorm to the same x, megatron/model/transformer.py:1195-1213): the statistics are shared,
+ * and since the backward is linear in g the gradient with respect to x is the single formula above with
+ *   g = dy1 * gamma1 + dy2 * gamma2
+ * evaluated in fp32 and rounded once (autograd would round each dx and add them: up to 1.5 ulp more).
+ * The parameter gradients are those of the two single calls.
+ */
+static int layernorm_dx(void* dx, const void* dy, const void* dy2, const void* x, const float* mean,
+                        const float* rstd, const void* gamma, const void* gamma2, int64_t rows, int64_t cols, int dt,
+                        int pdt)
+{
+    const size_t n = (size_t)(cols > 0 ? cols : 1);
+    float* g = (float*)malloc(sizeof(float) * n);
+    float* gx = (float*)malloc(sizeof(float) * n);
+    if (!g || !gx) {
+        free(g);
+        free(gx);
+        return -2;
+    }
+    for (int64_t r = 0; r < rows; ++r) {
+        for (int64_t c = 0; c < cols; ++c) {
+            const float xh = (load_elem(x, r * cols + c, dt) - mean[r]) * rstd[r];
+            g[c] = load_elem(dy, r * cols + c, dt) * (gamma ? load_param(gamma, c, pdt) : 1.0f);
+            if (dy2) g[c] = g[c] + load_elem(dy2, r * cols + c, dt) * (gamma2 ? load_param(gamma2, c, pdt) : 1.0f);
+            gx[c] = g[c] * xh;
+        }
+        const float s1 = pairwise_sum(g, cols), s2 = pairwise_sum(gx, cols);
+        for (int64_t c = 0; c < cols; ++c) {
+            const float xh = (load_elem(x, r * cols + c, dt) - mean[r]) * rstd[r];
+            const float t = (s1 + xh * s2) / (float)cols;
+            store_elem(dx, r * cols + c, dt, rstd[r] * (g[c] - t));
+        }
+    }
+    free(g);
+    free(gx);
+    return 0;
+}
+
+int oracle_layernorm_pair_dx(void* dx, const void* dy1, const void* dy2, const void* x, const float* mean,
+                             const float* rstd, const void* gamma1, const void* gamma2, int64_t rows, int64_t cols,
+                             int dt, int pdt)
+{
+    return layernorm_dx(dx, dy1, dy2, x, mean, rstd, gamma1, gamma2, rows, cols, dt, pdt);
 }

@@ -167,6 +167,19 @@ def test_argument_validation_of_the_layer_entry_points(hotpath):
     assert lib.nhp_layernorm_fwd(null, null, null, null, null, null, 1e-5, 4, 0, BF16, BF16, None) == 0
     assert lib.nhp_layernorm_bwd(q, null, null, p, p, null, p, p, null, 4, 8, BF16, BF16, None) == -3   # mean missing
     assert lib.nhp_layernorm_bwd(q, p, null, p, p, p, p, p, null, 4, 8, BF16, BF16, None) == -3          # workspace missing
+    # two LayerNorms of one input
+    q2 = ctypes.c_void_p(0x3000)
+    assert lib.nhp_layernorm_pair_fwd(q, q2, null, null, p, p, p, p, p, 1e-5, 4, 8, 4, F32, None) == -1
+    assert lib.nhp_layernorm_pair_fwd(q, q2, null, null, p, p, p, p, p, 1e-5, 4, 8, BF16, F16, None) == -1
+    assert lib.nhp_layernorm_pair_fwd(q, q2, null, null, p, p, p, p, p, 1e-5, 4, -8, BF16, F32, None) == -2
+    assert lib.nhp_layernorm_pair_fwd(q, null, null, null, p, p, p, p, p, 1e-5, 4, 8, BF16, F32, None) == -3   # y2 missing
+    assert lib.nhp_layernorm_pair_fwd(q, q, null, null, p, p, p, p, p, 1e-5, 4, 8, BF16, F32, None) == -6      # y1 is y2
+    assert lib.nhp_layernorm_pair_fwd(null, null, null, null, null, null, null, null, null, 1e-5, 0, 8, BF16, BF16, None) == 0
+    assert lib.nhp_layernorm_pair_bwd(q, null, null, null, null, p, null, p, p, p, p, p, null, 4, 8, BF16, BF16, None) == -3
+    assert lib.nhp_layernorm_pair_bwd(q, null, null, p, null, p, p, p, p, p, p, p, null, 4, 8, BF16, BF16, None) == -3  # workspace
+    assert lib.nhp_layernorm_pair_bwd(q, null, null, null, null, p, p, p, p, p, p, p, null, 4, 8, 7, BF16, None) == -1
+    assert lib.nhp_layernorm_pair_bwd_workspace_bytes(4096, 2048, BF16) == 2 * lib.nhp_norm_bwd_workspace_bytes(4096, 2048, BF16)
+    assert lib.nhp_layernorm_pair_bwd_workspace_bytes(4096, 2048, 9) == 0
     assert lib.nhp_rmsnorm_fwd(q, null, p, p, null, 1e-5, 3, 4, 8, BF16, BF16, None) == -2               # eps_mode
     assert lib.nhp_rmsnorm_partial_fwd(q, null, p, p, null, 1e-5, 1, 4, 8, 0, BF16, BF16, None) == -2    # no statistic columns
     assert lib.nhp_rmsnorm_partial_fwd(q, null, p, p, null, 1e-5, 1, 4, 8, 9, BF16, BF16, None) == -2    # more than the row has

@@ -136,6 +136,104 @@ def test_layernorm_vs_oracle(hotpath, shape, dtype, pd):
     util.assert_close_ulp_or_noise(db, want_db, 2, dy.float().abs().sum(0) * 32 * util.EPS32, "dbeta")
 
 
+def abi_layernorm_pair(hp, x, dy1, dy2, gamma1, beta1, gamma2, beta2, eps, want=(True, True, True, True)):
+    rows, cols = x.shape
+    code, pcode = hp.dtype_code(x, "t"), hp._DTYPE[gamma1.dtype]
+    y1, y2 = torch.empty_like(x), torch.empty_like(x)
+    mean = torch.empty(rows, dtype=torch.float32, device=x.device)
+    rstd = torch.empty_like(mean)
+    L = hp.lib()
+    rc = L.nhp_layernorm_pair_fwd(y1.data_ptr(), y2.data_ptr(), mean.data_ptr(), rstd.data_ptr(), x.data_ptr(), ptr(gamma1),
+                                  ptr(beta1), ptr(gamma2), ptr(beta2), eps, rows, cols, code, pcode, None)
+    assert rc == 0, L.nhp_status_string(rc)
+    dx = torch.empty_like(x)
+    grads = [torch.full((cols,), float("nan"), dtype=gamma1.dtype, device=x.device) if w else None for w in want]
+    ws = torch.empty(max(L.nhp_layernorm_pair_bwd_workspace_bytes(rows, cols, code), 1), dtype=torch.uint8, device=x.device)
+    rc = L.nhp_layernorm_pair_bwd(dx.data_ptr(), ptr(grads[0]), ptr(grads[1]), ptr(grads[2]), ptr(grads[3]), dy1.data_ptr(),
+                                  dy2.data_ptr(), x.data_ptr(), mean.data_ptr(), rstd.data_ptr(), ptr(gamma1), ptr(gamma2),
+                                  ws.data_ptr(), rows, cols, code, pcode, None)
+    assert rc == 0, L.nhp_status_string(rc)
+    return y1, y2, mean, rstd, dx, grads
+
+
+@pytest.mark.parametrize("pd", ["same", "fp32"])
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: f"{s[0]}x{s[1]}")
+def test_layernorm_pair_vs_oracle(hotpath, shape, dtype, pd):
+    rows, cols = shape
+    if pd == "fp32" and dtype == torch.float32:
+        pytest.skip("same case")
+    pdtype = dtype if pd == "same" else torch.float32
+    print(f"layernorm pair case {shape} {dtype} params {pdtype}", flush=True)
+    x, dy1, gamma1, beta1 = make(dtype, rows, cols, rows + cols, pdtype)
+    _, dy2, gamma2, beta2 = make(dtype, rows, cols, rows + cols + 1, pdtype)
+    eps = 1e-5
+    dev = [t.to(DEV) for t in (x, dy1, dy2, gamma1, beta1, gamma2, beta2)]
+    y1, y2, mean, rstd, dx, grads = abi_layernorm_pair(hotpath, *dev, eps)
+    # the statistics and outputs of two single launches (whose sums over a row may be formed in another order)
+    s1 = abi_layernorm(hotpath, dev[0], dev[1], dev[3], dev[4], eps)
+    s2 = abi_layernorm(hotpath, dev[0], dev[2], dev[5], dev[6], eps)
+    util.assert_close_ulp_or_noise(y1.cpu(), s1[0].cpu(), 1, out_noise(gamma1, x), "y1 vs single")
+    util.assert_close_ulp_or_noise(y2.cpu(), s2[0].cpu(), 1, out_noise(gamma2, x), "y2 vs single")
+    assert torch.allclose(mean, s1[1], rtol=0, atol=2e-6 * (1 + x.float().abs().max().item()))
+    assert torch.allclose(rstd, s1[2], rtol=1e-5, atol=0)
+    want_y1, want_y2, _, _ = oracle.layernorm_pair_fwd(x, gamma1, beta1, gamma2, beta2, eps)
+    util.assert_close_ulp_or_noise(y1.cpu(), want_y1, 2, out_noise(gamma1, x), "y1")
+    util.assert_close_ulp_or_noise(y2.cpu(), want_y2, 2, out_noise(gamma2, x), "y2")
+    mean, rstd = mean.cpu(), rstd.cpu()
+    want = oracle.layernorm_pair_bwd(dy1, dy2, x, mean, rstd, gamma1, gamma2)
+    noise = dx_noise(dy1, gamma1, rstd) + dx_noise(dy2, gamma2, rstd)
+    util.assert_close_ulp_or_noise(dx.cpu(), want[0], 2, noise, "dx")
+    xhat = ((x.float() - mean[:, None]) * rstd[:, None]).abs()
+    for i, dy in ((0, dy1), (2, dy2)):
+        util.assert_close_ulp_or_noise(grads[i].cpu(), want[1 + i], 2, (dy.float().abs() * xhat).sum(0) * 32 * util.EPS32,
+                                       f"dgamma{i // 2 + 1}")
+        util.assert_close_ulp_or_noise(grads[i + 1].cpu(), want[2 + i], 2, dy.float().abs().sum(0) * 32 * util.EPS32,
+                                       f"dbeta{i // 2 + 1}")
+    # and a second run reproduces every result (fixed summation order)
+    again = abi_layernorm_pair(hotpath, *dev, eps)
+    assert torch.equal(again[4], dx) and all(torch.equal(a, b) for a, b in zip(again[5], grads))
+
+
+def test_layernorm_pair_optional_gradients_and_module(hotpath):
+    from megatron.model.norms import LayerNorm, layer_norm_pair
+    x, dy1, gamma1, beta1 = [t.to(DEV) for t in make(torch.bfloat16, 67, 2048, 5, torch.float32)]
+    _, dy2, gamma2, beta2 = [t.to(DEV) for t in make(torch.bfloat16, 67, 2048, 6, torch.float32)]
+    full = abi_layernorm_pair(hotpath, x, dy1, dy2, gamma1, beta1, gamma2, beta2, 1e-5)
+    for want in ((False, False, False, False), (True, False, False, True), (False, True, True, False)):
+        part = abi_layernorm_pair(hotpath, x, dy1, dy2, gamma1, beta1, gamma2, beta2, 1e-5, want=want)
+        assert torch.equal(part[4], full[4])
+        for got, ref, w in zip(part[5], full[5], want):
+            assert (got is None) if not w else torch.equal(got, ref)
+    # the module-level helper against two separate modules, gradients through autograd
+    torch.manual_seed(3)
+    a, b = LayerNorm(2048, eps=1e-5).to(DEV), LayerNorm(2048, eps=1e-5).to(DEV)
+    with torch.no_grad():
+        a.weight.copy_(gamma1), a.bias.copy_(beta1), b.weight.copy_(gamma2), b.bias.copy_(beta2)
+    xa = x.view(1, 67, 2048).clone().requires_grad_(True)
+    y1, y2 = layer_norm_pair(xa, a, b)
+    (y1 * dy1.view_as(y1)).sum().backward(retain_graph=True)
+    only_first = xa.grad.clone()          # the second output unused so far: its gradient arrives as None / zeros
+    xa.grad = None
+    a.zero_grad(), b.zero_grad()
+    ((y1 * dy1.view_as(y1)).sum() + (y2 * dy2.view_as(y2)).sum()).backward()
+    pair_grads = [xa.grad.clone(), a.weight.grad.clone(), a.bias.grad.clone(), b.weight.grad.clone(), b.bias.grad.clone()]
+    assert torch.equal(pair_grads[0].view(67, 2048), full[4])
+    for got, ref in zip(pair_grads[1:], full[5]):
+        assert torch.equal(got, ref)
+    xb = x.view(1, 67, 2048).clone().requires_grad_(True)
+    a.zero_grad(), b.zero_grad()
+    z1, z2 = a(xb), b(xb)
+    assert util.ulp_distance(z1.cpu(), y1.cpu()).max() <= 1 and util.ulp_distance(z2.cpu(), y2.cpu()).max() <= 1
+    (z1 * dy1.view_as(z1)).sum().backward()
+    # (kernel-level parity is the test above; here only that the unused second output contributed nothing)
+    assert (xb.grad.float() - only_first.float()).abs().max() <= 2 ** -7 * only_first.float().abs().max()
+    # different settings fall back to two calls
+    c = LayerNorm(2048, eps=1e-6).to(DEV)
+    w1, w2 = layer_norm_pair(xb.detach(), a, c)
+    assert torch.equal(w1, a(xb.detach())) and torch.equal(w2, c(xb.detach()))
+
+
 @pytest.mark.parametrize("mode", [0, 1])
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
 @pytest.mark.parametrize("shape", [(5, 8), (70, 128), (129, 2048), (21, 4096), (19, 8192), (3, 32768), (11, 1000)],

@@ -219,6 +219,52 @@ def test_layernorm_backward_is_the_adjoint(dtype, pd):
     assert (dx32 * xhat).sum(-1).abs().max() < 1e-3
 
 
+@pytest.mark.parametrize("pd", ["same", "fp32"])
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_layernorm_pair_is_the_sum_of_two_layernorms(dtype, pd):
+    """Two LayerNorms of one input: outputs are the two single outputs, dx is the gradient of
+    y1.dy1 + y2.dy2 (float64 autograd through torch's layer_norm), rounded once."""
+    pdtype = dtype if pd == "same" else torch.float32
+    x, gamma1, beta1, dy1 = norm_inputs(dtype, seed=21, pdtype=pdtype)
+    _, gamma2, beta2, dy2 = norm_inputs(dtype, seed=22, pdtype=pdtype)
+    eps = 1e-5
+    y1, y2, mean, rstd = oracle.layernorm_pair_fwd(x, gamma1, beta1, gamma2, beta2, eps)
+    s1, m1, r1 = oracle.layernorm_fwd(x, gamma1, beta1, eps)
+    s2, _, _ = oracle.layernorm_fwd(x, gamma2, beta2, eps)
+    assert torch.equal(y1, s1) and torch.equal(y2, s2) and torch.equal(mean, m1) and torch.equal(rstd, r1)
+    dx, dg1, db1, dg2, db2 = oracle.layernorm_pair_bwd(dy1, dy2, x, mean, rstd, gamma1, gamma2)
+    xd = x.double().requires_grad_(True)
+    params = [t.double().requires_grad_(True) for t in (gamma1, beta1, gamma2, beta2)]
+    n = (x.size(-1),)
+    loss = (F.layer_norm(xd, n, params[0], params[1], eps) * dy1.double()).sum() + \
+           (F.layer_norm(xd, n, params[2], params[3], eps) * dy2.double()).sum()
+    loss.backward()
+    scale = ((dy1.float().abs() * gamma1.float().abs() + dy2.float().abs() * gamma2.float().abs()).sum(-1, keepdim=True)
+             * rstd[:, None] * 128 * util.EPS32)
+    util.assert_close_ulp_or_noise(dx, xd.grad.to(dtype), 1, scale.expand_as(dx.float()), "dx vs float64 autograd")
+    # parameter gradients are those of the single norms, bit for bit
+    _, w1, c1 = oracle.layernorm_bwd(dy1, x, mean, rstd, gamma1)
+    _, w2, c2 = oracle.layernorm_bwd(dy2, x, mean, rstd, gamma2)
+    assert torch.equal(dg1, w1) and torch.equal(db1, c1) and torch.equal(dg2, w2) and torch.equal(db2, c2)
+    for got, want in zip((dg1, db1, dg2, db2), params):
+        col = (dy1.float().abs() + dy2.float().abs()).sum(0) * 512 * util.EPS32
+        util.assert_close_ulp_or_noise(got, want.grad.to(pdtype), 1, col, "parameter gradient vs float64")
+    # a zero second gradient reduces it to the single backward, bit for bit; and swapping the two norms changes nothing
+    zero = torch.zeros_like(dy2)
+    single, _, _ = oracle.layernorm_bwd(dy1, x, mean, rstd, gamma1)
+    assert torch.equal(oracle.layernorm_pair_bwd(dy1, zero, x, mean, rstd, gamma1, gamma2)[0], single)
+    swapped = oracle.layernorm_pair_bwd(dy2, dy1, x, mean, rstd, gamma2, gamma1)[0]
+    util.assert_close_ulp_or_noise(swapped, dx, 1, scale.expand_as(dx.float()), "order of the two norms")
+    # one rounding: in fp32 the pair's dx equals the sum of the two single dx up to fp32 noise, and for 16-bit data it
+    # is at least as close to the float64 gradient as the rounded sum of two rounded gradients
+    d1, _, _ = oracle.layernorm_bwd(dy1, x, mean, rstd, gamma1)
+    d2, _, _ = oracle.layernorm_bwd(dy2, x, mean, rstd, gamma2)
+    two_step = (d1 + d2)
+    err_pair = (dx.double() - xd.grad).abs().mean()
+    err_two = (two_step.double() - xd.grad).abs().mean()
+    assert err_pair <= err_two * 1.001 + 1e-12
+
+
 @pytest.mark.parametrize("mode", [0, 1])
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
 def test_rmsnorm_forward(dtype, mode):
