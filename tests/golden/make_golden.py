@@ -121,6 +121,13 @@ def main():
         sdx, sds, _ = oracle.rmsnorm_bwd(dy, x, sinv, gvec, 1e-2, 2)
         put(name, part_y=py, part_inv=pinv, part_dx=pdx, part_dscale=pds, part_doffset=pdo, sn_y=sy, sn_inv=sinv,
             sn_dx=sdx, sn_dscale=sds)
+        # a second LayerNorm of the same input (the parallel-residual layer): one dx for both
+        gamma2 = (1 - 0.3 * torch.randn(24, generator=g)).to(dtype)
+        beta2 = (0.2 * torch.randn(24, generator=g)).to(dtype)
+        dy2 = util.randn((5, 24), dtype, seed + 2)
+        _, y2, _, _ = oracle.layernorm_pair_fwd(x, gamma, beta, gamma2, beta2, 1e-5)
+        pair_dx, _, _, pdg2, pdb2 = oracle.layernorm_pair_bwd(dy, dy2, x, mean, rstd, gamma, gamma2)
+        put(name, gamma2=gamma2, beta2=beta2, dy2=dy2, pair_y2=y2, pair_dx=pair_dx, pair_dgamma2=pdg2, pair_dbeta2=pdb2)
 
     for name, dtype, seed in (("gated_bf16", torch.bfloat16, 41), ("gated_fp16", torch.float16, 42),
                               ("gated_fp32", torch.float32, 43)):

@@ -78,6 +78,12 @@ def test_oracle_reproduces_norm_golden(name):
     assert same(sy, get(name, "sn_y")) and same(sinv, get(name, "sn_inv"))
     sdx, sds, _ = oracle.rmsnorm_bwd(dy, x, sinv, gvec, 1e-2, 2)
     assert same(sdx, get(name, "sn_dx")) and same(sds, get(name, "sn_dscale"))
+    gamma2, beta2, dy2 = (get(name, k) for k in ("gamma2", "beta2", "dy2"))
+    y1, y2, _, _ = oracle.layernorm_pair_fwd(x, gamma, beta, gamma2, beta2, 1e-5)
+    assert same(y1, get(name, "ln_y")) and same(y2, get(name, "pair_y2"))
+    pair = oracle.layernorm_pair_bwd(dy, dy2, x, mean, rstd, gamma, gamma2)
+    assert same(pair[0], get(name, "pair_dx")) and same(pair[1], get(name, "ln_dgamma")) and same(pair[2], get(name, "ln_dbeta"))
+    assert same(pair[3], get(name, "pair_dgamma2")) and same(pair[4], get(name, "pair_dbeta2"))
 
 
 GATED = ["gated_bf16", "gated_fp16", "gated_fp32"]
@@ -262,3 +268,26 @@ def test_gpu_matches_norm_golden(hotpath, name):
                              ws.data_ptr(), 1e-2, 2, rows, cols, code, code, None) == 0
     util.assert_close_ulp_or_noise(dx.cpu(), get(name, "sn_dx"), 2, dx_noise(gi.cpu()) * 2, name)
     util.assert_close_ulp_or_noise(dg.cpu(), get(name, "sn_dscale"), 2, col, name)
+
+    # two LayerNorms of one input
+    gamma2, beta2, dy2 = (get(name, k).cuda() for k in ("gamma2", "beta2", "dy2"))
+    y2 = torch.empty_like(x)
+    assert L.nhp_layernorm_pair_fwd(y.data_ptr(), y2.data_ptr(), mean.data_ptr(), rstd.data_ptr(), x.data_ptr(),
+                                    gamma.data_ptr(), beta.data_ptr(), gamma2.data_ptr(), beta2.data_ptr(), 1e-5, rows, cols,
+                                    code, code, None) == 0
+    util.assert_close_ulp_or_noise(y.cpu(), get(name, "ln_y"), 2, noise_y, name)
+    util.assert_close_ulp_or_noise(y2.cpu(), get(name, "pair_y2"), 2, (gamma2.float().abs().cpu() * 64 * util.EPS32).expand(rows, cols), name)
+    ws2 = torch.empty(max(L.nhp_layernorm_pair_bwd_workspace_bytes(rows, cols, code), 16), dtype=torch.uint8, device="cuda")
+    dg2, db2 = torch.empty_like(gamma), torch.empty_like(beta)
+    gm, gr = get(name, "ln_mean").cuda(), get(name, "ln_rstd").cuda()
+    assert L.nhp_layernorm_pair_bwd(dx.data_ptr(), dg.data_ptr(), db.data_ptr(), dg2.data_ptr(), db2.data_ptr(), dy.data_ptr(),
+                                    dy2.data_ptr(), x.data_ptr(), gm.data_ptr(), gr.data_ptr(), gamma.data_ptr(),
+                                    gamma2.data_ptr(), ws2.data_ptr(), rows, cols, code, code, None) == 0
+    both = ((dy.float().abs() * gamma.float().abs() + dy2.float().abs() * gamma2.float().abs()).sum(-1, keepdim=True).cpu()
+            * gr.cpu()[:, None] * 64 * util.EPS32).expand(rows, cols)
+    util.assert_close_ulp_or_noise(dx.cpu(), get(name, "pair_dx"), 2, both, name)
+    col2 = dy2.float().abs().sum(0).cpu() * 8 * 64 * util.EPS32
+    util.assert_close_ulp_or_noise(dg.cpu(), get(name, "ln_dgamma"), 2, col, name)
+    util.assert_close_ulp_or_noise(db.cpu(), get(name, "ln_dbeta"), 2, col, name)
+    util.assert_close_ulp_or_noise(dg2.cpu(), get(name, "pair_dgamma2"), 2, col2, name)
+    util.assert_close_ulp_or_noise(db2.cpu(), get(name, "pair_dbeta2"), 2, col2, name)
