@@ -1,6 +1,6 @@
 """Time one transformer layer (forward + backward) built from the fused kernels, on one GPU.
 
-    python gpt-neo-x_amd/layer_step.py [--config pythia-1.4b|llama2-7b] [--steps 20] [--warmup 5] [--dropout 0.0]
+    python gpt-neo-x_amd/layer_step.py [--config pythia-1.4b|llama2-7b|mistral-7b] [--steps 20] [--warmup 5] [--dropout 0.0]
 
 Prints one JSON line with the time per step. Under ``rocprofv3 --kernel-trace --stats`` the kernel table shows how
 the step divides between the library GEMMs and the kernels of libneox_hotpath.so (names starting with ``nhp::``).
@@ -23,6 +23,10 @@ CONFIGS = {
                         activation="gelu", rotary_pct=0.25, gpt_j_residual=True, use_bias=True, intermediate_size=None),
     "llama2-7b": dict(hidden_size=4096, num_attention_heads=32, seq_length=4096, batch=1, norm="rmsnorm",
                       activation="swiglu", rotary_pct=1.0, gpt_j_residual=False, use_bias=False, intermediate_size=11008 * 3),
+    # grouped-query attention (8 key/value heads for 32 query heads) and a sliding window of 4096 keys
+    "mistral-7b": dict(hidden_size=4096, num_attention_heads=32, num_kv_heads=8, seq_length=8192, batch=1, norm="rmsnorm",
+                       activation="swiglu", rotary_pct=1.0, gpt_j_residual=False, use_bias=False,
+                       intermediate_size=14336 * 3, sliding_window_width=4096),
 }
 
 
@@ -50,7 +54,7 @@ def main():
         attention_softmax_in_fp32=True, apply_query_key_layer_scaling=False, attention_dropout=a.dropout,
         hidden_dropout=a.dropout, bias_dropout_fusion=True, gpt_j_residual=c["gpt_j_residual"], gpt_j_tied=False,
         use_bias_in_mlp=c["use_bias"], use_bias_in_attn_linear=c["use_bias"], intermediate_size=c["intermediate_size"],
-        expansion_factor=None)
+        expansion_factor=None, num_kv_heads=c.get("num_kv_heads"), sliding_window_width=c.get("sliding_window_width"))
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
 

@@ -19,6 +19,13 @@ Everything between the two GEMMs that the reference runs as separate passes over
 the dropout (:592-593) -- is handed to ``FusedScaleMaskSoftmax`` and happens inside its
 kernel. Tensors are laid out as in the reference: q ``[sq, b, np, hn]``, k and v
 ``[sk, b, np, hn]``, result ``[b, np, sq, hn]``.
+
+Grouped-query attention (k and v with ``nkv < np`` heads): the reference repeats every k/v head
+``np / nkv`` times before the rotary embedding and the GEMMs (``gqa_project``,
+megatron/model/transformer.py:768-839). Here the heads are never repeated: the ``np / nkv`` query heads that
+share a k/v head are stacked along the row dimension of the GEMMs (``[b * nkv, (np / nkv) * sq, hn]``), which
+yields the same ``[b, np, sq, sk]`` scores, and the sum over the sharing heads in the gradients of k and v
+happens inside the GEMM instead of in a reduction pass.
 """
 import math
 
@@ -115,6 +122,8 @@ class CoreAttention(torch.nn.Module):
         projection, written by the context GEMM itself."""
         b, np_, sq, sk = query_layer.size(1), query_layer.size(2), query_layer.size(0), key_layer.size(0)
         hn = query_layer.size(3)
+        if key_layer.size(2) != np_:
+            return self._forward_grouped(query_layer, key_layer, value_layer, attention_mask, key_lengths, merged_heads)
         # [sq, b, np, hn] -> [sq, b * np, hn]
         q = query_layer.reshape(sq, b * np_, hn)
         k = key_layer.reshape(sk, b * np_, hn)
@@ -135,6 +144,33 @@ class CoreAttention(torch.nn.Module):
             return _ContextGemm.apply(probs.view(b * np_, sq, sk), v).view(sq, b, np_ * value_layer.size(3))
         context = torch.bmm(probs.view(b * np_, sq, sk), v.transpose(0, 1))
         return context.view(b, np_, sq, value_layer.size(3))
+
+    def _forward_grouped(self, query_layer, key_layer, value_layer, attention_mask, key_lengths, merged_heads):
+        """k and v ``[sk, b, nkv, hn]`` with ``nkv`` dividing ``np``: query head ``h`` attends with k/v head
+        ``h // (np / nkv)`` (the order ``torch.repeat_interleave(k, np / nkv, dim=2)`` produces)."""
+        sq, b, np_, hn = query_layer.shape
+        sk, nkv, hv = key_layer.size(0), key_layer.size(2), value_layer.size(3)
+        assert np_ % nkv == 0 and value_layer.size(2) == nkv, "query heads must be a multiple of the key/value heads"
+        group = np_ // nkv
+        # [sq, b, nkv, group, hn] -> [b * nkv, group * sq, hn]: no copy when q was written head-major
+        q = query_layer.view(sq, b, nkv, group, hn).permute(1, 2, 3, 0, 4).reshape(b * nkv, group * sq, hn)
+        k = key_layer.permute(1, 2, 0, 3).reshape(b * nkv, sk, hn)
+        v = value_layer.permute(1, 2, 0, 3).reshape(b * nkv, sk, hv)
+        if self.fold_scale:
+            scores = torch.bmm(q, k.transpose(1, 2))
+        else:
+            scores = torch.empty((b * nkv, group * sq, sk), dtype=q.dtype, device=q.device)
+            scores = torch.baddbmm(scores, q, k.transpose(1, 2), beta=0.0, alpha=self.gemm_alpha)
+        scores = scores.view(b, np_, sq, sk)
+        if self.use_cache and attention_mask is not None:
+            with torch.no_grad():
+                attention_mask = attention_mask[..., :sk, :sk]
+        bias = self.rpe(sq, sk) if self.rpe is not None else None
+        probs = self.scale_mask_softmax(scores, attention_mask, bias=bias, key_lengths=key_lengths)
+        context = torch.bmm(probs.view(b * nkv, group * sq, sk), v).view(b, np_, sq, hv)
+        if merged_heads:
+            return context.permute(2, 0, 1, 3).reshape(sq, b, np_ * hv)
+        return context
 
 
 def apply_rotary_to_query_key(query_layer, key_layer, rotary_emb, rotary_ndims=None, rope_fusion=True, bf16=False,
@@ -220,6 +256,69 @@ class _SplitRotaryQKV(torch.autograd.Function):
         else:
             gv.copy_(grad_v)
         return grad, None, None
+
+
+class _SplitRotaryGQA(torch.autograd.Function):
+    """``[sq, b, (np + 2 * nkv) * hn]`` (all query heads, then the key heads, then the value heads:
+    the layout of ``gqa_project``, megatron/model/transformer.py:774-794) -> rotated q ``[sq, b, np, hn]``,
+    rotated k ``[sq, b, nkv, hn]`` and v (a view). q and k are written head-major (storage ``[b, heads, sq, hn]``),
+    the layout in which the grouped GEMMs of ``CoreAttention`` take them without a copy. The backward writes the
+    three gradients into one buffer for the projection output."""
+
+    @staticmethod
+    def forward(ctx, mixed, cos, sin, np_, nkv):
+        import fused_rotary_positional_embedding as ext
+
+        sq, b, total = mixed.shape
+        hn = total // (np_ + 2 * nkv)
+        ctx.save_for_backward(cos, sin)
+        ctx.heads = (np_, nkv, hn)
+        q_in = mixed[..., :np_ * hn].view(sq, b, np_, hn)
+        k_in = mixed[..., np_ * hn:(np_ + nkv) * hn].view(sq, b, nkv, hn)
+        q_out = torch.empty((b, np_, sq, hn), dtype=mixed.dtype, device=mixed.device).permute(2, 0, 1, 3)
+        k_out = torch.empty((b, nkv, sq, hn), dtype=mixed.dtype, device=mixed.device).permute(2, 0, 1, 3)
+        ext.forward_cached_qk(q_in, k_in, cos, sin, False, out=(q_out, k_out))
+        return q_out, k_out, mixed[..., (np_ + nkv) * hn:].view(sq, b, nkv, hn)
+
+    @staticmethod
+    def backward(ctx, grad_q, grad_k, grad_v):
+        import fused_rotary_positional_embedding as ext
+
+        cos, sin = ctx.saved_tensors
+        np_, nkv, hn = ctx.heads
+        like = next(g for g in (grad_q, grad_k, grad_v) if g is not None)
+        sq, b = like.shape[:2]
+        grad = torch.empty((sq, b, (np_ + 2 * nkv) * hn), dtype=like.dtype, device=like.device)
+        gq = grad[..., :np_ * hn].view(sq, b, np_, hn)
+        gk = grad[..., np_ * hn:(np_ + nkv) * hn].view(sq, b, nkv, hn)
+        gv = grad[..., (np_ + nkv) * hn:].view(sq, b, nkv, hn)
+        if grad_q is not None and grad_k is not None:
+            ext.backward_cached_qk(grad_q, grad_k, cos, sin, False, out=(gq, gk))
+        else:
+            for dst, g in ((gq, grad_q), (gk, grad_k)):
+                if g is None:
+                    dst.zero_()
+                else:
+                    dst.copy_(ext.backward_cached(g, cos, sin, False))
+        if grad_v is None:
+            gv.zero_()
+        else:
+            gv.copy_(grad_v)
+        return grad, None, None, None, None
+
+
+def split_gqa_and_rotate(mixed_x_layer, rotary_emb, num_heads, num_kv_heads, layer_past=None):
+    """``split_qkv_and_rotate`` for grouped-query attention: ``mixed_x_layer`` is ``[sq, b, (np + 2 * nkv) * hn]``
+    as ``gqa_project`` lays it out (megatron/model/transformer.py:774-794); returns query ``[sq, b, np, hn]``,
+    key and value ``[sq, b, nkv, hn]`` -- the key/value heads are not repeated, ``CoreAttention`` groups the
+    query heads instead."""
+    seq_len = mixed_x_layer.shape[0]
+    offset = 0
+    if layer_past is not None and layer_past.numel() > 0:
+        offset = layer_past[0].shape[0]
+    cos, sin = rotary_emb(mixed_x_layer, seq_len=seq_len + offset)
+    rows = slice(offset, offset + seq_len)
+    return _SplitRotaryGQA.apply(mixed_x_layer, cos[rows], sin[rows], num_heads, num_kv_heads)
 
 
 def split_qkv_and_rotate(mixed_x_layer, rotary_emb, layer_past=None):

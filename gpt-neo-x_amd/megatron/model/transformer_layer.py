@@ -25,7 +25,8 @@ import torch
 import torch.nn.functional as F
 
 from .activations import Gated_Activation, get_activation
-from .attention_core import CoreAttention, apply_rotary_to_query_key, get_fusion_type, split_qkv_and_rotate
+from .attention_core import (CoreAttention, apply_rotary_to_query_key, get_fusion_type, split_gqa_and_rotate,
+                             split_qkv_and_rotate)
 from .fused_bias_dropout import bias_dropout_add_fused_inference, bias_dropout_add_fused_train, get_bias_dropout_add
 from .norms import get_norm, layer_norm_pair
 from .positional_embeddings import AliBi, RotaryEmbedding
@@ -88,7 +89,10 @@ class MLP(torch.nn.Module):
 
 class SelfAttention(torch.nn.Module):
     """``ParallelSelfAttention`` (megatron/model/transformer.py:326-959) with the unfused ("global") attention:
-    fused qkv projection, views split along the last dimension, rotary, CoreAttention, output projection."""
+    fused qkv projection, views split along the last dimension, rotary, CoreAttention, output projection.
+    With ``num_kv_heads`` below ``num_attention_heads`` (grouped-query attention, ``gqa_project``, :768-839)
+    the projection is ``[q heads | k heads | v heads]`` and the k/v heads are shared by groups of query heads
+    without being repeated."""
 
     def __init__(self, neox_args, attention_mask_func, layer_number, rpe=None, rotary=False):
         super().__init__()
@@ -98,7 +102,11 @@ class SelfAttention(torch.nn.Module):
         self.head_dim = neox_args.hidden_size // self.num_heads
         self.pos_emb = neox_args.pos_emb
         use_bias = getattr(neox_args, "use_bias_in_attn_linear", True)
-        self.query_key_value = Linear(neox_args.hidden_size, 3 * neox_args.hidden_size, bias=use_bias)
+        self.num_kv_heads = getattr(neox_args, "num_kv_heads", None) or self.num_heads
+        assert self.num_heads % self.num_kv_heads == 0, "num_kv_heads must divide num_attention_heads"
+        self.gqa = self.num_kv_heads != self.num_heads
+        self.query_key_value = Linear(neox_args.hidden_size, (self.num_heads + 2 * self.num_kv_heads) * self.head_dim,
+                                      bias=use_bias)
         slopes = AliBi(self.num_heads, 1, 0).slopes if self.pos_emb == "alibi" else None
         self.rotary_ndims = None
         self.rotary_emb = None
@@ -121,6 +129,8 @@ class SelfAttention(torch.nn.Module):
     def forward(self, hidden_states, attention_mask):
         sq, b = hidden_states.size(0), hidden_states.size(1)
         mixed, _ = self.query_key_value(hidden_states)
+        if self.gqa:
+            return self.dense(self.core(*self._gqa_project(mixed), attention_mask, merged_heads=True))
         # [sq, b, np * 3 * hn] -> [sq, b, np, 3 * hn] -> three views [sq, b, np, hn]
         mixed = mixed.view(sq, b, self.num_heads, 3 * self.head_dim)
         if self.rotary_emb is not None and self.rope_fusion:
@@ -133,6 +143,19 @@ class SelfAttention(torch.nn.Module):
         # [sq, b, np * hn], written in that layout by the context GEMM
         context = self.core(query, key, value, attention_mask, merged_heads=True)
         return self.dense(context)
+
+    def _gqa_project(self, mixed):
+        """``[sq, b, (np + 2 * nkv) * hn]`` -> q ``[sq, b, np, hn]``, k and v ``[sq, b, nkv, hn]``, q and k rotated."""
+        sq, b = mixed.shape[:2]
+        np_, nkv, hn = self.num_heads, self.num_kv_heads, self.head_dim
+        if self.rotary_emb is not None and self.rope_fusion:
+            return split_gqa_and_rotate(mixed, self.rotary_emb, np_, nkv)
+        query, key, value = torch.split(mixed, (np_ * hn, nkv * hn, nkv * hn), dim=-1)
+        query, key, value = query.view(sq, b, np_, hn), key.view(sq, b, nkv, hn), value.view(sq, b, nkv, hn)
+        if self.rotary_emb is not None:
+            query, key = apply_rotary_to_query_key(query, key, self.rotary_emb, rotary_ndims=self.rotary_ndims,
+                                                   rope_fusion=False, bf16=self.bf16)
+        return query, key, value
 
 
 class TransformerLayer(torch.nn.Module):

@@ -255,3 +255,85 @@ def test_merged_heads_output_equals_the_permuted_context():
     plain.backward(g)
     for a, e in ((qa, qb), (ka, kb), (va, vb)):
         assert torch.equal(util.raw_bits(a.grad), util.raw_bits(e.grad))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("merged", [False, True], ids=["bnsh", "merged"])
+def test_grouped_query_attention_equals_attention_with_repeated_heads(dtype, merged):
+    """k and v with fewer heads than q: the grouped GEMMs against what the reference does, repeat_interleave of
+    the k/v heads (gqa_project, megatron/model/transformer.py:820-837) followed by ordinary attention; textbook
+    fp32 attention on the repeated heads as the arbiter. The gradients of k and v are the sums over the query heads
+    that share them."""
+    from megatron.model.attention_core import CoreAttention
+    from megatron.model.fused_softmax import SoftmaxFusionTypes as T
+
+    sq, b, np_, nkv, hn = 256, 2, 8, 2, 64
+    lim = 2.0 ** (-7 if dtype == torch.bfloat16 else -9)
+    core = CoreAttention(hn, 1, dtype == torch.float16, dtype == torch.bfloat16, T.upper_triang, mask_func,
+                         attention_softmax_in_fp32=True)
+    mask = fb.causal_mask(sq, DEV)
+    q = util.randn((sq, b, np_, hn), dtype, seed=41).to(DEV).requires_grad_(True)
+    k = util.randn((sq, b, nkv, hn), dtype, seed=42).to(DEV).requires_grad_(True)
+    v = util.randn((sq, b, nkv, hn), dtype, seed=43).to(DEV).requires_grad_(True)
+    out = core(q, k, v, mask, merged_heads=merged)
+    shape = (sq, b, np_ * hn) if merged else (b, np_, sq, hn)
+    assert out.shape == shape and out.dtype == dtype
+    g = util.randn(shape, dtype, seed=44).to(DEV)
+    out.backward(g)
+
+    def repeated(t):
+        return torch.repeat_interleave(t, np_ // nkv, dim=2)
+
+    # the reference's way through the same module
+    q2, k2, v2 = (t.detach().clone().requires_grad_(True) for t in (q, k, v))
+    out2 = core(q2, repeated(k2), repeated(v2), mask, merged_heads=merged)
+    out2.backward(g)
+    # textbook fp32
+    q3, k3, v3 = (t.detach().clone().requires_grad_(True) for t in (q, k, v))
+    ref = textbook(q3, repeated(k3), repeated(v3), mask)
+    if merged:
+        ref = ref.permute(2, 0, 1, 3).reshape(shape)
+    ref.backward(g.float())
+    assert rel_err(out, ref) <= lim and rel_err(out2, ref) <= lim
+    for got, same, want in ((q.grad, q2.grad, q3.grad), (k.grad, k2.grad, k3.grad), (v.grad, v2.grad, v3.grad)):
+        assert got.shape == want.shape
+        assert rel_err(got, want) <= 2 * lim
+        # at least as close to the fp32 result as the repeat-and-reduce route
+        assert rel_err(got, want) <= 1.5 * rel_err(same, want) + 1e-6
+    # probabilities are identical whichever way the scores were formed up to the GEMM's own rounding
+    assert rel_err(out, out2) <= lim
+
+
+def test_split_gqa_and_rotate_matches_split_then_rotate():
+    """split_gqa_and_rotate against torch.split with the sizes of gqa_project followed by the rotary call site:
+    same q, k, v and the same gradient for the projection output; q and k come back head-major."""
+    from megatron.model.attention_core import apply_rotary_to_query_key, split_gqa_and_rotate
+    from megatron.model.positional_embeddings import RotaryEmbedding
+
+    dtype, sq, b, np_, nkv, hn = torch.bfloat16, 128, 2, 8, 2, 128
+    emb = RotaryEmbedding(hn, 256, base=10000, precision=dtype)
+    base = util.randn((sq, b, (np_ + 2 * nkv) * hn), dtype, seed=4).to(DEV)
+    ma = base.clone().requires_grad_(True)
+    mb = base.clone().requires_grad_(True)
+    qa, ka, va = split_gqa_and_rotate(ma, emb, np_, nkv)
+    assert qa.shape == (sq, b, np_, hn) and ka.shape == (sq, b, nkv, hn) and va.shape == (sq, b, nkv, hn)
+    assert qa.permute(1, 2, 0, 3).is_contiguous() and ka.permute(1, 2, 0, 3).is_contiguous()
+    q0, k0, v0 = torch.split(mb, (np_ * hn, nkv * hn, nkv * hn), dim=-1)
+    q0, k0, vb = q0.view(sq, b, np_, hn), k0.view(sq, b, nkv, hn), v0.view(sq, b, nkv, hn)
+    qb, kb = apply_rotary_to_query_key(q0, k0, emb, rope_fusion=True, one_launch=True)
+    for a, e in ((qa, qb), (ka, kb), (va, vb)):
+        assert a.shape == e.shape and torch.equal(util.raw_bits(a), util.raw_bits(e))
+    # gradients in the layouts the grouped GEMMs hand back: q head-major, k contiguous along the sequence
+    gq = util.randn((b, np_, sq, hn), dtype, seed=5).to(DEV).permute(2, 0, 1, 3)
+    gk = util.randn((b, nkv, hn, sq), dtype, seed=6).to(DEV).permute(3, 0, 1, 2)
+    gv = util.randn((b, nkv, sq, hn), dtype, seed=7).to(DEV).permute(2, 0, 1, 3)
+    torch.autograd.backward((qa, ka, va), (gq, gk, gv))
+    torch.autograd.backward((qb, kb, vb), (gq, gk, gv))
+    assert torch.equal(util.raw_bits(ma.grad), util.raw_bits(mb.grad))
+    # only the keys used
+    mc = base.clone().requires_grad_(True)
+    _, kc, _ = split_gqa_and_rotate(mc, emb, np_, nkv)
+    kc.backward(gk)
+    lo, hi = np_ * hn, (np_ + nkv) * hn
+    assert torch.equal(util.raw_bits(mc.grad[..., lo:hi]), util.raw_bits(ma.grad[..., lo:hi]))
+    assert mc.grad[..., :lo].abs().max().item() == 0 and mc.grad[..., hi:].abs().max().item() == 0

@@ -31,7 +31,7 @@ def args_for(**kw):
                 scaled_masked_softmax_fusion=False, attention_softmax_in_fp32=True, apply_query_key_layer_scaling=False,
                 attention_dropout=0.0, hidden_dropout=0.0, bias_dropout_fusion=True, gpt_j_residual=False,
                 gpt_j_tied=False, use_bias_in_mlp=True, use_bias_in_attn_linear=True, intermediate_size=None,
-                expansion_factor=None)
+                expansion_factor=None, num_kv_heads=None)
     base.update(kw)
     return types.SimpleNamespace(**base)
 
@@ -54,7 +54,13 @@ def reference_layer(layer, cfg, x, mask):
     def attention(t):
         sq, b = t.shape[:2]
         att = layer.attention
-        q, k, v = lin(att.query_key_value, t).view(sq, b, np_, 3 * hn).split(hn, dim=-1)
+        nkv = cfg.num_kv_heads or np_
+        if nkv == np_:
+            q, k, v = lin(att.query_key_value, t).view(sq, b, np_, 3 * hn).split(hn, dim=-1)
+        else:   # [q heads | k heads | v heads]; the k/v heads repeated for the query heads that share them
+            q, k, v = lin(att.query_key_value, t).split((np_ * hn, nkv * hn, nkv * hn), dim=-1)
+            q = q.view(sq, b, np_, hn)
+            k, v = (torch.repeat_interleave(u.view(sq, b, nkv, hn), np_ // nkv, dim=2) for u in (k, v))
         if att.rotary_emb is not None:
             nd = att.rotary_ndims or hn
             cos, sin = att.rotary_emb(t, seq_len=sq)
@@ -90,14 +96,17 @@ def rel_err(a, b):
     return ((a.float() - b.float()).norm() / b.float().norm()).item()
 
 
-@pytest.mark.parametrize("variant", ["pythia", "sequential", "llama"])
+@pytest.mark.parametrize("variant", ["pythia", "sequential", "llama", "gqa", "gqa-eager-rope"])
 def test_layer_matches_plain_torch(variant):
     from megatron.model.transformer_layer import TransformerLayer
 
     cfg = {"pythia": args_for(gpt_j_residual=True),
            "sequential": args_for(rotary_pct=1.0),
            "llama": args_for(norm="rmsnorm", activation="swiglu", rotary_pct=1.0, use_bias_in_mlp=False,
-                             use_bias_in_attn_linear=False)}[variant]
+                             use_bias_in_attn_linear=False),
+           "gqa": args_for(norm="rmsnorm", activation="swiglu", rotary_pct=1.0, use_bias_in_mlp=False,
+                           use_bias_in_attn_linear=False, num_kv_heads=2),
+           "gqa-eager-rope": args_for(num_kv_heads=4, rope_fusion=False)}[variant]
     torch.manual_seed(0)
     layer = TransformerLayer(cfg, mask_func, layer_number=3, rotary=True).to(DEV)
     with torch.no_grad():   # parameters away from their initial 1 / 0 so that every term matters
