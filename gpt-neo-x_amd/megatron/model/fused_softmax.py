@@ -208,7 +208,12 @@ class FusedScaleMaskSoftmax(nn.Module):
     def forward(self, input, mask, bias=None, key_lengths=None):
         assert input.dim() == 4  # [b, np, sq, sk]
         dropout = self.attention_dropout if self.training else 0.0
-        if self.is_kernel_available(mask, *input.size()):
+        if self.upper_triang_mask_fusion and input.size(2) != input.size(3):
+            # the last rows of a longer causal matrix (new positions after cached keys): the triangle the causal
+            # kernel implies does not apply, the caller's mask does. The reference asserts sq == sk here
+            # (fused_softmax.py:173) when its gate lets such a shape through.
+            probs = self._forward_rectangular(input, mask, bias, key_lengths)
+        elif self.is_kernel_available(mask, *input.size()):
             plain_causal = (self.upper_triang_mask_fusion and bias is None and key_lengths is None
                             and self.alibi_slopes is None)
             if dropout > 0.0 and plain_causal:
@@ -230,6 +235,17 @@ class FusedScaleMaskSoftmax(nn.Module):
         if dropout > 0.0:
             probs = torch.nn.functional.dropout(probs, p=dropout, training=True)
         return probs
+
+    def _forward_rectangular(self, input, mask, bias, key_lengths):
+        b, np, sq, sk = input.size()
+        general_ok = (self.input_in_float16 and mask is not None and sk > 16 and sq % 4 == 0 and (b * np) % 4 == 0
+                      and sq % self.get_batch_per_block(sq, sk, b, np) == 0 and self.alibi_slopes is None)
+        if not general_ok:
+            return self.forward_torch_softmax(input, mask, bias, key_lengths)
+        mask = self._mask_with_padding(mask, key_lengths, b, sk)
+        if bias is not None:
+            input = input + bias
+        return ScaledMaskedSoftmax.apply(input, mask, 1.0 if self.scale is None else self.scale)
 
     def is_kernel_available(self, mask, b, np, sq, sk):
         """The reference's conditions (fused_softmax.py:148-168) without ``sk <= 2048``."""

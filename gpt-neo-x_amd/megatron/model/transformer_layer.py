@@ -18,8 +18,9 @@ the GEMMs is one of the fused kernels:
 Both residual layouts of the reference are provided: the sequential one
 (``x = x + attn(ln1(x)); x = x + mlp(ln2(x))``, :1254-1318) and the parallel one of the
 GPT-J / Pythia configurations (``x = x + attn(ln1(x)) + mlp(ln2(x))``, :1195-1250).
-Left out: tensor / sequence / pipeline parallelism, mixture of experts, flash and sparse
-attention, key/value caching across calls, Transformer Engine layers.
+With ``use_cache`` a layer keeps the keys and values of the positions seen so far (``layer_past``) and the
+next call continues after them (inference, :916-935). Left out: tensor / sequence / pipeline parallelism,
+mixture of experts, flash and sparse attention, Transformer Engine layers.
 """
 import torch
 import torch.nn.functional as F
@@ -94,7 +95,7 @@ class SelfAttention(torch.nn.Module):
     the projection is ``[q heads | k heads | v heads]`` and the k/v heads are shared by groups of query heads
     without being repeated."""
 
-    def __init__(self, neox_args, attention_mask_func, layer_number, rpe=None, rotary=False):
+    def __init__(self, neox_args, attention_mask_func, layer_number, rpe=None, rotary=False, use_cache=False):
         super().__init__()
         self.fp16 = neox_args.precision == "fp16"
         self.bf16 = neox_args.precision == "bfloat16"
@@ -123,38 +124,51 @@ class SelfAttention(torch.nn.Module):
             attention_softmax_in_fp32=getattr(neox_args, "attention_softmax_in_fp32", False),
             apply_query_key_layer_scaling=getattr(neox_args, "apply_query_key_layer_scaling", False),
             use_mup=getattr(neox_args, "use_mup", False), attention_dropout=getattr(neox_args, "attention_dropout", 0.0),
-            sliding_window_width=getattr(neox_args, "sliding_window_width", None), alibi_slopes=slopes, rpe=rpe)
+            sliding_window_width=getattr(neox_args, "sliding_window_width", None), alibi_slopes=slopes, rpe=rpe,
+            use_cache=use_cache)
+        self.use_cache = use_cache
         self.dense = Linear(neox_args.hidden_size, neox_args.hidden_size, bias=use_bias, skip_bias_add=True)
 
-    def forward(self, hidden_states, attention_mask):
+    def forward(self, hidden_states, attention_mask, layer_past=None):
+        """Returns ``(output, bias)``; with ``use_cache`` the first item is ``[output, present]``, ``present`` the
+        stacked keys and values of all positions so far (megatron/model/transformer.py:916-958). ``layer_past``:
+        the ``present`` of the previous call; the rotary embedding then starts at the position after it and
+        ``attention_mask`` must hold the rows of the new positions over all keys."""
         sq, b = hidden_states.size(0), hidden_states.size(1)
         mixed, _ = self.query_key_value(hidden_states)
         if self.gqa:
-            return self.dense(self.core(*self._gqa_project(mixed), attention_mask, merged_heads=True))
-        # [sq, b, np * 3 * hn] -> [sq, b, np, 3 * hn] -> three views [sq, b, np, hn]
-        mixed = mixed.view(sq, b, self.num_heads, 3 * self.head_dim)
-        if self.rotary_emb is not None and self.rope_fusion:
-            query, key, value = split_qkv_and_rotate(mixed, self.rotary_emb)
+            query, key, value = self._gqa_project(mixed, layer_past)
         else:
-            query, key, value = torch.split(mixed, self.head_dim, dim=-1)
-            if self.rotary_emb is not None:
-                query, key = apply_rotary_to_query_key(query, key, self.rotary_emb, rotary_ndims=self.rotary_ndims,
-                                                       rope_fusion=False, bf16=self.bf16)
+            # [sq, b, np * 3 * hn] -> [sq, b, np, 3 * hn] -> three views [sq, b, np, hn]
+            mixed = mixed.view(sq, b, self.num_heads, 3 * self.head_dim)
+            if self.rotary_emb is not None and self.rope_fusion:
+                query, key, value = split_qkv_and_rotate(mixed, self.rotary_emb, layer_past=layer_past)
+            else:
+                query, key, value = torch.split(mixed, self.head_dim, dim=-1)
+                if self.rotary_emb is not None:
+                    query, key = apply_rotary_to_query_key(query, key, self.rotary_emb, rotary_ndims=self.rotary_ndims,
+                                                           rope_fusion=False, bf16=self.bf16, layer_past=layer_past)
+        if layer_past is not None and layer_past.numel() > 0:
+            past_key, past_value = layer_past
+            key = torch.cat((past_key.type_as(key), key), dim=0)
+            value = torch.cat((past_value.type_as(value), value), dim=0)
+        present = torch.stack((key, value)) if self.use_cache else None
         # [sq, b, np * hn], written in that layout by the context GEMM
         context = self.core(query, key, value, attention_mask, merged_heads=True)
-        return self.dense(context)
+        output, bias = self.dense(context)
+        return ([output, present] if self.use_cache else output), bias
 
-    def _gqa_project(self, mixed):
+    def _gqa_project(self, mixed, layer_past=None):
         """``[sq, b, (np + 2 * nkv) * hn]`` -> q ``[sq, b, np, hn]``, k and v ``[sq, b, nkv, hn]``, q and k rotated."""
         sq, b = mixed.shape[:2]
         np_, nkv, hn = self.num_heads, self.num_kv_heads, self.head_dim
         if self.rotary_emb is not None and self.rope_fusion:
-            return split_gqa_and_rotate(mixed, self.rotary_emb, np_, nkv)
+            return split_gqa_and_rotate(mixed, self.rotary_emb, np_, nkv, layer_past=layer_past)
         query, key, value = torch.split(mixed, (np_ * hn, nkv * hn, nkv * hn), dim=-1)
         query, key, value = query.view(sq, b, np_, hn), key.view(sq, b, nkv, hn), value.view(sq, b, nkv, hn)
         if self.rotary_emb is not None:
             query, key = apply_rotary_to_query_key(query, key, self.rotary_emb, rotary_ndims=self.rotary_ndims,
-                                                   rope_fusion=False, bf16=self.bf16)
+                                                   rope_fusion=False, bf16=self.bf16, layer_past=layer_past)
         return query, key, value
 
 
@@ -162,7 +176,7 @@ class TransformerLayer(torch.nn.Module):
     """``ParallelTransformerLayer.forward`` (megatron/model/transformer.py:1179-1321) on one GPU.
     Input and output ``[s, b, h]``."""
 
-    def __init__(self, neox_args, attention_mask_func, layer_number, rpe=None, rotary=False):
+    def __init__(self, neox_args, attention_mask_func, layer_number, rpe=None, rotary=False, use_cache=False):
         super().__init__()
         norm, eps = get_norm(neox_args)
         self.input_layernorm = norm(neox_args.hidden_size, eps=eps)
@@ -171,7 +185,10 @@ class TransformerLayer(torch.nn.Module):
         self.bias_dropout_fusion = getattr(neox_args, "bias_dropout_fusion", True)
         self.gpt_j_residual = getattr(neox_args, "gpt_j_residual", False)
         self.gpt_j_tied = getattr(neox_args, "gpt_j_tied", False)
-        self.attention = SelfAttention(neox_args, attention_mask_func, layer_number, rpe=rpe, rotary=rotary)
+        self.use_cache = use_cache
+        self.layer_past = None   # with use_cache: keys and values after the last call (transformer.py:1166, 1219-1225)
+        self.attention = SelfAttention(neox_args, attention_mask_func, layer_number, rpe=rpe, rotary=rotary,
+                                       use_cache=use_cache)
         self.mlp = MLP(neox_args)
 
     def _get_bias_dropout(self):
@@ -179,7 +196,14 @@ class TransformerLayer(torch.nn.Module):
             return bias_dropout_add_fused_train if self.training else bias_dropout_add_fused_inference
         return get_bias_dropout_add(self.training)
 
-    def forward(self, x, attention_mask):
+    def _attend(self, x, attention_mask, layer_past):
+        output, bias = self.attention(x, attention_mask, layer_past=layer_past)
+        if self.use_cache:
+            output, self.layer_past = output
+        return output, bias
+
+    def forward(self, x, attention_mask, layer_past=None):
+        layer_past = layer_past if layer_past is not None else self.layer_past
         bias_dropout_fn = self._get_bias_dropout()
         residual = x
         if self.gpt_j_residual:
@@ -188,7 +212,7 @@ class TransformerLayer(torch.nn.Module):
                 x1 = x2 = self.input_layernorm(x)
             else:
                 x1, x2 = layer_norm_pair(x, self.input_layernorm, self.post_attention_layernorm)
-            attention_output, attention_bias = self.attention(x1, attention_mask)
+            attention_output, attention_bias = self._attend(x1, attention_mask, layer_past)
             if attention_bias is not None:
                 attention_output = bias_dropout_fn(attention_output, bias=attention_bias, residual=None,
                                                    prob=self.hidden_dropout)
@@ -196,7 +220,7 @@ class TransformerLayer(torch.nn.Module):
             output = bias_dropout_fn(mlp_output, bias=mlp_bias, residual=attention_output, prob=self.hidden_dropout)
             return bias_dropout_add_fused_inference(output, None, residual, 0.0)  # residual + output
         # x = x + attn(ln1(x)); x = x + mlp(ln2(x))
-        attention_output, attention_bias = self.attention(self.input_layernorm(x), attention_mask)
+        attention_output, attention_bias = self._attend(self.input_layernorm(x), attention_mask, layer_past)
         attention_output = bias_dropout_fn(attention_output, bias=attention_bias, residual=residual,
                                            prob=self.hidden_dropout)
         mlp_output, mlp_bias = self.mlp(self.post_attention_layernorm(attention_output))

@@ -194,3 +194,37 @@ def test_layer_under_activation_checkpointing_reproduces_its_dropout_masks():
     assert torch.equal(out_a, out_b) and torch.equal(dx_a, dx_b)
     for n in grads_a:
         assert torch.equal(grads_a[n], grads_b[n]), n
+
+
+@pytest.mark.parametrize("variant", ["pythia", "gqa", "eager-rope"])
+def test_incremental_decoding_with_cached_keys_equals_the_full_pass(variant):
+    """use_cache (megatron/model/transformer.py:916-935, 1219-1225): feeding the sequence in pieces, each call
+    continuing after the cached keys and values, gives the hidden states of one pass over the whole sequence.
+    Pieces of 64 (masked kernel on a rectangular score matrix), 3 and 1 positions (torch branch of the softmax)."""
+    from megatron.model.transformer_layer import TransformerLayer
+
+    cfg = {"pythia": args_for(gpt_j_residual=True),
+           "gqa": args_for(norm="rmsnorm", activation="swiglu", rotary_pct=1.0, use_bias_in_mlp=False,
+                           use_bias_in_attn_linear=False, num_kv_heads=2),
+           "eager-rope": args_for(rope_fusion=False)}[variant]
+    torch.manual_seed(0)
+    layer = TransformerLayer(cfg, mask_func, layer_number=1, rotary=True, use_cache=True).to(DEV).to(torch.bfloat16).eval()
+    s, b, h = 136, 4, cfg.hidden_size
+    x = util.randn((s, b, h), torch.bfloat16, seed=1).to(DEV)
+    mask = fb.causal_mask(s, DEV)
+    nkv = cfg.num_kv_heads or cfg.num_attention_heads
+    with torch.no_grad():
+        full = layer(x, mask)
+        assert layer.layer_past.shape == (2, s, b, nkv, h // cfg.num_attention_heads)
+        layer.layer_past = None
+        pieces, start = [], 0
+        for n in (64, 64, 3, 1, 4):
+            rows = mask[..., start:start + n, :start + n]
+            pieces.append(layer(x[start:start + n], rows))
+            start += n
+            assert layer.layer_past.shape[1] == start
+        assert start == s
+    got = torch.cat(pieces, dim=0)
+    # the same arithmetic per position up to the order of the GEMMs' sums
+    assert rel_err(got, full) <= 2.0 ** -7
+    assert (got.float() - full.float()).abs().max() <= 2.0 ** -4 * full.float().abs().max()

@@ -355,3 +355,41 @@ def test_core_attention_scaling_and_torch_branch_on_cpu():
     cached = CoreAttention(hn, 1, False, False, T.none, mask_func, use_cache=True)
     big = fb.causal_mask(sq + 8, "cpu")
     assert torch.allclose(cached(q, k, v, big).double(), want, atol=1e-5)
+
+
+def test_grouped_query_attention_and_rectangular_scores_on_cpu():
+    """CoreAttention with fewer key/value heads than query heads (gqa_project, megatron/model/transformer.py:768-839)
+    in fp32 on the CPU against float64 attention over repeated heads, with gradients; and scores that are not
+    square (new positions after cached keys) under the causal fusion type, which take the caller's mask."""
+    from megatron.model.attention_core import CoreAttention
+    from megatron.model.fused_softmax import FusedScaleMaskSoftmax, SoftmaxFusionTypes as T
+
+    def mask_func(scores, mask):
+        return fb.fill_masked_with_dtype_min(scores, mask)
+
+    sq, b, np_, nkv, hn = 20, 2, 6, 2, 8
+    core = CoreAttention(hn, 1, False, False, T.none, mask_func)
+    q = util.randn((sq, b, np_, hn), torch.float32, seed=1).requires_grad_(True)
+    k = util.randn((sq, b, nkv, hn), torch.float32, seed=2).requires_grad_(True)
+    v = util.randn((sq, b, nkv, hn), torch.float32, seed=3).requires_grad_(True)
+    mask = fb.causal_mask(sq, "cpu")
+    g = util.randn((sq, b, np_ * hn), torch.float32, seed=4)
+    out = core(q, k, v, mask, merged_heads=True)
+    out.backward(g)
+    qd, kd, vd = (t.detach().double().requires_grad_(True) for t in (q, k, v))
+    kr, vr = (torch.repeat_interleave(t, np_ // nkv, dim=2) for t in (kd, vd))
+    scores = (qd.permute(1, 2, 0, 3) @ kr.permute(1, 2, 3, 0) / math.sqrt(hn)).masked_fill(mask, float("-inf"))
+    want = (torch.softmax(scores, -1) @ vr.permute(1, 2, 0, 3)).permute(2, 0, 1, 3).reshape(sq, b, np_ * hn)
+    want.backward(g.double())
+    assert torch.allclose(out.double(), want, atol=1e-5)
+    for got, ref in ((q.grad, qd.grad), (k.grad, kd.grad), (v.grad, vd.grad)):
+        assert got.shape == ref.shape and torch.allclose(got.double(), ref, atol=1e-5)
+    with pytest.raises(AssertionError):
+        core(q, k[:, :, :1].expand(sq, b, 4, hn), v, mask)   # 6 query heads over 4 key heads
+    # rows 12..19 of the 20 x 20 causal matrix
+    module = FusedScaleMaskSoftmax(False, False, T.upper_triang, mask_func, True, 0.5)
+    x = util.randn((b, np_, 8, sq), torch.float32, seed=5)
+    rows = mask[..., 12:, :]
+    got = module(x, rows)
+    ref = torch.softmax((x.double() * 0.5).masked_fill(rows, float("-inf")), -1)
+    assert torch.allclose(got.double(), ref, atol=1e-6)
