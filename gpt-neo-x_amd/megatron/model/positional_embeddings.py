@@ -176,3 +176,60 @@ class AliBi(torch.nn.Module):
     def forward(self, x):
         # x: [b, np, sq, sk]
         return x + self.bias(x.shape[-2], x.shape[-1], x.device, x.dtype)
+
+
+class RelativePositionBias(torch.nn.Module):
+    """T5 relative position bias: ``bias[0, h, q, k] = weight[bucket(k - q), h] * scale``
+    (``ParallelRelativePositionBias``, megatron/mpu/layers.py:215-381, for all heads on one GPU; built with
+    ``scale = sqrt(head_dim)`` by megatron/model/gpt2_model.py:228-240). ``forward(q_len, k_len)`` returns
+    ``[1, heads, q_len, k_len]``, the ``rpe`` argument of ``CoreAttention``, which hands it to the softmax kernel
+    as its bias operand.
+
+    Buckets (causal): distance ``n = max(q - k, 0)``; ``n`` itself below ``num_buckets / 2``, then logarithmic steps
+    up to ``max_distance``, the last bucket for everything beyond. Non-causal: half of the buckets per direction.
+    """
+
+    def __init__(self, scale, causal=True, num_buckets=32, max_distance=128, heads=8, init_method=None, neox_args=None):
+        super().__init__()
+        self.scale = scale
+        self.causal = causal
+        self.num_buckets = num_buckets
+        self.max_distance = max_distance
+        self.heads = heads
+        self.weight = torch.nn.Parameter(torch.empty(num_buckets, heads))
+        (init_method or torch.nn.init.xavier_normal_)(self.weight)
+        self._cached_lengths = None
+        self._cached_buckets = None
+
+    def relative_position_bucket(self, relative_position):
+        """Bucket index of ``relative_position = k - q`` (an integer tensor)."""
+        buckets = self.num_buckets
+        distance = -relative_position
+        base = torch.zeros_like(distance)
+        if self.causal:
+            distance = distance.clamp(min=0)
+        else:
+            buckets //= 2
+            base = (distance < 0).long() * buckets
+            distance = distance.abs()
+        exact = buckets // 2
+        # logarithmic part, in fp32 with the operation order of the reference (log of the ratio, divided by the
+        # log of the range, times the number of logarithmic buckets, truncated)
+        steps = torch.log(distance.float() / exact) / math.log(self.max_distance / exact) * (buckets - exact)
+        far = (exact + steps.long()).clamp(max=buckets - 1)
+        return base + torch.where(distance < exact, distance, far)
+
+    def buckets(self, q_len, k_len, device):
+        if self._cached_lengths != (q_len, k_len) or self._cached_buckets.device != torch.device(device):
+            q_pos = torch.arange(q_len, dtype=torch.long, device=device)
+            k_pos = torch.arange(k_len, dtype=torch.long, device=device)
+            self._cached_buckets = self.relative_position_bucket(k_pos[None, :] - q_pos[:, None])
+            self._cached_lengths = (q_len, k_len)
+        return self._cached_buckets
+
+    def forward(self, q_len, k_len):
+        values = torch.nn.functional.embedding(self.buckets(q_len, k_len, self.weight.device), self.weight)  # [q, k, h]
+        return values.movedim(2, 0).unsqueeze(0) * self.scale
+
+
+ParallelRelativePositionBias = RelativePositionBias

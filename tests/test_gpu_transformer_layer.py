@@ -73,7 +73,10 @@ def reference_layer(layer, cfg, x, mask):
 
             q, k = rot(q), rot(k)
         q, k, v = (u.permute(1, 2, 0, 3) for u in (q, k, v))
-        scores = (q @ k.transpose(-1, -2) / math.sqrt(hn)).masked_fill(mask, float("-inf"))
+        scores = q @ k.transpose(-1, -2) / math.sqrt(hn)
+        if att.core.rpe is not None:
+            scores = scores + att.core.rpe(sq, sq).float()
+        scores = scores.masked_fill(mask, float("-inf"))
         ctx = (torch.softmax(scores, -1) @ v).permute(2, 0, 1, 3).reshape(sq, b, h)
         return lin(att.dense, ctx)
 
@@ -96,7 +99,7 @@ def rel_err(a, b):
     return ((a.float() - b.float()).norm() / b.float().norm()).item()
 
 
-@pytest.mark.parametrize("variant", ["pythia", "sequential", "llama", "gqa", "gqa-eager-rope"])
+@pytest.mark.parametrize("variant", ["pythia", "sequential", "llama", "gqa", "gqa-eager-rope", "rpe"])
 def test_layer_matches_plain_torch(variant):
     from megatron.model.transformer_layer import TransformerLayer
 
@@ -106,9 +109,15 @@ def test_layer_matches_plain_torch(variant):
                              use_bias_in_attn_linear=False),
            "gqa": args_for(norm="rmsnorm", activation="swiglu", rotary_pct=1.0, use_bias_in_mlp=False,
                            use_bias_in_attn_linear=False, num_kv_heads=2),
-           "gqa-eager-rope": args_for(num_kv_heads=4, rope_fusion=False)}[variant]
+           "gqa-eager-rope": args_for(num_kv_heads=4, rope_fusion=False),
+           "rpe": args_for(pos_emb="rpe")}[variant]
     torch.manual_seed(0)
-    layer = TransformerLayer(cfg, mask_func, layer_number=3, rotary=True).to(DEV)
+    rpe = None
+    if variant == "rpe":   # T5 relative position bias shared by the layers, added inside the softmax kernel
+        from megatron.model.positional_embeddings import RelativePositionBias
+        rpe = RelativePositionBias(scale=math.sqrt(cfg.hidden_size // cfg.num_attention_heads), causal=True,
+                                   num_buckets=32, max_distance=128, heads=cfg.num_attention_heads)
+    layer = TransformerLayer(cfg, mask_func, layer_number=3, rpe=rpe, rotary=variant != "rpe").to(DEV)
     with torch.no_grad():   # parameters away from their initial 1 / 0 so that every term matters
         for name, p in layer.named_parameters():
             if p.dim() == 1:

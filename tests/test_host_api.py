@@ -393,3 +393,42 @@ def test_grouped_query_attention_and_rectangular_scores_on_cpu():
     got = module(x, rows)
     ref = torch.softmax((x.double() * 0.5).masked_fill(rows, float("-inf")), -1)
     assert torch.allclose(got.double(), ref, atol=1e-6)
+
+
+def test_relative_position_bias_buckets_and_values():
+    """RelativePositionBias (ParallelRelativePositionBias, megatron/mpu/layers.py:215-381): the T5 bucket function
+    pinned by its defining properties and by hand-computed boundaries, the bias by indexing the table directly."""
+    from megatron.model.positional_embeddings import ParallelRelativePositionBias, RelativePositionBias
+
+    assert ParallelRelativePositionBias is RelativePositionBias
+    torch.manual_seed(0)
+    rpe = RelativePositionBias(scale=8.0, causal=True, num_buckets=32, max_distance=128, heads=4)
+    assert rpe.weight.shape == (32, 4)
+    q_len = k_len = 300
+    b = rpe.buckets(q_len, k_len, "cpu")
+    assert b.shape == (q_len, k_len) and b.dtype == torch.long
+    q, k = torch.meshgrid(torch.arange(q_len), torch.arange(k_len), indexing="ij")
+    n = (q - k)
+    assert (b[n <= 0] == 0).all()                                   # the present and the future: bucket 0
+    assert torch.equal(b[(n > 0) & (n < 16)], n[(n > 0) & (n < 16)])  # one bucket per distance below num_buckets / 2
+    assert (b[n >= 128] == 31).all() and b.max() == 31                # everything from max_distance on: the last bucket
+    # Toeplitz and monotone in the distance
+    first_col = b[:, 0]
+    assert all(torch.equal(torch.diagonal(b, -d), first_col[d].expand(q_len - d)) for d in (1, 17, 64, 200))
+    assert (first_col[1:] >= first_col[:-1]).all()
+    # logarithmic part: bucket 16 + floor(log(n / 16) / log(8) * 16); boundaries by hand: 16 * 8^(j/16)
+    for n_val, want in ((16, 16), (18, 16), (19, 17), (22, 18), (32, 21), (45, 23), (46, 24), (64, 26), (91, 29), (127, 31)):
+        assert first_col[n_val].item() == want, (n_val, first_col[n_val].item(), want)
+    bias = rpe(q_len, k_len)
+    assert bias.shape == (1, 4, q_len, k_len)
+    for (h, qi, ki) in ((0, 5, 5), (1, 100, 3), (3, 299, 0), (2, 10, 200)):
+        assert bias[0, h, qi, ki].item() == pytest.approx(rpe.weight[b[qi, ki], h].item() * 8.0)
+    # non-causal: 16 buckets per direction
+    both = RelativePositionBias(scale=1.0, causal=False, num_buckets=32, max_distance=128, heads=2)
+    bb = both.buckets(200, 200, "cpu")
+    assert (bb[n[:200, :200] >= 0] < 16).all() and (bb[n[:200, :200] < 0] >= 16).all()
+    assert bb[0, 199].item() == 31 and bb[199, 0].item() == 15 and bb[7, 0].item() == 7 and bb[0, 7].item() == 16 + 7
+    # the gradient reaches the table
+    bias.sum().backward()
+    counts = torch.bincount(b.flatten(), minlength=32).float()
+    assert torch.allclose(rpe.weight.grad, (counts * 8.0)[:, None].expand(32, 4))
