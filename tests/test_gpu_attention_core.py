@@ -337,3 +337,73 @@ def test_split_gqa_and_rotate_matches_split_then_rotate():
     lo, hi = np_ * hn, (np_ + nkv) * hn
     assert torch.equal(util.raw_bits(mc.grad[..., lo:hi]), util.raw_bits(ma.grad[..., lo:hi]))
     assert mc.grad[..., :lo].abs().max().item() == 0 and mc.grad[..., hi:].abs().max().item() == 0
+
+
+@pytest.mark.parametrize("case", ["2048", "small-blocks-ragged", "fp16-alpha", "dropout", "alibi", "window", "window-dropout"])
+def test_blocked_causal_gemms_equal_the_dense_ones(case, monkeypatch):
+    """With the causal kernel the score, context and gradient GEMMs are computed on and below the diagonal blocks
+    only (nothing above is read, and the probabilities and their gradients are exact zeros there). Against the same
+    module with dense GEMMs, and against fp32 textbook attention; the uninitialised parts of the score tensor are
+    filled with NaN first to show that they are never used."""
+    from megatron.model import attention_core
+    from megatron.model.attention_core import CoreAttention
+    from megatron.model.fused_softmax import SoftmaxFusionTypes as T
+
+    dtype = torch.float16 if case == "fp16-alpha" else torch.bfloat16
+    sq, b, np_, hn = (2048, 1, 4, 64) if case == "2048" else (328, 2, 4, 64)
+    if case != "2048":
+        monkeypatch.setattr(attention_core, "causal_gemm_block", lambda s: 128)   # blocks of 128, 128 and 72 rows
+    real_empty = torch.empty
+
+    def poisoned_empty(*args, **kw):
+        t = real_empty(*args, **kw)
+        return t.fill_(float("nan")) if t.is_floating_point() else t
+
+    kw = dict(attention_softmax_in_fp32=True)
+    if case.endswith("dropout"):
+        kw["attention_dropout"] = 0.1
+    if case.startswith("window"):   # 100 keys: row blocks 2 and 3 start after key 0, and after key 128 for the last one
+        kw["sliding_window_width"] = 100
+    if case == "alibi":
+        from megatron.model.positional_embeddings import AliBi
+        kw["alibi_slopes"] = AliBi(np_, 1, 0).slopes
+    fp16, bf16 = dtype == torch.float16, dtype == torch.bfloat16
+    blocked = CoreAttention(hn, 1, fp16, bf16, T.upper_triang, mask_func, **kw).to(DEV)
+    dense = CoreAttention(hn, 1, fp16, bf16, T.upper_triang, mask_func, causal_gemm_blocks=False, **kw).to(DEV)
+    mask = fb.causal_mask(sq, DEV)
+    if case.startswith("window"):
+        pos = torch.arange(sq, device=DEV)
+        mask = mask | (pos.view(1, 1, sq, 1) - pos.view(1, 1, 1, sq) > 100)
+        assert attention_core._row_blocks(sq, 128, 100) == [(0, 128, 0), (128, 256, 0), (256, 328, 128)]
+        assert attention_core._column_blocks(sq, 128, 100) == [(0, 128, 228), (128, 256, 328), (256, 328, 328)]
+    q, k, v = qkv(dtype, sq, b, np_, hn, 51)
+    q2, k2, v2 = (t.detach().clone().requires_grad_(True) for t in (q, k, v))
+    assert blocked._causal_block(mask, b, np_, sq, sq, q) == (512 if case == "2048" else 128)
+    assert dense._causal_block(mask, b, np_, sq, sq, q) == 0
+    g = util.randn((sq, b, np_ * hn), dtype, seed=55).to(DEV)
+    torch.manual_seed(7)
+    monkeypatch.setattr(attention_core.torch, "empty", poisoned_empty)
+    out = blocked(q, k, v, mask, merged_heads=True)
+    out.backward(g)
+    monkeypatch.setattr(attention_core.torch, "empty", real_empty)
+    torch.manual_seed(7)   # the same dropout seed for the second module
+    out2 = dense(q2, k2, v2, mask, merged_heads=True)
+    out2.backward(g)
+    lim = 2.0 ** (-7 if dtype == torch.bfloat16 else -9)
+    for got, want in ((out, out2), (q.grad, q2.grad), (k.grad, k2.grad), (v.grad, v2.grad)):
+        assert torch.isfinite(got).all()
+        assert rel_err(got, want) <= lim / 4
+    if case in ("2048", "small-blocks-ragged", "fp16-alpha", "window"):
+        q3, k3, v3 = (t.detach().clone().requires_grad_(True) for t in (q, k, v))
+        ref = textbook(q3, k3, v3, mask).permute(2, 0, 1, 3).reshape(sq, b, np_ * hn)
+        ref.backward(g.float())
+        assert rel_err(out, ref) <= lim
+        for got, want in ((q.grad, q3.grad), (k.grad, k3.grad), (v.grad, v3.grad)):
+            assert rel_err(got, want) <= 2 * lim
+    # the [b, np, sq, hn] result as well
+    assert rel_err(blocked(q.detach(), k.detach(), v.detach(), mask).permute(2, 0, 1, 3).reshape(sq, b, np_ * hn)
+                   if not case.endswith("dropout") else out, out) <= lim / 4
+    # the dense GEMMs are kept where the causal kernel is not what runs
+    general = CoreAttention(hn, 1, fp16, bf16, T.general, mask_func, **kw).to(DEV)
+    assert general._causal_block(mask, b, np_, sq, sq, q) == 0
+    assert blocked._causal_block(mask, b, np_, sq, sq + 8, q) == 0
