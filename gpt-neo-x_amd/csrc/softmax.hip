@@ -161,6 +161,23 @@ __device__ __forceinline__ Band causal_band(uint32_t q, uint32_t window, bool ok
     return b;
 }
 
+// Columns [lo, hi) of row q that have to hold a value when the caller only consumes the result in square
+// blocks of 2^zshift rows and columns: from the start of the block that holds the first key visible to the
+// first row of q's block (column 0 without a window) to the end of the block that holds the diagonal.
+// zshift == 0: the whole row.
+__device__ __forceinline__ Band written_range(uint32_t q, uint32_t window, uint32_t n, uint32_t zshift)
+{
+    Band b;
+    b.lo = 0;
+    b.hi = n;
+    if (zshift != 0) {
+        b.hi = min(n, ((q >> zshift) + 1u) << zshift);
+        const uint32_t r0 = (q >> zshift) << zshift;
+        b.lo = r0 > window ? ((r0 - window) >> zshift) << zshift : 0u;
+    }
+    return b;
+}
+
 // Number of real keys of matrix `mat` ([batch * heads] matrices, one length per batch entry).
 __device__ __forceinline__ uint32_t key_limit(const int32_t* key_lengths, uint32_t mat, uint32_t heads)
 {
@@ -200,7 +217,7 @@ template <int DT, int L, int K, int W, int BW, int EXTRA>
 __global__ void __launch_bounds__((Geo<L, K, W, BW>::kThreads))
 causal_fwd_kernel(uint16_t* y, const uint16_t* x, float scale, uint32_t total_rows, uint32_t n, uint32_t window,
                   const float* slopes, const uint16_t* bias, const int32_t* key_lengths, uint32_t heads,
-                  uint16_t* dropped, DropoutKey dk)
+                  uint16_t* dropped, DropoutKey dk, uint32_t zshift)
 {
     using G = Geo<L, K, W, BW>;
     constexpr bool PER_HEAD = EXTRA == kPerHead;
@@ -291,12 +308,13 @@ causal_fwd_kernel(uint16_t* y, const uint16_t* x, float scale, uint32_t total_ro
 
     softmax_tile<L, K, W>(z, act, lds, wave, lane);
 
-    // The whole row is written in one go, zeros outside the band included:
-    // splitting a row's stores in time costs DRAM efficiency.
+    // The whole row is written in one go, zeros outside the band included (as far as the caller reads
+    // them): splitting a row's stores in time costs DRAM efficiency.
+    const Band wr = written_range(q, window, n, zshift);
 #pragma unroll
     for (int k = 0; k < K; ++k) {
         const uint32_t col = chunk_col<L, W>(k, w, l);
-        if (ok && col < n) {
+        if (ok && col < wr.hi && col >= wr.lo) {
             if ((act >> k & 1u) && col < band.hi && col + 8 > band.lo) {
                 const u32x4 py = pack8<DT>(z[k]);
                 store16_stream(yr + col, py);
@@ -483,7 +501,7 @@ template <int DT, int L, int K, int W, int BW, bool CAUSAL, int EXTRA>
 __global__ void __launch_bounds__((Geo<L, K, W, BW>::kThreads))
 softmax_bwd_kernel(uint16_t* dx, const uint16_t* dy, const uint16_t* y, float scale,
                    uint32_t total_rows, uint32_t n, uint32_t rows_per_matrix, uint32_t window,
-                   const int32_t* key_lengths, uint32_t heads, DropoutKey dk)
+                   const int32_t* key_lengths, uint32_t heads, DropoutKey dk, uint32_t zshift)
 {
     using G = Geo<L, K, W, BW>;
     __shared__ float lds[32];
@@ -560,10 +578,11 @@ softmax_bwd_kernel(uint16_t* dx, const uint16_t* dy, const uint16_t* y, float sc
     const uint32_t zw = Half2<DT>::pack(zv, zv);
 
     // the whole row is written in one go (see the forward kernel)
+    const Band wr = CAUSAL ? written_range(q, window, n, zshift) : Band{0u, n};
 #pragma unroll
     for (int k = 0; k < K; ++k) {
         const uint32_t col = chunk_col<L, W>(k, w, l);
-        if (ok && col < n) {
+        if (ok && col < wr.hi && col >= wr.lo) {
             u32x4 o;
             if ((act >> k & 1u) && col < band.hi && col + 8 > band.lo) {
 #pragma unroll
@@ -821,7 +840,7 @@ constexpr uint32_t kNoWindow = 0xffffffffu;
 template <int DT>
 static int causal_fwd(void* y, const void* x, float scale, int64_t batches, int64_t n, uint32_t window,
                       const float* slopes, const void* bias, const int32_t* kl, uint32_t heads, hipStream_t st,
-                      void* dropped = nullptr, const DropoutKey* drop = nullptr)
+                      void* dropped = nullptr, const DropoutKey* drop = nullptr, uint32_t zshift = 0)
 {
     const int64_t rows = batches * n;
     RowPlan p;
@@ -840,13 +859,13 @@ static int causal_fwd(void* y, const void* x, float scale, int64_t batches, int6
         if (!launch_fits(blocks, G::kThreads)) return NHP_ERR_SHAPE;                       \
         if (dp != nullptr)                                                                 \
             causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves, kDropout><<<blocks, G::kThreads, p.lds, st>>>( \
-                yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, nullptr, nullptr, nullptr, 1, dp, dk); \
+                yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, nullptr, nullptr, nullptr, 1, dp, dk, zshift); \
         else if (slopes != nullptr || bp != nullptr || kl != nullptr)                      \
             causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves, kPerHead><<<blocks, G::kThreads, p.lds, st>>>( \
-                yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, slopes, bp, kl, heads, nullptr, dk); \
+                yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, slopes, bp, kl, heads, nullptr, dk, zshift); \
         else                                                                               \
             causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves, kPlain><<<blocks, G::kThreads, p.lds, st>>>( \
-                yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, nullptr, nullptr, nullptr, 1, nullptr, dk); \
+                yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, nullptr, nullptr, nullptr, 1, nullptr, dk, zshift); \
     }
         NHP_FOR_PLAN(p);
 #undef CALL
@@ -861,7 +880,7 @@ static int causal_fwd(void* y, const void* x, float scale, int64_t batches, int6
 template <int DT, bool CAUSAL>
 static int softmax_bwd(void* dx, const void* dy, const void* y, float scale, int64_t rows, int64_t n,
                        int64_t rows_per_matrix, uint32_t window, const int32_t* kl, uint32_t heads, hipStream_t st,
-                       const DropoutKey* drop = nullptr)
+                       const DropoutKey* drop = nullptr, uint32_t zshift = 0)
 {
     RowPlan p;
     const DropoutKey dk = drop != nullptr ? *drop : DropoutKey{};
@@ -878,14 +897,15 @@ static int softmax_bwd(void* dx, const void* dy, const void* y, float scale, int
         if (dropout)                                                                       \
             softmax_bwd_kernel<DT, L_, K_, W_, kBlockWaves, CAUSAL, kDropout>                      \
                 <<<blocks, G::kThreads, p.lds, st>>>(dxp, dyp, yp, scale, (uint32_t)rows, (uint32_t)n, \
-                                                     (uint32_t)rows_per_matrix, window, nullptr, 1, dk); \
+                                                     (uint32_t)rows_per_matrix, window, nullptr, 1, dk, zshift); \
         else if (CAUSAL && kl != nullptr)                                                  \
             softmax_bwd_kernel<DT, L_, K_, W_, kBlockWaves, CAUSAL, CAUSAL ? kPerHead : kPlain>    \
                 <<<blocks, G::kThreads, p.lds, st>>>(dxp, dyp, yp, scale, (uint32_t)rows, (uint32_t)n, \
-                                                     (uint32_t)rows_per_matrix, window, kl, heads, dk); \
+                                                     (uint32_t)rows_per_matrix, window, kl, heads, dk, zshift); \
         else                                                                               \
             softmax_bwd_kernel<DT, L_, K_, W_, kBlockWaves, CAUSAL, kPlain><<<blocks, G::kThreads, p.lds, st>>>( \
-                dxp, dyp, yp, scale, (uint32_t)rows, (uint32_t)n, (uint32_t)rows_per_matrix, window, nullptr, 1, dk); \
+                dxp, dyp, yp, scale, (uint32_t)rows, (uint32_t)n, (uint32_t)rows_per_matrix, window, nullptr, 1, dk, \
+                zshift);                                                                   \
     }
         NHP_FOR_PLAN(p);
 #undef CALL
@@ -953,12 +973,23 @@ extern "C" {
 
 int64_t nhp_softmax_max_resident_row(void) { return kMaxResidentRow; }
 
-int nhp_causal_softmax_ex_fwd(void* y, const void* x, float scale, int64_t attn_batches, int64_t seq_len,
-                              int64_t window, const float* alibi_slopes, const void* bias,
-                              const int32_t* key_lengths, int64_t heads, int dtype, void* stream)
+// log2 of a block size given as 0 (no blocks: 0) or a power of two >= 8; -1 for anything else
+static int block_shift(int64_t zero_block)
+{
+    if (zero_block == 0) return 0;
+    if (zero_block < 8 || zero_block > ((int64_t)1 << 30) || (zero_block & (zero_block - 1)) != 0) return -1;
+    int shift = 0;
+    while (((int64_t)1 << shift) < zero_block) ++shift;
+    return shift;
+}
+
+int nhp_causal_softmax_blocks_fwd(void* y, const void* x, float scale, int64_t attn_batches, int64_t seq_len,
+                                  int64_t window, int64_t zero_block, const float* alibi_slopes, const void* bias,
+                                  const int32_t* key_lengths, int64_t heads, int dtype, void* stream)
 {
     if (dtype != NHP_F16 && dtype != NHP_BF16) return NHP_ERR_DTYPE;
-    if (attn_batches < 0 || seq_len < 0) return NHP_ERR_SHAPE;
+    const int zshift = block_shift(zero_block);
+    if (attn_batches < 0 || seq_len < 0 || zshift < 0) return NHP_ERR_SHAPE;
     const bool per_head = alibi_slopes != nullptr || bias != nullptr || key_lengths != nullptr;
     if (per_head && (heads < 1 || attn_batches % heads != 0)) return NHP_ERR_SHAPE;
     if (bias != nullptr && (bias == y)) return NHP_ERR_ALIAS;
@@ -968,9 +999,18 @@ int nhp_causal_softmax_ex_fwd(void* y, const void* x, float scale, int64_t attn_
     hipStream_t st = static_cast<hipStream_t>(stream);
     const uint32_t win = (window < 0 || window >= seq_len) ? kNoWindow : (uint32_t)window;
     const uint32_t hd = per_head ? (uint32_t)heads : 1u;
-    return dtype == NHP_BF16
-               ? causal_fwd<NHP_BF16>(y, x, scale, attn_batches, seq_len, win, alibi_slopes, bias, key_lengths, hd, st)
-               : causal_fwd<NHP_F16>(y, x, scale, attn_batches, seq_len, win, alibi_slopes, bias, key_lengths, hd, st);
+    return dtype == NHP_BF16 ? causal_fwd<NHP_BF16>(y, x, scale, attn_batches, seq_len, win, alibi_slopes, bias,
+                                                    key_lengths, hd, st, nullptr, nullptr, (uint32_t)zshift)
+                             : causal_fwd<NHP_F16>(y, x, scale, attn_batches, seq_len, win, alibi_slopes, bias,
+                                                   key_lengths, hd, st, nullptr, nullptr, (uint32_t)zshift);
+}
+
+int nhp_causal_softmax_ex_fwd(void* y, const void* x, float scale, int64_t attn_batches, int64_t seq_len,
+                              int64_t window, const float* alibi_slopes, const void* bias,
+                              const int32_t* key_lengths, int64_t heads, int dtype, void* stream)
+{
+    return nhp_causal_softmax_blocks_fwd(y, x, scale, attn_batches, seq_len, window, 0, alibi_slopes, bias, key_lengths,
+                                         heads, dtype, stream);
 }
 
 int nhp_causal_softmax_fwd(void* y, const void* x, float scale, int64_t attn_batches, int64_t seq_len,
@@ -980,12 +1020,13 @@ int nhp_causal_softmax_fwd(void* y, const void* x, float scale, int64_t attn_bat
                                      stream);
 }
 
-int nhp_causal_softmax_ex_bwd(void* dx, const void* dy, const void* y, float scale, int64_t attn_batches,
-                              int64_t seq_len, int64_t window, const int32_t* key_lengths, int64_t heads,
-                              int dtype, void* stream)
+int nhp_causal_softmax_blocks_bwd(void* dx, const void* dy, const void* y, float scale, int64_t attn_batches,
+                                  int64_t seq_len, int64_t window, int64_t zero_block, const int32_t* key_lengths,
+                                  int64_t heads, int dtype, void* stream)
 {
     if (dtype != NHP_F16 && dtype != NHP_BF16) return NHP_ERR_DTYPE;
-    if (attn_batches < 0 || seq_len < 0) return NHP_ERR_SHAPE;
+    const int zshift = block_shift(zero_block);
+    if (attn_batches < 0 || seq_len < 0 || zshift < 0) return NHP_ERR_SHAPE;
     if (key_lengths != nullptr && (heads < 1 || attn_batches % heads != 0)) return NHP_ERR_SHAPE;
     if (attn_batches == 0 || seq_len == 0) return NHP_OK;
     if (attn_batches > kMaxRows / seq_len - 1) return NHP_ERR_SHAPE;
@@ -995,9 +1036,18 @@ int nhp_causal_softmax_ex_bwd(void* dx, const void* dy, const void* y, float sca
     const int64_t rows = attn_batches * seq_len;
     const uint32_t win = (window < 0 || window >= seq_len) ? kNoWindow : (uint32_t)window;
     const uint32_t hd = key_lengths != nullptr ? (uint32_t)heads : 1u;
-    return dtype == NHP_BF16
-               ? softmax_bwd<NHP_BF16, true>(dx, dy, y, scale, rows, seq_len, seq_len, win, key_lengths, hd, st)
-               : softmax_bwd<NHP_F16, true>(dx, dy, y, scale, rows, seq_len, seq_len, win, key_lengths, hd, st);
+    return dtype == NHP_BF16 ? softmax_bwd<NHP_BF16, true>(dx, dy, y, scale, rows, seq_len, seq_len, win, key_lengths, hd,
+                                                           st, nullptr, (uint32_t)zshift)
+                             : softmax_bwd<NHP_F16, true>(dx, dy, y, scale, rows, seq_len, seq_len, win, key_lengths, hd,
+                                                          st, nullptr, (uint32_t)zshift);
+}
+
+int nhp_causal_softmax_ex_bwd(void* dx, const void* dy, const void* y, float scale, int64_t attn_batches,
+                              int64_t seq_len, int64_t window, const int32_t* key_lengths, int64_t heads,
+                              int dtype, void* stream)
+{
+    return nhp_causal_softmax_blocks_bwd(dx, dy, y, scale, attn_batches, seq_len, window, 0, key_lengths, heads, dtype,
+                                         stream);
 }
 
 int nhp_causal_softmax_bwd(void* dx, const void* dy, const void* y, float scale, int64_t attn_batches,
@@ -1006,12 +1056,13 @@ int nhp_causal_softmax_bwd(void* dx, const void* dy, const void* y, float scale,
     return nhp_causal_softmax_ex_bwd(dx, dy, y, scale, attn_batches, seq_len, -1, nullptr, 1, dtype, stream);
 }
 
-int nhp_causal_softmax_dropout_fwd(void* dropped, void* y, const void* x, float scale, int64_t attn_batches,
-                                   int64_t seq_len, int64_t window, float p, uint64_t seed, uint64_t offset, int dtype,
-                                   void* stream)
+int nhp_causal_softmax_dropout_blocks_fwd(void* dropped, void* y, const void* x, float scale, int64_t attn_batches,
+                                          int64_t seq_len, int64_t window, int64_t zero_block, float p, uint64_t seed,
+                                          uint64_t offset, int dtype, void* stream)
 {
     if (dtype != NHP_F16 && dtype != NHP_BF16) return NHP_ERR_DTYPE;
-    if (attn_batches < 0 || seq_len < 0 || !(p >= 0.0f && p < 1.0f)) return NHP_ERR_SHAPE;
+    const int zshift = block_shift(zero_block);
+    if (attn_batches < 0 || seq_len < 0 || !(p >= 0.0f && p < 1.0f) || zshift < 0) return NHP_ERR_SHAPE;
     if (attn_batches == 0 || seq_len == 0) return NHP_OK;
     if (attn_batches > kMaxRows / seq_len - 1) return NHP_ERR_SHAPE;
     if (!x || !y || !dropped) return NHP_ERR_NULL;
@@ -1019,17 +1070,27 @@ int nhp_causal_softmax_dropout_fwd(void* dropped, void* y, const void* x, float 
     hipStream_t st = static_cast<hipStream_t>(stream);
     const uint32_t win = (window < 0 || window >= seq_len) ? kNoWindow : (uint32_t)window;
     const DropoutKey dk = make_dropout_key(p, seed, offset);
-    return dtype == NHP_BF16
-               ? causal_fwd<NHP_BF16>(y, x, scale, attn_batches, seq_len, win, nullptr, nullptr, nullptr, 1, st, dropped, &dk)
-               : causal_fwd<NHP_F16>(y, x, scale, attn_batches, seq_len, win, nullptr, nullptr, nullptr, 1, st, dropped, &dk);
+    return dtype == NHP_BF16 ? causal_fwd<NHP_BF16>(y, x, scale, attn_batches, seq_len, win, nullptr, nullptr, nullptr, 1,
+                                                    st, dropped, &dk, (uint32_t)zshift)
+                             : causal_fwd<NHP_F16>(y, x, scale, attn_batches, seq_len, win, nullptr, nullptr, nullptr, 1,
+                                                   st, dropped, &dk, (uint32_t)zshift);
 }
 
-int nhp_causal_softmax_dropout_bwd(void* dx, const void* dy, const void* y, float scale, int64_t attn_batches,
+int nhp_causal_softmax_dropout_fwd(void* dropped, void* y, const void* x, float scale, int64_t attn_batches,
                                    int64_t seq_len, int64_t window, float p, uint64_t seed, uint64_t offset, int dtype,
                                    void* stream)
 {
+    return nhp_causal_softmax_dropout_blocks_fwd(dropped, y, x, scale, attn_batches, seq_len, window, 0, p, seed, offset,
+                                                 dtype, stream);
+}
+
+int nhp_causal_softmax_dropout_blocks_bwd(void* dx, const void* dy, const void* y, float scale, int64_t attn_batches,
+                                          int64_t seq_len, int64_t window, int64_t zero_block, float p, uint64_t seed,
+                                          uint64_t offset, int dtype, void* stream)
+{
     if (dtype != NHP_F16 && dtype != NHP_BF16) return NHP_ERR_DTYPE;
-    if (attn_batches < 0 || seq_len < 0 || !(p >= 0.0f && p < 1.0f)) return NHP_ERR_SHAPE;
+    const int zshift = block_shift(zero_block);
+    if (attn_batches < 0 || seq_len < 0 || !(p >= 0.0f && p < 1.0f) || zshift < 0) return NHP_ERR_SHAPE;
     if (attn_batches == 0 || seq_len == 0) return NHP_OK;
     if (attn_batches > kMaxRows / seq_len - 1) return NHP_ERR_SHAPE;
     if (!dx || !dy || !y) return NHP_ERR_NULL;
@@ -1039,8 +1100,16 @@ int nhp_causal_softmax_dropout_bwd(void* dx, const void* dy, const void* y, floa
     const uint32_t win = (window < 0 || window >= seq_len) ? kNoWindow : (uint32_t)window;
     const DropoutKey dk = make_dropout_key(p, seed, offset);
     return dtype == NHP_BF16
-               ? softmax_bwd<NHP_BF16, true>(dx, dy, y, scale, rows, seq_len, seq_len, win, nullptr, 1, st, &dk)
-               : softmax_bwd<NHP_F16, true>(dx, dy, y, scale, rows, seq_len, seq_len, win, nullptr, 1, st, &dk);
+               ? softmax_bwd<NHP_BF16, true>(dx, dy, y, scale, rows, seq_len, seq_len, win, nullptr, 1, st, &dk, (uint32_t)zshift)
+               : softmax_bwd<NHP_F16, true>(dx, dy, y, scale, rows, seq_len, seq_len, win, nullptr, 1, st, &dk, (uint32_t)zshift);
+}
+
+int nhp_causal_softmax_dropout_bwd(void* dx, const void* dy, const void* y, float scale, int64_t attn_batches,
+                                   int64_t seq_len, int64_t window, float p, uint64_t seed, uint64_t offset, int dtype,
+                                   void* stream)
+{
+    return nhp_causal_softmax_dropout_blocks_bwd(dx, dy, y, scale, attn_batches, seq_len, window, 0, p, seed, offset, dtype,
+                                                 stream);
 }
 
 int nhp_masked_softmax_fwd(void* y, const void* x, const uint8_t* mask, float scale, int64_t b,

@@ -45,6 +45,10 @@ def _declare(lib):
         "nhp_causal_softmax_ex_bwd": ([vp, vp, vp, f32, i64, i64, i64, vp, i64, ci, vp], ci),
         "nhp_causal_softmax_dropout_fwd": ([vp, vp, vp, f32, i64, i64, i64, f32, u64, u64, ci, vp], ci),
         "nhp_causal_softmax_dropout_bwd": ([vp, vp, vp, f32, i64, i64, i64, f32, u64, u64, ci, vp], ci),
+        "nhp_causal_softmax_blocks_fwd": ([vp, vp, f32, i64, i64, i64, i64, vp, vp, vp, i64, ci, vp], ci),
+        "nhp_causal_softmax_blocks_bwd": ([vp, vp, vp, f32, i64, i64, i64, i64, vp, i64, ci, vp], ci),
+        "nhp_causal_softmax_dropout_blocks_fwd": ([vp, vp, vp, f32, i64, i64, i64, i64, f32, u64, u64, ci, vp], ci),
+        "nhp_causal_softmax_dropout_blocks_bwd": ([vp, vp, vp, f32, i64, i64, i64, i64, f32, u64, u64, ci, vp], ci),
         "nhp_masked_softmax_dropout_fwd": ([vp, vp, vp, vp, f32, i64, i64, i64, i64, i64, f32, u64, u64, ci, vp], ci),
         "nhp_masked_softmax_dropout_bwd": ([vp, vp, vp, f32, i64, i64, f32, u64, u64, ci, vp], ci),
         "nhp_masked_softmax_fwd": ([vp, vp, vp, f32, i64, i64, i64, i64, i64, ci, vp], ci),

@@ -250,7 +250,10 @@ class CoreAttention(torch.nn.Module):
             window = None if window is None or window < 0 else int(window)
             scores = _CausalScoreGemm.apply(q.transpose(0, 1), k.transpose(0, 1), self.gemm_alpha, block, window)
             bias = self.rpe(sq, sk) if self.rpe is not None else None
-            probs = self.scale_mask_softmax(scores.view(b, np_, sq, sk), attention_mask, bias=bias, key_lengths=key_lengths)
+            # ... and is told that nobody reads the other blocks of its results, which it then does not write
+            zero_block = block if block & (block - 1) == 0 else 0
+            probs = self.scale_mask_softmax(scores.view(b, np_, sq, sk), attention_mask, bias=bias, key_lengths=key_lengths,
+                                            zero_block=zero_block)
             v = value_layer.reshape(sk, b * np_, value_layer.size(3)).transpose(0, 1)
             context = _CausalContextGemm.apply(probs.view(b * np_, sq, sk), v, block, window, merged_heads)
             if merged_heads:

@@ -60,12 +60,13 @@ class ScaledUpperTriangMaskedSoftmax(torch.autograd.Function):
     """
 
     @staticmethod
-    def forward(ctx, inputs, scale, window=None, alibi_slopes=None, bias=None, key_lengths=None):
+    def forward(ctx, inputs, scale, window=None, alibi_slopes=None, bias=None, key_lengths=None, zero_block=0):
         import scaled_upper_triang_masked_softmax_cuda as kernels
 
         factor = _scale_tensor(scale)
-        out = kernels.forward(inputs, factor[0], window, alibi_slopes, bias, key_lengths)
+        out = kernels.forward(inputs, factor[0], window, alibi_slopes, bias, key_lengths, zero_block)
         ctx.window = window
+        ctx.zero_block = zero_block
         ctx.key_lengths = key_lengths
         ctx.bias_shape = None if bias is None else tuple(bias.shape)
         ctx.save_for_backward(out, factor)
@@ -77,13 +78,28 @@ class ScaledUpperTriangMaskedSoftmax(torch.autograd.Function):
 
         out, factor = ctx.saved_tensors
         # in place on output_grads, like the reference kernel
-        grad = kernels.backward(output_grads, out, factor[0], ctx.window, ctx.key_lengths)
+        grad = kernels.backward(output_grads, out, factor[0], ctx.window, ctx.key_lengths, ctx.zero_block)
         grad_bias = None
         if ctx.bias_shape is not None and ctx.needs_input_grad[4]:
             # the bias is shared by the batch: its gradient is the batch sum of the score gradient
             heads, sq, sk = ctx.bias_shape[-3:]
-            grad_bias = grad.view(-1, heads, sq, sk).sum(dim=0).view(ctx.bias_shape)
-        return grad, None, None, None, grad_bias, None
+            full = grad
+            if ctx.zero_block:
+                # the blocks the kernel did not write hold no gradient: leave them out of the sum
+                full = torch.where(_written_blocks(sq, ctx.zero_block, ctx.window, grad.device), grad, torch.zeros_like(grad))
+            grad_bias = full.view(-1, heads, sq, sk).sum(dim=0).view(ctx.bias_shape)
+        return grad, None, None, None, grad_bias, None, None
+
+
+def _written_blocks(seq_len, zero_block, window, device):
+    """[seq_len, seq_len] bool: the part of every row that the causal kernels write when called with ``zero_block``."""
+    q = torch.arange(seq_len, device=device).view(seq_len, 1)
+    k = torch.arange(seq_len, device=device).view(1, seq_len)
+    hi = (q // zero_block + 1) * zero_block
+    lo = torch.zeros_like(q)
+    if window is not None and 0 <= window < seq_len:
+        lo = (q // zero_block * zero_block - window).clamp(min=0) // zero_block * zero_block
+    return (k < hi) & (k >= lo)
 
 
 class ScaledUpperTriangMaskedSoftmaxDropout(torch.autograd.Function):
@@ -91,12 +107,12 @@ class ScaledUpperTriangMaskedSoftmaxDropout(torch.autograd.Function):
     No counterpart in the reference, which runs ``torch.nn.Dropout`` on the probabilities."""
 
     @staticmethod
-    def forward(ctx, inputs, scale, prob, seed, window=None):
+    def forward(ctx, inputs, scale, prob, seed, window=None, zero_block=0):
         import scaled_upper_triang_masked_softmax_cuda as kernels
 
         factor = _scale_tensor(scale)
-        dropped, probs = kernels.forward_dropout(inputs, factor[0], prob, seed, window)
-        ctx.conf = (float(prob), int(seed), window)
+        dropped, probs = kernels.forward_dropout(inputs, factor[0], prob, seed, window, zero_block)
+        ctx.conf = (float(prob), int(seed), window, zero_block)
         ctx.save_for_backward(probs, factor)
         return dropped
 
@@ -105,8 +121,9 @@ class ScaledUpperTriangMaskedSoftmaxDropout(torch.autograd.Function):
         import scaled_upper_triang_masked_softmax_cuda as kernels
 
         probs, factor = ctx.saved_tensors
-        prob, seed, window = ctx.conf
-        return kernels.backward_dropout(output_grads, probs, factor[0], prob, seed, window), None, None, None, None
+        prob, seed, window, zero_block = ctx.conf
+        grad = kernels.backward_dropout(output_grads, probs, factor[0], prob, seed, window, zero_block)
+        return grad, None, None, None, None, None
 
 
 class ScaledMaskedSoftmax(torch.autograd.Function):
@@ -205,7 +222,10 @@ class FusedScaleMaskSoftmax(nn.Module):
             self.register_buffer("alibi_slopes", alibi_slopes.detach().float().clone(), persistent=False)
 
     # ------------------------------------------------------------------ dispatch
-    def forward(self, input, mask, bias=None, key_lengths=None):
+    def forward(self, input, mask, bias=None, key_lengths=None, zero_block=0):
+        """``zero_block`` (causal kernel only, ignored elsewhere): the caller reads the probabilities in square
+        blocks of that size and skips those without a visible (query, key) pair; the kernel then leaves them
+        unwritten (see ``scaled_upper_triang_masked_softmax_cuda.forward``)."""
         assert input.dim() == 4  # [b, np, sq, sk]
         dropout = self.attention_dropout if self.training else 0.0
         if self.upper_triang_mask_fusion and input.size(2) != input.size(3):
@@ -222,14 +242,14 @@ class FusedScaleMaskSoftmax(nn.Module):
                 factor = 1.0 if self.scale is None else self.scale
                 seed = int(torch.empty((), dtype=torch.int64).random_().item())  # CPU generator: no device sync
                 probs = ScaledUpperTriangMaskedSoftmaxDropout.apply(input.view(b * np, sq, sk), factor, dropout, seed,
-                                                                    self.sliding_window_width)
+                                                                    self.sliding_window_width, zero_block)
                 return probs.view(b, np, sq, sk)
             if (dropout > 0.0 and self.general_mask_fusion and bias is None and key_lengths is None
                     and self.alibi_slopes is None):
                 factor = 1.0 if self.scale is None else self.scale
                 seed = int(torch.empty((), dtype=torch.int64).random_().item())
                 return ScaledMaskedSoftmaxDropout.apply(input, mask, factor, dropout, seed)
-            probs = self.forward_fused_softmax(input, mask, bias, key_lengths)
+            probs = self.forward_fused_softmax(input, mask, bias, key_lengths, zero_block)
         else:
             probs = self.forward_torch_softmax(input, mask, bias, key_lengths)
         if dropout > 0.0:
@@ -275,7 +295,7 @@ class FusedScaleMaskSoftmax(nn.Module):
         padding = keys.view(1, 1, 1, sk) >= key_lengths.to(mask.device).view(b, 1, 1, 1)
         return (mask.bool() | padding).contiguous()
 
-    def forward_fused_softmax(self, input, mask, bias=None, key_lengths=None):
+    def forward_fused_softmax(self, input, mask, bias=None, key_lengths=None, zero_block=0):
         b, np, sq, sk = input.size()
         factor = 1.0 if self.scale is None else self.scale
         if not self.upper_triang_mask_fusion:
@@ -296,7 +316,8 @@ class FusedScaleMaskSoftmax(nn.Module):
             assert bias.shape[-3:] == (np, sq, sk) and bias.numel() == np * sq * sk, "bias must be [1, np, sq, sk]"
         if key_lengths is not None:
             assert key_lengths.shape == (b,), "key_lengths must be [b]"
-        probs = ScaledUpperTriangMaskedSoftmax.apply(flat, factor, self.sliding_window_width, slopes, bias, key_lengths)
+        probs = ScaledUpperTriangMaskedSoftmax.apply(flat, factor, self.sliding_window_width, slopes, bias, key_lengths,
+                                                     zero_block)
         return probs.view(b, np, sq, sk)
 
     def forward_torch_softmax(self, input, mask, bias=None, key_lengths=None):

@@ -25,7 +25,14 @@ def _key_lengths_arg(key_lengths, attn_batches, heads, who):
     return lengths, lengths.data_ptr(), attn_batches // batch
 
 
-def forward(input, scale_factor, window=None, alibi_slopes=None, bias=None, key_lengths=None):
+def _zero_block(zero_block):
+    zero_block = int(zero_block or 0)
+    if zero_block and (zero_block < 8 or zero_block & (zero_block - 1)):
+        raise RuntimeError("zero_block must be 0 or a power of two of at least 8")
+    return zero_block
+
+
+def forward(input, scale_factor, window=None, alibi_slopes=None, bias=None, key_lengths=None, zero_block=0):
     """softmax(scale * input) under an upper-triangular mask.
 
     input: [attn_batches, seq_len, seq_len] fp16/bf16 on the GPU. Returns a new
@@ -43,6 +50,10 @@ def forward(input, scale_factor, window=None, alibi_slopes=None, bias=None, key_
     key_lengths: integer tensor [batch] on the GPU, input being [batch * heads, s, s]:
         keys at or beyond a batch entry's length are padding and get probability 0
         (rows without any key left are all zeros).
+    zero_block: for a caller that reads the result in square blocks of this many rows and columns
+        and skips the blocks without a visible (query, key) pair: row q is only written from the
+        start of the block of the first key that the first row of its block sees to the end of the
+        block of the diagonal; the rest of the returned tensor is uninitialised. 0: every row whole.
     """
     if input.dim() != 3:
         raise RuntimeError("expected 3D tensor")
@@ -78,17 +89,18 @@ def forward(input, scale_factor, window=None, alibi_slopes=None, bias=None, key_
     lengths, lengths_ptr, heads = _key_lengths_arg(key_lengths, x.size(0), heads,
                                                    "scaled_upper_triang_masked_softmax_cuda.forward")
     with _hp.device_guard(x):
-        rc = _hp.lib().nhp_causal_softmax_ex_fwd(
+        rc = _hp.lib().nhp_causal_softmax_blocks_fwd(
             y.data_ptr(), x.data_ptr(), float(scale_factor), x.size(0), x.size(1),
-            -1 if window is None else int(window), slopes_ptr, bias_ptr, lengths_ptr, heads or 1,
+            -1 if window is None else int(window), _zero_block(zero_block), slopes_ptr, bias_ptr, lengths_ptr, heads or 1,
             _hp.dtype_code(x, "forward"), _hp.stream_of(x))
     _hp.check(rc, "scaled_upper_triang_masked_softmax_cuda.forward")
     return y
 
 
-def backward(output_grads, softmax_results, scale_factor, window=None, key_lengths=None):
+def backward(output_grads, softmax_results, scale_factor, window=None, key_lengths=None, zero_block=0):
     """Gradient w.r.t. the input of ``forward`` (pass the same ``window`` and ``key_lengths``;
-    AliBi and the bias tensor need nothing here).
+    AliBi and the bias tensor need nothing here; ``zero_block`` as in ``forward``: only that part
+    of every row is read and written).
 
     Works in place: the result is written into (the contiguous version of)
     ``output_grads`` and that tensor is returned, as in
@@ -109,15 +121,16 @@ def backward(output_grads, softmax_results, scale_factor, window=None, key_lengt
     lengths, lengths_ptr, heads = _key_lengths_arg(key_lengths, g.size(0), None,
                                                    "scaled_upper_triang_masked_softmax_cuda.backward")
     with _hp.device_guard(g):
-        rc = _hp.lib().nhp_causal_softmax_ex_bwd(
+        rc = _hp.lib().nhp_causal_softmax_blocks_bwd(
             g.data_ptr(), g.data_ptr(), y.data_ptr(), float(scale_factor), g.size(0), g.size(1),
-            -1 if window is None else int(window), lengths_ptr, heads or 1, _hp.dtype_code(g, "backward"),
+            -1 if window is None else int(window), _zero_block(zero_block), lengths_ptr, heads or 1,
+            _hp.dtype_code(g, "backward"),
             _hp.stream_of(g))
     _hp.check(rc, "scaled_upper_triang_masked_softmax_cuda.backward")
     return g
 
 
-def forward_dropout(input, scale_factor, p, seed, window=None):
+def forward_dropout(input, scale_factor, p, seed, window=None, zero_block=0):
     """``forward`` and attention dropout in one kernel: returns ``(dropped, probabilities)``.
 
     ``dropped = keep * probabilities / (1 - p)`` with the library's counter-based keep mask for
@@ -134,15 +147,16 @@ def forward_dropout(input, scale_factor, p, seed, window=None):
     y = torch.empty_like(x)
     dropped = torch.empty_like(x)
     with _hp.device_guard(x):
-        rc = _hp.lib().nhp_causal_softmax_dropout_fwd(
+        rc = _hp.lib().nhp_causal_softmax_dropout_blocks_fwd(
             dropped.data_ptr(), y.data_ptr(), x.data_ptr(), float(scale_factor), x.size(0), x.size(1),
-            -1 if window is None else int(window), float(p), int(seed), 0, _hp.dtype_code(x, "forward_dropout"),
+            -1 if window is None else int(window), _zero_block(zero_block), float(p), int(seed), 0,
+            _hp.dtype_code(x, "forward_dropout"),
             _hp.stream_of(x))
     _hp.check(rc, "scaled_upper_triang_masked_softmax_cuda.forward_dropout")
     return dropped, y
 
 
-def backward_dropout(output_grads, softmax_results, scale_factor, p, seed, window=None):
+def backward_dropout(output_grads, softmax_results, scale_factor, p, seed, window=None, zero_block=0):
     """Gradient of ``forward_dropout`` with respect to its input, given the gradient of ``dropped``;
     in place on ``output_grads`` like ``backward``."""
     if output_grads.dim() != 3 or softmax_results.dim() != 3:
@@ -156,9 +170,10 @@ def backward_dropout(output_grads, softmax_results, scale_factor, p, seed, windo
     g = output_grads.detach().contiguous()
     y = softmax_results.detach().contiguous()
     with _hp.device_guard(g):
-        rc = _hp.lib().nhp_causal_softmax_dropout_bwd(
+        rc = _hp.lib().nhp_causal_softmax_dropout_blocks_bwd(
             g.data_ptr(), g.data_ptr(), y.data_ptr(), float(scale_factor), g.size(0), g.size(1),
-            -1 if window is None else int(window), float(p), int(seed), 0, _hp.dtype_code(g, "backward_dropout"),
+            -1 if window is None else int(window), _zero_block(zero_block), float(p), int(seed), 0,
+            _hp.dtype_code(g, "backward_dropout"),
             _hp.stream_of(g))
     _hp.check(rc, "scaled_upper_triang_masked_softmax_cuda.backward_dropout")
     return g

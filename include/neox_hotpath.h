@@ -162,6 +162,40 @@ int nhp_causal_softmax_dropout_bwd(void* dx, const void* dy, const void* y, floa
                                    float p, uint64_t seed, uint64_t offset, int dtype, void* stream);
 
 /*
+ * The causal softmax entry points above for a caller that consumes the [seq_len, seq_len] matrices in
+ * square blocks of `zero_block` rows and columns and skips the blocks that hold no visible (query, key)
+ * pair -- the batched GEMMs either side of the softmax in ParallelSelfAttention.attention
+ * (megatron/model/transformer.py:556-621: baddbmm before, bmm after) computed block by block. Row q of
+ * y / dropped / dx is written from the start of the block that holds the first key visible to the first
+ * row of q's block (column 0 without a window) to the end of the block that holds the diagonal, zeros
+ * included; the columns outside that range are neither read nor written. zero_block: a power of two >= 8, or 0 for the whole row
+ * (then these are exactly nhp_causal_softmax_ex_* / nhp_causal_softmax_dropout_*). Rows that take the
+ * scalar kernels (seq_len not a multiple of 8, unaligned pointers) are written whole.
+ * Replaces scaled_upper_triang_masked_softmax_cuda.forward / backward
+ * (megatron/fused_kernels/scaled_upper_triang_masked_softmax.cpp:31-56), whose zeros above the diagonal
+ * are a third of the forward's memory traffic.
+ */
+int nhp_causal_softmax_blocks_fwd(void* y, const void* x, float scale, int64_t attn_batches,
+                                  int64_t seq_len, int64_t window, int64_t zero_block,
+                                  const float* alibi_slopes, const void* bias,
+                                  const int32_t* key_lengths, int64_t heads, int dtype, void* stream);
+
+int nhp_causal_softmax_blocks_bwd(void* dx, const void* dy, const void* y, float scale,
+                                  int64_t attn_batches, int64_t seq_len, int64_t window,
+                                  int64_t zero_block, const int32_t* key_lengths, int64_t heads,
+                                  int dtype, void* stream);
+
+int nhp_causal_softmax_dropout_blocks_fwd(void* dropped, void* y, const void* x, float scale,
+                                          int64_t attn_batches, int64_t seq_len, int64_t window,
+                                          int64_t zero_block, float p, uint64_t seed, uint64_t offset,
+                                          int dtype, void* stream);
+
+int nhp_causal_softmax_dropout_blocks_bwd(void* dx, const void* dy, const void* y, float scale,
+                                          int64_t attn_batches, int64_t seq_len, int64_t window,
+                                          int64_t zero_block, float p, uint64_t seed, uint64_t offset,
+                                          int dtype, void* stream);
+
+/*
  * The same for the padding-mask softmax: y as nhp_masked_softmax_fwd, dropped = keep ? y / (1 - p) : 0
  * over the flat element index of the [b, np, sq, sk] tensor; the backward is nhp_masked_softmax_bwd of
  * g = keep ? dy / (1 - p) : 0 (rows = b * np * sq).

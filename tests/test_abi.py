@@ -117,6 +117,7 @@ def test_argument_validation_of_the_layer_entry_points(hotpath):
     F16, BF16, F32 = hotpath.F16, hotpath.BF16, hotpath.F32
     p = ctypes.c_void_p(0x1000)  # never dereferenced
     q = ctypes.c_void_p(0x2000)
+    q2 = ctypes.c_void_p(0x3000)
     null = ctypes.c_void_p(0)
     # causal softmax variants: heads must divide attn_batches when a per-head operand is given
     assert lib.nhp_causal_softmax_ex_fwd(q, p, 1.0, 6, 8, -1, p, null, null, 4, BF16, None) == -2
@@ -125,6 +126,16 @@ def test_argument_validation_of_the_layer_entry_points(hotpath):
     assert lib.nhp_causal_softmax_ex_fwd(q, p, 1.0, 6, 8, -1, null, q, null, 3, BF16, None) == -6   # bias over the output
     assert lib.nhp_causal_softmax_ex_bwd(q, p, p, 1.0, 6, 8, -1, p, 4, BF16, None) == -2
     assert lib.nhp_causal_softmax_ex_fwd(null, null, 1.0, 0, 8, 3, null, null, null, 1, F16, None) == 0
+    # block-limited variants: the block size must be 0 or a power of two of at least 8
+    for bad in (4, 12, 100, -8):
+        assert lib.nhp_causal_softmax_blocks_fwd(q, p, 1.0, 6, 64, -1, bad, null, null, null, 1, BF16, None) == -2
+        assert lib.nhp_causal_softmax_blocks_bwd(q, p, p, 1.0, 6, 64, -1, bad, null, 1, BF16, None) == -2
+        assert lib.nhp_causal_softmax_dropout_blocks_fwd(q, q2, p, 1.0, 6, 64, -1, bad, 0.1, 1, 0, BF16, None) == -2
+        assert lib.nhp_causal_softmax_dropout_blocks_bwd(q, p, p, 1.0, 6, 64, -1, bad, 0.1, 1, 0, BF16, None) == -2
+    assert lib.nhp_causal_softmax_blocks_fwd(q, p, 1.0, 6, 64, -1, 16, null, null, null, 1, 5, None) == -1
+    assert lib.nhp_causal_softmax_blocks_fwd(null, p, 1.0, 6, 64, -1, 16, null, null, null, 1, BF16, None) == -3
+    assert lib.nhp_causal_softmax_blocks_fwd(null, null, 1.0, 0, 64, -1, 16, null, null, null, 1, BF16, None) == 0
+    assert lib.nhp_causal_softmax_blocks_bwd(q, p, q, 1.0, 6, 64, -1, 16, null, 1, BF16, None) == -6
     # bias + GeLU, bias + residual
     assert lib.nhp_bias_gelu_fwd(q, p, p, 4, 8, 9, None) == -1
     assert lib.nhp_bias_gelu_fwd(q, p, p, -1, 8, BF16, None) == -2
@@ -168,7 +179,6 @@ def test_argument_validation_of_the_layer_entry_points(hotpath):
     assert lib.nhp_layernorm_bwd(q, null, null, p, p, null, p, p, null, 4, 8, BF16, BF16, None) == -3   # mean missing
     assert lib.nhp_layernorm_bwd(q, p, null, p, p, p, p, p, null, 4, 8, BF16, BF16, None) == -3          # workspace missing
     # two LayerNorms of one input
-    q2 = ctypes.c_void_p(0x3000)
     assert lib.nhp_layernorm_pair_fwd(q, q2, null, null, p, p, p, p, p, 1e-5, 4, 8, 4, F32, None) == -1
     assert lib.nhp_layernorm_pair_fwd(q, q2, null, null, p, p, p, p, p, 1e-5, 4, 8, BF16, F16, None) == -1
     assert lib.nhp_layernorm_pair_fwd(q, q2, null, null, p, p, p, p, p, 1e-5, 4, -8, BF16, F32, None) == -2

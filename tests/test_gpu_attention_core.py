@@ -355,8 +355,14 @@ def test_blocked_causal_gemms_equal_the_dense_ones(case, monkeypatch):
         monkeypatch.setattr(attention_core, "causal_gemm_block", lambda s: 128)   # blocks of 128, 128 and 72 rows
     real_empty = torch.empty
 
+    real_empty_like = torch.empty_like
+
     def poisoned_empty(*args, **kw):
         t = real_empty(*args, **kw)
+        return t.fill_(float("nan")) if t.is_floating_point() else t
+
+    def poisoned_empty_like(*args, **kw):   # the softmax outputs, of which the kernel writes only the blocks in use
+        t = real_empty_like(*args, **kw)
         return t.fill_(float("nan")) if t.is_floating_point() else t
 
     kw = dict(attention_softmax_in_fp32=True)
@@ -383,9 +389,11 @@ def test_blocked_causal_gemms_equal_the_dense_ones(case, monkeypatch):
     g = util.randn((sq, b, np_ * hn), dtype, seed=55).to(DEV)
     torch.manual_seed(7)
     monkeypatch.setattr(attention_core.torch, "empty", poisoned_empty)
+    monkeypatch.setattr(attention_core.torch, "empty_like", poisoned_empty_like)
     out = blocked(q, k, v, mask, merged_heads=True)
     out.backward(g)
     monkeypatch.setattr(attention_core.torch, "empty", real_empty)
+    monkeypatch.setattr(attention_core.torch, "empty_like", real_empty_like)
     torch.manual_seed(7)   # the same dropout seed for the second module
     out2 = dense(q2, k2, v2, mask, merged_heads=True)
     out2.backward(g)

@@ -346,3 +346,73 @@ def test_masked_softmax_with_attention_dropout_vs_oracle(hotpath, case, pad_batc
     d0, y0 = ext.forward_dropout(x.to(DEV), mask.to(DEV), scale, 0.0, seed)
     plain = ext.forward(x.to(DEV), mask.to(DEV), scale)
     assert torch.equal(d0, y0) and torch.equal(y0, plain)
+
+
+# (attn_batches, seq_len, window, zero_block, variant)
+BLOCK_CASES = [(4, 2048, None, 512, "plain"), (2, 2048, 700, 256, "plain"), (2, 4096, 1000, 1024, "plain"),
+               (1, 8192, 4096, 1024, "plain"), (3, 328, 100, 128, "plain"), (2, 200, None, 64, "plain"),
+               (4, 2048, None, 512, "alibi"), (4, 1024, 300, 128, "lengths"), (2, 2048, 700, 256, "dropout"),
+               (4, 2048, None, 512, "dropout"), (2, 1001, None, 128, "plain"), (2, 64, None, 8, "plain")]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
+@pytest.mark.parametrize("case", BLOCK_CASES, ids=lambda c: f"a{c[0]}_s{c[1]}_w{c[2]}_z{c[3]}_{c[4]}")
+def test_block_limited_causal_softmax_writes_only_what_the_caller_reads(case, dtype):
+    """The zero_block variants (nhp_causal_softmax_blocks_*, nhp_causal_softmax_dropout_blocks_*): inside the range
+    of every row that a block-wise caller reads -- from the block of the first visible key to the block of the
+    diagonal -- bit-identical to the whole-row entry points (which the other tests hold to the oracle); outside of
+    it the output buffer keeps the sentinel it was filled with, i.e. is not written. Rows on the scalar path
+    (seq_len 1001) are written whole."""
+    import scaled_upper_triang_masked_softmax_cuda as ext
+    from megatron.model.fused_softmax import _written_blocks
+
+    a, s, window, zb, variant = case
+    print(f"blocks case {case} {dtype}", flush=True)
+    scale, p, seed = 1 / math.sqrt(128), 0.1, 77
+    x = util.randn((a, s, s), dtype, seed=s, std=2.0).to(DEV)
+    dy = util.randn((a, s, s), dtype, seed=s + 1).to(DEV)
+    kw = {}
+    if variant == "alibi":
+        kw["alibi_slopes"] = torch.tensor(fb.alibi_slopes(4), dtype=torch.float32, device=DEV)
+    if variant == "lengths":
+        kw["key_lengths"] = torch.tensor([700, 1024], dtype=torch.int32, device=DEV)
+    written = _written_blocks(s, zb, window, DEV)
+    if s % 8:
+        written = torch.ones_like(written)
+    # what the rows must hold: everything visible plus the zeros up to the block boundaries
+    visible = ~fb.causal_mask(s, sliding_window_width=window)[0, 0].to(DEV)
+    assert bool((written | ~visible).all())
+    sentinel = 0x7e01   # a NaN pattern in both 16-bit types
+    real_empty = torch.empty_like
+
+    def marked(t, **k):
+        out = real_empty(t, **k)
+        out.view(torch.int16).fill_(sentinel)
+        return out
+
+    def run(zero_block):
+        torch.empty_like = marked
+        try:
+            if variant == "dropout":
+                dropped, y = ext.forward_dropout(x, scale, p, seed, window, zero_block)
+                g = dy.clone()
+                if zero_block and s % 8 == 0:
+                    g.view(torch.int16)[:, ~written] = sentinel
+                dx = ext.backward_dropout(g, y, scale, p, seed, window, zero_block)
+                return dropped, y, dx
+            y = ext.forward(x, scale, window, kw.get("alibi_slopes"), None, kw.get("key_lengths"), zero_block)
+            g = dy.clone()
+            if zero_block and s % 8 == 0:   # the gradient outside the range is the caller's uninitialised memory
+                g.view(torch.int16)[:, ~written] = sentinel
+            dx = ext.backward(g, y, scale, window, kw.get("key_lengths"), zero_block)
+            return y, dx
+        finally:
+            torch.empty_like = real_empty
+
+    whole = run(0)
+    part = run(zb)
+    for got, want in zip(part, whole):
+        assert torch.equal(util.raw_bits(got)[:, written], util.raw_bits(want)[:, written])
+        if not bool(written.all()):
+            assert bool((util.raw_bits(got)[:, ~written] == sentinel).all()), "written outside the range"
+        assert not torch.isnan(got.float()[:, written]).any()
