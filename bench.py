@@ -21,6 +21,9 @@ the drop-in extension modules (which call libneox_hotpath.so):
   rope-kgrad-1.4b  rotary bwd on a gradient [2048,8,16,128] bf16 that is contiguous along the sequence (strides
                  (1, h*d*s, d*s, s)): the layout of the key gradient behind the score GEMM's backward
   mistral-window causal softmax fwd+bwd [64,8192,8192] bf16 with a 4096-key sliding window applied by index
+  causal-blocks-1.4b  causal softmax fwd+bwd [128,2048,2048] bf16 writing only the 512-column blocks on and below the
+                 diagonal (what the blocked attention GEMMs read); mistral-window-blocks: the same for mistral-window,
+                 1024-column blocks
   alibi-1.4b     causal softmax fwd+bwd [128,2048,2048] bf16 with the AliBi bias of 16 heads added in the kernel
   attn-dropout-1.4b  causal softmax + attention dropout (p = 0.1) in one kernel, fwd+bwd [128,2048,2048] bf16
   masked-dropout-c3  padding-masked softmax + attention dropout (p = 0.1) in one kernel, fwd+bwd on the masked-c3 tensors
@@ -194,12 +197,16 @@ def make_workload(name, torch, dev):
                "bytes_convention": "lower-triangle reads, dense writes (two dense outputs in the forward)"}
         return step, kernel_bytes, {}, "softmax_dropout_fwd", "bf16", cfg
 
-    if name in ("mistral-window", "alibi-1.4b", "rpe-bias-1.4b"):
+    if name in ("mistral-window", "alibi-1.4b", "rpe-bias-1.4b", "causal-blocks-1.4b", "mistral-window-blocks"):
         from megatron.model.positional_embeddings import AliBi
 
         bias = None
-        if name == "mistral-window":
+        zero_block = 0
+        if name in ("mistral-window", "mistral-window-blocks"):
             a, s, window, heads = 64, 8192, 4096, None
+            zero_block = 1024 if name.endswith("blocks") else 0
+        elif name == "causal-blocks-1.4b":
+            a, s, window, heads, zero_block = 128, 2048, None, None, 512
         else:
             a, s, window, heads = 128, 2048, None, 16
         scale = 1.0 / math.sqrt(128)
@@ -214,19 +221,27 @@ def make_workload(name, torch, dev):
             dy[i:i + 8] = randn((8, s, s), 1000 + i, torch.bfloat16)
         w = s if window is None else window
         band = sum(min(q, w) + 1 for q in range(s))  # keys read per matrix
-        fwd_b = a * band * 2 + a * s * s * 2
-        bwd_b = 2 * a * band * 2 + a * s * s * 2
+        written = s * s                               # elements written per matrix
+        if zero_block:
+            # every row from the block of the first key its block's first row sees to the block of the diagonal
+            written = sum((q // zero_block + 1) * zero_block - max(0, q // zero_block * zero_block - w) // zero_block * zero_block
+                          for q in range(s))
+        fwd_b = a * band * 2 + a * written * 2
+        bwd_b = 2 * a * band * 2 + a * written * 2
         if bias is not None:
             fwd_b += heads * band * 2  # each head's bias triangle once; the batch re-reads it from cache
         kernel_bytes = {"causal_softmax_fwd": fwd_b, "causal_softmax_bwd": bwd_b}
 
         def step(t):
-            y = t.run("causal_softmax_fwd", lambda: causal_ext.forward(x, scale, window, slopes, bias))
-            t.run("causal_softmax_bwd", lambda: causal_ext.backward(dy, y, scale, window))
+            y = t.run("causal_softmax_fwd", lambda: causal_ext.forward(x, scale, window, slopes, bias, None, zero_block))
+            t.run("causal_softmax_bwd", lambda: causal_ext.backward(dy, y, scale, window, None, zero_block))
 
         cfg = {"workload": name, "scores": [a, s, s], "window": window,
                "alibi_heads": None if slopes is None else heads, "bias": None if bias is None else list(bias.shape),
-               "bytes_convention": "reads of the attended band, dense writes"}
+               "bytes_convention": "reads of the attended band, dense writes" if not zero_block else
+               f"reads of the attended band, writes of the {zero_block}-column blocks a block-wise caller reads"}
+        if zero_block:
+            cfg["zero_block"] = zero_block
         return step, kernel_bytes, {}, "causal_softmax_bwd", "bf16", cfg
 
     if name in ("masked-c3", "masked-dropout-c3"):
