@@ -432,3 +432,32 @@ def test_relative_position_bias_buckets_and_values():
     bias.sum().backward()
     counts = torch.bincount(b.flatten(), minlength=32).float()
     assert torch.allclose(rpe.weight.grad, (counts * 8.0)[:, None].expand(32, 4))
+
+
+def test_causal_gemm_blocks_cover_what_is_visible_and_stay_inside_what_the_softmax_writes():
+    """The contract between the blocked attention GEMMs and the block-limited causal softmax, by brute force: every
+    visible (query, key) pair lies in a row block and in a column block (nothing needed is skipped), and every
+    element a block reads lies in the range the kernel writes for that row (nothing uninitialised is read)."""
+    from megatron.model import attention_core as ac
+    from megatron.model.fused_softmax import _written_blocks
+
+    assert ac.causal_gemm_block(1024) == 0 and ac.causal_gemm_block(2048) == 512 and ac.causal_gemm_block(4096) == 1024
+    for s, blk, window in ((64, 16, None), (64, 16, 5), (64, 16, 16), (64, 16, 17), (64, 16, 40), (72, 16, 20),
+                           (100, 32, 33), (100, 32, 0), (128, 8, 31), (50, 64, 10), (96, 32, 95), (96, 32, 200)):
+        visible = ~fb.causal_mask(s, "cpu", sliding_window_width=window)[0, 0]
+        eff = None if window is None or window >= s else window
+        written = _written_blocks(s, blk, eff, "cpu")
+        rows = torch.zeros((s, s), dtype=torch.bool)
+        for r0, r1, c0 in ac._row_blocks(s, blk, eff):
+            assert 0 <= c0 <= r0 < r1 <= s and c0 % blk == 0
+            rows[r0:r1, c0:r1] = True
+        cols = torch.zeros((s, s), dtype=torch.bool)
+        for c0, c1, r1 in ac._column_blocks(s, blk, eff):
+            assert 0 <= c0 < c1 <= r1 <= s
+            cols[c0:r1, c0:c1] = True
+        case = (s, blk, window)
+        assert bool((rows | ~visible).all()) and bool((cols | ~visible).all()), case     # nothing visible is skipped
+        assert bool((written | ~rows).all()) and bool((written | ~cols).all()), case     # nothing unwritten is read
+        assert bool((written | ~visible).all()), case
+        # and the blocks do save work: no block lies entirely above the diagonal
+        assert not bool(rows[0, blk:].any())
