@@ -22,8 +22,8 @@ the drop-in extension modules (which call libneox_hotpath.so):
                  (1, h*d*s, d*s, s)): the layout of the key gradient behind the score GEMM's backward
   mistral-window causal softmax fwd+bwd [64,8192,8192] bf16 with a 4096-key sliding window applied by index
   causal-blocks-1.4b  causal softmax fwd+bwd [128,2048,2048] bf16 writing only the 512-column blocks on and below the
-                 diagonal (what the blocked attention GEMMs read); mistral-window-blocks: the same for mistral-window,
-                 1024-column blocks
+                 diagonal (what the blocked attention GEMMs read); causal-blocks-7b: [32,4096,4096], 1024-column blocks;
+                 mistral-window-blocks: the same for mistral-window, 1024-column blocks
   alibi-1.4b     causal softmax fwd+bwd [128,2048,2048] bf16 with the AliBi bias of 16 heads added in the kernel
   attn-dropout-1.4b  causal softmax + attention dropout (p = 0.1) in one kernel, fwd+bwd [128,2048,2048] bf16
   masked-dropout-c3  padding-masked softmax + attention dropout (p = 0.1) in one kernel, fwd+bwd on the masked-c3 tensors
@@ -197,7 +197,8 @@ def make_workload(name, torch, dev):
                "bytes_convention": "lower-triangle reads, dense writes (two dense outputs in the forward)"}
         return step, kernel_bytes, {}, "softmax_dropout_fwd", "bf16", cfg
 
-    if name in ("mistral-window", "alibi-1.4b", "rpe-bias-1.4b", "causal-blocks-1.4b", "mistral-window-blocks"):
+    if name in ("mistral-window", "alibi-1.4b", "rpe-bias-1.4b", "causal-blocks-1.4b", "causal-blocks-7b",
+                "mistral-window-blocks"):
         from megatron.model.positional_embeddings import AliBi
 
         bias = None
@@ -207,6 +208,8 @@ def make_workload(name, torch, dev):
             zero_block = 1024 if name.endswith("blocks") else 0
         elif name == "causal-blocks-1.4b":
             a, s, window, heads, zero_block = 128, 2048, None, None, 512
+        elif name == "causal-blocks-7b":
+            a, s, window, heads, zero_block = 32, 4096, None, None, 1024
         else:
             a, s, window, heads = 128, 2048, None, 16
         scale = 1.0 / math.sqrt(128)

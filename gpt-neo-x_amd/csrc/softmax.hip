@@ -762,7 +762,10 @@ enum RowKind { kCausalFwd, kCausalFwdExtra, kCausalBwd, kMaskedFwd, kMaskedBwd }
 //   heads with one decoded mask row (measured at [16,32,1024,2048] fp16: 582 us
 //   with two waves per row and two heads, 615 with four heads, 633 with one,
 //   619 with one wave per row and two heads).
-static bool plan_row(int64_t n, RowKind kind, RowPlan& p)
+// blocks: the block-limited variants (a row's stores end with the block of the diagonal), for which other
+// shapes measured best than for whole rows: two chunks per lane in the backward as well (2048 keys: 312 -> 287 us,
+// 4096: 320 -> 282 us), and four waves of four chunks in the forward at 8192 keys (1508 -> 1243 us with a window).
+static bool plan_row(int64_t n, RowKind kind, RowPlan& p, bool blocks = false)
 {
     if (n < 8 || n % 8 != 0 || n > kMaxResidentRow) return false;
     const int64_t chunks = n / 8;
@@ -788,7 +791,7 @@ static bool plan_row(int64_t n, RowKind kind, RowPlan& p)
         W = 16;
         K = 8;
     } else {
-        K = (kind == kCausalFwd || kind == kCausalFwdExtra || kind == kMaskedFwd) ? 2 : 1;
+        K = (kind == kCausalFwd || kind == kCausalFwdExtra || kind == kMaskedFwd || (blocks && kind == kCausalBwd)) ? 2 : 1;
         while (8 * K < segs) K *= 2;
         static const int kWaves[] = {1, 2, 3, 4, 6, 8};
         W = 8;
@@ -797,6 +800,10 @@ static bool plan_row(int64_t n, RowKind kind, RowPlan& p)
                 W = w;
                 break;
             }
+        if (blocks && (kind == kCausalFwd || kind == kCausalFwdExtra) && segs > 8 && segs <= 16) {
+            K = 4;
+            W = 4;
+        }
     }
     p.W = tune("NHP_W", W);
     p.K = tune("NHP_K", K);
@@ -850,7 +857,7 @@ static int causal_fwd(void* y, const void* x, float scale, int64_t batches, int6
     const uint16_t* bp = static_cast<const uint16_t*>(bias);
     const DropoutKey dk = drop != nullptr ? *drop : DropoutKey{};
     const bool extras = slopes != nullptr || bp != nullptr;  // not dropout: its second output wants the two-wave shape
-    if (plan_row(n, extras ? kCausalFwdExtra : kCausalFwd, p) && aligned16(x) && aligned16(y) && aligned16(bias) &&
+    if (plan_row(n, extras ? kCausalFwdExtra : kCausalFwd, p, zshift != 0) && aligned16(x) && aligned16(y) && aligned16(bias) &&
         aligned16(dropped)) {
 #define CALL(L_, K_, W_)                                                                   \
     {                                                                                      \
@@ -888,7 +895,7 @@ static int softmax_bwd(void* dx, const void* dy, const void* y, float scale, int
     uint16_t* dxp = static_cast<uint16_t*>(dx);
     const uint16_t* dyp = static_cast<const uint16_t*>(dy);
     const uint16_t* yp = static_cast<const uint16_t*>(y);
-    if (plan_row(n, CAUSAL ? kCausalBwd : kMaskedBwd, p) && aligned16(dx) && aligned16(dy) && aligned16(y)) {
+    if (plan_row(n, CAUSAL ? kCausalBwd : kMaskedBwd, p, zshift != 0) && aligned16(dx) && aligned16(dy) && aligned16(y)) {
 #define CALL(L_, K_, W_)                                                                   \
     {                                                                                      \
         using G = Geo<L_, K_, W_, kBlockWaves>;                                            \

@@ -359,30 +359,28 @@ BLOCK_CASES = [(4, 2048, None, 512, "plain"), (2, 2048, 700, 256, "plain"), (2, 
 @pytest.mark.parametrize("case", BLOCK_CASES, ids=lambda c: f"a{c[0]}_s{c[1]}_w{c[2]}_z{c[3]}_{c[4]}")
 def test_block_limited_causal_softmax_writes_only_what_the_caller_reads(case, dtype):
     """The zero_block variants (nhp_causal_softmax_blocks_*, nhp_causal_softmax_dropout_blocks_*): inside the range
-    of every row that a block-wise caller reads -- from the block of the first visible key to the block of the
-    diagonal -- bit-identical to the whole-row entry points (which the other tests hold to the oracle); outside of
-    it the output buffer keeps the sentinel it was filled with, i.e. is not written. Rows on the scalar path
-    (seq_len 1001) are written whole."""
+    of every row that a block-wise caller reads -- from the block of the first key that the first row of the row's
+    block sees to the block of the diagonal -- the oracle's values to the tolerances of the whole-row entry points
+    (masked positions exactly +0); outside of it the output buffer keeps the sentinel it was filled with, i.e. is
+    not written, and sentinels (NaN patterns) planted there in the inputs of the backward do no harm. Rows on the
+    scalar path (seq_len 1001) are written whole."""
     import scaled_upper_triang_masked_softmax_cuda as ext
     from megatron.model.fused_softmax import _written_blocks
 
     a, s, window, zb, variant = case
     print(f"blocks case {case} {dtype}", flush=True)
     scale, p, seed = 1 / math.sqrt(128), 0.1, 77
-    x = util.randn((a, s, s), dtype, seed=s, std=2.0).to(DEV)
-    dy = util.randn((a, s, s), dtype, seed=s + 1).to(DEV)
-    kw = {}
+    x = util.randn((a, s, s), dtype, seed=s, std=2.0)
+    dy = util.randn((a, s, s), dtype, seed=s + 1)
+    slopes = lengths = None
     if variant == "alibi":
-        kw["alibi_slopes"] = torch.tensor(fb.alibi_slopes(4), dtype=torch.float32, device=DEV)
+        slopes = torch.tensor(fb.alibi_slopes(4), dtype=torch.float32)
     if variant == "lengths":
-        kw["key_lengths"] = torch.tensor([700, 1024], dtype=torch.int32, device=DEV)
-    written = _written_blocks(s, zb, window, DEV)
-    if s % 8:
-        written = torch.ones_like(written)
-    # what the rows must hold: everything visible plus the zeros up to the block boundaries
-    visible = ~fb.causal_mask(s, sliding_window_width=window)[0, 0].to(DEV)
-    assert bool((written | ~visible).all())
-    sentinel = 0x7e01   # a NaN pattern in both 16-bit types
+        lengths = torch.tensor([700, 1024], dtype=torch.int32)
+    written = _written_blocks(s, zb, window, "cpu") if s % 8 == 0 else torch.ones((s, s), dtype=torch.bool)
+    masked = fb.causal_mask(s, sliding_window_width=window)[0, 0]
+    assert bool((written | masked).all())          # everything visible lies inside the written range
+    sentinel = 0x7e01                              # a NaN pattern in both 16-bit types
     real_empty = torch.empty_like
 
     def marked(t, **k):
@@ -390,29 +388,43 @@ def test_block_limited_causal_softmax_writes_only_what_the_caller_reads(case, dt
         out.view(torch.int16).fill_(sentinel)
         return out
 
-    def run(zero_block):
-        torch.empty_like = marked
-        try:
-            if variant == "dropout":
-                dropped, y = ext.forward_dropout(x, scale, p, seed, window, zero_block)
-                g = dy.clone()
-                if zero_block and s % 8 == 0:
-                    g.view(torch.int16)[:, ~written] = sentinel
-                dx = ext.backward_dropout(g, y, scale, p, seed, window, zero_block)
-                return dropped, y, dx
-            y = ext.forward(x, scale, window, kw.get("alibi_slopes"), None, kw.get("key_lengths"), zero_block)
-            g = dy.clone()
-            if zero_block and s % 8 == 0:   # the gradient outside the range is the caller's uninitialised memory
-                g.view(torch.int16)[:, ~written] = sentinel
-            dx = ext.backward(g, y, scale, window, kw.get("key_lengths"), zero_block)
-            return y, dx
-        finally:
-            torch.empty_like = real_empty
+    def planted(t):                                # the caller's uninitialised memory outside the range
+        t = t.clone()
+        t.view(torch.int16)[:, ~written] = sentinel
+        return t.to(DEV)
 
-    whole = run(0)
-    part = run(zb)
-    for got, want in zip(part, whole):
-        assert torch.equal(util.raw_bits(got)[:, written], util.raw_bits(want)[:, written])
+    def check_range(got, what):
+        got = got.cpu()
         if not bool(written.all()):
-            assert bool((util.raw_bits(got)[:, ~written] == sentinel).all()), "written outside the range"
-        assert not torch.isnan(got.float()[:, written]).any()
+            assert bool((util.raw_bits(got)[:, ~written] == sentinel).all()), f"{what}: written outside the range"
+        zeros = written & masked
+        assert int(util.raw_bits(got)[:, zeros].abs().max() if zeros.any() else 0) == 0, f"{what}: zeros"
+        return got
+
+    def inside(got, want):                         # the oracle's values where nothing was written
+        return torch.where(written, got, want)
+
+    dl = None if lengths is None else lengths.to(DEV)
+    want_y = oracle.causal_softmax_fwd(x, scale, window=window, alibi_slopes=slopes, key_lengths=lengths)
+    torch.empty_like = marked
+    try:
+        if variant == "dropout":
+            dropped, y = ext.forward_dropout(x.to(DEV), scale, p, seed, window, zb)
+            dropped, y = check_range(dropped, "dropped"), check_range(y, "y")
+            util.assert_ulp_close(inside(y, want_y), want_y, 2, "y")
+            want_dropped = oracle.bias_dropout_add(inside(y, want_y), None, None, p, seed)
+            assert torch.equal(util.raw_bits(dropped)[:, written], util.raw_bits(want_dropped)[:, written])
+            dx = check_range(ext.backward_dropout(planted(dy), planted(want_y), scale, p, seed, window, zb), "dx")
+            want_dx = oracle.causal_softmax_dropout_bwd(dy, want_y, scale, p, seed, window=window)
+            g = oracle.bias_dropout_add(dy, None, None, p, seed)
+        else:
+            y = check_range(ext.forward(x.to(DEV), scale, window, None if slopes is None else slopes.to(DEV), None, dl,
+                                        zb), "y")
+            util.assert_ulp_close(inside(y, want_y), want_y, 2, "y")
+            dx = check_range(ext.backward(planted(dy), planted(want_y), scale, window, dl, zb), "dx")
+            want_dx = oracle.softmax_bwd(dy, want_y, scale, causal=True, window=window, key_lengths=lengths)
+            g = dy
+    finally:
+        torch.empty_like = real_empty
+    dead = want_y == 0                              # masked by the triangle, the window or the key lengths
+    util.assert_softmax_bwd_close(inside(dx, want_dx), want_dx, g.masked_fill(dead, 0), want_y, scale, "dx")
