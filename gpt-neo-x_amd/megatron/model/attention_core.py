@@ -198,7 +198,9 @@ class CoreAttention(torch.nn.Module):
             gradients of q and k. None (default): fold unless the scores are fp16 (there the scaled GEMM is
             what keeps them in range, the reason the reference scales twice) or the softmax is not in fp32.
         causal_gemm_blocks: with the causal kernel and sequences of 2048 positions or more, compute the two GEMMs
-            (and the four of the backward) only on and below the diagonal blocks.
+            (and the four of the backward) only on and below the diagonal blocks. The skipped parts of the score
+            and probability tensors and of their gradients stay uninitialised; switch this off for tools that
+            inspect those tensors (e.g. autograd's anomaly detection would report the stale NaN patterns in them).
     """
 
     def __init__(self, head_dim, layer_number, fp16, bf16, fusion_type, mask_func, attention_softmax_in_fp32=False,

@@ -461,3 +461,26 @@ def test_causal_gemm_blocks_cover_what_is_visible_and_stay_inside_what_the_softm
         assert bool((written | ~visible).all()), case
         # and the blocks do save work: no block lies entirely above the diagonal
         assert not bool(rows[0, blk:].any())
+
+
+def test_attention_mask_producers():
+    """get_attn_mask / get_ltor_masks_and_position_ids (megatron/utils.py:67-110): tril of ones, with a window
+    triu(diagonal=-width) of it, "< 0.5" -- written out with torch's own tril / triu here."""
+    from megatron.model.utils import get_fusion_type
+    from megatron.utils import get_attn_mask, get_ltor_masks_and_position_ids
+
+    assert callable(get_fusion_type)
+    for s, width in ((1, None), (7, None), (16, 0), (16, 3), (16, 15), (16, 40), (33, 8)):
+        ones = torch.tril(torch.ones((1, s, s))).view(1, 1, s, s)
+        if width is not None:
+            ones = torch.triu(ones, diagonal=-width)
+        want = ones < 0.5
+        got = get_attn_mask(s, "cpu", width)
+        assert got.dtype == torch.bool and got.shape == (1, 1, s, s) and torch.equal(got, want), (s, width)
+        assert torch.equal(got, fb.causal_mask(s, "cpu", sliding_window_width=width))
+    data = torch.tensor([[5, 0, 7, 0], [1, 2, 3, 4]])
+    mask, loss, pos = get_ltor_masks_and_position_ids(data, eod_token=0, eod_mask_loss=True, sliding_window_width=2)
+    assert torch.equal(mask, get_attn_mask(4, "cpu", 2))
+    assert torch.equal(loss, torch.tensor([[1.0, 0.0, 1.0, 0.0], [1.0, 1.0, 1.0, 1.0]]))
+    assert torch.equal(pos, torch.tensor([[0, 1, 2, 3], [0, 1, 2, 3]]))
+    assert get_ltor_masks_and_position_ids(data, 0)[1].sum() == 8
