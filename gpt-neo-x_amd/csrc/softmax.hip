@@ -762,9 +762,11 @@ enum RowKind { kCausalFwd, kCausalFwdExtra, kCausalBwd, kMaskedFwd, kMaskedBwd }
 //   heads with one decoded mask row (measured at [16,32,1024,2048] fp16: 582 us
 //   with two waves per row and two heads, 615 with four heads, 633 with one,
 //   619 with one wave per row and two heads).
-// blocks: the block-limited variants (a row's stores end with the block of the diagonal), for which other
-// shapes measured best than for whole rows: two chunks per lane in the backward as well (2048 keys: 312 -> 287 us,
-// 4096: 320 -> 282 us), and four waves of four chunks in the forward at 8192 keys (1508 -> 1243 us with a window).
+// The causal backward takes two chunks per lane like the forward kernels (measured by alternating shapes on the
+// same tensors: 4096 keys 350 -> 346 us), and at 2048 keys three waves per row, the first of which holds two of
+// the row's four segments (343 -> 335 us; block-limited 300 -> 282 us).
+// blocks: the block-limited variants (a row's stores end with the block of the diagonal): four waves of four
+// chunks in the forward at 8192 keys (1508 -> 1243 us with a window).
 static bool plan_row(int64_t n, RowKind kind, RowPlan& p, bool blocks = false)
 {
     if (n < 8 || n % 8 != 0 || n > kMaxResidentRow) return false;
@@ -791,7 +793,7 @@ static bool plan_row(int64_t n, RowKind kind, RowPlan& p, bool blocks = false)
         W = 16;
         K = 8;
     } else {
-        K = (kind == kCausalFwd || kind == kCausalFwdExtra || kind == kMaskedFwd || (blocks && kind == kCausalBwd)) ? 2 : 1;
+        K = (kind == kCausalFwd || kind == kCausalFwdExtra || kind == kMaskedFwd || kind == kCausalBwd) ? 2 : 1;
         while (8 * K < segs) K *= 2;
         static const int kWaves[] = {1, 2, 3, 4, 6, 8};
         W = 8;
@@ -800,6 +802,7 @@ static bool plan_row(int64_t n, RowKind kind, RowPlan& p, bool blocks = false)
                 W = w;
                 break;
             }
+        if (kind == kCausalBwd && segs == 4) W = 3;
         if (blocks && (kind == kCausalFwd || kind == kCausalFwdExtra) && segs > 8 && segs <= 16) {
             K = 4;
             W = 4;
