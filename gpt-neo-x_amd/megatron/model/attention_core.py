@@ -283,8 +283,8 @@ class CoreAttention(torch.nn.Module):
         """Block size for the blocked causal GEMMs, 0 when the scores do not go to the causal kernel (which is what
         guarantees that nothing above the diagonal is read or left non-zero) or are too small to gain."""
         softmax = self.scale_mask_softmax
-        if not self.causal_gemm_blocks or sq != sk or not like.is_cuda or self.use_cache:
-            return 0
+        if not self.causal_gemm_blocks or sq != sk or not like.is_cuda:
+            return 0   # (with cached keys sq != sk except for the first call, which is an ordinary causal pass)
         if not (softmax.upper_triang_mask_fusion and softmax.is_kernel_available(attention_mask, b, np_, sq, sk)):
             return 0
         return causal_gemm_block(sq)

@@ -428,3 +428,47 @@ def test_block_limited_causal_softmax_writes_only_what_the_caller_reads(case, dt
         torch.empty_like = real_empty
     dead = want_y == 0                              # masked by the triangle, the window or the key lengths
     util.assert_softmax_bwd_close(inside(dx, want_dx), want_dx, g.masked_fill(dead, 0), want_y, scale, "dx")
+
+
+def test_block_limited_causal_softmax_at_full_size():
+    """[128, 2048, 2048] bf16 (the Pythia-1.4B scores), blocks of 512: inside the written range the forward equals
+    the whole-row kernel bit for bit (same launch shape), every row sums to 1, the backward stays within the
+    tolerance of the whole-row backward (its row sums are formed by three waves instead of four), and the rest of
+    both outputs is left untouched."""
+    import scaled_upper_triang_masked_softmax_cuda as ext
+    from megatron.model.fused_softmax import _written_blocks
+
+    a, s, zb = 128, 2048, 512
+    scale = 1 / math.sqrt(128)
+    gen = torch.Generator(device=DEV).manual_seed(3)
+    x = (2 * torch.randn((a, s, s), generator=gen, device=DEV)).bfloat16()
+    dy = torch.randn((a, s, s), generator=gen, device=DEV).bfloat16()
+    written = _written_blocks(s, zb, None, DEV)
+    whole = ext.forward(x, scale)
+    real_empty = torch.empty_like
+    sentinel = 0x7e01
+
+    def marked(t, **k):
+        out = real_empty(t, **k)
+        out.view(torch.int16).fill_(sentinel)
+        return out
+
+    torch.empty_like = marked
+    try:
+        part = ext.forward(x, scale, None, None, None, None, zb)
+    finally:
+        torch.empty_like = real_empty
+    bits, want = part.view(torch.int16), whole.view(torch.int16)
+    assert bool(torch.where(written, bits == want, bits == sentinel).all())
+    sums = torch.where(written, part.float(), torch.zeros((), device=DEV)).sum(-1)
+    assert (sums - 1).abs().max().item() < 2048 * 2.0 ** -9
+    g = dy.clone()
+    g.view(torch.int16)[:, ~written] = sentinel           # the caller's uninitialised memory
+    got = ext.backward(g, part, scale, None, None, zb)      # in place on g
+    ref = ext.backward(dy.clone(), whole, scale)
+    gb = got.view(torch.int16)
+    assert bool((gb[:, ~written] == sentinel).all())
+    diff = torch.where(written, (got.float() - ref.float()).abs(), torch.zeros((), device=DEV))
+    bound = torch.where(written, ref.float().abs() * 2.0 ** -7 + 1e-6, torch.ones((), device=DEV))
+    assert bool((diff <= bound).all())
+    assert int(gb[:, written & (torch.arange(s, device=DEV)[None, :] > torch.arange(s, device=DEV)[:, None])].abs().max()) == 0
