@@ -31,7 +31,7 @@ def args_for(**kw):
                 scaled_masked_softmax_fusion=False, attention_softmax_in_fp32=True, apply_query_key_layer_scaling=False,
                 attention_dropout=0.0, hidden_dropout=0.0, bias_dropout_fusion=True, gpt_j_residual=False,
                 gpt_j_tied=False, use_bias_in_mlp=True, use_bias_in_attn_linear=True, intermediate_size=None,
-                expansion_factor=None, num_kv_heads=None)
+                expansion_factor=None, num_kv_heads=None, sliding_window_width=None)
     base.update(kw)
     return types.SimpleNamespace(**base)
 
@@ -99,7 +99,8 @@ def rel_err(a, b):
     return ((a.float() - b.float()).norm() / b.float().norm()).item()
 
 
-@pytest.mark.parametrize("variant", ["pythia", "sequential", "llama", "gqa", "gqa-eager-rope", "rpe"])
+@pytest.mark.parametrize("variant", ["pythia", "sequential", "llama", "gqa", "gqa-eager-rope", "rpe", "pythia-2048",
+                                     "mistral-2048"])
 def test_layer_matches_plain_torch(variant):
     from megatron.model.transformer_layer import TransformerLayer
 
@@ -110,7 +111,12 @@ def test_layer_matches_plain_torch(variant):
            "gqa": args_for(norm="rmsnorm", activation="swiglu", rotary_pct=1.0, use_bias_in_mlp=False,
                            use_bias_in_attn_linear=False, num_kv_heads=2),
            "gqa-eager-rope": args_for(num_kv_heads=4, rope_fusion=False),
-           "rpe": args_for(pos_emb="rpe")}[variant]
+           "rpe": args_for(pos_emb="rpe"),
+           # 2048 positions: the attention GEMMs and the softmax work on the blocks below the diagonal only
+           "pythia-2048": args_for(gpt_j_residual=True, seq_length=2048),
+           "mistral-2048": args_for(norm="rmsnorm", activation="swiglu", rotary_pct=1.0, use_bias_in_mlp=False,
+                                    use_bias_in_attn_linear=False, num_kv_heads=2, seq_length=2048,
+                                    sliding_window_width=700)}[variant]
     torch.manual_seed(0)
     rpe = None
     if variant == "rpe":   # T5 relative position bias shared by the layers, added inside the softmax kernel
@@ -123,10 +129,12 @@ def test_layer_matches_plain_torch(variant):
             if p.dim() == 1:
                 p.add_(0.1 * torch.randn_like(p))
     layer = layer.to(torch.bfloat16)
-    s, b, h = 256, 2, cfg.hidden_size
+    s, b, h = cfg.seq_length, 2, cfg.hidden_size
     x = util.randn((s, b, h), torch.bfloat16, seed=1).to(DEV).requires_grad_(True)
     g = util.randn((s, b, h), torch.bfloat16, seed=2).to(DEV)
-    mask = fb.causal_mask(s, DEV)
+    mask = fb.causal_mask(s, DEV, sliding_window_width=getattr(cfg, "sliding_window_width", None))
+    if s >= 2048:
+        assert layer.attention.core._causal_block(mask, b, cfg.num_attention_heads, s, s, x) == 512
     layer.train()
     out = layer(x, mask)
     assert out.shape == (s, b, h) and out.dtype == torch.bfloat16
