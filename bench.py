@@ -33,6 +33,7 @@ the drop-in extension modules (which call libneox_hotpath.so):
   swiglu-7b      SwiGLU forward and backward on the Llama-2 7B MLP activation [4096*4, 2*11008] -> [4096*4, 11008] bf16
   bias-residual-1.4b  residual + (x + bias) on the hidden state [2048*8, 2048] bf16
   bias-dropout-add-1.4b  residual + dropout(x + bias) with p = 0.1, and the dropout backward, same shape
+  bias-residual-pair-1.4b  residual + ((x1 + bias1) + (x2 + bias2)): the parallel-residual layer's three additions in one pass
   layernorm-1.4b  LayerNorm fwd and bwd (with the parameter gradients) on the hidden state [2048*8, 2048] bf16
   layernorm-pair-1.4b  the two LayerNorms of the parallel-residual layer in one launch each way, same hidden state
   rmsnorm-7b     RMSNorm fwd and bwd on [4096*4, 4096] bf16 (the Llama-2 7B hidden size)
@@ -493,6 +494,29 @@ def make_workload(name, torch, dev):
 
         cfg = {"workload": name, "hidden_state": [rows, cols], "dropout": 0.1, "mask": "regenerated (Philox4x32-10), not stored"}
         return step, kernel_bytes, {}, "bias_dropout_add", "bf16", cfg
+
+    if name == "bias-residual-pair-1.4b":
+        from megatron.fused_kernels import _hotpath as hp
+
+        lib = hp.lib()
+        rows, cols = 2048 * 8, 2048
+        sets = [tuple(randn((rows, cols), 10 * i + j, torch.bfloat16, 2.0) for j in range(3)) for i in range(5)]
+        b1, b2 = randn((cols,), 7, torch.bfloat16), randn((cols,), 8, torch.bfloat16)
+        out = torch.empty_like(sets[0][0])
+        kernel_bytes = {"bias_add_residual_pair": 4 * rows * cols * 2 + 2 * cols * 2}
+        state = {"i": 0}
+        stream = hp.stream_of(out)
+
+        def step(t):
+            x1, x2, res = sets[state["i"] % len(sets)]
+            state["i"] += 1
+            t.run("bias_add_residual_pair", lambda: hp.check(lib.nhp_bias_add_residual_pair(
+                out.data_ptr(), x1.data_ptr(), b1.data_ptr(), x2.data_ptr(), b2.data_ptr(), res.data_ptr(), rows, cols,
+                hp.BF16, stream), "bias_add_residual_pair"))
+
+        cfg = {"workload": name, "hidden_state": [rows, cols],
+               "bytes_convention": "three tensors read, one written, the two biases"}
+        return step, kernel_bytes, {}, "bias_add_residual_pair", "bf16", cfg
 
     if name == "bias-residual-1.4b":
         from megatron.model.fused_bias_dropout import bias_dropout_add_fused_inference

@@ -208,6 +208,93 @@ pointwise_scalar_kernel(void* out, const void* a, const void* b, const void* bia
     Elt<DT>::store(out, (int64_t)i, point_op<OP>(fa, fb, bv, has_b));
 }
 
+// ---------------------------------------------------------------------------
+// The three bias_dropout_add calls of the parallel-residual layer (dropout off) in one pass, each call
+// evaluated in fp32 and rounded once like nhp_bias_add_residual:
+//   t1 = round(x1 + bias1), t3 = round(t1 + (x2 + bias2)), out = round(residual + t3).
+// One step per workgroup, the tile shape of pointwise_kernel.
+// ---------------------------------------------------------------------------
+template <int DT>
+__device__ __forceinline__ void round_chunk(float (&v)[Elt<DT>::kVec])
+{
+    if constexpr (DT != NHP_F32) {
+        const u32x4 packed = float_to_chunk<DT>(v);
+        chunk_to_float<DT>(packed, v);
+    }
+}
+
+template <int DT, int TW, int U>
+__global__ void __launch_bounds__(kPwThreads)
+residual_pair_kernel(void* out, const void* x1, const void* bias1, const void* x2, const void* bias2,
+                     const void* residual, uint32_t rows, uint32_t cpr)
+{
+    constexpr int V = Elt<DT>::kVec;
+    constexpr int TR = kPwThreads / TW;
+    using S = typename Elt<DT>::storage;
+    const uint32_t tc = threadIdx.x % TW;
+    const uint32_t tr = threadIdx.x / TW;
+    const uint32_t cc = blockIdx.x * TW + tc;
+    if (cc >= cpr) return;
+    const size_t row_elems = (size_t)cpr * V;
+    u32x4 r1[U], r2[U], rr[U];
+    const uint32_t r = blockIdx.y * (TR * U) + tr;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const uint32_t row = r + u * TR;
+        const size_t off = (size_t)row * row_elems + (size_t)cc * V;
+        r1[u] = r2[u] = rr[u] = u32x4{0, 0, 0, 0};
+        if (row < rows) {
+            r1[u] = load16_stream(static_cast<const S*>(x1) + off);
+            r2[u] = load16_stream(static_cast<const S*>(x2) + off);
+            rr[u] = load16_stream(static_cast<const S*>(residual) + off);
+        }
+    }
+    float b1[V], b2[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) b1[j] = b2[j] = 0.0f;
+    if (bias1 != nullptr) chunk_to_float<DT>(load16(static_cast<const S*>(bias1) + (size_t)cc * V), b1);
+    if (bias2 != nullptr) chunk_to_float<DT>(load16(static_cast<const S*>(bias2) + (size_t)cc * V), b2);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const uint32_t row = r + u * TR;
+        if (row < rows) {
+            float t1[V], t2[V], fr[V];
+            chunk_to_float<DT>(r1[u], t1);
+            chunk_to_float<DT>(r2[u], t2);
+            chunk_to_float<DT>(rr[u], fr);
+            if (bias1 != nullptr) {
+#pragma unroll
+                for (int j = 0; j < V; ++j) t1[j] = t1[j] + b1[j];
+                round_chunk<DT>(t1);
+            }
+#pragma unroll
+            for (int j = 0; j < V; ++j) t1[j] = t1[j] + (t2[j] + b2[j]);
+            round_chunk<DT>(t1);
+#pragma unroll
+            for (int j = 0; j < V; ++j) t1[j] = fr[j] + t1[j];
+            store16_stream(static_cast<S*>(out) + (size_t)row * row_elems + (size_t)cc * V, float_to_chunk<DT>(t1));
+        }
+    }
+}
+
+template <int DT>
+__global__ void __launch_bounds__(kPwThreads)
+residual_pair_scalar_kernel(void* out, const void* x1, const void* bias1, const void* x2, const void* bias2,
+                            const void* residual, uint64_t total, uint64_t cols)
+{
+    const uint64_t i = (uint64_t)blockIdx.x * kPwThreads + threadIdx.x;
+    if (i >= total) return;
+    auto rounded = [](float v) {
+        typename Elt<DT>::storage tmp;
+        Elt<DT>::store(&tmp, 0, v);
+        return Elt<DT>::load(&tmp, 0);
+    };
+    float t1 = Elt<DT>::load(x1, (int64_t)i), t2 = Elt<DT>::load(x2, (int64_t)i);
+    if (bias1 != nullptr) t1 = rounded(t1 + Elt<DT>::load(bias1, (int64_t)(i % cols)));
+    if (bias2 != nullptr) t2 = t2 + Elt<DT>::load(bias2, (int64_t)(i % cols));
+    Elt<DT>::store(out, (int64_t)i, Elt<DT>::load(residual, (int64_t)i) + rounded(t1 + t2));
+}
+
 // one thread per column, rows in order (used after the scalar kernel has stored dx)
 template <int DT>
 __global__ void __launch_bounds__(kPwThreads)
@@ -349,6 +436,40 @@ static int run_pointwise(void* out, const void* a, const void* b, const void* bi
     return launch_result();
 }
 
+template <int DT>
+static int run_residual_pair(void* out, const void* x1, const void* bias1, const void* x2, const void* bias2,
+                             const void* residual, int64_t rows, int64_t cols, hipStream_t st)
+{
+    constexpr int V = Elt<DT>::kVec;
+    const bool chunked = cols % V == 0 && ptr_aligned16(out) && ptr_aligned16(x1) && ptr_aligned16(x2) &&
+                         ptr_aligned16(residual) && ptr_aligned16(bias1) && ptr_aligned16(bias2) &&
+                         rows < ((int64_t)1 << 31) && cols / V < ((int64_t)1 << 31);
+    if (chunked) {
+        const int64_t cpr = cols / V;
+        const TilePlan p = plan_tiles(rows, cpr, false);
+        if (p.steps > 65535u || !grid_fits((int64_t)p.col_tiles * p.steps, kPwThreads)) return NHP_ERR_SHAPE;
+        const dim3 grid(p.col_tiles, p.steps);
+#define CASE(TW_)                                                                                   \
+    case TW_:                                                                                       \
+        residual_pair_kernel<DT, TW_, kPwU><<<grid, kPwThreads, kPwLdsTwoInputs, st>>>(             \
+            out, x1, bias1, x2, bias2, residual, (uint32_t)rows, (uint32_t)cpr);                    \
+        break;
+        switch (p.tw) {
+            CASE(1) CASE(2) CASE(4) CASE(8) CASE(16) CASE(32) CASE(64)
+        default:
+            return NHP_ERR_SHAPE;
+        }
+#undef CASE
+        return launch_result();
+    }
+    const int64_t total = rows * cols;
+    const int64_t blocks = (total + kPwThreads - 1) / kPwThreads;
+    if (!grid_fits(blocks, kPwThreads)) return NHP_ERR_SHAPE;
+    residual_pair_scalar_kernel<DT><<<(uint32_t)blocks, kPwThreads, 0, st>>>(out, x1, bias1, x2, bias2, residual,
+                                                                            (uint64_t)total, (uint64_t)cols);
+    return launch_result();
+}
+
 template <int OP>
 static int dispatch_pointwise(void* out, const void* a, const void* b, const void* bias, void* dbias,
                               float* workspace, int64_t rows, int64_t cols, int dtype, hipStream_t st)
@@ -435,6 +556,23 @@ int nhp_bias_add_residual(void* out, const void* x, const void* bias, const void
     if (!out || !x) return NHP_ERR_NULL;
     return dispatch_pointwise<kBiasAddResidual>(out, x, residual, bias, nullptr, nullptr, rows, cols, dtype,
                                                 static_cast<hipStream_t>(stream));
+}
+
+int nhp_bias_add_residual_pair(void* out, const void* x1, const void* bias1, const void* x2, const void* bias2,
+                               const void* residual, int64_t rows, int64_t cols, int dtype, void* stream)
+{
+    if (int rc = check_shape(rows, cols, dtype)) return rc;
+    if (rows == 0 || cols == 0) return NHP_OK;
+    if (!out || !x1 || !x2 || !residual) return NHP_ERR_NULL;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+    case NHP_F16:
+        return run_residual_pair<NHP_F16>(out, x1, bias1, x2, bias2, residual, rows, cols, st);
+    case NHP_BF16:
+        return run_residual_pair<NHP_BF16>(out, x1, bias1, x2, bias2, residual, rows, cols, st);
+    default:
+        return run_residual_pair<NHP_F32>(out, x1, bias1, x2, bias2, residual, rows, cols, st);
+    }
 }
 
 }  // extern "C"

@@ -64,6 +64,7 @@ def _declare(lib):
         "nhp_bias_gelu_bwd": ([vp, vp, vp, vp, vp, vp, i64, i64, ci, vp], ci),
         "nhp_bias_gelu_bwd_workspace_bytes": ([i64, i64, ci], i64),
         "nhp_bias_add_residual": ([vp, vp, vp, vp, i64, i64, ci, vp], ci),
+        "nhp_bias_add_residual_pair": ([vp, vp, vp, vp, vp, vp, i64, i64, ci, vp], ci),
         "nhp_bias_dropout_add": ([vp, vp, vp, vp, i64, i64, f32, u64, u64, ci, vp], ci),
         "nhp_dropout_bwd": ([vp, vp, i64, i64, f32, u64, u64, ci, vp], ci),
         "nhp_philox4x32_10": ([pu32, pu32, pu32], None),

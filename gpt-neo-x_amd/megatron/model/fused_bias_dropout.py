@@ -101,6 +101,52 @@ class _BiasAddResidual(torch.autograd.Function):
         return grad, gb, grad if ctx.needs_input_grad[2] else None
 
 
+class _BiasAddResidualPair(torch.autograd.Function):
+    """``residual + ((x1 + bias1) + (x2 + bias2))`` in one pass, rounded as the three separate additions round.
+    The gradient passes through unchanged to ``x1``, ``x2`` and ``residual``; the two biases share one sum of it
+    over the rows."""
+
+    @staticmethod
+    def forward(ctx, x1, bias1, x2, bias2, residual):
+        what = "bias_add_residual_pair"
+        a, b1, res, rows, cols, exp1 = _prepare(x1, bias1, residual, what)
+        if res is None:
+            raise RuntimeError(f"{what}: a residual is required")
+        if x2.shape != x1.shape or x2.dtype != x1.dtype:
+            raise RuntimeError(f"{what}: x1 and x2 must have the same shape and dtype")
+        _hp.require_gpu(x2, what)
+        b2, exp2 = _bias_vector(bias2, x2, what)
+        c = x2.contiguous()
+        out = torch.empty_like(a)
+        with _hp.device_guard(a):
+            rc = _hp.lib().nhp_bias_add_residual_pair(
+                out.data_ptr(), a.data_ptr(), None if b1 is None else b1.data_ptr(), c.data_ptr(),
+                None if b2 is None else b2.data_ptr(), res.data_ptr(), rows, cols, _hp.dtype_code(a, what),
+                _hp.stream_of(a))
+        _hp.check(rc, what)
+        ctx.conf = (None if bias1 is None else bias1.shape, exp1, None if bias2 is None else bias2.shape, exp2)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad):
+        shape1, exp1, shape2, exp2 = ctx.conf
+        need1 = shape1 is not None and ctx.needs_input_grad[1]
+        need2 = shape2 is not None and ctx.needs_input_grad[3]
+        summed = _column_sum(grad) if (need1 and not exp1) or (need2 and not exp2) else None
+        g1 = (grad if exp1 else summed.view(shape1)) if need1 else None
+        g2 = (grad if exp2 else summed.view(shape2)) if need2 else None
+        return grad, g1, grad, g2, grad if ctx.needs_input_grad[4] else None
+
+
+def bias_add_residual_pair(x1: Tensor, bias1: Optional[Tensor], x2: Tensor, bias2: Optional[Tensor],
+                           residual: Tensor) -> Tensor:
+    """``residual + ((x1 + bias1) + (x2 + bias2))``: how the parallel-residual layer combines the outputs of its
+    attention and MLP branches (three ``bias_dropout_add`` calls in ParallelTransformerLayer.forward,
+    megatron/model/transformer.py:1229-1250) when dropout is off, in one kernel and with the reference's
+    roundings."""
+    return _BiasAddResidualPair.apply(x1, bias1, x2, bias2, residual)
+
+
 class _BiasDropoutAdd(torch.autograd.Function):
     """``residual + dropout(x + bias)`` with the mask regenerated from (seed, prob) in the backward."""
 

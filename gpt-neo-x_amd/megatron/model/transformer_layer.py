@@ -28,7 +28,8 @@ import torch.nn.functional as F
 from .activations import Gated_Activation, get_activation
 from .attention_core import (CoreAttention, apply_rotary_to_query_key, get_fusion_type, split_gqa_and_rotate,
                              split_qkv_and_rotate)
-from .fused_bias_dropout import bias_dropout_add_fused_inference, bias_dropout_add_fused_train, get_bias_dropout_add
+from .fused_bias_dropout import (bias_add_residual_pair, bias_dropout_add_fused_inference, bias_dropout_add_fused_train,
+                                 get_bias_dropout_add)
 from .norms import get_norm, layer_norm_pair
 from .positional_embeddings import AliBi, RotaryEmbedding
 
@@ -213,6 +214,10 @@ class TransformerLayer(torch.nn.Module):
             else:
                 x1, x2 = layer_norm_pair(x, self.input_layernorm, self.post_attention_layernorm)
             attention_output, attention_bias = self._attend(x1, attention_mask, layer_past)
+            if self.bias_dropout_fusion and (self.hidden_dropout == 0.0 or not self.training):
+                # no dropout: attention branch + MLP branch + residual in one pass
+                mlp_output, mlp_bias = self.mlp(x2)
+                return bias_add_residual_pair(attention_output, attention_bias, mlp_output, mlp_bias, residual)
             if attention_bias is not None:
                 attention_output = bias_dropout_fn(attention_output, bias=attention_bias, residual=None,
                                                    prob=self.hidden_dropout)

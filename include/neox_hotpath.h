@@ -415,6 +415,22 @@ int nhp_bias_add_residual(void* out, const void* x, const void* bias, const void
                           int64_t rows, int64_t cols, int dtype, void* stream);
 
 /*
+ * out = residual + ((x1 + bias1) + (x2 + bias2)), rounded where three nhp_bias_add_residual calls round
+ * (t1 = round(x1 + bias1), t3 = round(t1 + (x2 + bias2)), out = round(residual + t3)):
+ * the three element-wise passes with which the parallel-residual layer combines its two branches
+ *   attention_output = bias_dropout_fn(attention_output, attention_bias, residual=None)
+ *   output           = bias_dropout_fn(mlp_output, mlp_bias, residual=attention_output)
+ *   output           = residual + output
+ * (ParallelTransformerLayer.forward with gpt_j_residual, megatron/model/transformer.py:1229-1250,
+ * on bias_dropout_add, megatron/model/fused_bias_dropout.py:28-60) in one, with dropout off; the result
+ * is bit for bit that of three nhp_bias_add_residual calls. bias1 and bias2 may each be NULL (without
+ * bias1 there is no first rounding); out may alias x1, x2 or residual.
+ */
+int nhp_bias_add_residual_pair(void* out, const void* x1, const void* bias1, const void* x2,
+                               const void* bias2, const void* residual, int64_t rows, int64_t cols,
+                               int dtype, void* stream);
+
+/*
  * bias_dropout_add with dropout active (training and 0 < p < 1):
  *   out = residual + keep * (x + bias) / (1 - p),  dx = keep * g / (1 - p)
  * evaluated in fp32 and rounded once. The keep mask is not stored: element e

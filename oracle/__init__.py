@@ -482,3 +482,11 @@ def layernorm_pair_bwd(dy1, dy2, x, mean, rstd, gamma1, gamma2):
     _, dg1, db1 = layernorm_bwd(dy1, x, mean, rstd, gamma1, param_dtype=pdt)
     _, dg2, db2 = layernorm_bwd(dy2, x, mean, rstd, gamma2, param_dtype=pdt)
     return dx, dg1, db1, dg2, db2
+
+
+def bias_add_residual_pair(x1, bias1, x2, bias2, residual):
+    """residual + ((x1 + bias1) + (x2 + bias2)) as the parallel-residual layer's three bias_dropout_add calls with
+    dropout off, each evaluated in fp32 and rounded once (bias_add_residual): t1 = x1 + bias1 (skipped without
+    bias1), t3 = t1 + (x2 + bias2), result = residual + t3."""
+    t1 = x1 if bias1 is None else bias_add_residual(x1, bias1, None)
+    return bias_add_residual(bias_add_residual(x2, bias2, t1), None, residual)

@@ -178,6 +178,12 @@ def test_argument_validation_of_the_layer_entry_points(hotpath):
     assert lib.nhp_layernorm_fwd(null, null, null, null, null, null, 1e-5, 4, 0, BF16, BF16, None) == 0
     assert lib.nhp_layernorm_bwd(q, null, null, p, p, null, p, p, null, 4, 8, BF16, BF16, None) == -3   # mean missing
     assert lib.nhp_layernorm_bwd(q, p, null, p, p, p, p, p, null, 4, 8, BF16, BF16, None) == -3          # workspace missing
+    # attention branch + MLP branch + residual in one pass
+    assert lib.nhp_bias_add_residual_pair(q, p, p, p, p, p, 4, 8, 9, None) == -1
+    assert lib.nhp_bias_add_residual_pair(q, p, p, p, p, p, -4, 8, BF16, None) == -2
+    assert lib.nhp_bias_add_residual_pair(q, p, null, null, null, p, 4, 8, BF16, None) == -3   # x2 missing
+    assert lib.nhp_bias_add_residual_pair(q, p, null, p, null, null, 4, 8, BF16, None) == -3   # residual missing
+    assert lib.nhp_bias_add_residual_pair(null, null, null, null, null, null, 0, 8, BF16, None) == 0
     # two LayerNorms of one input
     assert lib.nhp_layernorm_pair_fwd(q, q2, null, null, p, p, p, p, p, 1e-5, 4, 8, 4, F32, None) == -1
     assert lib.nhp_layernorm_pair_fwd(q, q2, null, null, p, p, p, p, p, 1e-5, 4, 8, BF16, F16, None) == -1

@@ -187,6 +187,64 @@ def test_bias_add_residual_bit_exact(hotpath, shape, dtype):
         assert torch.equal(util.raw_bits(out.cpu()), util.raw_bits(oracle.bias_add_residual(x, b, r)))
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("shape", [(1, 8), (37, 96), (5, 1000), (300, 2048), (1000, 24), (64, 8192), (3, 1001)],
+                         ids=lambda s: f"{s[0]}x{s[1]}")
+def test_bias_add_residual_pair_bit_exact(hotpath, shape, dtype):
+    """nhp_bias_add_residual_pair against the oracle (three rounded additions) and against three
+    nhp_bias_add_residual launches, bit for bit; every combination of missing biases; in place on x1."""
+    rows, cols = shape
+    x1, x2, res = (util.randn((rows, cols), dtype, seed=10 + i, std=2.0) for i in range(3))
+    b1, b2 = (util.randn((cols,), dtype, seed=20 + i) for i in range(2))
+    L, code = hotpath.lib(), hotpath.dtype_code(x1, "t")
+    d1, d2, dr = x1.to(DEV), x2.to(DEV), res.to(DEV)
+    for ba, bb in ((b1, b2), (None, b2), (b1, None), (None, None)):
+        da = None if ba is None else ba.to(DEV)
+        db = None if bb is None else bb.to(DEV)
+        out = torch.empty((rows, cols), dtype=dtype, device=DEV)
+        assert L.nhp_bias_add_residual_pair(out.data_ptr(), d1.data_ptr(), ptr(da), d2.data_ptr(), ptr(db), dr.data_ptr(),
+                                            rows, cols, code, None) == 0
+        assert torch.equal(util.raw_bits(out.cpu()), util.raw_bits(oracle.bias_add_residual_pair(x1, ba, x2, bb, res)))
+        # the three launches it replaces
+        t1, t2, t3, o3 = (torch.empty_like(out) for _ in range(4))
+        if da is None:
+            t1 = d1
+        else:
+            assert L.nhp_bias_add_residual(t1.data_ptr(), d1.data_ptr(), ptr(da), None, rows, cols, code, None) == 0
+        assert L.nhp_bias_add_residual(t3.data_ptr(), d2.data_ptr(), ptr(db), t1.data_ptr(), rows, cols, code, None) == 0
+        assert L.nhp_bias_add_residual(o3.data_ptr(), t3.data_ptr(), None, dr.data_ptr(), rows, cols, code, None) == 0
+        assert torch.equal(util.raw_bits(out), util.raw_bits(o3))
+    inplace = d1.clone()
+    assert L.nhp_bias_add_residual_pair(inplace.data_ptr(), inplace.data_ptr(), ptr(b1.to(DEV)), d2.data_ptr(),
+                                        ptr(b2.to(DEV)), dr.data_ptr(), rows, cols, code, None) == 0
+    assert torch.equal(util.raw_bits(inplace.cpu()), util.raw_bits(oracle.bias_add_residual_pair(x1, b1, x2, b2, res)))
+
+
+def test_bias_add_residual_pair_function_and_gradients():
+    from megatron.model.fused_bias_dropout import bias_add_residual_pair, bias_dropout_add_fused_inference
+
+    dtype = torch.bfloat16
+    x1, x2, res = (util.randn((32, 4, 512), dtype, seed=30 + i, std=2.0).to(DEV).requires_grad_(True) for i in range(3))
+    b1, b2 = (util.randn((512,), dtype, seed=40 + i).to(DEV).requires_grad_(True) for i in range(2))
+    out = bias_add_residual_pair(x1, b1.expand_as(x1), x2, b2, res)     # one bias expanded as the reference passes it
+    g = util.randn((32, 4, 512), dtype, seed=50).to(DEV)
+    out.backward(g)
+    got = [t.grad.clone() for t in (x1, b1, x2, b2, res)]
+    for t in (x1, b1, x2, b2, res):
+        t.grad = None
+    a = bias_dropout_add_fused_inference(x1, b1.expand_as(x1), None, 0.0)
+    o = bias_dropout_add_fused_inference(x2, b2, a, 0.0)
+    ref = bias_dropout_add_fused_inference(o, None, res, 0.0)
+    assert torch.equal(util.raw_bits(out), util.raw_bits(ref))
+    ref.backward(g)
+    for mine, theirs in zip(got, (x1, b1, x2, b2, res)):
+        assert torch.equal(util.raw_bits(mine), util.raw_bits(theirs.grad))
+    with pytest.raises(RuntimeError):
+        bias_add_residual_pair(x1, b1, x2[:16], b2, res)
+    with pytest.raises(RuntimeError):
+        bias_add_residual_pair(x1, b1, x2, b2, None)
+
+
 def test_bias_dropout_add_functions():
     from megatron.model.fused_bias_dropout import (bias_dropout_add_fused_inference, bias_dropout_add_fused_train,
                                                     get_bias_dropout_add)

@@ -539,3 +539,26 @@ def test_bias_dropout_add_with_dropout(dtype):
     mean = sum(oracle.bias_dropout_add(v, None, None, 0.5, s) for s in range(400)) / 400
     assert (mean - 1).abs().max().item() < 0.5
     assert abs(mean.mean().item() - 1) < 0.05
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_bias_add_residual_pair_is_three_fused_calls(dtype):
+    """residual + ((x1 + b1) + (x2 + b2)) rounded where the parallel-residual layer's three bias_dropout_add calls
+    round when each runs as one fused function (fp32 inside, one rounding at its end; dropout off):
+    megatron/model/transformer.py:1229-1250, fused_bias_dropout.py:28-60. Written out with torch in fp32."""
+    rows, cols = 37, 48
+    x1, x2, res = (util.randn((rows, cols), dtype, seed=60 + i, std=2.0) for i in range(3))
+    b1, b2 = (util.randn((cols,), dtype, seed=70 + i) for i in range(2))
+
+    def call(x, bias, residual):      # one bias_dropout_add: fp32 inside, rounded once
+        v = x.float() if bias is None else x.float() + bias.float()
+        return (v if residual is None else residual.float() + v).to(dtype)
+
+    for ba, bb in ((b1, b2), (None, b2), (b1, None), (None, None)):
+        t1 = x1 if ba is None else call(x1, ba, None)
+        want = call(call(x2, bb, t1), None, res)
+        got = oracle.bias_add_residual_pair(x1, ba, x2, bb, res)
+        assert torch.equal(util.raw_bits(got), util.raw_bits(want)), (ba is None, bb is None)
+    if dtype != torch.float32:   # and the roundings matter: one rounding at the very end gives other bits somewhere
+        once = (res.float() + ((x1.float() + b1.float()) + (x2.float() + b2.float()))).to(dtype)
+        assert not torch.equal(util.raw_bits(once), util.raw_bits(oracle.bias_add_residual_pair(x1, b1, x2, b2, res)))
