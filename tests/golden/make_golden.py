@@ -95,7 +95,9 @@ def main():
         res = util.randn((6, 16), dtype, seed + 3, std=2.0)
         dx = oracle.bias_gelu_bwd(g, y, bias)
         put(name, y=y, bias=bias, g=g, res=res, out=oracle.bias_gelu_fwd(y, bias), dx=dx, dbias=oracle.column_sum(dx),
-            added=oracle.bias_add_residual(y, bias, res))
+            added=oracle.bias_add_residual(y, bias, res),
+            # attention branch y + bias, MLP branch g + bias, residual res (the parallel-residual layer's join)
+            added_pair=oracle.bias_add_residual_pair(y, bias, g, bias, res))
 
     for name, dtype, seed in (("norm_bf16", torch.bfloat16, 31), ("norm_fp16", torch.float16, 32),
                               ("norm_fp32", torch.float32, 33)):

@@ -53,6 +53,7 @@ def test_oracle_reproduces_gelu_golden(name):
     dx = oracle.bias_gelu_bwd(g, y, bias)
     assert same(dx, get(name, "dx")) and same(oracle.column_sum(dx), get(name, "dbias"))
     assert same(oracle.bias_add_residual(y, bias, res), get(name, "added"))
+    assert same(oracle.bias_add_residual_pair(y, bias, g, bias, res), get(name, "added_pair"))
 
 
 @pytest.mark.parametrize("name", NORM)
@@ -204,6 +205,10 @@ def test_gpu_matches_gelu_golden(hotpath, name):
     added = torch.empty_like(y)
     assert L.nhp_bias_add_residual(added.data_ptr(), y.data_ptr(), bias.data_ptr(), res.data_ptr(), rows, cols, code, None) == 0
     assert same(added.cpu(), get(name, "added"))
+    joined = torch.empty_like(added)
+    assert L.nhp_bias_add_residual_pair(joined.data_ptr(), y.data_ptr(), bias.data_ptr(), g.data_ptr(), bias.data_ptr(),
+                                        res.data_ptr(), rows, cols, code, None) == 0
+    assert same(joined.cpu(), get(name, "added_pair"))
 
 
 @pytest.mark.gpu
