@@ -226,7 +226,7 @@ __device__ __forceinline__ void round_chunk(float (&v)[Elt<DT>::kVec])
 template <int DT, int TW, int U>
 __global__ void __launch_bounds__(kPwThreads)
 residual_pair_kernel(void* out, const void* x1, const void* bias1, const void* x2, const void* bias2,
-                     const void* residual, uint32_t rows, uint32_t cpr)
+                     const void* residual, uint32_t rows, uint32_t cpr, uint32_t steps)
 {
     constexpr int V = Elt<DT>::kVec;
     constexpr int TR = kPwThreads / TW;
@@ -236,8 +236,10 @@ residual_pair_kernel(void* out, const void* x1, const void* bias1, const void* x
     const uint32_t cc = blockIdx.x * TW + tc;
     if (cc >= cpr) return;
     const size_t row_elems = (size_t)cpr * V;
+    // one step per workgroup unless the tensor has more steps than the grid may have rows
+    for (uint32_t step = blockIdx.y; step < steps; step += gridDim.y) {
     u32x4 r1[U], r2[U], rr[U];
-    const uint32_t r = blockIdx.y * (TR * U) + tr;
+    const uint32_t r = step * (TR * U) + tr;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const uint32_t row = r + u * TR;
@@ -274,6 +276,7 @@ residual_pair_kernel(void* out, const void* x1, const void* bias1, const void* x
             for (int j = 0; j < V; ++j) t1[j] = fr[j] + t1[j];
             store16_stream(static_cast<S*>(out) + (size_t)row * row_elems + (size_t)cc * V, float_to_chunk<DT>(t1));
         }
+    }
     }
 }
 
@@ -447,12 +450,12 @@ static int run_residual_pair(void* out, const void* x1, const void* bias1, const
     if (chunked) {
         const int64_t cpr = cols / V;
         const TilePlan p = plan_tiles(rows, cpr, false);
-        if (p.steps > 65535u || !grid_fits((int64_t)p.col_tiles * p.steps, kPwThreads)) return NHP_ERR_SHAPE;
-        const dim3 grid(p.col_tiles, p.steps);
+        if (!grid_fits((int64_t)p.col_tiles * p.grid_y, kPwThreads)) return NHP_ERR_SHAPE;
+        const dim3 grid(p.col_tiles, p.grid_y);
 #define CASE(TW_)                                                                                   \
     case TW_:                                                                                       \
         residual_pair_kernel<DT, TW_, kPwU><<<grid, kPwThreads, kPwLdsTwoInputs, st>>>(             \
-            out, x1, bias1, x2, bias2, residual, (uint32_t)rows, (uint32_t)cpr);                    \
+            out, x1, bias1, x2, bias2, residual, (uint32_t)rows, (uint32_t)cpr, p.steps);           \
         break;
         switch (p.tw) {
             CASE(1) CASE(2) CASE(4) CASE(8) CASE(16) CASE(32) CASE(64)

@@ -188,7 +188,8 @@ def test_bias_add_residual_bit_exact(hotpath, shape, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
-@pytest.mark.parametrize("shape", [(1, 8), (37, 96), (5, 1000), (300, 2048), (1000, 24), (64, 8192), (3, 1001)],
+@pytest.mark.parametrize("shape", [(1, 8), (37, 96), (5, 1000), (300, 2048), (1000, 24), (64, 8192), (3, 1001),
+                                   (600000, 8)],   # more row steps than a grid has rows: workgroups loop
                          ids=lambda s: f"{s[0]}x{s[1]}")
 def test_bias_add_residual_pair_bit_exact(hotpath, shape, dtype):
     """nhp_bias_add_residual_pair against the oracle (three rounded additions) and against three
