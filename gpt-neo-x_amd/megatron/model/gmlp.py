@@ -22,56 +22,70 @@ class TinyAttention(torch.nn.Module):
 
     def __init__(self, neox_args, d_attn, d_ff, mask_fn):
         super().__init__()
-        self.proj_qkv = torch.nn.Linear(d_ff * 2, 3 * d_attn)
-        self.proj_ffn = torch.nn.Linear(d_attn, d_ff)
+        softmax_in_fp32 = bool(getattr(neox_args, "attention_softmax_in_fp32", False))
         self.scale = d_attn ** -0.5
-        in_fp32 = getattr(neox_args, "attention_softmax_in_fp32", False)
-        self.fold_scale = bool(in_fp32)
+        self.fold_scale = softmax_in_fp32          # the softmax module only takes a scale when it works in fp32
+        self.proj_qkv = torch.nn.Linear(2 * d_ff, 3 * d_attn)
+        self.proj_ffn = torch.nn.Linear(d_attn, d_ff)
         self.softmax = FusedScaleMaskSoftmax(
-            input_in_fp16=neox_args.precision == "fp16", input_in_bf16=neox_args.precision == "bfloat16",
-            fusion_type=get_fusion_type(neox_args), mask_func=mask_fn, softmax_in_fp32=in_fp32,
-            scale=self.scale if self.fold_scale else None)
+            input_in_fp16=neox_args.precision == "fp16",
+            input_in_bf16=neox_args.precision == "bfloat16",
+            fusion_type=get_fusion_type(neox_args),
+            mask_func=mask_fn,
+            softmax_in_fp32=softmax_in_fp32,
+            scale=self.scale if self.fold_scale else None,
+        )
 
-    def forward(self, x, attention_mask):
-        q, k, v = torch.chunk(self.proj_qkv(x), 3, dim=-1)
-        scores = torch.bmm(q, k.transpose(1, 2)).unsqueeze(1)          # [b, 1, n, m]
+    def _probabilities(self, queries, keys, attention_mask):
+        """``[b, n, d] x [b, m, d] -> [b, n, m]`` attention weights; the softmax module wants a head dimension."""
+        scores = torch.bmm(queries, keys.transpose(1, 2))
         if not self.fold_scale:
             scores = scores * self.scale
-        mask = attention_mask[..., :scores.size(-2), :scores.size(-1)]
-        probs = self.softmax(scores, mask).squeeze(1)
-        return self.proj_ffn(torch.bmm(probs, v))
+        n, m = scores.shape[-2:]
+        return self.softmax(scores.unsqueeze(1), attention_mask[..., :n, :m]).squeeze(1)
+
+    def forward(self, x, attention_mask):
+        queries, keys, values = self.proj_qkv(x).chunk(3, dim=-1)
+        mixed = torch.bmm(self._probabilities(queries, keys, attention_mask), values)
+        return self.proj_ffn(mixed)
 
 
 class SpatialGatingUnit(torch.nn.Module):
     """``res * (W_causal . norm(gate) + b [+ tiny attention])`` with ``res, gate`` the two halves of the features
-    and ``W`` an ``s x s`` matrix mixing positions, its upper triangle zeroed (megatron/model/gmlp.py:57-94)."""
+    and ``W`` an ``s x s`` matrix mixing positions, its upper triangle zeroed (megatron/model/gmlp.py:57-94).
+    The mixing starts out as the identity on the bias alone: zero weights, unit bias."""
 
     def __init__(self, neox_args, d_ff, d_attn=None, causal=True, mask_fn=None):
         super().__init__()
+        norm_class, eps = get_norm(neox_args)
         self.causal = causal
-        self.use_attn = d_attn is not None
-        norm, eps = get_norm(neox_args)
-        self.norm = norm(d_ff, eps=eps)
+        self.norm = norm_class(d_ff, eps=eps)
         self.proj = torch.nn.Linear(neox_args.seq_length, neox_args.seq_length)
+        with torch.no_grad():
+            self.proj.weight.zero_()
+            self.proj.bias.fill_(1.0)
+        self.use_attn = d_attn is not None
         if self.use_attn:
             assert mask_fn is not None
-            self.attn = TinyAttention(neox_args, d_attn, d_ff, mask_fn)
-        torch.nn.init.zeros_(self.proj.weight)
-        torch.nn.init.constant_(self.proj.bias, 1.0)
+            self.attn = TinyAttention(neox_args=neox_args, d_attn=d_attn, d_ff=d_ff, mask_fn=mask_fn)
 
-    def forward(self, x, attention_mask):
-        n = x.shape[0]
-        x = x.transpose(0, 1)                                            # [s, b, d] -> [b, s, d]
-        res, gate = x.chunk(2, dim=-1)
-        gate = self.norm(gate)
+    def _mixing(self, n):
+        """Weights ``[n, n]`` and bias ``[n]`` of the mixing along the sequence for ``n`` positions; causal: a
+        position only receives from itself and earlier ones."""
         weight, bias = self.proj.weight, self.proj.bias
         if self.causal:
-            weight, bias = torch.tril(weight[:n, :n]), bias[:n]
-        # mixing along the sequence: [b, d, s] x W^T + b
-        gate = F.linear(gate.transpose(1, 2), weight, bias).transpose(1, 2)
+            return torch.tril(weight[:n, :n]), bias[:n]
+        return weight, bias
+
+    def forward(self, x, attention_mask):
+        batch_first = x.transpose(0, 1)                                   # [s, b, d] -> [b, s, d]
+        res, gate = batch_first.chunk(2, dim=-1)
+        weight, bias = self._mixing(x.shape[0])
+        # positions are mixed as the last dimension of [b, d, s]
+        gate = F.linear(self.norm(gate).transpose(1, 2), weight, bias).transpose(1, 2)
         if self.use_attn:
-            gate = gate + self.attn(x, attention_mask)
-        return (gate * res).transpose(0, 1)                              # -> [s, b, d]
+            gate = gate + self.attn(batch_first, attention_mask)
+        return (res * gate).transpose(0, 1)                               # -> [s, b, d]
 
 
 class GMLPBlock(torch.nn.Module):
