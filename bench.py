@@ -71,7 +71,7 @@ MEASURED_TRAFFIC_BYTES = {"pythia-1.4b": 2181026543, "mlp-gelu-1.4b": 838974329,
                           "layernorm-1.4b": 210897047, "masked-c3": 6442319672, "rope-c4": 541727652,
                           "llama2-7b-c5": 17247434494, "mistral-window": 15133130579,
                           "causal-blocks-1.4b": 1778443264, "mistral-window-blocks": 10569712988,
-                          "layernorm-pair-1.4b": 303302335, "bias-residual-pair-1.4b": 268494860}
+                          "layernorm-pair-1.4b": 303301529, "bias-residual-pair-1.4b": 268494848}
 
 
 def tri(n):
