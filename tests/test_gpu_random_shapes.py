@@ -222,3 +222,103 @@ def test_layer_kernels_random_shapes(hotpath, seed):
         assert L.nhp_gated_act_fwd(go.data_ptr(), xd.data_ptr(), bd.data_ptr(), rows, f, oracle.GATE_ACTS[act], code, None) == 0
         want_g = oracle.gated_act_fwd(x, act, bias)
         util.assert_close_ulp_or_noise(go.cpu(), want_g, 2, util.gated_noise(x, bias, act, want_g), f"gated {act}")
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_pair_kernels_random_shapes(hotpath, seed):
+    """The two kernels of the parallel-residual layer: two LayerNorms of one input (forward and backward) and the
+    join of the two branches with the residual, on boundary shapes."""
+    rng = random.Random(6000 + seed)
+    dtype = rng.choice(ALL)
+    rows, cols = boundary_int(rng, 1, 400), boundary_int(rng, 1, 5000)
+    pdtype = rng.choice((dtype, torch.float32))
+    L, code, pcode = hotpath.lib(), hotpath._DTYPE[dtype], hotpath._DTYPE[pdtype]
+    print(f"pair rows={rows} cols={cols} {dtype} params {pdtype}", flush=True)
+    x = util.randn((rows, cols), dtype, seed=seed, std=2.5) + 0.25
+    g1, g2 = (util.randn((rows, cols), dtype, seed=seed + 1 + i) for i in range(2))
+    gam1, gam2 = ((1 + 0.3 * util.randn((cols,), torch.float32, seed=seed + 3 + i)).to(pdtype) for i in range(2))
+    bet1, bet2 = ((0.2 * util.randn((cols,), torch.float32, seed=seed + 5 + i)).to(pdtype) for i in range(2))
+    dev = {k: v.to(DEV) for k, v in dict(x=x, g1=g1, g2=g2, gam1=gam1, gam2=gam2, bet1=bet1, bet2=bet2).items()}
+    # join of the branches: bit-exact, with a random choice of missing biases
+    b1 = util.randn((cols,), dtype, seed=seed + 7) if rng.random() < 0.7 else None
+    b2 = util.randn((cols,), dtype, seed=seed + 8) if rng.random() < 0.7 else None
+    d1, d2 = (None if b is None else b.to(DEV) for b in (b1, b2))
+    out = torch.empty_like(dev["x"])
+    assert L.nhp_bias_add_residual_pair(out.data_ptr(), dev["x"].data_ptr(), ptr(d1), dev["g1"].data_ptr(), ptr(d2),
+                                        dev["g2"].data_ptr(), rows, cols, code, None) == 0
+    assert torch.equal(util.raw_bits(out.cpu()), util.raw_bits(oracle.bias_add_residual_pair(x, b1, g1, b2, g2)))
+    # two LayerNorms of one input
+    y1, y2, dx = (torch.empty_like(dev["x"]) for _ in range(3))
+    mean, rstd = torch.empty(rows, device=DEV), torch.empty(rows, device=DEV)
+    grads = [torch.empty_like(dev["gam1"]) for _ in range(4)]
+    ws = torch.empty(max(L.nhp_layernorm_pair_bwd_workspace_bytes(rows, cols, code), 16), dtype=torch.uint8, device=DEV)
+    assert L.nhp_layernorm_pair_fwd(y1.data_ptr(), y2.data_ptr(), mean.data_ptr(), rstd.data_ptr(), dev["x"].data_ptr(),
+                                    dev["gam1"].data_ptr(), dev["bet1"].data_ptr(), dev["gam2"].data_ptr(),
+                                    dev["bet2"].data_ptr(), 1e-5, rows, cols, code, pcode, None) == 0
+    w1, w2, _, _ = oracle.layernorm_pair_fwd(x, gam1, bet1, gam2, bet2, 1e-5)
+    for got, want, gam in ((y1, w1, gam1), (y2, w2, gam2)):
+        util.assert_close_ulp_or_noise(got.cpu(), want, 2, (gam.float().abs() * 64 * util.EPS32).expand(rows, cols), "pair fwd")
+    assert L.nhp_layernorm_pair_bwd(dx.data_ptr(), grads[0].data_ptr(), grads[1].data_ptr(), grads[2].data_ptr(),
+                                    grads[3].data_ptr(), dev["g1"].data_ptr(), dev["g2"].data_ptr(), dev["x"].data_ptr(),
+                                    mean.data_ptr(), rstd.data_ptr(), dev["gam1"].data_ptr(), dev["gam2"].data_ptr(),
+                                    ws.data_ptr(), rows, cols, code, pcode, None) == 0
+    mc, rc = mean.cpu(), rstd.cpu()
+    want = oracle.layernorm_pair_bwd(g1, g2, x, mc, rc, gam1, gam2)
+    noise = (((g1.float().abs() * gam1.float().abs() + g2.float().abs() * gam2.float().abs()).sum(-1, keepdim=True))
+             * rc[:, None] * 64 * util.EPS32).expand(rows, cols)
+    util.assert_close_ulp_or_noise(dx.cpu(), want[0], 2, noise, "pair dx")
+    xhat = ((x.float() - mc[:, None]) * rc[:, None]).abs()
+    for i, g in ((0, g1), (2, g2)):
+        util.assert_close_ulp_or_noise(grads[i].cpu(), want[1 + i], 2, (g.float().abs() * xhat).sum(0) * 32 * util.EPS32, "dgamma")
+        util.assert_close_ulp_or_noise(grads[i + 1].cpu(), want[2 + i], 2, g.float().abs().sum(0) * 32 * util.EPS32, "dbeta")
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_block_limited_softmax_random_shapes(hotpath, seed):
+    """The causal softmax that writes only the blocks in use: random sequence length, window and block size; values
+    inside the written range against the oracle, a sentinel outside of it."""
+    import scaled_upper_triang_masked_softmax_cuda as ext
+    from megatron.model.fused_softmax import _written_blocks
+
+    rng = random.Random(7000 + seed)
+    dtype = rng.choice(HALF)
+    s = 8 * boundary_int(rng, 3, 300)
+    a = rng.randint(1, 3)
+    zb = 1 << rng.randint(3, 10)
+    window = rng.choice((None, None, rng.randint(0, s + 10)))
+    scale = rng.choice((1.0, 0.125, 1 / math.sqrt(128)))
+    print(f"blocks a={a} s={s} window={window} zero_block={zb} {dtype}", flush=True)
+    x = util.randn((a, s, s), dtype, seed=seed, std=2.0)
+    dy = util.randn((a, s, s), dtype, seed=seed + 1)
+    eff = None if window is None or window >= s else window
+    written = _written_blocks(s, zb, eff, "cpu")
+    masked = fb.causal_mask(s, sliding_window_width=window)[0, 0]
+    assert bool((written | masked).all())
+    sentinel = 0x7e01
+    want_y = oracle.causal_softmax_fwd(x, scale, window=window)
+    want_dx = oracle.softmax_bwd(dy, want_y, scale, causal=True, window=window)
+    real_empty = torch.empty_like
+
+    def marked(t, **k):
+        out = real_empty(t, **k)
+        out.view(torch.int16).fill_(sentinel)
+        return out
+
+    def planted(t):
+        t = t.clone()
+        t.view(torch.int16)[:, ~written] = sentinel
+        return t.to(DEV)
+
+    torch.empty_like = marked
+    try:
+        y = ext.forward(x.to(DEV), scale, window, None, None, None, zb).cpu()
+        dx = ext.backward(planted(dy), planted(want_y), scale, window, None, zb).cpu()
+    finally:
+        torch.empty_like = real_empty
+    for got in (y, dx):
+        if not bool(written.all()):
+            assert bool((util.raw_bits(got)[:, ~written] == sentinel).all())
+        zeros = written & masked
+        assert int(util.raw_bits(got)[:, zeros].abs().max() if zeros.any() else 0) == 0
+    util.assert_ulp_close(torch.where(written, y, want_y), want_y, 2, "y")
+    util.assert_softmax_bwd_close(torch.where(written, dx, want_dx), want_dx, dy.masked_fill(masked, 0), want_y, scale, "dx")
