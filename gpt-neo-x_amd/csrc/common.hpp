@@ -321,11 +321,24 @@ static inline DropoutKey make_dropout_key(float p, uint64_t seed, uint64_t offse
 }
 
 // ---------------------------------------------------------------------------
+// Launch-shape constants are written as NHP_TUNED_INT("NAME", default). This library
+// always takes the default; an experimental build can pre-include a header that
+// defines the macro differently (compiler option -include) to sweep the values.
+// ---------------------------------------------------------------------------
+#ifndef NHP_TUNED_INT
+#define NHP_TUNED_INT(name, def) (def)
+#endif
+
+// ---------------------------------------------------------------------------
 // Host-side launch checks
 // ---------------------------------------------------------------------------
 static inline bool ptr_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 // A grid of `blocks` workgroups of `threads` work-items must stay below 2^32 work-items.
 static inline bool grid_fits(int64_t blocks, int threads) { return blocks > 0 && blocks * threads < ((int64_t)1 << 32); }
+// hipGetLastError() returns and clears whatever error is pending on the calling thread, also one
+// left by an earlier call of the application's. launch_prepare() clears such a leftover before the
+// first launch of an entry point, so that launch_result() reports this library's launches only.
+static inline void launch_prepare() { (void)hipGetLastError(); }
 static inline int launch_result() { return hipGetLastError() == hipSuccess ? NHP_OK : NHP_ERR_LAUNCH; }
 
 }  // namespace nhp

@@ -105,6 +105,7 @@ dropout_scalar_kernel(DropArgs d, uint64_t total, uint64_t cols)
 template <int DT>
 static int dropout_launch(DropArgs d, int64_t rows, int64_t cols, hipStream_t st)
 {
+    launch_prepare();
     constexpr int V = Elt<DT>::kVec;
     const bool chunked = cols % V == 0 && ptr_aligned16(d.out) && ptr_aligned16(d.a) && ptr_aligned16(d.residual) &&
                          ptr_aligned16(d.bias) && rows < ((int64_t)1 << 31) && cols / V < ((int64_t)1 << 31);

@@ -169,6 +169,7 @@ template <int DT, int ACT, bool BWD>
 static int gated_launch(void* out, const void* in, const void* dy, const void* bias, int64_t rows, int64_t f,
                         hipStream_t st)
 {
+    launch_prepare();
     constexpr int V = Elt<DT>::kVec;
     const bool chunked = f % V == 0 && ptr_aligned16(out) && ptr_aligned16(in) && ptr_aligned16(dy) &&
                          ptr_aligned16(bias) && rows < ((int64_t)1 << 31) && f / V < ((int64_t)1 << 31);

@@ -20,8 +20,6 @@
 #include "common.hpp"
 #include "colsum.hpp"
 
-#include <cstdlib>
-
 namespace nhp {
 
 constexpr int kNormBlockWaves = 4;  // waves per workgroup when a wave holds whole rows
@@ -664,16 +662,6 @@ norm_param_grad_scalar_kernel(void* dgamma, void* dbeta, const void* dy, const v
 // ---------------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------------
-#ifdef NHP_TUNING
-static int norm_tune(const char* name, int def)
-{
-    const char* v = getenv(name);
-    return v ? atoi(v) : def;
-}
-#else
-static inline int norm_tune(const char*, int def) { return def; }
-#endif
-
 struct NormPlan {
     uint32_t L, logL;
     int K, W;
@@ -706,7 +694,7 @@ static bool plan_norm(int64_t cpr, bool backward, NormPlan& p, bool pair_fwd = f
             break;
         }
     }
-    const int tk = norm_tune("NHP_NORM_K", 0), tw = norm_tune("NHP_NORM_W", 0);
+    const int tk = NHP_TUNED_INT("NHP_NORM_K", 0), tw = NHP_TUNED_INT("NHP_NORM_W", 0);
     if (tk > 0 && tw > 0 && (int64_t)tk * tw >= segs) {
         p.K = tk;
         p.W = tw;
@@ -737,7 +725,7 @@ static uint32_t norm_bwd_grid(uint32_t row_blocks, bool param_grads, int waves_p
 {
     row_blocks = (row_blocks + kBwdU - 1) / kBwdU;  // a workgroup takes up to kBwdU row blocks per iteration
     if (!param_grads) return row_blocks;
-    const uint32_t cap = (uint32_t)norm_tune("NHP_NORM_GRID", (int)(kNormBwdWaves / (uint32_t)waves_per_block));
+    const uint32_t cap = (uint32_t)NHP_TUNED_INT("NHP_NORM_GRID", (int)(kNormBwdWaves / (uint32_t)waves_per_block));
     return row_blocks < cap ? row_blocks : cap;
 }
 
@@ -758,6 +746,7 @@ static int norm_fwd(void* y, float* mean, float* rstd, const void* x, const void
                     int eps_mode, int64_t rows, int64_t cols, int64_t stat, int pdt, hipStream_t st,
                     const NormSecond& second = NormSecond{})
 {
+    launch_prepare();
     constexpr int V = Elt<DT>::kVec;
     NormPlan p;
     const bool params_aligned = ptr_aligned16(gamma) && ptr_aligned16(beta) && ptr_aligned16(second.gamma2) &&
@@ -799,6 +788,7 @@ static int norm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, const v
                     const float* rstd, const void* gamma, void* workspace, float eps, int eps_mode, int64_t rows,
                     int64_t cols, int64_t stat, int pdt, hipStream_t st, const NormSecond& second = NormSecond{})
 {
+    launch_prepare();
     constexpr int V = Elt<DT>::kVec;
     NormPlan p;
     const bool pair = !RMS && second.dy2 != nullptr;

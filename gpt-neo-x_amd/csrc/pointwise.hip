@@ -313,16 +313,6 @@ column_sum_scalar_kernel(void* out, const void* dx, uint64_t rows, uint64_t cols
 // ---------------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------------
-#ifdef NHP_TUNING
-static int pw_tune(const char* name, int def)
-{
-    const char* v = getenv(name);
-    return v ? atoi(v) : def;
-}
-#else
-static inline int pw_tune(const char*, int def) { return def; }
-#endif
-
 struct TilePlan {
     int tw;          // chunk columns per workgroup (power of two <= 64)
     uint32_t steps;  // row steps of TR * U rows
@@ -345,12 +335,12 @@ static TilePlan plan_tiles(int64_t rows, int64_t cpr, bool colsum)
 {
     TilePlan p;
     p.tw = 1;
-    const int max_tw = pw_tune("NHP_PW_TW", kPwMaxTw);
+    const int max_tw = NHP_TUNED_INT("NHP_PW_TW", kPwMaxTw);
     while (p.tw < max_tw && p.tw < cpr) p.tw *= 2;
-    const int64_t step_rows = (int64_t)(kPwThreads / p.tw) * pw_tune("NHP_PW_U", colsum ? kPwColsumU : kPwU);
+    const int64_t step_rows = (int64_t)(kPwThreads / p.tw) * (colsum ? kPwColsumU : kPwU);
     p.steps = (uint32_t)((rows + step_rows - 1) / step_rows);
     p.col_tiles = (uint32_t)((cpr + p.tw - 1) / p.tw);
-    uint32_t cap = colsum ? (uint32_t)pw_tune("NHP_PW_GY", kPwColsumGridY) : 65535u;
+    uint32_t cap = colsum ? (uint32_t)NHP_TUNED_INT("NHP_PW_GY", kPwColsumGridY) : 65535u;
     if (cap == 0 || cap > 65535u) cap = 65535u;
     p.grid_y = p.steps < cap ? p.steps : cap;
     return p;
@@ -360,34 +350,19 @@ template <int DT, int OP, bool COLSUM>
 static int launch_tiled(void* out, const void* a, const void* b, const void* bias, float* partial, int64_t rows,
                         int64_t cpr, const TilePlan& p, hipStream_t st)
 {
+    launch_prepare();
     const dim3 grid(p.col_tiles, p.grid_y);
     if (!grid_fits((int64_t)p.col_tiles * p.grid_y, kPwThreads)) return NHP_ERR_SHAPE;
-    const uint32_t lds = (uint32_t)pw_tune("NHP_PW_LDS", (kNeedsB<OP> && b != nullptr) ? kPwLdsTwoInputs : 0);
+    const uint32_t lds = (uint32_t)NHP_TUNED_INT("NHP_PW_LDS", (kNeedsB<OP> && b != nullptr) ? kPwLdsTwoInputs : 0);
 #define CASE_U(TW_, U_)                                                                                  \
         pointwise_kernel<DT, OP, TW_, U_, COLSUM><<<grid, kPwThreads, lds, st>>>(                        \
             out, a, b, bias, partial, (uint32_t)rows, (uint32_t)cpr, p.steps);
-#ifdef NHP_TUNING
 #define CASE(TW_)                                                                                        \
     case TW_:                                                                                            \
-        switch (pw_tune("NHP_PW_U", COLSUM ? kPwColsumU : kPwU)) {                                                             \
-        case 1: CASE_U(TW_, 1) break;                                                                    \
-        case 2: CASE_U(TW_, 2) break;                                                                    \
-        case 4: CASE_U(TW_, 4) break;                                                                    \
-        case 8: CASE_U(TW_, 8) break;                                                                    \
-        default: return NHP_ERR_SHAPE;                                                                   \
-        }                                                                                                \
+        CASE_U(TW_, (COLSUM ? kPwColsumU : kPwU))                                                        \
         break;
-#else
-#define CASE(TW_)                                                                                        \
-    case TW_:                                                                                            \
-        CASE_U(TW_, (COLSUM ? kPwColsumU : kPwU))                                                                             \
-        break;
-#endif
     switch (p.tw) {
         CASE(1) CASE(2) CASE(4) CASE(8) CASE(16) CASE(32) CASE(64)
-#ifdef NHP_TUNING
-        CASE(128) CASE(256)
-#endif
     default:
         return NHP_ERR_SHAPE;
     }
@@ -401,6 +376,7 @@ template <int DT, int OP>
 static int run_pointwise(void* out, const void* a, const void* b, const void* bias, void* dbias, float* workspace,
                          int64_t rows, int64_t cols, hipStream_t st)
 {
+    launch_prepare();
     constexpr int V = Elt<DT>::kVec;
     const bool chunked = cols % V == 0 && ptr_aligned16(out) && ptr_aligned16(a) && ptr_aligned16(b) &&
                          ptr_aligned16(bias) && ptr_aligned16(workspace) && rows < ((int64_t)1 << 31) &&
@@ -443,6 +419,7 @@ template <int DT>
 static int run_residual_pair(void* out, const void* x1, const void* bias1, const void* x2, const void* bias2,
                              const void* residual, int64_t rows, int64_t cols, hipStream_t st)
 {
+    launch_prepare();
     constexpr int V = Elt<DT>::kVec;
     const bool chunked = cols % V == 0 && ptr_aligned16(out) && ptr_aligned16(x1) && ptr_aligned16(x2) &&
                          ptr_aligned16(residual) && ptr_aligned16(bias1) && ptr_aligned16(bias2) &&

@@ -24,8 +24,6 @@
 
 #include "common.hpp"
 
-#include <cstdlib>
-
 namespace nhp {
 
 // out = round(round(x*c) +/- round(r*s)); the three roundings of the scalar types.
@@ -374,30 +372,22 @@ static bool vector_ok(const RopeArgs& a, bool tables_ok)
     for (int i = 0; i < 3; ++i)
         if (a.is[i] % V != 0 || a.os[i] % V != 0) return false;
     if (!is_aligned16(a.in) || !is_aligned16(a.out)) return false;
-    if (a.s >= ((int64_t)1 << 31) || a.b * a.h >= ((int64_t)1 << 30)) return false;
+    // grid.x = s workgroups of 256 threads: a grid dimension must stay below 2^32 work-items
+    if (!grid_fits(a.s, 256) || a.b * a.h >= ((int64_t)1 << 30)) return false;
     return true;
 }
-
-#ifdef NHP_TUNING
-static int rope_tune(const char* name, int def)
-{
-    const char* v = getenv(name);
-    return v ? atoi(v) : def;
-}
-#else
-static inline int rope_tune(const char*, int def) { return def; }
-#endif
 
 template <int DT, bool BWD, typename Tables>
 static int rope_launch_scalar(const RopeArgs& a, const Tables& tab)
 {
+    launch_prepare();
     const int64_t total = a.s * a.b * a.h * a.d;
     const int64_t blocks = (total + 255) / 256;
     if (blocks >= ((int64_t)1 << 24)) return NHP_ERR_SHAPE;  // grid*block must stay below 2^32
     rope_scalar_kernel<DT, BWD, Tables><<<(uint32_t)blocks, 256, 0, a.st>>>(
         a.out, a.in, tab, total, a.b, a.h, a.d, a.d2, a.is[0], a.is[1], a.is[2], a.is[3], a.os[0], a.os[1],
         a.os[2], a.os[3]);
-    return hipGetLastError() == hipSuccess ? NHP_OK : NHP_ERR_LAUNCH;
+    return launch_result();
 }
 
 static RopeTensor rope_tensor(const RopeArgs& a)
@@ -412,6 +402,7 @@ static bool rope_flat(const RopeArgs& a) { return (a.is[1] == a.h * a.is[2]) && 
 template <int DT, bool BWD, typename Tables>
 static int rope_launch_vec(const RopeArgs& a, const RopeArgs* b, const Tables& tab)
 {
+    launch_prepare();
     constexpr int V = Elt<DT>::kVec;
     const int cpr = (int)(a.d / V);
     const int rpw = 64 / cpr;
@@ -424,19 +415,18 @@ static int rope_launch_vec(const RopeArgs& a, const RopeArgs* b, const Tables& t
     // iterations) with one set of cos/sin values; measured best on MI355X.
     const int64_t steps = (rows + rows_per_step - 1) / rows_per_step;
     int64_t splits = (steps + 3) / 4;
-    splits = rope_tune("NHP_ROPE_SPLITS", (int)splits);
+    splits = NHP_TUNED_INT("NHP_ROPE_SPLITS", (int)splits);
     if (splits < 1) splits = 1;
     if (splits > 65535) splits = 65535;
     dim3 grid((uint32_t)a.s, (uint32_t)splits, b ? 2u : 1u);
-    const uint32_t lds = (uint32_t)rope_tune("NHP_ROPE_LDS", 0);
     const bool flat = rope_flat(a) && (!b || rope_flat(*b));
     // two rows in flight per lane measured best (one is short of latency cover, four adds nothing)
     if (flat) {
-        rope_vec_kernel<DT, BWD, true, 2, Tables><<<grid, 256, lds, a.st>>>(pair, tab, cpr, (int)(a.d2 / V), rpw);
+        rope_vec_kernel<DT, BWD, true, 2, Tables><<<grid, 256, 0, a.st>>>(pair, tab, cpr, (int)(a.d2 / V), rpw);
     } else {
-        rope_vec_kernel<DT, BWD, false, 2, Tables><<<grid, 256, lds, a.st>>>(pair, tab, cpr, (int)(a.d2 / V), rpw);
+        rope_vec_kernel<DT, BWD, false, 2, Tables><<<grid, 256, 0, a.st>>>(pair, tab, cpr, (int)(a.d2 / V), rpw);
     }
-    return hipGetLastError() == hipSuccess ? NHP_OK : NHP_ERR_LAUNCH;
+    return launch_result();
 }
 
 // LDS row length (in chunks) of the transposing kernel: the XOR with the load chunk index needs a
@@ -467,6 +457,7 @@ static bool transposed_ok(const RopeArgs& a, bool tables_ok)
 template <int DT, bool BWD, typename Tables>
 static int rope_launch_transposed(const RopeArgs& a, const Tables& tab)
 {
+    launch_prepare();
     if constexpr (DT == NHP_F32) {
         return NHP_ERR_SHAPE;
     } else {
@@ -486,7 +477,7 @@ static int rope_launch_transposed(const RopeArgs& a, const Tables& tab)
             return NHP_ERR_SHAPE;
         }
 #undef CASE
-        return hipGetLastError() == hipSuccess ? NHP_OK : NHP_ERR_LAUNCH;
+        return launch_result();
     }
 }
 

@@ -35,8 +35,6 @@
 
 #include "common.hpp"
 
-#include <cstdlib>
-
 namespace nhp {
 
 constexpr float kExpBias = 64.0f;
@@ -731,22 +729,10 @@ scalar_bwd_kernel(uint16_t* dx, const uint16_t* dy, const uint16_t* y, float sca
 // ---------------------------------------------------------------------------
 struct RowPlan {
     int L, K, W;
-    uint32_t lds;  // dynamic LDS bytes, only used to bound the number of resident workgroups
 };
 
 constexpr int64_t kMaxResidentRow = 65536;
 constexpr int kBlockWaves = 4;  // waves per workgroup when a wave owns whole rows
-
-#ifdef NHP_TUNING
-// Tuning builds read overrides from the environment on every call.
-static int tune(const char* name, int def)
-{
-    const char* v = getenv(name);
-    return v ? atoi(v) : def;
-}
-#else
-static inline int tune(const char*, int def) { return def; }
-#endif
 
 enum RowKind { kCausalFwd, kCausalFwdExtra, kCausalBwd, kMaskedFwd, kMaskedBwd };
 
@@ -771,7 +757,6 @@ static bool plan_row(int64_t n, RowKind kind, RowPlan& p, bool blocks = false)
 {
     if (n < 8 || n % 8 != 0 || n > kMaxResidentRow) return false;
     const int64_t chunks = n / 8;
-    p.lds = (uint32_t)tune("NHP_LDS", 0);
     if (chunks <= 64) {
         int L = 1;
         while (L < chunks) L *= 2;
@@ -811,8 +796,8 @@ static bool plan_row(int64_t n, RowKind kind, RowPlan& p, bool blocks = false)
             W = 4;
         }
     }
-    p.W = tune("NHP_W", W);
-    p.K = tune("NHP_K", K);
+    p.W = NHP_TUNED_INT("NHP_W", W);
+    p.K = NHP_TUNED_INT("NHP_K", K);
     if ((int64_t)p.W * p.K < segs) p.K = (int)((segs + p.W - 1) / p.W);
     return true;
 }
@@ -842,11 +827,6 @@ static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t
 // The runtime rejects launches of 2^32 or more threads per grid dimension.
 static inline bool launch_fits(int64_t blocks, int threads) { return blocks * threads < ((int64_t)1 << 32); }
 
-static inline int launch_status()
-{
-    return hipGetLastError() == hipSuccess ? NHP_OK : NHP_ERR_LAUNCH;
-}
-
 constexpr int64_t kMaxRows = (int64_t)1 << 31;  // row and block ids are 32-bit on the device
 constexpr uint32_t kNoWindow = 0xffffffffu;
 
@@ -855,6 +835,7 @@ static int causal_fwd(void* y, const void* x, float scale, int64_t batches, int6
                       const float* slopes, const void* bias, const int32_t* kl, uint32_t heads, hipStream_t st,
                       void* dropped = nullptr, const DropoutKey* drop = nullptr, uint32_t zshift = 0)
 {
+    launch_prepare();
     const int64_t rows = batches * n;
     RowPlan p;
     uint16_t* yp = static_cast<uint16_t*>(y);
@@ -871,13 +852,13 @@ static int causal_fwd(void* y, const void* x, float scale, int64_t batches, int6
         const uint32_t blocks = (uint32_t)((rows + G::kRowsPerBlock - 1) / G::kRowsPerBlock); \
         if (!launch_fits(blocks, G::kThreads)) return NHP_ERR_SHAPE;                       \
         if (dp != nullptr)                                                                 \
-            causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves, kDropout><<<blocks, G::kThreads, p.lds, st>>>( \
+            causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves, kDropout><<<blocks, G::kThreads, 0, st>>>( \
                 yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, nullptr, nullptr, nullptr, 1, dp, dk, zshift); \
         else if (slopes != nullptr || bp != nullptr || kl != nullptr)                      \
-            causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves, kPerHead><<<blocks, G::kThreads, p.lds, st>>>( \
+            causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves, kPerHead><<<blocks, G::kThreads, 0, st>>>( \
                 yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, slopes, bp, kl, heads, nullptr, dk, zshift); \
         else                                                                               \
-            causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves, kPlain><<<blocks, G::kThreads, p.lds, st>>>( \
+            causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves, kPlain><<<blocks, G::kThreads, 0, st>>>( \
                 yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, nullptr, nullptr, nullptr, 1, nullptr, dk, zshift); \
     }
         NHP_FOR_PLAN(p);
@@ -887,7 +868,7 @@ static int causal_fwd(void* y, const void* x, float scale, int64_t batches, int6
         scalar_fwd_kernel<DT, 0><<<(uint32_t)rows, kScalarThreads, 0, st>>>(
             yp, xp, nullptr, scale, (uint64_t)n, (uint64_t)n, 1, 0, window, slopes, bp, kl, heads, dp, dk);
     }
-    return launch_status();
+    return launch_result();
 }
 
 template <int DT, bool CAUSAL>
@@ -895,6 +876,7 @@ static int softmax_bwd(void* dx, const void* dy, const void* y, float scale, int
                        int64_t rows_per_matrix, uint32_t window, const int32_t* kl, uint32_t heads, hipStream_t st,
                        const DropoutKey* drop = nullptr, uint32_t zshift = 0)
 {
+    launch_prepare();
     RowPlan p;
     const DropoutKey dk = drop != nullptr ? *drop : DropoutKey{};
     const bool dropout = drop != nullptr;
@@ -909,14 +891,14 @@ static int softmax_bwd(void* dx, const void* dy, const void* y, float scale, int
         if (!launch_fits(blocks, G::kThreads)) return NHP_ERR_SHAPE;                       \
         if (dropout)                                                                       \
             softmax_bwd_kernel<DT, L_, K_, W_, kBlockWaves, CAUSAL, kDropout>                      \
-                <<<blocks, G::kThreads, p.lds, st>>>(dxp, dyp, yp, scale, (uint32_t)rows, (uint32_t)n, \
+                <<<blocks, G::kThreads, 0, st>>>(dxp, dyp, yp, scale, (uint32_t)rows, (uint32_t)n, \
                                                      (uint32_t)rows_per_matrix, window, nullptr, 1, dk, zshift); \
         else if (CAUSAL && kl != nullptr)                                                  \
             softmax_bwd_kernel<DT, L_, K_, W_, kBlockWaves, CAUSAL, CAUSAL ? kPerHead : kPlain>    \
-                <<<blocks, G::kThreads, p.lds, st>>>(dxp, dyp, yp, scale, (uint32_t)rows, (uint32_t)n, \
+                <<<blocks, G::kThreads, 0, st>>>(dxp, dyp, yp, scale, (uint32_t)rows, (uint32_t)n, \
                                                      (uint32_t)rows_per_matrix, window, kl, heads, dk, zshift); \
         else                                                                               \
-            softmax_bwd_kernel<DT, L_, K_, W_, kBlockWaves, CAUSAL, kPlain><<<blocks, G::kThreads, p.lds, st>>>( \
+            softmax_bwd_kernel<DT, L_, K_, W_, kBlockWaves, CAUSAL, kPlain><<<blocks, G::kThreads, 0, st>>>( \
                 dxp, dyp, yp, scale, (uint32_t)rows, (uint32_t)n, (uint32_t)rows_per_matrix, window, nullptr, 1, dk, \
                 zshift);                                                                   \
     }
@@ -928,7 +910,7 @@ static int softmax_bwd(void* dx, const void* dy, const void* y, float scale, int
             dxp, dyp, yp, scale, (uint64_t)n, (uint64_t)rows_per_matrix, window, CAUSAL ? kl : nullptr, heads,
             dropout ? 1 : 0, dk);
     }
-    return launch_status();
+    return launch_result();
 }
 
 // Heads a wave walks over with one decoded mask row. Two amortise the decoding;
@@ -940,6 +922,7 @@ static int masked_fwd(void* y, const void* x, const uint8_t* mask, float scale, 
                       int64_t sq, int64_t n, int64_t pad_batches, hipStream_t st, void* dropped = nullptr,
                       const DropoutKey* drop = nullptr)
 {
+    launch_prepare();
     uint16_t* dp = static_cast<uint16_t*>(dropped);
     const DropoutKey dk = drop != nullptr ? *drop : DropoutKey{};
     const int64_t bq_rows = b * sq;
@@ -953,18 +936,18 @@ static int masked_fwd(void* y, const void* x, const uint8_t* mask, float scale, 
     {                                                                                      \
         using G = Geo<L_, K_, W_, kBlockWaves>;                                            \
         const int64_t rb = (bq_rows + G::kRowsPerBlock - 1) / G::kRowsPerBlock;            \
-        const uint32_t hpw = (uint32_t)tune("NHP_HPW", (int)pick_heads_per_wave(np));       \
+        const uint32_t hpw = (uint32_t)NHP_TUNED_INT("NHP_HPW", (int)pick_heads_per_wave(np));       \
         const uint32_t hgs = (uint32_t)((np + hpw - 1) / hpw);                             \
         if (rb * hgs >= kMaxRows || !launch_fits(rb * hgs, G::kThreads)) return NHP_ERR_SHAPE; \
-        int64_t tile = tune("NHP_MASK_TILE", (int)((sq + G::kRowsPerBlock - 1) / G::kRowsPerBlock)); \
+        int64_t tile = NHP_TUNED_INT("NHP_MASK_TILE", (int)((sq + G::kRowsPerBlock - 1) / G::kRowsPerBlock)); \
         if (tile < 1) tile = 1;                                                            \
         if (tile > rb) tile = rb;                                                          \
         if (dp != nullptr)                                                                 \
-            masked_fwd_kernel<DT, L_, K_, W_, kBlockWaves, true><<<(uint32_t)(rb * hgs), G::kThreads, p.lds, st>>>( \
+            masked_fwd_kernel<DT, L_, K_, W_, kBlockWaves, true><<<(uint32_t)(rb * hgs), G::kThreads, 0, st>>>( \
                 yp, xp, mask, scale, (uint32_t)bq_rows, (uint32_t)sq, (uint32_t)np, (uint32_t)n, hpw, hgs, \
                 per_batch, (uint32_t)rb, (uint32_t)tile, dp, dk);                          \
         else                                                                               \
-            masked_fwd_kernel<DT, L_, K_, W_, kBlockWaves, false><<<(uint32_t)(rb * hgs), G::kThreads, p.lds, st>>>( \
+            masked_fwd_kernel<DT, L_, K_, W_, kBlockWaves, false><<<(uint32_t)(rb * hgs), G::kThreads, 0, st>>>( \
                 yp, xp, mask, scale, (uint32_t)bq_rows, (uint32_t)sq, (uint32_t)np, (uint32_t)n, hpw, hgs, \
                 per_batch, (uint32_t)rb, (uint32_t)tile, nullptr, dk);                     \
     }
@@ -975,7 +958,7 @@ static int masked_fwd(void* y, const void* x, const uint8_t* mask, float scale, 
         scalar_fwd_kernel<DT, 1><<<(uint32_t)(b * np * sq), kScalarThreads, 0, st>>>(
             yp, xp, mask, scale, (uint64_t)n, (uint64_t)sq, (uint64_t)np, per_batch, kNoWindow, nullptr, nullptr, nullptr, 1, dp, dk);
     }
-    return launch_status();
+    return launch_result();
 }
 
 }  // namespace nhp
