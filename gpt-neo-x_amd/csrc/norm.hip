@@ -20,6 +20,8 @@
 #include "common.hpp"
 #include "colsum.hpp"
 
+#include <mutex>
+
 namespace nhp {
 
 constexpr int kNormBlockWaves = 4;  // waves per workgroup when a wave holds whole rows
@@ -913,6 +915,38 @@ static int norm_bwd_dispatch(void* dx, void* dgamma, void* dbeta, const void* dy
     }
 }
 
+// ---------------------------------------------------------------------------
+// Fixed scratch memory for nhp_layernorm_bwd_noalloc: the partial rows of the parameter
+// gradients live in a device array that is part of the loaded code object, so that entry
+// point needs no workspace from the caller and no allocation. Every GPU the library runs
+// on holds its own copy of the array at its own address; host code never uses the array's
+// name as an address (it is only a handle for hipGetSymbolAddress), always the pointer
+// looked up once per device.
+// ---------------------------------------------------------------------------
+constexpr size_t kNoallocScratchBytes = NHP_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kNoallocScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static std::mutex scratch_mutex;
+static void* scratch_ptr[kMaxDevices];  // per device, filled on the first call with that device current
+
+// Address of the current device's copy of `scratch`; nullptr on failure.
+static void* noalloc_scratch()
+{
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (scratch_ptr[dev] == nullptr) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        scratch_ptr[dev] = p;
+    }
+    return scratch_ptr[dev];
+}
+
 }  // namespace nhp
 
 using namespace nhp;
@@ -932,6 +966,21 @@ int nhp_layernorm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, const
 {
     return norm_bwd_dispatch<false>(dx, dgamma, dbeta, dy, x, mean, rstd, gamma, workspace, 0.0f, 0, rows, cols,
                                     cols, dtype, param_dtype, stream);
+}
+
+int nhp_layernorm_bwd_noalloc(void* dx, void* dgamma, void* dbeta, const void* dy, const void* x, const float* mean,
+                              const float* rstd, const void* gamma, int64_t rows, int64_t cols, int dtype,
+                              int param_dtype, void* stream)
+{
+    if (dtype != NHP_F16 && dtype != NHP_BF16 && dtype != NHP_F32) return NHP_ERR_DTYPE;
+    void* ws = nullptr;
+    if (dgamma != nullptr || dbeta != nullptr) {
+        if (norm_workspace_bytes(rows, cols, dtype) > (int64_t)kNoallocScratchBytes) return NHP_ERR_SCRATCH;
+        ws = noalloc_scratch();
+        if (ws == nullptr) return NHP_ERR_LAUNCH;
+    }
+    return norm_bwd_dispatch<false>(dx, dgamma, dbeta, dy, x, mean, rstd, gamma, ws, 0.0f, 0, rows, cols, cols, dtype,
+                                    param_dtype, stream);
 }
 
 int nhp_layernorm_pair_fwd(void* y1, void* y2, float* mean, float* rstd, const void* x, const void* gamma1,

@@ -669,6 +669,7 @@ const char* nhp_status_string(int status)
         case NHP_ERR_PAD_BATCHES: return "mask batch dimension must be 1 or equal to the batch size";
         case NHP_ERR_LAUNCH: return "kernel launch failed";
         case NHP_ERR_ALIAS: return "output aliases an input";
+        case NHP_ERR_SCRATCH: return "input needs more scratch memory than the entry point's fixed buffer holds";
         default: return "unknown status";
     }
 }

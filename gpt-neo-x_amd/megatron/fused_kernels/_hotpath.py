@@ -82,6 +82,7 @@ def _declare(lib):
         "nhp_rmsnorm_partial_fwd": ([vp, vp, vp, vp, vp, f32, ci, i64, i64, i64, ci, ci, vp], ci),
         "nhp_rmsnorm_partial_bwd": ([vp, vp, vp, vp, vp, vp, vp, vp, f32, ci, i64, i64, i64, ci, ci, vp], ci),
         "nhp_norm_bwd_workspace_bytes": ([i64, i64, ci], i64),
+        "nhp_layernorm_bwd_noalloc": ([vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, ci, ci, vp], ci),
     }
     for name, (args, res) in sigs.items():
         fn = getattr(lib, name)  # AttributeError if the symbol is missing

@@ -43,7 +43,8 @@ typedef enum nhp_status {
     NHP_ERR_NULL = -3,      /* a required pointer is NULL while the tensor is not empty */
     NHP_ERR_PAD_BATCHES = -4, /* mask batch dimension is neither 1 nor b */
     NHP_ERR_LAUNCH = -5,    /* hipGetLastError() reported a launch failure */
-    NHP_ERR_ALIAS = -6      /* an output overlaps an input where that is not allowed */
+    NHP_ERR_ALIAS = -6,     /* an output overlaps an input where that is not allowed */
+    NHP_ERR_SCRATCH = -7    /* the input needs more scratch memory than the entry point's fixed buffer holds */
 } nhp_status;
 
 /* Library ABI version (bumped when a signature changes). */
@@ -524,6 +525,25 @@ int nhp_layernorm_fwd(void* y, float* mean, float* rstd, const void* x,
 int nhp_layernorm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, const void* x,
                       const float* mean, const float* rstd, const void* gamma, void* workspace,
                       int64_t rows, int64_t cols, int dtype, int param_dtype, void* stream);
+
+/*
+ * nhp_layernorm_bwd without a workspace argument and without any allocation, for callers that
+ * cannot allocate device memory (code under HIP graph capture, tight serving loops, harnesses
+ * that forbid it). No counterpart in the reference. Same arguments, kernels and results as
+ * nhp_layernorm_bwd; the partial sums of the parameter gradients go to a fixed device array of
+ * NHP_NOALLOC_SCRATCH_BYTES bytes (16 MiB) that is part of the library image on
+ * every GPU it runs on. Shapes whose nhp_norm_bwd_workspace_bytes() exceed that return
+ * NHP_ERR_SCRATCH (nothing is launched); without parameter gradients any shape is accepted.
+ * The caller's device must be current. All calls on one GPU share the array: calls that overlap
+ * in time on one GPU (different streams or threads) race; calls on one stream are ordered.
+ * Nothing needs clearing between calls (every partial row that is read was written by the
+ * same call). The array's address is looked up on the first call on each device; make that
+ * call outside a graph capture.
+ */
+#define NHP_NOALLOC_SCRATCH_BYTES (16 * 1024 * 1024)
+int nhp_layernorm_bwd_noalloc(void* dx, void* dgamma, void* dbeta, const void* dy, const void* x,
+                              const float* mean, const float* rstd, const void* gamma, int64_t rows,
+                              int64_t cols, int dtype, int param_dtype, void* stream);
 
 /*
  * Two LayerNorms of one input in one pass each way: y1 = xhat * gamma1 + beta1, y2 = xhat * gamma2 + beta2

@@ -41,6 +41,11 @@ def test_every_header_comment_cites_the_reference():
             continue
         if name.endswith("_workspace_bytes"):  # size query, documented with the function it serves
             continue
+        if name == "nhp_layernorm_bwd_noalloc":
+            # the one entry point without a counterpart in the reference: its comment must say so
+            before = text[: text.index(name + "(")]
+            assert "No counterpart in the reference" in before[before.rindex("/*"):]
+            continue
         before = text[: text.index(name + "(")]
         comment = before[before.rindex("/*") :]
         # the backward/forward pairs of the rotary functions share one comment
@@ -53,11 +58,11 @@ def test_status_strings_and_version(hotpath):
     assert lib.nhp_abi_version() == hotpath.ABI_VERSION
     assert lib.nhp_status_string(0) == b"ok"
     seen = set()
-    for code in range(-6, 0):
+    for code in range(-7, 0):
         s = lib.nhp_status_string(code)
         assert s and s != b"unknown status"
         seen.add(s)
-    assert len(seen) == 6
+    assert len(seen) == 7
     assert lib.nhp_status_string(-99) == b"unknown status"
     assert lib.nhp_softmax_max_resident_row() == 65536
 
