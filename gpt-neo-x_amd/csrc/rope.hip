@@ -5,14 +5,19 @@
 // elements of every head vector are rotated with the angle of position s,
 // the remaining d - d2 are copied.
 //
-// Vector kernel. A head vector is cut into 16-byte chunks (V = 8 elements for
+// Vector kernels. A head vector is cut into 16-byte chunks (V = 8 elements for
 // 16-bit data, 4 for fp32) and every lane owns one chunk, so a wave-wide load
 // or store moves up to 1 KiB of consecutive head vectors. The rotation pairs
 // element i with i + d2/2, i.e. a chunk with the chunk d2/(2V) lanes away in
 // the same wave; the partner's data is fetched with ds_bpermute (no memory
-// traffic). Chunks of the pass-through tail are copied by their lanes. A
-// workgroup stays on one sequence position and walks over the (batch, head)
-// rows, re-using the cos/sin values it loaded (or computed) once.
+// traffic). Chunks of the pass-through tail are copied by their lanes.
+//   rope_lean_kernel: cached tables, head vectors of a power-of-two number of
+//     chunks. Two chunks per thread, no loop, every load issued before the first
+//     wait: the shape a plain streaming copy runs fastest in on this GPU.
+//   rope_vec_kernel: everything else with unit feature stride (angles evaluated
+//     on the device, other head sizes). A workgroup stays on one sequence
+//     position and walks over the (batch, head) rows, re-using the cos/sin
+//     values it loaded (or computed) once.
 //
 // Transposing kernel, for 16-bit inputs that are contiguous along the sequence
 // instead of along the features (see rope_tr_kernel). Everything else (odd
@@ -213,6 +218,105 @@ rope_vec_kernel(RopePair pair, Tables tab, int cpr, int rot_chunks, int rpw)
 }
 
 // ---------------------------------------------------------------------------
+// Lean vector kernel (cached tables only)
+//   grid  = (ceil(rows * CPR / 512), s, tensors), block = 256 threads
+//   thread t of workgroup x owns chunks x * 512 + t and x * 512 + 256 + t of
+//   position blockIdx.y, counted over the position's rows * CPR chunks;
+//   CPR = 2^LOG_CPR chunks per head vector, so both chunks have the same
+//   place in their head vectors and share one pair of table chunks.
+// Consecutive workgroups sweep consecutive memory. Every load (tables, then
+// data) is issued before anything waits: lanes outside the rotary part load
+// table chunk 0 and discard the result, a second row beyond the end re-loads
+// the last row and is not stored, so that no load sits in a divergent region
+// (where the compiler would have to wait for it on the spot, or would sink it
+// behind the wait for the data). Needs d2 > 0.
+// ---------------------------------------------------------------------------
+constexpr int kLeanThreads = 256;
+constexpr int kLeanU = 2;
+
+template <int DT, bool BWD, int LOG_CPR, bool FLAT, typename Tables>
+__global__ void __launch_bounds__(kLeanThreads)
+rope_lean_kernel(RopeTensor ta, RopeTensor tb, Tables tab, int rot_chunks)
+{
+    constexpr int V = Elt<DT>::kVec;
+    constexpr int CPR = 1 << LOG_CPR;
+    constexpr int T = kLeanThreads, U = kLeanU;
+    using S = typename Elt<DT>::storage;
+    // both tensors' descriptions arrive with the kernel arguments; blockIdx.z picks one
+    const bool second = blockIdx.z != 0;
+    const S* const in = static_cast<const S*>(second ? tb.in : ta.in);
+    S* const out = static_cast<S*>(second ? tb.out : ta.out);
+    const int rows = second ? tb.rows : ta.rows;
+    const int h = second ? tb.h : ta.h;
+    const int64_t is_s = second ? tb.is_s : ta.is_s, is_b = second ? tb.is_b : ta.is_b, is_h = second ? tb.is_h : ta.is_h;
+    const int64_t os_s = second ? tb.os_s : ta.os_s, os_b = second ? tb.os_b : ta.os_b, os_h = second ? tb.os_h : ta.os_h;
+
+    const int lane = threadIdx.x & 63;
+    const int64_t pos = blockIdx.y;
+    const int i0 = (int)blockIdx.x * (T * U) + (int)threadIdx.x;
+    const int c = i0 & (CPR - 1);
+    const int r0 = i0 >> LOG_CPR;
+    if (r0 < rows) {
+        const int half = rot_chunks >> 1;
+        const bool is_rot = c < rot_chunks;
+        const bool first = c < half;
+        const int partner_lane = is_rot ? (first ? lane + half : lane - half) : lane;
+        // cos of the own chunk; sin of the own chunk (forward) or of the partner's (backward)
+        const int tc = is_rot ? c : 0;
+        const int ts = is_rot ? (BWD ? (first ? c + half : c - half) : c) : 0;
+        // addresses first, then all loads back to back
+        const S* ip = in + pos * is_s + c * V;
+        S* op = out + pos * os_s + c * V;
+        int64_t src[U], dst[U];
+        bool on[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int r = r0 + u * (T >> LOG_CPR);
+            on[u] = r < rows;
+            const int rr = on[u] ? r : rows - 1;
+            if (FLAT) {
+                src[u] = rr * is_h;
+                dst[u] = rr * os_h;
+            } else {
+                const int bi = rr / h;
+                const int hi = rr - bi * h;
+                src[u] = bi * is_b + hi * is_h;
+                dst[u] = bi * os_b + hi * os_h;
+            }
+        }
+        float cv[V], sv[V], unused[V];
+        tab.get_vec(pos, (int64_t)tc * V, cv, unused);
+        tab.get_vec(pos, (int64_t)ts * V, unused, sv);
+        u32x4 raw[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) raw[u] = load16_stream(ip + src[u]);
+        // forward: first half subtracts, backward: second half subtracts
+        const bool negate = BWD ? !first : first;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            u32x4 praw;
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                praw[k] = (uint32_t)__builtin_amdgcn_ds_bpermute(partner_lane << 2, (int)raw[u][k]);
+            float x[V], pr[V], y[V];
+            chunk_to_float<DT>(raw[u], x);
+            chunk_to_float<DT>(praw, pr);
+#pragma unroll
+            for (int v = 0; v < V; ++v)
+                y[v] = negate ? rot<DT, true>(x[v], cv[v], pr[v], sv[v]) : rot<DT>(x[v], cv[v], pr[v], sv[v]);
+            const u32x4 rotated = float_to_chunk<DT>(y);
+            u32x4 res;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) res[k] = is_rot ? rotated[k] : raw[u][k];
+            // The value passes through an opaque statement: without it the compiler folds the select into
+            // the store and the store loses its non-temporal hint.
+            asm volatile("" : "+v"(res));
+            if (on[u]) store16_stream(op + dst[u], res);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Transposing kernel: the input is contiguous along the sequence (stride_s == 1,
 // features stride_d apart), the output along the features. This is the layout in
 // which the gradient of the keys arrives from the backward of the score GEMM
@@ -399,12 +503,51 @@ static bool rope_flat(const RopeArgs& a) { return (a.is[1] == a.h * a.is[2]) && 
 
 // Launches the vector kernel for one tensor (b == nullptr) or for two tensors
 // that share s, d, d2 and the tables (q and k; their head counts may differ).
+template <typename T>
+struct IsCachedTables { static constexpr bool value = false; };
+template <int DT, int CS>
+struct IsCachedTables<CachedTables<DT, CS>> { static constexpr bool value = true; };
+
+// log2 of a power of two in 2..64, else -1
+static int log2_chunks(int64_t cpr)
+{
+    for (int l = 1; l <= 6; ++l)
+        if (cpr == ((int64_t)1 << l)) return l;
+    return -1;
+}
+
 template <int DT, bool BWD, typename Tables>
 static int rope_launch_vec(const RopeArgs& a, const RopeArgs* b, const Tables& tab)
 {
     launch_prepare();
     constexpr int V = Elt<DT>::kVec;
     const int cpr = (int)(a.d / V);
+    if constexpr (IsCachedTables<Tables>::value) {
+        const int log_cpr = log2_chunks(cpr);
+        const int64_t most_rows = (b && b->b * b->h > a.b * a.h) ? b->b * b->h : a.b * a.h;
+        // grid.y holds the position; chunk numbers inside a position are 32-bit
+        if (log_cpr > 0 && a.d2 > 0 && a.s <= 65535 && most_rows * cpr < ((int64_t)1 << 31)) {
+            const RopeTensor ta = rope_tensor(a);
+            const RopeTensor tb = b ? rope_tensor(*b) : ta;
+            const int64_t rows = most_rows;
+            const int64_t per_pos = (rows * cpr + kLeanThreads * kLeanU - 1) / (kLeanThreads * kLeanU);
+            const dim3 grid((uint32_t)per_pos, (uint32_t)a.s, b ? 2u : 1u);
+            const bool flat = rope_flat(a) && (!b || rope_flat(*b));
+            const int rot_chunks = (int)(a.d2 / V);
+#define LEAN(LC_)                                                                                             \
+    case LC_:                                                                                                 \
+        if (flat)                                                                                             \
+            rope_lean_kernel<DT, BWD, LC_, true, Tables><<<grid, kLeanThreads, 0, a.st>>>(ta, tb, tab, rot_chunks);  \
+        else                                                                                                  \
+            rope_lean_kernel<DT, BWD, LC_, false, Tables><<<grid, kLeanThreads, 0, a.st>>>(ta, tb, tab, rot_chunks); \
+        break;
+            switch (log_cpr) {
+                LEAN(1) LEAN(2) LEAN(3) LEAN(4) LEAN(5) LEAN(6)
+            }
+#undef LEAN
+            return launch_result();
+        }
+    }
     const int rpw = 64 / cpr;
     const int rows_per_step = 4 * rpw;
     RopePair pair;
