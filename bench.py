@@ -29,6 +29,10 @@ the drop-in extension modules (which call libneox_hotpath.so):
   masked-dropout-c3  padding-masked softmax + attention dropout (p = 0.1) in one kernel, fwd+bwd on the masked-c3 tensors
   rpe-bias-1.4b  causal softmax fwd+bwd [128,2048,2048] bf16 with a bias tensor [16,2048,2048] added in the kernel
 
+  hbm-probes     kernels that only move data (libneox_probe.so): a plain streaming copy of 64 MiB, 128 MiB and
+                 1 GiB tensors, and the causal softmax forward's access pattern (lower-triangle reads, dense writes)
+                 at [128,2048,2048] and [64,8192,8192]: what the memory system gives for those patterns and sizes
+
   mlp-gelu-1.4b  bias + tanh-GeLU fwd and bwd (with the bias gradient) on the MLP activation [2048*8, 8192] bf16
   swiglu-7b      SwiGLU forward and backward on the Llama-2 7B MLP activation [4096*4, 2*11008] -> [4096*4, 11008] bf16
   bias-residual-1.4b  residual + (x + bias) on the hidden state [2048*8, 2048] bf16
@@ -64,14 +68,37 @@ for p in (ROOT, os.path.join(ROOT, "gpt-neo-x_amd")):
 METRIC = "achieved HBM GB/s (% of MI355X peak), causal softmax+rotary fwd/bwd, 1.4B shape"
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per launch of each workload's dominant kernel measured with
-# rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE; profiles/pythia-1.4b_step_hbm_traffic.txt,
-# profiles/layer_neighbours_hbm_traffic.txt, profiles/other_workloads_hbm_traffic.txt).
-MEASURED_TRAFFIC_BYTES = {"pythia-1.4b": 2181026543, "mlp-gelu-1.4b": 838974329, "swiglu-7b": 1803563138,
-                          "layernorm-1.4b": 210897047, "masked-c3": 6442319672, "rope-c4": 541727652,
-                          "llama2-7b-c5": 17247434494, "mistral-window": 15133130579,
-                          "causal-blocks-1.4b": 1778443264, "mistral-window-blocks": 10569712988,
-                          "layernorm-pair-1.4b": 303301529, "bias-residual-pair-1.4b": 268494848}
+TRAFFIC_TABLE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+# Workloads whose dominant kernel has no geometry query: a revision label that is changed by hand whenever
+# that kernel's launch shape or data flow changes, so that a traffic figure measured before is dropped.
+KERNEL_REVISIONS = {"mlp-gelu-1.4b": "bias_gelu_bwd r1", "swiglu-7b": "gated_bwd r1", "layernorm-1.4b": "norm_bwd r1",
+                    "rope-c4": "rope_lean r1", "layernorm-pair-1.4b": "norm_pair_bwd r1",
+                    "bias-residual-pair-1.4b": "bias_add_residual_pair r1"}
+
+
+def measured_traffic(workload, signature):
+    """HBM bytes per launch of the workload's dominant kernel as measured with rocprofv3 --pmc
+    (FETCH_SIZE, WRITE_SIZE), from the tracked table profiles/hbm_traffic.json. A figure belongs to
+    one kernel instantiation: it is returned only when the table's signature for the workload equals
+    the signature of the kernel that runs now (None otherwise, and when the workload is not listed)."""
+    try:
+        with open(TRAFFIC_TABLE) as f:
+            entry = json.load(f)["workloads"].get(workload)
+    except (OSError, ValueError, KeyError):
+        return None
+    if not entry or entry.get("signature") != signature:
+        return None
+    return entry["bytes"]
+
+
+def softmax_signature(lib, row_len, kind):
+    """'L<lanes> K<chunks per lane> W<waves per row>' of the kernel the library launches for such rows."""
+    import ctypes
+
+    l, k, w = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    if lib.nhp_softmax_geometry(row_len, kind, ctypes.byref(l), ctypes.byref(k), ctypes.byref(w)) != 0:
+        return "scalar"
+    return f"L{l.value} K{k.value} W{w.value}"
 
 
 def tri(n):
@@ -120,7 +147,7 @@ class Timer:
         self.pairs = {}
 
 
-def make_workload(name, torch, dev):
+def make_workload(name, torch, dev, fresh_dy=False):
     import fused_rotary_positional_embedding as rope_ext
     import scaled_masked_softmax_cuda as masked_ext
     import scaled_upper_triang_masked_softmax_cuda as causal_ext
@@ -156,6 +183,11 @@ def make_workload(name, torch, dev):
                         "rope_bwd": 2 * rb}
         dense = {"causal_softmax_fwd": 2 * a * s * s * 2, "causal_softmax_bwd": 3 * a * s * s * 2}
 
+        # --fresh-dy: the backward works in place, so without this its input shrinks from step to step
+        # (dx ~ 0.09 * y * dy); with it the upstream gradient is restored from a pristine copy before
+        # every backward, outside the backward's event bracket (the copy is part of the step's wall time)
+        dy0 = dy.clone() if fresh_dy else None
+
         def step(t):
             def rope_f():
                 rope_ext.forward_cached(q, cos, sin, False)
@@ -167,13 +199,19 @@ def make_workload(name, torch, dev):
 
             t.run("rope_fwd", rope_f)
             y = t.run("causal_softmax_fwd", lambda: causal_ext.forward(x, scale))
-            # in place on dy, as the reference does; its values shrink from step
-            # to step, which does not change the work done
+            if fresh_dy:
+                dy.copy_(dy0)
+            # in place on dy, as the reference does
             t.run("causal_softmax_bwd", lambda: causal_ext.backward(dy, y, scale))
             t.run("rope_bwd", rope_b)
 
+        from megatron.fused_kernels import _hotpath as hp
+
         cfg = {"workload": name, "scores": [a, s, s], "qk": [s, b, h, d], "rotary_dim": d2,
-               "scale": "1/sqrt(%d)" % d, "bytes_convention": "causal-min (reads of the lower triangle, dense writes)"}
+               "scale": "1/sqrt(%d)" % d, "bytes_convention": "causal-min (reads of the lower triangle, dense writes)",
+               "dominant_kernel_signature": "softmax_bwd causal " + softmax_signature(hp.lib(), s, 2)}
+        if fresh_dy:
+            cfg["fresh_dy"] = True
         return step, kernel_bytes, dense, "causal_softmax_bwd", "bf16", cfg
 
     if name == "attn-dropout-1.4b":
@@ -248,6 +286,10 @@ def make_workload(name, torch, dev):
                f"reads of the attended band, writes of the {zero_block}-column blocks a block-wise caller reads"}
         if zero_block:
             cfg["zero_block"] = zero_block
+        from megatron.fused_kernels import _hotpath as hp
+
+        cfg["dominant_kernel_signature"] = "softmax_bwd causal " + softmax_signature(hp.lib(), s, 2) + \
+            (f" blocks{zero_block}" if zero_block else "")
         return step, kernel_bytes, {}, "causal_softmax_bwd", "bf16", cfg
 
     if name in ("masked-c3", "masked-dropout-c3"):
@@ -290,9 +332,59 @@ def make_workload(name, torch, dev):
                    "bytes_convention": "dense (tensor read + mask once + probabilities and dropped probabilities written; "
                                        "3x tensor backward)"}
             return step_dropout, kernel_bytes, {}, "masked_softmax_dropout_bwd", "f16", cfg
+        from megatron.fused_kernels import _hotpath as hp
+
+        # The forward never reads a group of 8 keys that is all padding (37 % of this workload's keys):
+        # its bytes are the reads of the live groups + the mask once + the dense write, which is what the
+        # kernel moves; the dense convention (2x tensor) is printed beside it.
+        dense_fwd = kernel_bytes["masked_softmax_fwd"]
+        kernel_bytes["masked_softmax_fwd"] = needed["masked_softmax_fwd"][1]
+        needed = {"masked_softmax_fwd": ("GB/s_dense_convention", dense_fwd)}
         cfg = {"workload": name, "scores": [b, np_, sq, sk], "mask": [b, 1, sq, sk],
-               "bytes_convention": "dense (2x tensor forward + mask once, 3x tensor backward)"}
+               "bytes_convention": "forward: unmasked 8-key groups read + mask once + dense write; backward: 3x tensor",
+               "dominant_kernel_signature": "softmax_bwd plain " + softmax_signature(hp.lib(), sk, 4)}
         return step, kernel_bytes, needed, "masked_softmax_bwd", "f16", cfg
+
+    if name == "hbm-probes":
+        import ctypes
+
+        from megatron.fused_kernels import _hotpath as hp
+
+        path = os.path.join(os.path.dirname(hp.LIB_PATH), "libneox_probe.so")
+        plib = ctypes.CDLL(path)
+        vp, i64 = ctypes.c_void_p, ctypes.c_int64
+        plib.nhp_probe_copy.argtypes = [vp, vp, i64, ctypes.c_int, vp]
+        plib.nhp_probe_causal_pattern.argtypes = [vp, vp, i64, i64, vp]
+        kernel_bytes = {}
+        runs = []
+        for mib in (64, 128, 1024):
+            nsets = max(2, 1024 // mib)  # rotate over more than the last-level cache holds
+            bufs = [(torch.full((mib << 19,), 1.0, dtype=torch.bfloat16, device=dev),
+                     torch.empty((mib << 19,), dtype=torch.bfloat16, device=dev)) for _ in range(nsets)]
+            key = f"copy_{mib}MiB"
+            kernel_bytes[key] = 2 * (mib << 20)
+            runs.append((key, bufs, mib))
+        pat = []
+        for a, s in ((128, 2048), (64, 8192)):
+            x = torch.empty((a, s, s), dtype=torch.bfloat16, device=dev)
+            x.fill_(1.0)
+            y = torch.empty_like(x)
+            key = f"causal_pattern_{a}x{s}x{s}"
+            kernel_bytes[key] = causal_bytes(a, s)[0]
+            pat.append((key, x, y, a, s))
+        state = {"i": 0}
+        stream = hp.stream_of(pat[0][1])
+
+        def step(t):
+            state["i"] += 1
+            for key, bufs, mib in runs:
+                src, dst = bufs[state["i"] % len(bufs)]
+                t.run(key, lambda: hp.check(plib.nhp_probe_copy(dst.data_ptr(), src.data_ptr(), mib << 20, 256, stream), key))
+            for key, x, y, a, s in pat:
+                t.run(key, lambda: hp.check(plib.nhp_probe_causal_pattern(y.data_ptr(), x.data_ptr(), a, s, stream), key))
+
+        cfg = {"workload": name, "what": "data movement only; bytes as the kernels they stand for are priced"}
+        return step, kernel_bytes, {}, "copy_1024MiB", "u8", cfg
 
     if name == "rope-qk-1.4b":
         s, b, h, d, d2 = 2048, 8, 16, 128, 32
@@ -680,6 +772,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="pythia-1.4b")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--fresh-dy", action="store_true",
+                    help="pythia-1.4b / llama2-7b-c5: restore the upstream gradient from a pristine copy before every "
+                         "in-place backward (the copy runs outside the backward's event bracket)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="run one plain 1 GiB device copy first (reference for scaling rocprofv3 --pmc byte counters)")
     args = ap.parse_args()
@@ -705,7 +800,8 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    step, kernel_bytes, dense_bytes, dominant, dtype, cfg = make_workload(args.workload, torch, dev)
+    step, kernel_bytes, dense_bytes, dominant, dtype, cfg = make_workload(args.workload, torch, dev, args.fresh_dy)
+    signature = cfg.get("dominant_kernel_signature", KERNEL_REVISIONS.get(args.workload))
     # Timed region: K steps; only the dominant kernel is bracketed by events
     # (every event record is one more packet between the kernels).
     timer = Timer(torch, only=dominant)
@@ -760,7 +856,7 @@ def main():
         "bytes_per_step": step_bytes,
         "kernels": kernels,
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": dom["GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": dom["frac_of_peak"], "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "frac": dom["frac_of_peak"], "traffic": measured_traffic(args.workload, signature),
                      "algorithmic_bytes": kernel_bytes[dominant], "avg_launch_ms": dom["ms"],
                      "min_launch_ms": round(dominant_spread[0], 4), "median_launch_ms": round(dominant_spread[1], 4),
                      "max_launch_ms": round(dominant_spread[2], 4)},

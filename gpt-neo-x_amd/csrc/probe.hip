@@ -1,0 +1,89 @@
+// Data-movement probes for gfx950: kernels that only move bytes, in the access patterns of the
+// library's kernels, so that a kernel's time can be set against what the memory system gives for
+// its pattern and size. Built into libneox_probe.so, which only bench.py loads; nothing of the
+// library proper depends on it.
+//
+//   nhp_probe_copy            plain streaming copy, one 16-byte chunk per thread, no loop: the
+//                             fastest copy shape measured on MI355X (more bytes per thread, grid-
+//                             stride loops and XCD-contiguous orders are all slower)
+//   nhp_probe_causal_pattern  the causal softmax forward's traffic: row q of every [n, n] matrix
+//                             is read up to the 16-byte chunk that holds column q and written in
+//                             full; two waves per row, two chunks per lane for n = 2048, as the
+//                             forward kernel is launched
+
+#include "common.hpp"
+
+namespace nhp {
+
+__global__ void __launch_bounds__(1024)
+probe_copy_kernel(u32x4* out, const u32x4* in, size_t chunks)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < chunks) store16_stream(out + i, load16_stream(in + i));
+}
+
+// K chunks per lane, W waves per row (chunk c of a row belongs to (k, w, l) with c = (k*W + w)*64 + l,
+// the softmax kernels' layout); workgroup = one row.
+template <int K, int W>
+__global__ void __launch_bounds__(W * 64)
+probe_causal_pattern_kernel(uint16_t* y, const uint16_t* x, uint32_t n)
+{
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const uint32_t row = blockIdx.x;
+    const uint32_t q = row % n;
+    const int w = (int)((wave + blockIdx.x) % W);
+    const uint16_t* xr = x + (size_t)row * n;
+    uint16_t* yr = y + (size_t)row * n;
+    u32x4 raw[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const uint32_t col = (uint32_t)((k * W + w) * 64 + lane) * 8u;
+        raw[k] = u32x4{0, 0, 0, 0};
+        if (col < n && col <= q) raw[k] = load16_stream(xr + col);
+    }
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const uint32_t col = (uint32_t)((k * W + w) * 64 + lane) * 8u;
+        if (col < n) store16_stream(yr + col, raw[k]);
+    }
+}
+
+}  // namespace nhp
+
+using namespace nhp;
+
+extern "C" {
+
+// Copies `bytes` (a multiple of 16) from in to out with workgroups of `threads` (64..1024) threads.
+int nhp_probe_copy(void* out, const void* in, int64_t bytes, int threads, void* stream)
+{
+    if (bytes < 0 || bytes % 16 != 0 || threads < 64 || threads > 1024 || threads % 64 != 0) return NHP_ERR_SHAPE;
+    if (bytes == 0) return NHP_OK;
+    if (!out || !in) return NHP_ERR_NULL;
+    const int64_t chunks = bytes / 16;
+    const int64_t blocks = (chunks + threads - 1) / threads;
+    if (!grid_fits(blocks, threads)) return NHP_ERR_SHAPE;
+    launch_prepare();
+    probe_copy_kernel<<<(uint32_t)blocks, threads, 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<u32x4*>(out), static_cast<const u32x4*>(in), (size_t)chunks);
+    return launch_result();
+}
+
+// y, x: [batches, n, n] 16-bit elements, n = 2048 (two waves of two chunks per lane) or 8192
+// (eight waves of two chunks per lane).
+int nhp_probe_causal_pattern(void* y, const void* x, int64_t batches, int64_t n, void* stream)
+{
+    if (batches < 1 || (n != 2048 && n != 8192) || batches * n >= ((int64_t)1 << 31)) return NHP_ERR_SHAPE;
+    if (!y || !x) return NHP_ERR_NULL;
+    launch_prepare();
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const uint32_t rows = (uint32_t)(batches * n);
+    if (n == 2048)
+        probe_causal_pattern_kernel<2, 2><<<rows, 128, 0, st>>>(static_cast<uint16_t*>(y), static_cast<const uint16_t*>(x), 2048u);
+    else
+        probe_causal_pattern_kernel<2, 8><<<rows, 512, 0, st>>>(static_cast<uint16_t*>(y), static_cast<const uint16_t*>(x), 8192u);
+    return launch_result();
+}
+
+}  // extern "C"

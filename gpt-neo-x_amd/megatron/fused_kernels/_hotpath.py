@@ -39,6 +39,7 @@ def _declare(lib):
         "nhp_abi_version": ([], ci),
         "nhp_status_string": ([ci], ctypes.c_char_p),
         "nhp_softmax_max_resident_row": ([], i64),
+        "nhp_softmax_geometry": ([i64, ci, ctypes.POINTER(ci), ctypes.POINTER(ci), ctypes.POINTER(ci)], ci),
         "nhp_causal_softmax_fwd": ([vp, vp, f32, i64, i64, ci, vp], ci),
         "nhp_causal_softmax_bwd": ([vp, vp, vp, f32, i64, i64, ci, vp], ci),
         "nhp_causal_softmax_ex_fwd": ([vp, vp, f32, i64, i64, i64, vp, vp, vp, i64, ci, vp], ci),

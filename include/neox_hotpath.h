@@ -57,6 +57,13 @@ const char* nhp_status_string(int status);
  * take a slower streaming kernel but are still supported. */
 int64_t nhp_softmax_max_resident_row(void);
 
+/* Launch geometry the softmax kernels use for rows of `row_len` elements, for profiling
+ * records (a measured figure belongs to one kernel instantiation): lanes per row L, 16-byte
+ * chunks per lane K, waves per row W. `kind`: 0 causal forward, 1 causal forward with AliBi
+ * or a bias tensor, 2 causal backward, 3 padding-mask forward, 4 padding-mask backward.
+ * Returns NHP_ERR_SHAPE when such rows take the scalar kernel. */
+int nhp_softmax_geometry(int64_t row_len, int kind, int* lanes, int* chunks, int* waves);
+
 /* ------------------------------------------------------------------------
  * Scaled upper-triangular (causal) masked softmax
  * ---------------------------------------------------------------------- */

@@ -37,7 +37,7 @@ def test_library_exports_every_declared_symbol(hotpath):
 def test_every_header_comment_cites_the_reference():
     text = open(HEADER).read()
     for name in declared_functions():
-        if name in ("nhp_abi_version", "nhp_status_string", "nhp_softmax_max_resident_row"):
+        if name in ("nhp_abi_version", "nhp_status_string", "nhp_softmax_max_resident_row", "nhp_softmax_geometry"):
             continue
         if name.endswith("_workspace_bytes"):  # size query, documented with the function it serves
             continue
@@ -65,6 +65,12 @@ def test_status_strings_and_version(hotpath):
     assert len(seen) == 7
     assert lib.nhp_status_string(-99) == b"unknown status"
     assert lib.nhp_softmax_max_resident_row() == 65536
+    L, K, W = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    for kind in range(5):
+        assert lib.nhp_softmax_geometry(2048, kind, ctypes.byref(L), ctypes.byref(K), ctypes.byref(W)) == 0
+        assert L.value == 64 and L.value * K.value * W.value * 8 >= 2048
+    assert lib.nhp_softmax_geometry(2047, 0, ctypes.byref(L), ctypes.byref(K), ctypes.byref(W)) == -2  # scalar kernel
+    assert lib.nhp_softmax_geometry(2048, 9, ctypes.byref(L), ctypes.byref(K), ctypes.byref(W)) == -2
 
 
 def test_batch_per_block_matches_reference_formula(hotpath):

@@ -166,3 +166,49 @@ def test_rotary_cache_recipe():
     want = math.cos(p * base ** (-2 * j / dim))
     assert abs(cos[p, 0, 0, j].float().item() - want) <= 2.0**-8
     assert torch.equal(cos, ang.cos().to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+def test_rounding_boundary_marks_cover_every_fp32_perturbation(dtype):
+    """util.near_rounding_boundary: an fp32 value that rounds differently to `dtype` after moving
+    by up to 2 fp32 spacings must be marked; and only a small share of values is marked."""
+    g = torch.Generator().manual_seed(11)
+    ang = torch.rand(200000, generator=g, dtype=torch.float64) * 4000.0 - 2000.0
+    v = torch.cos(ang)
+    marked = util.near_rounding_boundary(v, dtype)
+    v32 = v.float()
+    base = v32.to(dtype)
+    raw = v32.view(torch.int32)
+    for k in (-2, -1, 1, 2):
+        moved = (raw + k).view(torch.float32)
+        flips = moved.to(dtype).view(torch.int16) != base.view(torch.int16)
+        assert not (flips & ~marked).any(), k
+    assert 0 < float(marked.float().mean()) < (0.002 if dtype == torch.bfloat16 else 0.01)
+    # exact midpoints and exact representable values
+    one = torch.tensor([1.0], dtype=dtype)
+    nxt = (one.view(torch.int16) + 1).view(dtype)
+    mid = (one.double() + nxt.double()) / 2
+    assert util.near_rounding_boundary(mid, dtype).all()
+    assert not util.near_rounding_boundary(one.double(), dtype).any()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32], ids=["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("backward", [False, True], ids=["fwd", "bwd"])
+def test_freqs_tolerance_holds_between_two_host_sincos(dtype, backward):
+    """The comparison used for the device's angle variant, exercised on the CPU: the oracle (libm
+    sincosf) against the same rotation with tables from torch's cos / sin (another fp32 routine).
+    They may differ only on elements marked as resting on a table rounding boundary."""
+    s, b, h, d, d2 = 64, 2, 3, 64, 48
+    g = torch.Generator().manual_seed(5)
+    ang = ((torch.rand((s, 1, 1, d2), generator=g) * 20.0 - 10.0) *
+           torch.where(torch.arange(s) % 2 == 0, 1.0, 700.0).view(s, 1, 1, 1)).contiguous()
+    t = util.randn((s, b, h, d), dtype, seed=3)
+    want = oracle.rope_freqs(t, ang, backward=backward)
+    got = oracle.rope_cached(t, ang.cos().to(dtype).contiguous(), ang.sin().to(dtype).contiguous(), backward=backward)
+    util.assert_rope_freqs_close(got, want, t, ang, backward, "host sincos pair")
+    # a wrong angle index on a handful of elements is caught: swap two positions' angles
+    bad_ang = ang.clone()
+    bad_ang[[3, 4]] = ang[[4, 3]]
+    bad = oracle.rope_cached(t, bad_ang.cos().to(dtype).contiguous(), bad_ang.sin().to(dtype).contiguous(), backward=backward)
+    with pytest.raises(AssertionError):
+        util.assert_rope_freqs_close(bad, want, t, ang, backward, "swapped angles")

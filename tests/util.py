@@ -63,7 +63,74 @@ def ulp_size(t):
     return torch.pow(2.0, e - mant)
 
 
-def assert_softmax_bwd_close(got, want, dy, y, scale, what=""):
+def near_rounding_boundary(v64, dtype, slack_ulp32=3):
+    """Bool tensor: the float64 values v64 lie within `slack_ulp32` fp32 spacings of a point where
+    rounding to `dtype` (fp16 / bf16) switches from one representable value to the next. Two fp32
+    evaluations of such a value that differ in the last places (device sincosf against libm) may
+    round to different `dtype` values; everywhere else they round to the same one."""
+    r = v64.to(torch.float32).to(dtype)                       # nearest representable value
+    bits = ordered_bits(r)
+    def from_ordered(o):
+        mag = o.abs().to(torch.int16)
+        raw = torch.where(o < 0, mag | torch.tensor(-32768, dtype=torch.int16), mag)
+        return raw.view(dtype).double()
+    up, down = from_ordered(bits + 1), from_ordered(bits - 1)
+    rd = r.double()
+    dist = torch.minimum((v64 - (rd + up) / 2).abs(), (v64 - (rd + down) / 2).abs())
+    ulp32 = torch.pow(2.0, torch.floor(torch.log2(v64.abs().clamp(min=2.0**-126))) - 23)
+    return dist <= slack_ulp32 * ulp32
+
+
+def rope_freqs_marked(freqs, dtype, backward):
+    """[s, 1, 1, d2] bool: elements of a rotary result computed from angles whose cos or sin table
+    entry (cos[i], sin[i] in the forward; cos[i], sin[partner(i)] in the backward) sits on a rounding
+    boundary of `dtype` in the sense of near_rounding_boundary. fp32 data: nothing is marked (the
+    table entries are not narrowed; the comparison is made in fp32 spacings)."""
+    f64 = freqs.double()
+    if dtype == torch.float32:
+        return torch.zeros_like(f64, dtype=torch.bool)
+    mc = near_rounding_boundary(torch.cos(f64), dtype)
+    ms = near_rounding_boundary(torch.sin(f64), dtype)
+    if backward:
+        d2 = freqs.size(-1)
+        h2 = d2 // 2
+        i = torch.arange(d2)
+        partner = torch.where(i + h2 < d2, i + h2, i + h2 - d2)   # the reference kernel's index, also for odd d2
+        ms = ms[..., partner]
+    return mc | ms
+
+
+def assert_rope_freqs_close(got, want, t, freqs, backward, what="", max_marked_share=0.02):
+    """Rotary from angles against the oracle. The only arithmetic that may differ between the two is
+    sincosf (device library against libm, both accurate to a few fp32 spacings); the three roundings
+    after it are the same. So wherever both table entries of an element are clear of a rounding
+    boundary of the data dtype the results must be bit-identical; on the marked elements (a fraction
+    of a per cent) one table entry may have rounded the other way, which moves the result by at most
+    one spacing of the data dtype at the magnitude of the inputs per entry: 2 spacings at max |t| of
+    the head vector. fp32 data: 2 fp32 spacings at that magnitude everywhere."""
+    got, want = got.cpu(), want.cpu()
+    d2 = freqs.size(-1)
+    marked = rope_freqs_marked(freqs.cpu(), got.dtype, backward).expand(got.shape[:-1] + (d2,))
+    g, w = got[..., :d2], want[..., :d2]
+    scale_ref = t.cpu().float().abs().amax(dim=-1, keepdim=True).expand_as(g.float())
+    wide_ok = (g.float() - w.float()).abs() <= 2 * ulp_size(scale_ref.to(got.dtype))
+    if got.dtype == torch.float32:
+        assert wide_ok.all(), f"{what}: {int((~wide_ok).sum())} fp32 elements out of tolerance"
+        return 0.0
+    same = raw_bits(g.contiguous()) == raw_bits(w.contiguous())
+    bad_clear = ~same & ~marked
+    assert not bad_clear.any(), (f"{what}: {int(bad_clear.sum())} elements differ from the oracle although their "
+                                 "table entries are clear of a rounding boundary")
+    assert (wide_ok | ~marked).all(), f"{what}: a marked element is off by more than two spacings at input magnitude"
+    share = float(marked.float().mean())
+    assert share <= max_marked_share, f"{what}: {share:.4f} of the elements rest on the wide tolerance"
+    return share
+
+
+BWD_NOISE_SHARES = []  # (what, share of elements beyond 2 ulp, worst ulp distance) of every backward comparison
+
+
+def assert_softmax_bwd_close(got, want, dy, y, scale, what="", max_noise_share=0.05):
     """Backward tolerance: 2 ulp of the output dtype, plus the rounding noise of
     an fp32 row sum. dx = scale*(g - y*S) cancels, so an S that differs by a few
     fp32 ulp of sum|g| (a different summation order) moves dx by
@@ -82,6 +149,11 @@ def assert_softmax_bwd_close(got, want, dy, y, scale, what=""):
         raise AssertionError(
             f"{what}: element {idx}: got {got.flatten()[idx].item()!r} want {want.flatten()[idx].item()!r} "
             f"noise {noise.flatten()[idx].item():.3e}")
+    # how much of the result rests on the noise clause rather than on the 2-ulp bound: recorded so that a
+    # regression (a kernel that drifts away from the oracle) shows up as a growing share, and bounded
+    share = float((~ok_ulp).float().mean()) if got.numel() else 0.0
+    BWD_NOISE_SHARES.append((what, share, int(ulp_distance(got, want).max()) if got.numel() else 0))
+    assert share <= max_noise_share, f"{what}: {share:.4f} of the elements are beyond 2 ulp (noise clause)"
     return int(ulp_distance(got, want).max())
 
 
