@@ -292,6 +292,42 @@ def make_workload(name, torch, dev, fresh_dy=False):
             (f" blocks{zero_block}" if zero_block else "")
         return step, kernel_bytes, {}, "causal_softmax_bwd", "bf16", cfg
 
+    if name == "masked-extras-1.4b":
+        # The padding-mask kernel doing what its caller otherwise does in passes of its own: relative-position bias,
+        # AliBi and the padding keys of right-padded sequences, under the decoder's causal mask given as a tensor.
+        from megatron.model.positional_embeddings import AliBi
+
+        b, np_, s = 8, 16, 2048
+        scale = 1.0 / math.sqrt(128)
+        x = torch.empty((b, np_, s, s), dtype=torch.bfloat16, device=dev)
+        dy = torch.empty_like(x)
+        for i in range(b):
+            x[i] = randn((np_, s, s), i, torch.bfloat16, 2.0)
+            dy[i] = randn((np_, s, s), 1000 + i, torch.bfloat16)
+        bias = randn((np_, s, s), 77, torch.bfloat16, 1.0)
+        slopes = AliBi(np_, mp_size=1, mp_rank=0).slopes.float().to(dev)
+        idx = torch.arange(s, device=dev)
+        mask = (idx[None, :] > idx[:, None]).view(1, 1, s, s).contiguous()
+        lengths = torch.tensor([2048, 1900, 1024, 2048, 1500, 2000, 777, 2048], dtype=torch.int32, device=dev)
+        n = x.numel()
+        # 8-key groups with a visible key: those of the triangle that start below the sequence's length
+        starts = torch.arange(0, s, 8, device=dev)
+        live = ((starts[None, None, :] <= idx[None, :, None]) & (starts[None, None, :] < lengths[:, None, None].long()))
+        live_chunks = int(live.sum().item())
+        bias_chunks = int((starts[None, :] <= idx[:, None]).sum().item())
+        fwd_b = live_chunks * 16 * np_ + bias_chunks * 16 * np_ + mask.numel() + n * 2
+        kernel_bytes = {"masked_softmax_ex_fwd": fwd_b, "masked_softmax_bwd": 3 * n * 2}
+
+        def step(t):
+            y = t.run("masked_softmax_ex_fwd", lambda: masked_ext.forward(x, mask, scale, slopes, bias, lengths))
+            t.run("masked_softmax_bwd", lambda: masked_ext.backward(dy, y, scale))
+
+        cfg = {"workload": name, "scores": [b, np_, s, s], "mask": [1, 1, s, s], "alibi_heads": np_, "bias": [np_, s, s],
+               "key_lengths": lengths.tolist(),
+               "bytes_convention": "forward: 8-key groups with a visible key read + each head's bias groups once + "
+                                   "mask once + dense write; backward: 3x tensor"}
+        return step, kernel_bytes, {}, "masked_softmax_bwd", "bf16", cfg
+
     if name in ("masked-c3", "masked-dropout-c3"):
         b, np_, sq, sk = 16, 32, 1024, 2048
         scale = 1.0 / math.sqrt(128)

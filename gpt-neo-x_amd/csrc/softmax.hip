@@ -209,7 +209,7 @@ __device__ __forceinline__ uint32_t active_slots(const Band& band, int w)
 // registers for loads in flight): kPerHead = bias tensor, AliBi, key lengths;
 // kDropout = a second output `dropped` = dropout(y) (y, the probabilities, is
 // still written: the backward needs it).
-enum CausalExtra { kPlain = 0, kPerHead = 1, kDropout = 2 };
+enum CausalExtra { kPlain = 0, kPerHead = 1, kDropout = 2, kPerHeadDropout = 3 };  // bit flags
 
 template <int DT, int L, int K, int W, int BW, int EXTRA>
 __global__ void __launch_bounds__((Geo<L, K, W, BW>::kThreads))
@@ -218,7 +218,8 @@ causal_fwd_kernel(uint16_t* y, const uint16_t* x, float scale, uint32_t total_ro
                   uint16_t* dropped, DropoutKey dk, uint32_t zshift)
 {
     using G = Geo<L, K, W, BW>;
-    constexpr bool PER_HEAD = EXTRA == kPerHead;
+    constexpr bool PER_HEAD = (EXTRA & kPerHead) != 0;
+    constexpr bool DROPOUT = (EXTRA & kDropout) != 0;
     __shared__ float lds[32];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -316,7 +317,7 @@ causal_fwd_kernel(uint16_t* y, const uint16_t* x, float scale, uint32_t total_ro
             if ((act >> k & 1u) && col < band.hi && col + 8 > band.lo) {
                 const u32x4 py = pack8<DT>(z[k]);
                 store16_stream(yr + col, py);
-                if constexpr (EXTRA == kDropout) {
+                if constexpr (DROPOUT) {
                     // dropout of the stored (rounded) probabilities, as the separate dropout kernel would see them
                     float f[8];
                     unpack8<DT>(py, f);
@@ -327,7 +328,7 @@ causal_fwd_kernel(uint16_t* y, const uint16_t* x, float scale, uint32_t total_ro
                 }
             } else {
                 store16_stream(yr + col, u32x4{0, 0, 0, 0});
-                if constexpr (EXTRA == kDropout) store16_stream(dropped + (size_t)row * n + col, u32x4{0, 0, 0, 0});
+                if constexpr (DROPOUT) store16_stream(dropped + (size_t)row * n + col, u32x4{0, 0, 0, 0});
             }
         }
     }
@@ -339,12 +340,19 @@ causal_fwd_kernel(uint16_t* y, const uint16_t* x, float scale, uint32_t total_ro
 // fetched and decoded once per head group.
 // ---------------------------------------------------------------------------
 // DROP: also write dropped = dropout(y), as the causal kernel does.
-template <int DT, int L, int K, int W, int BW, bool DROP>
+// PER_HEAD: what the caller of the reference adds to the scores, or folds into the mask, before this
+// softmax (megatron/model/transformer.py:580-588), done here instead of in passes of their own:
+//   bias [np, sq, n] in the scores' dtype (attention_scores += rpe): added in the storage dtype;
+//   AliBi slopes [np] (sq == n): the bias -(q - k) * slope for k <= q, nothing above the diagonal, with
+//     the roundings of AliBi.forward (megatron/model/positional_embeddings.py:219-257);
+//   key_lengths [b]: keys k >= key_lengths[b] count as masked (as if their mask bytes were 1).
+template <int DT, int L, int K, int W, int BW, bool DROP, bool PER_HEAD>
 __global__ void __launch_bounds__((Geo<L, K, W, BW>::kThreads))
 masked_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float scale,
                   uint32_t bq_rows, uint32_t sq, uint32_t np, uint32_t n,
                   uint32_t heads_per_wave, uint32_t head_groups, int mask_per_batch, uint32_t row_blocks,
-                  uint32_t tile, uint16_t* dropped, DropoutKey dk)
+                  uint32_t tile, uint16_t* dropped, DropoutKey dk, const float* slopes, const uint16_t* bias,
+                  const int32_t* key_lengths)
 {
     using G = Geo<L, K, W, BW>;
     __shared__ float lds[2][32];
@@ -394,6 +402,18 @@ masked_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
             const u32x2 v = load8(mrow + col);
             mb[k][0] = v[0];
             mb[k][1] = v[1];
+            if (PER_HEAD && key_lengths != nullptr) {
+                // bytes of the keys at or beyond the sequence's length become 1
+                const int32_t len = key_lengths[bi];
+                const uint32_t limit = len < 0 ? 0u : (uint32_t)len;
+                const uint32_t valid = limit > col ? limit - col : 0u;  // leading keys of the chunk that are real
+                if (valid < 8u) {
+                    const uint64_t beyond = ~(uint64_t)0 << (8u * valid);
+                    const uint64_t bytes = ((((uint64_t)mb[k][1] << 32) | mb[k][0]) & ~beyond) | (0x0101010101010101ull & beyond);
+                    mb[k][0] = (uint32_t)bytes;
+                    mb[k][1] = (uint32_t)(bytes >> 32);
+                }
+            }
         }
         dead[k] = inb && (mb[k][0] == 0x01010101u) && (mb[k][1] == 0x01010101u);
         live[k] = inb && !dead[k];
@@ -413,6 +433,42 @@ masked_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
             const uint32_t col = chunk_col<L, W>(k, w, l);
             raw[k] = u32x4{0, 0, 0, 0};
             if (live[k]) raw[k] = load16_stream(xr + col);
+        }
+        if constexpr (PER_HEAD) {
+            if (bias != nullptr) {
+                const uint16_t* br = bias + ((size_t)h * sq + qi) * n;
+#pragma unroll
+                for (int k = 0; k < K; ++k) {
+                    if (live[k]) {
+                        const u32x4 rb = load16(br + chunk_col<L, W>(k, w, l));  // re-used by every batch entry
+                        float f[8], g[8];
+                        unpack8<DT>(raw[k], f);
+                        unpack8<DT>(rb, g);
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) f[j] = f[j] + g[j];
+                        raw[k] = pack8<DT>(f);
+                    }
+                }
+            }
+            if (slopes != nullptr) {
+                const float slope = Half2<DT>::round(slopes[h]);
+#pragma unroll
+                for (int k = 0; k < K; ++k) {
+                    const uint32_t col = chunk_col<L, W>(k, w, l);
+                    if (live[k] && col <= qi) {
+                        float f[8];
+                        unpack8<DT>(raw[k], f);
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) {
+                            if (col + j <= qi) {
+                                const float dist = Half2<DT>::round(-(float)((int)qi - (int)(col + j)));
+                                f[j] = Half2<DT>::round(f[j] + Half2<DT>::round(dist * slope));
+                            }
+                        }
+                        raw[k] = pack8<DT>(f);
+                    }
+                }
+            }
         }
 
         // Chunks whose eight columns are all masked hold eight copies of the fill value:
@@ -515,7 +571,7 @@ softmax_bwd_kernel(uint16_t* dx, const uint16_t* dy, const uint16_t* y, float sc
     Band band;
     if constexpr (CAUSAL) {
         band = causal_band(q, window, ok,
-                           (EXTRA == kPerHead && ok) ? key_limit(key_lengths, mat, heads) : 0xffffffffu);
+                           ((EXTRA & kPerHead) != 0 && ok) ? key_limit(key_lengths, mat, heads) : 0xffffffffu);
     } else {
         band.lo = 0;
         band.hi = ok ? n : 0;
@@ -533,7 +589,7 @@ softmax_bwd_kernel(uint16_t* dx, const uint16_t* dy, const uint16_t* y, float sc
         if ((act >> k & 1u) && col < band.hi && col + 8 > band.lo) {
             rg[k] = load16_stream(dy + base + col);
             ry[k] = load16_stream(y + base + col);
-            if constexpr (EXTRA == kDropout) {
+            if constexpr ((EXTRA & kDropout) != 0) {
                 float f[8];
                 unpack8<DT>(rg[k], f);
                 const Philox rnd = dropout_bits(dk, (uint64_t)base + col);
@@ -635,6 +691,7 @@ scalar_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
     uint64_t lo = 0, hi = n;
     float slope = 0.0f;
     const uint16_t* br = nullptr;
+    uint64_t key_end = ~(uint64_t)0;  // MODE 1: keys at or beyond it count as masked
     if (MODE == 0) {
         hi = min(q + 1, (uint64_t)key_limit(key_lengths, (uint32_t)(row / sq), heads));
         lo = (q > window) ? q - window : 0;
@@ -642,18 +699,22 @@ scalar_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
         if (bias != nullptr) br = bias + (((row / sq) % heads) * sq + q) * n;
     } else {
         const uint64_t bi = row / (sq * np);
+        const uint64_t head = (row / sq) % np;
         mrow = mask + (mask_per_batch ? (bi * sq + q) : q) * n;
+        if (slopes != nullptr) slope = Half2<DT>::round(slopes[head]);
+        if (bias != nullptr) br = bias + (head * sq + q) * n;
+        if (key_lengths != nullptr) key_end = key_limit(key_lengths, (uint32_t)bi, 1);
     }
     // scaled logit of column c (lo <= c < hi)
     auto logit = [&](uint64_t c) {
         float f = Half2<DT>::from_bits(xr[c]);
-        if (MODE == 0 && br != nullptr) f = Half2<DT>::round(f + Half2<DT>::from_bits(br[c]));
-        if (MODE == 0 && slopes != nullptr) {
+        if (br != nullptr) f = Half2<DT>::round(f + Half2<DT>::from_bits(br[c]));
+        if (slopes != nullptr && (MODE == 0 || c <= q)) {
             const float dist = Half2<DT>::round(-(float)((int64_t)q - (int64_t)c));
             f = Half2<DT>::round(f + Half2<DT>::round(dist * slope));
         }
         float z = f * scale;
-        if (MODE == 1 && mrow[c] == 1) z = kMaskFill;
+        if (MODE == 1 && (mrow[c] == 1 || c >= key_end)) z = kMaskFill;
         return z;
     };
 
@@ -851,10 +912,14 @@ static int causal_fwd(void* y, const void* x, float scale, int64_t batches, int6
         using G = Geo<L_, K_, W_, kBlockWaves>;                                            \
         const uint32_t blocks = (uint32_t)((rows + G::kRowsPerBlock - 1) / G::kRowsPerBlock); \
         if (!launch_fits(blocks, G::kThreads)) return NHP_ERR_SHAPE;                       \
-        if (dp != nullptr)                                                                 \
+        const bool per_head = slopes != nullptr || bp != nullptr || kl != nullptr;         \
+        if (dp != nullptr && per_head)                                                     \
+            causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves, kPerHeadDropout><<<blocks, G::kThreads, 0, st>>>( \
+                yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, slopes, bp, kl, heads, dp, dk, zshift); \
+        else if (dp != nullptr)                                                            \
             causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves, kDropout><<<blocks, G::kThreads, 0, st>>>( \
                 yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, nullptr, nullptr, nullptr, 1, dp, dk, zshift); \
-        else if (slopes != nullptr || bp != nullptr || kl != nullptr)                      \
+        else if (per_head)                                                                 \
             causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves, kPerHead><<<blocks, G::kThreads, 0, st>>>( \
                 yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, slopes, bp, kl, heads, nullptr, dk, zshift); \
         else                                                                               \
@@ -889,7 +954,11 @@ static int softmax_bwd(void* dx, const void* dy, const void* y, float scale, int
         using G = Geo<L_, K_, W_, kBlockWaves>;                                            \
         const uint32_t blocks = (uint32_t)((rows + G::kRowsPerBlock - 1) / G::kRowsPerBlock); \
         if (!launch_fits(blocks, G::kThreads)) return NHP_ERR_SHAPE;                       \
-        if (dropout)                                                                       \
+        if (dropout && CAUSAL && kl != nullptr)                                            \
+            softmax_bwd_kernel<DT, L_, K_, W_, kBlockWaves, CAUSAL, CAUSAL ? kPerHeadDropout : kDropout> \
+                <<<blocks, G::kThreads, 0, st>>>(dxp, dyp, yp, scale, (uint32_t)rows, (uint32_t)n, \
+                                                 (uint32_t)rows_per_matrix, window, kl, heads, dk, zshift); \
+        else if (dropout)                                                                  \
             softmax_bwd_kernel<DT, L_, K_, W_, kBlockWaves, CAUSAL, kDropout>                      \
                 <<<blocks, G::kThreads, 0, st>>>(dxp, dyp, yp, scale, (uint32_t)rows, (uint32_t)n, \
                                                      (uint32_t)rows_per_matrix, window, nullptr, 1, dk, zshift); \
@@ -917,10 +986,18 @@ static int softmax_bwd(void* dx, const void* dy, const void* y, float scale, int
 // more make the access order less sequential and measured slower.
 static uint32_t pick_heads_per_wave(int64_t np) { return (uint32_t)(np < 2 ? np : 2); }
 
+// The extras of the padding-mask forward (all optional).
+struct MaskedExtras {
+    const float* slopes = nullptr;       // [np] AliBi slopes (needs sq == sk)
+    const void* bias = nullptr;          // [np, sq, sk] in the scores' dtype
+    const int32_t* key_lengths = nullptr;  // [b]
+    bool any() const { return slopes != nullptr || bias != nullptr || key_lengths != nullptr; }
+};
+
 template <int DT>
 static int masked_fwd(void* y, const void* x, const uint8_t* mask, float scale, int64_t b, int64_t np,
                       int64_t sq, int64_t n, int64_t pad_batches, hipStream_t st, void* dropped = nullptr,
-                      const DropoutKey* drop = nullptr)
+                      const DropoutKey* drop = nullptr, const MaskedExtras& ex = MaskedExtras{})
 {
     launch_prepare();
     uint16_t* dp = static_cast<uint16_t*>(dropped);
@@ -930,33 +1007,40 @@ static int masked_fwd(void* y, const void* x, const uint8_t* mask, float scale, 
     RowPlan p;
     uint16_t* yp = static_cast<uint16_t*>(y);
     const uint16_t* xp = static_cast<const uint16_t*>(x);
+    const uint16_t* bp = static_cast<const uint16_t*>(ex.bias);
     const bool mask_ok = (reinterpret_cast<uintptr_t>(mask) & 7u) == 0;
-    if (plan_row(n, kMaskedFwd, p) && aligned16(x) && aligned16(y) && aligned16(dropped) && mask_ok) {
+    if (plan_row(n, kMaskedFwd, p) && aligned16(x) && aligned16(y) && aligned16(dropped) && aligned16(ex.bias) && mask_ok) {
+#define LAUNCH_MASKED(L_, K_, W_, DROP_, PH_)                                                         \
+    masked_fwd_kernel<DT, L_, K_, W_, kBlockWaves, DROP_, PH_><<<(uint32_t)(rb * hgs), Geo<L_, K_, W_, kBlockWaves>::kThreads, 0, st>>>( \
+        yp, xp, mask, scale, (uint32_t)bq_rows, (uint32_t)sq, (uint32_t)np, (uint32_t)n, hpw, hgs, per_batch, \
+        (uint32_t)rb, (uint32_t)tile, DROP_ ? dp : nullptr, dk, ex.slopes, bp, ex.key_lengths)
 #define CALL(L_, K_, W_)                                                                   \
     {                                                                                      \
         using G = Geo<L_, K_, W_, kBlockWaves>;                                            \
         const int64_t rb = (bq_rows + G::kRowsPerBlock - 1) / G::kRowsPerBlock;            \
-        const uint32_t hpw = (uint32_t)NHP_TUNED_INT("NHP_HPW", (int)pick_heads_per_wave(np));       \
+        const uint32_t hpw = (uint32_t)NHP_TUNED_INT("NHP_HPW", (int)pick_heads_per_wave(np)); \
         const uint32_t hgs = (uint32_t)((np + hpw - 1) / hpw);                             \
         if (rb * hgs >= kMaxRows || !launch_fits(rb * hgs, G::kThreads)) return NHP_ERR_SHAPE; \
         int64_t tile = NHP_TUNED_INT("NHP_MASK_TILE", (int)((sq + G::kRowsPerBlock - 1) / G::kRowsPerBlock)); \
         if (tile < 1) tile = 1;                                                            \
         if (tile > rb) tile = rb;                                                          \
-        if (dp != nullptr)                                                                 \
-            masked_fwd_kernel<DT, L_, K_, W_, kBlockWaves, true><<<(uint32_t)(rb * hgs), G::kThreads, 0, st>>>( \
-                yp, xp, mask, scale, (uint32_t)bq_rows, (uint32_t)sq, (uint32_t)np, (uint32_t)n, hpw, hgs, \
-                per_batch, (uint32_t)rb, (uint32_t)tile, dp, dk);                          \
+        if (dp != nullptr && ex.any())                                                     \
+            LAUNCH_MASKED(L_, K_, W_, true, true);                                                     \
+        else if (dp != nullptr)                                                            \
+            LAUNCH_MASKED(L_, K_, W_, true, false);                                                    \
+        else if (ex.any())                                                                 \
+            LAUNCH_MASKED(L_, K_, W_, false, true);                                                    \
         else                                                                               \
-            masked_fwd_kernel<DT, L_, K_, W_, kBlockWaves, false><<<(uint32_t)(rb * hgs), G::kThreads, 0, st>>>( \
-                yp, xp, mask, scale, (uint32_t)bq_rows, (uint32_t)sq, (uint32_t)np, (uint32_t)n, hpw, hgs, \
-                per_batch, (uint32_t)rb, (uint32_t)tile, nullptr, dk);                     \
+            LAUNCH_MASKED(L_, K_, W_, false, false);                                                   \
     }
         NHP_FOR_PLAN(p);
 #undef CALL
+#undef LAUNCH_MASKED
     } else {
         if (!launch_fits(b * np * sq, kScalarThreads)) return NHP_ERR_SHAPE;
         scalar_fwd_kernel<DT, 1><<<(uint32_t)(b * np * sq), kScalarThreads, 0, st>>>(
-            yp, xp, mask, scale, (uint64_t)n, (uint64_t)sq, (uint64_t)np, per_batch, kNoWindow, nullptr, nullptr, nullptr, 1, dp, dk);
+            yp, xp, mask, scale, (uint64_t)n, (uint64_t)sq, (uint64_t)np, per_batch, kNoWindow, ex.slopes, bp,
+            ex.key_lengths, 1, dp, dk);
     }
     return launch_result();
 }
@@ -968,6 +1052,17 @@ using namespace nhp;
 extern "C" {
 
 int64_t nhp_softmax_max_resident_row(void) { return kMaxResidentRow; }
+
+int nhp_softmax_geometry(int64_t row_len, int kind, int* lanes, int* chunks, int* waves)
+{
+    static const RowKind kKinds[] = {kCausalFwd, kCausalFwdExtra, kCausalBwd, kMaskedFwd, kMaskedBwd};
+    RowPlan p;
+    if (kind < 0 || kind > 4 || !plan_row(row_len, kKinds[kind], p)) return NHP_ERR_SHAPE;
+    if (lanes) *lanes = p.L;
+    if (chunks) *chunks = p.K;
+    if (waves) *waves = p.W;
+    return NHP_OK;
+}
 
 // log2 of a block size given as 0 (no blocks: 0) or a power of two >= 8; -1 for anything else
 static int block_shift(int64_t zero_block)
@@ -1052,24 +1147,37 @@ int nhp_causal_softmax_bwd(void* dx, const void* dy, const void* y, float scale,
     return nhp_causal_softmax_ex_bwd(dx, dy, y, scale, attn_batches, seq_len, -1, nullptr, 1, dtype, stream);
 }
 
-int nhp_causal_softmax_dropout_blocks_fwd(void* dropped, void* y, const void* x, float scale, int64_t attn_batches,
-                                          int64_t seq_len, int64_t window, int64_t zero_block, float p, uint64_t seed,
-                                          uint64_t offset, int dtype, void* stream)
+int nhp_causal_softmax_ex_dropout_fwd(void* dropped, void* y, const void* x, float scale, int64_t attn_batches,
+                                      int64_t seq_len, int64_t window, int64_t zero_block, const float* alibi_slopes,
+                                      const void* bias, const int32_t* key_lengths, int64_t heads, float p,
+                                      uint64_t seed, uint64_t offset, int dtype, void* stream)
 {
     if (dtype != NHP_F16 && dtype != NHP_BF16) return NHP_ERR_DTYPE;
     const int zshift = block_shift(zero_block);
     if (attn_batches < 0 || seq_len < 0 || !(p >= 0.0f && p < 1.0f) || zshift < 0) return NHP_ERR_SHAPE;
+    const bool per_head = alibi_slopes != nullptr || bias != nullptr || key_lengths != nullptr;
+    if (per_head && (heads < 1 || attn_batches % heads != 0)) return NHP_ERR_SHAPE;
+    if (bias != nullptr && (bias == y || bias == dropped)) return NHP_ERR_ALIAS;
     if (attn_batches == 0 || seq_len == 0) return NHP_OK;
     if (attn_batches > kMaxRows / seq_len - 1) return NHP_ERR_SHAPE;
     if (!x || !y || !dropped) return NHP_ERR_NULL;
     if (dropped == y || dropped == x) return NHP_ERR_ALIAS;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const uint32_t win = (window < 0 || window >= seq_len) ? kNoWindow : (uint32_t)window;
+    const uint32_t hd = per_head ? (uint32_t)heads : 1u;
     const DropoutKey dk = make_dropout_key(p, seed, offset);
-    return dtype == NHP_BF16 ? causal_fwd<NHP_BF16>(y, x, scale, attn_batches, seq_len, win, nullptr, nullptr, nullptr, 1,
-                                                    st, dropped, &dk, (uint32_t)zshift)
-                             : causal_fwd<NHP_F16>(y, x, scale, attn_batches, seq_len, win, nullptr, nullptr, nullptr, 1,
-                                                   st, dropped, &dk, (uint32_t)zshift);
+    return dtype == NHP_BF16 ? causal_fwd<NHP_BF16>(y, x, scale, attn_batches, seq_len, win, alibi_slopes, bias, key_lengths,
+                                                    hd, st, dropped, &dk, (uint32_t)zshift)
+                             : causal_fwd<NHP_F16>(y, x, scale, attn_batches, seq_len, win, alibi_slopes, bias, key_lengths,
+                                                   hd, st, dropped, &dk, (uint32_t)zshift);
+}
+
+int nhp_causal_softmax_dropout_blocks_fwd(void* dropped, void* y, const void* x, float scale, int64_t attn_batches,
+                                          int64_t seq_len, int64_t window, int64_t zero_block, float p, uint64_t seed,
+                                          uint64_t offset, int dtype, void* stream)
+{
+    return nhp_causal_softmax_ex_dropout_fwd(dropped, y, x, scale, attn_batches, seq_len, window, zero_block, nullptr,
+                                             nullptr, nullptr, 1, p, seed, offset, dtype, stream);
 }
 
 int nhp_causal_softmax_dropout_fwd(void* dropped, void* y, const void* x, float scale, int64_t attn_batches,
@@ -1080,13 +1188,14 @@ int nhp_causal_softmax_dropout_fwd(void* dropped, void* y, const void* x, float 
                                                  dtype, stream);
 }
 
-int nhp_causal_softmax_dropout_blocks_bwd(void* dx, const void* dy, const void* y, float scale, int64_t attn_batches,
-                                          int64_t seq_len, int64_t window, int64_t zero_block, float p, uint64_t seed,
-                                          uint64_t offset, int dtype, void* stream)
+int nhp_causal_softmax_ex_dropout_bwd(void* dx, const void* dy, const void* y, float scale, int64_t attn_batches,
+                                      int64_t seq_len, int64_t window, int64_t zero_block, const int32_t* key_lengths,
+                                      int64_t heads, float p, uint64_t seed, uint64_t offset, int dtype, void* stream)
 {
     if (dtype != NHP_F16 && dtype != NHP_BF16) return NHP_ERR_DTYPE;
     const int zshift = block_shift(zero_block);
     if (attn_batches < 0 || seq_len < 0 || !(p >= 0.0f && p < 1.0f) || zshift < 0) return NHP_ERR_SHAPE;
+    if (key_lengths != nullptr && (heads < 1 || attn_batches % heads != 0)) return NHP_ERR_SHAPE;
     if (attn_batches == 0 || seq_len == 0) return NHP_OK;
     if (attn_batches > kMaxRows / seq_len - 1) return NHP_ERR_SHAPE;
     if (!dx || !dy || !y) return NHP_ERR_NULL;
@@ -1094,10 +1203,19 @@ int nhp_causal_softmax_dropout_blocks_bwd(void* dx, const void* dy, const void* 
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int64_t rows = attn_batches * seq_len;
     const uint32_t win = (window < 0 || window >= seq_len) ? kNoWindow : (uint32_t)window;
+    const uint32_t hd = key_lengths != nullptr ? (uint32_t)heads : 1u;
     const DropoutKey dk = make_dropout_key(p, seed, offset);
     return dtype == NHP_BF16
-               ? softmax_bwd<NHP_BF16, true>(dx, dy, y, scale, rows, seq_len, seq_len, win, nullptr, 1, st, &dk, (uint32_t)zshift)
-               : softmax_bwd<NHP_F16, true>(dx, dy, y, scale, rows, seq_len, seq_len, win, nullptr, 1, st, &dk, (uint32_t)zshift);
+               ? softmax_bwd<NHP_BF16, true>(dx, dy, y, scale, rows, seq_len, seq_len, win, key_lengths, hd, st, &dk, (uint32_t)zshift)
+               : softmax_bwd<NHP_F16, true>(dx, dy, y, scale, rows, seq_len, seq_len, win, key_lengths, hd, st, &dk, (uint32_t)zshift);
+}
+
+int nhp_causal_softmax_dropout_blocks_bwd(void* dx, const void* dy, const void* y, float scale, int64_t attn_batches,
+                                          int64_t seq_len, int64_t window, int64_t zero_block, float p, uint64_t seed,
+                                          uint64_t offset, int dtype, void* stream)
+{
+    return nhp_causal_softmax_ex_dropout_bwd(dx, dy, y, scale, attn_batches, seq_len, window, zero_block, nullptr, 1, p,
+                                             seed, offset, dtype, stream);
 }
 
 int nhp_causal_softmax_dropout_bwd(void* dx, const void* dy, const void* y, float scale, int64_t attn_batches,
@@ -1108,19 +1226,47 @@ int nhp_causal_softmax_dropout_bwd(void* dx, const void* dy, const void* y, floa
                                                  stream);
 }
 
+// Shared argument checks of the padding-mask forward entry points.
+static int masked_fwd_check(const void* y, const void* x, const uint8_t* mask, int64_t b, int64_t np, int64_t sq,
+                            int64_t sk, int64_t pad_batches, const MaskedExtras& ex, int dtype, bool& empty)
+{
+    empty = false;
+    if (dtype != NHP_F16 && dtype != NHP_BF16) return NHP_ERR_DTYPE;
+    if (b < 0 || np < 0 || sq < 0 || sk < 0) return NHP_ERR_SHAPE;
+    if (ex.slopes != nullptr && sq != sk) return NHP_ERR_SHAPE;  // the AliBi bias is defined on square scores
+    if (b == 0 || np == 0 || sq == 0 || sk == 0) {
+        empty = true;
+        return NHP_OK;
+    }
+    if (pad_batches != 1 && pad_batches != b) return NHP_ERR_PAD_BATCHES;
+    if (b > kMaxRows / np - 1 || b * np > kMaxRows / sq - 1) return NHP_ERR_SHAPE;
+    if (!x || !y || !mask) return NHP_ERR_NULL;
+    if (ex.bias != nullptr && ex.bias == y) return NHP_ERR_ALIAS;
+    return NHP_OK;
+}
+
+int nhp_masked_softmax_ex_fwd(void* y, const void* x, const uint8_t* mask, float scale, int64_t b, int64_t np,
+                              int64_t sq, int64_t sk, int64_t pad_batches, const float* alibi_slopes, const void* bias,
+                              const int32_t* key_lengths, int dtype, void* stream)
+{
+    MaskedExtras ex;
+    ex.slopes = alibi_slopes;
+    ex.bias = bias;
+    ex.key_lengths = key_lengths;
+    bool empty;
+    const int rc = masked_fwd_check(y, x, mask, b, np, sq, sk, pad_batches, ex, dtype, empty);
+    if (rc != NHP_OK || empty) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    return dtype == NHP_BF16 ? masked_fwd<NHP_BF16>(y, x, mask, scale, b, np, sq, sk, pad_batches, st, nullptr, nullptr, ex)
+                             : masked_fwd<NHP_F16>(y, x, mask, scale, b, np, sq, sk, pad_batches, st, nullptr, nullptr, ex);
+}
+
 int nhp_masked_softmax_fwd(void* y, const void* x, const uint8_t* mask, float scale, int64_t b,
                            int64_t np, int64_t sq, int64_t sk, int64_t pad_batches, int dtype,
                            void* stream)
 {
-    if (dtype != NHP_F16 && dtype != NHP_BF16) return NHP_ERR_DTYPE;
-    if (b < 0 || np < 0 || sq < 0 || sk < 0) return NHP_ERR_SHAPE;
-    if (b == 0 || np == 0 || sq == 0 || sk == 0) return NHP_OK;
-    if (pad_batches != 1 && pad_batches != b) return NHP_ERR_PAD_BATCHES;
-    if (b > kMaxRows / np - 1 || b * np > kMaxRows / sq - 1) return NHP_ERR_SHAPE;
-    if (!x || !y || !mask) return NHP_ERR_NULL;
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    return dtype == NHP_BF16 ? masked_fwd<NHP_BF16>(y, x, mask, scale, b, np, sq, sk, pad_batches, st)
-                             : masked_fwd<NHP_F16>(y, x, mask, scale, b, np, sq, sk, pad_batches, st);
+    return nhp_masked_softmax_ex_fwd(y, x, mask, scale, b, np, sq, sk, pad_batches, nullptr, nullptr, nullptr, dtype,
+                                     stream);
 }
 
 int nhp_masked_softmax_bwd(void* dx, const void* dy, const void* y, float scale, int64_t rows, int64_t sk,
@@ -1138,21 +1284,33 @@ int nhp_masked_softmax_bwd(void* dx, const void* dy, const void* y, float scale,
                              : softmax_bwd<NHP_F16, false>(dx, dy, y, scale, rows, sk, rows, kNoWindow, nullptr, 1, st);
 }
 
+int nhp_masked_softmax_ex_dropout_fwd(void* dropped, void* y, const void* x, const uint8_t* mask, float scale,
+                                      int64_t b, int64_t np, int64_t sq, int64_t sk, int64_t pad_batches,
+                                      const float* alibi_slopes, const void* bias, const int32_t* key_lengths, float p,
+                                      uint64_t seed, uint64_t offset, int dtype, void* stream)
+{
+    MaskedExtras ex;
+    ex.slopes = alibi_slopes;
+    ex.bias = bias;
+    ex.key_lengths = key_lengths;
+    bool empty;
+    if (!(p >= 0.0f && p < 1.0f)) return (dtype != NHP_F16 && dtype != NHP_BF16) ? NHP_ERR_DTYPE : NHP_ERR_SHAPE;
+    const int rc = masked_fwd_check(y, x, mask, b, np, sq, sk, pad_batches, ex, dtype, empty);
+    if (rc != NHP_OK || empty) return rc;
+    if (!dropped) return NHP_ERR_NULL;
+    if (dropped == y || dropped == x || (bias != nullptr && dropped == bias)) return NHP_ERR_ALIAS;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const DropoutKey dk = make_dropout_key(p, seed, offset);
+    return dtype == NHP_BF16 ? masked_fwd<NHP_BF16>(y, x, mask, scale, b, np, sq, sk, pad_batches, st, dropped, &dk, ex)
+                             : masked_fwd<NHP_F16>(y, x, mask, scale, b, np, sq, sk, pad_batches, st, dropped, &dk, ex);
+}
+
 int nhp_masked_softmax_dropout_fwd(void* dropped, void* y, const void* x, const uint8_t* mask, float scale,
                                    int64_t b, int64_t np, int64_t sq, int64_t sk, int64_t pad_batches, float p,
                                    uint64_t seed, uint64_t offset, int dtype, void* stream)
 {
-    if (dtype != NHP_F16 && dtype != NHP_BF16) return NHP_ERR_DTYPE;
-    if (b < 0 || np < 0 || sq < 0 || sk < 0 || !(p >= 0.0f && p < 1.0f)) return NHP_ERR_SHAPE;
-    if (b == 0 || np == 0 || sq == 0 || sk == 0) return NHP_OK;
-    if (pad_batches != 1 && pad_batches != b) return NHP_ERR_PAD_BATCHES;
-    if (b > kMaxRows / np - 1 || b * np > kMaxRows / sq - 1) return NHP_ERR_SHAPE;
-    if (!x || !y || !mask || !dropped) return NHP_ERR_NULL;
-    if (dropped == y || dropped == x) return NHP_ERR_ALIAS;
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    const DropoutKey dk = make_dropout_key(p, seed, offset);
-    return dtype == NHP_BF16 ? masked_fwd<NHP_BF16>(y, x, mask, scale, b, np, sq, sk, pad_batches, st, dropped, &dk)
-                             : masked_fwd<NHP_F16>(y, x, mask, scale, b, np, sq, sk, pad_batches, st, dropped, &dk);
+    return nhp_masked_softmax_ex_dropout_fwd(dropped, y, x, mask, scale, b, np, sq, sk, pad_batches, nullptr, nullptr,
+                                             nullptr, p, seed, offset, dtype, stream);
 }
 
 int nhp_masked_softmax_dropout_bwd(void* dx, const void* dy, const void* y, float scale, int64_t rows, int64_t sk,

@@ -53,6 +53,10 @@ def _declare(lib):
         "nhp_masked_softmax_dropout_fwd": ([vp, vp, vp, vp, f32, i64, i64, i64, i64, i64, f32, u64, u64, ci, vp], ci),
         "nhp_masked_softmax_dropout_bwd": ([vp, vp, vp, f32, i64, i64, f32, u64, u64, ci, vp], ci),
         "nhp_masked_softmax_fwd": ([vp, vp, vp, f32, i64, i64, i64, i64, i64, ci, vp], ci),
+        "nhp_masked_softmax_ex_fwd": ([vp, vp, vp, f32, i64, i64, i64, i64, i64, vp, vp, vp, ci, vp], ci),
+        "nhp_masked_softmax_ex_dropout_fwd": ([vp, vp, vp, vp, f32, i64, i64, i64, i64, i64, vp, vp, vp, f32, u64, u64, ci, vp], ci),
+        "nhp_causal_softmax_ex_dropout_fwd": ([vp, vp, vp, f32, i64, i64, i64, i64, vp, vp, vp, i64, f32, u64, u64, ci, vp], ci),
+        "nhp_causal_softmax_ex_dropout_bwd": ([vp, vp, vp, f32, i64, i64, i64, i64, vp, i64, f32, u64, u64, ci, vp], ci),
         "nhp_masked_softmax_bwd": ([vp, vp, vp, f32, i64, i64, ci, vp], ci),
         "nhp_softmax_batch_per_block": ([i64, i64, i64, i64], ci),
         "nhp_rope_cached_fwd": ([vp, vp, vp, vp, i64, i64, i64, i64, i64, p64, p64, ci, ci, vp], ci),

@@ -15,22 +15,23 @@ all of it widening:
   held in registers, longer ones stream);
 * ``scale`` reaches the forward kernel in fp32 (the reference's CUDA dispatcher
   narrows it to the input dtype first);
-* two optional constructor arguments let the causal kernel do by index what its
-  caller otherwise does with tensors: ``sliding_window_width`` (the reference's
-  causal kernel never looks at the mask, so a sliding window is lost on its
-  fused branch) and ``alibi_slopes`` (the AliBi bias is formed inside the kernel
-  instead of by a separate ``scores + alibi_matrix`` pass). Both default to off;
+* two optional constructor arguments let the kernels do by index what their
+  caller otherwise does with tensors: ``sliding_window_width`` (causal kernel; the
+  reference's causal kernel never looks at the mask, so a sliding window is lost on
+  its fused branch) and ``alibi_slopes`` (the AliBi bias is formed inside either
+  kernel instead of by a separate ``scores + alibi_matrix`` pass). Both default to off;
 * ``forward(input, mask, bias=None)``: an optional additive bias ``[1, np, sq, sk]``
   (the relative-position bias the caller adds with ``attention_scores += rpe``)
-  is read by the causal kernel instead of being added in a pass of its own;
+  is read by the kernel beside the scores instead of being added in a pass of its own;
 * ``forward(..., key_lengths=None)``: an integer tensor ``[b]`` of real key counts for
-  right-padded batches. The causal kernel masks the padding keys by index (the
-  reference's ignores the mask, so padding is attended to on its fused branch); the
-  other branches merge ``k >= key_lengths[b]`` into the mask they are given;
+  right-padded batches. Both kernels mask the padding keys by index (the reference's
+  causal kernel ignores the mask, so padding is attended to on its fused branch); the
+  torch branch merges ``k >= key_lengths[b]`` into the mask it is given;
 * constructor argument ``attention_dropout`` (default 0): in training mode the module returns
-  ``dropout(probabilities)``; on the causal fused branch softmax and dropout are one kernel and
-  the keep mask (the library's counter-based generator, seeded from torch's CPU generator) is
-  regenerated in the backward instead of being stored. The caller must then not apply its own dropout.
+  ``dropout(probabilities)``; on the fused branches softmax and dropout are one kernel, with or
+  without the extras above, and the keep mask (the library's counter-based generator, seeded from
+  torch's CPU generator) is regenerated in the backward instead of being stored. The caller must
+  then not apply its own dropout.
 """
 import enum
 
@@ -82,12 +83,12 @@ class ScaledUpperTriangMaskedSoftmax(torch.autograd.Function):
         grad_bias = None
         if ctx.bias_shape is not None and ctx.needs_input_grad[4]:
             # the bias is shared by the batch: its gradient is the batch sum of the score gradient
-            heads, sq, sk = ctx.bias_shape[-3:]
             full = grad
             if ctx.zero_block:
                 # the blocks the kernel did not write hold no gradient: leave them out of the sum
+                sq = ctx.bias_shape[-2]
                 full = torch.where(_written_blocks(sq, ctx.zero_block, ctx.window, grad.device), grad, torch.zeros_like(grad))
-            grad_bias = full.view(-1, heads, sq, sk).sum(dim=0).view(ctx.bias_shape)
+            grad_bias = _batch_sum(full, ctx.bias_shape)
         return grad, None, None, None, grad_bias, None, None
 
 
@@ -102,17 +103,28 @@ def _written_blocks(seq_len, zero_block, window, device):
     return (k < hi) & (k >= lo)
 
 
+def _batch_sum(grad, bias_shape):
+    """Gradient of a bias shared by the batch: the batch sum of the score gradient, in the bias's shape."""
+    heads, sq, sk = bias_shape[-3:]
+    return grad.view(-1, heads, sq, sk).sum(dim=0).view(bias_shape)
+
+
 class ScaledUpperTriangMaskedSoftmaxDropout(torch.autograd.Function):
-    """``dropout(softmax(scale * x))`` under the causal mask in one kernel forward and one backward.
+    """``dropout(softmax(scale * x))`` under the causal mask in one kernel forward and one backward, with the
+    same optional extras as ``ScaledUpperTriangMaskedSoftmax``.
     No counterpart in the reference, which runs ``torch.nn.Dropout`` on the probabilities."""
 
     @staticmethod
-    def forward(ctx, inputs, scale, prob, seed, window=None, zero_block=0):
+    def forward(ctx, inputs, scale, prob, seed, window=None, zero_block=0, alibi_slopes=None, bias=None,
+                key_lengths=None):
         import scaled_upper_triang_masked_softmax_cuda as kernels
 
         factor = _scale_tensor(scale)
-        dropped, probs = kernels.forward_dropout(inputs, factor[0], prob, seed, window, zero_block)
+        dropped, probs = kernels.forward_dropout(inputs, factor[0], prob, seed, window, zero_block, alibi_slopes, bias,
+                                                 key_lengths)
         ctx.conf = (float(prob), int(seed), window, zero_block)
+        ctx.key_lengths = key_lengths
+        ctx.bias_shape = None if bias is None else tuple(bias.shape)
         ctx.save_for_backward(probs, factor)
         return dropped
 
@@ -122,20 +134,31 @@ class ScaledUpperTriangMaskedSoftmaxDropout(torch.autograd.Function):
 
         probs, factor = ctx.saved_tensors
         prob, seed, window, zero_block = ctx.conf
-        grad = kernels.backward_dropout(output_grads, probs, factor[0], prob, seed, window, zero_block)
-        return grad, None, None, None, None, None
+        grad = kernels.backward_dropout(output_grads, probs, factor[0], prob, seed, window, zero_block, ctx.key_lengths)
+        grad_bias = None
+        if ctx.bias_shape is not None and ctx.needs_input_grad[7]:
+            full = grad
+            if zero_block:
+                sq = ctx.bias_shape[-2]
+                full = torch.where(_written_blocks(sq, zero_block, window, grad.device), grad, torch.zeros_like(grad))
+            grad_bias = _batch_sum(full, ctx.bias_shape)
+        return grad, None, None, None, None, None, None, grad_bias, None
 
 
 class ScaledMaskedSoftmax(torch.autograd.Function):
     """``softmax(where(mask, -10000, scale * x))`` over the last dimension of
-    ``[b, np, sq, sk]`` scores with a ``[1 or b, 1, sq, sk]`` mask."""
+    ``[b, np, sq, sk]`` scores with a ``[1 or b, 1, sq, sk]`` mask.
+
+    ``alibi_slopes``, ``bias`` and ``key_lengths`` are optional extras (see
+    ``scaled_masked_softmax_cuda.forward``); the reference signature is ``apply(inputs, mask, scale)``."""
 
     @staticmethod
-    def forward(ctx, inputs, mask, scale):
+    def forward(ctx, inputs, mask, scale, alibi_slopes=None, bias=None, key_lengths=None):
         import scaled_masked_softmax_cuda as kernels
 
         factor = _scale_tensor(scale)
-        out = kernels.forward(inputs, mask, factor[0])
+        out = kernels.forward(inputs, mask, factor[0], alibi_slopes, bias, key_lengths)
+        ctx.bias_shape = None if bias is None else tuple(bias.shape)
         ctx.save_for_backward(out, factor)
         return out
 
@@ -144,7 +167,11 @@ class ScaledMaskedSoftmax(torch.autograd.Function):
         import scaled_masked_softmax_cuda as kernels
 
         out, factor = ctx.saved_tensors
-        return kernels.backward(output_grads, out, factor[0]), None, None
+        grad = kernels.backward(output_grads, out, factor[0])
+        grad_bias = None
+        if ctx.bias_shape is not None and ctx.needs_input_grad[4]:
+            grad_bias = _batch_sum(grad, ctx.bias_shape)
+        return grad, None, None, None, grad_bias, None
 
 
 class ScaledMaskedSoftmaxDropout(torch.autograd.Function):
@@ -152,12 +179,13 @@ class ScaledMaskedSoftmaxDropout(torch.autograd.Function):
     No counterpart in the reference, which runs ``torch.nn.Dropout`` on the probabilities."""
 
     @staticmethod
-    def forward(ctx, inputs, mask, scale, prob, seed):
+    def forward(ctx, inputs, mask, scale, prob, seed, alibi_slopes=None, bias=None, key_lengths=None):
         import scaled_masked_softmax_cuda as kernels
 
         factor = _scale_tensor(scale)
-        dropped, probs = kernels.forward_dropout(inputs, mask, factor[0], prob, seed)
+        dropped, probs = kernels.forward_dropout(inputs, mask, factor[0], prob, seed, alibi_slopes, bias, key_lengths)
         ctx.conf = (float(prob), int(seed))
+        ctx.bias_shape = None if bias is None else tuple(bias.shape)
         ctx.save_for_backward(probs, factor)
         return dropped
 
@@ -167,7 +195,11 @@ class ScaledMaskedSoftmaxDropout(torch.autograd.Function):
 
         probs, factor = ctx.saved_tensors
         prob, seed = ctx.conf
-        return kernels.backward_dropout(output_grads, probs, factor[0], prob, seed), None, None, None, None
+        grad = kernels.backward_dropout(output_grads, probs, factor[0], prob, seed)
+        grad_bias = None
+        if ctx.bias_shape is not None and ctx.needs_input_grad[6]:
+            grad_bias = _batch_sum(grad, ctx.bias_shape)
+        return grad, None, None, None, None, None, grad_bias, None
 
 
 class FusedScaleMaskSoftmax(nn.Module):
@@ -190,7 +222,7 @@ class FusedScaleMaskSoftmax(nn.Module):
             roundings, so the caller must not add it.
         attention_dropout: (extension) dropout probability applied to the
             probabilities in training mode; fused with the softmax on both
-            kernel branches (unless a bias, AliBi or key lengths are in play).
+            kernel branches, whatever else (bias, AliBi, key lengths) is in play.
             The caller must not apply its own dropout.
     """
 
@@ -232,40 +264,18 @@ class FusedScaleMaskSoftmax(nn.Module):
             # the last rows of a longer causal matrix (new positions after cached keys): the triangle the causal
             # kernel implies does not apply, the caller's mask does. The reference asserts sq == sk here
             # (fused_softmax.py:173) when its gate lets such a shape through.
-            probs = self._forward_rectangular(input, mask, bias, key_lengths)
+            if self._rectangular_kernel_available(mask, *input.size()):
+                return self._forward_general(input, mask, bias, key_lengths, dropout)
         elif self.is_kernel_available(mask, *input.size()):
-            plain_causal = (self.upper_triang_mask_fusion and bias is None and key_lengths is None
-                            and self.alibi_slopes is None)
-            if dropout > 0.0 and plain_causal:
-                b, np, sq, sk = input.size()
-                assert sq == sk, "causal mask is only for self attention"
-                factor = 1.0 if self.scale is None else self.scale
-                seed = int(torch.empty((), dtype=torch.int64).random_().item())  # CPU generator: no device sync
-                probs = ScaledUpperTriangMaskedSoftmaxDropout.apply(input.view(b * np, sq, sk), factor, dropout, seed,
-                                                                    self.sliding_window_width, zero_block)
-                return probs.view(b, np, sq, sk)
-            if (dropout > 0.0 and self.general_mask_fusion and bias is None and key_lengths is None
-                    and self.alibi_slopes is None):
-                factor = 1.0 if self.scale is None else self.scale
-                seed = int(torch.empty((), dtype=torch.int64).random_().item())
-                return ScaledMaskedSoftmaxDropout.apply(input, mask, factor, dropout, seed)
-            probs = self.forward_fused_softmax(input, mask, bias, key_lengths, zero_block)
-        else:
-            probs = self.forward_torch_softmax(input, mask, bias, key_lengths)
+            return self.forward_fused_softmax(input, mask, bias, key_lengths, zero_block, dropout)
+        probs = self.forward_torch_softmax(input, mask, bias, key_lengths)
         if dropout > 0.0:
             probs = torch.nn.functional.dropout(probs, p=dropout, training=True)
         return probs
 
-    def _forward_rectangular(self, input, mask, bias, key_lengths):
-        b, np, sq, sk = input.size()
-        general_ok = (self.input_in_float16 and mask is not None and sk > 16 and sq % 4 == 0 and (b * np) % 4 == 0
-                      and sq % self.get_batch_per_block(sq, sk, b, np) == 0 and self.alibi_slopes is None)
-        if not general_ok:
-            return self.forward_torch_softmax(input, mask, bias, key_lengths)
-        mask = self._mask_with_padding(mask, key_lengths, b, sk)
-        if bias is not None:
-            input = input + bias
-        return ScaledMaskedSoftmax.apply(input, mask, 1.0 if self.scale is None else self.scale)
+    def _rectangular_kernel_available(self, mask, b, np, sq, sk):
+        return (self.input_in_float16 and mask is not None and sk > 16 and sq % 4 == 0 and (b * np) % 4 == 0
+                and sq % self.get_batch_per_block(sq, sk, b, np) == 0 and self.alibi_slopes is None)
 
     def is_kernel_available(self, mask, b, np, sq, sk):
         """The reference's conditions (fused_softmax.py:148-168) without ``sk <= 2048``."""
@@ -295,29 +305,52 @@ class FusedScaleMaskSoftmax(nn.Module):
         padding = keys.view(1, 1, 1, sk) >= key_lengths.to(mask.device).view(b, 1, 1, 1)
         return (mask.bool() | padding).contiguous()
 
-    def forward_fused_softmax(self, input, mask, bias=None, key_lengths=None, zero_block=0):
+    @staticmethod
+    def _dropout_seed():
+        # drawn from torch's CPU generator: repeatable under torch.manual_seed, no device synchronisation
+        return int(torch.empty((), dtype=torch.int64).random_().item())
+
+    def _slopes_on(self, device):
+        slopes = self.alibi_slopes
+        if slopes is not None and slopes.device != device:
+            slopes = slopes.to(device)
+        return slopes
+
+    def _forward_general(self, input, mask, bias, key_lengths, dropout):
+        """The padding-mask kernel; bias, AliBi, key lengths and dropout all happen inside it."""
+        b, np, sq, sk = input.size()
+        factor = 1.0 if self.scale is None else self.scale
+        if bias is not None:
+            assert bias.shape[-3:] == (np, sq, sk) and bias.numel() == np * sq * sk, "bias must be [1, np, sq, sk]"
+        if key_lengths is not None:
+            assert key_lengths.shape == (b,), "key_lengths must be [b]"
+        slopes = self._slopes_on(input.device)
+        if dropout > 0.0:
+            return ScaledMaskedSoftmaxDropout.apply(input, mask, factor, dropout, self._dropout_seed(), slopes, bias,
+                                                    key_lengths)
+        return ScaledMaskedSoftmax.apply(input, mask, factor, slopes, bias, key_lengths)
+
+    def forward_fused_softmax(self, input, mask, bias=None, key_lengths=None, zero_block=0, dropout=0.0):
         b, np, sq, sk = input.size()
         factor = 1.0 if self.scale is None else self.scale
         if not self.upper_triang_mask_fusion:
-            mask = self._mask_with_padding(mask, key_lengths, b, sk)
-            if bias is not None:
-                input = input + bias
-            if self.alibi_slopes is not None:
-                input = self._add_alibi(input)
-            return ScaledMaskedSoftmax.apply(input, mask, factor)
+            return self._forward_general(input, mask, bias, key_lengths, dropout)
 
         assert sq == sk, "causal mask is only for self attention"
-        slopes = self.alibi_slopes
-        if slopes is not None and slopes.device != input.device:
-            slopes = slopes.to(input.device)
+        slopes = self._slopes_on(input.device)
         # the kernel takes [attn_batches, sq, sk]; the causal mask is implied by the indices
         flat = input.view(b * np, sq, sk)
         if bias is not None:
             assert bias.shape[-3:] == (np, sq, sk) and bias.numel() == np * sq * sk, "bias must be [1, np, sq, sk]"
         if key_lengths is not None:
             assert key_lengths.shape == (b,), "key_lengths must be [b]"
-        probs = ScaledUpperTriangMaskedSoftmax.apply(flat, factor, self.sliding_window_width, slopes, bias, key_lengths,
-                                                     zero_block)
+        if dropout > 0.0:
+            probs = ScaledUpperTriangMaskedSoftmaxDropout.apply(flat, factor, dropout, self._dropout_seed(),
+                                                                self.sliding_window_width, zero_block, slopes, bias,
+                                                                key_lengths)
+        else:
+            probs = ScaledUpperTriangMaskedSoftmax.apply(flat, factor, self.sliding_window_width, slopes, bias,
+                                                         key_lengths, zero_block)
         return probs.view(b, np, sq, sk)
 
     def forward_torch_softmax(self, input, mask, bias=None, key_lengths=None):

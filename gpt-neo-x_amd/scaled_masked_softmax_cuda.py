@@ -32,21 +32,60 @@ def _checked_forward_args(input, mask, name):
     return input.contiguous(), mask.contiguous()
 
 
-def forward(input, mask, scale_factor):
+def _extras(x, alibi_slopes, bias, key_lengths, name):
+    """Pointers (and the tensors that keep them alive) of the optional operands of ``forward``."""
+    b, np_, sq, sk = x.shape
+    keep = []
+    slopes_ptr = bias_ptr = lengths_ptr = None
+    if alibi_slopes is not None:
+        if alibi_slopes.dtype != torch.float32 or alibi_slopes.dim() != 1 or alibi_slopes.numel() != np_:
+            raise RuntimeError("alibi_slopes must be a float32 tensor with one slope per head")
+        if sq != sk:
+            raise RuntimeError("the AliBi bias needs query_seq_len == key_seq_len")
+        _hp.require_gpu(alibi_slopes, name)
+        keep.append(alibi_slopes.contiguous())
+        slopes_ptr = keep[-1].data_ptr()
+    if bias is not None:
+        if bias.dim() == 4 and bias.size(0) == 1:
+            bias = bias[0]
+        if bias.shape != (np_, sq, sk) or bias.dtype != x.dtype:
+            raise RuntimeError("bias must be [heads, query_seq_len, key_seq_len] in the dtype of the input")
+        _hp.require_gpu(bias, name)
+        keep.append(bias.contiguous())
+        bias_ptr = keep[-1].data_ptr()
+    if key_lengths is not None:
+        if key_lengths.dim() != 1 or key_lengths.numel() != b or key_lengths.is_floating_point():
+            raise RuntimeError("key_lengths must be an integer tensor with one entry per batch entry")
+        _hp.require_gpu(key_lengths, name)
+        keep.append(key_lengths.to(torch.int32).contiguous())
+        lengths_ptr = keep[-1].data_ptr()
+    return keep, slopes_ptr, bias_ptr, lengths_ptr
+
+
+def forward(input, mask, scale_factor, alibi_slopes=None, bias=None, key_lengths=None):
     """softmax(where(mask == 1, -10000, scale * input)) over the last dim.
 
     input: [b, np, sq, sk] fp16/bf16; mask: [1 or b, 1, sq, sk], one byte per
     element (bool or uint8). Checks follow scaled_masked_softmax.cpp:33-42 and
     scaled_masked_softmax_cuda.cu:46-51; sk is not limited to 2048.
+
+    Three optional arguments go beyond the reference function; each stands for a pass over the scores
+    (or the mask) that the caller otherwise makes first (megatron/model/transformer.py:580-588):
+    alibi_slopes: fp32 [np] on the GPU, needs sq == sk: ``scores + alibi_matrix`` in the storage dtype;
+    bias: [np, sq, sk] (or [1, np, sq, sk]) in the input's dtype: ``scores += bias`` in the storage dtype;
+    key_lengths: integer [b] on the GPU: keys at or beyond a batch entry's length count as masked.
     """
-    x, m = _checked_forward_args(input, mask, "scaled_masked_softmax_cuda.forward")
+    name = "scaled_masked_softmax_cuda.forward"
+    x, m = _checked_forward_args(input, mask, name)
     b, np_, sq, sk = x.shape
+    keep, slopes_ptr, bias_ptr, lengths_ptr = _extras(x, alibi_slopes, bias, key_lengths, name)
     y = torch.empty_like(x)
     with _hp.device_guard(x):
-        rc = _hp.lib().nhp_masked_softmax_fwd(
+        rc = _hp.lib().nhp_masked_softmax_ex_fwd(
             y.data_ptr(), x.data_ptr(), m.data_ptr(), float(scale_factor), b, np_, sq, sk, m.size(0),
-            _hp.dtype_code(x, "forward"), _hp.stream_of(x))
-    _hp.check(rc, "scaled_masked_softmax_cuda.forward")
+            slopes_ptr, bias_ptr, lengths_ptr, _hp.dtype_code(x, "forward"), _hp.stream_of(x))
+    _hp.check(rc, name)
+    del keep
     return y
 
 
@@ -79,7 +118,7 @@ def _check_prob(p, name):
         raise RuntimeError(f"{name}: dropout probability has to be in [0, 1), got {p}")
 
 
-def forward_dropout(input, mask, scale_factor, p, seed):
+def forward_dropout(input, mask, scale_factor, p, seed, alibi_slopes=None, bias=None, key_lengths=None):
     """(not in the reference module) ``forward`` and attention dropout in one kernel: returns
     ``(dropped, probs)`` with ``dropped = keep ? probs / (1 - p) : 0``; the keep mask is generated from
     ``seed`` over the flat element index and is regenerated by ``backward_dropout``."""
@@ -87,13 +126,15 @@ def forward_dropout(input, mask, scale_factor, p, seed):
     _check_prob(p, name)
     x, m = _checked_forward_args(input, mask, name)
     b, np_, sq, sk = x.shape
+    keep, slopes_ptr, bias_ptr, lengths_ptr = _extras(x, alibi_slopes, bias, key_lengths, name)
     y = torch.empty_like(x)
     dropped = torch.empty_like(x)
     with _hp.device_guard(x):
-        rc = _hp.lib().nhp_masked_softmax_dropout_fwd(
+        rc = _hp.lib().nhp_masked_softmax_ex_dropout_fwd(
             dropped.data_ptr(), y.data_ptr(), x.data_ptr(), m.data_ptr(), float(scale_factor), b, np_, sq, sk, m.size(0),
-            float(p), int(seed), 0, _hp.dtype_code(x, name), _hp.stream_of(x))
+            slopes_ptr, bias_ptr, lengths_ptr, float(p), int(seed), 0, _hp.dtype_code(x, name), _hp.stream_of(x))
     _hp.check(rc, name)
+    del keep
     return dropped, y
 
 

@@ -25,6 +25,39 @@ def _key_lengths_arg(key_lengths, attn_batches, heads, who):
     return lengths, lengths.data_ptr(), attn_batches // batch
 
 
+def _per_head_args(x, alibi_slopes, bias, key_lengths, who):
+    """Pointers of the optional per-head operands of the forward kernels, the tensors that keep them alive,
+    and the number of heads per batch entry they imply (None without any of them)."""
+    keep = []
+    slopes_ptr, heads = None, None
+    if alibi_slopes is not None:
+        if alibi_slopes.dtype != torch.float32 or alibi_slopes.dim() != 1:
+            raise RuntimeError("alibi_slopes must be a 1-D float32 tensor")
+        _hp.require_gpu(alibi_slopes, who)
+        alibi_slopes = alibi_slopes.contiguous()
+        keep.append(alibi_slopes)
+        slopes_ptr, heads = alibi_slopes.data_ptr(), alibi_slopes.numel()
+        if heads == 0 or x.size(0) % heads != 0:
+            raise RuntimeError("attn_batches must be a multiple of the number of AliBi slopes")
+    bias_ptr = None
+    if bias is not None:
+        if bias.dim() == 4 and bias.size(0) == 1:
+            bias = bias[0]
+        if bias.dim() != 3 or bias.size(1) != x.size(1) or bias.size(2) != x.size(2) or bias.dtype != x.dtype:
+            raise RuntimeError("bias must be [heads, seq_len, seq_len] in the dtype of the input")
+        _hp.require_gpu(bias, who)
+        if alibi_slopes is not None and bias.size(0) != heads:
+            raise RuntimeError("bias and alibi_slopes must have the same number of heads")
+        bias = bias.contiguous()
+        keep.append(bias)
+        bias_ptr, heads = bias.data_ptr(), bias.size(0)
+        if heads == 0 or x.size(0) % heads != 0:
+            raise RuntimeError("attn_batches must be a multiple of the number of bias heads")
+    lengths, lengths_ptr, heads = _key_lengths_arg(key_lengths, x.size(0), heads, who)
+    keep.append(lengths)
+    return keep, slopes_ptr, bias_ptr, lengths_ptr, heads
+
+
 def _zero_block(zero_block):
     zero_block = int(zero_block or 0)
     if zero_block and (zero_block < 8 or zero_block & (zero_block - 1)):
@@ -64,30 +97,8 @@ def forward(input, scale_factor, window=None, alibi_slopes=None, bias=None, key_
     _hp.require_gpu(input, "scaled_upper_triang_masked_softmax_cuda.forward")
     x = input.contiguous()
     y = torch.empty_like(x)
-    slopes_ptr, heads = None, None
-    if alibi_slopes is not None:
-        if alibi_slopes.dtype != torch.float32 or alibi_slopes.dim() != 1:
-            raise RuntimeError("alibi_slopes must be a 1-D float32 tensor")
-        _hp.require_gpu(alibi_slopes, "scaled_upper_triang_masked_softmax_cuda.forward")
-        alibi_slopes = alibi_slopes.contiguous()
-        slopes_ptr, heads = alibi_slopes.data_ptr(), alibi_slopes.numel()
-        if heads == 0 or x.size(0) % heads != 0:
-            raise RuntimeError("attn_batches must be a multiple of the number of AliBi slopes")
-    bias_ptr = None
-    if bias is not None:
-        if bias.dim() == 4 and bias.size(0) == 1:
-            bias = bias[0]
-        if bias.dim() != 3 or bias.size(1) != x.size(1) or bias.size(2) != x.size(2) or bias.dtype != x.dtype:
-            raise RuntimeError("bias must be [heads, seq_len, seq_len] in the dtype of the input")
-        _hp.require_gpu(bias, "scaled_upper_triang_masked_softmax_cuda.forward")
-        if alibi_slopes is not None and bias.size(0) != heads:
-            raise RuntimeError("bias and alibi_slopes must have the same number of heads")
-        bias = bias.contiguous()
-        bias_ptr, heads = bias.data_ptr(), bias.size(0)
-        if heads == 0 or x.size(0) % heads != 0:
-            raise RuntimeError("attn_batches must be a multiple of the number of bias heads")
-    lengths, lengths_ptr, heads = _key_lengths_arg(key_lengths, x.size(0), heads,
-                                                   "scaled_upper_triang_masked_softmax_cuda.forward")
+    keep, slopes_ptr, bias_ptr, lengths_ptr, heads = _per_head_args(
+        x, alibi_slopes, bias, key_lengths, "scaled_upper_triang_masked_softmax_cuda.forward")
     with _hp.device_guard(x):
         rc = _hp.lib().nhp_causal_softmax_blocks_fwd(
             y.data_ptr(), x.data_ptr(), float(scale_factor), x.size(0), x.size(1),
@@ -130,50 +141,56 @@ def backward(output_grads, softmax_results, scale_factor, window=None, key_lengt
     return g
 
 
-def forward_dropout(input, scale_factor, p, seed, window=None, zero_block=0):
+def forward_dropout(input, scale_factor, p, seed, window=None, zero_block=0, alibi_slopes=None, bias=None,
+                    key_lengths=None):
     """``forward`` and attention dropout in one kernel: returns ``(dropped, probabilities)``.
 
     ``dropped = keep * probabilities / (1 - p)`` with the library's counter-based keep mask for
     ``seed`` (see ``nhp_causal_softmax_dropout_fwd``); ``probabilities`` is what ``forward`` returns
-    and what ``backward_dropout`` needs. Not part of the reference's extension module."""
+    and what ``backward_dropout`` needs. ``alibi_slopes``, ``bias`` and ``key_lengths`` as in ``forward``.
+    Not part of the reference's extension module."""
+    who = "scaled_upper_triang_masked_softmax_cuda.forward_dropout"
     if input.dim() != 3:
         raise RuntimeError("expected 3D tensor")
     if input.dtype not in _HALF:
         raise RuntimeError("Only fp16 and bf16 are supported")
     if input.size(1) != input.size(2):
         raise RuntimeError("expected a square [attn_batches, seq_len, seq_len] tensor")
-    _hp.require_gpu(input, "scaled_upper_triang_masked_softmax_cuda.forward_dropout")
+    _hp.require_gpu(input, who)
     x = input.contiguous()
     y = torch.empty_like(x)
     dropped = torch.empty_like(x)
+    keep, slopes_ptr, bias_ptr, lengths_ptr, heads = _per_head_args(x, alibi_slopes, bias, key_lengths, who)
     with _hp.device_guard(x):
-        rc = _hp.lib().nhp_causal_softmax_dropout_blocks_fwd(
+        rc = _hp.lib().nhp_causal_softmax_ex_dropout_fwd(
             dropped.data_ptr(), y.data_ptr(), x.data_ptr(), float(scale_factor), x.size(0), x.size(1),
-            -1 if window is None else int(window), _zero_block(zero_block), float(p), int(seed), 0,
-            _hp.dtype_code(x, "forward_dropout"),
-            _hp.stream_of(x))
-    _hp.check(rc, "scaled_upper_triang_masked_softmax_cuda.forward_dropout")
+            -1 if window is None else int(window), _zero_block(zero_block), slopes_ptr, bias_ptr, lengths_ptr,
+            heads or 1, float(p), int(seed), 0, _hp.dtype_code(x, "forward_dropout"), _hp.stream_of(x))
+    _hp.check(rc, who)
+    del keep
     return dropped, y
 
 
-def backward_dropout(output_grads, softmax_results, scale_factor, p, seed, window=None, zero_block=0):
-    """Gradient of ``forward_dropout`` with respect to its input, given the gradient of ``dropped``;
-    in place on ``output_grads`` like ``backward``."""
+def backward_dropout(output_grads, softmax_results, scale_factor, p, seed, window=None, zero_block=0, key_lengths=None):
+    """Gradient of ``forward_dropout`` with respect to its input, given the gradient of ``dropped``
+    (pass the same ``window``, ``zero_block`` and ``key_lengths``); in place on ``output_grads`` like ``backward``."""
+    who = "scaled_upper_triang_masked_softmax_cuda.backward_dropout"
     if output_grads.dim() != 3 or softmax_results.dim() != 3:
         raise RuntimeError("expected 3D tensor")
     if output_grads.dtype not in _HALF or softmax_results.dtype not in _HALF:
         raise RuntimeError("Only fp16 and bf16 are supported")
     if output_grads.shape != softmax_results.shape or output_grads.dtype != softmax_results.dtype:
         raise RuntimeError("output_grads and softmax_results must have the same shape and dtype")
-    _hp.require_gpu(output_grads, "scaled_upper_triang_masked_softmax_cuda.backward_dropout")
-    _hp.require_gpu(softmax_results, "scaled_upper_triang_masked_softmax_cuda.backward_dropout")
+    _hp.require_gpu(output_grads, who)
+    _hp.require_gpu(softmax_results, who)
     g = output_grads.detach().contiguous()
     y = softmax_results.detach().contiguous()
+    lengths, lengths_ptr, heads = _key_lengths_arg(key_lengths, g.size(0), None, who)
     with _hp.device_guard(g):
-        rc = _hp.lib().nhp_causal_softmax_dropout_blocks_bwd(
+        rc = _hp.lib().nhp_causal_softmax_ex_dropout_bwd(
             g.data_ptr(), g.data_ptr(), y.data_ptr(), float(scale_factor), g.size(0), g.size(1),
-            -1 if window is None else int(window), _zero_block(zero_block), float(p), int(seed), 0,
-            _hp.dtype_code(g, "backward_dropout"),
-            _hp.stream_of(g))
-    _hp.check(rc, "scaled_upper_triang_masked_softmax_cuda.backward_dropout")
+            -1 if window is None else int(window), _zero_block(zero_block), lengths_ptr, heads or 1, float(p),
+            int(seed), 0, _hp.dtype_code(g, "backward_dropout"), _hp.stream_of(g))
+    _hp.check(rc, who)
+    del lengths
     return g

@@ -204,6 +204,57 @@ int nhp_causal_softmax_dropout_blocks_bwd(void* dx, const void* dy, const void* 
                                           int dtype, void* stream);
 
 /*
+ * Attention dropout together with the per-head extras of nhp_causal_softmax_ex_fwd (AliBi slopes, additive
+ * bias tensor, key lengths; any of them may be NULL) and the block-limited writing of
+ * nhp_causal_softmax_blocks_fwd, in one kernel: the scores pass through bias, AliBi, scaling, the band
+ * mask, the softmax and the dropout exactly as in the entry points that do one of these at a time. The
+ * backward takes the gradient of `dropped`, with the key lengths of the forward.
+ *
+ * Replaces, in ParallelSelfAttention.attention (megatron/model/transformer.py:580-593), the sequence
+ * `attention_scores += rpe`, `alibi_embed(attention_scores)`, scale_mask_softmax (the fused branch:
+ * megatron/fused_kernels/scaled_upper_triang_masked_softmax.cpp:31-56) and attention_dropout.
+ */
+int nhp_causal_softmax_ex_dropout_fwd(void* dropped, void* y, const void* x, float scale,
+                                      int64_t attn_batches, int64_t seq_len, int64_t window,
+                                      int64_t zero_block, const float* alibi_slopes, const void* bias,
+                                      const int32_t* key_lengths, int64_t heads, float p, uint64_t seed,
+                                      uint64_t offset, int dtype, void* stream);
+
+int nhp_causal_softmax_ex_dropout_bwd(void* dx, const void* dy, const void* y, float scale,
+                                      int64_t attn_batches, int64_t seq_len, int64_t window,
+                                      int64_t zero_block, const int32_t* key_lengths, int64_t heads,
+                                      float p, uint64_t seed, uint64_t offset, int dtype, void* stream);
+
+/*
+ * nhp_masked_softmax_fwd with what the caller of the reference does to the scores and the mask before
+ * the padding-mask softmax (megatron/model/transformer.py:580-588), done inside the kernel instead of in
+ * full passes over [b, np, sq, sk] (any of the three may be NULL):
+ *   bias         [np, sq, sk] in the scores' dtype, shared by the batch (`attention_scores += rpe`): added
+ *                in the storage dtype, as the eager in-place addition leaves it in memory;
+ *   alibi_slopes [np] fp32, needs sq == sk: the AliBi bias -(q - k) * slope for k <= q and nothing above
+ *                the diagonal, with the roundings of AliBi.forward
+ *                (megatron/model/positional_embeddings.py:219-257), after the bias;
+ *   key_lengths  [b] int32: keys k >= key_lengths[b] count as masked (as if their mask bytes were 1).
+ * Results are bit-identical to nhp_masked_softmax_fwd on scores and a mask prepared that way. The
+ * backward is nhp_masked_softmax_bwd (it takes no mask). The _dropout variant also writes
+ * dropped = dropout(y) as nhp_masked_softmax_dropout_fwd does; its backward is
+ * nhp_masked_softmax_dropout_bwd.
+ *
+ * Replaces scaled_masked_softmax_cuda.forward (megatron/fused_kernels/scaled_masked_softmax.cpp:33-42)
+ * together with those preparations.
+ */
+int nhp_masked_softmax_ex_fwd(void* y, const void* x, const uint8_t* mask, float scale, int64_t b,
+                              int64_t np, int64_t sq, int64_t sk, int64_t pad_batches,
+                              const float* alibi_slopes, const void* bias, const int32_t* key_lengths,
+                              int dtype, void* stream);
+
+int nhp_masked_softmax_ex_dropout_fwd(void* dropped, void* y, const void* x, const uint8_t* mask,
+                                      float scale, int64_t b, int64_t np, int64_t sq, int64_t sk,
+                                      int64_t pad_batches, const float* alibi_slopes, const void* bias,
+                                      const int32_t* key_lengths, float p, uint64_t seed,
+                                      uint64_t offset, int dtype, void* stream);
+
+/*
  * The same for the padding-mask softmax: y as nhp_masked_softmax_fwd, dropped = keep ? y / (1 - p) : 0
  * over the flat element index of the [b, np, sq, sk] tensor; the backward is nhp_masked_softmax_bwd of
  * g = keep ? dy / (1 - p) : 0 (rows = b * np * sq).

@@ -132,9 +132,35 @@ def causal_softmax_fwd(x, scale, window=None, alibi_slopes=None, bias=None, key_
     return y
 
 
-def masked_softmax_fwd(x, mask, scale):
-    """x: [b, np, sq, sk]; mask: [1 or b, 1, sq, sk] bool/uint8 (value 1 masks)."""
+def prepared_masked_inputs(x, mask, alibi_slopes=None, bias=None, key_lengths=None):
+    """What the caller of the padding-mask softmax does to its operands beforehand
+    (megatron/model/transformer.py:580-588), as eager torch statements in the scores' dtype:
+    `attention_scores += rpe` (bias [np, sq, sk] or [1, np, sq, sk]), then AliBi.forward
+    (megatron/model/positional_embeddings.py:219-257, sq == sk), and the padding keys
+    k >= key_lengths[b] merged into the mask. Returns (scores, mask [b or 1, 1, sq, sk] bool)."""
+    from . import fallback_semantics as fb
+
+    b, np_, sq, sk = x.shape
+    if bias is not None:
+        x = x + bias.view(1, np_, sq, sk)
+    if alibi_slopes is not None:
+        assert sq == sk
+        x = fb.alibi_add(x, alibi_slopes)
+    m = mask.bool() if mask.dtype != torch.bool else mask
+    if key_lengths is not None:
+        assert key_lengths.numel() == b
+        keys = torch.arange(sk)
+        m = m | (keys.view(1, 1, 1, sk) >= key_lengths.clamp(min=0).view(b, 1, 1, 1))
+    return x, m
+
+
+def masked_softmax_fwd(x, mask, scale, alibi_slopes=None, bias=None, key_lengths=None):
+    """x: [b, np, sq, sk]; mask: [1 or b, 1, sq, sk] bool/uint8 (value 1 masks).
+    alibi_slopes (fp32 [np]), bias ([np, sq, sk] in x.dtype) and key_lengths (integer [b]) are applied
+    as prepared_masked_inputs does, i.e. the result is the plain softmax of the prepared operands."""
     assert x.dim() == 4 and mask.dim() == 4
+    if alibi_slopes is not None or bias is not None or key_lengths is not None:
+        x, mask = prepared_masked_inputs(x, mask, alibi_slopes, bias, key_lengths)
     x = _cpu_contig(x)
     m = _cpu_contig(mask).view(torch.uint8) if mask.dtype == torch.bool else _cpu_contig(mask)
     assert m.dtype == torch.uint8
@@ -410,10 +436,14 @@ def bias_dropout_add(x, bias, residual, p, seed, offset=0):
     return out
 
 
-def causal_softmax_dropout_fwd(x, scale, p, seed, offset=0, window=None):
-    """Returns (dropped, y): the probabilities y and dropout(y) with the mask of dropout_mask over x's flat index."""
+def causal_softmax_dropout_fwd(x, scale, p, seed, offset=0, window=None, alibi_slopes=None, bias=None, key_lengths=None):
+    """Returns (dropped, y): the probabilities y and dropout(y) with the mask of dropout_mask over x's flat index.
+    With AliBi slopes, a bias or key lengths: causal_softmax_fwd with them, then the dropout of its stored result."""
     assert x.dim() == 3 and x.size(1) == x.size(2)
     x = _cpu_contig(x)
+    if alibi_slopes is not None or bias is not None or key_lengths is not None:
+        y = causal_softmax_fwd(x, scale, window, alibi_slopes, bias, key_lengths)
+        return _dropout_of_stored(y, p, seed, offset), y
     y, dropped = torch.empty_like(x), torch.empty_like(x)
     _check(lib().oracle_causal_softmax_dropout_fwd(dropped.data_ptr(), y.data_ptr(), x.data_ptr(), float(scale), x.size(0),
                                                    x.size(1), -1 if window is None else int(window), float(p), int(seed),
@@ -421,9 +451,11 @@ def causal_softmax_dropout_fwd(x, scale, p, seed, offset=0, window=None):
     return dropped, y
 
 
-def causal_softmax_dropout_bwd(dy, y, scale, p, seed, offset=0, window=None):
+def causal_softmax_dropout_bwd(dy, y, scale, p, seed, offset=0, window=None, key_lengths=None):
     """Gradient with respect to the scores, given the gradient of dropout(y)."""
     dy, y = _cpu_contig(dy), _cpu_contig(y)
+    if key_lengths is not None:
+        return softmax_bwd(_dropout_of_stored(dy, p, seed, offset), y, scale, True, window, key_lengths)
     dx = torch.empty_like(dy)
     _check(lib().oracle_causal_softmax_dropout_bwd(dx.data_ptr(), dy.data_ptr(), y.data_ptr(), float(scale), dy.size(0),
                                                    dy.size(1), -1 if window is None else int(window), float(p), int(seed),
@@ -442,11 +474,11 @@ def _dropout_of_stored(t, p, seed, offset):
     return torch.where(keep, scaled, torch.zeros_like(scaled))
 
 
-def masked_softmax_dropout_fwd(x, mask, scale, p, seed, offset=0):
+def masked_softmax_dropout_fwd(x, mask, scale, p, seed, offset=0, alibi_slopes=None, bias=None, key_lengths=None):
     """Returns (dropped, y) for the padding-mask softmax followed by attention dropout
     (megatron/model/transformer.py:588-593): the composition of masked_softmax_fwd and the dropout of its
     stored result, the mask taken over the flat index of the [b, np, sq, sk] tensor."""
-    y = masked_softmax_fwd(x, mask, scale)
+    y = masked_softmax_fwd(x, mask, scale, alibi_slopes, bias, key_lengths)
     return _dropout_of_stored(y, p, seed, offset), y
 
 

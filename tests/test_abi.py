@@ -137,6 +137,22 @@ def test_argument_validation_of_the_layer_entry_points(hotpath):
     assert lib.nhp_causal_softmax_ex_fwd(q, p, 1.0, 6, 8, -1, null, q, null, 3, BF16, None) == -6   # bias over the output
     assert lib.nhp_causal_softmax_ex_bwd(q, p, p, 1.0, 6, 8, -1, p, 4, BF16, None) == -2
     assert lib.nhp_causal_softmax_ex_fwd(null, null, 1.0, 0, 8, 3, null, null, null, 1, F16, None) == 0
+    # the same extras with dropout, and on the padding-mask softmax
+    assert lib.nhp_causal_softmax_ex_dropout_fwd(q, q2, p, 1.0, 6, 8, -1, 0, p, null, null, 4, 0.1, 1, 0, BF16, None) == -2
+    assert lib.nhp_causal_softmax_ex_dropout_fwd(q, q2, p, 1.0, 6, 8, -1, 0, null, q2, null, 3, 0.1, 1, 0, BF16, None) == -6
+    assert lib.nhp_causal_softmax_ex_dropout_fwd(q, q2, p, 1.0, 6, 8, -1, 0, null, q, null, 3, 0.1, 1, 0, BF16, None) == -6
+    assert lib.nhp_causal_softmax_ex_dropout_fwd(q, q2, p, 1.0, 6, 8, -1, 0, null, null, null, 1, 1.0, 1, 0, BF16, None) == -2
+    assert lib.nhp_causal_softmax_ex_dropout_bwd(q, p, p, 1.0, 6, 8, -1, 0, p, 4, 0.1, 1, 0, BF16, None) == -2
+    assert lib.nhp_causal_softmax_ex_dropout_bwd(null, null, null, 1.0, 0, 8, -1, 0, null, 1, 0.1, 1, 0, BF16, None) == 0
+    assert lib.nhp_masked_softmax_ex_fwd(q, p, p, 1.0, 2, 2, 8, 16, 1, p, null, null, BF16, None) == -2   # AliBi needs sq == sk
+    assert lib.nhp_masked_softmax_ex_fwd(q, p, p, 1.0, 2, 2, 8, 16, 1, null, q, null, BF16, None) == -6   # bias over the output
+    assert lib.nhp_masked_softmax_ex_fwd(q, p, p, 1.0, 2, 2, 8, 16, 3, null, null, p, BF16, None) == -4
+    assert lib.nhp_masked_softmax_ex_fwd(q, p, p, 1.0, 2, 2, 8, 16, 1, null, null, null, F32, None) == -1
+    assert lib.nhp_masked_softmax_ex_fwd(null, null, null, 1.0, 2, 0, 8, 16, 1, null, null, null, F16, None) == 0
+    assert lib.nhp_masked_softmax_ex_dropout_fwd(q2, q, p, p, 1.0, 2, 2, 8, 16, 1, null, q2, null, 0.1, 1, 0, BF16, None) == -6
+    assert lib.nhp_masked_softmax_ex_dropout_fwd(q, q, p, p, 1.0, 2, 2, 8, 16, 1, null, null, null, 0.1, 1, 0, BF16, None) == -6
+    assert lib.nhp_masked_softmax_ex_dropout_fwd(null, q, p, p, 1.0, 2, 2, 8, 16, 1, null, null, null, 0.1, 1, 0, BF16, None) == -3
+    assert lib.nhp_masked_softmax_ex_dropout_fwd(q2, q, p, p, 1.0, 2, 2, 8, 16, 1, null, null, null, -0.5, 1, 0, BF16, None) == -2
     # block-limited variants: the block size must be 0 or a power of two of at least 8
     for bad in (4, 12, 100, -8):
         assert lib.nhp_causal_softmax_blocks_fwd(q, p, 1.0, 6, 64, -1, bad, null, null, null, 1, BF16, None) == -2

@@ -306,7 +306,7 @@ def test_module_with_attention_dropout():
     assert (yg.detach().cpu().float() - want_gd.float()).abs().max().item() <= 2.0**-7 * want_gd.float().abs().max().item()
     want_gdx = oracle.masked_softmax_dropout_bwd(dy, want_gy, scale, p, seed)
     assert (xg.grad.cpu().float() - want_gdx.float()).norm().item() <= 2.0**-6 * want_gdx.float().norm().item()
-    # with a bias the module falls back to torch's dropout after the kernel: same rate
+    # with a bias it is still one kernel, and the same rate
     yb = g(x.to(DEV), mask, bias=torch.zeros((1, np_, s, s), dtype=dtype, device=DEV))
     zero_rate = ((yb == 0) & ~mask).float().sum().item() / (~mask).expand_as(yb).float().sum().item()
     assert abs(zero_rate - p) < 0.02
@@ -472,3 +472,191 @@ def test_block_limited_causal_softmax_at_full_size():
     bound = torch.where(written, ref.float().abs() * 2.0 ** -7 + 1e-6, torch.ones((), device=DEV))
     assert bool((diff <= bound).all())
     assert int(gb[:, written & (torch.arange(s, device=DEV)[None, :] > torch.arange(s, device=DEV)[:, None])].abs().max()) == 0
+
+
+# ---------------------------------------------------------------------------
+# The padding-mask softmax with bias / AliBi / key lengths inside the kernel, and both softmax kernels with
+# those extras and attention dropout at once.
+# ---------------------------------------------------------------------------
+def abi_masked_ex_fwd(hp, x, mask, scale, slopes=None, bias=None, key_lengths=None, dropout=None):
+    """nhp_masked_softmax_ex_fwd, or with dropout=(p, seed) nhp_masked_softmax_ex_dropout_fwd -> (dropped, y)."""
+    b, np_, sq, sk = x.shape
+    y = torch.empty_like(x)
+    m = mask.view(torch.uint8) if mask.dtype == torch.bool else mask
+    extras = (None if slopes is None else slopes.data_ptr(), None if bias is None else bias.data_ptr(),
+              None if key_lengths is None else key_lengths.data_ptr())
+    if dropout is None:
+        rc = hp.lib().nhp_masked_softmax_ex_fwd(y.data_ptr(), x.data_ptr(), m.data_ptr(), scale, b, np_, sq, sk, m.size(0),
+                                                *extras, hp.dtype_code(x, "t"), None)
+        assert rc == 0, hp.lib().nhp_status_string(rc)
+        return y
+    dropped = torch.empty_like(x)
+    rc = hp.lib().nhp_masked_softmax_ex_dropout_fwd(dropped.data_ptr(), y.data_ptr(), x.data_ptr(), m.data_ptr(), scale, b,
+                                                    np_, sq, sk, m.size(0), *extras, dropout[0], dropout[1], 0,
+                                                    hp.dtype_code(x, "t"), None)
+    assert rc == 0, hp.lib().nhp_status_string(rc)
+    return dropped, y
+
+
+# (b, np, sq, sk, extras): every forward geometry of the padding-mask kernel incl. the scalar fallback (sk = 1001, 24);
+# "a" AliBi (square scores only), "b" bias tensor, "l" key lengths
+MASKED_EX_CASES = [
+    (2, 3, 64, 64, "a"), (2, 3, 64, 64, "abl"), (3, 2, 5, 200, "bl"), (2, 2, 512, 512, "al"), (2, 2, 12, 512, "b"),
+    (4, 2, 4, 1024, "l"), (2, 4, 1024, 1024, "ab"), (2, 4, 16, 2048, "bl"), (1, 2, 2048, 2048, "abl"), (1, 2, 4, 4096, "bl"),
+    (1, 2, 2, 8192, "b"), (2, 2, 6, 1001, "bl"), (2, 2, 1001, 1001, "abl"), (2, 1, 3, 24, "l"), (2, 3, 24, 24, "a"),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
+@pytest.mark.parametrize("pad_batches", ["one", "each"])
+@pytest.mark.parametrize("case", MASKED_EX_CASES, ids=lambda c: "x".join(map(str, c)))
+def test_masked_softmax_with_extras_vs_oracle(hotpath, case, pad_batches, dtype):
+    """nhp_masked_softmax_ex_fwd against the oracle's composition (eager preparation of scores and mask, then
+    the plain padding-mask softmax): 2 ulp, masked keys exactly what the plain kernel leaves there, the scores
+    and bias entries of whole chunks of padding keys never read, and bit-identical to the plain entry point
+    given the prepared operands."""
+    b, np_, sq, sk, extras = case
+    print(f"masked ex case {case} {pad_batches} {dtype}", flush=True)
+    scale = 1 / math.sqrt(128)
+    x = util.randn((b, np_, sq, sk), dtype, seed=sk + sq, std=2.0)
+    mask = util.padding_mask(b, sq, sk, seed=sk, lo=sk // 2)
+    if sq == sk:
+        mask = mask | fb.causal_mask(sk)                  # the decoder's mask: causal and padding
+    if pad_batches == "one":
+        mask = mask[:1].contiguous()
+    slopes = torch.tensor(fb.alibi_slopes(max(np_, 2))[:np_], dtype=torch.float32) if "a" in extras else None
+    bias = util.randn((np_, sq, sk), dtype, seed=sk + 7, std=1.5) if "b" in extras else None
+    lengths = None
+    if "l" in extras:
+        lengths = torch.randint(sk // 3, sk + 1, (b,), generator=torch.Generator().manual_seed(sk), dtype=torch.int32)
+        lengths[0] = sk - 3                               # a length that cuts a 16-byte chunk
+        if b > 1:
+            lengths[-1] = 0                               # a sequence without keys: uniform rows
+    want = oracle.masked_softmax_fwd(x, mask, scale, slopes, bias, lengths)
+    xp, bp = x.clone(), None if bias is None else bias.clone()
+    if lengths is not None:
+        # whole chunks of padding keys are not read, neither from the scores nor from the bias
+        chunk_start = torch.arange(sk) // 8 * 8
+        beyond = chunk_start.view(1, 1, 1, sk) >= lengths.view(b, 1, 1, 1)
+        xp[beyond.expand_as(xp)] = float("nan")
+        if bp is not None:
+            bp[(chunk_start.view(1, 1, sk) >= int(lengths.max())).expand_as(bp)] = float("inf")
+    dev = lambda t: None if t is None else t.to(DEV)
+    got = abi_masked_ex_fwd(hotpath, xp.to(DEV), mask.to(DEV), scale, dev(slopes), dev(bp), dev(lengths)).cpu()
+    assert not torch.isnan(got.float()).any()
+    util.assert_ulp_close(got, want, 2, "fwd")
+    # the same kernel arithmetic as the plain entry point on prepared operands
+    xs, ms = oracle.prepared_masked_inputs(x, mask, slopes, bias, lengths)
+    plain = util.abi_masked_fwd(hotpath, xs.to(DEV), ms.contiguous().to(DEV), scale).cpu()
+    assert torch.equal(util.raw_bits(got), util.raw_bits(plain))
+    if lengths is not None and b > 1:
+        assert torch.equal(got[-1], torch.full_like(got[-1], 1.0 / sk))
+    # with dropout on top: the same probabilities, and the oracle's dropout of them
+    p, seed = 0.2, 99 + sk
+    dropped, y = abi_masked_ex_fwd(hotpath, xp.to(DEV), mask.to(DEV), scale, dev(slopes), dev(bp), dev(lengths), (p, seed))
+    assert torch.equal(util.raw_bits(y.cpu()), util.raw_bits(got))
+    assert torch.equal(util.raw_bits(dropped.cpu()), util.raw_bits(oracle.bias_dropout_add(got, None, None, p, seed)))
+
+
+# (batch, heads, seq_len, window, extras, zero_block)
+CAUSAL_EX_DROPOUT_CASES = [
+    (2, 2, 64, None, "abl", 0), (1, 3, 200, 63, "a", 0), (2, 2, 512, None, "bl", 0), (2, 4, 1024, 100, "al", 0),
+    (2, 3, 2048, None, "abl", 0), (1, 2, 4096, 1000, "l", 0), (1, 1, 8192, None, "a", 0), (2, 2, 1001, None, "abl", 0),
+    (2, 2, 2048, None, "bl", 512),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
+@pytest.mark.parametrize("case", CAUSAL_EX_DROPOUT_CASES, ids=lambda c: "_".join(map(str, c)))
+def test_causal_softmax_with_extras_and_dropout_vs_oracle(hotpath, case, dtype):
+    """nhp_causal_softmax_ex_dropout_fwd/bwd through the extension module: the probabilities are those of the
+    entry point without dropout bit for bit (and within 2 ulp of the oracle), `dropped` is the oracle's dropout of
+    them, the backward meets the oracle's (dropout backward, then the softmax backward under the same band)."""
+    import scaled_upper_triang_masked_softmax_cuda as ext
+    from megatron.model.fused_softmax import _written_blocks
+
+    batch, heads, s, window, extras, zb = case
+    print(f"causal ex dropout case {case} {dtype}", flush=True)
+    a = batch * heads
+    scale, p, seed = 1 / math.sqrt(128), 0.1, 555 + s
+    x = util.randn((a, s, s), dtype, seed=s + 3, std=2.0)
+    dy = util.randn((a, s, s), dtype, seed=s + 4)
+    slopes = torch.tensor(fb.alibi_slopes(max(heads, 2))[:heads], dtype=torch.float32) if "a" in extras else None
+    bias = util.randn((heads, s, s), dtype, seed=s + 5, std=1.5) if "b" in extras else None
+    lengths = torch.tensor([s - 5, s // 3][:batch], dtype=torch.int32) if "l" in extras else None
+    dev = lambda t: None if t is None else t.to(DEV)
+    want_y = oracle.causal_softmax_fwd(x, scale, window, slopes, bias, lengths)
+    written = _written_blocks(s, zb, window, "cpu") if zb else torch.ones((s, s), dtype=torch.bool)
+    dropped, y = ext.forward_dropout(x.to(DEV), scale, p, seed, window, zb, dev(slopes), dev(bias), dev(lengths))
+    no_drop = ext.forward(x.to(DEV), scale, window, dev(slopes), dev(bias), dev(lengths), zb)
+    y, dropped, no_drop = y.cpu(), dropped.cpu(), no_drop.cpu()
+    assert torch.equal(util.raw_bits(y)[:, written], util.raw_bits(no_drop)[:, written])
+    y = torch.where(written, y, want_y)
+    util.assert_ulp_close(y, want_y, 2, "y")
+    want_dropped = oracle.bias_dropout_add(y, None, None, p, seed)
+    assert torch.equal(util.raw_bits(dropped)[:, written], util.raw_bits(want_dropped)[:, written])
+    dead = want_y == 0
+    assert int(util.raw_bits(dropped)[:, written][dead[:, written]].abs().max()) == 0
+    want_dx = oracle.causal_softmax_dropout_bwd(dy, want_y, scale, p, seed, window=window, key_lengths=lengths)
+    got_dx = ext.backward_dropout(dy.to(DEV).clone(), want_y.to(DEV), scale, p, seed, window, zb, dev(lengths)).cpu()
+    got_dx = torch.where(written, got_dx, want_dx)
+    masked = fb.causal_mask(s, sliding_window_width=window)[0, 0].expand(a, s, s).clone()
+    if lengths is not None:
+        masked |= padded_mask(s, lengths, window).repeat_interleave(heads, dim=0)
+    assert int(util.raw_bits(got_dx)[masked].abs().max()) == 0
+    g = oracle.bias_dropout_add(dy, None, None, p, seed)
+    util.assert_softmax_bwd_close(got_dx, want_dx, g.masked_fill(masked, 0), want_y, scale, "bwd")
+
+
+@pytest.mark.parametrize("fusion", ["upper_triang", "general"])
+def test_module_fuses_every_extra_and_dropout_into_one_kernel(fusion, monkeypatch):
+    """FusedScaleMaskSoftmax with a bias, AliBi, key lengths and attention dropout together on a fused branch:
+    no element-wise torch pass over the scores is left (torch's dropout, add and arange are made to raise), the
+    result is the oracle's for the seed the module drew, and the gradients of scores and bias match autograd
+    through the torch branch given the same keep mask."""
+    from megatron.model.fused_softmax import FusedScaleMaskSoftmax, SoftmaxFusionTypes as T
+
+    dtype, b, np_, s, scale, p = torch.bfloat16, 2, 4, 256, 0.125, 0.25
+    slopes = torch.tensor(fb.alibi_slopes(np_), dtype=torch.float32)
+    x = util.randn((b, np_, s, s), dtype, seed=1, std=2.0)
+    rpe = util.randn((1, np_, s, s), dtype, seed=2)
+    dy = util.randn((b, np_, s, s), dtype, seed=3)
+    lengths = torch.tensor([s, 100], dtype=torch.int32)
+    mask = fb.causal_mask(s, DEV)
+    m = FusedScaleMaskSoftmax(False, True, T[fusion], fb.fill_masked_with_dtype_min, True, scale, alibi_slopes=slopes,
+                              attention_dropout=p).to(DEV)
+    torch.manual_seed(5)
+    seed = int(torch.empty((), dtype=torch.int64).random_().item())
+    torch.manual_seed(5)
+    xd, bd, ld = x.to(DEV).requires_grad_(True), rpe.to(DEV).requires_grad_(True), lengths.to(DEV)
+
+    def forbidden(*a, **k):
+        raise AssertionError("a torch pass over the scores on the fused branch")
+
+    with monkeypatch.context() as mp:
+        mp.setattr(torch.nn.functional, "dropout", forbidden)
+        mp.setattr(m, "_add_alibi", forbidden)
+        mp.setattr(m, "_mask_with_padding", forbidden)
+        out = m(xd, mask, bias=bd, key_lengths=ld)
+    out.backward(dy.to(DEV).clone())
+    if fusion == "upper_triang":
+        want_d, want_y = oracle.causal_softmax_dropout_fwd(x.view(-1, s, s), scale, p, seed, alibi_slopes=slopes,
+                                                           bias=rpe[0], key_lengths=lengths)
+    else:
+        want_d, want_y = oracle.masked_softmax_dropout_fwd(x, mask.cpu(), scale, p, seed, alibi_slopes=slopes,
+                                                           bias=rpe[0], key_lengths=lengths)
+    want_d, want_y = want_d.view_as(x), want_y.view_as(x)
+    keep = oracle.dropout_mask(x.numel(), p, seed).view_as(x)
+    got = out.detach().cpu()
+    assert int(util.raw_bits(got)[~keep].abs().max()) == 0
+    assert (got.float() - want_d.float()).abs().max().item() <= 2.0**-7 * want_d.float().abs().max().item()
+    # gradients: float64 autograd of the same function with the same keep mask
+    x64, b64 = x.double().requires_grad_(True), rpe.double().requires_grad_(True)
+    z = fb.alibi_add((x64 + b64), slopes.double()) * scale
+    full = mask.cpu() | (torch.arange(s).view(1, 1, 1, s) >= lengths.view(b, 1, 1, 1))
+    probs = torch.softmax(z.masked_fill(full, -10000.0), -1)
+    (probs * keep / (1 - p)).backward(dy.double())
+    gx, gb = xd.grad.cpu().double(), bd.grad.cpu().double()
+    assert (gx - x64.grad).norm().item() <= 2.0**-6 * x64.grad.norm().item()
+    assert (gb - b64.grad).norm().item() <= 2.0**-5 * b64.grad.norm().item()
+    assert bd.grad.shape == rpe.shape

@@ -285,3 +285,85 @@ def test_masked_softmax_with_attention_dropout_is_the_composition(dtype):
     assert err <= 4 * 2.0 ** (-8 if dtype == torch.bfloat16 else -11) * xd.grad.abs().max().item()
     d0, y0 = oracle.masked_softmax_dropout_fwd(x, mask, scale, 0.0, seed)
     assert torch.equal(util.raw_bits(d0), util.raw_bits(plain)) and torch.equal(util.raw_bits(y0), util.raw_bits(plain))
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_padding_mask_softmax_with_extras_is_the_composition(dtype):
+    """The padding-mask softmax with a bias tensor, AliBi slopes and key lengths is the plain one on operands
+    prepared by the caller's eager statements (transformer.py:580-588). Two independent statements must meet:
+    given the causal mask, it equals the causal kernel semantics (C) with the same extras on every row that keeps
+    a key (a row without keys is 1/sk here and zeros there): exact zeros in the same places, and probabilities
+    within 1 ulp (the two sum a row's exponentials over different lengths, hence in a different order)."""
+    b, heads, s, scale = 3, 4, 72, 0.3
+    slopes = torch.tensor(fb.alibi_slopes(heads), dtype=torch.float32)
+    x = util.randn((b, heads, s, s), dtype, seed=11, std=2.0)
+    bias = util.randn((heads, s, s), dtype, seed=12, std=1.5)
+    lengths = torch.tensor([s, 29, 0], dtype=torch.int32)
+    mask = fb.causal_mask(s)
+    for use_slopes, use_bias, use_len in [(1, 0, 0), (0, 1, 0), (0, 0, 1), (1, 1, 1)]:
+        kw = dict(alibi_slopes=slopes if use_slopes else None, bias=bias if use_bias else None,
+                  key_lengths=lengths if use_len else None)
+        general = oracle.masked_softmax_fwd(x, mask, scale, **kw)
+        causal = oracle.causal_softmax_fwd(x.view(-1, s, s), scale, **kw).view_as(x)
+        has_key = torch.ones(b, 1, s, 1, dtype=torch.bool)
+        if use_len:
+            has_key = (lengths.view(b, 1, 1, 1) > 0).expand(b, 1, s, 1)
+        rows = has_key.expand_as(x)
+        assert torch.equal(util.raw_bits(general)[rows] == 0, util.raw_bits(causal)[rows] == 0)
+        util.assert_ulp_close(general[rows], causal[rows], 1, str((use_slopes, use_bias, use_len)))
+        if use_len:
+            # the sequence without any key: every row uniform, exactly fl(1/sk)
+            assert torch.equal(general[2], torch.full_like(general[2], 1.0 / s))
+    # the prepared operands themselves: in-place add, AliBi.forward, merged padding
+    xs, m = oracle.prepared_masked_inputs(x, mask, slopes, bias, lengths)
+    assert torch.equal(util.raw_bits(xs), util.raw_bits(fb.alibi_add(x + bias, slopes)))
+    assert bool(m[1, 0, :, 29:].all()) and not bool(m[1, 0, 40, :29].any()) and bool(m[2].all())
+    assert torch.equal(m[0], mask[0])
+    # a [b, 1, sq, sk] mask and a uint8 mask work the same
+    per_batch = mask.expand(b, 1, s, s).contiguous()
+    a = oracle.masked_softmax_fwd(x, per_batch.to(torch.uint8), scale, slopes, bias, lengths)
+    assert torch.equal(util.raw_bits(a), util.raw_bits(oracle.masked_softmax_fwd(x, mask, scale, slopes, bias, lengths)))
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_rectangular_scores_with_bias_and_key_lengths(dtype):
+    """sq != sk (new positions after cached keys): bias and key lengths against float64 brute force."""
+    b, heads, sq, sk, scale = 2, 3, 5, 40, 0.25
+    x = util.randn((b, heads, sq, sk), dtype, seed=21, std=2.0)
+    bias = util.randn((heads, sq, sk), dtype, seed=22)
+    lengths = torch.tensor([33, 40], dtype=torch.int32)
+    mask = util.padding_mask(b, sq, sk, seed=23, lo=20)
+    got = oracle.masked_softmax_fwd(x, mask, scale, bias=bias, key_lengths=lengths)
+    z = (x + bias).double() * float(torch.tensor(scale, dtype=torch.float32))
+    full = mask.expand(b, heads, sq, sk) | (torch.arange(sk).view(1, 1, 1, sk) >= lengths.view(b, 1, 1, 1))
+    want = f64_softmax_rows(z.masked_fill(full, -10000.0))
+    util.assert_ulp_close(got, want.to(dtype), 1, "rectangular")
+    assert int(util.raw_bits(got)[full & ~full.all(-1, keepdim=True)].abs().max()) == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_causal_softmax_dropout_with_extras_is_the_composition(dtype):
+    """Dropout after the causal softmax with extras: same probabilities as without dropout, dropped = the C
+    oracle's dropout of them; with trivial extras the composed route equals the single C function."""
+    b, heads, s, scale, p, seed = 2, 2, 40, 0.3, 0.25, 77
+    x = util.randn((b * heads, s, s), dtype, seed=31, std=2.0)
+    dy = util.randn((b * heads, s, s), dtype, seed=32)
+    slopes = torch.tensor(fb.alibi_slopes(heads), dtype=torch.float32)
+    bias = util.randn((heads, s, s), dtype, seed=33)
+    lengths = torch.tensor([s, 17], dtype=torch.int32)
+    dropped, y = oracle.causal_softmax_dropout_fwd(x, scale, p, seed, window=9, alibi_slopes=slopes, bias=bias,
+                                                   key_lengths=lengths)
+    plain = oracle.causal_softmax_fwd(x, scale, window=9, alibi_slopes=slopes, bias=bias, key_lengths=lengths)
+    assert torch.equal(util.raw_bits(y), util.raw_bits(plain))
+    assert torch.equal(util.raw_bits(dropped), util.raw_bits(oracle.bias_dropout_add(plain, None, None, p, seed)))
+    # zero bias: the composed route against the C function that does softmax and dropout at once
+    d1, y1 = oracle.causal_softmax_dropout_fwd(x, scale, p, seed, window=9, bias=torch.zeros_like(bias))
+    d2, y2 = oracle.causal_softmax_dropout_fwd(x, scale, p, seed, window=9)
+    assert torch.equal(util.raw_bits(d1), util.raw_bits(d2)) and torch.equal(util.raw_bits(y1), util.raw_bits(y2))
+    # backward: all lengths full = the C function; shorter lengths zero the padding columns
+    full = torch.tensor([s, s], dtype=torch.int32)
+    g1 = oracle.causal_softmax_dropout_bwd(dy, y2, scale, p, seed, window=9, key_lengths=full)
+    g2 = oracle.causal_softmax_dropout_bwd(dy, y2, scale, p, seed, window=9)
+    assert torch.equal(util.raw_bits(g1), util.raw_bits(g2))
+    g3 = oracle.causal_softmax_dropout_bwd(dy, y, scale, p, seed, window=9, key_lengths=lengths)
+    assert int(util.raw_bits(g3)[heads:, :, 17:].abs().max()) == 0
