@@ -322,17 +322,47 @@ rope_lean_kernel(RopeTensor ta, RopeTensor tb, Tables tab, int rot_chunks)
 // which the gradient of the keys arrives from the backward of the score GEMM
 // (q k^T hands its second operand's gradient over as [b, h, d, s]).
 //   grid  = (b * h rows, ceil(s / 64)), block = 256 threads
-//   phase 1: 16-byte loads along s (8 lanes cover the 64 positions of one
-//            feature), written to LDS transposed, one 16-bit element at a time;
-//            the chunk slot of a feature is XOR-ed with the load chunk index so
-//            that the 8 lanes of a feature hit 8 different bank groups
+//   phase 1: 16-byte loads along s. A wave covers, per pass, the 8 features of one
+//            output chunk (lane >> 3) by the 64 positions of the tile (8 lanes of 8
+//            positions each). The 8 x 8 block of 16-bit elements that 8 lanes 8 apart
+//            hold is transposed in registers (one DPP exchange, then the row and
+//            half-wave swaps of gfx950), after which every lane owns one whole output
+//            chunk and writes it to LDS with one 16-byte store; the chunk slot is
+//            XOR-ed with the position group so that neither side conflicts
 //   phase 2: one lane per (position, feature chunk) reads its chunk and the
-//            partner chunk from LDS, rotates, and stores 16 bytes
+//            partner chunk from LDS, rotates, and stores 16 bytes. With a partial
+//            rotary dimension the rotation is done first, in place in LDS, by as
+//            many lanes as there are rotating chunk pairs (all of them busy), and
+//            the tile is then copied out without arithmetic
 // 16-bit data only; P = ceil(d / 32) load passes, all in flight together.
 // Requires: s % 8 == 0, stride_d and the batch / head strides multiples of 8,
 // output stride_d == 1, aligned pointers and tables, d % 8 == 0, d2 % 16 == 0.
 // ---------------------------------------------------------------------------
 constexpr int kTrTile = 64;  // positions per workgroup
+
+// In: lane (f, g) = (lane >> 3, lane & 7) holds element j = 0..7 of row f of an 8 x 8 block of
+// 16-bit values (one block per g), two per register, the lower-indexed one in bits 0..15.
+// Out: the same lane holds row f of the transposed block. `sel` is the byte selector of the
+// first stage: 0x05040100 in lanes with even f, 0x03020706 in lanes with odd f.
+__device__ __forceinline__ u32x4 transpose_8x8_halfwords(const u32x4& r, uint32_t sel)
+{
+    // lanes f and f ^ 1 (8 apart: a rotation by 8 inside a row of 16 lanes): afterwards register k holds
+    // column 2k + (f & 1) of the row pair (f & ~1, f | 1)
+    uint32_t t[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const uint32_t other = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)r[k], 0x128, 0xF, 0xF, false);  // row_ror:8
+        t[k] = __builtin_amdgcn_perm(other, r[k], sel);
+    }
+    // lanes f and f ^ 2 (16 apart): the odd rows of 16 lanes of the first register change places with the
+    // even rows of the second
+    const auto a = __builtin_amdgcn_permlane16_swap(t[0], t[1], false, false);
+    const auto b = __builtin_amdgcn_permlane16_swap(t[2], t[3], false, false);
+    // lanes f and f ^ 4 (32 apart): the upper half-wave of the first register with the lower of the second
+    const auto c = __builtin_amdgcn_permlane32_swap(a[0], b[0], false, false);
+    const auto d = __builtin_amdgcn_permlane32_swap(a[1], b[1], false, false);
+    return u32x4{c[0], d[0], c[1], d[1]};
+}
 
 template <int DT, bool BWD, int P, typename Tables>
 __global__ void __launch_bounds__(256)
@@ -341,42 +371,80 @@ rope_tr_kernel(RopeTensor T, Tables tab, int s, int cpr, int rot_chunks, int row
     static_assert(DT != NHP_F32, "16-bit data");
     constexpr int V = 8;
     extern __shared__ u32x4 tile[];  // [kTrTile][row_chunks] chunks of 8 elements
-    uint16_t* tile16 = reinterpret_cast<uint16_t*>(tile);
     const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = blockIdx.x;
     const int s0 = blockIdx.y * kTrTile;
     const int bi = r / T.h;
     const int hi = r - bi * T.h;
-    const int d = cpr * V;
     const uint16_t* in = static_cast<const uint16_t*>(T.in) + bi * T.is_b + hi * T.is_h;
     uint16_t* out = static_cast<uint16_t*>(T.out) + bi * T.os_b + hi * T.os_h;
 
-    const int sc = tid & 7;   // which 8 positions of the tile
-    const int dr = tid >> 3;  // feature within a pass of 32
+    const int sc = lane & 7;  // which 8 positions of the tile
+    const int f = lane >> 3;  // feature within the output chunk of this wave and pass
     const int pos8 = s0 + sc * 8;
     u32x4 raw[P];
 #pragma unroll
     for (int p = 0; p < P; ++p) {
-        const int di = p * 32 + dr;
+        const int c = p * 4 + wave;  // output chunk: wave-uniform
         raw[p] = u32x4{0, 0, 0, 0};
-        if (di < d && pos8 < s) raw[p] = load16_stream(in + (int64_t)di * is_d + pos8);
+        if (c < cpr && pos8 < s) raw[p] = load16_stream(in + (int64_t)(c * V + f) * is_d + pos8);
     }
-    const int row_elems = row_chunks * V;
+    const uint32_t sel = (f & 1) ? 0x03020706u : 0x05040100u;
 #pragma unroll
     for (int p = 0; p < P; ++p) {
-        const int di = p * 32 + dr;
-        if (di < d) {
-            const int slot = ((di >> 3) ^ sc) * V + (di & 7);
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const uint32_t word = raw[p][j >> 1];
-                tile16[(sc * 8 + j) * row_elems + slot] = (uint16_t)((j & 1) ? (word >> 16) : (word & 0xffffu));
-            }
+        const int c = p * 4 + wave;
+        if (c < cpr) {
+            // afterwards this lane holds the 8 features of chunk c at position sc * 8 + f of the tile
+            tile[(sc * 8 + f) * row_chunks + (c ^ sc)] = transpose_8x8_halfwords(raw[p], sel);
         }
     }
     __syncthreads();
 
     const int half = rot_chunks / 2;
+    if (rot_chunks > 0 && rot_chunks < cpr) {
+        // Partial rotary dimension: rotate in place in LDS, one work item per pair of chunks (c, c + half), so
+        // that every lane that does arithmetic is busy; then copy the tile out whole head vectors at a time
+        // (storing the rotated chunks straight from these lanes, 32 bytes at a time, measured 20 % slower).
+        for (int idx = tid; idx < kTrTile * half; idx += 256) {
+            const int row = idx / half;
+            const int c = idx - row * half;
+            const int pc = c + half;
+            const int pos = s0 + row;
+            if (pos >= s) continue;
+            const int swz = row >> 3;
+            u32x4* pa = &tile[row * row_chunks + (c ^ swz)];
+            u32x4* pb = &tile[row * row_chunks + (pc ^ swz)];
+            float ca[V], sa[V], cb[V], sb[V], xa[V], xb[V], ya[V], yb[V];
+            tab.get_vec(pos, (int64_t)c * V, ca, sa);
+            tab.get_vec(pos, (int64_t)pc * V, cb, sb);
+            chunk_to_float<DT>(*pa, xa);
+            chunk_to_float<DT>(*pb, xb);
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                if (!BWD) {
+                    ya[v] = rot<DT, true>(xa[v], ca[v], xb[v], sa[v]);
+                    yb[v] = rot<DT, false>(xb[v], cb[v], xa[v], sb[v]);
+                } else {
+                    ya[v] = rot<DT, false>(xa[v], ca[v], xb[v], sb[v]);
+                    yb[v] = rot<DT, true>(xb[v], cb[v], xa[v], sa[v]);
+                }
+            }
+            *pa = float_to_chunk<DT>(ya);
+            *pb = float_to_chunk<DT>(yb);
+        }
+        __syncthreads();
+        for (int idx = tid; idx < kTrTile * cpr; idx += 256) {
+            const int row = idx / cpr;
+            const int c = idx - row * cpr;
+            const int pos = s0 + row;
+            if (pos >= s) continue;
+            store16_stream(out + (int64_t)pos * T.os_s + (int64_t)c * V, tile[row * row_chunks + (c ^ (row >> 3))]);
+        }
+        return;
+    }
+
     for (int idx = tid; idx < kTrTile * cpr; idx += 256) {
         const int row = idx / cpr;
         const int c = idx - row * cpr;
@@ -744,6 +812,32 @@ static int rope_cached_qk(void* q_out, void* k_out, const void* q_in, const void
     return NHP_ERR_DTYPE;
 }
 
+template <bool BWD>
+static int rope_freqs_qk(void* q_out, void* k_out, const void* q_in, const void* k_in, const float* freqs, int64_t s,
+                         int64_t b, int64_t hq, int64_t hk, int64_t d, int64_t d2, const int64_t* qis,
+                         const int64_t* kis, const int64_t* qos, const int64_t* kos, int dtype, void* stream)
+{
+    if (dtype != NHP_F16 && dtype != NHP_BF16 && dtype != NHP_F32) return NHP_ERR_DTYPE;
+    bool empty_q, empty_k;
+    int rc = check_common(q_out, q_in, s, b, hq, d, d2, qis, qos, empty_q);
+    if (rc != NHP_OK) return rc;
+    rc = check_common(k_out, k_in, s, b, hk, d, d2, kis, kos, empty_k);
+    if (rc != NHP_OK) return rc;
+    if (empty_q || empty_k) {
+        if (!empty_q) return rope_freqs<BWD>(q_out, q_in, freqs, s, b, hq, d, d2, qis, qos, dtype, stream);
+        if (!empty_k) return rope_freqs<BWD>(k_out, k_in, freqs, s, b, hk, d, d2, kis, kos, dtype, stream);
+        return NHP_OK;
+    }
+    if (q_out == k_in || k_out == q_in || q_out == k_out) return NHP_ERR_ALIAS;
+    if (d2 > 0 && !freqs) return NHP_ERR_NULL;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    RopeArgs q{q_out, q_in, s, b, hq, d, d2, {qis[0], qis[1], qis[2], qis[3]}, {qos[0], qos[1], qos[2], qos[3]}, st};
+    RopeArgs k{k_out, k_in, s, b, hk, d, d2, {kis[0], kis[1], kis[2], kis[3]}, {kos[0], kos[1], kos[2], kos[3]}, st};
+    if (dtype == NHP_BF16) return rope_launch_pair<NHP_BF16, BWD>(q, k, FreqTable<NHP_BF16>{freqs, d2}, true);
+    if (dtype == NHP_F16) return rope_launch_pair<NHP_F16, BWD>(q, k, FreqTable<NHP_F16>{freqs, d2}, true);
+    return rope_launch_pair<NHP_F32, BWD>(q, k, FreqTable<NHP_F32>{freqs, d2}, true);
+}
+
 }  // namespace nhp
 
 using namespace nhp;
@@ -798,6 +892,24 @@ int nhp_rope_cached_qk_bwd(void* q_out, void* k_out, const void* q_in, const voi
 {
     return rope_cached_qk<true>(q_out, k_out, q_in, k_in, cos, sin, s, b, hq, hk, d, d2, q_in_stride, k_in_stride,
                                 q_out_stride, k_out_stride, dtype, cs_dtype, stream);
+}
+
+int nhp_rope_freqs_qk_fwd(void* q_out, void* k_out, const void* q_in, const void* k_in, const float* freqs, int64_t s,
+                          int64_t b, int64_t hq, int64_t hk, int64_t d, int64_t d2, const int64_t q_in_stride[4],
+                          const int64_t k_in_stride[4], const int64_t q_out_stride[4], const int64_t k_out_stride[4],
+                          int dtype, void* stream)
+{
+    return rope_freqs_qk<false>(q_out, k_out, q_in, k_in, freqs, s, b, hq, hk, d, d2, q_in_stride, k_in_stride,
+                                q_out_stride, k_out_stride, dtype, stream);
+}
+
+int nhp_rope_freqs_qk_bwd(void* q_out, void* k_out, const void* q_in, const void* k_in, const float* freqs, int64_t s,
+                          int64_t b, int64_t hq, int64_t hk, int64_t d, int64_t d2, const int64_t q_in_stride[4],
+                          const int64_t k_in_stride[4], const int64_t q_out_stride[4], const int64_t k_out_stride[4],
+                          int dtype, void* stream)
+{
+    return rope_freqs_qk<true>(q_out, k_out, q_in, k_in, freqs, s, b, hq, hk, d, d2, q_in_stride, k_in_stride,
+                               q_out_stride, k_out_stride, dtype, stream);
 }
 
 int nhp_abi_version(void) { return 1; }

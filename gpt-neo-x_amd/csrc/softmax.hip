@@ -146,7 +146,8 @@ __device__ __forceinline__ void locate_row(uint32_t block, uint32_t rows_per_mat
 // The columns of row q that take part in a causal softmax: [lo, hi) with
 // hi = min(q + 1, limit) and lo = max(0, q - window) (window = 0xffffffff: no
 // lower bound; limit = the number of real keys of the row's batch entry).
-// hi <= lo is an empty band: the row is written as zeros.
+// hi <= lo is an empty band (possible with key lengths only): the forward writes 1/n in every
+// column of such a row, the backward zeros.
 struct Band {
     uint32_t lo, hi;
 };
@@ -310,11 +311,27 @@ causal_fwd_kernel(uint16_t* y, const uint16_t* x, float scale, uint32_t total_ro
     // The whole row is written in one go, zeros outside the band included (as far as the caller reads
     // them): splitting a row's stores in time costs DRAM efficiency.
     const Band wr = written_range(q, window, n, zshift);
+    // A row that the key lengths leave without any key: 1/n in every column, what the softmax over a
+    // row of equal fill values gives on the reference's torch branch (megatron/model/fused_softmax.py:184-199).
+    uint32_t fill = 0;
+    if constexpr (PER_HEAD) {
+        if (ok && band.hi == 0) fill = Half2<DT>::pack(1.0f / (float)n, 1.0f / (float)n);
+    }
 #pragma unroll
     for (int k = 0; k < K; ++k) {
         const uint32_t col = chunk_col<L, W>(k, w, l);
         if (ok && col < wr.hi && col >= wr.lo) {
-            if ((act >> k & 1u) && col < band.hi && col + 8 > band.lo) {
+            if (PER_HEAD && fill != 0) {
+                store16_stream(yr + col, u32x4{fill, fill, fill, fill});
+                if constexpr (DROPOUT) {
+                    const float v = Half2<DT>::lo(fill);
+                    float f[8];
+                    const Philox rnd = dropout_bits(dk, (uint64_t)row * n + col);
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) f[j] = random16(rnd, j) < dk.threshold ? v * dk.scale : 0.0f;
+                    store16_stream(dropped + (size_t)row * n + col, pack8<DT>(f));
+                }
+            } else if ((act >> k & 1u) && col < band.hi && col + 8 > band.lo) {
                 const u32x4 py = pack8<DT>(z[k]);
                 store16_stream(yr + col, py);
                 if constexpr (DROPOUT) {
@@ -730,8 +747,9 @@ scalar_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
 
     // every thread reads and then writes the columns it owns, after the last
     // reduction barrier: y may alias x
+    const bool no_key = MODE == 0 && hi <= lo;  // only key lengths can empty a causal band: a uniform row
     for (uint64_t c = threadIdx.x; c < n; c += kScalarThreads) {
-        float p = 0.0f;
+        float p = no_key ? 1.0f / (float)n : 0.0f;
         if (c >= lo && c < hi) p = exp2_raw(fmaf(logit(c) - m, kLog2e, kExpBias)) * inv;
         yr[c] = Half2<DT>::to_bits(p);
         if (dropped != nullptr) {

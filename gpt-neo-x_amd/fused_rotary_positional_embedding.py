@@ -154,3 +154,42 @@ def backward_cached_qk(grad_q, grad_k, cos, sin, transpose_output, out=None):
     ``out``: optional ``(q_result, k_result)`` tensors to write into (any strides) instead of new ones."""
     return _run_cached_qk("fused_rotary_positional_embedding.backward_cached_qk", _hp.lib().nhp_rope_cached_qk_bwd,
                           grad_q, grad_k, cos, sin, transpose_output, out)
+
+
+def _run_freqs_qk(name, fn, q, k, freqs, transpose_output):
+    for t, what in ((q, "q"), (k, "k")):
+        _check(t.dim() == 4, "expected 4D tensor")
+        _check(t.size(0) == freqs.size(0), f"expected {what} and freqs tensor have the same sequence length")
+        _check(t.size(3) >= freqs.size(3),
+               f"expected the last dim of the {what} tensor equals or is greater than the freqs tensor")
+        _check(t.dtype in _FLOATS, f"{name}: unsupported dtype {t.dtype}")
+        _hp.require_gpu(t, name)
+    _check(freqs.dim() == 4, "expected 4D tensor")
+    _check(freqs.size(1) == 1 and freqs.size(2) == 1, "expected the second and third dims of the freqs tensor equal 1")
+    _check(freqs.dtype == torch.float32, "Dtype of the freqs tensor must be float")
+    _check(q.dtype == k.dtype and q.device == k.device, "q and k must have the same dtype and device")
+    _check(q.size(0) == k.size(0) and q.size(1) == k.size(1) and q.size(3) == k.size(3),
+           "q and k must agree in sequence length, batch size and head dimension")
+    _hp.require_gpu(freqs, name)
+    f = freqs.contiguous()
+    q_out = _new_output(q, transpose_output)
+    k_out = _new_output(k, transpose_output)
+    s, b, hq, d = q.shape
+    with _hp.device_guard(q):
+        rc = fn(q_out.data_ptr(), k_out.data_ptr(), q.data_ptr(), k.data_ptr(), f.data_ptr(), s, b, hq, k.size(2), d,
+                f.size(3), _hp.strides4(q), _hp.strides4(k), _hp.strides4(q_out), _hp.strides4(k_out),
+                _hp.dtype_code(q, name), _hp.stream_of(q))
+    _hp.check(rc, name)
+    return q_out, k_out
+
+
+def forward_qk(q, k, freqs, transpose_output):
+    """(not in the reference module) ``forward`` for q and k in one launch; k may have fewer heads."""
+    return _run_freqs_qk("fused_rotary_positional_embedding.forward_qk", _hp.lib().nhp_rope_freqs_qk_fwd, q, k, freqs,
+                         transpose_output)
+
+
+def backward_qk(grad_q, grad_k, freqs, transpose_output):
+    """(not in the reference module) ``backward`` for the gradients of q and k in one launch."""
+    return _run_freqs_qk("fused_rotary_positional_embedding.backward_qk", _hp.lib().nhp_rope_freqs_qk_bwd, grad_q, grad_k,
+                         freqs, transpose_output)

@@ -63,6 +63,8 @@ def _declare(lib):
         "nhp_rope_cached_bwd": ([vp, vp, vp, vp, i64, i64, i64, i64, i64, p64, p64, ci, ci, vp], ci),
         "nhp_rope_cached_qk_fwd": ([vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, p64, p64, p64, p64, ci, ci, vp], ci),
         "nhp_rope_cached_qk_bwd": ([vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, p64, p64, p64, p64, ci, ci, vp], ci),
+        "nhp_rope_freqs_qk_fwd": ([vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, p64, p64, p64, p64, ci, vp], ci),
+        "nhp_rope_freqs_qk_bwd": ([vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, p64, p64, p64, p64, ci, vp], ci),
         "nhp_rope_freqs_fwd": ([vp, vp, vp, i64, i64, i64, i64, i64, p64, p64, ci, vp], ci),
         "nhp_rope_freqs_bwd": ([vp, vp, vp, i64, i64, i64, i64, i64, p64, p64, ci, vp], ci),
         "nhp_bias_gelu_fwd": ([vp, vp, vp, i64, i64, ci, vp], ci),

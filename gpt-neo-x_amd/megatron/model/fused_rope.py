@@ -70,6 +70,29 @@ class FusedRoPEQKCachedFunc(torch.autograd.Function):
         return gq, gk, None, None, None
 
 
+class FusedRoPEQKFunc(torch.autograd.Function):
+    """RoPE of q and k from float32 angles in a single kernel launch."""
+
+    @staticmethod
+    def forward(ctx, q, k, freqs, transpose_output_memory=False):
+        ctx.transpose_output_memory = transpose_output_memory
+        ctx.save_for_backward(freqs)
+        return _kernels().forward_qk(q, k, freqs, transpose_output_memory)
+
+    @staticmethod
+    def backward(ctx, grad_q, grad_k):
+        (freqs,) = ctx.saved_tensors
+        gq, gk = _kernels().backward_qk(grad_q, grad_k, freqs, ctx.transpose_output_memory)
+        return gq, gk, None, None
+
+
+def fused_apply_rotary_pos_emb_qk(
+    q: torch.Tensor, k: torch.Tensor, freqs: torch.Tensor, transpose_output_memory: bool = False
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``fused_apply_rotary_pos_emb`` for q ``[s, b, hq, d]`` and k ``[s, b, hk, d]`` in one launch."""
+    return FusedRoPEQKFunc.apply(q, k, freqs, transpose_output_memory)
+
+
 def fused_apply_rotary_pos_emb(
     t: torch.Tensor, freqs: torch.Tensor, transpose_output_memory: bool = False
 ) -> torch.Tensor:

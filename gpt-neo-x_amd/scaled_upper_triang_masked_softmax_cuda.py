@@ -82,7 +82,7 @@ def forward(input, scale_factor, window=None, alibi_slopes=None, bias=None, key_
         `scores += bias` would (e.g. a relative-position bias shared by the batch).
     key_lengths: integer tensor [batch] on the GPU, input being [batch * heads, s, s]:
         keys at or beyond a batch entry's length are padding and get probability 0
-        (rows without any key left are all zeros).
+        (a row without any key left is 1/seq_len in every column, as on the torch branch).
     zero_block: for a caller that reads the result in square blocks of this many rows and columns
         and skips the blocks without a visible (query, key) pair: row q is only written from the
         start of the block of the first key that the first row of its block sees to the end of the

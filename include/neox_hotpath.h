@@ -124,7 +124,9 @@ int nhp_causal_softmax_bwd(void* dx, const void* dy, const void* y, float scale,
  *      diagonal, i.e. the mask `causal | (k >= len)` handed to
  *      FusedScaleMaskSoftmax.forward (megatron/model/fused_softmax.py:140-146),
  *      which the reference's causal kernel ignores. Padding keys are never
- *      read. A row left without any key (length 0) is written as zeros.
+ *      read. A row left without any key (length 0, or a window that starts in
+ *      the padding) is 1/seq_len in every column, as the softmax of the
+ *      reference's torch branch over a row of equal fill values.
  *      Values below 0 count as 0, values above seq_len as seq_len.
  *
  * The backward takes the same window and key_lengths (masked positions get
@@ -401,6 +403,27 @@ int nhp_rope_freqs_bwd(void* out, const void* in, const float* freqs,
                        int64_t s, int64_t b, int64_t h, int64_t d, int64_t d2,
                        const int64_t in_stride[4], const int64_t out_stride[4],
                        int dtype, void* stream);
+
+/*
+ * q and k in one launch from the angles, as nhp_rope_cached_qk_fwd / _bwd do from the tables:
+ * exactly nhp_rope_freqs_fwd / _bwd applied to (q_out, q_in) and (k_out, k_in). Fused form of the
+ * two calls of fused_apply_rotary_pos_emb (megatron/model/fused_rope.py:61-76) that a caller makes
+ * for the query and the key of a layer (megatron/model/transformer.py:898-910 does so with the
+ * cached variant).
+ */
+int nhp_rope_freqs_qk_fwd(void* q_out, void* k_out, const void* q_in, const void* k_in,
+                          const float* freqs,
+                          int64_t s, int64_t b, int64_t hq, int64_t hk, int64_t d, int64_t d2,
+                          const int64_t q_in_stride[4], const int64_t k_in_stride[4],
+                          const int64_t q_out_stride[4], const int64_t k_out_stride[4],
+                          int dtype, void* stream);
+
+int nhp_rope_freqs_qk_bwd(void* q_out, void* k_out, const void* q_in, const void* k_in,
+                          const float* freqs,
+                          int64_t s, int64_t b, int64_t hq, int64_t hk, int64_t d, int64_t d2,
+                          const int64_t q_in_stride[4], const int64_t k_in_stride[4],
+                          const int64_t q_out_stride[4], const int64_t k_out_stride[4],
+                          int dtype, void* stream);
 
 /* ------------------------------------------------------------------------
  * Element-wise neighbours of attention in the transformer layer

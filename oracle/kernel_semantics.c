@@ -19,9 +19,7 @@
  *     dispatcher narrows it to the input dtype first
  *     (scaled_upper_triang_masked_softmax.h:368, scaled_masked_softmax.h:358);
  *     pass an already narrowed value to reproduce that.
- * Two definitions that are this build's own, for variants the reference's kernels do not have:
- *   - with key lengths, a row that keeps no key at all is written as zeros (the torch
- *     fallback given the merged mask yields 1/s there; see oracle_causal_softmax_ex_fwd);
+ * One definition that is this build's own, for a variant the reference's kernels do not have:
  *   - the attention-dropout mask is the counter-based one of layer_semantics.c: which
  *     elements torch's generator would drop is PARITY UNPINNED by construction, everything
  *     else about oracle_causal_softmax_dropout_fwd/bwd is the composition of pinned parts.
@@ -79,9 +77,8 @@ static void softmax_row(float* z, int64_t n)
  *     of batch entry b = matrix / heads are padding and masked like the keys
  *     above the diagonal (the mask `causal | (k >= len)` given to
  *     forward_torch_softmax, fused_softmax.py:184-199). A row that keeps no
- *     key at all is written as zeros (the fallback's softmax over a row of
- *     equal fill values would give 1/s there; attention to padding only is
- *     meaningless either way and zeros keep the output finite).
+ *     key at all is 1/s in every column, above the diagonal too: what that
+ *     fallback's softmax over a row of equal fill values gives.
  */
 int oracle_causal_softmax_ex_fwd(void* y, const void* x, float scale, int64_t batches, int64_t s,
                                  int64_t window, const float* slopes, const void* bias,
@@ -101,7 +98,7 @@ int oracle_causal_softmax_ex_fwd(void* y, const void* x, float scale, int64_t ba
                 if (len < hi) hi = len;
             }
             if (hi <= lo) {
-                for (int64_t k = 0; k < s; ++k) store_elem(y, base + k, dt, 0.0f);
+                for (int64_t k = 0; k < s; ++k) store_elem(y, base + k, dt, 1.0f / (float)s);
                 continue;
             }
             for (int64_t k = lo; k < hi; ++k) {

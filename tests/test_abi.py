@@ -115,6 +115,10 @@ def test_argument_validation_needs_no_gpu(hotpath):
     assert lib.nhp_rope_cached_fwd(o, p, null, p, 1, 1, 1, 8, 8, st, st, BF16, BF16, None) == -3
     assert lib.nhp_rope_freqs_fwd(o, p, null, 1, 1, 1, 8, 8, st, st, BF16, None) == -3
     assert lib.nhp_rope_freqs_fwd(o, p, p, 1, 1, 1, 8, 8, None, st, BF16, None) == -3
+    assert lib.nhp_rope_freqs_qk_fwd(o, ctypes.c_void_p(0xa000), p, p, null, 1, 1, 1, 1, 8, 8, st, st, st, st, BF16, None) == -3
+    assert lib.nhp_rope_freqs_qk_fwd(o, o, p, p, p, 1, 1, 1, 1, 8, 8, st, st, st, st, BF16, None) == -6
+    assert lib.nhp_rope_freqs_qk_bwd(null, null, null, null, null, 0, 1, 1, 1, 8, 8, st, st, st, st, F16, None) == 0
+    assert lib.nhp_rope_freqs_qk_bwd(o, ctypes.c_void_p(0xa000), p, p, p, 1, 1, 1, 1, 8, 16, st, st, st, st, F16, None) == -2
     # mask batch dimension
     assert lib.nhp_masked_softmax_fwd(p, p, p, 1.0, 4, 1, 2, 8, 3, F16, None) == -4
     # aliasing that is not allowed: dx over y, rotary in place

@@ -261,3 +261,61 @@ def test_rope_input_contiguous_along_the_sequence(hotpath, shape, dtype, cs_fp32
         want = oracle.rope_cached(t[8:].contiguous(), cos[: s - 8].contiguous(), sin[: s - 8].contiguous(), backward=True)
         got = util.abi_rope_cached(hotpath, w, cos[: s - 8].contiguous().to(DEV), sin[: s - 8].contiguous().to(DEV), True)
         assert torch.equal(util.raw_bits(got.cpu()), util.raw_bits(want))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("shape", [(64, 2, 3, 128, 128), (200, 2, 4, 128, 32), (136, 2, 2, 96, 48), (256, 1, 2, 256, 256)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_rope_from_angles_on_input_contiguous_along_the_sequence(hotpath, shape, dtype):
+    """The angles variant on the sequence-major layout takes the transposing kernel as well: same results as on
+    the contiguous copy of the input bit for bit, and the oracle's to the tolerance of the angles variant."""
+    s, b, h, d, d2 = shape
+    say(f"rope freqs sequence-major {shape} {dtype}")
+    base = util.randn((b, h, d, s), dtype, seed=s + d + 1)
+    t = base.permute(3, 0, 1, 2)
+    t_d = base.to(DEV).permute(3, 0, 1, 2)
+    ang = (util.randn((s, 1, 1, d2), torch.float32, seed=d2 + 5) * 3.0).contiguous()
+    for backward in (False, True):
+        got = util.abi_rope_freqs(hotpath, t_d, ang.to(DEV), backward)
+        same = util.abi_rope_freqs(hotpath, t_d.contiguous(), ang.to(DEV), backward)
+        assert torch.equal(util.raw_bits(got.cpu()), util.raw_bits(same.cpu())), backward
+        want = oracle.rope_freqs(t.contiguous(), ang, backward=backward)
+        util.assert_rope_freqs_close(got.cpu(), want, t.contiguous(), ang, backward, f"seq-major freqs bwd={backward}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("shape", [(16, 2, 8, 8, 128, 128), (16, 2, 8, 2, 128, 32), (9, 3, 5, 1, 64, 16), (7, 2, 4, 4, 24, 8)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_rope_from_angles_qk_single_launch_equals_two_calls(hotpath, shape, dtype):
+    """nhp_rope_freqs_qk_* against two nhp_rope_freqs_* calls bit for bit (same device sine and cosine), forward and
+    backward, on views of a fused projection, and through the autograd function against the per-tensor function."""
+    from megatron.model.fused_rope import fused_apply_rotary_pos_emb, fused_apply_rotary_pos_emb_qk
+
+    s, b, hq, hk, d, d2 = shape
+    buf = util.randn((s, b, hq + 2 * hk, d), dtype, seed=s + d).to(DEV)
+    q, k = buf[:, :, :hq], buf[:, :, hq : hq + hk]
+    ang = (util.randn((s, 1, 1, d2), torch.float32, seed=d2 + 9) * 5.0).contiguous().to(DEV)
+    L = hotpath.lib()
+    for backward in (False, True):
+        for transpose in (False, True):
+            want_q = util.abi_rope_freqs(hotpath, q, ang, backward, transpose)
+            want_k = util.abi_rope_freqs(hotpath, k, ang, backward, transpose)
+            got_q = util._rope_out(q, transpose)
+            got_k = util._rope_out(k, transpose)
+            fn = L.nhp_rope_freqs_qk_bwd if backward else L.nhp_rope_freqs_qk_fwd
+            rc = fn(got_q.data_ptr(), got_k.data_ptr(), q.data_ptr(), k.data_ptr(), ang.data_ptr(), s, b, hq, hk, d, d2,
+                    hotpath.strides4(q), hotpath.strides4(k), hotpath.strides4(got_q), hotpath.strides4(got_k),
+                    hotpath.dtype_code(q, "t"), None)
+            assert rc == 0
+            torch.cuda.synchronize()
+            assert torch.equal(util.raw_bits(got_q.cpu()), util.raw_bits(want_q.cpu()))
+            assert torch.equal(util.raw_bits(got_k.cpu()), util.raw_bits(want_k.cpu()))
+    qd, kd = q.detach().clone().requires_grad_(True), k.detach().clone().requires_grad_(True)
+    qe, ke = q.detach().clone().requires_grad_(True), k.detach().clone().requires_grad_(True)
+    gq, gk = util.randn(q.shape, dtype, seed=1).to(DEV), util.randn(k.shape, dtype, seed=2).to(DEV)
+    fq, fk = fused_apply_rotary_pos_emb_qk(qd, kd, ang)
+    torch.autograd.backward([fq, fk], [gq, gk])
+    oq, ok = fused_apply_rotary_pos_emb(qe, ang), fused_apply_rotary_pos_emb(ke, ang)
+    torch.autograd.backward([oq, ok], [gq, gk])
+    for a_, b_ in ((fq, oq), (fk, ok), (qd.grad, qe.grad), (kd.grad, ke.grad)):
+        assert torch.equal(util.raw_bits(a_.detach().cpu()), util.raw_bits(b_.detach().cpu()))
