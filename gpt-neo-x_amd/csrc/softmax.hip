@@ -451,41 +451,19 @@ masked_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
             raw[k] = u32x4{0, 0, 0, 0};
             if (live[k]) raw[k] = load16_stream(xr + col);
         }
+        // the bias chunks are requested with the scores; both are used in the logit loop below
+        u32x4 rbias[PER_HEAD ? K : 1];
+        float slope = 0.0f;
         if constexpr (PER_HEAD) {
             if (bias != nullptr) {
                 const uint16_t* br = bias + ((size_t)h * sq + qi) * n;
 #pragma unroll
                 for (int k = 0; k < K; ++k) {
-                    if (live[k]) {
-                        const u32x4 rb = load16(br + chunk_col<L, W>(k, w, l));  // re-used by every batch entry
-                        float f[8], g[8];
-                        unpack8<DT>(raw[k], f);
-                        unpack8<DT>(rb, g);
-#pragma unroll
-                        for (int j = 0; j < 8; ++j) f[j] = f[j] + g[j];
-                        raw[k] = pack8<DT>(f);
-                    }
+                    rbias[k] = u32x4{0, 0, 0, 0};
+                    if (live[k]) rbias[k] = load16(br + chunk_col<L, W>(k, w, l));  // re-used by every batch entry
                 }
             }
-            if (slopes != nullptr) {
-                const float slope = Half2<DT>::round(slopes[h]);
-#pragma unroll
-                for (int k = 0; k < K; ++k) {
-                    const uint32_t col = chunk_col<L, W>(k, w, l);
-                    if (live[k] && col <= qi) {
-                        float f[8];
-                        unpack8<DT>(raw[k], f);
-#pragma unroll
-                        for (int j = 0; j < 8; ++j) {
-                            if (col + j <= qi) {
-                                const float dist = Half2<DT>::round(-(float)((int)qi - (int)(col + j)));
-                                f[j] = Half2<DT>::round(f[j] + Half2<DT>::round(dist * slope));
-                            }
-                        }
-                        raw[k] = pack8<DT>(f);
-                    }
-                }
-            }
+            if (slopes != nullptr) slope = Half2<DT>::round(slopes[h]);
         }
 
         // Chunks whose eight columns are all masked hold eight copies of the fill value:
@@ -497,6 +475,28 @@ masked_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
             if (live[k]) {
                 float f[8];
                 unpack8<DT>(raw[k], f);
+                if constexpr (PER_HEAD) {
+                    if (bias != nullptr) {
+                        float g[8];
+                        unpack8<DT>(rbias[k], g);
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) f[j] = Half2<DT>::round(f[j] + g[j]);
+                    }
+                    const uint32_t col = chunk_col<L, W>(k, w, l);
+                    if (slopes != nullptr && col <= qi) {
+                        // -(q - k) for the chunk's first column; formed anew for every head (an opaque value)
+                        // so that the 8 K distances are not kept in registers across the loop over the heads
+                        // Above the diagonal the AliBi matrix is 0: the distance is clamped there, which
+                        // leaves the score as it is (a -0 becomes +0, the same logit).
+                        float d0 = (float)((int)col - (int)qi);
+                        asm volatile("" : "+v"(d0));
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) {
+                            const float dist = Half2<DT>::round(fminf(d0 + (float)j, 0.0f));
+                            f[j] = Half2<DT>::round(f[j] + Half2<DT>::round(dist * slope));
+                        }
+                    }
+                }
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     const uint32_t byte = (mb[k][j >> 2] >> (8 * (j & 3))) & 0xffu;
@@ -813,7 +813,7 @@ struct RowPlan {
 constexpr int64_t kMaxResidentRow = 65536;
 constexpr int kBlockWaves = 4;  // waves per workgroup when a wave owns whole rows
 
-enum RowKind { kCausalFwd, kCausalFwdExtra, kCausalBwd, kMaskedFwd, kMaskedBwd };
+enum RowKind { kCausalFwd, kCausalFwdExtra, kCausalBwd, kMaskedFwd, kMaskedBwd, kMaskedFwdExtra };
 
 // Geometry for rows of n elements, from measurements on MI355X. HBM efficiency
 // drops when too many different rows are in flight per CU, and a row should be
@@ -847,7 +847,7 @@ static bool plan_row(int64_t n, RowKind kind, RowPlan& p, bool blocks = false)
     p.L = 64;
     const int64_t segs = (chunks + 63) / 64;  // 1 KiB segments per row
     int W, K;
-    if (kind == kCausalFwdExtra && segs <= 4) {
+    if ((kind == kCausalFwdExtra || kind == kMaskedFwdExtra) && segs <= 4) {
         // Causal forward with per-element extra work (AliBi, bias tensor):
         // without a barrier in the row the extra instructions of one wave overlap the loads of the
         // others (measured at 2048: the extras cost 30-45 us with two waves per row, 15-20 us with one)
@@ -857,7 +857,10 @@ static bool plan_row(int64_t n, RowKind kind, RowPlan& p, bool blocks = false)
         W = 16;
         K = 8;
     } else {
-        K = (kind == kCausalFwd || kind == kCausalFwdExtra || kind == kMaskedFwd || kind == kCausalBwd) ? 2 : 1;
+        K = (kind == kCausalFwd || kind == kCausalFwdExtra || kind == kMaskedFwd || kind == kMaskedFwdExtra ||
+             kind == kCausalBwd)
+                ? 2
+                : 1;
         while (8 * K < segs) K *= 2;
         static const int kWaves[] = {1, 2, 3, 4, 6, 8};
         W = 8;
@@ -1027,7 +1030,9 @@ static int masked_fwd(void* y, const void* x, const uint8_t* mask, float scale, 
     const uint16_t* xp = static_cast<const uint16_t*>(x);
     const uint16_t* bp = static_cast<const uint16_t*>(ex.bias);
     const bool mask_ok = (reinterpret_cast<uintptr_t>(mask) & 7u) == 0;
-    if (plan_row(n, kMaskedFwd, p) && aligned16(x) && aligned16(y) && aligned16(dropped) && aligned16(ex.bias) && mask_ok) {
+    // AliBi and the bias tensor are per-element work: one wave per row, as in the causal kernel
+    const RowKind kind = (ex.slopes != nullptr || ex.bias != nullptr) ? kMaskedFwdExtra : kMaskedFwd;
+    if (plan_row(n, kind, p) && aligned16(x) && aligned16(y) && aligned16(dropped) && aligned16(ex.bias) && mask_ok) {
 #define LAUNCH_MASKED(L_, K_, W_, DROP_, PH_)                                                         \
     masked_fwd_kernel<DT, L_, K_, W_, kBlockWaves, DROP_, PH_><<<(uint32_t)(rb * hgs), Geo<L_, K_, W_, kBlockWaves>::kThreads, 0, st>>>( \
         yp, xp, mask, scale, (uint32_t)bq_rows, (uint32_t)sq, (uint32_t)np, (uint32_t)n, hpw, hgs, per_batch, \

@@ -237,7 +237,9 @@ int nhp_causal_softmax_ex_dropout_bwd(void* dx, const void* dy, const void* y, f
  *                the diagonal, with the roundings of AliBi.forward
  *                (megatron/model/positional_embeddings.py:219-257), after the bias;
  *   key_lengths  [b] int32: keys k >= key_lengths[b] count as masked (as if their mask bytes were 1).
- * Results are bit-identical to nhp_masked_softmax_fwd on scores and a mask prepared that way. The
+ * Results are those of nhp_masked_softmax_fwd on scores and a mask prepared that way (bit-identical with
+ * key_lengths alone; with AliBi or a bias the kernel takes another launch shape, hence another summation
+ * order: within 1 ulp, zeros in the same places). The
  * backward is nhp_masked_softmax_bwd (it takes no mask). The _dropout variant also writes
  * dropped = dropout(y) as nhp_masked_softmax_dropout_fwd does; its backward is
  * nhp_masked_softmax_dropout_bwd.

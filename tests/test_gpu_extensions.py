@@ -519,8 +519,8 @@ MASKED_EX_CASES = [
 def test_masked_softmax_with_extras_vs_oracle(hotpath, case, pad_batches, dtype):
     """nhp_masked_softmax_ex_fwd against the oracle's composition (eager preparation of scores and mask, then
     the plain padding-mask softmax): 2 ulp, masked keys exactly what the plain kernel leaves there, the scores
-    and bias entries of whole chunks of padding keys never read, and bit-identical to the plain entry point
-    given the prepared operands."""
+    and bias entries of whole chunks of padding keys never read, and the plain entry point's result on the
+    prepared operands (bit for bit with key lengths alone, within 1 ulp when AliBi or a bias change the launch shape)."""
     b, np_, sq, sk, extras = case
     print(f"masked ex case {case} {pad_batches} {dtype}", flush=True)
     scale = 1 / math.sqrt(128)
@@ -554,7 +554,12 @@ def test_masked_softmax_with_extras_vs_oracle(hotpath, case, pad_batches, dtype)
     # the same kernel arithmetic as the plain entry point on prepared operands
     xs, ms = oracle.prepared_masked_inputs(x, mask, slopes, bias, lengths)
     plain = util.abi_masked_fwd(hotpath, xs.to(DEV), ms.contiguous().to(DEV), scale).cpu()
-    assert torch.equal(util.raw_bits(got), util.raw_bits(plain))
+    if slopes is None and bias is None:
+        assert torch.equal(util.raw_bits(got), util.raw_bits(plain))
+    else:
+        # per-element extras take a launch shape of their own (one wave per row): another summation order
+        util.assert_ulp_close(got, plain, 1, "vs the plain entry point on prepared operands")
+        assert torch.equal(util.raw_bits(got) == 0, util.raw_bits(plain) == 0)
     if lengths is not None and b > 1:
         assert torch.equal(got[-1], torch.full_like(got[-1], 1.0 / sk))
     # with dropout on top: the same probabilities, and the oracle's dropout of them
