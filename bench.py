@@ -7,7 +7,8 @@ A step is one pass of the hot path over one batch of synthetic input, through
 the drop-in extension modules (which call libneox_hotpath.so):
 
   pythia-1.4b (default; the configuration the headline metric is quoted on)
-      rotary fwd on q and k  [s=2048, b=8, h=16, d=128] bf16, rotary_pct 0.25
+      rotary fwd on q and k  [s=2048, b=8, h=16, d=128] bf16, rotary_pct 0.25 (both tensors in one
+                             launch; --rope-per-tensor: one launch each, the reference's call style)
       causal softmax fwd     [b*h=128, 2048, 2048] bf16, scale 1/sqrt(128)
       causal softmax bwd     same shape, in place on the upstream gradient
       rotary bwd on dq, dk
@@ -31,7 +32,9 @@ the drop-in extension modules (which call libneox_hotpath.so):
 
   hbm-probes     kernels that only move data (libneox_probe.so): a plain streaming copy of 64 MiB, 128 MiB and
                  1 GiB tensors, and the causal softmax forward's access pattern (lower-triangle reads, dense writes)
-                 at [128,2048,2048] and [64,8192,8192]: what the memory system gives for those patterns and sizes
+                 at [128,2048,2048] and [64,8192,8192], and the layout change of the transposing rotary kernel
+                 ([128,128,2048] contiguous along the sequence -> [2048,128,128]): what the memory system gives for
+                 those patterns and sizes
 
   mlp-gelu-1.4b  bias + tanh-GeLU fwd and bwd (with the bias gradient) on the MLP activation [2048*8, 8192] bf16
   swiglu-7b      SwiGLU forward and backward on the Llama-2 7B MLP activation [4096*4, 2*11008] -> [4096*4, 11008] bf16
@@ -147,7 +150,7 @@ class Timer:
         self.pairs = {}
 
 
-def make_workload(name, torch, dev, fresh_dy=False):
+def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False):
     import fused_rotary_positional_embedding as rope_ext
     import scaled_masked_softmax_cuda as masked_ext
     import scaled_upper_triang_masked_softmax_cuda as causal_ext
@@ -179,8 +182,11 @@ def make_workload(name, torch, dev, fresh_dy=False):
         dy = randn((a, s, s), 1, torch.bfloat16)
         fwd_b, bwd_b = causal_bytes(a, s)
         rb = rope_bytes(s, b, h, d, d2)
-        kernel_bytes = {"rope_fwd": 2 * rb, "causal_softmax_fwd": fwd_b, "causal_softmax_bwd": bwd_b,
-                        "rope_bwd": 2 * rb}
+        # q and k share one launch and one read of the tables (--rope-per-tensor: one launch per tensor,
+        # the reference's call style, each reading the tables)
+        rope_b = 2 * rb if rope_per_tensor else 2 * rb - 2 * s * d2 * 2
+        kernel_bytes = {"rope_fwd": rope_b, "causal_softmax_fwd": fwd_b, "causal_softmax_bwd": bwd_b,
+                        "rope_bwd": rope_b}
         dense = {"causal_softmax_fwd": 2 * a * s * s * 2, "causal_softmax_bwd": 3 * a * s * s * 2}
 
         # --fresh-dy: the backward works in place, so without this its input shrinks from step to step
@@ -190,12 +196,18 @@ def make_workload(name, torch, dev, fresh_dy=False):
 
         def step(t):
             def rope_f():
-                rope_ext.forward_cached(q, cos, sin, False)
-                rope_ext.forward_cached(k, cos, sin, False)
+                if rope_per_tensor:
+                    rope_ext.forward_cached(q, cos, sin, False)
+                    rope_ext.forward_cached(k, cos, sin, False)
+                else:
+                    rope_ext.forward_cached_qk(q, k, cos, sin, False)
 
             def rope_b():
-                rope_ext.backward_cached(dq, cos, sin, False)
-                rope_ext.backward_cached(dk, cos, sin, False)
+                if rope_per_tensor:
+                    rope_ext.backward_cached(dq, cos, sin, False)
+                    rope_ext.backward_cached(dk, cos, sin, False)
+                else:
+                    rope_ext.backward_cached_qk(dq, dk, cos, sin, False)
 
             t.run("rope_fwd", rope_f)
             y = t.run("causal_softmax_fwd", lambda: causal_ext.forward(x, scale))
@@ -210,6 +222,7 @@ def make_workload(name, torch, dev, fresh_dy=False):
         cfg = {"workload": name, "scores": [a, s, s], "qk": [s, b, h, d], "rotary_dim": d2,
                "scale": "1/sqrt(%d)" % d, "bytes_convention": "causal-min (reads of the lower triangle, dense writes)",
                "dominant_kernel_signature": "softmax_bwd causal " + softmax_signature(hp.lib(), s, 2)}
+        cfg["rotary_launches"] = "one per tensor" if rope_per_tensor else "q and k in one launch"
         if fresh_dy:
             cfg["fresh_dy"] = True
         return step, kernel_bytes, dense, "causal_softmax_bwd", "bf16", cfg
@@ -408,6 +421,12 @@ def make_workload(name, torch, dev, fresh_dy=False):
             key = f"causal_pattern_{a}x{s}x{s}"
             kernel_bytes[key] = causal_bytes(a, s)[0]
             pat.append((key, x, y, a, s))
+        plib.nhp_probe_seq_major_pattern.argtypes = [vp, vp, i64, i64, vp]
+        # the key gradient's layout change at the Pythia-1.4B shape: [b*h = 128, d = 128, s = 2048] -> [s, b*h, d]
+        tr_rows, tr_s = 128, 2048
+        tr_bufs = [(torch.full((tr_rows, 128, tr_s), 1.0, dtype=torch.bfloat16, device=dev),
+                    torch.empty((tr_s, tr_rows, 128), dtype=torch.bfloat16, device=dev)) for _ in range(8)]
+        kernel_bytes["seq_major_pattern_128x128x2048"] = 2 * tr_rows * 128 * tr_s * 2
         state = {"i": 0}
         stream = hp.stream_of(pat[0][1])
 
@@ -418,6 +437,9 @@ def make_workload(name, torch, dev, fresh_dy=False):
                 t.run(key, lambda: hp.check(plib.nhp_probe_copy(dst.data_ptr(), src.data_ptr(), mib << 20, 256, stream), key))
             for key, x, y, a, s in pat:
                 t.run(key, lambda: hp.check(plib.nhp_probe_causal_pattern(y.data_ptr(), x.data_ptr(), a, s, stream), key))
+            src, dst = tr_bufs[state["i"] % len(tr_bufs)]
+            t.run("seq_major_pattern_128x128x2048", lambda: hp.check(
+                plib.nhp_probe_seq_major_pattern(dst.data_ptr(), src.data_ptr(), tr_rows, tr_s, stream), "seq_major_pattern"))
 
         cfg = {"workload": name, "what": "data movement only; bytes as the kernels they stand for are priced"}
         return step, kernel_bytes, {}, "copy_1024MiB", "u8", cfg
@@ -811,6 +833,9 @@ def main():
     ap.add_argument("--fresh-dy", action="store_true",
                     help="pythia-1.4b / llama2-7b-c5: restore the upstream gradient from a pristine copy before every "
                          "in-place backward (the copy runs outside the backward's event bracket)")
+    ap.add_argument("--rope-per-tensor", action="store_true",
+                    help="pythia-1.4b / llama2-7b-c5: rotate q and k with one launch each (the reference's call style) "
+                         "instead of both in one launch")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="run one plain 1 GiB device copy first (reference for scaling rocprofv3 --pmc byte counters)")
     args = ap.parse_args()
@@ -836,7 +861,7 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    step, kernel_bytes, dense_bytes, dominant, dtype, cfg = make_workload(args.workload, torch, dev, args.fresh_dy)
+    step, kernel_bytes, dense_bytes, dominant, dtype, cfg = make_workload(args.workload, torch, dev, args.fresh_dy, args.rope_per_tensor)
     signature = cfg.get("dominant_kernel_signature", KERNEL_REVISIONS.get(args.workload))
     # Timed region: K steps; only the dominant kernel is bracketed by events
     # (every event record is one more packet between the kernels).

@@ -10,6 +10,11 @@
 //                             is read up to the 16-byte chunk that holds column q and written in
 //                             full; two waves per row, two chunks per lane for n = 2048, as the
 //                             forward kernel is launched
+//   nhp_probe_seq_major_pattern  the traffic of the transposing rotary kernel: a [rows, 128, s]
+//                             tensor (contiguous along s) is read in runs of 64 positions per
+//                             feature and written as [s, rows, 128], whole 256-byte head vectors,
+//                             through one 16-byte LDS store and load per chunk and one barrier;
+//                             the data is not transposed (what arrives where is not the point)
 
 #include "common.hpp"
 
@@ -49,6 +54,30 @@ probe_causal_pattern_kernel(uint16_t* y, const uint16_t* x, uint32_t n)
     }
 }
 
+// One workgroup per (row, 64 positions): thread t loads 16 bytes (8 positions) of features
+// (t >> 3) + 32 p, p = 0..3, stages them in LDS, and stores the tile as 64 head vectors of 256 bytes.
+__global__ void __launch_bounds__(256)
+probe_seq_major_kernel(uint16_t* out, const uint16_t* in, uint32_t rows, uint32_t s)
+{
+    __shared__ u32x4 tile[64 * 16];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t r = blockIdx.x;
+    const uint32_t s0 = blockIdx.y * 64u;
+    const uint32_t sc = tid & 7u, dr = tid >> 3;
+    u32x4 raw[4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) raw[p] = load16_stream(in + ((size_t)r * 128u + p * 32u + dr) * s + s0 + sc * 8u);
+#pragma unroll
+    for (int p = 0; p < 4; ++p) tile[(p * 256u + tid) ^ ((tid >> 4) & 7u)] = raw[p];
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t idx = i * 256u + tid;
+        const uint32_t row = idx >> 4, c = idx & 15u;
+        store16_stream(out + ((size_t)(s0 + row) * rows + r) * 128u + c * 8u, tile[idx ^ (row & 7u)]);
+    }
+}
+
 }  // namespace nhp
 
 using namespace nhp;
@@ -83,6 +112,17 @@ int nhp_probe_causal_pattern(void* y, const void* x, int64_t batches, int64_t n,
         probe_causal_pattern_kernel<2, 2><<<rows, 128, 0, st>>>(static_cast<uint16_t*>(y), static_cast<const uint16_t*>(x), 2048u);
     else
         probe_causal_pattern_kernel<2, 8><<<rows, 512, 0, st>>>(static_cast<uint16_t*>(y), static_cast<const uint16_t*>(x), 8192u);
+    return launch_result();
+}
+
+// in: [rows, 128, s], out: [s, rows, 128], 16-bit elements; s a multiple of 64.
+int nhp_probe_seq_major_pattern(void* out, const void* in, int64_t rows, int64_t s, void* stream)
+{
+    if (rows < 1 || s < 64 || s % 64 != 0 || s / 64 > 65535 || rows >= ((int64_t)1 << 24)) return NHP_ERR_SHAPE;
+    if (!out || !in) return NHP_ERR_NULL;
+    launch_prepare();
+    probe_seq_major_kernel<<<dim3((uint32_t)rows, (uint32_t)(s / 64)), 256, 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<uint16_t*>(out), static_cast<const uint16_t*>(in), (uint32_t)rows, (uint32_t)s);
     return launch_result();
 }
 

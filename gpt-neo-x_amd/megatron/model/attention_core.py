@@ -254,8 +254,8 @@ class CoreAttention(torch.nn.Module):
             bias = self.rpe(sq, sk) if self.rpe is not None else None
             # ... and is told that nobody reads the other blocks of its results, which it then does not write
             zero_block = block if block & (block - 1) == 0 else 0
-            probs = self.scale_mask_softmax(scores.view(b, np_, sq, sk), attention_mask, bias=bias, key_lengths=key_lengths,
-                                            zero_block=zero_block)
+            probs = self.scale_mask_softmax._forward_block_limited(scores.view(b, np_, sq, sk), attention_mask, bias,
+                                                                   key_lengths, zero_block)
             v = value_layer.reshape(sk, b * np_, value_layer.size(3)).transpose(0, 1)
             context = _CausalContextGemm.apply(probs.view(b * np_, sq, sk), v, block, window, merged_heads)
             if merged_heads:

@@ -181,16 +181,18 @@ class _BiasDropoutAdd(torch.autograd.Function):
         return dx, gb, grad if ctx.needs_input_grad[2] else None, None, None
 
 
-def _fresh_seed():
-    # from torch's CPU generator: no device synchronisation, repeatable under torch.manual_seed
-    return int(torch.empty((), dtype=torch.int64).random_().item())
+def _fresh_seed(device):
+    # from the device's CUDA generator, read on the host: follows torch.manual_seed, no synchronisation
+    from . import dropout_rng
+
+    return dropout_rng.next_seed(device)
 
 
 def bias_dropout_add(x: Tensor, bias: Tensor, residual: Optional[Tensor], prob: float, training: bool) -> Tensor:
     if training and prob > 0.0:
         if not prob < 1.0:
             raise ValueError(f"dropout probability has to be between 0 and 1, but got {prob}")
-        return _BiasDropoutAdd.apply(x, bias, residual, prob, _fresh_seed())
+        return _BiasDropoutAdd.apply(x, bias, residual, prob, _fresh_seed(x.device))
     return _BiasAddResidual.apply(x, bias, residual)
 
 

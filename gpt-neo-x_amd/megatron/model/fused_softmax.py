@@ -30,7 +30,7 @@ all of it widening:
 * constructor argument ``attention_dropout`` (default 0): in training mode the module returns
   ``dropout(probabilities)``; on the fused branches softmax and dropout are one kernel, with or
   without the extras above, and the keep mask (the library's counter-based generator, seeded from
-  torch's CPU generator) is regenerated in the backward instead of being stored. The caller must
+  the device's CUDA generator, see ``megatron.model.dropout_rng``) is regenerated in the backward instead of being stored. The caller must
   then not apply its own dropout.
 """
 import enum
@@ -39,6 +39,7 @@ import torch
 from torch import nn
 
 from ..fused_kernels import load_fused_kernels
+from . import dropout_rng
 
 
 class SoftmaxFusionTypes(enum.Enum):
@@ -254,10 +255,18 @@ class FusedScaleMaskSoftmax(nn.Module):
             self.register_buffer("alibi_slopes", alibi_slopes.detach().float().clone(), persistent=False)
 
     # ------------------------------------------------------------------ dispatch
-    def forward(self, input, mask, bias=None, key_lengths=None, zero_block=0):
-        """``zero_block`` (causal kernel only, ignored elsewhere): the caller reads the probabilities in square
-        blocks of that size and skips those without a visible (query, key) pair; the kernel then leaves them
-        unwritten (see ``scaled_upper_triang_masked_softmax_cuda.forward``)."""
+    def forward(self, input, mask, bias=None, key_lengths=None):
+        return self._dispatch(input, mask, bias, key_lengths, 0)
+
+    def _forward_block_limited(self, input, mask, bias, key_lengths, zero_block):
+        """For a caller that reads the probabilities (and their gradient) only in square blocks of ``zero_block``
+        rows and columns and skips the blocks without a visible (query, key) pair: the causal kernel then leaves
+        those blocks of its results UNWRITTEN (see ``scaled_upper_triang_masked_softmax_cuda.forward``); the other
+        branches ignore the hint. Not part of the module's public surface: a dense consumer of the result would
+        read uninitialised memory."""
+        return self._dispatch(input, mask, bias, key_lengths, zero_block)
+
+    def _dispatch(self, input, mask, bias, key_lengths, zero_block):
         assert input.dim() == 4  # [b, np, sq, sk]
         dropout = self.attention_dropout if self.training else 0.0
         if self.upper_triang_mask_fusion and input.size(2) != input.size(3):
@@ -306,9 +315,9 @@ class FusedScaleMaskSoftmax(nn.Module):
         return (mask.bool() | padding).contiguous()
 
     @staticmethod
-    def _dropout_seed():
-        # drawn from torch's CPU generator: repeatable under torch.manual_seed, no device synchronisation
-        return int(torch.empty((), dtype=torch.int64).random_().item())
+    def _dropout_seed(device):
+        # from the device's CUDA generator, read on the host: follows torch.manual_seed, no synchronisation
+        return dropout_rng.next_seed(device)
 
     def _slopes_on(self, device):
         slopes = self.alibi_slopes
@@ -326,7 +335,7 @@ class FusedScaleMaskSoftmax(nn.Module):
             assert key_lengths.shape == (b,), "key_lengths must be [b]"
         slopes = self._slopes_on(input.device)
         if dropout > 0.0:
-            return ScaledMaskedSoftmaxDropout.apply(input, mask, factor, dropout, self._dropout_seed(), slopes, bias,
+            return ScaledMaskedSoftmaxDropout.apply(input, mask, factor, dropout, self._dropout_seed(input.device), slopes, bias,
                                                     key_lengths)
         return ScaledMaskedSoftmax.apply(input, mask, factor, slopes, bias, key_lengths)
 
@@ -345,7 +354,7 @@ class FusedScaleMaskSoftmax(nn.Module):
         if key_lengths is not None:
             assert key_lengths.shape == (b,), "key_lengths must be [b]"
         if dropout > 0.0:
-            probs = ScaledUpperTriangMaskedSoftmaxDropout.apply(flat, factor, dropout, self._dropout_seed(),
+            probs = ScaledUpperTriangMaskedSoftmaxDropout.apply(flat, factor, dropout, self._dropout_seed(input.device),
                                                                 self.sliding_window_width, zero_block, slopes, bias,
                                                                 key_lengths)
         else:

@@ -280,8 +280,10 @@ def test_module_with_attention_dropout():
     dy = util.randn((b, np_, s, s), dtype, seed=2)
     mask = fb.causal_mask(s, DEV)
     m = FusedScaleMaskSoftmax(False, True, T.upper_triang, fb.fill_masked_with_dtype_min, True, scale, attention_dropout=p)
+    from megatron.model import dropout_rng
+
     torch.manual_seed(3)
-    seed = int(torch.empty((), dtype=torch.int64).random_().item())
+    seed = dropout_rng.next_seed()  # what the module will draw
     torch.manual_seed(3)
     xd = x.to(DEV).requires_grad_(True)
     out = m(xd, mask)
@@ -636,8 +638,10 @@ def test_module_fuses_every_extra_and_dropout_into_one_kernel(fusion, monkeypatc
     mask = fb.causal_mask(s, DEV)
     m = FusedScaleMaskSoftmax(False, True, T[fusion], fb.fill_masked_with_dtype_min, True, scale, alibi_slopes=slopes,
                               attention_dropout=p).to(DEV)
+    from megatron.model import dropout_rng
+
     torch.manual_seed(5)
-    seed = int(torch.empty((), dtype=torch.int64).random_().item())
+    seed = dropout_rng.next_seed()  # what the module will draw
     torch.manual_seed(5)
     xd, bd, ld = x.to(DEV).requires_grad_(True), rpe.to(DEV).requires_grad_(True), lengths.to(DEV)
 

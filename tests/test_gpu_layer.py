@@ -301,8 +301,10 @@ def test_bias_dropout_add_training_functions():
     x = util.randn((64, 4, 1024), dtype, seed=1, std=2.0).to(DEV).requires_grad_(True)
     bias = util.randn((1024,), dtype, seed=2).to(DEV).requires_grad_(True)
     res = util.randn((64, 4, 1024), dtype, seed=3, std=2.0).to(DEV).requires_grad_(True)
+    from megatron.model import dropout_rng
+
     torch.manual_seed(5)
-    seed = int(torch.empty((), dtype=torch.int64).random_().item())  # what the function will draw
+    seed = dropout_rng.next_seed()  # what the module will draw
     torch.manual_seed(5)
     out = bias_dropout_add_fused_train(x, bias, res, p)
     dropped = ~oracle.dropout_mask(x.numel(), p, seed).view(x.shape).to(DEV)
@@ -509,3 +511,27 @@ def test_column_sum_vs_oracle(hotpath, shape, dtype):
     again = torch.empty_like(out)
     assert L.nhp_column_sum(again.data_ptr(), xd.data_ptr(), ws.data_ptr(), rows, cols, code, None) == 0
     assert torch.equal(util.raw_bits(out), util.raw_bits(again))
+
+
+def test_dropout_seeds_follow_the_cuda_generator():
+    """dropout_rng.next_seed: restarted by torch.manual_seed, saved and restored with the CUDA generator state,
+    advancing only that generator (torch's CPU stream, hence data order, is untouched), no two alike."""
+    from megatron.model import dropout_rng as rng
+
+    torch.manual_seed(11)
+    cpu_before = torch.get_rng_state().clone()
+    a = [rng.next_seed() for _ in range(3)]
+    assert torch.equal(torch.get_rng_state(), cpu_before)
+    assert len(set(a)) == 3 and all(0 <= v < 2**63 for v in a)
+    torch.manual_seed(11)
+    assert [rng.next_seed(torch.device(DEV, 0)) for _ in range(3)] == a
+    torch.manual_seed(12)
+    assert rng.next_seed() not in a
+    state = torch.cuda.get_rng_state()
+    b = rng.next_seed()
+    torch.cuda.set_rng_state(state)
+    assert rng.next_seed() == b
+    # torch's own device random numbers and the seeds share one stream: neither repeats the other
+    torch.manual_seed(11)
+    torch.rand(4, device=DEV)
+    assert rng.next_seed() != a[0]
