@@ -422,6 +422,12 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False):
             kernel_bytes[key] = causal_bytes(a, s)[0]
             pat.append((key, x, y, a, s))
         plib.nhp_probe_seq_major_pattern.argtypes = [vp, vp, i64, i64, vp]
+        plib.nhp_probe_streams.argtypes = [vp, vp, vp, vp, i64, ctypes.c_int, ctypes.c_int, vp]
+        # 64 MiB streams (the hidden state [16384, 2048] bf16 of the layer kernels): n inputs -> one or no output
+        mixes = [("read_64MiB", 1, 0), ("write_64MiB", 0, 1), ("read2_write1_64MiB", 2, 1), ("read3_write1_64MiB", 3, 1)]
+        mix_bufs = [[torch.full((64 << 19,), 1.0, dtype=torch.bfloat16, device=dev) for _ in range(4)] for _ in range(4)]
+        for key, n_in, w in mixes:
+            kernel_bytes[key] = (n_in + w) * (64 << 20)
         # the key gradient's layout change at the Pythia-1.4B shape: [b*h = 128, d = 128, s = 2048] -> [s, b*h, d]
         tr_rows, tr_s = 128, 2048
         tr_bufs = [(torch.full((tr_rows, 128, tr_s), 1.0, dtype=torch.bfloat16, device=dev),
@@ -437,6 +443,10 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False):
                 t.run(key, lambda: hp.check(plib.nhp_probe_copy(dst.data_ptr(), src.data_ptr(), mib << 20, 256, stream), key))
             for key, x, y, a, s in pat:
                 t.run(key, lambda: hp.check(plib.nhp_probe_causal_pattern(y.data_ptr(), x.data_ptr(), a, s, stream), key))
+            bufs4 = mix_bufs[state["i"] % len(mix_bufs)]
+            for key, n_in, w in mixes:
+                t.run(key, lambda: hp.check(plib.nhp_probe_streams(bufs4[3].data_ptr(), bufs4[0].data_ptr(), bufs4[1].data_ptr(),
+                                                                   bufs4[2].data_ptr(), 64 << 20, n_in, w, stream), key))
             src, dst = tr_bufs[state["i"] % len(tr_bufs)]
             t.run("seq_major_pattern_128x128x2048", lambda: hp.check(
                 plib.nhp_probe_seq_major_pattern(dst.data_ptr(), src.data_ptr(), tr_rows, tr_s, stream), "seq_major_pattern"))

@@ -6,6 +6,10 @@
 //   nhp_probe_copy            plain streaming copy, one 16-byte chunk per thread, no loop: the
 //                             fastest copy shape measured on MI355X (more bytes per thread, grid-
 //                             stride loops and XCD-contiguous orders are all slower)
+//   nhp_probe_streams         n_in input streams (0..3) and one or no output stream of the same size, one
+//                             16-byte chunk of each per thread: the traffic mix of the element-wise and
+//                             normalisation backward kernels (two or three tensors in, one out) and of a
+//                             pure reduction (one tensor in, nothing out)
 //   nhp_probe_causal_pattern  the causal softmax forward's traffic: row q of every [n, n] matrix
 //                             is read up to the 16-byte chunk that holds column q and written in
 //                             full; two waves per row, two chunks per lane for n = 2048, as the
@@ -25,6 +29,28 @@ probe_copy_kernel(u32x4* out, const u32x4* in, size_t chunks)
 {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < chunks) store16_stream(out + i, load16_stream(in + i));
+}
+
+// out = in0 ^ in1 ^ in2 (as many as given); without an output the value is only consumed.
+template <int N_IN, bool WRITE>
+__global__ void __launch_bounds__(256)
+probe_streams_kernel(u32x4* out, const u32x4* in0, const u32x4* in1, const u32x4* in2, size_t chunks)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= chunks) return;
+    u32x4 v = u32x4{1, 2, 3, 4};
+    u32x4 a, b, c;
+    if (N_IN > 0) a = load16_stream(in0 + i);
+    if (N_IN > 1) b = load16_stream(in1 + i);
+    if (N_IN > 2) c = load16_stream(in2 + i);
+    if (N_IN > 0) v ^= a;
+    if (N_IN > 1) v ^= b;
+    if (N_IN > 2) v ^= c;
+    if (WRITE) {
+        store16_stream(out + i, v);
+    } else if ((v[0] ^ v[1] ^ v[2] ^ v[3]) == 0x9e3779b9u && v[0] == 0x12345678u) {
+        out[0] = v;  // practically never: keeps the loads alive
+    }
 }
 
 // K chunks per lane, W waves per row (chunk c of a row belongs to (k, w, l) with c = (k*W + w)*64 + l,
@@ -97,6 +123,34 @@ int nhp_probe_copy(void* out, const void* in, int64_t bytes, int threads, void* 
     probe_copy_kernel<<<(uint32_t)blocks, threads, 0, static_cast<hipStream_t>(stream)>>>(
         static_cast<u32x4*>(out), static_cast<const u32x4*>(in), (size_t)chunks);
     return launch_result();
+}
+
+// `bytes` (a multiple of 16) per stream; n_in = 0..3 inputs, with_out = 1: one output of that size, 0: none
+// (out must still point to at least 16 writable bytes).
+int nhp_probe_streams(void* out, const void* in0, const void* in1, const void* in2, int64_t bytes, int n_in,
+                      int with_out, void* stream)
+{
+    if (bytes < 0 || bytes % 16 != 0 || n_in < 0 || n_in > 3 || (n_in == 0 && !with_out)) return NHP_ERR_SHAPE;
+    if (bytes == 0) return NHP_OK;
+    if (!out || (n_in > 0 && !in0) || (n_in > 1 && !in1) || (n_in > 2 && !in2)) return NHP_ERR_NULL;
+    const int64_t chunks = bytes / 16;
+    const int64_t blocks = (chunks + 255) / 256;
+    if (!grid_fits(blocks, 256)) return NHP_ERR_SHAPE;
+    launch_prepare();
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    u32x4* o = static_cast<u32x4*>(out);
+    const u32x4* a = static_cast<const u32x4*>(in0);
+    const u32x4* b = static_cast<const u32x4*>(in1);
+    const u32x4* c = static_cast<const u32x4*>(in2);
+#define NHP_PROBE_CASE(N_, W_)                                                                           \
+    if (n_in == N_ && (with_out != 0) == W_) {                                                           \
+        probe_streams_kernel<N_, W_><<<(uint32_t)blocks, 256, 0, st>>>(o, a, b, c, (size_t)chunks);      \
+        return launch_result();                                                                          \
+    }
+    NHP_PROBE_CASE(0, true) NHP_PROBE_CASE(1, true) NHP_PROBE_CASE(2, true) NHP_PROBE_CASE(3, true)
+    NHP_PROBE_CASE(1, false) NHP_PROBE_CASE(2, false) NHP_PROBE_CASE(3, false)
+#undef NHP_PROBE_CASE
+    return NHP_ERR_SHAPE;
 }
 
 // y, x: [batches, n, n] 16-bit elements, n = 2048 (two waves of two chunks per lane) or 8192

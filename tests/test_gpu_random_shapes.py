@@ -322,3 +322,59 @@ def test_block_limited_softmax_random_shapes(hotpath, seed):
         assert int(util.raw_bits(got)[:, zeros].abs().max() if zeros.any() else 0) == 0
     util.assert_ulp_close(torch.where(written, y, want_y), want_y, 2, "y")
     util.assert_softmax_bwd_close(torch.where(written, dx, want_dx), want_dx, dy.masked_fill(masked, 0), want_y, scale, "dx")
+
+
+@pytest.mark.parametrize("seed", range(20))
+def test_softmax_extras_with_dropout_random_shapes(hotpath, seed):
+    """Both softmax kernels with a random subset of {AliBi, bias tensor, key lengths} and attention dropout, on
+    shapes around the launch-geometry boundaries, through the extension modules: probabilities within 2 ulp of the
+    oracle's composition, zeros (and uniform rows) where it has them, `dropped` exactly the oracle's dropout of the
+    stored probabilities, the causal backward with key lengths against the oracle."""
+    import scaled_masked_softmax_cuda as mext
+    import scaled_upper_triang_masked_softmax_cuda as cext
+
+    rng = random.Random(7000 + seed)
+    dtype = rng.choice(HALF)
+    b, heads = rng.randint(1, 3), rng.randint(1, 4)
+    s = boundary_int(rng, 2, 1100)
+    scale = rng.choice((1.0, 0.125, 1 / math.sqrt(128)))
+    p, sd = rng.choice((0.1, 0.5)), rng.randint(0, 1 << 40)
+    use = {k: rng.random() < 0.6 for k in "abl"}
+    print(f"extras b={b} heads={heads} s={s} {dtype} use={use} p={p}", flush=True)
+    slopes = torch.tensor(fb.alibi_slopes(max(heads, 2))[:heads], dtype=torch.float32) if use["a"] else None
+    bias = util.randn((heads, s, s), dtype, seed=seed + 2, std=1.5) if use["b"] else None
+    lengths = torch.tensor([rng.choice((0, s, rng.randint(0, s))) for _ in range(b)], dtype=torch.int32) if use["l"] else None
+    x = util.randn((b, heads, s, s), dtype, seed=seed, std=2.0)
+    dy = util.randn((b, heads, s, s), dtype, seed=seed + 1)
+    dev = lambda t: None if t is None else t.to(DEV)
+
+    # causal kernel
+    want = oracle.causal_softmax_fwd(x.view(-1, s, s), scale, None, slopes, bias, lengths)
+    dropped, y = [t.cpu() for t in cext.forward_dropout(x.view(-1, s, s).to(DEV), scale, p, sd, None, 0, dev(slopes), dev(bias),
+                                                         dev(lengths))]
+    assert torch.equal(util.raw_bits(y) == 0, util.raw_bits(want) == 0)
+    util.assert_ulp_close(y, want, 2, "causal y")
+    assert torch.equal(util.raw_bits(dropped), util.raw_bits(oracle.bias_dropout_add(y, None, None, p, sd)))
+    want_dx = oracle.causal_softmax_dropout_bwd(dy.view(-1, s, s), want, scale, p, sd, key_lengths=lengths)
+    got_dx = cext.backward_dropout(dy.view(-1, s, s).to(DEV).clone(), want.to(DEV), scale, p, sd, None, 0, dev(lengths)).cpu()
+    g = oracle.bias_dropout_add(dy.view(-1, s, s), None, None, p, sd)
+    keys = torch.arange(s)
+    masked = fb.causal_mask(s)[0, 0].expand(b * heads, s, s).clone()
+    if lengths is not None:
+        masked |= (keys.view(1, 1, s) >= lengths.clamp(0, s).view(b, 1, 1)).repeat_interleave(heads, dim=0)
+    assert int(util.raw_bits(got_dx)[masked].abs().max() if masked.any() else 0) == 0
+    util.assert_softmax_bwd_close(got_dx, want_dx, g.masked_fill(masked, 0), want, scale, "causal dx")
+
+    # padding-mask kernel (sq > 1 is a precondition of the reference's entry point)
+    if s > 1:
+        mask = util.padding_mask(b, s, s, seed=seed, lo=1) | fb.causal_mask(s)
+        if rng.random() < 0.5:
+            mask = mask[:1].contiguous()
+        want_m = oracle.masked_softmax_fwd(x, mask, scale, slopes, bias, lengths)
+        dropped_m, y_m = [t.cpu() for t in mext.forward_dropout(x.to(DEV), mask.to(DEV), scale, p, sd, dev(slopes), dev(bias),
+                                                                 dev(lengths))]
+        util.assert_ulp_close(y_m, want_m, 2, "masked y")
+        assert torch.equal(util.raw_bits(y_m) == 0, util.raw_bits(want_m) == 0)
+        assert torch.equal(util.raw_bits(dropped_m), util.raw_bits(oracle.bias_dropout_add(y_m, None, None, p, sd)))
+        plain = mext.forward(x.to(DEV), mask.to(DEV), scale, dev(slopes), dev(bias), dev(lengths)).cpu()
+        assert torch.equal(util.raw_bits(plain), util.raw_bits(y_m))
