@@ -150,7 +150,21 @@ class Timer:
         self.pairs = {}
 
 
-def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False):
+def grad_ring(torch, pristine, launches):
+    """Copies of the upstream gradient for an in-place backward, made before the timed region: launch i works on
+    copy i, so every backward sees the same pristine values instead of the shrinking results of its predecessors
+    (dx ~ 0.09 * y * dy: after a few generations the buffer holds zeros, which move measurably faster than data).
+    As many copies as `launches`, or as fit into the free device memory beside a reserve for the step's own
+    results (then the ring wraps and later launches see once-processed data)."""
+    free, _ = torch.cuda.mem_get_info(pristine.device)
+    per = pristine.numel() * pristine.element_size()
+    reserve = max(8 << 30, 3 * per)
+    count = max(1, min(launches, (free - reserve) // per))
+    ring = [pristine] + [pristine.clone() for _ in range(int(count) - 1)]
+    return ring
+
+
+def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False, launches=1, decaying_dy=False):
     import fused_rotary_positional_embedding as rope_ext
     import scaled_masked_softmax_cuda as masked_ext
     import scaled_upper_triang_masked_softmax_cuda as causal_ext
@@ -189,6 +203,10 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False):
                         "rope_bwd": rope_b}
         dense = {"causal_softmax_fwd": 2 * a * s * s * 2, "causal_softmax_bwd": 3 * a * s * s * 2}
 
+        # The backward works in place. By default every launch gets a pristine copy of the upstream gradient from a
+        # ring filled beforehand (--decaying-dy: one buffer, each launch works on its predecessor's result).
+        ring = [dy] if (decaying_dy or fresh_dy) else grad_ring(torch, dy, launches)
+        ring_state = {"i": 0}
         # --fresh-dy: the backward works in place, so without this its input shrinks from step to step
         # (dx ~ 0.09 * y * dy); with it the upstream gradient is restored from a pristine copy before
         # every backward, outside the backward's event bracket (the copy is part of the step's wall time)
@@ -211,10 +229,12 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False):
 
             t.run("rope_fwd", rope_f)
             y = t.run("causal_softmax_fwd", lambda: causal_ext.forward(x, scale))
+            g = ring[ring_state["i"] % len(ring)]
+            ring_state["i"] += 1
             if fresh_dy:
-                dy.copy_(dy0)
-            # in place on dy, as the reference does
-            t.run("causal_softmax_bwd", lambda: causal_ext.backward(dy, y, scale))
+                g.copy_(dy0)
+            # in place on the gradient buffer, as the reference does
+            t.run("causal_softmax_bwd", lambda: causal_ext.backward(g, y, scale))
             t.run("rope_bwd", rope_b)
 
         from megatron.fused_kernels import _hotpath as hp
@@ -223,8 +243,9 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False):
                "scale": "1/sqrt(%d)" % d, "bytes_convention": "causal-min (reads of the lower triangle, dense writes)",
                "dominant_kernel_signature": "softmax_bwd causal " + softmax_signature(hp.lib(), s, 2)}
         cfg["rotary_launches"] = "one per tensor" if rope_per_tensor else "q and k in one launch"
-        if fresh_dy:
-            cfg["fresh_dy"] = True
+        cfg["upstream_gradient"] = ("restored by a copy before every backward" if fresh_dy else
+                                    "one buffer, results fed back (decays to zeros)" if len(ring) == 1 else
+                                    f"ring of {len(ring)} pristine copies for {launches} launches")
         return step, kernel_bytes, dense, "causal_softmax_bwd", "bf16", cfg
 
     if name == "attn-dropout-1.4b":
@@ -363,9 +384,14 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False):
         live_chunks = int((~mask.view(b, sq, sk // 8, 8).all(dim=-1)).sum().item())
         needed = {"masked_softmax_fwd": ("GB/s_unmasked_reads_only", live_chunks * 16 * np_ + mask.numel() + n * 2)}
 
+        ring = [dy] if decaying_dy else grad_ring(torch, dy, launches)
+        ring_state = {"i": 0}
+
         def step(t):
             y = t.run("masked_softmax_fwd", lambda: masked_ext.forward(x, mask, scale))
-            t.run("masked_softmax_bwd", lambda: masked_ext.backward(dy, y, scale))
+            g = ring[ring_state["i"] % len(ring)]
+            ring_state["i"] += 1
+            t.run("masked_softmax_bwd", lambda: masked_ext.backward(g, y, scale))
 
         if name == "masked-dropout-c3":
             kernel_bytes = {"masked_softmax_dropout_fwd": 3 * n * 2 + mask.numel(), "masked_softmax_dropout_bwd": 3 * n * 2}
@@ -390,6 +416,8 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False):
         kernel_bytes["masked_softmax_fwd"] = needed["masked_softmax_fwd"][1]
         needed = {"masked_softmax_fwd": ("GB/s_dense_convention", dense_fwd)}
         cfg = {"workload": name, "scores": [b, np_, sq, sk], "mask": [b, 1, sq, sk],
+               "upstream_gradient": f"ring of {len(ring)} pristine copies for {launches} launches" if len(ring) > 1 else
+               "one buffer, results fed back (decays to zeros)",
                "bytes_convention": "forward: unmasked 8-key groups read + mask once + dense write; backward: 3x tensor",
                "dominant_kernel_signature": "softmax_bwd plain " + softmax_signature(hp.lib(), sk, 4)}
         return step, kernel_bytes, needed, "masked_softmax_bwd", "f16", cfg
@@ -408,15 +436,17 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False):
         runs = []
         for mib in (64, 128, 1024):
             nsets = max(2, 1024 // mib)  # rotate over more than the last-level cache holds
-            bufs = [(torch.full((mib << 19,), 1.0, dtype=torch.bfloat16, device=dev),
-                     torch.empty((mib << 19,), dtype=torch.bfloat16, device=dev)) for _ in range(nsets)]
+            # random data, not a constant: what the bytes hold changes the time measurably (zeros move ~4 % faster)
+            bufs = [(randn((mib << 19,), 300 + j, torch.bfloat16),
+                     torch.empty((mib << 19,), dtype=torch.bfloat16, device=dev)) for j in range(nsets)]
             key = f"copy_{mib}MiB"
             kernel_bytes[key] = 2 * (mib << 20)
             runs.append((key, bufs, mib))
         pat = []
         for a, s in ((128, 2048), (64, 8192)):
             x = torch.empty((a, s, s), dtype=torch.bfloat16, device=dev)
-            x.fill_(1.0)
+            for j in range(a):
+                x[j] = randn((s, s), 400 + j, torch.bfloat16)
             y = torch.empty_like(x)
             key = f"causal_pattern_{a}x{s}x{s}"
             kernel_bytes[key] = causal_bytes(a, s)[0]
@@ -425,13 +455,13 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False):
         plib.nhp_probe_streams.argtypes = [vp, vp, vp, vp, i64, ctypes.c_int, ctypes.c_int, vp]
         # 64 MiB streams (the hidden state [16384, 2048] bf16 of the layer kernels): n inputs -> one or no output
         mixes = [("read_64MiB", 1, 0), ("write_64MiB", 0, 1), ("read2_write1_64MiB", 2, 1), ("read3_write1_64MiB", 3, 1)]
-        mix_bufs = [[torch.full((64 << 19,), 1.0, dtype=torch.bfloat16, device=dev) for _ in range(4)] for _ in range(4)]
+        mix_bufs = [[randn((64 << 19,), 600 + 4 * i + j, torch.bfloat16) for j in range(4)] for i in range(4)]
         for key, n_in, w in mixes:
             kernel_bytes[key] = (n_in + w) * (64 << 20)
         # the key gradient's layout change at the Pythia-1.4B shape: [b*h = 128, d = 128, s = 2048] -> [s, b*h, d]
         tr_rows, tr_s = 128, 2048
-        tr_bufs = [(torch.full((tr_rows, 128, tr_s), 1.0, dtype=torch.bfloat16, device=dev),
-                    torch.empty((tr_s, tr_rows, 128), dtype=torch.bfloat16, device=dev)) for _ in range(8)]
+        tr_bufs = [(randn((tr_rows, 128, tr_s), 500 + j, torch.bfloat16),
+                    torch.empty((tr_s, tr_rows, 128), dtype=torch.bfloat16, device=dev)) for j in range(8)]
         kernel_bytes["seq_major_pattern_128x128x2048"] = 2 * tr_rows * 128 * tr_s * 2
         state = {"i": 0}
         stream = hp.stream_of(pat[0][1])
@@ -842,7 +872,11 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--fresh-dy", action="store_true",
                     help="pythia-1.4b / llama2-7b-c5: restore the upstream gradient from a pristine copy before every "
-                         "in-place backward (the copy runs outside the backward's event bracket)")
+                         "in-place backward (the copy runs outside the backward's event bracket but inside the step)")
+    ap.add_argument("--decaying-dy", action="store_true",
+                    help="pythia-1.4b / llama2-7b-c5 / masked-c3: one gradient buffer, every in-place backward works on "
+                         "the result of the one before (the data decay to zeros); default: a ring of pristine copies "
+                         "filled before the timed region, one per launch as far as device memory allows")
     ap.add_argument("--rope-per-tensor", action="store_true",
                     help="pythia-1.4b / llama2-7b-c5: rotate q and k with one launch each (the reference's call style) "
                          "instead of both in one launch")
@@ -871,7 +905,9 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    step, kernel_bytes, dense_bytes, dominant, dtype, cfg = make_workload(args.workload, torch, dev, args.fresh_dy, args.rope_per_tensor)
+    step, kernel_bytes, dense_bytes, dominant, dtype, cfg = make_workload(
+        args.workload, torch, dev, args.fresh_dy, args.rope_per_tensor,
+        launches=args.warmup + args.steps + min(args.steps, 20), decaying_dy=args.decaying_dy)
     signature = cfg.get("dominant_kernel_signature", KERNEL_REVISIONS.get(args.workload))
     # Timed region: K steps; only the dominant kernel is bracketed by events
     # (every event record is one more packet between the kernels).
