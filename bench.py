@@ -158,8 +158,9 @@ def grad_ring(torch, pristine, launches):
     results (then the ring wraps and later launches see once-processed data)."""
     free, _ = torch.cuda.mem_get_info(pristine.device)
     per = pristine.numel() * pristine.element_size()
-    reserve = max(8 << 30, 3 * per)
-    count = max(1, min(launches, (free - reserve) // per))
+    reserve = max(16 << 30, 6 * per)
+    budget = min(free - reserve, 160 << 30)
+    count = max(1, min(launches, budget // per))
     ring = [pristine] + [pristine.clone() for _ in range(int(count) - 1)]
     return ring
 
@@ -261,12 +262,14 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False, launc
         bwd_b = 2 * a * tri(s) * 2 + n * 2
         kernel_bytes = {"softmax_dropout_fwd": fwd_b, "softmax_dropout_bwd": bwd_b}
         state = {"i": 0}
+        ring = [dy] if decaying_dy else grad_ring(torch, dy, launches)
 
         def step(t):
             state["i"] += 1
             seed = state["i"]
             dropped, y = t.run("softmax_dropout_fwd", lambda: causal_ext.forward_dropout(x, scale, 0.1, seed))
-            t.run("softmax_dropout_bwd", lambda: causal_ext.backward_dropout(dy, y, scale, 0.1, seed))
+            g = ring[state["i"] % len(ring)]
+            t.run("softmax_dropout_bwd", lambda: causal_ext.backward_dropout(g, y, scale, 0.1, seed))
 
         cfg = {"workload": name, "scores": [a, s, s], "dropout": 0.1, "mask": "regenerated (Philox4x32-10), not stored",
                "bytes_convention": "lower-triangle reads, dense writes (two dense outputs in the forward)"}
@@ -310,9 +313,14 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False, launc
             fwd_b += heads * band * 2  # each head's bias triangle once; the batch re-reads it from cache
         kernel_bytes = {"causal_softmax_fwd": fwd_b, "causal_softmax_bwd": bwd_b}
 
+        ring = [dy] if decaying_dy else grad_ring(torch, dy, launches)
+        ring_state = {"i": 0}
+
         def step(t):
             y = t.run("causal_softmax_fwd", lambda: causal_ext.forward(x, scale, window, slopes, bias, None, zero_block))
-            t.run("causal_softmax_bwd", lambda: causal_ext.backward(dy, y, scale, window, None, zero_block))
+            g = ring[ring_state["i"] % len(ring)]
+            ring_state["i"] += 1
+            t.run("causal_softmax_bwd", lambda: causal_ext.backward(g, y, scale, window, None, zero_block))
 
         cfg = {"workload": name, "scores": [a, s, s], "window": window,
                "alibi_heads": None if slopes is None else heads, "bias": None if bias is None else list(bias.shape),
@@ -352,9 +360,14 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False, launc
         fwd_b = live_chunks * 16 * np_ + bias_chunks * 16 * np_ + mask.numel() + n * 2
         kernel_bytes = {"masked_softmax_ex_fwd": fwd_b, "masked_softmax_bwd": 3 * n * 2}
 
+        ring = [dy] if decaying_dy else grad_ring(torch, dy, launches)
+        ring_state = {"i": 0}
+
         def step(t):
             y = t.run("masked_softmax_ex_fwd", lambda: masked_ext.forward(x, mask, scale, slopes, bias, lengths))
-            t.run("masked_softmax_bwd", lambda: masked_ext.backward(dy, y, scale))
+            g = ring[ring_state["i"] % len(ring)]
+            ring_state["i"] += 1
+            t.run("masked_softmax_bwd", lambda: masked_ext.backward(g, y, scale))
 
         cfg = {"workload": name, "scores": [b, np_, s, s], "mask": [1, 1, s, s], "alibi_heads": np_, "bias": [np_, s, s],
                "key_lengths": lengths.tolist(),
@@ -401,7 +414,8 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False, launc
                 state["i"] += 1
                 seed = 1000 + state["i"]
                 _, y = t.run("masked_softmax_dropout_fwd", lambda: masked_ext.forward_dropout(x, mask, scale, 0.1, seed))
-                t.run("masked_softmax_dropout_bwd", lambda: masked_ext.backward_dropout(dy, y, scale, 0.1, seed))
+                g = ring[state["i"] % len(ring)]
+                t.run("masked_softmax_dropout_bwd", lambda: masked_ext.backward_dropout(g, y, scale, 0.1, seed))
 
             cfg = {"workload": name, "scores": [b, np_, sq, sk], "mask": [b, 1, sq, sk], "dropout": 0.1,
                    "bytes_convention": "dense (tensor read + mask once + probabilities and dropped probabilities written; "
@@ -874,7 +888,7 @@ def main():
                     help="pythia-1.4b / llama2-7b-c5: restore the upstream gradient from a pristine copy before every "
                          "in-place backward (the copy runs outside the backward's event bracket but inside the step)")
     ap.add_argument("--decaying-dy", action="store_true",
-                    help="pythia-1.4b / llama2-7b-c5 / masked-c3: one gradient buffer, every in-place backward works on "
+                    help="workloads with an in-place softmax backward: one gradient buffer, every in-place backward works on "
                          "the result of the one before (the data decay to zeros); default: a ring of pristine copies "
                          "filled before the timed region, one per launch as far as device memory allows")
     ap.add_argument("--rope-per-tensor", action="store_true",
