@@ -153,7 +153,8 @@ class Timer:
 def grad_ring(torch, pristine, launches):
     """Copies of the upstream gradient for an in-place backward, made before the timed region: launch i works on
     copy i, so every backward sees the same pristine values instead of the shrinking results of its predecessors
-    (dx ~ 0.09 * y * dy: after a few generations the buffer holds zeros, which move measurably faster than data).
+    (dx ~ 0.09 * y * dy: after a few generations the buffer holds zeros, which a plain copy moves ~3 % faster than
+    data). Every launch also meets another placement of its gradient buffer, so the average is one over placements.
     As many copies as `launches`, or as fit into the free device memory beside a reserve for the step's own
     results (then the ring wraps and later launches see once-processed data)."""
     free, _ = torch.cuda.mem_get_info(pristine.device)
@@ -450,7 +451,7 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False, launc
         runs = []
         for mib in (64, 128, 1024):
             nsets = max(2, 1024 // mib)  # rotate over more than the last-level cache holds
-            # random data, not a constant: what the bytes hold changes the time measurably (zeros move ~4 % faster)
+            # random data: what the bytes hold changes the time measurably (a copy of zeros is ~3 % faster)
             bufs = [(randn((mib << 19,), 300 + j, torch.bfloat16),
                      torch.empty((mib << 19,), dtype=torch.bfloat16, device=dev)) for j in range(nsets)]
             key = f"copy_{mib}MiB"
