@@ -435,9 +435,11 @@ int nhp_rope_freqs_qk_bwd(void* q_out, void* k_out, const void* q_in, const void
  * functions calls. Tensors are dense [rows, cols] (rows = all leading
  * dimensions flattened), the bias is [cols]. dtype: NHP_F16, NHP_BF16 or
  * NHP_F32, the same for every operand. Operands are widened to fp32, the
- * expression is evaluated in fp32 in the order of the reference's source and
- * rounded once to the storage type (what a fused TorchScript kernel does;
- * eager 16-bit torch rounds after every operator). Outputs may alias inputs.
+ * expression is evaluated in fp32 and rounded once to the storage type (what
+ * a fused TorchScript kernel does; eager 16-bit torch rounds after every
+ * operator). The tanh-GeLU is evaluated in an algebraically equal form without
+ * tanh (see pointwise.hip); results agree with the written formula to 2
+ * representable values or the fp32 noise of `1 + tanh`. Outputs may alias inputs.
  * ---------------------------------------------------------------------- */
 
 /*

@@ -79,6 +79,14 @@ def test_bias_gelu_edge_cases(hotpath, dtype):
     got = abi_gelu_fwd(hotpath, v.to(DEV), None).cpu()
     want = oracle.bias_gelu_fwd(v, None)
     util.assert_ulp_close(got, want, 2, "special values")
+    # the derivative stays finite (0 on the far left, 1 on the far right) wherever x * x is finite
+    big = [0.0, -0.0, 1.0, 30.0, -30.0, 1e4, -1e4] + ([] if dtype == torch.float16 else [1e13, -1e13, 1e15, -1e15, 1e18, -1e18])
+    v = torch.tensor([big + [0.5] * (16 - len(big))], dtype=dtype)
+    g = torch.full_like(v, 1.5)
+    dx, _ = abi_gelu_bwd(hotpath, g.to(DEV), v.to(DEV), None, with_dbias=False)
+    want = oracle.bias_gelu_bwd(g, v, None)
+    assert torch.isfinite(dx.cpu().float()).all()
+    util.assert_ulp_close(dx.cpu(), want, 2, "derivative at large inputs")
     y = util.randn((40, 256), dtype, seed=1, std=3.0)
     yd = y.to(DEV)
     inplace = abi_gelu_fwd(hotpath, yd, None, out=yd).cpu()
