@@ -84,6 +84,16 @@ struct Half2<NHP_F16> {
     }
 };
 
+// Two values rounded to the storage type with one packed conversion (three instructions for the pair
+// instead of four).
+template <int DT>
+__device__ __forceinline__ void round_pair(float& a, float& b)
+{
+    const uint32_t w = Half2<DT>::pack(a, b);
+    a = Half2<DT>::lo(w);
+    b = Half2<DT>::hi(w);
+}
+
 // Unpack the eight elements of a 16-byte chunk.
 template <int DT>
 __device__ __forceinline__ void unpack8(const u32x4& raw, float (&f)[8])

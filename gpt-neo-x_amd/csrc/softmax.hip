@@ -282,10 +282,17 @@ causal_fwd_kernel(uint16_t* y, const uint16_t* x, float scale, uint32_t total_ro
             float f[8];
             unpack8<DT>(raw[k], f);
             if (alibi) {
+                // -(q - k) from the chunk's first column; every rounding takes two elements at a time
+                const float d0 = (float)((int)col - (int)q);
 #pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const float dist = Half2<DT>::round(-(float)((int)q - (int)(col + j)));
-                    f[j] = Half2<DT>::round(f[j] + Half2<DT>::round(dist * slope));
+                for (int j = 0; j < 8; j += 2) {
+                    float da = d0 + (float)j, db = d0 + (float)(j + 1);
+                    round_pair<DT>(da, db);
+                    float pa = da * slope, pb = db * slope;
+                    round_pair<DT>(pa, pb);
+                    f[j] = f[j] + pa;
+                    f[j + 1] = f[j + 1] + pb;
+                    round_pair<DT>(f[j], f[j + 1]);
                 }
             }
 #pragma unroll
@@ -480,7 +487,11 @@ masked_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
                         float g[8];
                         unpack8<DT>(rbias[k], g);
 #pragma unroll
-                        for (int j = 0; j < 8; ++j) f[j] = Half2<DT>::round(f[j] + g[j]);
+                        for (int j = 0; j < 8; j += 2) {
+                            f[j] = f[j] + g[j];
+                            f[j + 1] = f[j + 1] + g[j + 1];
+                            round_pair<DT>(f[j], f[j + 1]);
+                        }
                     }
                     const uint32_t col = chunk_col<L, W>(k, w, l);
                     if (slopes != nullptr && col <= qi) {
@@ -491,9 +502,14 @@ masked_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
                         float d0 = (float)((int)col - (int)qi);
                         asm volatile("" : "+v"(d0));
 #pragma unroll
-                        for (int j = 0; j < 8; ++j) {
-                            const float dist = Half2<DT>::round(fminf(d0 + (float)j, 0.0f));
-                            f[j] = Half2<DT>::round(f[j] + Half2<DT>::round(dist * slope));
+                        for (int j = 0; j < 8; j += 2) {
+                            float da = fminf(d0 + (float)j, 0.0f), db = fminf(d0 + (float)(j + 1), 0.0f);
+                            round_pair<DT>(da, db);
+                            float pa = da * slope, pb = db * slope;
+                            round_pair<DT>(pa, pb);
+                            f[j] = f[j] + pa;
+                            f[j + 1] = f[j + 1] + pb;
+                            round_pair<DT>(f[j], f[j + 1]);
                         }
                     }
                 }
