@@ -19,6 +19,8 @@ the drop-in extension modules (which call libneox_hotpath.so):
                  the attention layer slices q and k from), rotary_pct 1.0; one launch per tensor, then q and k
                  in one launch
   rope-qk-1.4b   rotary fwd+bwd on q,k [2048,8,16,128] bf16, rotary_pct 0.25, q and k in one launch
+  rope-freqs-1.4b  the same tensors through the entry points that take the angles (fp32) and evaluate sin/cos on the
+                 device, per tensor and q and k in one launch
   rope-kgrad-1.4b  rotary bwd on a gradient [2048,8,16,128] bf16 that is contiguous along the sequence (strides
                  (1, h*d*s, d*s, s)): the layout of the key gradient behind the score GEMM's backward
   mistral-window causal softmax fwd+bwd [64,8192,8192] bf16 with a 4096-key sliding window applied by index
@@ -514,6 +516,29 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False, launc
 
         cfg = {"workload": name, "qk": [s, b, h, d], "rotary_dim": d2}
         return step, kernel_bytes, {}, "rope_qk_fwd", "bf16", cfg
+
+    if name == "rope-freqs-1.4b":
+        # the entry points that take the angles and evaluate sin/cos on the device (fused_apply_rotary_pos_emb)
+        s, b, h, d, d2 = 2048, 8, 16, 128, 32
+        sets = [rope_setup(s, b, h, d, d2, 50 + 10 * i) for i in range(4)]
+        inv_freq = 1.0 / (10000 ** (torch.arange(0, d2, 2, device=dev, dtype=torch.float32) / d2))
+        ang = torch.outer(torch.arange(s, device=dev, dtype=torch.float32), inv_freq)
+        freqs = torch.cat((ang, ang), dim=-1).view(s, 1, 1, d2).contiguous()
+        per = 2 * s * b * h * d * 2 + s * d2 * 4  # tensor in and out + the fp32 angles
+        kernel_bytes = {"rope_freqs_fwd": per, "rope_freqs_bwd": per, "rope_freqs_qk_fwd": 2 * per - s * d2 * 4,
+                        "rope_freqs_qk_bwd": 2 * per - s * d2 * 4}
+        state = {"i": 0}
+
+        def step(t):
+            q, k, dq, dk, _, _ = sets[state["i"] % len(sets)]
+            state["i"] += 1
+            t.run("rope_freqs_fwd", lambda: rope_ext.forward(q, freqs, False))
+            t.run("rope_freqs_bwd", lambda: rope_ext.backward(dq, freqs, False))
+            t.run("rope_freqs_qk_fwd", lambda: rope_ext.forward_qk(q, k, freqs, False))
+            t.run("rope_freqs_qk_bwd", lambda: rope_ext.backward_qk(dq, dk, freqs, False))
+
+        cfg = {"workload": name, "t": [s, b, h, d], "rotary_dim": d2, "angles": "fp32 [s,1,1,rotary_dim], sin/cos on the device"}
+        return step, kernel_bytes, {}, "rope_freqs_qk_fwd", "bf16", cfg
 
     if name == "mlp-gelu-1.4b":
         # through the C ABI with preallocated outputs and workspace

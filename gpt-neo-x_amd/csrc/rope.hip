@@ -11,13 +11,16 @@
 // element i with i + d2/2, i.e. a chunk with the chunk d2/(2V) lanes away in
 // the same wave; the partner's data is fetched with ds_bpermute (no memory
 // traffic). Chunks of the pass-through tail are copied by their lanes.
-//   rope_lean_kernel: cached tables, head vectors of a power-of-two number of
-//     chunks. Two chunks per thread, no loop, every load issued before the first
-//     wait: the shape a plain streaming copy runs fastest in on this GPU.
-//   rope_vec_kernel: everything else with unit feature stride (angles evaluated
-//     on the device, other head sizes). A workgroup stays on one sequence
-//     position and walks over the (batch, head) rows, re-using the cos/sin
-//     values it loaded (or computed) once.
+//   rope_lean_kernel: head vectors of a power-of-two number of chunks. Two
+//     chunks per thread, no loop, every load issued before the first wait: the
+//     shape a plain streaming copy runs fastest in on this GPU.
+//   rope_vec_kernel: other head sizes with unit feature stride. A workgroup
+//     stays on one sequence position and walks over the (batch, head) rows,
+//     re-using the cos/sin values it loaded once.
+//   When the angles are given instead of cached tables, a workgroup of either
+//   kernel first evaluates sin and cos of its position, one rotary feature per
+//   thread, into LDS (sincosf costs a few hundred instructions: evaluated per
+//   lane it made these kernels compute-bound).
 //
 // Transposing kernel, for 16-bit inputs that are contiguous along the sequence
 // instead of along the features (see rope_tr_kernel). Everything else (odd
@@ -48,6 +51,7 @@ __device__ __forceinline__ float rot(float x, float c, float r, float s)
 // ---------------------------------------------------------------------------
 template <int DT, int CS>  // CS: dtype of the cached tables
 struct CachedTables {
+    static constexpr bool kEvaluate = false;
     const void* cos;
     const void* sin;
     int64_t d2;
@@ -84,6 +88,9 @@ struct CachedTables {
 
 template <int DT>
 struct FreqTable {
+    // sin and cos are evaluated on the device: the vector kernels do it once per workgroup and
+    // position, into LDS, instead of once per lane
+    static constexpr bool kEvaluate = true;
     const float* freqs;
     int64_t d2;
     __device__ __forceinline__ void get(int64_t pos, int64_t i, float& c, float& s) const
@@ -100,6 +107,36 @@ struct FreqTable {
         for (int v = 0; v < Elt<DT>::kVec; ++v) get(pos, i + v, c[v], s[v]);
     }
 };
+
+// Rotary features a vector kernel can take: d <= 64 chunks of at most 8 elements.
+constexpr int kMaxRotary = 512;
+
+// cos/sin of position `pos` for the workgroup: with evaluated tables the first d2 threads compute one
+// value each into LDS (every thread of the workgroup has to call this: it holds a barrier).
+template <typename Tables>
+__device__ __forceinline__ void stage_tables(const Tables& tab, int64_t pos, int d2, float* tcos, float* tsin)
+{
+    if constexpr (Tables::kEvaluate) {
+        for (int i = (int)threadIdx.x; i < d2; i += (int)blockDim.x) tab.get(pos, i, tcos[i], tsin[i]);
+        __syncthreads();
+    }
+}
+
+// V consecutive values of the staged tables, or of the cached ones.
+template <int DT, typename Tables>
+__device__ __forceinline__ void table_chunk(const Tables& tab, int64_t pos, int e, const float* tcos, const float* tsin,
+                                            float (&c)[Elt<DT>::kVec], float (&s)[Elt<DT>::kVec])
+{
+    if constexpr (Tables::kEvaluate) {
+#pragma unroll
+        for (int v = 0; v < Elt<DT>::kVec; ++v) {
+            c[v] = tcos[e + v];
+            s[v] = tsin[e + v];
+        }
+    } else {
+        tab.get_vec(pos, (int64_t)e, c, s);
+    }
+}
 
 // ---------------------------------------------------------------------------
 // Vector kernel
@@ -143,6 +180,8 @@ rope_vec_kernel(RopePair pair, Tables tab, int cpr, int rot_chunks, int rpw)
     const int c = lane - rl * cpr;    // chunk within the head vector
     const bool lane_on = rl < rpw;
     const int64_t pos = blockIdx.x;
+    __shared__ float tcos[Tables::kEvaluate ? kMaxRotary : 1], tsin[Tables::kEvaluate ? kMaxRotary : 1];
+    stage_tables(tab, pos, rot_chunks * V, tcos, tsin);
 
     const int half = rot_chunks / 2;
     const bool is_rot = c < rot_chunks;
@@ -159,10 +198,10 @@ rope_vec_kernel(RopePair pair, Tables tab, int cpr, int rot_chunks, int rpw)
     if (lane_on && is_rot) {
         float unused[V];
         if (!BWD) {
-            tab.get_vec(pos, (int64_t)c * V, cv, sv);
+            table_chunk<DT>(tab, pos, c * V, tcos, tsin, cv, sv);
         } else {
-            tab.get_vec(pos, (int64_t)c * V, cv, unused);
-            tab.get_vec(pos, (int64_t)(first ? c + half : c - half) * V, unused, sv);
+            table_chunk<DT>(tab, pos, c * V, tcos, tsin, cv, unused);
+            table_chunk<DT>(tab, pos, (first ? c + half : c - half) * V, tcos, tsin, unused, sv);
         }
     }
     // forward: first half subtracts, backward: second half subtracts
@@ -218,7 +257,7 @@ rope_vec_kernel(RopePair pair, Tables tab, int cpr, int rot_chunks, int rpw)
 }
 
 // ---------------------------------------------------------------------------
-// Lean vector kernel (cached tables only)
+// Lean vector kernel
 //   grid  = (ceil(rows * CPR / 512), s, tensors), block = 256 threads
 //   thread t of workgroup x owns chunks x * 512 + t and x * 512 + 256 + t of
 //   position blockIdx.y, counted over the position's rows * CPR chunks;
@@ -253,6 +292,8 @@ rope_lean_kernel(RopeTensor ta, RopeTensor tb, Tables tab, int rot_chunks)
 
     const int lane = threadIdx.x & 63;
     const int64_t pos = blockIdx.y;
+    __shared__ float tcos[Tables::kEvaluate ? kMaxRotary : 1], tsin[Tables::kEvaluate ? kMaxRotary : 1];
+    stage_tables(tab, pos, rot_chunks * V, tcos, tsin);
     const int i0 = (int)blockIdx.x * (T * U) + (int)threadIdx.x;
     const int c = i0 & (CPR - 1);
     const int r0 = i0 >> LOG_CPR;
@@ -285,8 +326,8 @@ rope_lean_kernel(RopeTensor ta, RopeTensor tb, Tables tab, int rot_chunks)
             }
         }
         float cv[V], sv[V], unused[V];
-        tab.get_vec(pos, (int64_t)tc * V, cv, unused);
-        tab.get_vec(pos, (int64_t)ts * V, unused, sv);
+        table_chunk<DT>(tab, pos, tc * V, tcos, tsin, cv, unused);
+        table_chunk<DT>(tab, pos, ts * V, tcos, tsin, unused, sv);
         u32x4 raw[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) raw[u] = load16_stream(ip + src[u]);
@@ -571,11 +612,6 @@ static bool rope_flat(const RopeArgs& a) { return (a.is[1] == a.h * a.is[2]) && 
 
 // Launches the vector kernel for one tensor (b == nullptr) or for two tensors
 // that share s, d, d2 and the tables (q and k; their head counts may differ).
-template <typename T>
-struct IsCachedTables { static constexpr bool value = false; };
-template <int DT, int CS>
-struct IsCachedTables<CachedTables<DT, CS>> { static constexpr bool value = true; };
-
 // log2 of a power of two in 2..64, else -1
 static int log2_chunks(int64_t cpr)
 {
@@ -590,7 +626,7 @@ static int rope_launch_vec(const RopeArgs& a, const RopeArgs* b, const Tables& t
     launch_prepare();
     constexpr int V = Elt<DT>::kVec;
     const int cpr = (int)(a.d / V);
-    if constexpr (IsCachedTables<Tables>::value) {
+    {
         const int log_cpr = log2_chunks(cpr);
         const int64_t most_rows = (b && b->b * b->h > a.b * a.h) ? b->b * b->h : a.b * a.h;
         // grid.y holds the position; chunk numbers inside a position are 32-bit
