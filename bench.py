@@ -526,7 +526,9 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False, launc
         freqs = torch.cat((ang, ang), dim=-1).view(s, 1, 1, d2).contiguous()
         per = 2 * s * b * h * d * 2 + s * d2 * 4  # tensor in and out + the fp32 angles
         kernel_bytes = {"rope_freqs_fwd": per, "rope_freqs_bwd": per, "rope_freqs_qk_fwd": 2 * per - s * d2 * 4,
-                        "rope_freqs_qk_bwd": 2 * per - s * d2 * 4}
+                        "rope_freqs_qk_bwd": 2 * per - s * d2 * 4, "rope_freqs_bwd_seq_major": per}
+        # a gradient that is contiguous along the sequence, as in rope-kgrad-1.4b
+        gsm = [randn((b, h, d, s), 120 + i, torch.bfloat16).permute(3, 0, 1, 2) for i in range(4)]
         state = {"i": 0}
 
         def step(t):
@@ -536,6 +538,8 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False, launc
             t.run("rope_freqs_bwd", lambda: rope_ext.backward(dq, freqs, False))
             t.run("rope_freqs_qk_fwd", lambda: rope_ext.forward_qk(q, k, freqs, False))
             t.run("rope_freqs_qk_bwd", lambda: rope_ext.backward_qk(dq, dk, freqs, False))
+            g = gsm[state["i"] % len(gsm)]
+            t.run("rope_freqs_bwd_seq_major", lambda: rope_ext.backward(g, freqs, False))
 
         cfg = {"workload": name, "t": [s, b, h, d], "rotary_dim": d2, "angles": "fp32 [s,1,1,rotary_dim], sin/cos on the device"}
         return step, kernel_bytes, {}, "rope_freqs_qk_fwd", "bf16", cfg
