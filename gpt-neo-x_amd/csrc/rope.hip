@@ -407,113 +407,146 @@ __device__ __forceinline__ u32x4 transpose_8x8_halfwords(const u32x4& r, uint32_
 
 template <int DT, bool BWD, int P, typename Tables>
 __global__ void __launch_bounds__(256)
-rope_tr_kernel(RopeTensor T, Tables tab, int s, int cpr, int rot_chunks, int row_chunks, int64_t is_d)
+rope_tr_kernel(RopeTensor T, Tables tab, int s, int cpr, int rot_chunks, int row_chunks, int64_t is_d, int rows_per_wg)
 {
     static_assert(DT != NHP_F32, "16-bit data");
     constexpr int V = 8;
+    constexpr bool EVAL = Tables::kEvaluate;
     extern __shared__ u32x4 tile[];  // [kTrTile][row_chunks] chunks of 8 elements
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int r = blockIdx.x;
     const int s0 = blockIdx.y * kTrTile;
-    const int bi = r / T.h;
-    const int hi = r - bi * T.h;
-    const uint16_t* in = static_cast<const uint16_t*>(T.in) + bi * T.is_b + hi * T.is_h;
-    uint16_t* out = static_cast<uint16_t*>(T.out) + bi * T.os_b + hi * T.os_h;
+
+    // Angles instead of cached tables: cos and sin of the tile's positions are evaluated once, as pairs of
+    // 16-bit values behind the tile, and serve rows_per_wg (batch, head) rows; the first barrier of the
+    // row loop makes them visible.
+    uint32_t* const staged = reinterpret_cast<uint32_t*>(tile + kTrTile * row_chunks);  // [kTrTile][d2]
+    const int d2 = rot_chunks * V;
+    if constexpr (EVAL) {
+        for (int i = tid; i < kTrTile * d2; i += 256) {
+            const int row = i / d2;
+            float c = 0.0f, sn = 0.0f;
+            if (s0 + row < s) tab.get(s0 + row, i - row * d2, c, sn);
+            staged[i] = Half2<DT>::pack(c, sn);
+        }
+    }
+    // cos and sin of chunk `chunk` at tile row `row` (position pos)
+    auto fetch = [&](int row, int pos, int chunk, float (&c)[V], float (&sn)[V]) {
+        if constexpr (EVAL) {
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                const uint32_t w = staged[row * d2 + chunk * V + v];
+                c[v] = Half2<DT>::lo(w);
+                sn[v] = Half2<DT>::hi(w);
+            }
+        } else {
+            tab.get_vec(pos, (int64_t)chunk * V, c, sn);
+        }
+    };
 
     const int sc = lane & 7;  // which 8 positions of the tile
     const int f = lane >> 3;  // feature within the output chunk of this wave and pass
     const int pos8 = s0 + sc * 8;
-    u32x4 raw[P];
-#pragma unroll
-    for (int p = 0; p < P; ++p) {
-        const int c = p * 4 + wave;  // output chunk: wave-uniform
-        raw[p] = u32x4{0, 0, 0, 0};
-        if (c < cpr && pos8 < s) raw[p] = load16_stream(in + (int64_t)(c * V + f) * is_d + pos8);
-    }
     const uint32_t sel = (f & 1) ? 0x03020706u : 0x05040100u;
-#pragma unroll
-    for (int p = 0; p < P; ++p) {
-        const int c = p * 4 + wave;
-        if (c < cpr) {
-            // afterwards this lane holds the 8 features of chunk c at position sc * 8 + f of the tile
-            tile[(sc * 8 + f) * row_chunks + (c ^ sc)] = transpose_8x8_halfwords(raw[p], sel);
-        }
-    }
-    __syncthreads();
-
     const int half = rot_chunks / 2;
-    if (rot_chunks > 0 && rot_chunks < cpr) {
-        // Partial rotary dimension: rotate in place in LDS, one work item per pair of chunks (c, c + half), so
-        // that every lane that does arithmetic is busy; then copy the tile out whole head vectors at a time
-        // (storing the rotated chunks straight from these lanes, 32 bytes at a time, measured 20 % slower).
-        for (int idx = tid; idx < kTrTile * half; idx += 256) {
-            const int row = idx / half;
-            const int c = idx - row * half;
-            const int pc = c + half;
-            const int pos = s0 + row;
-            if (pos >= s) continue;
-            const int swz = row >> 3;
-            u32x4* pa = &tile[row * row_chunks + (c ^ swz)];
-            u32x4* pb = &tile[row * row_chunks + (pc ^ swz)];
-            float ca[V], sa[V], cb[V], sb[V], xa[V], xb[V], ya[V], yb[V];
-            tab.get_vec(pos, (int64_t)c * V, ca, sa);
-            tab.get_vec(pos, (int64_t)pc * V, cb, sb);
-            chunk_to_float<DT>(*pa, xa);
-            chunk_to_float<DT>(*pb, xb);
+
+    const int r_begin = blockIdx.x * rows_per_wg;
+    const int r_end = min(T.rows, r_begin + rows_per_wg);
+    for (int r = r_begin; r < r_end; ++r) {
+        if (r != r_begin) __syncthreads();  // the previous row's copy-out still reads the tile
+        const int bi = r / T.h;
+        const int hi = r - bi * T.h;
+        const uint16_t* in = static_cast<const uint16_t*>(T.in) + bi * T.is_b + hi * T.is_h;
+        uint16_t* out = static_cast<uint16_t*>(T.out) + bi * T.os_b + hi * T.os_h;
+
+        u32x4 raw[P];
 #pragma unroll
-            for (int v = 0; v < V; ++v) {
-                if (!BWD) {
-                    ya[v] = rot<DT, true>(xa[v], ca[v], xb[v], sa[v]);
-                    yb[v] = rot<DT, false>(xb[v], cb[v], xa[v], sb[v]);
-                } else {
-                    ya[v] = rot<DT, false>(xa[v], ca[v], xb[v], sb[v]);
-                    yb[v] = rot<DT, true>(xb[v], cb[v], xa[v], sa[v]);
-                }
+        for (int p = 0; p < P; ++p) {
+            const int c = p * 4 + wave;  // output chunk: wave-uniform
+            raw[p] = u32x4{0, 0, 0, 0};
+            if (c < cpr && pos8 < s) raw[p] = load16_stream(in + (int64_t)(c * V + f) * is_d + pos8);
+        }
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            const int c = p * 4 + wave;
+            if (c < cpr) {
+                // afterwards this lane holds the 8 features of chunk c at position sc * 8 + f of the tile
+                tile[(sc * 8 + f) * row_chunks + (c ^ sc)] = transpose_8x8_halfwords(raw[p], sel);
             }
-            *pa = float_to_chunk<DT>(ya);
-            *pb = float_to_chunk<DT>(yb);
         }
         __syncthreads();
-        for (int idx = tid; idx < kTrTile * cpr; idx += 256) {
-            const int row = idx / cpr;
-            const int c = idx - row * cpr;
-            const int pos = s0 + row;
-            if (pos >= s) continue;
-            store16_stream(out + (int64_t)pos * T.os_s + (int64_t)c * V, tile[row * row_chunks + (c ^ (row >> 3))]);
-        }
-        return;
-    }
 
-    for (int idx = tid; idx < kTrTile * cpr; idx += 256) {
-        const int row = idx / cpr;
-        const int c = idx - row * cpr;
-        const int pos = s0 + row;
-        if (pos >= s) continue;
-        const int swz = row >> 3;
-        const u32x4 x = tile[row * row_chunks + (c ^ swz)];
-        u32x4 res = x;
-        if (c < rot_chunks) {
-            const bool first = c < half;
-            const int pc = first ? c + half : c - half;
-            const u32x4 px = tile[row * row_chunks + (pc ^ swz)];
-            float cv[V], sv[V], unused[V], xf[V], pf[V], y[V];
-            if (!BWD) {
-                tab.get_vec(pos, (int64_t)c * V, cv, sv);
-            } else {
-                tab.get_vec(pos, (int64_t)c * V, cv, unused);
-                tab.get_vec(pos, (int64_t)pc * V, unused, sv);
-            }
-            const bool negate = BWD ? !first : first;
-            chunk_to_float<DT>(x, xf);
-            chunk_to_float<DT>(px, pf);
+        if (rot_chunks > 0 && rot_chunks < cpr) {
+            // Partial rotary dimension: rotate in place in LDS, one work item per pair of chunks (c, c + half), so
+            // that every lane that does arithmetic is busy; then copy the tile out whole head vectors at a time
+            // (storing the rotated chunks straight from these lanes, 32 bytes at a time, measured 20 % slower).
+            for (int idx = tid; idx < kTrTile * half; idx += 256) {
+                const int row = idx / half;
+                const int c = idx - row * half;
+                const int pc = c + half;
+                const int pos = s0 + row;
+                if (pos >= s) continue;
+                const int swz = row >> 3;
+                u32x4* pa = &tile[row * row_chunks + (c ^ swz)];
+                u32x4* pb = &tile[row * row_chunks + (pc ^ swz)];
+                float ca[V], sa[V], cb[V], sb[V], xa[V], xb[V], ya[V], yb[V];
+                fetch(row, pos, c, ca, sa);
+                fetch(row, pos, pc, cb, sb);
+                chunk_to_float<DT>(*pa, xa);
+                chunk_to_float<DT>(*pb, xb);
 #pragma unroll
-            for (int v = 0; v < V; ++v)
-                y[v] = negate ? rot<DT, true>(xf[v], cv[v], pf[v], sv[v]) : rot<DT>(xf[v], cv[v], pf[v], sv[v]);
-            res = float_to_chunk<DT>(y);
+                for (int v = 0; v < V; ++v) {
+                    if (!BWD) {
+                        ya[v] = rot<DT, true>(xa[v], ca[v], xb[v], sa[v]);
+                        yb[v] = rot<DT, false>(xb[v], cb[v], xa[v], sb[v]);
+                    } else {
+                        ya[v] = rot<DT, false>(xa[v], ca[v], xb[v], sb[v]);
+                        yb[v] = rot<DT, true>(xb[v], cb[v], xa[v], sa[v]);
+                    }
+                }
+                *pa = float_to_chunk<DT>(ya);
+                *pb = float_to_chunk<DT>(yb);
+            }
+            __syncthreads();
+            for (int idx = tid; idx < kTrTile * cpr; idx += 256) {
+                const int row = idx / cpr;
+                const int c = idx - row * cpr;
+                const int pos = s0 + row;
+                if (pos >= s) continue;
+                store16_stream(out + (int64_t)pos * T.os_s + (int64_t)c * V, tile[row * row_chunks + (c ^ (row >> 3))]);
+            }
+        } else {
+            for (int idx = tid; idx < kTrTile * cpr; idx += 256) {
+                const int row = idx / cpr;
+                const int c = idx - row * cpr;
+                const int pos = s0 + row;
+                if (pos >= s) continue;
+                const int swz = row >> 3;
+                const u32x4 x = tile[row * row_chunks + (c ^ swz)];
+                u32x4 res = x;
+                if (c < rot_chunks) {
+                    const bool first = c < half;
+                    const int pc = first ? c + half : c - half;
+                    const u32x4 px = tile[row * row_chunks + (pc ^ swz)];
+                    float cv[V], sv[V], unused[V], xf[V], pf[V], y[V];
+                    if (!BWD) {
+                        fetch(row, pos, c, cv, sv);
+                    } else {
+                        fetch(row, pos, c, cv, unused);
+                        fetch(row, pos, pc, unused, sv);
+                    }
+                    const bool negate = BWD ? !first : first;
+                    chunk_to_float<DT>(x, xf);
+                    chunk_to_float<DT>(px, pf);
+#pragma unroll
+                    for (int v = 0; v < V; ++v)
+                        y[v] = negate ? rot<DT, true>(xf[v], cv[v], pf[v], sv[v]) : rot<DT>(xf[v], cv[v], pf[v], sv[v]);
+                    res = float_to_chunk<DT>(y);
+                }
+                store16_stream(out + (int64_t)pos * T.os_s + (int64_t)c * V, res);
+            }
         }
-        store16_stream(out + (int64_t)pos * T.os_s + (int64_t)c * V, res);
     }
 }
 
@@ -685,10 +718,19 @@ static int tr_row_chunks(int64_t cpr)
     return n + 1;
 }
 
-template <int DT>
+// Dynamic LDS of the transposing kernel: the tile, and behind it the evaluated (cos, sin) pairs of its positions.
+template <typename Tables>
+static int64_t tr_lds_bytes(const RopeArgs& a)
+{
+    const int64_t tile = (int64_t)kTrTile * tr_row_chunks(a.d / 8) * 16;
+    return tile + (Tables::kEvaluate ? (int64_t)kTrTile * a.d2 * 4 : 0);
+}
+
+template <int DT, typename Tables>
 static bool transposed_ok(const RopeArgs& a, bool tables_ok)
 {
     if (DT == NHP_F32 || !tables_ok) return false;
+    if (tr_lds_bytes<Tables>(a) > 65536) return false;
     if (a.is[0] != 1 || a.os[3] != 1 || a.is[3] % 8 != 0) return false;
     if (a.s % 8 != 0 || a.d % 8 != 0 || a.d2 % 16 != 0 || a.d > 256) return false;
     const int64_t passes = (a.d + 31) / 32;
@@ -710,13 +752,21 @@ static int rope_launch_transposed(const RopeArgs& a, const Tables& tab)
     } else {
         const int cpr = (int)(a.d / 8);
         const int row_chunks = tr_row_chunks(cpr);
-        const uint32_t lds = (uint32_t)(kTrTile * row_chunks * 16);
-        const dim3 grid((uint32_t)(a.b * a.h), (uint32_t)((a.s + kTrTile - 1) / kTrTile));
+        const uint32_t lds = (uint32_t)tr_lds_bytes<Tables>(a);
+        const int64_t rows = a.b * a.h, tiles = (a.s + kTrTile - 1) / kTrTile;
+        // Evaluated tables are shared by several rows per workgroup, as many as leave about a thousand
+        // workgroups (at most 8); cached tables: one row per workgroup.
+        int rows_per_wg = 1;
+        if (Tables::kEvaluate) {
+            const int64_t want = rows * tiles / 1024;
+            rows_per_wg = (int)(want < 1 ? 1 : want > 8 ? 8 : want);
+        }
+        const dim3 grid((uint32_t)((rows + rows_per_wg - 1) / rows_per_wg), (uint32_t)tiles);
         const RopeTensor t = rope_tensor(a);
 #define CASE(P_)                                                                                              \
     case P_:                                                                                                  \
         rope_tr_kernel<DT, BWD, P_, Tables><<<grid, 256, lds, a.st>>>(t, tab, (int)a.s, cpr, (int)(a.d2 / 8),   \
-                                                                      row_chunks, a.is[3]);                   \
+                                                                      row_chunks, a.is[3], rows_per_wg);      \
         break;
         switch ((int)((a.d + 31) / 32)) {
             CASE(2) CASE(3) CASE(4) CASE(8)
@@ -732,7 +782,7 @@ template <int DT, bool BWD, typename Tables>
 static int rope_launch(const RopeArgs& a, const Tables& tab, bool tables_ok)
 {
     if (vector_ok<DT>(a, tables_ok)) return rope_launch_vec<DT, BWD>(a, nullptr, tab);
-    if (transposed_ok<DT>(a, tables_ok)) return rope_launch_transposed<DT, BWD>(a, tab);
+    if (transposed_ok<DT, Tables>(a, tables_ok)) return rope_launch_transposed<DT, BWD>(a, tab);
     return rope_launch_scalar<DT, BWD>(a, tab);
 }
 

@@ -283,6 +283,23 @@ def test_rope_from_angles_on_input_contiguous_along_the_sequence(hotpath, shape,
         util.assert_rope_freqs_close(got.cpu(), want, t.contiguous(), ang, backward, f"seq-major freqs bwd={backward}")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("shape", [(200, 10, 103, 64, 32), (72, 3, 1367, 64, 64), (2048, 2, 16, 128, 32)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_rope_from_angles_sequence_major_many_rows(hotpath, shape, dtype):
+    """With many (batch, head) rows a workgroup of the transposing kernel evaluates the sines and cosines of its
+    64 positions once and serves several rows with them (4, 8 and 1 rows per workgroup for these shapes, the
+    last group ragged): bit for bit the result of the contiguous layout, which takes the other vector kernel."""
+    s, b, h, d, d2 = shape
+    say(f"rope freqs sequence-major, many rows {shape} {dtype}")
+    t_d = util.randn((b, h, d, s), dtype, seed=s + h).to(DEV).permute(3, 0, 1, 2)
+    ang = (util.randn((s, 1, 1, d2), torch.float32, seed=d2 + 6) * 3.0).contiguous().to(DEV)
+    for backward in (False, True):
+        got = util.abi_rope_freqs(hotpath, t_d, ang, backward)
+        same = util.abi_rope_freqs(hotpath, t_d.contiguous(), ang, backward)
+        assert torch.equal(util.raw_bits(got), util.raw_bits(same)), backward
+
+
 @pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16", "fp32"])
 @pytest.mark.parametrize("shape", [(16, 2, 8, 8, 128, 128), (16, 2, 8, 2, 128, 32), (9, 3, 5, 1, 64, 16), (7, 2, 4, 4, 24, 8)],
                          ids=lambda s: "x".join(map(str, s)))
