@@ -19,6 +19,8 @@ the drop-in extension modules (which call libneox_hotpath.so):
                  the attention layer slices q and k from), rotary_pct 1.0; one launch per tensor, then q and k
                  in one launch
   rope-qk-1.4b   rotary fwd+bwd on q,k [2048,8,16,128] bf16, rotary_pct 0.25, q and k in one launch
+  rope-neox-20b  rotary fwd+bwd on q,k [2048,4,64,96] bf16 with 24 rotary dimensions (the reference's 20B configuration):
+                 half the rotary dimension is not a whole number of 16-byte chunks
   rope-freqs-1.4b  the same tensors through the entry points that take the angles (fp32) and evaluate sin/cos on the
                  device, per tensor and q and k in one launch
   rope-kgrad-1.4b  rotary bwd on a gradient [2048,8,16,128] bf16 that is contiguous along the sequence (strides
@@ -511,6 +513,26 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False, launc
         def step(t):
             q, k, dq, dk, cos, sin = sets[state["i"] % len(sets)]
             state["i"] += 1
+            t.run("rope_qk_fwd", lambda: rope_ext.forward_cached_qk(q, k, cos, sin, False))
+            t.run("rope_qk_bwd", lambda: rope_ext.backward_cached_qk(dq, dk, cos, sin, False))
+
+        cfg = {"workload": name, "qk": [s, b, h, d], "rotary_dim": d2}
+        return step, kernel_bytes, {}, "rope_qk_fwd", "bf16", cfg
+
+    if name == "rope-neox-20b":
+        # the 20B configuration of the reference (configs/20B.yml): 64 heads of 96, rotary_pct 0.25 -> 24 rotary
+        # dimensions, whose half (12) is not a whole number of 16-byte chunks
+        s, b, h, d, d2 = 2048, 4, 64, 96, 24
+        sets = [rope_setup(s, b, h, d, d2, 70 + 10 * i) for i in range(4)]
+        rb = rope_bytes(s, b, h, d, d2)
+        kernel_bytes = {"rope_fwd": rb, "rope_bwd": rb, "rope_qk_fwd": 2 * rb - 2 * s * d2 * 2, "rope_qk_bwd": 2 * rb - 2 * s * d2 * 2}
+        state = {"i": 0}
+
+        def step(t):
+            q, k, dq, dk, cos, sin = sets[state["i"] % len(sets)]
+            state["i"] += 1
+            t.run("rope_fwd", lambda: rope_ext.forward_cached(q, cos, sin, False))
+            t.run("rope_bwd", lambda: rope_ext.backward_cached(dq, cos, sin, False))
             t.run("rope_qk_fwd", lambda: rope_ext.forward_cached_qk(q, k, cos, sin, False))
             t.run("rope_qk_bwd", lambda: rope_ext.backward_cached_qk(dq, dk, cos, sin, False))
 

@@ -22,6 +22,10 @@
 //   thread, into LDS (sincosf costs a few hundred instructions: evaluated per
 //   lane it made these kernels compute-bound).
 //
+//   rope_gather_kernel: rotary dimensions whose half is not a whole number of
+//     chunks (24 of 96, 20 of 80) or unaligned tables; partner elements are
+//     picked from LDS one by one.
+//
 // Transposing kernel, for 16-bit inputs that are contiguous along the sequence
 // instead of along the features (see rope_tr_kernel). Everything else (odd
 // sizes, unaligned pointers, other strides) takes the scalar kernel.
@@ -253,6 +257,123 @@ rope_vec_kernel(RopePair pair, Tables tab, int cpr, int rot_chunks, int rpw)
             }
             if (on[u]) store16_stream(op + dst_off[u], res);
         }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Gather kernel: rotary dimensions whose half is not a whole number of chunks
+// (d2 = 24 of 96, 20 of 80: a quarter of the head sizes 96 and 80), or tables
+// that are not 16-byte aligned. The launch shape of rope_vec_kernel; a lane
+// still owns one chunk, but the partner of element i, i +- d2/2, may sit
+// anywhere in up to two other chunks of the head vector, so every lane puts
+// its chunk into LDS and picks its partner elements from there one by one
+// (the lanes of a head vector share a wave, whose LDS accesses execute in
+// order: a wave-level fence is all the synchronisation needed). cos and sin of
+// the position are staged in LDS by the workgroup whatever their source.
+// Requires: stride_d == 1 on both sides, d % V == 0, d <= 64 V, d2 even, every
+// other stride a multiple of V, 16-byte aligned base pointers.
+// ---------------------------------------------------------------------------
+template <int DT, bool BWD, bool FLAT, int U, typename Tables>
+__global__ void __launch_bounds__(256)
+rope_gather_kernel(RopePair pair, Tables tab, int cpr, int d2, int rpw)
+{
+    const RopeTensor& T = pair.t[blockIdx.z];
+    void* const out = T.out;
+    const void* const in = T.in;
+    const int rows = T.rows, h = T.h;
+    const int64_t is_s = T.is_s, is_b = T.is_b, is_h = T.is_h, os_s = T.os_s, os_b = T.os_b, os_h = T.os_h;
+    constexpr int V = Elt<DT>::kVec;
+    using S = typename Elt<DT>::storage;
+    __shared__ float tcos[kMaxRotary], tsin[kMaxRotary];
+    __shared__ u32x4 stage[U][256];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int rl = lane / cpr;
+    const int c = lane - rl * cpr;
+    const bool lane_on = rl < rpw;
+    const int64_t pos = blockIdx.x;
+
+    for (int i = (int)threadIdx.x; i < d2; i += 256) tab.get(pos, i, tcos[i], tsin[i]);
+    __syncthreads();
+
+    // per element of the own chunk: cos, the sine the formula takes (its own forward, the partner's
+    // backward), the sign, and where the partner sits among the staged elements of the head vector
+    const int h2 = d2 / 2;
+    const int vec0 = ((int)threadIdx.x - c) * V;  // first staged element of this lane's head vector
+    float cv[V], sv[V];
+    int src[V];
+    bool neg[V];
+    bool any = false;
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+        const int i = c * V + v;
+        const bool rot_on = lane_on && i < d2;
+        const bool first = i < h2;
+        const int pi = first ? i + h2 : i - h2;
+        cv[v] = rot_on ? tcos[i] : 0.0f;
+        sv[v] = rot_on ? tsin[BWD ? pi : i] : 0.0f;
+        neg[v] = BWD ? !first : first;
+        src[v] = rot_on ? vec0 + pi : -1;
+        any = any || rot_on;
+    }
+
+    const S* ip = static_cast<const S*>(in) + pos * is_s + (int64_t)c * V;
+    S* op = static_cast<S*>(out) + pos * os_s + (int64_t)c * V;
+    const int rows_per_step = 4 * rpw;
+    const int stride = rows_per_step * (int)gridDim.y;
+    for (int r0 = (int)blockIdx.y * rows_per_step + wave * rpw + rl; r0 < rows; r0 += stride * U) {
+        u32x4 raw[U];
+        int64_t dst_off[U];
+        bool on[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int r = r0 + u * stride;
+            on[u] = lane_on && r < rows;
+            raw[u] = u32x4{0, 0, 0, 0};
+            dst_off[u] = 0;
+            if (on[u]) {
+                if (FLAT) {
+                    raw[u] = load16_stream(ip + r * is_h);
+                    dst_off[u] = r * os_h;
+                } else {
+                    const int bi = r / h;
+                    const int hi = r - bi * h;
+                    raw[u] = load16_stream(ip + bi * is_b + hi * is_h);
+                    dst_off[u] = bi * os_b + hi * os_h;
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) stage[u][threadIdx.x] = raw[u];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            u32x4 res = raw[u];
+            if (any) {
+                const S* staged = reinterpret_cast<const S*>(&stage[u][0]);
+                float x[V], y[V];
+                chunk_to_float<DT>(raw[u], x);
+#pragma unroll
+                for (int v = 0; v < V; ++v) {
+                    y[v] = x[v];
+                    if (src[v] >= 0) {
+                        float pr;
+                        if constexpr (DT == NHP_F32)
+                            pr = staged[src[v]];
+                        else
+                            pr = Half2<DT>::from_bits(staged[src[v]]);
+                        y[v] = neg[v] ? rot<DT, true>(x[v], cv[v], pr, sv[v]) : rot<DT>(x[v], cv[v], pr, sv[v]);
+                    }
+                }
+                res = float_to_chunk<DT>(y);
+            }
+            if (on[u]) store16_stream(op + dst_off[u], res);
+        }
+        // the next iteration overwrites the staged chunks: its stores follow these loads in program order
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
     }
 }
 
@@ -623,6 +744,21 @@ static bool vector_ok(const RopeArgs& a, bool tables_ok)
     return true;
 }
 
+// What rope_gather_kernel takes: the chunked layout of the vector kernels with any even rotary
+// dimension and any table alignment.
+template <int DT>
+static bool gather_ok(const RopeArgs& a)
+{
+    constexpr int V = Elt<DT>::kVec;
+    if (a.is[3] != 1 || a.os[3] != 1) return false;
+    if (a.d % V != 0 || a.d2 % 2 != 0 || a.d2 == 0 || a.d > 64 * V) return false;
+    for (int i = 0; i < 3; ++i)
+        if (a.is[i] % V != 0 || a.os[i] % V != 0) return false;
+    if (!is_aligned16(a.in) || !is_aligned16(a.out)) return false;
+    if (!grid_fits(a.s, 256) || a.b * a.h >= ((int64_t)1 << 30)) return false;
+    return true;
+}
+
 template <int DT, bool BWD, typename Tables>
 static int rope_launch_scalar(const RopeArgs& a, const Tables& tab)
 {
@@ -709,6 +845,31 @@ static int rope_launch_vec(const RopeArgs& a, const RopeArgs* b, const Tables& t
     return launch_result();
 }
 
+// One tensor (b == nullptr) or q and k through rope_gather_kernel.
+template <int DT, bool BWD, typename Tables>
+static int rope_launch_gather(const RopeArgs& a, const RopeArgs* b, const Tables& tab)
+{
+    launch_prepare();
+    constexpr int V = Elt<DT>::kVec;
+    const int cpr = (int)(a.d / V);
+    const int rpw = 64 / cpr;
+    const int rows_per_step = 4 * rpw;
+    RopePair pair;
+    pair.t[0] = rope_tensor(a);
+    pair.t[1] = b ? rope_tensor(*b) : pair.t[0];
+    const int rows = (b && pair.t[1].rows > pair.t[0].rows) ? pair.t[1].rows : pair.t[0].rows;
+    const int64_t steps = (rows + rows_per_step - 1) / rows_per_step;
+    int64_t splits = (steps + 3) / 4;  // about four steps per workgroup, as in rope_vec_kernel
+    if (splits < 1) splits = 1;
+    if (splits > 65535) splits = 65535;
+    const dim3 grid((uint32_t)a.s, (uint32_t)splits, b ? 2u : 1u);
+    if (rope_flat(a) && (!b || rope_flat(*b)))
+        rope_gather_kernel<DT, BWD, true, 2, Tables><<<grid, 256, 0, a.st>>>(pair, tab, cpr, (int)a.d2, rpw);
+    else
+        rope_gather_kernel<DT, BWD, false, 2, Tables><<<grid, 256, 0, a.st>>>(pair, tab, cpr, (int)a.d2, rpw);
+    return launch_result();
+}
+
 // LDS row length (in chunks) of the transposing kernel: the XOR with the load chunk index needs a
 // power-of-two number of slots (at least 8), one more chunk staggers the rows over the banks.
 static int tr_row_chunks(int64_t cpr)
@@ -783,6 +944,7 @@ static int rope_launch(const RopeArgs& a, const Tables& tab, bool tables_ok)
 {
     if (vector_ok<DT>(a, tables_ok)) return rope_launch_vec<DT, BWD>(a, nullptr, tab);
     if (transposed_ok<DT, Tables>(a, tables_ok)) return rope_launch_transposed<DT, BWD>(a, tab);
+    if (gather_ok<DT>(a)) return rope_launch_gather<DT, BWD>(a, nullptr, tab);
     return rope_launch_scalar<DT, BWD>(a, tab);
 }
 
@@ -791,6 +953,9 @@ template <int DT, bool BWD, typename Tables>
 static int rope_launch_pair(const RopeArgs& q, const RopeArgs& k, const Tables& tab, bool tables_ok)
 {
     if (vector_ok<DT>(q, tables_ok) && vector_ok<DT>(k, tables_ok)) return rope_launch_vec<DT, BWD>(q, &k, tab);
+    if (!vector_ok<DT>(q, tables_ok) && !vector_ok<DT>(k, tables_ok) && gather_ok<DT>(q) && gather_ok<DT>(k) &&
+        !transposed_ok<DT, Tables>(q, tables_ok) && !transposed_ok<DT, Tables>(k, tables_ok))
+        return rope_launch_gather<DT, BWD>(q, &k, tab);
     const int rc = rope_launch<DT, BWD>(q, tab, tables_ok);
     if (rc != NHP_OK) return rc;
     return rope_launch<DT, BWD>(k, tab, tables_ok);

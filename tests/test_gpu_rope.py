@@ -46,6 +46,11 @@ SHAPES = [
     (5, 2, 33, 128, 64), (4, 1, 2, 256, 256), (7, 2, 2, 32, 16), (3, 2, 2, 24, 8), (6, 2, 3, 20, 10),
     (4, 2, 2, 16, 6), (4, 2, 2, 15, 7), (64, 4, 16, 128, 32), (33, 5, 40, 128, 128),
 ]
+# rotary dimensions whose half is not a whole number of 16-byte chunks (a quarter of the head sizes 96 and 80, the
+# rotary slice passed on its own, an odd half) take the gather kernel; several row steps per workgroup, ragged rows
+GATHER_SHAPES = [(33, 2, 5, 96, 24), (17, 3, 4, 80, 20), (16, 2, 3, 24, 24), (12, 1, 7, 512, 40), (5, 3, 47, 96, 24),
+                 (9, 2, 2, 48, 6), (6, 2, 70, 32, 12)]
+SHAPES = SHAPES + GATHER_SHAPES
 DTYPES = [torch.bfloat16, torch.float16, torch.float32]
 
 
@@ -109,7 +114,7 @@ def test_rope_matches_eager_torch(hotpath, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16", "fp32"])
-@pytest.mark.parametrize("shape", SHAPES[:8] + SHAPES[-2:], ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("shape", SHAPES[:8] + SHAPES[12:14] + GATHER_SHAPES[:3], ids=lambda s: "x".join(map(str, s)))
 def test_rope_freqs_vs_oracle(hotpath, shape, dtype):
     s, b, h, d, d2 = shape
     say(f"rope freqs {shape} {dtype}")
@@ -163,7 +168,8 @@ def test_rope_full_size_properties(hotpath):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16", "fp32"])
-@pytest.mark.parametrize("shape", [(16, 2, 8, 8, 128, 128), (16, 2, 8, 2, 128, 32), (9, 3, 5, 1, 64, 16), (7, 2, 4, 4, 24, 8)],
+@pytest.mark.parametrize("shape", [(16, 2, 8, 8, 128, 128), (16, 2, 8, 2, 128, 32), (9, 3, 5, 1, 64, 16), (7, 2, 4, 4, 24, 8),
+                                   (11, 2, 6, 2, 96, 24)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_rope_qk_single_launch_equals_two_calls(hotpath, shape, dtype):
     """q and k (k possibly with fewer heads) through nhp_rope_cached_qk_* give the
@@ -301,7 +307,8 @@ def test_rope_from_angles_sequence_major_many_rows(hotpath, shape, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16", "fp32"])
-@pytest.mark.parametrize("shape", [(16, 2, 8, 8, 128, 128), (16, 2, 8, 2, 128, 32), (9, 3, 5, 1, 64, 16), (7, 2, 4, 4, 24, 8)],
+@pytest.mark.parametrize("shape", [(16, 2, 8, 8, 128, 128), (16, 2, 8, 2, 128, 32), (9, 3, 5, 1, 64, 16), (7, 2, 4, 4, 24, 8),
+                                   (11, 2, 6, 2, 96, 24)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_rope_from_angles_qk_single_launch_equals_two_calls(hotpath, shape, dtype):
     """nhp_rope_freqs_qk_* against two nhp_rope_freqs_* calls bit for bit (same device sine and cosine), forward and
