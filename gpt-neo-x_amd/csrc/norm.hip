@@ -354,12 +354,14 @@ constexpr int bwd_waves()
     return g < W ? W : g;
 }
 
-constexpr int kBwdU = 2;      // row blocks in flight per iteration of the backward loop
-constexpr int kBwdUPair = 1;  // the same with two incoming gradients
+// Row blocks in flight per iteration of the backward loop: two, or one where the registers of a second
+// would cost a resident workgroup (two incoming gradients; rows of 10 or more KiB-segments: 93 instead of
+// 145 VGPRs at K = 2, W = 8, 146 -> 130 us at [16384, 6144]).
+constexpr int bwd_rows_in_flight(int k, int w, bool pair) { return (pair || k * w >= 10) ? 1 : 2; }
 
 // PAIR (LayerNorm only): g = dy * gamma + dy2 * gamma2, one dx for both norms, and the parameter
 // gradients of the second norm beside those of the first.
-template <int DT, int K, int W, bool RMS, bool PAIR = false, int U = (PAIR ? kBwdUPair : kBwdU)>
+template <int DT, int K, int W, bool RMS, bool PAIR = false, int U = bwd_rows_in_flight(K, W, PAIR)>
 __global__ void __launch_bounds__((bwd_waves<K, W, Elt<DT>::kVec>() * kWave))
 norm_bwd_kernel(NormBwdArgs a)
 {
@@ -670,7 +672,9 @@ struct NormPlan {
 };
 
 // (K, W) pairs that are compiled
-#define NHP_NORM_GEOMETRIES(X) X(1, 1) X(2, 1) X(4, 1) X(1, 2) X(2, 2) X(1, 4) X(2, 4) X(2, 8) X(4, 8) X(4, 16)
+#define NHP_NORM_GEOMETRIES(X) X(1, 1) X(2, 1) X(4, 1) X(1, 2) X(2, 2) X(1, 4) X(2, 4) X(2, 5) X(2, 8) X(4, 8) X(4, 16)
+// forward only: rows of 5-6 and 12 chunks per lane (hidden sizes 2560, 3072, 6144) without idle waves
+#define NHP_NORM_FWD_GEOMETRIES(X) X(2, 3) X(2, 6)
 
 // Geometry for rows of cpr chunks: a wave reads 1-2 KiB of a row (1 KiB of each of its two
 // inputs in the backward); returns false when the row does not fit.
@@ -684,15 +688,21 @@ static bool plan_norm(int64_t cpr, bool backward, NormPlan& p, bool pair_fwd = f
         ++p.logL;
     }
     const int64_t segs = (cpr + p.L - 1) / p.L;  // 16-byte chunks per lane over the whole row
-    static const int fwd_table[][2] = {{1, 1}, {2, 1}, {2, 2}, {2, 4}, {2, 8}, {4, 8}, {4, 16}};
-    static const int bwd_table[][2] = {{1, 1}, {1, 2}, {1, 4}, {2, 4}, {2, 8}, {4, 8}, {4, 16}};
+    // workgroups of 3, 5 and 6 waves measured 6-9 % faster than the next power of two at 2560, 3072 and 5120
+    // columns in the forward; in the backward only the 5 waves at 5120 columns gain (8 %)
+    static const int fwd_table[][2] = {{1, 1}, {2, 1}, {2, 2}, {2, 3}, {2, 4}, {2, 5}, {2, 6}, {2, 8}, {4, 8}, {4, 16}};
+    static const int bwd_table[][2] = {{1, 1}, {1, 2}, {1, 4}, {2, 4}, {2, 5}, {2, 8}, {4, 8}, {4, 16}};
     // a forward that writes two results: a whole row of up to 4 chunks per lane in one wave measured faster
     static const int pair_fwd_table[][2] = {{1, 1}, {2, 1}, {4, 1}, {2, 4}, {2, 8}, {4, 8}, {4, 16}};
     p.K = p.W = 0;
-    for (const auto& kw : (backward ? bwd_table : pair_fwd ? pair_fwd_table : fwd_table)) {
-        if ((int64_t)kw[0] * kw[1] >= segs) {
-            p.K = kw[0];
-            p.W = kw[1];
+    const int(*table)[2] = backward ? bwd_table : pair_fwd ? pair_fwd_table : fwd_table;
+    const size_t count = backward   ? sizeof(bwd_table) / sizeof(bwd_table[0])
+                         : pair_fwd ? sizeof(pair_fwd_table) / sizeof(pair_fwd_table[0])
+                                    : sizeof(fwd_table) / sizeof(fwd_table[0]);
+    for (size_t i = 0; i < count; ++i) {
+        if ((int64_t)table[i][0] * table[i][1] >= segs) {
+            p.K = table[i][0];
+            p.W = table[i][1];
             break;
         }
     }
@@ -723,11 +733,14 @@ static int bwd_waves_of(const NormPlan& p, int v)
 // that the second kernel has to read): 4096 waves in all, 16 per CU.
 constexpr uint32_t kNormBwdWaves = 4096;
 
-static uint32_t norm_bwd_grid(uint32_t row_blocks, bool param_grads, int waves_per_block)
+static uint32_t norm_bwd_grid(uint32_t row_blocks, bool param_grads, int waves_per_block, int in_flight)
 {
-    row_blocks = (row_blocks + kBwdU - 1) / kBwdU;  // a workgroup takes up to kBwdU row blocks per iteration
+    row_blocks = (row_blocks + in_flight - 1) / in_flight;  // a workgroup takes that many row blocks per iteration
     if (!param_grads) return row_blocks;
-    const uint32_t cap = (uint32_t)NHP_TUNED_INT("NHP_NORM_GRID", (int)(kNormBwdWaves / (uint32_t)waves_per_block));
+    // a whole number of workgroups per CU (256 CUs): a ragged last round costs more than the waves it adds
+    uint32_t cap = kNormBwdWaves / (uint32_t)waves_per_block / 256u * 256u;
+    if (cap == 0) cap = 256;
+    cap = (uint32_t)NHP_TUNED_INT("NHP_NORM_GRID", (int)cap);
     return row_blocks < cap ? row_blocks : cap;
 }
 
@@ -766,6 +779,7 @@ static int norm_fwd(void* y, float* mean, float* rstd, const void* x, const void
         return launch_result();                                                        \
     }
         NHP_NORM_GEOMETRIES(X)
+        NHP_NORM_FWD_GEOMETRIES(X)
 #undef X
         return NHP_ERR_SHAPE;
     }
@@ -782,7 +796,8 @@ static int64_t norm_workspace_bytes(int64_t rows, int64_t cols, int dtype)
     NormPlan p;
     if (rows <= 0 || cols <= 0 || cols % v != 0 || !plan_norm(cols / v, true, p)) return 0;
     const int waves = bwd_waves_of(p, v);
-    return 2 * (int64_t)norm_bwd_grid(norm_row_blocks(rows, p, waves), true, waves) * cols * (int64_t)sizeof(float);
+    // sized for one row block in flight, the variant with the most workgroups
+    return 2 * (int64_t)norm_bwd_grid(norm_row_blocks(rows, p, waves), true, waves, 1) * cols * (int64_t)sizeof(float);
 }
 
 template <int DT, bool RMS>
@@ -800,7 +815,7 @@ static int norm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, const v
         plan_norm(cols / V, true, p)) {
         const int waves = bwd_waves_of(p, V);
         const uint32_t row_blocks = norm_row_blocks(rows, p, waves);
-        const uint32_t grid = norm_bwd_grid(row_blocks, want_params, waves);
+        const uint32_t grid = norm_bwd_grid(row_blocks, want_params, waves, bwd_rows_in_flight(p.K, p.W, pair));
         const size_t part = (size_t)grid * cols;
         float* part_g = want_params ? static_cast<float*>(workspace) : nullptr;
         float* part_b = want_params ? part_g + part : nullptr;

@@ -108,7 +108,9 @@ def dx_noise(dy, gamma, factor):
 
 # rows, cols: every geometry (lanes per row 1..64, 1..16 waves per row), partial row blocks, scalar fallbacks
 SHAPES = [(5, 8), (9, 16), (33, 64), (70, 128), (300, 512), (37, 1024), (129, 2048), (21, 4096), (19, 8192),
-          (7, 16384), (3, 32768), (11, 1000), (4, 65536), (13, 2056), (1, 24)]
+          (7, 16384), (3, 32768), (11, 1000), (4, 65536), (13, 2056), (1, 24),
+          # hidden sizes that are not a power of two: workgroups of 3, 5 and 6 waves per row
+          (23, 2560), (17, 3072), (13, 5120), (11, 6144), (9, 1536)]
 
 
 @pytest.mark.parametrize("pd", ["same", "fp32"])
@@ -523,9 +525,11 @@ def test_mixed_fused_classes_match_torch(one_p):
     assert (rms.scale.grad.float() - sr.grad).norm() <= lim * sr.grad.norm()
 
 
-def test_layernorm_full_size(hotpath):
-    """The hidden state of the 1.4B configuration, [2048*8, 2048] bf16 with fp32 parameters."""
-    rows, cols = 2048 * 8, 2048
+@pytest.mark.parametrize("cols", [2048, 2560, 5120, 6144], ids=lambda c: f"hidden{c}")
+def test_layernorm_full_size(hotpath, cols):
+    """The hidden state of the 1.4B configuration, [2048*8, 2048] bf16 with fp32 parameters, and the hidden sizes of
+    the 2.8B, 12B and 20B configurations (workgroups of 3, 5 and 6 or 8 waves per row, a bounded grid that loops)."""
+    rows = 2048 * 8
     gen = torch.Generator(device=DEV).manual_seed(0)
     x = (torch.randn((rows, cols), generator=gen, device=DEV) * 2 + 0.5).bfloat16()
     dy = torch.randn((rows, cols), generator=gen, device=DEV).bfloat16()
