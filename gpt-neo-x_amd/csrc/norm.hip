@@ -678,7 +678,7 @@ struct NormPlan {
 
 // Geometry for rows of cpr chunks: a wave reads 1-2 KiB of a row (1 KiB of each of its two
 // inputs in the backward); returns false when the row does not fit.
-static bool plan_norm(int64_t cpr, bool backward, NormPlan& p, bool pair_fwd = false)
+static bool plan_norm(int64_t cpr, bool backward, NormPlan& p, bool pair = false)
 {
     if (cpr < 1) return false;
     p.L = 1;
@@ -692,13 +692,16 @@ static bool plan_norm(int64_t cpr, bool backward, NormPlan& p, bool pair_fwd = f
     // columns in the forward; in the backward only the 5 waves at 5120 columns gain (8 %)
     static const int fwd_table[][2] = {{1, 1}, {2, 1}, {2, 2}, {2, 3}, {2, 4}, {2, 5}, {2, 6}, {2, 8}, {4, 8}, {4, 16}};
     static const int bwd_table[][2] = {{1, 1}, {1, 2}, {1, 4}, {2, 4}, {2, 5}, {2, 8}, {4, 8}, {4, 16}};
+    // two incoming gradients: the 5 waves at 5120 columns lose (254 against 222 us)
+    static const int pair_bwd_table[][2] = {{1, 1}, {1, 2}, {1, 4}, {2, 4}, {2, 8}, {4, 8}, {4, 16}};
     // a forward that writes two results: a whole row of up to 4 chunks per lane in one wave measured faster
     static const int pair_fwd_table[][2] = {{1, 1}, {2, 1}, {4, 1}, {2, 4}, {2, 8}, {4, 8}, {4, 16}};
     p.K = p.W = 0;
-    const int(*table)[2] = backward ? bwd_table : pair_fwd ? pair_fwd_table : fwd_table;
-    const size_t count = backward   ? sizeof(bwd_table) / sizeof(bwd_table[0])
-                         : pair_fwd ? sizeof(pair_fwd_table) / sizeof(pair_fwd_table[0])
-                                    : sizeof(fwd_table) / sizeof(fwd_table[0]);
+    const int(*table)[2] = backward ? (pair ? pair_bwd_table : bwd_table) : pair ? pair_fwd_table : fwd_table;
+    const size_t count = backward ? (pair ? sizeof(pair_bwd_table) / sizeof(pair_bwd_table[0])
+                                          : sizeof(bwd_table) / sizeof(bwd_table[0]))
+                         : pair   ? sizeof(pair_fwd_table) / sizeof(pair_fwd_table[0])
+                                  : sizeof(fwd_table) / sizeof(fwd_table[0]);
     for (size_t i = 0; i < count; ++i) {
         if ((int64_t)table[i][0] * table[i][1] >= segs) {
             p.K = table[i][0];
@@ -790,11 +793,11 @@ static int norm_fwd(void* y, float* mean, float* rstd, const void* x, const void
     return launch_result();
 }
 
-static int64_t norm_workspace_bytes(int64_t rows, int64_t cols, int dtype)
+static int64_t norm_workspace_bytes(int64_t rows, int64_t cols, int dtype, bool pair = false)
 {
     const int v = dtype == NHP_F32 ? 4 : 8;
     NormPlan p;
-    if (rows <= 0 || cols <= 0 || cols % v != 0 || !plan_norm(cols / v, true, p)) return 0;
+    if (rows <= 0 || cols <= 0 || cols % v != 0 || !plan_norm(cols / v, true, p, pair)) return 0;
     const int waves = bwd_waves_of(p, v);
     // sized for one row block in flight, the variant with the most workgroups
     return 2 * (int64_t)norm_bwd_grid(norm_row_blocks(rows, p, waves), true, waves, 1) * cols * (int64_t)sizeof(float);
@@ -812,7 +815,7 @@ static int norm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, const v
     const bool want_params = dgamma != nullptr || dbeta != nullptr || second.dgamma2 != nullptr || second.dbeta2 != nullptr;
     if (cols % V == 0 && ptr_aligned16(dx) && ptr_aligned16(dy) && ptr_aligned16(x) && ptr_aligned16(gamma) &&
         ptr_aligned16(second.dy2) && ptr_aligned16(second.gamma2) && ptr_aligned16(workspace) &&
-        plan_norm(cols / V, true, p)) {
+        plan_norm(cols / V, true, p, pair)) {
         const int waves = bwd_waves_of(p, V);
         const uint32_t row_blocks = norm_row_blocks(rows, p, waves);
         const uint32_t grid = norm_bwd_grid(row_blocks, want_params, waves, bwd_rows_in_flight(p.K, p.W, pair));
@@ -1030,7 +1033,7 @@ int nhp_layernorm_pair_bwd(void* dx, void* dgamma1, void* dbeta1, void* dgamma2,
 int64_t nhp_layernorm_pair_bwd_workspace_bytes(int64_t rows, int64_t cols, int dtype)
 {
     if (dtype != NHP_F16 && dtype != NHP_BF16 && dtype != NHP_F32) return 0;
-    return 2 * norm_workspace_bytes(rows, cols, dtype);
+    return 2 * norm_workspace_bytes(rows, cols, dtype, true);
 }
 
 int nhp_rmsnorm_fwd(void* y, float* inv, const void* x, const void* scale, const void* offset, float eps,
