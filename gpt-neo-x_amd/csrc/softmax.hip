@@ -359,6 +359,68 @@ causal_fwd_kernel(uint16_t* y, const uint16_t* x, float scale, uint32_t total_ro
 }
 
 // ---------------------------------------------------------------------------
+// Causal forward for rows of at most 64 chunks (512 keys), plain variant. One chunk per lane
+// covers such a row, and half of the chunks are above the diagonal and never loaded: a wave
+// of the general kernel has a few hundred bytes in flight. Here a lane takes the same chunk
+// of R rows (64 / L rows apart), all loads issued first; every row is reduced on its own with
+// the arithmetic of softmax_tile, so the results are the same bits. Measured at 1 GiB of
+// scores: 53 -> 63 % of the HBM peak at 256 keys, 62 -> 65 % at 512 (eight rows in flight, or
+// four chunks per lane with masked slots skipped by the whole wave, gain nothing more).
+// ---------------------------------------------------------------------------
+constexpr int kShortRows = 4;  // rows in flight per lane (8 measured slower)
+
+template <int DT, int L, int R>
+__global__ void __launch_bounds__(256)
+causal_fwd_short_kernel(uint16_t* y, const uint16_t* x, float scale, uint32_t total_rows, uint32_t n, uint32_t window)
+{
+    constexpr int RPW = kWave / L;  // rows per wave and step
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int l = lane & (L - 1);
+    const uint32_t col = (uint32_t)l * 8u;
+    const uint32_t row0 = (blockIdx.x * 4u + (uint32_t)wave) * (uint32_t)(RPW * R) + (uint32_t)(lane / L);
+    uint32_t q = row0 % n;
+
+    u32x4 raw[R];
+    Band band[R];
+    bool ok[R];
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        const uint32_t row = row0 + (uint32_t)(i * RPW);
+        ok[i] = row < total_rows && col < n;
+        band[i] = causal_band(q, window, ok[i]);
+        raw[i] = u32x4{0, 0, 0, 0};
+        if (col < band[i].hi && col + 8 > band[i].lo) raw[i] = load16_stream(x + (size_t)row * n + col);
+        q += RPW;
+        while (q >= n) q -= n;
+    }
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        float z[8];
+        unpack8<DT>(raw[i], z);
+        float m = kNegInf;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            z[j] = (col + j < band[i].hi && col + j >= band[i].lo) ? z[j] * scale : kNegInf;
+            m = fmaxf(m, z[j]);
+        }
+        m = group_reduce<OpMax, L>(m);
+        float sum = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            z[j] = exp2_raw(fmaf(z[j] - m, kLog2e, kExpBias));
+            sum += z[j];
+        }
+        sum = group_reduce<OpSum, L>(sum);
+        const float inv = 1.0f / sum;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) z[j] *= inv;
+        // lanes of rows beyond the tensor hold m = -inf and NaNs: not stored
+        if (ok[i]) store16_stream(y + (size_t)(row0 + (uint32_t)(i * RPW)) * n + col, pack8<DT>(z));
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Padding-mask forward. A wave owns the rows (b, q) of its lanes and walks
 // over `heads_per_wave` heads with them, so the mask bytes of a row are
 // fetched and decoded once per head group.
@@ -942,8 +1004,28 @@ static int causal_fwd(void* y, const void* x, float scale, int64_t batches, int6
     const uint16_t* bp = static_cast<const uint16_t*>(bias);
     const DropoutKey dk = drop != nullptr ? *drop : DropoutKey{};
     const bool extras = slopes != nullptr || bp != nullptr;  // not dropout: its second output wants the two-wave shape
-    if (plan_row(n, extras ? kCausalFwdExtra : kCausalFwd, p, zshift != 0) && aligned16(x) && aligned16(y) && aligned16(bias) &&
-        aligned16(dropped)) {
+    const bool planned = plan_row(n, extras ? kCausalFwdExtra : kCausalFwd, p, zshift != 0) && aligned16(x) &&
+                         aligned16(y) && aligned16(bias) && aligned16(dropped);
+    // short rows, nothing but the mask, and enough rows for a thousand workgroups of 4 waves x R rows
+    if (planned && p.K == 1 && p.W == 1 && !extras && kl == nullptr && dp == nullptr && zshift == 0 &&
+        rows * p.L >= (int64_t)1024 * 256 * kShortRows) {
+        const int64_t rows_per_block = (int64_t)4 * (kWave / p.L) * kShortRows;
+        const uint32_t blocks = (uint32_t)((rows + rows_per_block - 1) / rows_per_block);
+        if (!launch_fits(blocks, 256)) return NHP_ERR_SHAPE;
+#define SHORT(L_)                                                                                      \
+    case L_:                                                                                           \
+        causal_fwd_short_kernel<DT, L_, kShortRows><<<blocks, 256, 0, st>>>(yp, xp, scale, (uint32_t)rows, \
+                                                                           (uint32_t)n, window);       \
+        break;
+        switch (p.L) {
+            SHORT(1) SHORT(2) SHORT(4) SHORT(8) SHORT(16) SHORT(32) SHORT(64)
+        default:
+            return NHP_ERR_SHAPE;
+        }
+#undef SHORT
+        return launch_result();
+    }
+    if (planned) {
 #define CALL(L_, K_, W_)                                                                   \
     {                                                                                      \
         using G = Geo<L_, K_, W_, kBlockWaves>;                                            \

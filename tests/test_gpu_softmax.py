@@ -64,6 +64,28 @@ def test_causal_forward_backward_vs_oracle(hotpath, shape, dtype):
     assert torch.equal(util.raw_bits(g.cpu()), util.raw_bits(got_dx_cpu))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("n,batches", [(512, 33), (504, 33), (256, 130), (136, 490), (64, 2050), (24, 21900), (8, 131100)],
+                         ids=lambda v: str(v))
+def test_causal_forward_short_rows_many_rows(hotpath, n, batches, dtype):
+    """Rows of at most 512 keys in tensors with enough rows take a kernel of their own (four rows in flight per lane,
+    the last workgroup ragged). Bit for bit the result of the same matrices handed over in groups small enough for
+    the general kernel, which is the one the other tests compare with the oracle; a few matrices against the oracle
+    here as well."""
+    say(f"causal short rows n={n} batches={batches} {dtype}")
+    x = util.randn((batches, n, n), dtype, seed=n, std=2.0).to(DEV)
+    scale = 0.11
+    got = util.abi_causal_fwd(hotpath, x, scale)
+    step = max(1, (1 << 20) // (4 * n * max(8, n // 8)))  # far below the row count that selects the short-row kernel
+    for b0 in list(range(0, batches, max(1, batches // 5)))[:5] + [batches - step]:
+        part = util.abi_causal_fwd(hotpath, x[b0:b0 + step].contiguous(), scale)
+        assert torch.equal(util.raw_bits(got[b0:b0 + step]), util.raw_bits(part)), b0
+    for b0 in (0, batches - 1):
+        want = oracle.causal_softmax_fwd(x[b0:b0 + 1].cpu(), scale)
+        util.assert_ulp_close(got[b0:b0 + 1].cpu(), want, 2, f"matrix {b0}")
+        assert (got[b0].cpu().float().triu(1) == 0).all()
+
+
 def test_causal_forward_in_place(hotpath):
     x = util.randn((4, 512, 512), torch.bfloat16, seed=5, std=2.0).to(DEV)
     want = util.abi_causal_fwd(hotpath, x, 0.125)
