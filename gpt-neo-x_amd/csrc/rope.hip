@@ -498,7 +498,8 @@ rope_lean_kernel(RopeTensor ta, RopeTensor tb, Tables tab, int rot_chunks)
 //            the tile is then copied out without arithmetic
 // 16-bit data only; P = ceil(d / 32) load passes, all in flight together.
 // Requires: s % 8 == 0, stride_d and the batch / head strides multiples of 8,
-// output stride_d == 1, aligned pointers and tables, d % 8 == 0, d2 % 16 == 0.
+// output stride_d == 1, aligned pointers, d % 8 == 0, and d2 % 16 == 0 with
+// aligned tables or any other even d2 (rotated element by element in LDS).
 // ---------------------------------------------------------------------------
 constexpr int kTrTile = 64;  // positions per workgroup
 
@@ -528,7 +529,7 @@ __device__ __forceinline__ u32x4 transpose_8x8_halfwords(const u32x4& r, uint32_
 
 template <int DT, bool BWD, int P, typename Tables>
 __global__ void __launch_bounds__(256)
-rope_tr_kernel(RopeTensor T, Tables tab, int s, int cpr, int rot_chunks, int row_chunks, int64_t is_d, int rows_per_wg)
+rope_tr_kernel(RopeTensor T, Tables tab, int s, int cpr, int d2, int row_chunks, int64_t is_d, int rows_per_wg)
 {
     static_assert(DT != NHP_F32, "16-bit data");
     constexpr int V = 8;
@@ -543,7 +544,7 @@ rope_tr_kernel(RopeTensor T, Tables tab, int s, int cpr, int rot_chunks, int row
     // 16-bit values behind the tile, and serve rows_per_wg (batch, head) rows; the first barrier of the
     // row loop makes them visible.
     uint32_t* const staged = reinterpret_cast<uint32_t*>(tile + kTrTile * row_chunks);  // [kTrTile][d2]
-    const int d2 = rot_chunks * V;
+    const int rot_chunks = d2 / V;  // whole rotating chunks; d2 % 16 != 0: the rotation goes element by element
     if constexpr (EVAL) {
         for (int i = tid; i < kTrTile * d2; i += 256) {
             const int row = i / d2;
@@ -563,6 +564,16 @@ rope_tr_kernel(RopeTensor T, Tables tab, int s, int cpr, int rot_chunks, int row
             }
         } else {
             tab.get_vec(pos, (int64_t)chunk * V, c, sn);
+        }
+    };
+    // the same for one element
+    auto fetch1 = [&](int row, int pos, int i, float& c, float& sn) {
+        if constexpr (EVAL) {
+            const uint32_t w = staged[row * d2 + i];
+            c = Half2<DT>::lo(w);
+            sn = Half2<DT>::hi(w);
+        } else {
+            tab.get(pos, i, c, sn);
         }
     };
 
@@ -598,7 +609,49 @@ rope_tr_kernel(RopeTensor T, Tables tab, int s, int cpr, int rot_chunks, int row
         }
         __syncthreads();
 
-        if (rot_chunks > 0 && rot_chunks < cpr) {
+        if (d2 % (2 * V) != 0) {
+            // Half the rotary dimension is not a whole number of chunks (24 of 96, 20 of 80): element i pairs with
+            // i + d2/2 somewhere in the middle of another chunk. The pairs are disjoint, so one work item rotates
+            // up to 8 of them in place, element by element, and the tile is copied out afterwards.
+            const int h2 = d2 / 2;
+            const int groups = (h2 + V - 1) / V;
+            for (int idx = tid; idx < kTrTile * groups; idx += 256) {
+                const int row = idx / groups;
+                const int i0 = (idx - row * groups) * V;
+                const int pos = s0 + row;
+                if (pos >= s) continue;
+                const int swz = row >> 3;
+                uint16_t* const base = reinterpret_cast<uint16_t*>(&tile[row * row_chunks]);
+                const int cnt = (h2 - i0 < V) ? h2 - i0 : V;
+                for (int e = 0; e < cnt; ++e) {
+                    const int ia = i0 + e, ib = ia + h2;
+                    uint16_t* const pa = base + ((((ia >> 3) ^ swz) << 3) | (ia & 7));
+                    uint16_t* const pb = base + ((((ib >> 3) ^ swz) << 3) | (ib & 7));
+                    float ca, sa, cb, sb;
+                    fetch1(row, pos, ia, ca, sa);
+                    fetch1(row, pos, ib, cb, sb);
+                    const float xa = Half2<DT>::from_bits(*pa), xb = Half2<DT>::from_bits(*pb);
+                    float ya, yb;
+                    if (!BWD) {
+                        ya = rot<DT, true>(xa, ca, xb, sa);
+                        yb = rot<DT, false>(xb, cb, xa, sb);
+                    } else {
+                        ya = rot<DT, false>(xa, ca, xb, sb);
+                        yb = rot<DT, true>(xb, cb, xa, sa);
+                    }
+                    *pa = Half2<DT>::to_bits(ya);
+                    *pb = Half2<DT>::to_bits(yb);
+                }
+            }
+            __syncthreads();
+            for (int idx = tid; idx < kTrTile * cpr; idx += 256) {
+                const int row = idx / cpr;
+                const int c = idx - row * cpr;
+                const int pos = s0 + row;
+                if (pos >= s) continue;
+                store16_stream(out + (int64_t)pos * T.os_s + (int64_t)c * V, tile[row * row_chunks + (c ^ (row >> 3))]);
+            }
+        } else if (rot_chunks > 0 && rot_chunks < cpr) {
             // Partial rotary dimension: rotate in place in LDS, one work item per pair of chunks (c, c + half), so
             // that every lane that does arithmetic is busy; then copy the tile out whole head vectors at a time
             // (storing the rotated chunks straight from these lanes, 32 bytes at a time, measured 20 % slower).
@@ -890,10 +943,12 @@ static int64_t tr_lds_bytes(const RopeArgs& a)
 template <int DT, typename Tables>
 static bool transposed_ok(const RopeArgs& a, bool tables_ok)
 {
-    if (DT == NHP_F32 || !tables_ok) return false;
+    if (DT == NHP_F32) return false;
+    // whole rotating chunks are fetched from the tables 16 bytes at a time; otherwise element by element
+    if (a.d2 % 16 == 0 ? !tables_ok : a.d2 % 2 != 0) return false;
     if (tr_lds_bytes<Tables>(a) > 65536) return false;
     if (a.is[0] != 1 || a.os[3] != 1 || a.is[3] % 8 != 0) return false;
-    if (a.s % 8 != 0 || a.d % 8 != 0 || a.d2 % 16 != 0 || a.d > 256) return false;
+    if (a.s % 8 != 0 || a.d % 8 != 0 || a.d > 256) return false;
     const int64_t passes = (a.d + 31) / 32;
     if (passes != 2 && passes != 3 && passes != 4 && passes != 8) return false;
     if (a.is[1] % 8 != 0 || a.is[2] % 8 != 0) return false;
@@ -926,7 +981,7 @@ static int rope_launch_transposed(const RopeArgs& a, const Tables& tab)
         const RopeTensor t = rope_tensor(a);
 #define CASE(P_)                                                                                              \
     case P_:                                                                                                  \
-        rope_tr_kernel<DT, BWD, P_, Tables><<<grid, 256, lds, a.st>>>(t, tab, (int)a.s, cpr, (int)(a.d2 / 8),   \
+        rope_tr_kernel<DT, BWD, P_, Tables><<<grid, 256, lds, a.st>>>(t, tab, (int)a.s, cpr, (int)a.d2,         \
                                                                       row_chunks, a.is[3], rows_per_wg);      \
         break;
         switch ((int)((a.d + 31) / 32)) {

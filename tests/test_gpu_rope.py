@@ -238,7 +238,9 @@ def test_fused_qk_function_matches_eager_apply_with_offset(dtype, offset):
 # (s, b, h, d, d2): tile boundaries (s around 64), every number of load passes, partial rotary, shapes the
 # transposing kernel refuses (s not a multiple of 8, d beyond 256) and that fall back to the scalar kernel
 SEQ_MAJOR = [(64, 2, 3, 128, 128), (200, 2, 4, 128, 32), (72, 1, 5, 64, 64), (136, 2, 2, 96, 48), (8, 2, 2, 80, 16),
-             (256, 1, 2, 256, 256), (120, 3, 2, 128, 64), (30, 2, 2, 128, 32), (16, 1, 2, 512, 64)]
+             (256, 1, 2, 256, 256), (120, 3, 2, 128, 64), (30, 2, 2, 128, 32), (16, 1, 2, 512, 64),
+             # half the rotary dimension is not a whole number of chunks: rotated element by element
+             (72, 2, 3, 96, 24), (136, 1, 4, 80, 20), (64, 2, 2, 64, 8), (40, 1, 3, 96, 96 - 8), (200, 2, 2, 128, 6)]
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
@@ -270,7 +272,8 @@ def test_rope_input_contiguous_along_the_sequence(hotpath, shape, dtype, cs_fp32
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
-@pytest.mark.parametrize("shape", [(64, 2, 3, 128, 128), (200, 2, 4, 128, 32), (136, 2, 2, 96, 48), (256, 1, 2, 256, 256)],
+@pytest.mark.parametrize("shape", [(64, 2, 3, 128, 128), (200, 2, 4, 128, 32), (136, 2, 2, 96, 48), (256, 1, 2, 256, 256),
+                                   (72, 2, 3, 96, 24), (136, 1, 4, 80, 20)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_rope_from_angles_on_input_contiguous_along_the_sequence(hotpath, shape, dtype):
     """The angles variant on the sequence-major layout takes the transposing kernel as well: same results as on
@@ -290,7 +293,7 @@ def test_rope_from_angles_on_input_contiguous_along_the_sequence(hotpath, shape,
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
-@pytest.mark.parametrize("shape", [(200, 10, 103, 64, 32), (72, 3, 1367, 64, 64), (2048, 2, 16, 128, 32)],
+@pytest.mark.parametrize("shape", [(200, 10, 103, 64, 32), (72, 3, 1367, 64, 64), (2048, 2, 16, 128, 32), (136, 5, 99, 96, 24)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_rope_from_angles_sequence_major_many_rows(hotpath, shape, dtype):
     """With many (batch, head) rows a workgroup of the transposing kernel evaluates the sines and cosines of its
