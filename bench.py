@@ -477,6 +477,12 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False, launc
         mix_bufs = [[randn((64 << 19,), 600 + 4 * i + j, torch.bfloat16) for j in range(4)] for i in range(4)]
         for key, n_in, w in mixes:
             kernel_bytes[key] = (n_in + w) * (64 << 20)
+        # the backward's stream mix at its real footprints: two inputs, the result written over the first
+        # (on the tensors of the pattern probes: 1 GiB each, and 4 and 8 GiB of the 8 GiB ones)
+        inplace = [("read2_write1_in_place_1GiB", 0, 1 << 30), ("read2_write1_in_place_4GiB", 1, 4 << 30),
+                   ("read2_write1_in_place_8GiB", 1, 8 << 30)]
+        for key, _, nbytes in inplace:
+            kernel_bytes[key] = 3 * nbytes
         # the key gradient's layout change at the Pythia-1.4B shape: [b*h = 128, d = 128, s = 2048] -> [s, b*h, d]
         tr_rows, tr_s = 128, 2048
         tr_bufs = [(randn((tr_rows, 128, tr_s), 500 + j, torch.bfloat16),
@@ -496,6 +502,10 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False, launc
             for key, n_in, w in mixes:
                 t.run(key, lambda: hp.check(plib.nhp_probe_streams(bufs4[3].data_ptr(), bufs4[0].data_ptr(), bufs4[1].data_ptr(),
                                                                    bufs4[2].data_ptr(), 64 << 20, n_in, w, stream), key))
+            for key, which, nbytes in inplace:
+                _, x, y, _, _ = pat[which]
+                t.run(key, lambda: hp.check(plib.nhp_probe_streams(y.data_ptr(), y.data_ptr(), x.data_ptr(), x.data_ptr(),
+                                                                   nbytes, 2, 1, stream), key))
             src, dst = tr_bufs[state["i"] % len(tr_bufs)]
             t.run("seq_major_pattern_128x128x2048", lambda: hp.check(
                 plib.nhp_probe_seq_major_pattern(dst.data_ptr(), src.data_ptr(), tr_rows, tr_s, stream), "seq_major_pattern"))
