@@ -913,6 +913,7 @@ static int rope_launch_gather(const RopeArgs& a, const RopeArgs* b, const Tables
     const int rows = (b && pair.t[1].rows > pair.t[0].rows) ? pair.t[1].rows : pair.t[0].rows;
     const int64_t steps = (rows + rows_per_step - 1) / rows_per_step;
     int64_t splits = (steps + 3) / 4;  // about four steps per workgroup, as in rope_vec_kernel
+    splits = NHP_TUNED_INT("NHP_ROPE_SPLITS", (int)splits);
     if (splits < 1) splits = 1;
     if (splits > 65535) splits = 65535;
     const dim3 grid((uint32_t)a.s, (uint32_t)splits, b ? 2u : 1u);
