@@ -955,6 +955,14 @@ static bool plan_row(int64_t n, RowKind kind, RowPlan& p, bool blocks = false)
             K = 4;
             W = 4;
         }
+        // Rows of 8200..16384 keys: the kernels compiled for 8 chunks per lane (half of the slots unused here,
+        // 89-100 VGPRs, 4-5 waves per SIMD) beat 4 chunks x 6 or 8 waves at full occupancy: fewer rows in
+        // flight at a time (backward 67.9 -> 72.1 % of the HBM peak at 16384 keys, 69.3 -> 71.6 % at 12288;
+        // forward 66.9 -> 69.6 % at 16384, but 71.3 -> 68.6 % at 12288).
+        if (segs > 16 && segs <= 32 && (kind == kCausalBwd || (kind == kCausalFwd && segs > 24))) {
+            K = 8;
+            W = 8;
+        }
     }
     p.W = NHP_TUNED_INT("NHP_W", W);
     p.K = NHP_TUNED_INT("NHP_K", K);
