@@ -736,13 +736,16 @@ static int bwd_waves_of(const NormPlan& p, int v)
 // that the second kernel has to read): 4096 waves in all, 16 per CU.
 constexpr uint32_t kNormBwdWaves = 4096;
 
-static uint32_t norm_bwd_grid(uint32_t row_blocks, bool param_grads, int waves_per_block, int in_flight)
+static uint32_t norm_bwd_grid(uint32_t row_blocks, bool param_grads, int waves_per_block, int in_flight,
+                              bool one_per_cu = false)
 {
     row_blocks = (row_blocks + in_flight - 1) / in_flight;  // a workgroup takes that many row blocks per iteration
     if (!param_grads) return row_blocks;
     // a whole number of workgroups per CU (256 CUs): a ragged last round costs more than the waves it adds
     uint32_t cap = kNormBwdWaves / (uint32_t)waves_per_block / 256u * 256u;
-    if (cap == 0) cap = 256;
+    // two gradients and two chunks per lane, or four chunks per lane: 158-163 VGPRs, one 8-wave workgroup per
+    // CU is resident; a second round of workgroups costs more than it brings (244 -> 225 us at [16384, 6144])
+    if (cap == 0 || one_per_cu) cap = 256;
     cap = (uint32_t)NHP_TUNED_INT("NHP_NORM_GRID", (int)cap);
     return row_blocks < cap ? row_blocks : cap;
 }
@@ -818,7 +821,8 @@ static int norm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, const v
         plan_norm(cols / V, true, p, pair)) {
         const int waves = bwd_waves_of(p, V);
         const uint32_t row_blocks = norm_row_blocks(rows, p, waves);
-        const uint32_t grid = norm_bwd_grid(row_blocks, want_params, waves, bwd_rows_in_flight(p.K, p.W, pair));
+        const uint32_t grid = norm_bwd_grid(row_blocks, want_params, waves, bwd_rows_in_flight(p.K, p.W, pair),
+                                            (pair && p.K >= 2) || p.K >= 4);
         const size_t part = (size_t)grid * cols;
         float* part_g = want_params ? static_cast<float*>(workspace) : nullptr;
         float* part_b = want_params ? part_g + part : nullptr;
