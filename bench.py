@@ -34,7 +34,7 @@ the drop-in extension modules (which call libneox_hotpath.so):
   masked-dropout-c3  padding-masked softmax + attention dropout (p = 0.1) in one kernel, fwd+bwd on the masked-c3 tensors
   rpe-bias-1.4b  causal softmax fwd+bwd [128,2048,2048] bf16 with a bias tensor [16,2048,2048] added in the kernel
 
-  hbm-probes     kernels that only move data (libneox_probe.so): a plain streaming copy of 64 MiB, 128 MiB and
+  hbm-probes     kernels that only move data (bench_probes/libneox_probe.so): a plain streaming copy of 64 MiB, 128 MiB and
                  1 GiB tensors, and the causal softmax forward's access pattern (lower-triangle reads, dense writes)
                  at [128,2048,2048] and [64,8192,8192], and the layout change of the transposing rotary kernel
                  ([128,128,2048] contiguous along the sequence -> [2048,128,128]): what the memory system gives for
@@ -446,7 +446,7 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False, launc
 
         from megatron.fused_kernels import _hotpath as hp
 
-        path = os.path.join(os.path.dirname(hp.LIB_PATH), "libneox_probe.so")
+        path = os.path.join(ROOT, "bench_probes", "libneox_probe.so")
         plib = ctypes.CDLL(path)
         vp, i64 = ctypes.c_void_p, ctypes.c_int64
         plib.nhp_probe_copy.argtypes = [vp, vp, i64, ctypes.c_int, vp]

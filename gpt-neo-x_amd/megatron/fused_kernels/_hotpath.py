@@ -138,6 +138,17 @@ def dtype_code(t, what):
         raise RuntimeError(f"{what}: unsupported dtype {t.dtype}") from None
 
 
+def forward_scale(scale_factor, t, narrow):
+    """The factor the forward softmax kernels multiply the scores by. With ``narrow`` it is first rounded
+    to t's dtype (round to nearest even) and widened again, which is what the reference's CUDA dispatchers do
+    by taking ``const input_t scale`` (scaled_upper_triang_masked_softmax.h:368, scaled_masked_softmax.h:358);
+    without it the fp32 value is used as it is, like the reference's backward and its torch branch."""
+    value = float(scale_factor)
+    if narrow:
+        value = float(torch.tensor(value, dtype=torch.float32).to(t.dtype))
+    return value
+
+
 def require_gpu(t, what):
     if t.device.type != "cuda":
         raise RuntimeError(f"{what}: expected a tensor on the GPU, got device {t.device}")

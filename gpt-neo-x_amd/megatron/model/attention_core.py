@@ -32,15 +32,7 @@ import math
 import torch
 
 from .fused_softmax import FusedScaleMaskSoftmax, SoftmaxFusionTypes
-
-
-def get_fusion_type(neox_args):
-    """``SoftmaxFusionTypes`` member for the two fusion flags (megatron/model/utils.py:356-362)."""
-    if neox_args.scaled_upper_triang_masked_softmax_fusion:
-        return SoftmaxFusionTypes.upper_triang
-    if neox_args.scaled_masked_softmax_fusion:
-        return SoftmaxFusionTypes.general
-    return SoftmaxFusionTypes.none
+from .utils import get_fusion_type  # noqa: F401  (also reachable from here, where its caller lives)
 
 
 class _ContextGemm(torch.autograd.Function):

@@ -11,7 +11,10 @@ in the reference (megatron/model/transformer.py:592-593, megatron/model/fused_bi
 * ``torch.cuda.get_rng_state`` / ``set_rng_state`` save and restore it (checkpointing, activation
   recomputation), and a region that swaps the CUDA generator state, like the reference's
   ``mpu.get_cuda_rng_tracker().fork()``, gives the fused dropout inside it that region's stream;
-* the CPU generator, hence data order, is not affected.
+* the CPU generator, hence data order, is not affected;
+* a seed is a host value fixed at call time, so it cannot be drawn while a HIP graph is being
+  captured (every replay would reuse the one mask): ``next_seed`` raises there. Capture the
+  kernels through their extension functions with a seed of the caller's choosing instead.
 
 Which elements are dropped for a given seed is the library's own definition (see
 ``nhp_bias_dropout_add`` in include/neox_hotpath.h), not torch's.
@@ -34,6 +37,9 @@ def next_seed(device=None):
     index = torch.cuda.current_device() if device is None else torch.device(device).index
     if index is None:
         index = torch.cuda.current_device()
+    if torch.cuda.is_current_stream_capturing():
+        raise RuntimeError("dropout seeds are drawn on the host and cannot be drawn during graph capture: "
+                           "every replay would repeat one mask; pass an explicit seed to the extension functions")
     gen = torch.cuda.default_generators[index]
     seed, offset = gen.initial_seed(), gen.get_offset()
     gen.set_offset(offset + 4)  # Philox offsets advance in steps of four

@@ -5,10 +5,19 @@ Surface of GPT-NeoX's ``megatron/model/fused_bias_dropout.py``:
 ``bias_dropout_add_fused_train`` (:45-50), ``bias_dropout_add_fused_inference``
 (:53-58). The whole expression ``residual + dropout(x + bias)`` is one gfx950
 kernel, evaluated in fp32 and rounded once. With dropout active the keep mask
-comes from the library's own counter-based generator (Philox4x32-10, seeded
-per call from torch's CPU generator, so ``torch.manual_seed`` makes runs
-repeatable); it is regenerated in the backward instead of being stored. Which
-elements are dropped therefore differs from what torch's dropout would pick.
+comes from the library's own counter-based generator (Philox4x32-10 over the
+flat element index, seeded per call from the device's CUDA generator, see
+``dropout_rng``, so ``torch.manual_seed`` makes runs repeatable); it is
+regenerated in the backward instead of being stored.
+
+Parity of the keep mask is unpinned against the reference by construction: WHICH
+elements are dropped for a given seed is this library's definition, not that of
+``torch.nn.functional.dropout`` (which the reference calls and which draws its
+mask from torch's generator stream in its own order). Everything else is pinned:
+the generator against the published Philox4x32-10 known answers, the keep rate,
+and ``keep ? (x + bias) / (1 - p) : 0`` plus the residual bit for bit given the mask.
+With dropout off (``training=False`` or ``prob=0``, the setting of every
+configuration the reference ships) results do not depend on any of this.
 """
 from typing import Optional
 

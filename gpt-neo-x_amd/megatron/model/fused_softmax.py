@@ -13,8 +13,9 @@ all of it widening:
 
 * key lengths above 2048 stay on the fused branch (rows up to 65536 keys are
   held in registers, longer ones stream);
-* ``scale`` reaches the forward kernel in fp32 (the reference's CUDA dispatcher
-  narrows it to the input dtype first);
+* ``scale`` reaches the forward kernel in fp32 by default, as on the reference's torch
+  branch; the reference's CUDA dispatcher narrows it to the input dtype first, which the
+  constructor argument ``narrow_forward_scale=True`` reproduces;
 * two optional constructor arguments let the kernels do by index what their
   caller otherwise does with tensors: ``sliding_window_width`` (causal kernel; the
   reference's causal kernel never looks at the mask, so a sliding window is lost on
@@ -62,25 +63,27 @@ class ScaledUpperTriangMaskedSoftmax(torch.autograd.Function):
     """
 
     @staticmethod
-    def forward(ctx, inputs, scale, window=None, alibi_slopes=None, bias=None, key_lengths=None, zero_block=0):
+    def forward(ctx, inputs, scale, window=None, alibi_slopes=None, bias=None, key_lengths=None, zero_block=0,
+                narrow_scale=False):
         import scaled_upper_triang_masked_softmax_cuda as kernels
 
         factor = _scale_tensor(scale)
-        out = kernels.forward(inputs, factor[0], window, alibi_slopes, bias, key_lengths, zero_block)
+        out = kernels.forward(inputs, factor[0], window, alibi_slopes, bias, key_lengths, zero_block,
+                              narrow_scale=narrow_scale)
         ctx.window = window
         ctx.zero_block = zero_block
-        ctx.key_lengths = key_lengths
         ctx.bias_shape = None if bias is None else tuple(bias.shape)
-        ctx.save_for_backward(out, factor)
+        _save(ctx, out, factor, key_lengths)
         return out
 
     @staticmethod
     def backward(ctx, output_grads):
         import scaled_upper_triang_masked_softmax_cuda as kernels
 
-        out, factor = ctx.saved_tensors
-        # in place on output_grads, like the reference kernel
-        grad = kernels.backward(output_grads, out, factor[0], ctx.window, ctx.key_lengths, ctx.zero_block)
+        out, factor, key_lengths = _saved(ctx)
+        # in place on output_grads, like the reference kernel; the backward's factor is never narrowed
+        # (scaled_upper_triang_masked_softmax.h:467 takes acc_t)
+        grad = kernels.backward(output_grads, out, factor[0], ctx.window, key_lengths, ctx.zero_block)
         grad_bias = None
         if ctx.bias_shape is not None and ctx.needs_input_grad[4]:
             # the bias is shared by the batch: its gradient is the batch sum of the score gradient
@@ -90,7 +93,23 @@ class ScaledUpperTriangMaskedSoftmax(torch.autograd.Function):
                 sq = ctx.bias_shape[-2]
                 full = torch.where(_written_blocks(sq, ctx.zero_block, ctx.window, grad.device), grad, torch.zeros_like(grad))
             grad_bias = _batch_sum(full, ctx.bias_shape)
-        return grad, None, None, None, grad_bias, None, None
+        return grad, None, None, None, grad_bias, None, None, None
+
+
+def _save(ctx, out, factor, key_lengths):
+    """Keeps the tensors of a forward for its backward; the key lengths go through save_for_backward as well, so
+    that autograd notices an in-place change between the two."""
+    ctx.has_key_lengths = key_lengths is not None
+    if ctx.has_key_lengths:
+        ctx.save_for_backward(out, factor, key_lengths)
+    else:
+        ctx.save_for_backward(out, factor)
+
+
+def _saved(ctx):
+    if ctx.has_key_lengths:
+        return ctx.saved_tensors
+    return ctx.saved_tensors + (None,)
 
 
 def _written_blocks(seq_len, zero_block, window, device):
@@ -117,25 +136,24 @@ class ScaledUpperTriangMaskedSoftmaxDropout(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, inputs, scale, prob, seed, window=None, zero_block=0, alibi_slopes=None, bias=None,
-                key_lengths=None):
+                key_lengths=None, narrow_scale=False):
         import scaled_upper_triang_masked_softmax_cuda as kernels
 
         factor = _scale_tensor(scale)
         dropped, probs = kernels.forward_dropout(inputs, factor[0], prob, seed, window, zero_block, alibi_slopes, bias,
-                                                 key_lengths)
+                                                 key_lengths, narrow_scale=narrow_scale)
         ctx.conf = (float(prob), int(seed), window, zero_block)
-        ctx.key_lengths = key_lengths
         ctx.bias_shape = None if bias is None else tuple(bias.shape)
-        ctx.save_for_backward(probs, factor)
+        _save(ctx, probs, factor, key_lengths)
         return dropped
 
     @staticmethod
     def backward(ctx, output_grads):
         import scaled_upper_triang_masked_softmax_cuda as kernels
 
-        probs, factor = ctx.saved_tensors
+        probs, factor, key_lengths = _saved(ctx)
         prob, seed, window, zero_block = ctx.conf
-        grad = kernels.backward_dropout(output_grads, probs, factor[0], prob, seed, window, zero_block, ctx.key_lengths)
+        grad = kernels.backward_dropout(output_grads, probs, factor[0], prob, seed, window, zero_block, key_lengths)
         grad_bias = None
         if ctx.bias_shape is not None and ctx.needs_input_grad[7]:
             full = grad
@@ -143,7 +161,7 @@ class ScaledUpperTriangMaskedSoftmaxDropout(torch.autograd.Function):
                 sq = ctx.bias_shape[-2]
                 full = torch.where(_written_blocks(sq, zero_block, window, grad.device), grad, torch.zeros_like(grad))
             grad_bias = _batch_sum(full, ctx.bias_shape)
-        return grad, None, None, None, None, None, None, grad_bias, None
+        return grad, None, None, None, None, None, None, grad_bias, None, None
 
 
 class ScaledMaskedSoftmax(torch.autograd.Function):
@@ -154,11 +172,11 @@ class ScaledMaskedSoftmax(torch.autograd.Function):
     ``scaled_masked_softmax_cuda.forward``); the reference signature is ``apply(inputs, mask, scale)``."""
 
     @staticmethod
-    def forward(ctx, inputs, mask, scale, alibi_slopes=None, bias=None, key_lengths=None):
+    def forward(ctx, inputs, mask, scale, alibi_slopes=None, bias=None, key_lengths=None, narrow_scale=False):
         import scaled_masked_softmax_cuda as kernels
 
         factor = _scale_tensor(scale)
-        out = kernels.forward(inputs, mask, factor[0], alibi_slopes, bias, key_lengths)
+        out = kernels.forward(inputs, mask, factor[0], alibi_slopes, bias, key_lengths, narrow_scale=narrow_scale)
         ctx.bias_shape = None if bias is None else tuple(bias.shape)
         ctx.save_for_backward(out, factor)
         return out
@@ -172,7 +190,7 @@ class ScaledMaskedSoftmax(torch.autograd.Function):
         grad_bias = None
         if ctx.bias_shape is not None and ctx.needs_input_grad[4]:
             grad_bias = _batch_sum(grad, ctx.bias_shape)
-        return grad, None, None, None, grad_bias, None
+        return grad, None, None, None, grad_bias, None, None
 
 
 class ScaledMaskedSoftmaxDropout(torch.autograd.Function):
@@ -180,11 +198,13 @@ class ScaledMaskedSoftmaxDropout(torch.autograd.Function):
     No counterpart in the reference, which runs ``torch.nn.Dropout`` on the probabilities."""
 
     @staticmethod
-    def forward(ctx, inputs, mask, scale, prob, seed, alibi_slopes=None, bias=None, key_lengths=None):
+    def forward(ctx, inputs, mask, scale, prob, seed, alibi_slopes=None, bias=None, key_lengths=None,
+                narrow_scale=False):
         import scaled_masked_softmax_cuda as kernels
 
         factor = _scale_tensor(scale)
-        dropped, probs = kernels.forward_dropout(inputs, mask, factor[0], prob, seed, alibi_slopes, bias, key_lengths)
+        dropped, probs = kernels.forward_dropout(inputs, mask, factor[0], prob, seed, alibi_slopes, bias, key_lengths,
+                                                 narrow_scale=narrow_scale)
         ctx.conf = (float(prob), int(seed))
         ctx.bias_shape = None if bias is None else tuple(bias.shape)
         ctx.save_for_backward(probs, factor)
@@ -200,7 +220,7 @@ class ScaledMaskedSoftmaxDropout(torch.autograd.Function):
         grad_bias = None
         if ctx.bias_shape is not None and ctx.needs_input_grad[6]:
             grad_bias = _batch_sum(grad, ctx.bias_shape)
-        return grad, None, None, None, None, None, grad_bias, None
+        return grad, None, None, None, None, None, grad_bias, None, None
 
 
 class FusedScaleMaskSoftmax(nn.Module):
@@ -225,10 +245,18 @@ class FusedScaleMaskSoftmax(nn.Module):
             probabilities in training mode; fused with the softmax on both
             kernel branches, whatever else (bias, AliBi, key lengths) is in play.
             The caller must not apply its own dropout.
+        narrow_forward_scale: (extension, default False) on the fused branches round ``scale`` to
+            the scores' dtype before the forward kernel uses it, which is what the reference's CUDA
+            forward dispatchers do (``const input_t scale``, scaled_upper_triang_masked_softmax.h:368,
+            scaled_masked_softmax.h:358). True: results follow the reference's fused kernels.
+            False: the fp32 value is used, results follow the reference's torch branch
+            (``forward_torch_softmax``). The backward uses the fp32 value either way, as the
+            reference's does. Only factors that are not representable in the scores' dtype differ:
+            1/sqrt(128) becomes 0.08837890625 (1.07e-4 smaller), 1/sqrt(64) is exact.
     """
 
     def __init__(self, input_in_fp16, input_in_bf16, fusion_type, mask_func, softmax_in_fp32, scale,
-                 sliding_window_width=None, alibi_slopes=None, attention_dropout=0.0):
+                 sliding_window_width=None, alibi_slopes=None, attention_dropout=0.0, narrow_forward_scale=False):
         super().__init__()
         assert isinstance(fusion_type, SoftmaxFusionTypes), f"Invalid fusion type {fusion_type}"
         assert scale is None or softmax_in_fp32, "softmax should be in fp32 when scaled"
@@ -248,6 +276,7 @@ class FusedScaleMaskSoftmax(nn.Module):
 
         assert 0.0 <= attention_dropout < 1.0, "attention_dropout must be in [0, 1)"
         self.attention_dropout = float(attention_dropout)
+        self.narrow_forward_scale = bool(narrow_forward_scale)
         self.sliding_window_width = sliding_window_width
         if alibi_slopes is None:
             self.alibi_slopes = None
@@ -336,8 +365,8 @@ class FusedScaleMaskSoftmax(nn.Module):
         slopes = self._slopes_on(input.device)
         if dropout > 0.0:
             return ScaledMaskedSoftmaxDropout.apply(input, mask, factor, dropout, self._dropout_seed(input.device), slopes, bias,
-                                                    key_lengths)
-        return ScaledMaskedSoftmax.apply(input, mask, factor, slopes, bias, key_lengths)
+                                                    key_lengths, self.narrow_forward_scale)
+        return ScaledMaskedSoftmax.apply(input, mask, factor, slopes, bias, key_lengths, self.narrow_forward_scale)
 
     def forward_fused_softmax(self, input, mask, bias=None, key_lengths=None, zero_block=0, dropout=0.0):
         b, np, sq, sk = input.size()
@@ -356,10 +385,10 @@ class FusedScaleMaskSoftmax(nn.Module):
         if dropout > 0.0:
             probs = ScaledUpperTriangMaskedSoftmaxDropout.apply(flat, factor, dropout, self._dropout_seed(input.device),
                                                                 self.sliding_window_width, zero_block, slopes, bias,
-                                                                key_lengths)
+                                                                key_lengths, self.narrow_forward_scale)
         else:
             probs = ScaledUpperTriangMaskedSoftmax.apply(flat, factor, self.sliding_window_width, slopes, bias,
-                                                         key_lengths, zero_block)
+                                                         key_lengths, zero_block, self.narrow_forward_scale)
         return probs.view(b, np, sq, sk)
 
     def forward_torch_softmax(self, input, mask, bias=None, key_lengths=None):

@@ -11,6 +11,13 @@ fused RMSNorm variants do; the Python ``RMSNorm`` of the reference, run eagerly
 on 16-bit tensors, rounds after every operator and so differs by a few units in
 the last place.
 
+The reference's three classes are plain torch modules that work on any device.
+That is kept: a tensor that is not on a GPU is normalised with the reference's
+own torch expressions (``torch.nn.functional.layer_norm``, the statements of
+``RMSNorm.forward`` and ``ScaleNorm.forward``), with autograd's backward. A
+tensor on a GPU always takes the kernels; if the library is missing that raises,
+there is no torch path for GPU tensors.
+
 Not provided: the Transformer Engine classes (``te_rmsnorm``, ``te_layernorm``).
 """
 import numbers
@@ -200,6 +207,9 @@ class LayerNorm(torch.nn.Module):
     def forward(self, input):
         if input.size(-1) != self.normalized_shape[0]:
             raise RuntimeError(f"LayerNorm: expected last dimension {self.normalized_shape[0]}, got {input.size(-1)}")
+        if input.device.type != "cuda":
+            # off the GPU: torch's own LayerNorm, which is the reference's class (megatron/model/norms.py:16)
+            return torch.nn.functional.layer_norm(input, self.normalized_shape, self.weight, self.bias, self.eps)
         return _LayerNormFunction.apply(input, self.weight, self.bias, self.eps)
 
     def extra_repr(self):
@@ -287,8 +297,28 @@ class RMSNorm(torch.nn.Module):
     def forward(self, x):
         if x.size(-1) != self.d:
             raise RuntimeError(f"RMSNorm: expected last dimension {self.d}, got {x.size(-1)}")
+        if x.device.type != "cuda":
+            return self._forward_torch(x)
         return _RMSNormFunction.apply(x, self.scale, self.offset, self.eps, 0 if self.fused_eps else 1,
                                       self.partial_size)
+
+    def _forward_torch(self, x):
+        """Off the GPU: the statements of the reference's ``RMSNorm.forward`` (megatron/model/norms.py:82-107), every
+        operator in the tensors' own dtypes; with ``fused_eps`` the fused definition evaluated in fp32."""
+        if self.fused_eps:
+            stat = x.float() if self.partial_size is None else x.float()[..., : self.partial_size]
+            inv = torch.rsqrt(stat.pow(2).mean(dim=-1, keepdim=True) + self.eps)
+            out = x.float() * inv * self.scale.float()
+            if self.offset is not None:
+                out = out + self.offset.float()
+            return out.to(x.dtype)
+        measured = x if self.partial_size is None else x[..., : self.partial_size]
+        count = self.d if self.partial_size is None else self.partial_size
+        rms = measured.norm(2, dim=-1, keepdim=True) * count ** -0.5
+        normed = x / (rms + self.eps)
+        if self.offset is not None:
+            return self.scale * normed + self.offset  # the reference does not cast back on this branch
+        return (self.scale * normed).to(x.dtype)
 
 
 class ScaleNorm(torch.nn.Module):
@@ -303,6 +333,9 @@ class ScaleNorm(torch.nn.Module):
         self.eps = eps
 
     def forward(self, x):
+        if x.device.type != "cuda":
+            # off the GPU: the reference's two statements (megatron/model/norms.py:116-119)
+            return x / torch.norm(x, dim=-1, keepdim=True).clamp(min=self.eps) * self.g
         g = self.g if self.g.dtype in (x.dtype, torch.float32) else self.g.to(x.dtype)
         return _RMSNormFunction.apply(x, g.expand(x.size(-1)), None, self.eps, 2, None)
 

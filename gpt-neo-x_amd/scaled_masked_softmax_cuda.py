@@ -62,7 +62,7 @@ def _extras(x, alibi_slopes, bias, key_lengths, name):
     return keep, slopes_ptr, bias_ptr, lengths_ptr
 
 
-def forward(input, mask, scale_factor, alibi_slopes=None, bias=None, key_lengths=None):
+def forward(input, mask, scale_factor, alibi_slopes=None, bias=None, key_lengths=None, *, narrow_scale=False):
     """softmax(where(mask == 1, -10000, scale * input)) over the last dim.
 
     input: [b, np, sq, sk] fp16/bf16; mask: [1 or b, 1, sq, sk], one byte per
@@ -74,6 +74,9 @@ def forward(input, mask, scale_factor, alibi_slopes=None, bias=None, key_lengths
     alibi_slopes: fp32 [np] on the GPU, needs sq == sk: ``scores + alibi_matrix`` in the storage dtype;
     bias: [np, sq, sk] (or [1, np, sq, sk]) in the input's dtype: ``scores += bias`` in the storage dtype;
     key_lengths: integer [b] on the GPU: keys at or beyond a batch entry's length count as masked.
+    narrow_scale (keyword only): round ``scale_factor`` to the input's dtype before use, as the reference's CUDA
+    forward does (scaled_masked_softmax.h:358 takes ``const input_t scale``); by default the fp32 value is used,
+    as in the reference's backward and torch branch.
     """
     name = "scaled_masked_softmax_cuda.forward"
     x, m = _checked_forward_args(input, mask, name)
@@ -82,8 +85,8 @@ def forward(input, mask, scale_factor, alibi_slopes=None, bias=None, key_lengths
     y = torch.empty_like(x)
     with _hp.device_guard(x):
         rc = _hp.lib().nhp_masked_softmax_ex_fwd(
-            y.data_ptr(), x.data_ptr(), m.data_ptr(), float(scale_factor), b, np_, sq, sk, m.size(0),
-            slopes_ptr, bias_ptr, lengths_ptr, _hp.dtype_code(x, "forward"), _hp.stream_of(x))
+            y.data_ptr(), x.data_ptr(), m.data_ptr(), _hp.forward_scale(scale_factor, x, narrow_scale), b, np_, sq, sk,
+            m.size(0), slopes_ptr, bias_ptr, lengths_ptr, _hp.dtype_code(x, "forward"), _hp.stream_of(x))
     _hp.check(rc, name)
     del keep
     return y
@@ -118,7 +121,8 @@ def _check_prob(p, name):
         raise RuntimeError(f"{name}: dropout probability has to be in [0, 1), got {p}")
 
 
-def forward_dropout(input, mask, scale_factor, p, seed, alibi_slopes=None, bias=None, key_lengths=None):
+def forward_dropout(input, mask, scale_factor, p, seed, alibi_slopes=None, bias=None, key_lengths=None, *,
+                    narrow_scale=False):
     """(not in the reference module) ``forward`` and attention dropout in one kernel: returns
     ``(dropped, probs)`` with ``dropped = keep ? probs / (1 - p) : 0``; the keep mask is generated from
     ``seed`` over the flat element index and is regenerated by ``backward_dropout``."""
@@ -131,8 +135,8 @@ def forward_dropout(input, mask, scale_factor, p, seed, alibi_slopes=None, bias=
     dropped = torch.empty_like(x)
     with _hp.device_guard(x):
         rc = _hp.lib().nhp_masked_softmax_ex_dropout_fwd(
-            dropped.data_ptr(), y.data_ptr(), x.data_ptr(), m.data_ptr(), float(scale_factor), b, np_, sq, sk, m.size(0),
-            slopes_ptr, bias_ptr, lengths_ptr, float(p), int(seed), 0, _hp.dtype_code(x, name), _hp.stream_of(x))
+            dropped.data_ptr(), y.data_ptr(), x.data_ptr(), m.data_ptr(), _hp.forward_scale(scale_factor, x, narrow_scale),
+            b, np_, sq, sk, m.size(0), slopes_ptr, bias_ptr, lengths_ptr, float(p), int(seed), 0, _hp.dtype_code(x, name), _hp.stream_of(x))
     _hp.check(rc, name)
     del keep
     return dropped, y

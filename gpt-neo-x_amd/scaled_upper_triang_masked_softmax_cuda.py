@@ -65,7 +65,8 @@ def _zero_block(zero_block):
     return zero_block
 
 
-def forward(input, scale_factor, window=None, alibi_slopes=None, bias=None, key_lengths=None, zero_block=0):
+def forward(input, scale_factor, window=None, alibi_slopes=None, bias=None, key_lengths=None, zero_block=0, *,
+            narrow_scale=False):
     """softmax(scale * input) under an upper-triangular mask.
 
     input: [attn_batches, seq_len, seq_len] fp16/bf16 on the GPU. Returns a new
@@ -87,6 +88,10 @@ def forward(input, scale_factor, window=None, alibi_slopes=None, bias=None, key_
         and skips the blocks without a visible (query, key) pair: row q is only written from the
         start of the block of the first key that the first row of its block sees to the end of the
         block of the diagonal; the rest of the returned tensor is uninitialised. 0: every row whole.
+    narrow_scale (keyword only): round ``scale_factor`` to the input's dtype before use, as the reference's
+        CUDA forward does (scaled_upper_triang_masked_softmax.h:368 takes ``const input_t scale``): results
+        then follow the reference's fused kernel; by default the fp32 value is used, as in the reference's
+        backward and torch branch. 1/sqrt(128) narrows to 0.08837890625 in fp16 and bf16 (-1.07e-4 relative).
     """
     if input.dim() != 3:
         raise RuntimeError("expected 3D tensor")
@@ -101,7 +106,7 @@ def forward(input, scale_factor, window=None, alibi_slopes=None, bias=None, key_
         x, alibi_slopes, bias, key_lengths, "scaled_upper_triang_masked_softmax_cuda.forward")
     with _hp.device_guard(x):
         rc = _hp.lib().nhp_causal_softmax_blocks_fwd(
-            y.data_ptr(), x.data_ptr(), float(scale_factor), x.size(0), x.size(1),
+            y.data_ptr(), x.data_ptr(), _hp.forward_scale(scale_factor, x, narrow_scale), x.size(0), x.size(1),
             -1 if window is None else int(window), _zero_block(zero_block), slopes_ptr, bias_ptr, lengths_ptr, heads or 1,
             _hp.dtype_code(x, "forward"), _hp.stream_of(x))
     _hp.check(rc, "scaled_upper_triang_masked_softmax_cuda.forward")
@@ -142,12 +147,12 @@ def backward(output_grads, softmax_results, scale_factor, window=None, key_lengt
 
 
 def forward_dropout(input, scale_factor, p, seed, window=None, zero_block=0, alibi_slopes=None, bias=None,
-                    key_lengths=None):
+                    key_lengths=None, *, narrow_scale=False):
     """``forward`` and attention dropout in one kernel: returns ``(dropped, probabilities)``.
 
     ``dropped = keep * probabilities / (1 - p)`` with the library's counter-based keep mask for
     ``seed`` (see ``nhp_causal_softmax_dropout_fwd``); ``probabilities`` is what ``forward`` returns
-    and what ``backward_dropout`` needs. ``alibi_slopes``, ``bias`` and ``key_lengths`` as in ``forward``.
+    and what ``backward_dropout`` needs. ``alibi_slopes``, ``bias``, ``key_lengths`` and ``narrow_scale`` as in ``forward``.
     Not part of the reference's extension module."""
     who = "scaled_upper_triang_masked_softmax_cuda.forward_dropout"
     if input.dim() != 3:
@@ -163,8 +168,8 @@ def forward_dropout(input, scale_factor, p, seed, window=None, zero_block=0, ali
     keep, slopes_ptr, bias_ptr, lengths_ptr, heads = _per_head_args(x, alibi_slopes, bias, key_lengths, who)
     with _hp.device_guard(x):
         rc = _hp.lib().nhp_causal_softmax_ex_dropout_fwd(
-            dropped.data_ptr(), y.data_ptr(), x.data_ptr(), float(scale_factor), x.size(0), x.size(1),
-            -1 if window is None else int(window), _zero_block(zero_block), slopes_ptr, bias_ptr, lengths_ptr,
+            dropped.data_ptr(), y.data_ptr(), x.data_ptr(), _hp.forward_scale(scale_factor, x, narrow_scale), x.size(0),
+            x.size(1), -1 if window is None else int(window), _zero_block(zero_block), slopes_ptr, bias_ptr, lengths_ptr,
             heads or 1, float(p), int(seed), 0, _hp.dtype_code(x, "forward_dropout"), _hp.stream_of(x))
     _hp.check(rc, who)
     del keep

@@ -225,3 +225,103 @@ def test_load_is_idempotent_and_reports_the_native_library():
     assert fk._hotpath.lib().nhp_abi_version() == fk._hotpath.ABI_VERSION
     # the shared object is mapped into this process
     assert any("libneox_hotpath.so" in line for line in open("/proc/self/maps"))
+
+
+def test_baseline_config_c1_whole_tensor_through_the_module():
+    """The first configuration of the benchmark set exactly as written: causal forward on scores
+    [b=4, h=8, 512, 512] bf16 ~ N(0, 4), scale 1/sqrt(64), seed 0, through FusedScaleMaskSoftmax;
+    every element against the oracle (<= 2 ulp), exact zeros above the diagonal, and against the
+    reference's torch branch (what that configuration runs on the CPU)."""
+    from megatron.model.fused_softmax import SoftmaxFusionTypes as T
+
+    b, np_, s = 4, 8, 512
+    scale = 1 / math.sqrt(64)
+    g = torch.Generator().manual_seed(0)
+    x = (torch.randn((b, np_, s, s), generator=g) * 2).to(torch.bfloat16)
+    mask = fb.causal_mask(s, DEV)
+    m = make(T.upper_triang, torch.bfloat16, scale)
+    assert m.is_kernel_available(mask, b, np_, s, s)
+    y = m(x.to(DEV), mask).cpu()
+    assert y.shape == (b, np_, s, s) and y.dtype == torch.bfloat16
+    want = oracle.causal_softmax_fwd(x.view(-1, s, s), scale).view(b, np_, s, s)
+    util.assert_ulp_close(y, want, 2, "C1 fused vs kernel-semantics oracle")  # 2 bf16 ulp
+    above = torch.triu(torch.ones(s, s, dtype=torch.bool), diagonal=1)
+    assert int(util.raw_bits(y)[..., above].abs().max()) == 0, "masked positions must be +0 bit for bit"
+    fallback = fb.torch_softmax_fallback(x, mask.cpu(), scale)
+    util.assert_ulp_close(y, fallback, 2, "C1 fused vs the torch branch")
+    # 0.125 is representable in bf16: the reference kernel's narrowing of the factor changes nothing here
+    m_narrow = FusedNarrow(T.upper_triang, torch.bfloat16, scale)
+    assert torch.equal(util.raw_bits(m_narrow(x.to(DEV), mask).cpu()), util.raw_bits(y))
+
+
+def FusedNarrow(fusion, dtype, scale):
+    from megatron.model.fused_softmax import FusedScaleMaskSoftmax
+
+    return FusedScaleMaskSoftmax(dtype == torch.float16, dtype == torch.bfloat16, fusion, mask_func, True, scale,
+                                 narrow_forward_scale=True)
+
+
+def _c3_style_scores(shape, seed):
+    """fp16 ~ N(0, 9) with 1 % of the entries at +-60, as the padding-mask configuration of the benchmark set."""
+    x = util.randn(shape, torch.float16, seed=seed, std=3.0)
+    g = torch.Generator().manual_seed(seed + 1)
+    hit = torch.rand(shape, generator=g) < 0.01
+    sign = torch.where(torch.rand(shape, generator=g) < 0.5, -60.0, 60.0).to(torch.float16)
+    return torch.where(hit, sign, x)
+
+
+@pytest.mark.parametrize("fusion", ["upper_triang", "general"])
+def test_narrow_forward_scale_follows_the_reference_kernel(fusion):
+    """narrow_forward_scale=True: the forward factor is rounded to the scores' dtype first, as the reference's
+    CUDA dispatchers do (scaled_upper_triang_masked_softmax.h:368, scaled_masked_softmax.h:358): within 2 ulp of
+    the kernel-semantics oracle called with the narrowed factor, on +-60 outliers where the two factors give
+    results up to 3 fp16 ulp apart. Default: within 2 ulp of the oracle with the fp32 factor (= the torch branch).
+    The backward uses the fp32 factor in both settings (:467 / :457 take acc_t)."""
+    from megatron.model.fused_softmax import SoftmaxFusionTypes as T
+
+    scale = 1 / math.sqrt(128)
+    narrowed = float(torch.tensor(scale).to(torch.float16))
+    assert narrowed == 0.08837890625
+    if fusion == "upper_triang":
+        b, np_, sq, sk = 2, 4, 1024, 1024
+        mask = fb.causal_mask(sq, "cpu")
+        ref = lambda x, f: oracle.causal_softmax_fwd(x.view(-1, sq, sk), f).view(b, np_, sq, sk)
+    else:
+        b, np_, sq, sk = 4, 4, 64, 2048
+        mask = util.padding_mask(b, sq, sk, seed=9, full_batch=1)
+        ref = lambda x, f: oracle.masked_softmax_fwd(x, mask, f)
+    x = _c3_style_scores((b, np_, sq, sk), seed=21)
+    dy = util.randn((b, np_, sq, sk), torch.float16, seed=23)
+    want_full, want_narrow = ref(x, scale), ref(x, narrowed)
+    assert int(util.ulp_distance(want_full, want_narrow).max()) >= 2, "the inputs must tell the two factors apart"
+
+    results = {}
+    for narrow in (False, True):
+        m = (FusedNarrow if narrow else make)(getattr(T, fusion), torch.float16, scale)
+        xd = x.to(DEV).requires_grad_(True)
+        y = m(xd, mask.to(DEV))
+        y.backward(dy.to(DEV))
+        yc = y.detach().cpu()
+        util.assert_ulp_close(yc, want_narrow if narrow else want_full, 2, f"forward, narrow={narrow}")  # 2 fp16 ulp
+        want_dx = oracle.softmax_bwd(dy.view(-1, sq, sk), yc.view(-1, sq, sk), scale, fusion == "upper_triang")
+        util.assert_softmax_bwd_close(xd.grad.cpu().view(-1, sq, sk), want_dx, dy.view(-1, sq, sk), yc.view(-1, sq, sk),
+                                      scale, f"backward with the fp32 factor, narrow={narrow}")
+        results[narrow] = yc
+    assert not torch.equal(util.raw_bits(results[False]), util.raw_bits(results[True]))
+
+
+def test_extension_forward_narrow_scale_keyword():
+    import scaled_masked_softmax_cuda as masked_ext
+    import scaled_upper_triang_masked_softmax_cuda as causal_ext
+
+    scale = 1 / math.sqrt(128)
+    narrowed = 0.08837890625
+    x = _c3_style_scores((4, 512, 512), seed=31).to(DEV)
+    got = causal_ext.forward(x, scale, narrow_scale=True)
+    same = causal_ext.forward(x, narrowed)
+    assert torch.equal(util.raw_bits(got.cpu()), util.raw_bits(same.cpu()))
+    xb = x.bfloat16().view(1, 4, 512, 512)
+    mask = util.padding_mask(1, 512, 512, seed=3).to(DEV)
+    got = masked_ext.forward(xb, mask, scale, narrow_scale=True)
+    same = masked_ext.forward(xb, mask, narrowed)  # the bf16 rounding of 1/sqrt(128) is the same number
+    assert torch.equal(util.raw_bits(got.cpu()), util.raw_bits(same.cpu()))

@@ -214,6 +214,64 @@ def test_load_fused_kernels_exits_when_not_installed(hotpath, monkeypatch, tmp_p
 
 
 # ---------------------------------------------------------------------------
+# the reference's get_norm classes are torch modules that run on any device (megatron/model/norms.py:16,54-119)
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_norm_modules_off_the_gpu_follow_the_reference_expressions(dtype):
+    from megatron.model import norms
+
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn((3, 5, 32), generator=g) * 2 + 0.5).to(dtype)
+    dy = torch.randn((3, 5, 32), generator=g).to(dtype)
+
+    def grads(module, inp):
+        inp = inp.clone().requires_grad_(True)
+        out = module(inp)
+        out.backward(dy.to(out.dtype))
+        return out.detach(), inp.grad, [p.grad.clone() for p in module.parameters()]
+
+    # LayerNorm: torch's own class is the reference's
+    ours, theirs = norms.LayerNorm(32, eps=1e-5).to(dtype), torch.nn.LayerNorm(32, eps=1e-5).to(dtype)
+    with torch.no_grad():
+        for p in (ours.weight, theirs.weight):
+            p.copy_(torch.linspace(0.5, 1.5, 32))
+        for p in (ours.bias, theirs.bias):
+            p.copy_(torch.linspace(-1, 1, 32))
+    for a, b in zip(grads(ours, x)[:2], grads(theirs, x)[:2]):
+        assert a.dtype == b.dtype and torch.equal(a, b)
+
+    # RMSNorm, full and partial, with and without offset: x / (||x[:k]|| / sqrt(k) + eps) * scale [+ offset]
+    for p_frac, bias in ((-1.0, False), (0.5, False), (-1.0, True)):
+        m = norms.RMSNorm(32, p=p_frac, eps=1e-8, bias=bias).to(dtype)
+        with torch.no_grad():
+            m.scale.copy_(torch.linspace(0.5, 1.5, 32))
+        out, dx, _ = grads(m, x)
+        k = 32 if p_frac < 0 else 16
+        x64 = x.double().requires_grad_(True)
+        rms = x64[..., :k].pow(2).sum(-1, keepdim=True).sqrt() / math.sqrt(k)
+        want = m.scale.detach().double() * (x64 / (rms + 1e-8))
+        want.backward(dy.double())
+        tol = 1e-5 if dtype == torch.float32 else 6e-2
+        assert out.dtype == dtype and out.shape == x.shape
+        assert (out.double() - want.detach()).abs().max().item() <= tol * max(1.0, want.detach().abs().max().item())
+        assert (dx.double() - x64.grad).abs().max().item() <= tol * max(1.0, x64.grad.abs().max().item())
+    fused = norms.RMSNorm(32, eps=1e-6, fused_eps=True).to(dtype)
+    want = (x.float() * torch.rsqrt(x.float().pow(2).mean(-1, keepdim=True) + 1e-6)).to(dtype)
+    assert torch.equal(fused(x).detach(), want)
+
+    # ScaleNorm: x / max(||x||, eps) * g, clamped rows included
+    sn = norms.ScaleNorm(32, eps=1e-5).to(dtype)
+    with torch.no_grad():
+        sn.g.fill_(1.5)
+    xs = x.clone()
+    xs[0, 0] = 0
+    out = sn(xs).detach()
+    want = xs.double() / xs.double().norm(dim=-1, keepdim=True).clamp(min=1e-5) * 1.5
+    assert out.dtype == dtype and float(out[0, 0].abs().sum()) == 0
+    assert (out.double() - want).abs().max().item() <= (1e-5 if dtype == torch.float32 else 3e-2)
+
+
+# ---------------------------------------------------------------------------
 # element-wise and normalisation modules: names, parameters, errors (no GPU needed)
 # ---------------------------------------------------------------------------
 def test_layer_modules_surface_and_errors():
@@ -239,8 +297,6 @@ def test_layer_modules_surface_and_errors():
     assert norms.LayerNorm((16,), elementwise_affine=False).weight is None
     with pytest.raises(NotImplementedError):
         norms.LayerNorm((4, 16))
-    with pytest.raises(RuntimeError, match="GPU"):
-        ln(torch.zeros(2, 16))
     rms = norms.RMSNorm(16, eps=1e-8)
     assert [n for n, _ in rms.named_parameters()] == ["scale"] and rms.offset is None
     assert sorted(n for n, _ in norms.RMSNorm(16, bias=True).named_parameters()) == ["offset", "scale"]
@@ -505,3 +561,26 @@ def test_block_limited_softmax_is_not_part_of_the_public_forward():
 
     assert list(inspect.signature(FusedScaleMaskSoftmax.forward).parameters) == ["self", "input", "mask", "bias", "key_lengths"]
     assert hasattr(FusedScaleMaskSoftmax, "_forward_block_limited")
+
+
+def test_forward_scale_narrowing_helper_and_constructor_flag():
+    """The opt-in that reproduces the reference's `const input_t scale` (scaled_upper_triang_masked_softmax.h:368,
+    scaled_masked_softmax.h:358): rounding to the scores' dtype, round to nearest even, on the host."""
+    from megatron.fused_kernels import _hotpath as hp
+    from megatron.model.fused_softmax import FusedScaleMaskSoftmax, SoftmaxFusionTypes
+
+    s128 = 1 / math.sqrt(128)
+    for dtype in (torch.float16, torch.bfloat16):
+        t = torch.zeros(1, dtype=dtype)
+        assert hp.forward_scale(s128, t, False) == s128
+        assert hp.forward_scale(s128, t, True) == 0.08837890625
+        assert hp.forward_scale(0.125, t, True) == 0.125
+        assert hp.forward_scale(torch.tensor([0.3])[0], t, True) == float(torch.tensor(0.3).to(dtype))
+    # 1 + 2^-8 is a tie in bf16 (8 significant bits): to even, i.e. down; 1 + 3 * 2^-8 ties up
+    bf = torch.zeros(1, dtype=torch.bfloat16)
+    assert hp.forward_scale(1 + 2.0**-8, bf, True) == 1.0
+    assert hp.forward_scale(1 + 3 * 2.0**-8, bf, True) == 1 + 2.0**-6
+    m = FusedScaleMaskSoftmax(True, False, SoftmaxFusionTypes.none, lambda s, k: s, True, s128)
+    assert m.narrow_forward_scale is False
+    m = FusedScaleMaskSoftmax(True, False, SoftmaxFusionTypes.none, lambda s, k: s, True, s128, narrow_forward_scale=True)
+    assert m.narrow_forward_scale is True
