@@ -513,6 +513,50 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False, launc
         cfg = {"workload": name, "what": "data movement only; bytes as the kernels they stand for are priced"}
         return step, kernel_bytes, {}, "copy_1024MiB", "u8", cfg
 
+    if name == "causal-c1":
+        # scores [b=4, h=8, 512, 512] bf16 ~ N(0, 4), scale 1/sqrt(64): 16 MiB per tensor, so the launches rotate over
+        # 16 buffer pairs (512 MiB in all, twice the last-level cache). A launch lasts a few microseconds, less
+        # than the host needs to issue it: each bracket holds 16 launches issued while the GPU is still busy
+        # with a 1 GiB copy, so that they run back to back and the bracket measures the GPU's time.
+        a, s = 32, 512
+        scale = 1.0 / math.sqrt(64)
+        sets = [randn((a, s, s), 700 + i, torch.bfloat16, 2.0) for i in range(16)]
+        filler = (torch.empty(1 << 29, dtype=torch.bfloat16, device=dev), torch.empty(1 << 29, dtype=torch.bfloat16, device=dev))
+        fwd_b, _ = causal_bytes(a, s)
+        kernel_bytes = {"causal_softmax_fwd": 16 * fwd_b}
+
+        def step(t):
+            filler[1].copy_(filler[0])
+            t.run("causal_softmax_fwd", lambda: [causal_ext.forward(x, scale) for x in sets])
+
+        cfg = {"workload": name, "scores": [a, s, s], "scale": "1/sqrt(64)", "launches_per_bracket": 16,
+               "bytes_convention": "causal-min (reads of the lower triangle, dense writes)"}
+        return step, kernel_bytes, {"causal_softmax_fwd": 16 * 2 * a * s * s * 2}, "causal_softmax_fwd", "bf16", cfg
+
+    if name == "rope-styles-1.4b":
+        # the rotary leg of the default workload in both call styles: one launch per tensor (the reference's
+        # fused_apply_rotary_pos_emb_cached, called for q and then for k) and q and k in one launch
+        s, b, h, d, d2 = 2048, 8, 16, 128, 32
+        sets = [rope_setup(s, b, h, d, d2, 50 + 10 * i) for i in range(4)]
+        rb = rope_bytes(s, b, h, d, d2)
+        one = 2 * rb - 2 * s * d2 * 2
+        kernel_bytes = {"rope_fwd_per_tensor": 2 * rb, "rope_bwd_per_tensor": 2 * rb, "rope_fwd_one_launch": one,
+                        "rope_bwd_one_launch": one}
+        state = {"i": 0}
+
+        def step(t):
+            q, k, dq, dk, cos, sin = sets[state["i"] % len(sets)]
+            state["i"] += 1
+            t.run("rope_fwd_per_tensor", lambda: (rope_ext.forward_cached(q, cos, sin, False),
+                                                  rope_ext.forward_cached(k, cos, sin, False)))
+            t.run("rope_bwd_per_tensor", lambda: (rope_ext.backward_cached(dq, cos, sin, False),
+                                                  rope_ext.backward_cached(dk, cos, sin, False)))
+            t.run("rope_fwd_one_launch", lambda: rope_ext.forward_cached_qk(q, k, cos, sin, False))
+            t.run("rope_bwd_one_launch", lambda: rope_ext.backward_cached_qk(dq, dk, cos, sin, False))
+
+        cfg = {"workload": name, "qk": [s, b, h, d], "rotary_dim": d2}
+        return step, kernel_bytes, {}, "rope_fwd_per_tensor", "bf16", cfg
+
     if name == "rope-qk-1.4b":
         s, b, h, d, d2 = 2048, 8, 16, 128, 32
         sets = [rope_setup(s, b, h, d, d2, 50 + 10 * i) for i in range(4)]  # rotate buffers: 64 MiB tensors fit the cache
@@ -939,6 +983,85 @@ def cpu_baseline(torch):
                       f"{med * 1e3:.1f} ms each, same algorithmic-byte convention"}
 
 
+def measure_workload(name, torch, dev, steps, warmup):
+    """Event-brackets every kernel of a workload over `steps` steps after `warmup`: per kernel the algorithmic
+    bytes, mean and median bracket in microseconds, GB/s and the fraction of the HBM peak. The workload's tensors
+    are released afterwards."""
+    import gc
+
+    step, kernel_bytes, other, _, dtype, cfg = make_workload(name, torch, dev, launches=warmup + steps)
+    timer = Timer(torch)
+    for _ in range(warmup):
+        step(timer)
+    torch.cuda.synchronize()
+    timer.reset()
+    for _ in range(steps):
+        step(timer)
+    torch.cuda.synchronize()
+    avg = timer.averages_ms()
+    per = cfg.get("launches_per_bracket", 1)
+    out = {}
+    for key, nbytes in kernel_bytes.items():
+        gbs = nbytes / (avg[key] * 1e-3) / 1e9
+        out[key] = {"bytes": nbytes // per, "us": round(avg[key] * 1e3 / per, 2),
+                    "median_us": round(timer.spread_ms(key)[1] * 1e3 / per, 2), "GB/s": round(gbs, 1),
+                    "frac_of_peak": round(gbs / HBM_PEAK_GBS, 4)}
+        if key in other:
+            label, nb = other[key] if isinstance(other[key], tuple) else ("GB/s_dense_convention", other[key])
+            out[key][label] = round(nb / (avg[key] * 1e-3) / 1e9, 1)
+    del step, timer
+    gc.collect()
+    torch.cuda.empty_cache()
+    return {"dtype": dtype, "workload": cfg, "steps": steps, "warmup": warmup, "kernels": out}
+
+
+def cpu_fallback_c1(torch):
+    """The first configuration as the reference runs it without its kernels: forward_torch_softmax on the host cores,
+    scores [4,8,512,512] bf16 ~ N(0,4), scale 1/sqrt(64), causal mask, seed 0."""
+    from oracle import fallback_semantics as fb
+
+    torch.set_num_threads(os.cpu_count() or 1)
+    g = torch.Generator().manual_seed(0)
+    x = (torch.randn((4, 8, 512, 512), generator=g) * 2).bfloat16()
+    mask = fb.causal_mask(512)
+    scale = 1.0 / math.sqrt(64)
+    fb.torch_softmax_fallback(x, mask, scale)
+    times = []
+    for _ in range(9):
+        t0 = time.perf_counter()
+        fb.torch_softmax_fallback(x, mask, scale)
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    nbytes = causal_bytes(32, 512)[0]
+    return {"ms": round(med * 1e3, 3), "min_ms": round(times[0] * 1e3, 3), "bytes": nbytes,
+            "GB/s": round(nbytes / med / 1e9, 2), "cores": torch.get_num_threads(), "kind": "port",
+            "what": "reference torch branch (fp32 softmax, masked_fill with the dtype minimum), median of 9 runs"}
+
+
+def baseline_configs(torch, dev, with_cpu):
+    """Every configuration of the benchmark set beside the headline one, each kernel event-bracketed on its
+    real tensors: C1 (HIP kernel, and the torch branch on the host cores), the rotary leg of C2 in both call
+    styles, C3, C4 (both rotary fractions, one launch per tensor; and q, k as views of one fused projection
+    buffer, per tensor and in one launch), C5, and the sliding-window variant of C5's scores."""
+    out = {}
+    c1 = measure_workload("causal-c1", torch, dev, steps=10, warmup=3)
+    if with_cpu:
+        c1["cpu_fallback"] = cpu_fallback_c1(torch)
+    out["C1 causal fwd [4,8,512,512] bf16"] = c1
+    out["C2 rotary leg, both call styles [2048,8,16,128] rotary_pct 0.25"] = measure_workload(
+        "rope-styles-1.4b", torch, dev, steps=20, warmup=5)
+    out["C3 padding-mask softmax fwd+bwd [16,32,1024,2048] fp16"] = measure_workload("masked-c3", torch, dev, steps=12, warmup=3)
+    out["C4 rotary fwd+bwd [4096,4,32,128] rotary_pct 1.0 and 0.25, one launch per tensor"] = measure_workload(
+        "rope-c4", torch, dev, steps=20, warmup=5)
+    out["C4 rotary on q,k sliced from a fused [4096,4,32,384] buffer"] = measure_workload(
+        "rope-c4-qkv-view", torch, dev, steps=20, warmup=5)
+    out["C5 rotary [8192,2,32,128] + causal fwd+bwd [64,8192,8192] bf16"] = measure_workload(
+        "llama2-7b-c5", torch, dev, steps=8, warmup=2)
+    out["C5 scores with a 4096-key sliding window"] = measure_workload("mistral-window", torch, dev, steps=8, warmup=2)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -946,6 +1069,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="pythia-1.4b")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="default workload: leave out the `configs` object (the other configurations of the benchmark set, "
+                         "measured after the timed region)")
     ap.add_argument("--fresh-dy", action="store_true",
                     help="pythia-1.4b / llama2-7b-c5: restore the upstream gradient from a pristine copy before every "
                          "in-place backward (the copy runs outside the backward's event bracket but inside the step)")
@@ -1048,6 +1174,13 @@ def main():
     }
     if args.workload == "pythia-1.4b" and not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch)
+    if args.workload == "pythia-1.4b" and not args.no_configs:
+        import gc
+
+        del step, timer, full
+        gc.collect()
+        torch.cuda.empty_cache()
+        out["configs"] = baseline_configs(torch, dev, not args.no_cpu_baseline)
     print(json.dumps(out), flush=True)
 
 

@@ -735,17 +735,20 @@ static int bwd_waves_of(const NormPlan& p, int v)
 // With parameter gradients the backward grid is bounded (every workgroup writes a partial row
 // that the second kernel has to read): 4096 waves in all, 16 per CU.
 constexpr uint32_t kNormBwdWaves = 4096;
+// Compute units of an MI355X. The grid bounds below are whole rounds of workgroups over this many CUs; on a
+// part with another count they stay correct and only lose the "no ragged last round" property.
+constexpr uint32_t kCUs = 256;
 
 static uint32_t norm_bwd_grid(uint32_t row_blocks, bool param_grads, int waves_per_block, int in_flight,
                               bool one_per_cu = false)
 {
     row_blocks = (row_blocks + in_flight - 1) / in_flight;  // a workgroup takes that many row blocks per iteration
     if (!param_grads) return row_blocks;
-    // a whole number of workgroups per CU (256 CUs): a ragged last round costs more than the waves it adds
-    uint32_t cap = kNormBwdWaves / (uint32_t)waves_per_block / 256u * 256u;
+    // a whole number of workgroups per CU: a ragged last round costs more than the waves it adds
+    uint32_t cap = kNormBwdWaves / (uint32_t)waves_per_block / kCUs * kCUs;
     // two gradients and two chunks per lane, or four chunks per lane: 158-163 VGPRs, one 8-wave workgroup per
     // CU is resident; a second round of workgroups costs more than it brings (244 -> 225 us at [16384, 6144])
-    if (cap == 0 || one_per_cu) cap = 256;
+    if (cap == 0 || one_per_cu) cap = kCUs;
     cap = (uint32_t)NHP_TUNED_INT("NHP_NORM_GRID", (int)cap);
     return row_blocks < cap ? row_blocks : cap;
 }
@@ -809,7 +812,8 @@ static int64_t norm_workspace_bytes(int64_t rows, int64_t cols, int dtype, bool 
 template <int DT, bool RMS>
 static int norm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, const void* x, const float* mean,
                     const float* rstd, const void* gamma, void* workspace, float eps, int eps_mode, int64_t rows,
-                    int64_t cols, int64_t stat, int pdt, hipStream_t st, const NormSecond& second = NormSecond{})
+                    int64_t cols, int64_t stat, int pdt, hipStream_t st, const NormSecond& second = NormSecond{},
+                    uint32_t max_partial_rows = 0)
 {
     launch_prepare();
     constexpr int V = Elt<DT>::kVec;
@@ -821,8 +825,10 @@ static int norm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, const v
         plan_norm(cols / V, true, p, pair)) {
         const int waves = bwd_waves_of(p, V);
         const uint32_t row_blocks = norm_row_blocks(rows, p, waves);
-        const uint32_t grid = norm_bwd_grid(row_blocks, want_params, waves, bwd_rows_in_flight(p.K, p.W, pair),
-                                            (pair && p.K >= 2) || p.K >= 4);
+        uint32_t grid = norm_bwd_grid(row_blocks, want_params, waves, bwd_rows_in_flight(p.K, p.W, pair),
+                                      (pair && p.K >= 2) || p.K >= 4);
+        // a caller with a fixed workspace: fewer workgroups, each striding over more row blocks
+        if (want_params && max_partial_rows != 0 && grid > max_partial_rows) grid = max_partial_rows;
         const size_t part = (size_t)grid * cols;
         float* part_g = want_params ? static_cast<float*>(workspace) : nullptr;
         float* part_b = want_params ? part_g + part : nullptr;
@@ -914,7 +920,7 @@ template <bool RMS>
 static int norm_bwd_dispatch(void* dx, void* dgamma, void* dbeta, const void* dy, const void* x, const float* mean,
                              const float* rstd, const void* gamma, void* workspace, float eps, int eps_mode,
                              int64_t rows, int64_t cols, int64_t stat, int dtype, int pdt, void* stream,
-                             const NormSecond& second = NormSecond{})
+                             const NormSecond& second = NormSecond{}, uint32_t max_partial_rows = 0)
 {
     if (int rc = norm_check(rows, cols, dtype, pdt)) return rc;
     if (RMS && (eps_mode < 0 || eps_mode > 2)) return NHP_ERR_SHAPE;
@@ -927,13 +933,13 @@ static int norm_bwd_dispatch(void* dx, void* dgamma, void* dbeta, const void* dy
     switch (dtype) {
     case NHP_F16:
         return norm_bwd<NHP_F16, RMS>(dx, dgamma, dbeta, dy, x, mean, rstd, gamma, workspace, eps, eps_mode, rows,
-                                      cols, stat, pdt, st, second);
+                                      cols, stat, pdt, st, second, max_partial_rows);
     case NHP_BF16:
         return norm_bwd<NHP_BF16, RMS>(dx, dgamma, dbeta, dy, x, mean, rstd, gamma, workspace, eps, eps_mode, rows,
-                                       cols, stat, pdt, st, second);
+                                       cols, stat, pdt, st, second, max_partial_rows);
     default:
         return norm_bwd<NHP_F32, RMS>(dx, dgamma, dbeta, dy, x, mean, rstd, gamma, workspace, eps, eps_mode, rows,
-                                      cols, stat, pdt, st, second);
+                                      cols, stat, pdt, st, second, max_partial_rows);
     }
 }
 
@@ -996,13 +1002,20 @@ int nhp_layernorm_bwd_noalloc(void* dx, void* dgamma, void* dbeta, const void* d
 {
     if (dtype != NHP_F16 && dtype != NHP_BF16 && dtype != NHP_F32) return NHP_ERR_DTYPE;
     void* ws = nullptr;
-    if (dgamma != nullptr || dbeta != nullptr) {
-        if (norm_workspace_bytes(rows, cols, dtype) > (int64_t)kNoallocScratchBytes) return NHP_ERR_SCRATCH;
+    uint32_t max_partial_rows = 0;
+    if ((dgamma != nullptr || dbeta != nullptr) && rows > 0 && cols > 0) {
+        // The fixed array holds two fp32 partial rows (dgamma, dbeta) per workgroup: where nhp_layernorm_bwd
+        // would use more workgroups than fit, this entry point launches fewer (each strides over more row
+        // blocks; the sums are then formed in another order, within rounding of nhp_layernorm_bwd's).
+        // Rows too long for even 8 workgroups are refused.
+        const int64_t fit = (int64_t)kNoallocScratchBytes / (2 * cols * (int64_t)sizeof(float));
+        if (fit < 8) return NHP_ERR_SCRATCH;
+        max_partial_rows = (uint32_t)(fit < (int64_t)kNormBwdWaves ? fit : (int64_t)kNormBwdWaves);
         ws = noalloc_scratch();
         if (ws == nullptr) return NHP_ERR_LAUNCH;
     }
     return norm_bwd_dispatch<false>(dx, dgamma, dbeta, dy, x, mean, rstd, gamma, ws, 0.0f, 0, rows, cols, cols, dtype,
-                                    param_dtype, stream);
+                                    param_dtype, stream, NormSecond{}, max_partial_rows);
 }
 
 int nhp_layernorm_pair_fwd(void* y1, void* y2, float* mean, float* rstd, const void* x, const void* gamma1,

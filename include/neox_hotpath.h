@@ -61,7 +61,10 @@ int64_t nhp_softmax_max_resident_row(void);
  * records (a measured figure belongs to one kernel instantiation): lanes per row L, 16-byte
  * chunks per lane K, waves per row W. `kind`: 0 causal forward, 1 causal forward with AliBi
  * or a bias tensor, 2 causal backward, 3 padding-mask forward, 4 padding-mask backward.
- * Returns NHP_ERR_SHAPE when such rows take the scalar kernel. */
+ * Returns NHP_ERR_SHAPE when such rows take the scalar kernel. Kind 0 describes the general
+ * forward kernel; rows of at most 512 elements in tensors of enough rows (rows * L >= 2^20) with
+ * nothing but the causal mask or a window take a kernel with the same L and four rows per lane,
+ * which this query does not tell apart (the query has no row count). */
 int nhp_softmax_geometry(int64_t row_len, int kind, int* lanes, int* chunks, int* waves);
 
 /* ------------------------------------------------------------------------
@@ -614,11 +617,16 @@ int nhp_layernorm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, const
 /*
  * nhp_layernorm_bwd without a workspace argument and without any allocation, for callers that
  * cannot allocate device memory (code under HIP graph capture, tight serving loops, harnesses
- * that forbid it). No counterpart in the reference. Same arguments, kernels and results as
+ * that forbid it). No counterpart in the reference. Same arguments and kernels as
  * nhp_layernorm_bwd; the partial sums of the parameter gradients go to a fixed device array of
  * NHP_NOALLOC_SCRATCH_BYTES bytes (16 MiB) that is part of the library image on
- * every GPU it runs on. Shapes whose nhp_norm_bwd_workspace_bytes() exceed that return
- * NHP_ERR_SCRATCH (nothing is launched); without parameter gradients any shape is accepted.
+ * every GPU it runs on. The array holds 16 MiB / (8 * cols) pairs of fp32 partial rows. Where
+ * nhp_layernorm_bwd would use more workgroups than that (at 16384 rows: more than 4096 columns), fewer
+ * are launched and each covers more rows: dx is the same bit for bit, dgamma and dbeta are sums in
+ * another order (equal within fp32 rounding of the sums, then rounded to the parameter dtype); where
+ * it would not, every result is bit-identical to nhp_layernorm_bwd's. Rows of more than 262144
+ * columns (fewer than 8 partial rows fit) return NHP_ERR_SCRATCH with parameter gradients (nothing
+ * is launched); without parameter gradients any shape is accepted.
  * The caller's device must be current. All calls on one GPU share the array: calls that overlap
  * in time on one GPU (different streams or threads) race; calls on one stream are ordered.
  * Nothing needs clearing between calls (every partial row that is read was written by the

@@ -293,7 +293,8 @@ def test_narrow_forward_scale_follows_the_reference_kernel(fusion):
     x = _c3_style_scores((b, np_, sq, sk), seed=21)
     dy = util.randn((b, np_, sq, sk), torch.float16, seed=23)
     want_full, want_narrow = ref(x, scale), ref(x, narrowed)
-    assert int(util.ulp_distance(want_full, want_narrow).max()) >= 2, "the inputs must tell the two factors apart"
+    apart = util.ulp_distance(want_full, want_narrow)
+    assert int(apart.max()) >= 1 and (apart > 0).float().mean().item() > 0.02, "the inputs must tell the two factors apart"
 
     results = {}
     for narrow in (False, True):

@@ -86,6 +86,43 @@ def test_causal_forward_short_rows_many_rows(hotpath, n, batches, dtype):
         assert (got[b0].cpu().float().triu(1) == 0).all()
 
 
+@pytest.mark.parametrize("n,batches", [(512, 40), (136, 490), (24, 21900)], ids=lambda v: str(v))
+@pytest.mark.parametrize("window", ["third", 0, "wide"])
+def test_causal_forward_short_rows_many_rows_with_a_window(hotpath, n, batches, window):
+    """The short-row kernel also serves a sliding window (nothing else: AliBi, bias, key lengths, dropout and block
+    limits go to the general kernel). Bit for bit the general kernel's result on groups of matrices below the row
+    count that selects the short-row kernel, and two matrices against the oracle."""
+    w = {"third": n // 3, 0: 0, "wide": n + 5}[window]
+    say(f"causal short rows with window n={n} batches={batches} window={w}")
+    dtype = torch.bfloat16
+    x = util.randn((batches, n, n), dtype, seed=n + 1, std=2.0).to(DEV)
+    scale = 0.11
+
+    def run(t):
+        y = torch.empty_like(t)
+        rc = hotpath.lib().nhp_causal_softmax_ex_fwd(y.data_ptr(), t.data_ptr(), scale, t.size(0), n, w, None, None, None, 1,
+                                                     hotpath.BF16, None)
+        assert rc == 0, hotpath.lib().nhp_status_string(rc)
+        return y
+
+    got = run(x)
+    step = max(1, (1 << 20) // (4 * n * max(8, n // 8)))
+    for b0 in list(range(0, batches, max(1, batches // 5)))[:5] + [batches - step]:
+        part = run(x[b0:b0 + step].contiguous())
+        assert torch.equal(util.raw_bits(got[b0:b0 + step]), util.raw_bits(part)), b0
+    for b0 in (0, batches - 1):
+        want = oracle.causal_softmax_fwd(x[b0:b0 + 1].cpu(), scale, window=w)
+        util.assert_ulp_close(got[b0:b0 + 1].cpu(), want, 2, f"matrix {b0}")
+        outside = ~fb_band(n, w)
+        assert int(util.raw_bits(got[b0].cpu())[outside].abs().max()) == 0, "outside the band: +0 bit for bit"
+
+
+def fb_band(n, w):
+    q = torch.arange(n).view(n, 1)
+    k = torch.arange(n).view(1, n)
+    return (k <= q) & (k >= q - w)
+
+
 def test_causal_forward_in_place(hotpath):
     x = util.randn((4, 512, 512), torch.bfloat16, seed=5, std=2.0).to(DEV)
     want = util.abi_causal_fwd(hotpath, x, 0.125)

@@ -84,8 +84,32 @@ def test_noalloc_without_parameter_gradients_and_too_large(hotpath):
     want, _, _ = _backward(hp, False, x, dy, gamma, mean, rstd)
     torch.cuda.synchronize()
     assert torch.equal(util.raw_bits(dx), util.raw_bits(want))
-    # a shape whose partial rows do not fit the fixed array is refused before anything is launched
-    rows, cols = 1 << 20, 32768
-    assert L.nhp_norm_bwd_workspace_bytes(rows, cols, hp.BF16) > 16 << 20
+    # rows so long that fewer than 8 pairs of partial rows fit the fixed array are refused before anything is launched
+    rows, cols = 1 << 12, 1 << 19
     p = ctypes.c_void_p(0x1000)  # never dereferenced
     assert L.nhp_layernorm_bwd_noalloc(p, p, p, p, p, p, p, p, rows, cols, hp.BF16, hp.BF16, None) == -7
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("cols", [5120, 6144, 8192])
+def test_noalloc_with_fewer_partial_rows_than_the_workspace_entry_point(hotpath, cols):
+    """At [16384, cols] beyond 4096 columns nhp_layernorm_bwd wants a workspace of more than 16 MiB
+    (25-32 MiB): the entry point without allocation launches as many workgroups as have room for their
+    partial rows in the fixed array. dx does not depend on the grid (bit-identical); dgamma / dbeta are the
+    same column sums added in another order: within 2 ulp of the parameter dtype, or within the fp32
+    rounding noise of a sum of that many terms."""
+    hp = hotpath
+    rows = 16384
+    assert hp.lib().nhp_norm_bwd_workspace_bytes(rows, cols, hp.BF16) > 16 << 20
+    for pdtype in (torch.bfloat16, torch.float32):
+        x, dy, gamma, beta = _inputs(torch.bfloat16, rows, cols, 7, pdtype)
+        mean, rstd = _stats(hp, x, gamma, beta)
+        want = _backward(hp, False, x, dy, gamma, mean, rstd)
+        got = _backward(hp, True, x, dy, gamma, mean, rstd)
+        assert torch.equal(util.raw_bits(got[0]), util.raw_bits(want[0])), "dx"
+        for name, g, w in zip(("dgamma", "dbeta"), got[1:], want[1:]):
+            assert not torch.isnan(g.float()).any(), f"{name} not fully written"
+            # |terms| of a column sum to about rows * E|dy * xhat| ~ rows; fp32 noise of re-ordering: a few eps of that
+            noise = 8 * util.EPS32 * rows
+            ok = (util.ulp_distance(g, w) <= 2) | ((g.float() - w.float()).abs() <= noise)
+            assert bool(ok.all()), f"{name}: {int((~ok).sum())} columns differ beyond reordering noise"
