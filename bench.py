@@ -470,6 +470,9 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False, launc
             key = f"causal_pattern_{a}x{s}x{s}"
             kernel_bytes[key] = causal_bytes(a, s)[0]
             pat.append((key, x, y, a, s))
+        plib.nhp_probe_causal_bwd_pattern.argtypes = [vp, vp, i64, i64, vp]
+        for _, _, _, a, s in pat:
+            kernel_bytes[f"causal_bwd_pattern_{a}x{s}x{s}"] = causal_bytes(a, s)[1]
         plib.nhp_probe_seq_major_pattern.argtypes = [vp, vp, i64, i64, vp]
         plib.nhp_probe_streams.argtypes = [vp, vp, vp, vp, i64, ctypes.c_int, ctypes.c_int, vp]
         # 64 MiB streams (the hidden state [16384, 2048] bf16 of the layer kernels): n inputs -> one or no output
@@ -488,16 +491,34 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False, launc
         tr_bufs = [(randn((tr_rows, 128, tr_s), 500 + j, torch.bfloat16),
                     torch.empty((tr_s, tr_rows, 128), dtype=torch.bfloat16, device=dev)) for j in range(8)]
         kernel_bytes["seq_major_pattern_128x128x2048"] = 2 * tr_rows * 128 * tr_s * 2
+        # q and k as slices of a fused projection buffer [4096, 4, 32, 3 * 128] bf16: 256-byte head vectors 768 bytes
+        # apart copied to one contiguous tensor (one tensor per launch), and 512-byte (q|k) runs split over two
+        plib.nhp_probe_strided_runs.argtypes = [vp, vp, vp, i64, ctypes.c_int, i64, ctypes.c_int, vp]
+        qkv_rows = 4096 * 4 * 32
+        qkv_bufs = [(randn((qkv_rows, 384), 650 + j, torch.bfloat16),
+                     torch.empty((qkv_rows, 128), dtype=torch.bfloat16, device=dev),
+                     torch.empty((qkv_rows, 128), dtype=torch.bfloat16, device=dev)) for j in range(3)]
+        kernel_bytes["strided_256_of_768_bytes_128MiB"] = 2 * qkv_rows * 256
+        kernel_bytes["strided_512_of_768_bytes_split_2x128MiB"] = 4 * qkv_rows * 256
         state = {"i": 0}
         stream = hp.stream_of(pat[0][1])
 
         def step(t):
             state["i"] += 1
+            src, o0, o1 = qkv_bufs[state["i"] % len(qkv_bufs)]
+            t.run("strided_256_of_768_bytes_128MiB", lambda: hp.check(plib.nhp_probe_strided_runs(
+                o0.data_ptr(), None, src.data_ptr(), qkv_rows, 16, 48, 0, stream), "strided runs"))
+            t.run("strided_512_of_768_bytes_split_2x128MiB", lambda: hp.check(plib.nhp_probe_strided_runs(
+                o0.data_ptr(), o1.data_ptr(), src.data_ptr(), qkv_rows, 32, 48, 1, stream), "strided runs, split"))
             for key, bufs, mib in runs:
                 src, dst = bufs[state["i"] % len(bufs)]
                 t.run(key, lambda: hp.check(plib.nhp_probe_copy(dst.data_ptr(), src.data_ptr(), mib << 20, 256, stream), key))
             for key, x, y, a, s in pat:
                 t.run(key, lambda: hp.check(plib.nhp_probe_causal_pattern(y.data_ptr(), x.data_ptr(), a, s, stream), key))
+            for _, x, y, a, s in pat:
+                # two triangles read, the first tensor's rows overwritten (XOR of random data stays random)
+                t.run(f"causal_bwd_pattern_{a}x{s}x{s}", lambda: hp.check(
+                    plib.nhp_probe_causal_bwd_pattern(y.data_ptr(), x.data_ptr(), a, s, stream), "causal bwd pattern"))
             bufs4 = mix_bufs[state["i"] % len(mix_bufs)]
             for key, n_in, w in mixes:
                 t.run(key, lambda: hp.check(plib.nhp_probe_streams(bufs4[3].data_ptr(), bufs4[0].data_ptr(), bufs4[1].data_ptr(),

@@ -14,11 +14,19 @@
 //                             is read up to the 16-byte chunk that holds column q and written in
 //                             full; two waves per row, two chunks per lane for n = 2048, as the
 //                             forward kernel is launched
+//   nhp_probe_causal_bwd_pattern  the causal softmax backward's traffic: the rows of two tensors read up to
+//                             the diagonal, the first tensor's rows overwritten in full
 //   nhp_probe_seq_major_pattern  the traffic of the transposing rotary kernel: a [rows, 128, s]
 //                             tensor (contiguous along s) is read in runs of 64 positions per
 //                             feature and written as [s, rows, 128], whole 256-byte head vectors,
 //                             through one 16-byte LDS store and load per chunk and one barrier;
 //                             the data is not transposed (what arrives where is not the point)
+//   nhp_probe_strided_runs    the traffic of the rotary kernels on q and k given as slices of one fused
+//                             projection buffer [.., 3 * d]: runs of 2^k chunks that lie a fixed distance
+//                             apart are read and written either to one contiguous output (one tensor per
+//                             launch: 256 of every 768 bytes at d = 128) or, split in halves, to two
+//                             contiguous outputs (q and k in one pass: 512 of every 768 bytes); two chunks
+//                             per thread, all loads first, as rope_lean_kernel is launched
 
 #include "common.hpp"
 
@@ -82,6 +90,37 @@ probe_causal_pattern_kernel(uint16_t* y, const uint16_t* x, uint32_t n)
     }
 }
 
+// The causal softmax backward's traffic: row q of every [n, n] matrix of g and of y is read up to the chunk
+// that holds column q, and the row of g is overwritten in full (in place, as the library's backward works).
+template <int K, int W>
+__global__ void __launch_bounds__(W * 64)
+probe_causal_bwd_pattern_kernel(uint16_t* g, const uint16_t* y, uint32_t n)
+{
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const uint32_t row = blockIdx.x;
+    const uint32_t q = row % n;
+    const int w = (int)((wave + blockIdx.x) % W);
+    uint16_t* gr = g + (size_t)row * n;
+    const uint16_t* yr = y + (size_t)row * n;
+    u32x4 a[K], b[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const uint32_t col = (uint32_t)((k * W + w) * 64 + lane) * 8u;
+        a[k] = u32x4{0, 0, 0, 0};
+        b[k] = u32x4{0, 0, 0, 0};
+        if (col < n && col <= q) {
+            a[k] = load16_stream(gr + col);
+            b[k] = load16_stream(yr + col);
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const uint32_t col = (uint32_t)((k * W + w) * 64 + lane) * 8u;
+        if (col < n) store16_stream(gr + col, a[k] ^ b[k]);
+    }
+}
+
 // One workgroup per (row, 64 positions): thread t loads 16 bytes (8 positions) of features
 // (t >> 3) + 32 p, p = 0..3, stages them in LDS, and stores the tile as 64 head vectors of 256 bytes.
 __global__ void __launch_bounds__(256)
@@ -106,11 +145,65 @@ probe_seq_major_kernel(uint16_t* out, const uint16_t* in, uint32_t rows, uint32_
     }
 }
 
+// Run r holds chunks [r * stride, r * stride + 2^LOG_RUN). SPLIT: the first half of every run goes to out0,
+// the second to out1 (each contiguous); otherwise the whole run to out0.
+template <int LOG_RUN, bool SPLIT>
+__global__ void __launch_bounds__(256)
+probe_strided_runs_kernel(u32x4* out0, u32x4* out1, const u32x4* in, uint32_t runs, uint32_t stride)
+{
+    constexpr uint32_t RUN = 1u << LOG_RUN, HALF = RUN / 2;
+    const uint32_t i0 = blockIdx.x * 512u + threadIdx.x;
+    u32x4 raw[2];
+    bool on[2];
+    size_t dst[2];
+    bool second[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+        const uint32_t i = i0 + u * 256u;
+        const uint32_t r = i >> LOG_RUN, c = i & (RUN - 1);
+        on[u] = r < runs;
+        const uint32_t rr = on[u] ? r : runs - 1;
+        raw[u] = load16_stream(in + (size_t)rr * stride + c);
+        second[u] = SPLIT && c >= HALF;
+        dst[u] = SPLIT ? (size_t)rr * HALF + (c & (HALF - 1)) : (size_t)rr * RUN + c;
+    }
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+        if (on[u]) store16_stream((second[u] ? out1 : out0) + dst[u], raw[u]);
+}
+
 }  // namespace nhp
 
 using namespace nhp;
 
 extern "C" {
+
+// `runs` runs of `run_chunks` (16 or 32) 16-byte chunks, `stride_chunks` apart in `in`. split = 0: copied to out0
+// back to back; split = 1: first halves to out0, second halves to out1.
+int nhp_probe_strided_runs(void* out0, void* out1, const void* in, int64_t runs, int run_chunks, int64_t stride_chunks,
+                           int split, void* stream)
+{
+    if (runs < 1 || (run_chunks != 16 && run_chunks != 32) || stride_chunks < run_chunks ||
+        stride_chunks >= ((int64_t)1 << 31) || runs * run_chunks >= ((int64_t)1 << 31))
+        return NHP_ERR_SHAPE;
+    if (!out0 || !in || (split && !out1)) return NHP_ERR_NULL;
+    const int64_t blocks = (runs * run_chunks + 511) / 512;
+    if (!grid_fits(blocks, 256)) return NHP_ERR_SHAPE;
+    launch_prepare();
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    u32x4* o0 = static_cast<u32x4*>(out0);
+    u32x4* o1 = static_cast<u32x4*>(out1);
+    const u32x4* ip = static_cast<const u32x4*>(in);
+    if (run_chunks == 16 && !split)
+        probe_strided_runs_kernel<4, false><<<(uint32_t)blocks, 256, 0, st>>>(o0, o1, ip, (uint32_t)runs, (uint32_t)stride_chunks);
+    else if (run_chunks == 32 && split)
+        probe_strided_runs_kernel<5, true><<<(uint32_t)blocks, 256, 0, st>>>(o0, o1, ip, (uint32_t)runs, (uint32_t)stride_chunks);
+    else if (run_chunks == 32)
+        probe_strided_runs_kernel<5, false><<<(uint32_t)blocks, 256, 0, st>>>(o0, o1, ip, (uint32_t)runs, (uint32_t)stride_chunks);
+    else
+        probe_strided_runs_kernel<4, true><<<(uint32_t)blocks, 256, 0, st>>>(o0, o1, ip, (uint32_t)runs, (uint32_t)stride_chunks);
+    return launch_result();
+}
 
 // Copies `bytes` (a multiple of 16) from in to out with workgroups of `threads` (64..1024) threads.
 int nhp_probe_copy(void* out, const void* in, int64_t bytes, int threads, void* stream)
@@ -168,6 +261,21 @@ int nhp_probe_causal_pattern(void* y, const void* x, int64_t batches, int64_t n,
         probe_causal_pattern_kernel<2, 2><<<rows, 128, 0, st>>>(static_cast<uint16_t*>(y), static_cast<const uint16_t*>(x), 2048u);
     else
         probe_causal_pattern_kernel<2, 8><<<rows, 512, 0, st>>>(static_cast<uint16_t*>(y), static_cast<const uint16_t*>(x), 8192u);
+    return launch_result();
+}
+
+// g (overwritten), y: [batches, n, n] 16-bit elements, n = 2048 (two waves of two chunks per lane) or 8192 (eight waves).
+int nhp_probe_causal_bwd_pattern(void* g, const void* y, int64_t batches, int64_t n, void* stream)
+{
+    if (batches < 1 || (n != 2048 && n != 8192) || batches * n >= ((int64_t)1 << 31)) return NHP_ERR_SHAPE;
+    if (!g || !y) return NHP_ERR_NULL;
+    launch_prepare();
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const uint32_t rows = (uint32_t)(batches * n);
+    if (n == 2048)
+        probe_causal_bwd_pattern_kernel<2, 2><<<rows, 128, 0, st>>>(static_cast<uint16_t*>(g), static_cast<const uint16_t*>(y), 2048u);
+    else
+        probe_causal_bwd_pattern_kernel<2, 8><<<rows, 512, 0, st>>>(static_cast<uint16_t*>(g), static_cast<const uint16_t*>(y), 8192u);
     return launch_result();
 }
 

@@ -394,16 +394,22 @@ rope_gather_kernel(RopePair pair, Tables tab, int cpr, int d2, int rpw)
 constexpr int kLeanThreads = 256;
 constexpr int kLeanU = 2;
 
-template <int DT, bool BWD, int LOG_CPR, bool FLAT, typename Tables>
+// JOINT: q and k are slices of one buffer with k's head vectors directly behind q's (k.in == q.in + d, equal
+// strides, equal row counts: how the attention layer slices them from its fused projection,
+// megatron/model/transformer.py:852-866). The two head vectors of a row are then read as one run of 2 * CPR
+// chunks, whose first half goes to q's output and whose second half to k's: one pass over the buffer instead
+// of two that each pick every third head vector. `ta` describes q (and both inputs), `tb.out` is k's output.
+template <int DT, bool BWD, int LOG_CPR, bool FLAT, typename Tables, bool JOINT = false>
 __global__ void __launch_bounds__(kLeanThreads)
 rope_lean_kernel(RopeTensor ta, RopeTensor tb, Tables tab, int rot_chunks)
 {
     constexpr int V = Elt<DT>::kVec;
     constexpr int CPR = 1 << LOG_CPR;
+    constexpr int LOG_RUN = LOG_CPR + (JOINT ? 1 : 0);  // chunks a row contributes: one head vector, or q's and k's
     constexpr int T = kLeanThreads, U = kLeanU;
     using S = typename Elt<DT>::storage;
     // both tensors' descriptions arrive with the kernel arguments; blockIdx.z picks one
-    const bool second = blockIdx.z != 0;
+    const bool second = !JOINT && blockIdx.z != 0;
     const S* const in = static_cast<const S*>(second ? tb.in : ta.in);
     S* const out = static_cast<S*>(second ? tb.out : ta.out);
     const int rows = second ? tb.rows : ta.rows;
@@ -416,8 +422,9 @@ rope_lean_kernel(RopeTensor ta, RopeTensor tb, Tables tab, int rot_chunks)
     __shared__ float tcos[Tables::kEvaluate ? kMaxRotary : 1], tsin[Tables::kEvaluate ? kMaxRotary : 1];
     stage_tables(tab, pos, rot_chunks * V, tcos, tsin);
     const int i0 = (int)blockIdx.x * (T * U) + (int)threadIdx.x;
-    const int c = i0 & (CPR - 1);
-    const int r0 = i0 >> LOG_CPR;
+    const int cj = i0 & ((1 << LOG_RUN) - 1);  // chunk within the row's run
+    const int c = cj & (CPR - 1);              // chunk within its head vector
+    const int r0 = i0 >> LOG_RUN;
     if (r0 < rows) {
         const int half = rot_chunks >> 1;
         const bool is_rot = c < rot_chunks;
@@ -427,13 +434,13 @@ rope_lean_kernel(RopeTensor ta, RopeTensor tb, Tables tab, int rot_chunks)
         const int tc = is_rot ? c : 0;
         const int ts = is_rot ? (BWD ? (first ? c + half : c - half) : c) : 0;
         // addresses first, then all loads back to back
-        const S* ip = in + pos * is_s + c * V;
-        S* op = out + pos * os_s + c * V;
+        const S* ip = in + pos * is_s + cj * V;
+        S* op = ((JOINT && cj >= CPR) ? static_cast<S*>(tb.out) : out) + pos * os_s + c * V;
         int64_t src[U], dst[U];
         bool on[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int r = r0 + u * (T >> LOG_CPR);
+            const int r = r0 + u * (T >> LOG_RUN);
             on[u] = r < rows;
             const int rr = on[u] ? r : rows - 1;
             if (FLAT) {
@@ -832,6 +839,19 @@ static RopeTensor rope_tensor(const RopeArgs& a)
 
 static bool rope_flat(const RopeArgs& a) { return (a.is[1] == a.h * a.is[2]) && (a.os[1] == a.h * a.os[2]); }
 
+// q and k as adjacent slices of one buffer: k's head vector of a row starts where q's ends, all input strides
+// and all output strides agree, same batch and head counts (no grouped-query attention).
+template <int DT>
+static bool rope_adjacent(const RopeArgs& q, const RopeArgs& k)
+{
+    using S = typename Elt<DT>::storage;
+    if (q.b != k.b || q.h != k.h || q.d != k.d) return false;
+    if (static_cast<const S*>(k.in) != static_cast<const S*>(q.in) + q.d) return false;
+    for (int i = 0; i < 3; ++i)
+        if (q.is[i] != k.is[i] || q.os[i] != k.os[i]) return false;
+    return 2 * q.b * q.h * (q.d / Elt<DT>::kVec) < ((int64_t)1 << 31);
+}
+
 // Launches the vector kernel for one tensor (b == nullptr) or for two tensors
 // that share s, d, d2 and the tables (q and k; their head counts may differ).
 // log2 of a power of two in 2..64, else -1
@@ -856,10 +876,27 @@ static int rope_launch_vec(const RopeArgs& a, const RopeArgs* b, const Tables& t
             const RopeTensor ta = rope_tensor(a);
             const RopeTensor tb = b ? rope_tensor(*b) : ta;
             const int64_t rows = most_rows;
-            const int64_t per_pos = (rows * cpr + kLeanThreads * kLeanU - 1) / (kLeanThreads * kLeanU);
-            const dim3 grid((uint32_t)per_pos, (uint32_t)a.s, b ? 2u : 1u);
             const bool flat = rope_flat(a) && (!b || rope_flat(*b));
             const int rot_chunks = (int)(a.d2 / V);
+            if (b && rope_adjacent<DT>(a, *b) && NHP_TUNED_INT("NHP_ROPE_JOINT", 1) != 0) {
+                // k's head vectors lie directly behind q's: one pass over runs of 2 * cpr chunks
+                const int64_t per_pos = (rows * 2 * cpr + kLeanThreads * kLeanU - 1) / (kLeanThreads * kLeanU);
+                const dim3 grid((uint32_t)per_pos, (uint32_t)a.s, 1u);
+#define LEAN(LC_)                                                                                             \
+    case LC_:                                                                                                 \
+        if (flat)                                                                                             \
+            rope_lean_kernel<DT, BWD, LC_, true, Tables, true><<<grid, kLeanThreads, 0, a.st>>>(ta, tb, tab, rot_chunks);  \
+        else                                                                                                  \
+            rope_lean_kernel<DT, BWD, LC_, false, Tables, true><<<grid, kLeanThreads, 0, a.st>>>(ta, tb, tab, rot_chunks); \
+        break;
+                switch (log_cpr) {
+                    LEAN(1) LEAN(2) LEAN(3) LEAN(4) LEAN(5) LEAN(6)
+                }
+#undef LEAN
+                return launch_result();
+            }
+            const int64_t per_pos = (rows * cpr + kLeanThreads * kLeanU - 1) / (kLeanThreads * kLeanU);
+            const dim3 grid((uint32_t)per_pos, (uint32_t)a.s, b ? 2u : 1u);
 #define LEAN(LC_)                                                                                             \
     case LC_:                                                                                                 \
         if (flat)                                                                                             \

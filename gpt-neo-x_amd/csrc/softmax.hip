@@ -39,6 +39,9 @@ namespace nhp {
 
 constexpr float kExpBias = 64.0f;
 constexpr float kMaskFill = -10000.0f;  // scaled_masked_softmax.h:180-184 of the reference
+// Row blocks of one head that are taken for every batch entry in turn when a bias tensor is shared by the
+// batch (batch_interleaved_block); 0: all row blocks of a matrix.
+constexpr int kBiasShareGroup = 0;
 
 template <int L, int K, int W, int BW>
 struct Geo {
@@ -143,6 +146,29 @@ __device__ __forceinline__ void locate_row(uint32_t block, uint32_t rows_per_mat
     }
 }
 
+// Workgroup order for a bias tensor [heads, n_q, n] that the `batch` entries of the batch share. In
+// row-major order the matrices that share a head's bias are a whole batch entry apart and every one of
+// them fetches that bias from HBM again. Here `group` consecutive row blocks of one head are taken for every
+// batch entry in turn (group * batch workgroups), then the head's next row blocks: workgroup id -> block
+// number of the row-major order. The library uses group = all row blocks of a matrix, i.e. the matrices
+// in the order (head, batch entry): the batch entries of a head then follow each other, each XCD sees the
+// same eighth of the bias rows again one matrix later and finds them in its L2 (2048 keys: 1 MiB per XCD
+// and head; the scores pass through with streaming hints), which took the fetched bytes from 1.8 x to
+// 1.03 x the algorithmic ones at [8 * 16, 2048, 2048] and 0-2 % off the time. Smaller groups save the same
+// bytes but interleave the DRAM streams of `batch` matrices and cost 10 % (groups of 8 or 64 blocks).
+__device__ __forceinline__ uint32_t batch_interleaved_block(uint32_t id, uint32_t blocks_per_matrix, uint32_t heads,
+                                                            uint32_t batch, uint32_t group)
+{
+    const uint32_t span = group * batch;
+    const uint32_t g = id / span;  // (head, row-block group), head-major
+    const uint32_t t = id - g * span;
+    const uint32_t j = t / group, r = t - j * group;
+    const uint32_t groups_per_matrix = blocks_per_matrix / group;
+    const uint32_t head = g / groups_per_matrix;
+    const uint32_t qg = g - head * groups_per_matrix;
+    return (j * heads + head) * blocks_per_matrix + qg * group + r;
+}
+
 // The columns of row q that take part in a causal softmax: [lo, hi) with
 // hi = min(q + 1, limit) and lo = max(0, q - window) (window = 0xffffffff: no
 // lower bound; limit = the number of real keys of the row's batch entry).
@@ -216,7 +242,7 @@ template <int DT, int L, int K, int W, int BW, int EXTRA>
 __global__ void __launch_bounds__((Geo<L, K, W, BW>::kThreads))
 causal_fwd_kernel(uint16_t* y, const uint16_t* x, float scale, uint32_t total_rows, uint32_t n, uint32_t window,
                   const float* slopes, const uint16_t* bias, const int32_t* key_lengths, uint32_t heads,
-                  uint16_t* dropped, DropoutKey dk, uint32_t zshift)
+                  uint16_t* dropped, DropoutKey dk, uint32_t zshift, uint32_t share_batch, uint32_t share_group)
 {
     using G = Geo<L, K, W, BW>;
     constexpr bool PER_HEAD = (EXTRA & kPerHead) != 0;
@@ -230,8 +256,12 @@ causal_fwd_kernel(uint16_t* y, const uint16_t* x, float scale, uint32_t total_ro
     // and wave i of every workgroup sits on the same SIMD of its CU.
     const int w = (W > 1) ? (int)((wave + blockIdx.x) % W) : 0;
 
+    // share_batch > 1 (only with a bias tensor): the batch entries of a head follow each other
+    uint32_t block = blockIdx.x;
+    if (PER_HEAD && share_batch > 1)
+        block = batch_interleaved_block(block, n / (uint32_t)G::kRowsPerBlock, heads, share_batch, share_group);
     uint32_t row, q, mat;
-    locate_row<G>(blockIdx.x, n, wave, lane, L, row, q, mat);
+    locate_row<G>(block, n, wave, lane, L, row, q, mat);
     const bool ok = row < total_rows;
     // columns [lo, hi) take part
     const Band band = causal_band(q, window, ok, (PER_HEAD && ok) ? key_limit(key_lengths, mat, heads) : 0xffffffffu);
@@ -438,7 +468,7 @@ masked_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
                   uint32_t bq_rows, uint32_t sq, uint32_t np, uint32_t n,
                   uint32_t heads_per_wave, uint32_t head_groups, int mask_per_batch, uint32_t row_blocks,
                   uint32_t tile, uint16_t* dropped, DropoutKey dk, const float* slopes, const uint16_t* bias,
-                  const int32_t* key_lengths)
+                  const int32_t* key_lengths, uint32_t share_batch, uint32_t share_group)
 {
     using G = Geo<L, K, W, BW>;
     __shared__ float lds[2][32];
@@ -451,13 +481,25 @@ masked_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
     // sequence), then the next head group on the same rows, then the next tile.
     // Neighbouring workgroups thus work on consecutive score rows (what HBM
     // likes best), and a mask row is used again one tile later, from L2.
+    // With a bias tensor shared by `share_batch` batch entries (a tile is then exactly one batch entry's
+    // row blocks): `share_group` row blocks of one head group for every batch entry in turn, so that the
+    // matrices sharing a bias follow each other (see batch_interleaved_block).
     const uint32_t id = blockIdx.x;
-    const uint32_t per_tile = tile * head_groups;
-    const uint32_t t = id / per_tile;
-    const uint32_t r = id - t * per_tile;
-    const uint32_t tile_rows = (t * tile + tile <= row_blocks) ? tile : row_blocks - t * tile;
-    const uint32_t hg = r / tile_rows;
-    const uint32_t rb = t * tile + (r - hg * tile_rows);
+    uint32_t hg, rb;
+    if (PER_HEAD && share_batch > 1) {
+        const uint32_t flat = batch_interleaved_block(id, tile, head_groups, share_batch, share_group);
+        const uint32_t m = flat / tile;  // batch entry * head_groups + head group
+        const uint32_t bi_ = m / head_groups;
+        hg = m - bi_ * head_groups;
+        rb = bi_ * tile + (flat - m * tile);
+    } else {
+        const uint32_t per_tile = tile * head_groups;
+        const uint32_t t = id / per_tile;
+        const uint32_t r = id - t * per_tile;
+        const uint32_t tile_rows = (t * tile + tile <= row_blocks) ? tile : row_blocks - t * tile;
+        hg = r / tile_rows;
+        rb = t * tile + (r - hg * tile_rows);
+    }
 
     uint32_t local;
     if constexpr (G::kRowsPerBlock == 1) {
@@ -505,6 +547,12 @@ masked_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
         live[k] = inb && !dead[k];
         any_dead = any_dead || dead[k];
     }
+    // Slots in which no lane of the wave has a masked key among its live columns skip the per-element
+    // selection below (most slots: a padding mask has one ragged chunk per row, a causal one per slot row).
+    bool mixed[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k)
+        mixed[k] = __builtin_amdgcn_ballot_w64(live[k] && (mb[k][0] | mb[k][1]) != 0u) != 0ull;
 
     const uint32_t h_begin = hg * heads_per_wave;
     const uint32_t h_end = (h_begin + heads_per_wave < np) ? h_begin + heads_per_wave : np;
@@ -575,11 +623,19 @@ masked_fwd_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, float sca
                         }
                     }
                 }
+                if (mixed[k]) {
 #pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const uint32_t byte = (mb[k][j >> 2] >> (8 * (j & 3))) & 0xffu;
-                    z[k][j] = (byte == 1u) ? kMaskFill : f[j] * scale;
-                    m = fmaxf(m, z[k][j]);
+                    for (int j = 0; j < 8; ++j) {
+                        const uint32_t byte = (mb[k][j >> 2] >> (8 * (j & 3))) & 0xffu;
+                        z[k][j] = (byte == 1u) ? kMaskFill : f[j] * scale;
+                        m = fmaxf(m, z[k][j]);
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        z[k][j] = f[j] * scale;
+                        m = fmaxf(m, z[k][j]);
+                    }
                 }
             }
         }
@@ -1040,18 +1096,25 @@ static int causal_fwd(void* y, const void* x, float scale, int64_t batches, int6
         const uint32_t blocks = (uint32_t)((rows + G::kRowsPerBlock - 1) / G::kRowsPerBlock); \
         if (!launch_fits(blocks, G::kThreads)) return NHP_ERR_SHAPE;                       \
         const bool per_head = slopes != nullptr || bp != nullptr || kl != nullptr;         \
+        /* a bias shared by several batch entries: their workgroups are interleaved (whole groups only) */ \
+        uint32_t sgroup = (uint32_t)NHP_TUNED_INT("NHP_BIAS_GROUP", kBiasShareGroup);        \
+        if (sgroup == 0) sgroup = (uint32_t)(n / G::kRowsPerBlock);                        \
+        uint32_t sbatch = 0;                                                               \
+        if (bp != nullptr && heads > 0 && batches / heads > 1 && sgroup > 0 && n % G::kRowsPerBlock == 0 && \
+            (n / G::kRowsPerBlock) % sgroup == 0 && NHP_TUNED_INT("NHP_BIAS_SHARE", 1) != 0)   \
+            sbatch = (uint32_t)(batches / heads);                                          \
         if (dp != nullptr && per_head)                                                     \
             causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves, kPerHeadDropout><<<blocks, G::kThreads, 0, st>>>( \
-                yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, slopes, bp, kl, heads, dp, dk, zshift); \
+                yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, slopes, bp, kl, heads, dp, dk, zshift, sbatch, sgroup); \
         else if (dp != nullptr)                                                            \
             causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves, kDropout><<<blocks, G::kThreads, 0, st>>>( \
-                yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, nullptr, nullptr, nullptr, 1, dp, dk, zshift); \
+                yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, nullptr, nullptr, nullptr, 1, dp, dk, zshift, 0, 0); \
         else if (per_head)                                                                 \
             causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves, kPerHead><<<blocks, G::kThreads, 0, st>>>( \
-                yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, slopes, bp, kl, heads, nullptr, dk, zshift); \
+                yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, slopes, bp, kl, heads, nullptr, dk, zshift, sbatch, sgroup); \
         else                                                                               \
             causal_fwd_kernel<DT, L_, K_, W_, kBlockWaves, kPlain><<<blocks, G::kThreads, 0, st>>>( \
-                yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, nullptr, nullptr, nullptr, 1, nullptr, dk, zshift); \
+                yp, xp, scale, (uint32_t)rows, (uint32_t)n, window, nullptr, nullptr, nullptr, 1, nullptr, dk, zshift, 0, 0); \
     }
         NHP_FOR_PLAN(p);
 #undef CALL
@@ -1142,7 +1205,7 @@ static int masked_fwd(void* y, const void* x, const uint8_t* mask, float scale, 
 #define LAUNCH_MASKED(L_, K_, W_, DROP_, PH_)                                                         \
     masked_fwd_kernel<DT, L_, K_, W_, kBlockWaves, DROP_, PH_><<<(uint32_t)(rb * hgs), Geo<L_, K_, W_, kBlockWaves>::kThreads, 0, st>>>( \
         yp, xp, mask, scale, (uint32_t)bq_rows, (uint32_t)sq, (uint32_t)np, (uint32_t)n, hpw, hgs, per_batch, \
-        (uint32_t)rb, (uint32_t)tile, DROP_ ? dp : nullptr, dk, ex.slopes, bp, ex.key_lengths)
+        (uint32_t)rb, (uint32_t)tile, DROP_ ? dp : nullptr, dk, ex.slopes, bp, ex.key_lengths, sbatch, sgroup)
 #define CALL(L_, K_, W_)                                                                   \
     {                                                                                      \
         using G = Geo<L_, K_, W_, kBlockWaves>;                                            \
@@ -1153,6 +1216,13 @@ static int masked_fwd(void* y, const void* x, const uint8_t* mask, float scale, 
         int64_t tile = NHP_TUNED_INT("NHP_MASK_TILE", (int)((sq + G::kRowsPerBlock - 1) / G::kRowsPerBlock)); \
         if (tile < 1) tile = 1;                                                            \
         if (tile > rb) tile = rb;                                                          \
+        /* a bias shared by several batch entries: their workgroups are interleaved (tile = one batch entry) */ \
+        uint32_t sgroup = (uint32_t)NHP_TUNED_INT("NHP_BIAS_GROUP", kBiasShareGroup);        \
+        if (sgroup == 0) sgroup = (uint32_t)tile;                                          \
+        uint32_t sbatch = 0;                                                               \
+        if (bp != nullptr && b > 1 && sgroup > 0 && sq % G::kRowsPerBlock == 0 && tile == sq / G::kRowsPerBlock && \
+            tile % sgroup == 0 && NHP_TUNED_INT("NHP_BIAS_SHARE", 1) != 0)                  \
+            sbatch = (uint32_t)b;                                                          \
         if (dp != nullptr && ex.any())                                                     \
             LAUNCH_MASKED(L_, K_, W_, true, true);                                                     \
         else if (dp != nullptr)                                                            \

@@ -137,6 +137,31 @@ def test_additive_bias_forward_vs_oracle(hotpath, dtype, s, window, with_alibi):
     assert torch.equal(util.raw_bits(via_abi), util.raw_bits(got))
 
 
+@pytest.mark.parametrize("b,heads,s", [(3, 2, 512), (5, 1, 1024), (2, 3, 2048), (3, 2, 4096), (3, 2, 200)])
+def test_bias_shared_by_the_batch_workgroup_order(hotpath, b, heads, s):
+    """With a bias tensor and more than one batch entry the forward kernels take the matrices in the order
+    (head, batch entry), so that the matrices sharing a head's bias follow each other and find it in cache;
+    batch sizes that are not powers of two, one head, rows of several waves, and a row count that does not
+    fill its last workgroup (plain order). Every matrix against the oracle, causal and padding-mask kernel."""
+    import scaled_masked_softmax_cuda as masked_ext
+    import scaled_upper_triang_masked_softmax_cuda as ext
+
+    dtype, scale = torch.bfloat16, 0.11
+    print(f"shared bias b={b} heads={heads} s={s}", flush=True)
+    x = util.randn((b * heads, s, s), dtype, seed=s + b, std=2.0)
+    bias = util.randn((heads, s, s), dtype, seed=s + 1, std=1.5)
+    want = oracle.causal_softmax_fwd(x, scale, bias=bias)
+    got = ext.forward(x.to(DEV), scale, None, None, bias.to(DEV)).cpu()
+    util.assert_ulp_close(got, want, 2, "causal, shared bias")
+    sq = s // 8
+    xm = util.randn((b, heads, sq, s), dtype, seed=s + b + 1, std=2.0)
+    bm = util.randn((heads, sq, s), dtype, seed=s + 2, std=1.5)
+    mask = util.padding_mask(b, sq, s, seed=s, lo=s // 2)
+    want = oracle.masked_softmax_fwd(xm, mask, scale, None, bm, None)
+    got = masked_ext.forward(xm.to(DEV), mask.to(DEV), scale, None, bm.to(DEV)).cpu()
+    util.assert_ulp_close(got, want, 2, "padding mask, shared bias")
+
+
 def test_module_with_relative_position_bias_and_its_gradient():
     """FusedScaleMaskSoftmax(input, mask, bias): probabilities and the gradients of the
     scores and of the (batch-shared, learned) bias against autograd through the unfused path."""

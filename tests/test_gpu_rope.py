@@ -199,6 +199,58 @@ def test_rope_qk_single_launch_equals_two_calls(hotpath, shape, dtype):
             assert torch.equal(util.raw_bits(got_k.cpu()), util.raw_bits(oracle.rope_cached(k.cpu(), cos.cpu(), sin.cpu(), backward, transpose)))
 
 
+# (s, b, h, d, d2): head vectors of 2..64 chunks, rows that do not fill the last workgroup, partial rotary dimensions
+FUSED_QKV = [(16, 2, 8, 128, 128), (16, 2, 8, 128, 32), (5, 3, 7, 64, 64), (9, 1, 3, 32, 16), (3, 2, 5, 16, 16),
+             (4, 2, 3, 256, 64), (3, 1, 2, 512, 512), (6, 2, 33, 128, 64), (64, 4, 16, 128, 128)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("shape", FUSED_QKV, ids=lambda s: "x".join(map(str, s)))
+def test_rope_qk_sliced_from_a_fused_projection(hotpath, shape, dtype):
+    """q and k the way the attention layer slices them (megatron/model/transformer.py:852-866): last-dimension
+    slices [..., :d] and [..., d:2d] of one [s, b, h, 3d] buffer, so k's head vector lies directly behind q's.
+    The two-tensor entry points then read each (q|k) pair as one run; results are the oracle's bit for bit, in
+    both directions and output layouts, with cached tables and with angles. Slices in another order, or with
+    unequal strides, take the ordinary two-tensor launch and give the same bits."""
+    s, b, h, d, d2 = shape
+    say(f"rope q,k sliced from a fused buffer {shape} {dtype}")
+    buf = util.randn((s, b, h, 3 * d), dtype, seed=s + d + d2).to(DEV)
+    q, k, v = buf[..., :d], buf[..., d:2 * d], buf[..., 2 * d:]
+    assert k.data_ptr() == q.data_ptr() + d * buf.element_size() and q.stride() == k.stride()
+    cos, sin, ang = generic_tables(d2, s, dtype, seed=d2)
+    cos_d, sin_d, ang_d = cos.to(DEV), sin.to(DEV), ang.to(DEV)
+    L = hotpath.lib()
+    code = hotpath.dtype_code(q, "t")
+    for backward in (False, True):
+        for transpose in (False, True):
+            want_q = oracle.rope_cached(q.cpu(), cos, sin, backward, transpose)
+            want_k = oracle.rope_cached(k.cpu(), cos, sin, backward, transpose)
+            for first, second, want_first, want_second in ((q, k, want_q, want_k), (k, q, want_k, want_q), (k, v, want_k, None)):
+                got_a, got_b = util._rope_out(first, transpose), util._rope_out(second, transpose)
+                fn = L.nhp_rope_cached_qk_bwd if backward else L.nhp_rope_cached_qk_fwd
+                rc = fn(got_a.data_ptr(), got_b.data_ptr(), first.data_ptr(), second.data_ptr(), cos_d.data_ptr(),
+                        sin_d.data_ptr(), s, b, h, h, d, d2, hotpath.strides4(first), hotpath.strides4(second),
+                        hotpath.strides4(got_a), hotpath.strides4(got_b), code, code, None)
+                assert rc == 0, L.nhp_status_string(rc)
+                torch.cuda.synchronize()
+                assert torch.equal(util.raw_bits(got_a.cpu()), util.raw_bits(want_first)), (backward, transpose)
+                if want_second is not None:
+                    assert torch.equal(util.raw_bits(got_b.cpu()), util.raw_bits(want_second)), (backward, transpose)
+            # the angles variant: the same bits as its single-tensor entry point (same device sine and cosine)
+            got_a, got_b = util._rope_out(q, transpose), util._rope_out(k, transpose)
+            fn = L.nhp_rope_freqs_qk_bwd if backward else L.nhp_rope_freqs_qk_fwd
+            rc = fn(got_a.data_ptr(), got_b.data_ptr(), q.data_ptr(), k.data_ptr(), ang_d.data_ptr(), s, b, h, h, d, d2,
+                    hotpath.strides4(q), hotpath.strides4(k), hotpath.strides4(got_a), hotpath.strides4(got_b), code, None)
+            assert rc == 0, L.nhp_status_string(rc)
+            torch.cuda.synchronize()
+            assert torch.equal(util.raw_bits(got_a.cpu()),
+                               util.raw_bits(util.abi_rope_freqs(hotpath, q, ang_d, backward, transpose).cpu()))
+            assert torch.equal(util.raw_bits(got_b.cpu()),
+                               util.raw_bits(util.abi_rope_freqs(hotpath, k, ang_d, backward, transpose).cpu()))
+    # the buffer itself is untouched, v included
+    assert torch.equal(util.raw_bits(buf.cpu()), util.raw_bits(util.randn((s, b, h, 3 * d), dtype, seed=s + d + d2)))
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 @pytest.mark.parametrize("offset", [0, 5])
 def test_fused_qk_function_matches_eager_apply_with_offset(dtype, offset):
