@@ -124,21 +124,34 @@ def rope_bytes(s, b, h, d, d2, e=2, e_cs=2):
 
 class Timer:
     """Event-times named kernels on the current stream. `only` restricts the
-    bracketing to one name (the others run unbracketed, without event records)."""
+    bracketing to one name (the others run unbracketed, without event records).
+    `chain`: a kernel that directly follows a bracketed one takes that bracket's closing
+    event as its opening event (one event record between two kernels instead of two: every
+    record is a packet the GPU has to process between them, about 2 us). The workload
+    must then issue nothing else between two run() calls; `unchain()` says that it did."""
 
-    def __init__(self, torch, only=None):
+    def __init__(self, torch, only=None, chain=False):
         self.torch = torch
         self.only = only
+        self.chain = chain
+        self.last = None
         self.pairs = {}
+
+    def unchain(self):
+        self.last = None
 
     def run(self, name, fn):
         if self.only is not None and name != self.only:
+            self.last = None
             return fn()
-        a = self.torch.cuda.Event(enable_timing=True)
+        a = self.last if (self.chain and self.last is not None) else None
+        if a is None:
+            a = self.torch.cuda.Event(enable_timing=True)
+            a.record()
         b = self.torch.cuda.Event(enable_timing=True)
-        a.record()
         out = fn()
         b.record()
+        self.last = b
         self.pairs.setdefault(name, []).append((a, b))
         return out
 
@@ -152,6 +165,7 @@ class Timer:
 
     def reset(self):
         self.pairs = {}
+        self.last = None
 
 
 def grad_ring(torch, pristine, launches):
@@ -239,6 +253,7 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False, launc
             ring_state["i"] += 1
             if fresh_dy:
                 g.copy_(dy0)
+                t.unchain()
             # in place on the gradient buffer, as the reference does
             t.run("causal_softmax_bwd", lambda: causal_ext.backward(g, y, scale))
             t.run("rope_bwd", rope_b)
@@ -1011,12 +1026,14 @@ def measure_workload(name, torch, dev, steps, warmup):
     import gc
 
     step, kernel_bytes, other, _, dtype, cfg = make_workload(name, torch, dev, launches=warmup + steps)
-    timer = Timer(torch)
+    timer = Timer(torch, chain=True)
     for _ in range(warmup):
+        timer.unchain()  # a step may begin with work of its own (picking buffers, a copy)
         step(timer)
     torch.cuda.synchronize()
     timer.reset()
     for _ in range(steps):
+        timer.unchain()
         step(timer)
     torch.cuda.synchronize()
     avg = timer.averages_ms()

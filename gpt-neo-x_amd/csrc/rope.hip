@@ -11,20 +11,20 @@
 // element i with i + d2/2, i.e. a chunk with the chunk d2/(2V) lanes away in
 // the same wave; the partner's data is fetched with ds_bpermute (no memory
 // traffic). Chunks of the pass-through tail are copied by their lanes.
-//   rope_lean_kernel: head vectors of a power-of-two number of chunks. Two
-//     chunks per thread, no loop, every load issued before the first wait: the
-//     shape a plain streaming copy runs fastest in on this GPU.
-//   rope_vec_kernel: other head sizes with unit feature stride. A workgroup
-//     stays on one sequence position and walks over the (batch, head) rows,
-//     re-using the cos/sin values it loaded once.
+//   rope_lean_kernel: two chunks per thread, no loop, every load issued before
+//     the first wait: the shape a plain streaming copy runs fastest in on this
+//     GPU. Head vectors of any number of chunks up to 64.
+//   rope_vec_kernel: what the lean kernel's grid cannot hold (more than 65535
+//     positions) and calls without a rotary part. A workgroup stays on one sequence
+//     position and walks over the (batch, head) rows, re-using the cos/sin values it loaded once.
 //   When the angles are given instead of cached tables, a workgroup of either
 //   kernel first evaluates sin and cos of its position, one rotary feature per
 //   thread, into LDS (sincosf costs a few hundred instructions: evaluated per
 //   lane it made these kernels compute-bound).
 //
-//   rope_gather_kernel: rotary dimensions whose half is not a whole number of
-//     chunks (24 of 96, 20 of 80) or unaligned tables; partner elements are
-//     picked from LDS one by one.
+//   Rotary dimensions whose half is not a whole number of chunks (24 of 96,
+//     20 of 80) or unaligned tables: partner elements are picked from LDS one by
+//     one, by a variant of the lean kernel (rope_gather_kernel beyond its grid).
 //
 // Transposing kernel, for 16-bit inputs that are contiguous along the sequence
 // instead of along the features (see rope_tr_kernel). Everything else (odd
@@ -379,34 +379,42 @@ rope_gather_kernel(RopePair pair, Tables tab, int cpr, int d2, int rpw)
 
 // ---------------------------------------------------------------------------
 // Lean vector kernel
-//   grid  = (ceil(rows * CPR / 512), s, tensors), block = 256 threads
-//   thread t of workgroup x owns chunks x * 512 + t and x * 512 + 256 + t of
-//   position blockIdx.y, counted over the position's rows * CPR chunks;
-//   CPR = 2^LOG_CPR chunks per head vector, so both chunks have the same
-//   place in their head vectors and share one pair of table chunks.
+//   grid  = (ceil(rows / (8 * RPW)), s, tensors), block = 256 threads = 4 waves
+//   A head vector is CPR chunks; a wave holds RPW = 64 / CPR whole head vectors (its last 64 - RPW * CPR lanes
+//   idle when CPR is not a power of two: 4 of 64 at 12 chunks), consecutive waves consecutive rows, and every
+//   thread owns the same chunk of two rows, 4 * RPW rows apart, so that both share one pair of table chunks.
+//   LOG_CPR >= 0: CPR = 2^LOG_CPR at compile time; LOG_CPR < 0: any CPR <= 64, passed as an argument.
 // Consecutive workgroups sweep consecutive memory. Every load (tables, then
 // data) is issued before anything waits: lanes outside the rotary part load
 // table chunk 0 and discard the result, a second row beyond the end re-loads
 // the last row and is not stored, so that no load sits in a divergent region
 // (where the compiler would have to wait for it on the spot, or would sink it
 // behind the wait for the data). Needs d2 > 0.
-// ---------------------------------------------------------------------------
-constexpr int kLeanThreads = 256;
-constexpr int kLeanU = 2;
-
+//
 // JOINT: q and k are slices of one buffer with k's head vectors directly behind q's (k.in == q.in + d, equal
 // strides, equal row counts: how the attention layer slices them from its fused projection,
 // megatron/model/transformer.py:852-866). The two head vectors of a row are then read as one run of 2 * CPR
 // chunks, whose first half goes to q's output and whose second half to k's: one pass over the buffer instead
 // of two that each pick every third head vector. `ta` describes q (and both inputs), `tb.out` is k's output.
-template <int DT, bool BWD, int LOG_CPR, bool FLAT, typename Tables, bool JOINT = false>
+//
+// GATHER: rotary dimensions whose half is not a whole number of chunks (24 of 96, 20 of 80: a quarter of
+// the head sizes 96 and 80), or tables that are not 16-byte aligned. The partner of element i, i +- d2/2, may
+// sit anywhere in up to two other chunks of the head vector, so every lane puts its chunks into LDS and
+// picks its partner elements from there one by one (the lanes of a head vector share a wave, whose LDS
+// accesses execute in order: a wave-level fence is all the synchronisation needed); cos and sin of the
+// position are staged in LDS by the workgroup whatever their source. `rot_arg` is then d2, else d2 / V.
+// ---------------------------------------------------------------------------
+constexpr int kLeanThreads = 256;
+constexpr int kLeanU = 2;
+
+template <int DT, bool BWD, int LOG_CPR, bool FLAT, typename Tables, bool JOINT = false, bool GATHER = false>
 __global__ void __launch_bounds__(kLeanThreads)
-rope_lean_kernel(RopeTensor ta, RopeTensor tb, Tables tab, int rot_chunks)
+rope_lean_kernel(RopeTensor ta, RopeTensor tb, Tables tab, int rot_arg, int cpr_arg)
 {
+    static_assert(!(JOINT && (GATHER || LOG_CPR < 0)), "the joint variant exists for power-of-two head vectors only");
     constexpr int V = Elt<DT>::kVec;
-    constexpr int CPR = 1 << LOG_CPR;
-    constexpr int LOG_RUN = LOG_CPR + (JOINT ? 1 : 0);  // chunks a row contributes: one head vector, or q's and k's
-    constexpr int T = kLeanThreads, U = kLeanU;
+    constexpr int U = kLeanU;
+    constexpr bool STAGED = GATHER || Tables::kEvaluate;  // cos and sin come from LDS
     using S = typename Elt<DT>::storage;
     // both tensors' descriptions arrive with the kernel arguments; blockIdx.z picks one
     const bool second = !JOINT && blockIdx.z != 0;
@@ -417,30 +425,34 @@ rope_lean_kernel(RopeTensor ta, RopeTensor tb, Tables tab, int rot_chunks)
     const int64_t is_s = second ? tb.is_s : ta.is_s, is_b = second ? tb.is_b : ta.is_b, is_h = second ? tb.is_h : ta.is_h;
     const int64_t os_s = second ? tb.os_s : ta.os_s, os_b = second ? tb.os_b : ta.os_b, os_h = second ? tb.os_h : ta.os_h;
 
+    const int cpr = LOG_CPR >= 0 ? (1 << (LOG_CPR >= 0 ? LOG_CPR : 0)) : cpr_arg;  // chunks per head vector
+    const int run = JOINT ? 2 * cpr : cpr;  // chunks a row contributes: one head vector, or q's and k's
+    const int rpw = 64 / run;               // rows per wave
     const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int rl = lane / run;              // row within the wave
+    const int cj = lane - rl * run;         // chunk within the row's run
+    const int c = JOINT ? (cj & (cpr - 1)) : cj;  // chunk within its head vector
     const int64_t pos = blockIdx.y;
-    __shared__ float tcos[Tables::kEvaluate ? kMaxRotary : 1], tsin[Tables::kEvaluate ? kMaxRotary : 1];
-    stage_tables(tab, pos, rot_chunks * V, tcos, tsin);
-    const int i0 = (int)blockIdx.x * (T * U) + (int)threadIdx.x;
-    const int cj = i0 & ((1 << LOG_RUN) - 1);  // chunk within the row's run
-    const int c = cj & (CPR - 1);              // chunk within its head vector
-    const int r0 = i0 >> LOG_RUN;
-    if (r0 < rows) {
-        const int half = rot_chunks >> 1;
-        const bool is_rot = c < rot_chunks;
-        const bool first = c < half;
-        const int partner_lane = is_rot ? (first ? lane + half : lane - half) : lane;
-        // cos of the own chunk; sin of the own chunk (forward) or of the partner's (backward)
-        const int tc = is_rot ? c : 0;
-        const int ts = is_rot ? (BWD ? (first ? c + half : c - half) : c) : 0;
+    const int d2 = GATHER ? rot_arg : rot_arg * V;
+    __shared__ float tcos[STAGED ? kMaxRotary : 1], tsin[STAGED ? kMaxRotary : 1];
+    __shared__ u32x4 stage[GATHER ? U : 1][GATHER ? kLeanThreads : 1];
+    if constexpr (GATHER) {
+        for (int i = (int)threadIdx.x; i < d2; i += kLeanThreads) tab.get(pos, i, tcos[i], tsin[i]);
+        __syncthreads();
+    } else {
+        stage_tables(tab, pos, d2, tcos, tsin);
+    }
+    const int r0 = ((int)blockIdx.x * (4 * U) + wave) * rpw + rl;
+    if (rl < rpw && r0 < rows) {
         // addresses first, then all loads back to back
         const S* ip = in + pos * is_s + cj * V;
-        S* op = ((JOINT && cj >= CPR) ? static_cast<S*>(tb.out) : out) + pos * os_s + c * V;
+        S* op = ((JOINT && cj >= cpr) ? static_cast<S*>(tb.out) : out) + pos * os_s + c * V;
         int64_t src[U], dst[U];
         bool on[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int r = r0 + u * (T >> LOG_RUN);
+            const int r = r0 + u * 4 * rpw;
             on[u] = r < rows;
             const int rr = on[u] ? r : rows - 1;
             if (FLAT) {
@@ -453,34 +465,97 @@ rope_lean_kernel(RopeTensor ta, RopeTensor tb, Tables tab, int rot_chunks)
                 dst[u] = bi * os_b + hi * os_h;
             }
         }
-        float cv[V], sv[V], unused[V];
-        table_chunk<DT>(tab, pos, tc * V, tcos, tsin, cv, unused);
-        table_chunk<DT>(tab, pos, ts * V, tcos, tsin, unused, sv);
-        u32x4 raw[U];
+        if constexpr (!GATHER) {
+            const int rot_chunks = rot_arg;
+            const int half = rot_chunks >> 1;
+            const bool is_rot = c < rot_chunks;
+            const bool first = c < half;
+            const int partner_lane = is_rot ? (first ? lane + half : lane - half) : lane;
+            // cos of the own chunk; sin of the own chunk (forward) or of the partner's (backward)
+            const int tc = is_rot ? c : 0;
+            const int ts = is_rot ? (BWD ? (first ? c + half : c - half) : c) : 0;
+            float cv[V], sv[V], unused[V];
+            table_chunk<DT>(tab, pos, tc * V, tcos, tsin, cv, unused);
+            table_chunk<DT>(tab, pos, ts * V, tcos, tsin, unused, sv);
+            u32x4 raw[U];
 #pragma unroll
-        for (int u = 0; u < U; ++u) raw[u] = load16_stream(ip + src[u]);
-        // forward: first half subtracts, backward: second half subtracts
-        const bool negate = BWD ? !first : first;
+            for (int u = 0; u < U; ++u) raw[u] = load16_stream(ip + src[u]);
+            // forward: first half subtracts, backward: second half subtracts
+            const bool negate = BWD ? !first : first;
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            u32x4 praw;
+            for (int u = 0; u < U; ++u) {
+                u32x4 praw;
 #pragma unroll
-            for (int k = 0; k < 4; ++k)
-                praw[k] = (uint32_t)__builtin_amdgcn_ds_bpermute(partner_lane << 2, (int)raw[u][k]);
-            float x[V], pr[V], y[V];
-            chunk_to_float<DT>(raw[u], x);
-            chunk_to_float<DT>(praw, pr);
+                for (int k = 0; k < 4; ++k)
+                    praw[k] = (uint32_t)__builtin_amdgcn_ds_bpermute(partner_lane << 2, (int)raw[u][k]);
+                float x[V], pr[V], y[V];
+                chunk_to_float<DT>(raw[u], x);
+                chunk_to_float<DT>(praw, pr);
 #pragma unroll
-            for (int v = 0; v < V; ++v)
-                y[v] = negate ? rot<DT, true>(x[v], cv[v], pr[v], sv[v]) : rot<DT>(x[v], cv[v], pr[v], sv[v]);
-            const u32x4 rotated = float_to_chunk<DT>(y);
-            u32x4 res;
+                for (int v = 0; v < V; ++v)
+                    y[v] = negate ? rot<DT, true>(x[v], cv[v], pr[v], sv[v]) : rot<DT>(x[v], cv[v], pr[v], sv[v]);
+                const u32x4 rotated = float_to_chunk<DT>(y);
+                u32x4 res;
 #pragma unroll
-            for (int k = 0; k < 4; ++k) res[k] = is_rot ? rotated[k] : raw[u][k];
-            // The value passes through an opaque statement: without it the compiler folds the select into
-            // the store and the store loses its non-temporal hint.
-            asm volatile("" : "+v"(res));
-            if (on[u]) store16_stream(op + dst[u], res);
+                for (int k = 0; k < 4; ++k) res[k] = is_rot ? rotated[k] : raw[u][k];
+                // The value passes through an opaque statement: without it the compiler folds the select into
+                // the store and the store loses its non-temporal hint.
+                asm volatile("" : "+v"(res));
+                if (on[u]) store16_stream(op + dst[u], res);
+            }
+        } else {
+            u32x4 raw[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) raw[u] = load16_stream(ip + src[u]);
+            // per element of the own chunk: cos, the sine the formula takes (its own forward, the partner's
+            // backward), the sign, and where the partner sits among the staged elements of the head vector
+            const int h2 = d2 >> 1;
+            const int vec0 = ((int)threadIdx.x - c) * V;  // first staged element of this lane's head vector
+            float cv[V], sv[V];
+            int from[V];
+            bool neg[V];
+            bool any = false;
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                const int i = c * V + v;
+                const bool rot_on = i < d2;
+                const bool first = i < h2;
+                const int pi = first ? i + h2 : i - h2;
+                cv[v] = rot_on ? tcos[i] : 0.0f;
+                sv[v] = rot_on ? tsin[BWD ? pi : i] : 0.0f;
+                neg[v] = BWD ? !first : first;
+                from[v] = rot_on ? vec0 + pi : -1;
+                any = any || rot_on;
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) stage[u][threadIdx.x] = raw[u];
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                u32x4 res = raw[u];
+                if (any) {
+                    const S* staged = reinterpret_cast<const S*>(&stage[u][0]);
+                    float x[V], y[V];
+                    chunk_to_float<DT>(raw[u], x);
+#pragma unroll
+                    for (int v = 0; v < V; ++v) {
+                        y[v] = x[v];
+                        if (from[v] >= 0) {
+                            float pr;
+                            if constexpr (DT == NHP_F32)
+                                pr = staged[from[v]];
+                            else
+                                pr = Half2<DT>::from_bits(staged[from[v]]);
+                            y[v] = neg[v] ? rot<DT, true>(x[v], cv[v], pr, sv[v]) : rot<DT>(x[v], cv[v], pr, sv[v]);
+                        }
+                    }
+                    res = float_to_chunk<DT>(y);
+                }
+                asm volatile("" : "+v"(res));
+                if (on[u]) store16_stream(op + dst[u], res);
+            }
         }
     }
 }
@@ -662,9 +737,12 @@ rope_tr_kernel(RopeTensor T, Tables tab, int s, int cpr, int d2, int row_chunks,
             // Partial rotary dimension: rotate in place in LDS, one work item per pair of chunks (c, c + half), so
             // that every lane that does arithmetic is busy; then copy the tile out whole head vectors at a time
             // (storing the rotated chunks straight from these lanes, 32 bytes at a time, measured 20 % slower).
+            // Consecutive work items take consecutive tile rows (positions) of one chunk pair: the rows of the
+            // tile are 4 banks apart, so the 8 lanes of a 16-byte LDS access pass fall on distinct banks (with
+            // the pair index running fastest two neighbouring rows overlapped in half of their banks).
             for (int idx = tid; idx < kTrTile * half; idx += 256) {
-                const int row = idx / half;
-                const int c = idx - row * half;
+                const int c = idx / kTrTile;
+                const int row = idx - c * kTrTile;
                 const int pc = c + half;
                 const int pos = s0 + row;
                 if (pos >= s) continue;
@@ -672,7 +750,7 @@ rope_tr_kernel(RopeTensor T, Tables tab, int s, int cpr, int d2, int row_chunks,
                 u32x4* pa = &tile[row * row_chunks + (c ^ swz)];
                 u32x4* pb = &tile[row * row_chunks + (pc ^ swz)];
                 float ca[V], sa[V], cb[V], sb[V], xa[V], xb[V], ya[V], yb[V];
-                fetch(row, pos, c, ca, sa);
+                fetch(row, pos, c, ca, sa);  // requesting these before the barrier, with the data, measured 3 % slower
                 fetch(row, pos, pc, cb, sb);
                 chunk_to_float<DT>(*pa, xa);
                 chunk_to_float<DT>(*pb, xb);
@@ -871,41 +949,43 @@ static int rope_launch_vec(const RopeArgs& a, const RopeArgs* b, const Tables& t
     {
         const int log_cpr = log2_chunks(cpr);
         const int64_t most_rows = (b && b->b * b->h > a.b * a.h) ? b->b * b->h : a.b * a.h;
-        // grid.y holds the position; chunk numbers inside a position are 32-bit
-        if (log_cpr > 0 && a.d2 > 0 && a.s <= 65535 && most_rows * cpr < ((int64_t)1 << 31)) {
+        // grid.y holds the position; row numbers inside a position are 32-bit
+        if (cpr >= 2 && cpr <= 64 && a.d2 > 0 && a.s <= 65535 && most_rows * cpr < ((int64_t)1 << 31)) {
             const RopeTensor ta = rope_tensor(a);
             const RopeTensor tb = b ? rope_tensor(*b) : ta;
             const int64_t rows = most_rows;
             const bool flat = rope_flat(a) && (!b || rope_flat(*b));
             const int rot_chunks = (int)(a.d2 / V);
-            if (b && rope_adjacent<DT>(a, *b) && NHP_TUNED_INT("NHP_ROPE_JOINT", 1) != 0) {
+            if (log_cpr > 0 && log_cpr < 6 && b && rope_adjacent<DT>(a, *b)) {
                 // k's head vectors lie directly behind q's: one pass over runs of 2 * cpr chunks
-                const int64_t per_pos = (rows * 2 * cpr + kLeanThreads * kLeanU - 1) / (kLeanThreads * kLeanU);
-                const dim3 grid((uint32_t)per_pos, (uint32_t)a.s, 1u);
+                const int64_t rows_per_wg = (int64_t)4 * kLeanU * (64 / (2 * cpr));
+                const dim3 grid((uint32_t)((rows + rows_per_wg - 1) / rows_per_wg), (uint32_t)a.s, 1u);
 #define LEAN(LC_)                                                                                             \
     case LC_:                                                                                                 \
         if (flat)                                                                                             \
-            rope_lean_kernel<DT, BWD, LC_, true, Tables, true><<<grid, kLeanThreads, 0, a.st>>>(ta, tb, tab, rot_chunks);  \
+            rope_lean_kernel<DT, BWD, LC_, true, Tables, true><<<grid, kLeanThreads, 0, a.st>>>(ta, tb, tab, rot_chunks, cpr);  \
         else                                                                                                  \
-            rope_lean_kernel<DT, BWD, LC_, false, Tables, true><<<grid, kLeanThreads, 0, a.st>>>(ta, tb, tab, rot_chunks); \
+            rope_lean_kernel<DT, BWD, LC_, false, Tables, true><<<grid, kLeanThreads, 0, a.st>>>(ta, tb, tab, rot_chunks, cpr); \
         break;
                 switch (log_cpr) {
-                    LEAN(1) LEAN(2) LEAN(3) LEAN(4) LEAN(5) LEAN(6)
+                    LEAN(1) LEAN(2) LEAN(3) LEAN(4) LEAN(5)
                 }
 #undef LEAN
                 return launch_result();
             }
-            const int64_t per_pos = (rows * cpr + kLeanThreads * kLeanU - 1) / (kLeanThreads * kLeanU);
-            const dim3 grid((uint32_t)per_pos, (uint32_t)a.s, b ? 2u : 1u);
+            const int64_t rows_per_wg = (int64_t)4 * kLeanU * (64 / cpr);
+            const dim3 grid((uint32_t)((rows + rows_per_wg - 1) / rows_per_wg), (uint32_t)a.s, b ? 2u : 1u);
 #define LEAN(LC_)                                                                                             \
     case LC_:                                                                                                 \
         if (flat)                                                                                             \
-            rope_lean_kernel<DT, BWD, LC_, true, Tables><<<grid, kLeanThreads, 0, a.st>>>(ta, tb, tab, rot_chunks);  \
+            rope_lean_kernel<DT, BWD, LC_, true, Tables><<<grid, kLeanThreads, 0, a.st>>>(ta, tb, tab, rot_chunks, cpr);  \
         else                                                                                                  \
-            rope_lean_kernel<DT, BWD, LC_, false, Tables><<<grid, kLeanThreads, 0, a.st>>>(ta, tb, tab, rot_chunks); \
+            rope_lean_kernel<DT, BWD, LC_, false, Tables><<<grid, kLeanThreads, 0, a.st>>>(ta, tb, tab, rot_chunks, cpr); \
         break;
             switch (log_cpr) {
                 LEAN(1) LEAN(2) LEAN(3) LEAN(4) LEAN(5) LEAN(6)
+            default:  // not a power of two: the chunk count is a kernel argument
+                LEAN(-1)
             }
 #undef LEAN
             return launch_result();
@@ -948,6 +1028,18 @@ static int rope_launch_gather(const RopeArgs& a, const RopeArgs* b, const Tables
     pair.t[0] = rope_tensor(a);
     pair.t[1] = b ? rope_tensor(*b) : pair.t[0];
     const int rows = (b && pair.t[1].rows > pair.t[0].rows) ? pair.t[1].rows : pair.t[0].rows;
+    if (a.s <= 65535 && (int64_t)rows * cpr < ((int64_t)1 << 31)) {
+        // the launch shape of the lean kernel: two rows per thread, no loop
+        const int64_t rows_per_wg = (int64_t)4 * kLeanU * rpw;
+        const dim3 lgrid((uint32_t)((rows + rows_per_wg - 1) / rows_per_wg), (uint32_t)a.s, b ? 2u : 1u);
+        if (rope_flat(a) && (!b || rope_flat(*b)))
+            rope_lean_kernel<DT, BWD, -1, true, Tables, false, true><<<lgrid, kLeanThreads, 0, a.st>>>(
+                pair.t[0], pair.t[1], tab, (int)a.d2, cpr);
+        else
+            rope_lean_kernel<DT, BWD, -1, false, Tables, false, true><<<lgrid, kLeanThreads, 0, a.st>>>(
+                pair.t[0], pair.t[1], tab, (int)a.d2, cpr);
+        return launch_result();
+    }
     const int64_t steps = (rows + rows_per_step - 1) / rows_per_step;
     int64_t splits = (steps + 3) / 4;  // about four steps per workgroup, as in rope_vec_kernel
     splits = NHP_TUNED_INT("NHP_ROPE_SPLITS", (int)splits);

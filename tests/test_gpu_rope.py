@@ -199,6 +199,31 @@ def test_rope_qk_single_launch_equals_two_calls(hotpath, shape, dtype):
             assert torch.equal(util.raw_bits(got_k.cpu()), util.raw_bits(oracle.rope_cached(k.cpu(), cos.cpu(), sin.cpu(), backward, transpose)))
 
 
+@pytest.mark.parametrize("d,d2", [(16, 16), (32, 8), (24, 12), (16, 6), (8, 8), (32, 0)], ids=lambda v: str(v))
+def test_rope_more_positions_than_a_grid_dimension_and_no_rotary_part(hotpath, d, d2):
+    """The two-rows-per-thread kernel keeps the position in a grid dimension (at most 65535) and needs a rotary
+    part; longer sequences, head vectors of a single chunk and d2 = 0 take the looping vector kernels (or, for
+    a rotary half that is not a whole number of chunks, their gathering variant). Bit-exact like the others."""
+    dtype = torch.bfloat16
+    s, b, h = (65536 + 40, 1, 3) if d2 else (40, 2, 3)
+    t = util.randn((s, b, h, d), dtype, seed=d + d2)
+    cos, sin, _ = generic_tables(max(d2, 2), s, dtype, seed=d2)
+    cos, sin = cos[..., :d2].contiguous(), sin[..., :d2].contiguous()
+    td, cos_d, sin_d = t.to(DEV), cos.to(DEV), sin.to(DEV)
+    for backward in (False, True):
+        out = util._rope_out(td, False)
+        fn = hotpath.lib().nhp_rope_cached_bwd if backward else hotpath.lib().nhp_rope_cached_fwd
+        rc = fn(out.data_ptr(), td.data_ptr(), cos_d.data_ptr(), sin_d.data_ptr(), s, b, h, d, d2,
+                hotpath.strides4(td), hotpath.strides4(out), hotpath.BF16, hotpath.BF16, None)
+        assert rc == 0, hotpath.lib().nhp_status_string(rc)
+        torch.cuda.synchronize()
+        if d2:
+            want = oracle.rope_cached(t, cos, sin, backward)
+        else:
+            want = t
+        assert torch.equal(util.raw_bits(out.cpu()), util.raw_bits(want)), backward
+
+
 # (s, b, h, d, d2): head vectors of 2..64 chunks, rows that do not fill the last workgroup, partial rotary dimensions
 FUSED_QKV = [(16, 2, 8, 128, 128), (16, 2, 8, 128, 32), (5, 3, 7, 64, 64), (9, 1, 3, 32, 16), (3, 2, 5, 16, 16),
              (4, 2, 3, 256, 64), (3, 1, 2, 512, 512), (6, 2, 33, 128, 64), (64, 4, 16, 128, 128)]
