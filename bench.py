@@ -79,7 +79,7 @@ TRAFFIC_TABLE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
 # Workloads whose dominant kernel has no geometry query: a revision label that is changed by hand whenever
 # that kernel's launch shape or data flow changes, so that a traffic figure measured before is dropped.
 KERNEL_REVISIONS = {"mlp-gelu-1.4b": "bias_gelu_bwd r1", "swiglu-7b": "gated_bwd r1", "layernorm-1.4b": "norm_bwd r1",
-                    "rope-c4": "rope_lean r1", "layernorm-pair-1.4b": "norm_pair_bwd r1",
+                    "rope-c4": "rope_lean r2", "layernorm-pair-1.4b": "norm_pair_bwd r1",
                     "bias-residual-pair-1.4b": "bias_add_residual_pair r1"}
 
 

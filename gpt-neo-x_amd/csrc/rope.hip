@@ -503,6 +503,63 @@ rope_lean_kernel(RopeTensor ta, RopeTensor tb, Tables tab, int rot_arg, int cpr_
                 asm volatile("" : "+v"(res));
                 if (on[u]) store16_stream(op + dst[u], res);
             }
+        } else if ((d2 >> 1) % (4 / (int)sizeof(S)) == 0 && d2 % (4 / (int)sizeof(S)) == 0) {
+            // Half the rotary dimension is a whole number of 32-bit words (12 of 24 elements, 10 of 20): the
+            // partner of every word of the own chunk is a whole word somewhere in the head vector. Four 32-bit
+            // LDS reads with addresses fixed per lane replace the chunk exchange of the plain variant; the
+            // arithmetic is then the same, a whole chunk at a time. The sign of the rotated term is folded
+            // into the sine (r * (-s) is -(r * s) exactly, and a + (-b) is a - b).
+            constexpr int E = 4 / (int)sizeof(S);  // elements per word
+            u32x4 raw[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) raw[u] = load16_stream(ip + src[u]);
+            const int h2 = d2 >> 1;
+            const int h2w = h2 / E, d2w = d2 / E;
+            const int vecw0 = ((int)threadIdx.x - c) * 4;  // first staged word of this lane's head vector
+            int from[4];
+            bool turns[4];
+            float cv[V], sv[V];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int w = c * 4 + k;
+                turns[k] = w < d2w;
+                const bool first = w < h2w;
+                const int pw = turns[k] ? (first ? w + h2w : w - h2w) : w;
+                // lanes outside the rotary part read a word they do not use: one per lane and bank (their own
+                // chunk's words, 4 words apart from lane to lane, would make every such read a 4-way bank conflict)
+                from[k] = turns[k] ? vecw0 + pw : (int)threadIdx.x;
+                const bool negate = BWD ? !first : first;
+#pragma unroll
+                for (int e = 0; e < E; ++e) {
+                    const int i = w * E + e, pi = pw * E + e;
+                    cv[k * E + e] = turns[k] ? tcos[i] : 0.0f;
+                    const float sn = turns[k] ? tsin[BWD ? pi : i] : 0.0f;
+                    sv[k * E + e] = negate ? -sn : sn;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) stage[u][threadIdx.x] = raw[u];
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const uint32_t* words = reinterpret_cast<const uint32_t*>(&stage[u][0]);
+                u32x4 praw;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) praw[k] = words[from[k]];
+                float x[V], pr[V], y[V];
+                chunk_to_float<DT>(raw[u], x);
+                chunk_to_float<DT>(praw, pr);
+#pragma unroll
+                for (int v = 0; v < V; ++v) y[v] = rot<DT>(x[v], cv[v], pr[v], sv[v]);
+                const u32x4 rotated = float_to_chunk<DT>(y);
+                u32x4 res;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) res[k] = turns[k] ? rotated[k] : raw[u][k];
+                asm volatile("" : "+v"(res));
+                if (on[u]) store16_stream(op + dst[u], res);
+            }
         } else {
             u32x4 raw[U];
 #pragma unroll

@@ -154,7 +154,15 @@ def require_gpu(t, what):
         raise RuntimeError(f"{what}: expected a tensor on the GPU, got device {t.device}")
 
 
+# torch's direct accessor of the current stream's handle (what its own launchers use): about a microsecond
+# less per call than building a torch.cuda.Stream object first
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_of(t):
+    """The HIP stream torch would launch on for t's device right now, as a handle for the C ABI."""
+    if _raw_stream is not None:
+        return ctypes.c_void_p(_raw_stream(t.device.index))
     return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
 
 
