@@ -34,8 +34,8 @@ the drop-in extension modules (which call libneox_hotpath.so):
   masked-dropout-c3  padding-masked softmax + attention dropout (p = 0.1) in one kernel, fwd+bwd on the masked-c3 tensors
   rpe-bias-1.4b  causal softmax fwd+bwd [128,2048,2048] bf16 with a bias tensor [16,2048,2048] added in the kernel
 
-  hbm-probes     kernels that only move data (bench_probes/libneox_probe.so): a plain streaming copy of 64 MiB, 128 MiB and
-                 1 GiB tensors, and the causal softmax forward's access pattern (lower-triangle reads, dense writes)
+  hbm-probes     kernels that only move data (bench_probes/libneox_probe.so): a plain streaming copy of 16 MiB, 64 MiB,
+                 128 MiB and 1 GiB tensors, and the causal softmax forward's access pattern (lower-triangle reads, dense writes)
                  at [128,2048,2048] and [64,8192,8192], and the layout change of the transposing rotary kernel
                  ([128,128,2048] contiguous along the sequence -> [2048,128,128]): what the memory system gives for
                  those patterns and sizes
@@ -468,7 +468,7 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False, launc
         plib.nhp_probe_causal_pattern.argtypes = [vp, vp, i64, i64, vp]
         kernel_bytes = {}
         runs = []
-        for mib in (64, 128, 1024):
+        for mib in (16, 64, 128, 1024):  # 16 MiB: the tensor size of the [4,8,512,512] configuration
             nsets = max(2, 1024 // mib)  # rotate over more than the last-level cache holds
             # random data: what the bytes hold changes the time measurably (a copy of zeros is ~3 % faster)
             bufs = [(randn((mib << 19,), 300 + j, torch.bfloat16),
