@@ -118,6 +118,64 @@ def test_rope_random_shapes(hotpath, seed):
         assert torch.equal(util.raw_bits(got), util.raw_bits(want)), ("sequence-major", backward)
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_rope_two_tensor_launches_random_shapes(hotpath, seed):
+    """q and k through the two-tensor entry points in the layouts a caller may hand over: separate tensors, slices
+    of one buffer along the heads (k possibly with fewer heads), slices along the features in the order of a fused
+    projection (k directly behind q: read as one run per row) or in another order, both output layouts, both
+    table sources. Bit-exact against the oracle (cached tables) or the single-tensor entry point (angles)."""
+    rng = random.Random(3300 + seed)
+    dtype = rng.choice(ALL)
+    s, b, h = rng.randint(1, 40), rng.randint(1, 3), rng.randint(1, 6)
+    d = rng.choice((8, 16, 32, 64, 96, 128, 256, 80, 24))
+    d2 = rng.choice([v for v in (d, d // 2, d // 4, 8, 6) if 2 <= v <= d and v % 2 == 0])
+    layout = rng.choice(("separate", "heads", "features", "features-reversed", "features-gap"))
+    hk = h
+    if layout == "separate":
+        hk = rng.randint(1, h)
+        q = util.randn((s, b, h, d), dtype, seed=seed).to(DEV)
+        k = util.randn((s, b, hk, d), dtype, seed=seed + 50).to(DEV)
+    elif layout == "heads":
+        hk = rng.randint(1, h)
+        buf = util.randn((s, b, h + 2 * hk, d), dtype, seed=seed).to(DEV)
+        q, k = buf[:, :, :h], buf[:, :, h:h + hk]
+    else:
+        buf = util.randn((s, b, h, 4 * d), dtype, seed=seed).to(DEV)
+        if layout == "features":
+            q, k = buf[..., :d], buf[..., d:2 * d]
+        elif layout == "features-reversed":
+            q, k = buf[..., d:2 * d], buf[..., :d]
+        else:
+            q, k = buf[..., :d], buf[..., 2 * d:3 * d]
+    transpose = rng.random() < 0.4
+    print(f"rope two tensors s={s} b={b} h={h} hk={hk} d={d} d2={d2} {dtype} {layout} transpose={transpose}", flush=True)
+    g = torch.Generator().manual_seed(seed)
+    ang = (torch.rand((s, 1, 1, d2), generator=g) * 20 - 10).contiguous()
+    cs = torch.float32 if rng.random() < 0.3 else dtype
+    cos, sin = ang.cos().to(cs), ang.sin().to(cs)
+    cos_d, sin_d, ang_d = cos.to(DEV), sin.to(DEV), ang.to(DEV)
+    L = hotpath.lib()
+    code = hotpath.dtype_code(q, "t")
+    for backward in (False, True):
+        got_q, got_k = util._rope_out(q, transpose), util._rope_out(k, transpose)
+        fn = L.nhp_rope_cached_qk_bwd if backward else L.nhp_rope_cached_qk_fwd
+        rc = fn(got_q.data_ptr(), got_k.data_ptr(), q.data_ptr(), k.data_ptr(), cos_d.data_ptr(), sin_d.data_ptr(), s, b, h, hk,
+                d, d2, hotpath.strides4(q), hotpath.strides4(k), hotpath.strides4(got_q), hotpath.strides4(got_k), code,
+                hotpath.dtype_code(cos_d, "c"), None)
+        assert rc == 0, L.nhp_status_string(rc)
+        torch.cuda.synchronize()
+        assert torch.equal(util.raw_bits(got_q.cpu()), util.raw_bits(oracle.rope_cached(q.cpu(), cos, sin, backward, transpose)))
+        assert torch.equal(util.raw_bits(got_k.cpu()), util.raw_bits(oracle.rope_cached(k.cpu(), cos, sin, backward, transpose)))
+        got_q, got_k = util._rope_out(q, transpose), util._rope_out(k, transpose)
+        fn = L.nhp_rope_freqs_qk_bwd if backward else L.nhp_rope_freqs_qk_fwd
+        rc = fn(got_q.data_ptr(), got_k.data_ptr(), q.data_ptr(), k.data_ptr(), ang_d.data_ptr(), s, b, h, hk, d, d2,
+                hotpath.strides4(q), hotpath.strides4(k), hotpath.strides4(got_q), hotpath.strides4(got_k), code, None)
+        assert rc == 0, L.nhp_status_string(rc)
+        torch.cuda.synchronize()
+        assert torch.equal(util.raw_bits(got_q.cpu()), util.raw_bits(util.abi_rope_freqs(hotpath, q, ang_d, backward, transpose).cpu()))
+        assert torch.equal(util.raw_bits(got_k.cpu()), util.raw_bits(util.abi_rope_freqs(hotpath, k, ang_d, backward, transpose).cpu()))
+
+
 @pytest.mark.parametrize("seed", range(12))
 def test_rope_sequence_major_random_shapes(hotpath, seed):
     """Shapes inside and around the conditions of the transposing kernel (s a multiple of 8 or not, every head
