@@ -488,6 +488,18 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False, launc
         plib.nhp_probe_causal_bwd_pattern.argtypes = [vp, vp, i64, i64, vp]
         for _, _, _, a, s in pat:
             kernel_bytes[f"causal_bwd_pattern_{a}x{s}x{s}"] = causal_bytes(a, s)[1]
+        # the padding-mask forward's pattern on the tensors of masked-c3 (scores [16,32,1024,2048], 37 % padding keys)
+        plib.nhp_probe_masked_pattern.argtypes = [vp, vp, vp, i64, i64, i64, vp]
+        mb, mnp, msq, msk = 16, 32, 1024, 2048
+        g0 = torch.Generator().manual_seed(0)
+        mvalid = torch.randint(512, msk + 1, (mb,), generator=g0)
+        mmask = (torch.arange(msk)[None, :] >= mvalid[:, None])[:, None, None, :].expand(mb, 1, msq, msk).contiguous()
+        mmask[7] = True
+        mmask = mmask.to(dev)
+        mlive = int((~mmask.view(mb, msq, msk // 8, 8).all(dim=-1)).sum().item())
+        mx = pat[1][1].view(-1)[: mb * mnp * msq * msk].view(mb, mnp, msq, msk)   # 2 GiB of the 8 GiB random tensor
+        my = pat[1][2].view(-1)[: mb * mnp * msq * msk].view(mb, mnp, msq, msk)
+        kernel_bytes["masked_pattern_16x32x1024x2048"] = mlive * 16 * mnp + mmask.numel() + mx.numel() * 2
         plib.nhp_probe_seq_major_pattern.argtypes = [vp, vp, i64, i64, vp]
         plib.nhp_probe_streams.argtypes = [vp, vp, vp, vp, i64, ctypes.c_int, ctypes.c_int, vp]
         # 64 MiB streams (the hidden state [16384, 2048] bf16 of the layer kernels): n inputs -> one or no output
@@ -534,6 +546,8 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False, launc
                 # two triangles read, the first tensor's rows overwritten (XOR of random data stays random)
                 t.run(f"causal_bwd_pattern_{a}x{s}x{s}", lambda: hp.check(
                     plib.nhp_probe_causal_bwd_pattern(y.data_ptr(), x.data_ptr(), a, s, stream), "causal bwd pattern"))
+            t.run("masked_pattern_16x32x1024x2048", lambda: hp.check(plib.nhp_probe_masked_pattern(
+                my.data_ptr(), mx.data_ptr(), mmask.data_ptr(), mb, mnp, msq, stream), "masked pattern"))
             bufs4 = mix_bufs[state["i"] % len(mix_bufs)]
             for key, n_in, w in mixes:
                 t.run(key, lambda: hp.check(plib.nhp_probe_streams(bufs4[3].data_ptr(), bufs4[0].data_ptr(), bufs4[1].data_ptr(),

@@ -16,6 +16,8 @@
 //                             forward kernel is launched
 //   nhp_probe_causal_bwd_pattern  the causal softmax backward's traffic: the rows of two tensors read up to
 //                             the diagonal, the first tensor's rows overwritten in full
+//   nhp_probe_masked_pattern  the padding-mask softmax forward's traffic at [b, np, sq, 2048]: the mask row, the
+//                             chunks of the scores that are not all padding, the whole row written
 //   nhp_probe_seq_major_pattern  the traffic of the transposing rotary kernel: a [rows, 128, s]
 //                             tensor (contiguous along s) is read in runs of 64 positions per
 //                             feature and written as [s, rows, 128], whole 256-byte head vectors,
@@ -118,6 +120,45 @@ probe_causal_bwd_pattern_kernel(uint16_t* g, const uint16_t* y, uint32_t n)
     for (int k = 0; k < K; ++k) {
         const uint32_t col = (uint32_t)((k * W + w) * 64 + lane) * 8u;
         if (col < n) store16_stream(gr + col, a[k] ^ b[k]);
+    }
+}
+
+// The padding-mask softmax forward's traffic at 2048 keys: a workgroup of two waves takes one (batch entry,
+// query) row for two heads: it reads the row's 2048 mask bytes, then for each head the 16-byte chunks of the
+// scores whose 8 mask bytes are not all 1, and writes the whole row (two chunks per lane and wave, as the
+// library's kernel is launched; workgroups ordered (batch entry, head pair, query)).
+__global__ void __launch_bounds__(128)
+probe_masked_pattern_kernel(uint16_t* y, const uint16_t* x, const uint8_t* mask, uint32_t sq, uint32_t np)
+{
+    constexpr uint32_t n = 2048;
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t pairs = np / 2;
+    const uint32_t id = blockIdx.x;
+    const uint32_t bi = id / (pairs * sq);
+    const uint32_t r = id - bi * pairs * sq;
+    const uint32_t hp = r / sq, qi = r - hp * sq;
+    const uint8_t* mrow = mask + ((size_t)bi * sq + qi) * n;
+    bool live[2];
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        const uint32_t col = ((k * 2 + wave) * 64 + lane) * 8u;
+        const u32x2 v = load8(mrow + col);
+        live[k] = !(v[0] == 0x01010101u && v[1] == 0x01010101u);
+    }
+    for (uint32_t h = hp * 2; h < hp * 2 + 2; ++h) {
+        const size_t base = (((size_t)bi * np + h) * sq + qi) * n;
+        u32x4 raw[2];
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            const uint32_t col = ((k * 2 + wave) * 64 + lane) * 8u;
+            raw[k] = u32x4{0, 0, 0, 0};
+            if (live[k]) raw[k] = load16_stream(x + base + col);
+        }
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            const uint32_t col = ((k * 2 + wave) * 64 + lane) * 8u;
+            store16_stream(y + base + col, raw[k]);
+        }
     }
 }
 
@@ -276,6 +317,18 @@ int nhp_probe_causal_bwd_pattern(void* g, const void* y, int64_t batches, int64_
         probe_causal_bwd_pattern_kernel<2, 2><<<rows, 128, 0, st>>>(static_cast<uint16_t*>(g), static_cast<const uint16_t*>(y), 2048u);
     else
         probe_causal_bwd_pattern_kernel<2, 8><<<rows, 512, 0, st>>>(static_cast<uint16_t*>(g), static_cast<const uint16_t*>(y), 8192u);
+    return launch_result();
+}
+
+// y, x: [b, np, sq, 2048] 16-bit elements, mask: [b, 1, sq, 2048] bytes (1 = masked); np even.
+int nhp_probe_masked_pattern(void* y, const void* x, const void* mask, int64_t b, int64_t np, int64_t sq, void* stream)
+{
+    if (b < 1 || np < 2 || np % 2 != 0 || sq < 1 || b * (np / 2) * sq >= ((int64_t)1 << 31)) return NHP_ERR_SHAPE;
+    if (!y || !x || !mask) return NHP_ERR_NULL;
+    launch_prepare();
+    probe_masked_pattern_kernel<<<(uint32_t)(b * (np / 2) * sq), 128, 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<uint16_t*>(y), static_cast<const uint16_t*>(x), static_cast<const uint8_t*>(mask), (uint32_t)sq,
+        (uint32_t)np);
     return launch_result();
 }
 
