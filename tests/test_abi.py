@@ -246,3 +246,41 @@ def test_missing_library_fails_loudly(hotpath, monkeypatch, tmp_path):
     monkeypatch.setattr(hotpath, "LIB_PATH", str(tmp_path / "libneox_hotpath.so"))
     with pytest.raises(ImportError):
         hotpath.lib()
+
+
+def test_probe_library_exports_and_validates():
+    """bench.py's data-movement probes (bench_probes/libneox_probe.so, measurement equipment, not part of the
+    product library): every entry point bench.py binds exists, and bad arguments are refused before any launch."""
+    import ctypes
+    import subprocess
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    path = os.path.join(root, "bench_probes", "libneox_probe.so")
+    if not os.path.exists(path):
+        subprocess.run(["make", "-C", os.path.dirname(path)], check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+    lib = ctypes.CDLL(path)
+    vp, i64, ci = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+    sigs = {
+        "nhp_probe_copy": [vp, vp, i64, ci, vp],
+        "nhp_probe_streams": [vp, vp, vp, vp, i64, ci, ci, vp],
+        "nhp_probe_causal_pattern": [vp, vp, i64, i64, vp],
+        "nhp_probe_causal_bwd_pattern": [vp, vp, i64, i64, vp],
+        "nhp_probe_masked_pattern": [vp, vp, vp, i64, i64, i64, vp],
+        "nhp_probe_strided_runs": [vp, vp, vp, i64, ci, i64, ci, vp],
+        "nhp_probe_seq_major_pattern": [vp, vp, i64, i64, vp],
+    }
+    for name, args in sigs.items():
+        fn = getattr(lib, name)
+        fn.argtypes = args
+        fn.restype = ci
+    p = ctypes.c_void_p(0x1000)  # never dereferenced: every call below is refused
+    shape, null = -2, -3
+    assert lib.nhp_probe_copy(p, p, 24, 256, None) == shape          # not a multiple of 16 bytes
+    assert lib.nhp_probe_copy(None, p, 32, 256, None) == null
+    assert lib.nhp_probe_streams(p, p, p, p, 32, 4, 1, None) == shape
+    assert lib.nhp_probe_causal_pattern(p, p, 1, 1000, None) == shape
+    assert lib.nhp_probe_causal_bwd_pattern(p, None, 1, 2048, None) == null
+    assert lib.nhp_probe_masked_pattern(p, p, p, 1, 3, 8, None) == shape  # odd number of heads
+    assert lib.nhp_probe_strided_runs(p, None, p, 8, 24, 48, 0, None) == shape
+    assert lib.nhp_probe_strided_runs(p, None, p, 8, 32, 48, 1, None) == null
+    assert lib.nhp_probe_seq_major_pattern(p, p, 4, 100, None) == shape
