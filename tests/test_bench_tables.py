@@ -51,3 +51,25 @@ def test_algorithmic_byte_formulas(bench):
     assert bench.causal_bytes(64, 8192) == (12885426176, 17180917760)
     assert bench.rope_bytes(2048, 8, 16, 128, 32) == 134479872
     assert bench.tri(2048) == 2048 * 2049 // 2
+
+
+@pytest.mark.gpu
+def test_bench_measures_a_configuration_and_releases_its_tensors(bench):
+    """bench.py's per-configuration measurement (what fills the `configs` object of its default line) on its two
+    smallest workloads: every kernel reports bytes, a positive bracket and a fraction of the peak below 1, the
+    16 launches of the [4,8,512,512] bracket are divided out, and the tensors are released afterwards."""
+    import torch
+
+    dev = torch.device("cuda:0")
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated(dev)
+    c1 = bench.measure_workload("causal-c1", torch, dev, steps=2, warmup=1)
+    k = c1["kernels"]["causal_softmax_fwd"]
+    assert k["bytes"] == bench.causal_bytes(32, 512)[0] == 25182208
+    assert 1.0 < k["us"] < 100.0 and 0.0 < k["frac_of_peak"] < 1.0
+    rope = bench.measure_workload("rope-styles-1.4b", torch, dev, steps=2, warmup=1)
+    assert set(rope["kernels"]) == {"rope_fwd_per_tensor", "rope_bwd_per_tensor", "rope_fwd_one_launch", "rope_bwd_one_launch"}
+    for v in rope["kernels"].values():
+        assert v["bytes"] > 2 * 2048 * 8 * 16 * 128 * 2 * 2 and 10.0 < v["us"] < 1000.0 and 0.0 < v["frac_of_peak"] < 1.0
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated(dev) <= before + (1 << 20)
