@@ -374,6 +374,10 @@ int nhp_rope_cached_bwd(void* out, const void* in, const void* cos, const void* 
  * pass-through features after; with d2 < d the copy happens inside the
  * kernel. A position `offset` (KV-cache decoding, transformer.py:893-896) is
  * expressed by passing cos + offset*d2 and sin + offset*d2.
+ * When q_in and k_in are the slices [..., 0:d] and [..., d:2d] of one fused
+ * projection buffer (k_in == q_in + d elements, equal strides, hq == hk: how
+ * transformer.py:852-866 produces them) and the outputs share their strides,
+ * each row's q and k head vectors are read as one run; nothing else changes.
  */
 int nhp_rope_cached_qk_fwd(void* q_out, void* k_out, const void* q_in, const void* k_in,
                            const void* cos, const void* sin,
