@@ -45,7 +45,8 @@ the drop-in extension modules (which call libneox_hotpath.so):
   bias-residual-1.4b  residual + (x + bias) on the hidden state [2048*8, 2048] bf16
   bias-dropout-add-1.4b  residual + dropout(x + bias) with p = 0.1, and the dropout backward, same shape
   bias-residual-pair-1.4b  residual + ((x1 + bias1) + (x2 + bias2)): the parallel-residual layer's three additions in one pass
-  layernorm-1.4b  LayerNorm fwd and bwd (with the parameter gradients) on the hidden state [2048*8, 2048] bf16
+  layernorm-1.4b  LayerNorm fwd and bwd (with the parameter gradients, and for frozen parameters without) on the hidden
+                 state [2048*8, 2048] bf16
   layernorm-pair-1.4b  the two LayerNorms of the parallel-residual layer in one launch each way, same hidden state
   rmsnorm-7b     RMSNorm fwd and bwd on [4096*4, 4096] bf16 (the Llama-2 7B hidden size)
 
@@ -78,7 +79,7 @@ HBM_PEAK_GBS = 8000.0
 TRAFFIC_TABLE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
 # Workloads whose dominant kernel has no geometry query: a revision label that is changed by hand whenever
 # that kernel's launch shape or data flow changes, so that a traffic figure measured before is dropped.
-KERNEL_REVISIONS = {"mlp-gelu-1.4b": "bias_gelu_bwd r1", "swiglu-7b": "gated_bwd r1", "layernorm-1.4b": "norm_bwd r1",
+KERNEL_REVISIONS = {"mlp-gelu-1.4b": "bias_gelu_bwd r1", "swiglu-7b": "gated_bwd r1", "layernorm-1.4b": "norm_bwd r2",
                     "rope-c4": "rope_lean r2", "layernorm-pair-1.4b": "norm_pair_bwd r1",
                     "bias-residual-pair-1.4b": "bias_add_residual_pair r1"}
 
@@ -759,7 +760,8 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False, launc
         stats = rows * 4 * (2 if layer else 1)
         nparam = 2 if layer else 1
         kernel_bytes = {"norm_fwd": 2 * n * 2 + nparam * cols * 2 + stats,
-                        "norm_bwd": 3 * n * 2 + stats + (1 + nparam) * cols * 2}
+                        "norm_bwd": 3 * n * 2 + stats + (1 + nparam) * cols * 2,
+                        "norm_bwd_frozen_parameters": 3 * n * 2 + stats + cols * 2}
         state = {"i": 0}
         stream = hp.stream_of(y)
 
@@ -772,13 +774,16 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False, launc
                                          rows, cols, hp.BF16, hp.BF16, stream)
             hp.check(rc, "norm forward")
 
-        def bwd(x, g):
+        def bwd(x, g, params=True):
+            # params = False: the gradient of the input alone (frozen or absent parameters): another instantiation,
+            # one row block per workgroup, no column sums
+            dg, db = (dgamma.data_ptr(), dbeta.data_ptr()) if params else (None, None)
             if layer:
-                rc = lib.nhp_layernorm_bwd(dx.data_ptr(), dgamma.data_ptr(), dbeta.data_ptr(), g.data_ptr(), x.data_ptr(),
+                rc = lib.nhp_layernorm_bwd(dx.data_ptr(), dg, db, g.data_ptr(), x.data_ptr(),
                                            mean.data_ptr(), rstd.data_ptr(), gamma.data_ptr(), ws.data_ptr(), rows, cols,
                                            hp.BF16, hp.BF16, stream)
             else:
-                rc = lib.nhp_rmsnorm_bwd(dx.data_ptr(), dgamma.data_ptr(), None, g.data_ptr(), x.data_ptr(), rstd.data_ptr(),
+                rc = lib.nhp_rmsnorm_bwd(dx.data_ptr(), dg, None, g.data_ptr(), x.data_ptr(), rstd.data_ptr(),
                                          gamma.data_ptr(), ws.data_ptr(), 1e-8, 1, rows, cols, hp.BF16, hp.BF16, stream)
             hp.check(rc, "norm backward")
 
@@ -787,6 +792,7 @@ def make_workload(name, torch, dev, fresh_dy=False, rope_per_tensor=False, launc
             state["i"] += 1
             t.run("norm_fwd", lambda: fwd(x))
             t.run("norm_bwd", lambda: bwd(x, g))
+            t.run("norm_bwd_frozen_parameters", lambda: bwd(x, g, False))
 
         cfg = {"workload": name, "hidden_state": [rows, cols], "parameters": "bf16", "parameter_gradients": True,
                "bytes_convention": "every tensor element read or written once, plus the fp32 row statistics"}

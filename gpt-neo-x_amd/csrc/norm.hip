@@ -345,11 +345,16 @@ struct NormBwdArgs {
 // Waves per workgroup of the backward kernel: as many row groups as the LDS buffer of the final
 // accumulator reduction (K * V floats per thread, at most 32 KiB) and 512 threads allow (workgroups
 // of 1024 threads measured slower), or the W waves of one row if that is more.
-template <int K, int W, int V>
+// Without parameter gradients (PARAMS = false: nothing is carried from row to row, a workgroup is only the
+// unit that shares a barrier) at most 4 waves: the row groups of a workgroup then wait for each other less,
+// 39.2 -> 34.9 us at [16384, 2048], 75.2 -> 67.9 us at [16384, 4096]. With parameter gradients smaller
+// workgroups mean more partial rows and lose (42.3 -> 51.5 us at 2048 columns).
+template <int K, int W, int V, bool PARAMS = true>
 constexpr int bwd_waves()
 {
     int g = 8192 / (K * V) / kWave;  // threads by the LDS bound, in waves
-    if (g > 8) g = 8;
+    const int cap = PARAMS ? 8 : 4;
+    if (g > cap) g = cap;
     g = g / W * W;                    // whole row groups
     return g < W ? W : g;
 }
@@ -361,13 +366,14 @@ constexpr int bwd_rows_in_flight(int k, int w, bool pair) { return (pair || k * 
 
 // PAIR (LayerNorm only): g = dy * gamma + dy2 * gamma2, one dx for both norms, and the parameter
 // gradients of the second norm beside those of the first.
-template <int DT, int K, int W, bool RMS, bool PAIR = false, int U = bwd_rows_in_flight(K, W, PAIR)>
-__global__ void __launch_bounds__((bwd_waves<K, W, Elt<DT>::kVec>() * kWave))
+// PARAMS = false: no parameter gradients are wanted; the column sums and everything around them are left out.
+template <int DT, int K, int W, bool RMS, bool PAIR = false, bool PARAMS = true, int U = bwd_rows_in_flight(K, W, PAIR)>
+__global__ void __launch_bounds__((bwd_waves<K, W, Elt<DT>::kVec, PARAMS>() * kWave))
 norm_bwd_kernel(NormBwdArgs a)
 {
     static_assert(!PAIR || !RMS, "pairs of LayerNorms only");
     constexpr int V = Elt<DT>::kVec;
-    constexpr int G = bwd_waves<K, W, V>();
+    constexpr int G = bwd_waves<K, W, V, PARAMS>();
     constexpr int T = G * kWave;
     constexpr int GROUPS = G / W;
     using S = typename Elt<DT>::storage;
@@ -378,7 +384,7 @@ norm_bwd_kernel(NormBwdArgs a)
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const size_t cols = (size_t)a.cpr * V;
     const float n = RMS ? (float)a.stat : (float)cols;
-    const bool param_grads = a.part_g != nullptr;
+    const bool param_grads = PARAMS && a.part_g != nullptr;
 
     // this thread's chunk columns do not depend on the row block
     const RowSlot first = locate<W, G>(0, a.rows, a.L, a.logL, wave, lane);
@@ -464,13 +470,17 @@ norm_bwd_kernel(NormBwdArgs a)
                         float g = fg[j] * gam[k][j];
                         if constexpr (PAIR) {
                             g = g + fg2[j] * gam2[k][j];
-                            acc_g2[k][j] += fg2[j] * xh;
-                            acc_b2[k][j] += fg2[j];
+                            if constexpr (PARAMS) {
+                                acc_g2[k][j] += fg2[j] * xh;
+                                acc_b2[k][j] += fg2[j];
+                            }
                         }
                         s1[u] += g;
                         s2[u] += g * xh;
-                        acc_g[k][j] += fg[j] * xh;
-                        acc_b[k][j] += fg[j];
+                        if constexpr (PARAMS) {
+                            acc_g[k][j] += fg[j] * xh;
+                            acc_b[k][j] += fg[j];
+                        }
                     }
                 }
             }
@@ -531,7 +541,9 @@ norm_bwd_kernel(NormBwdArgs a)
     }
 
     if (!param_grads) return;
-    if constexpr (W > 1 && GROUPS == 1) {
+    if constexpr (!PARAMS) {
+        return;
+    } else if constexpr (W > 1 && GROUPS == 1) {
         // one row group: every thread owns its columns alone
 #pragma unroll
         for (int k = 0; k < K; ++k) {
@@ -724,10 +736,11 @@ static uint32_t norm_row_blocks(int64_t rows, const NormPlan& p, int waves)
     return (uint32_t)((rows + rows_per_block - 1) / rows_per_block);
 }
 
-static int bwd_waves_of(const NormPlan& p, int v)
+static int bwd_waves_of(const NormPlan& p, int v, bool params = true)
 {
     int g = 8192 / (p.K * v) / kWave;
-    if (g > 8) g = 8;
+    const int cap = params ? 8 : 4;
+    if (g > cap) g = cap;
     g = g / p.W * p.W;
     return g < p.W ? p.W : g;
 }
@@ -823,7 +836,7 @@ static int norm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, const v
     if (cols % V == 0 && ptr_aligned16(dx) && ptr_aligned16(dy) && ptr_aligned16(x) && ptr_aligned16(gamma) &&
         ptr_aligned16(second.dy2) && ptr_aligned16(second.gamma2) && ptr_aligned16(workspace) &&
         plan_norm(cols / V, true, p, pair)) {
-        const int waves = bwd_waves_of(p, V);
+        const int waves = bwd_waves_of(p, V, want_params);
         const uint32_t row_blocks = norm_row_blocks(rows, p, waves);
         uint32_t grid = norm_bwd_grid(row_blocks, want_params, waves, bwd_rows_in_flight(p.K, p.W, pair),
                                       (pair && p.K >= 2) || p.K >= 4);
@@ -843,12 +856,19 @@ static int norm_bwd(void* dx, void* dgamma, void* dbeta, const void* dy, const v
 #define X(K_, W_)                                                                      \
     if (!launched && p.K == K_ && p.W == W_) {                                         \
         if constexpr (!RMS) {                                                          \
-            if (pair)                                                                  \
-                norm_bwd_kernel<DT, K_, W_, false, true><<<grid, threads, 0, st>>>(a); \
+            if (pair && want_params)                                                   \
+                norm_bwd_kernel<DT, K_, W_, false, true, true><<<grid, threads, 0, st>>>(a); \
+            else if (pair)                                                             \
+                norm_bwd_kernel<DT, K_, W_, false, true, false><<<grid, threads, 0, st>>>(a); \
+            else if (want_params)                                                      \
+                norm_bwd_kernel<DT, K_, W_, false, false, true><<<grid, threads, 0, st>>>(a); \
             else                                                                       \
-                norm_bwd_kernel<DT, K_, W_, false, false><<<grid, threads, 0, st>>>(a); \
+                norm_bwd_kernel<DT, K_, W_, false, false, false><<<grid, threads, 0, st>>>(a); \
         } else {                                                                       \
-            norm_bwd_kernel<DT, K_, W_, RMS><<<grid, threads, 0, st>>>(a);             \
+            if (want_params)                                                           \
+                norm_bwd_kernel<DT, K_, W_, RMS, false, true><<<grid, threads, 0, st>>>(a); \
+            else                                                                       \
+                norm_bwd_kernel<DT, K_, W_, RMS, false, false><<<grid, threads, 0, st>>>(a); \
         }                                                                              \
         launched = true;                                                               \
     }

@@ -53,7 +53,7 @@ def abi_layernorm(hp, x, dy, gamma, beta, eps, want_params=True):
     return y, mean, rstd, dx, dg, db
 
 
-def abi_rmsnorm(hp, x, dy, scale, offset, eps, mode, stat=None):
+def abi_rmsnorm(hp, x, dy, scale, offset, eps, mode, stat=None, want_params=True):
     if stat is not None:
         return abi_rmsnorm_partial(hp, x, dy, scale, offset, eps, mode, stat)
     rows, cols = x.shape
@@ -66,10 +66,10 @@ def abi_rmsnorm(hp, x, dy, scale, offset, eps, mode, stat=None):
     assert rc == 0, L.nhp_status_string(rc)
     dx = torch.empty_like(x)
     pd = scale.dtype if scale is not None else x.dtype
-    ds = torch.full((cols,), float("nan"), dtype=pd, device=x.device)
-    do = torch.full((cols,), float("nan"), dtype=pd, device=x.device)
+    ds = torch.full((cols,), float("nan"), dtype=pd, device=x.device) if want_params else None
+    do = torch.full((cols,), float("nan"), dtype=pd, device=x.device) if want_params else None
     ws = torch.empty(max(L.nhp_norm_bwd_workspace_bytes(rows, cols, code), 1), dtype=torch.uint8, device=x.device)
-    rc = L.nhp_rmsnorm_bwd(dx.data_ptr(), ds.data_ptr(), do.data_ptr(), dy.data_ptr(), x.data_ptr(), inv.data_ptr(),
+    rc = L.nhp_rmsnorm_bwd(dx.data_ptr(), ptr(ds), ptr(do), dy.data_ptr(), x.data_ptr(), inv.data_ptr(),
                            ptr(scale), ws.data_ptr(), eps, mode, rows, cols, code, pcode, None)
     assert rc == 0, L.nhp_status_string(rc)
     return y, inv, dx, ds, do
@@ -136,6 +136,9 @@ def test_layernorm_vs_oracle(hotpath, shape, dtype, pd):
     col = (dy.float().abs() * ((x.float() - mean[:, None]) * rstd[:, None]).abs()).sum(0) * 32 * util.EPS32
     util.assert_close_ulp_or_noise(dg, want_dg, 2, col, "dgamma")
     util.assert_close_ulp_or_noise(db, want_db, 2, dy.float().abs().sum(0) * 32 * util.EPS32, "dbeta")
+    # without parameter gradients another instantiation runs (smaller workgroups, no column sums): the same dx bit for bit
+    alone = abi_layernorm(hotpath, x.to(DEV), dy.to(DEV), gamma.to(DEV), beta.to(DEV), eps, want_params=False)[3].cpu()
+    assert torch.equal(util.raw_bits(alone), util.raw_bits(dx)), "dx without parameter gradients"
 
 
 def abi_layernorm_pair(hp, x, dy1, dy2, gamma1, beta1, gamma2, beta2, eps, want=(True, True, True, True)):
@@ -195,6 +198,9 @@ def test_layernorm_pair_vs_oracle(hotpath, shape, dtype, pd):
     # and a second run reproduces every result (fixed summation order)
     again = abi_layernorm_pair(hotpath, *dev, eps)
     assert torch.equal(again[4], dx) and all(torch.equal(a, b) for a, b in zip(again[5], grads))
+    # without any parameter gradient (another instantiation: smaller workgroups, no column sums) the same dx bit for bit
+    alone = abi_layernorm_pair(hotpath, *dev, eps, want=(False, False, False, False))
+    assert torch.equal(util.raw_bits(alone[4]), util.raw_bits(dx)), "dx without parameter gradients"
 
 
 def test_layernorm_pair_optional_gradients_and_module(hotpath):
@@ -255,6 +261,8 @@ def test_rmsnorm_vs_oracle(hotpath, shape, dtype, mode):
     col = (dy.float().abs() * (x.float() * inv[:, None]).abs()).sum(0) * 32 * util.EPS32
     util.assert_close_ulp_or_noise(ds, want_ds, 2, col, "dscale")
     util.assert_close_ulp_or_noise(do, want_do, 2, dy.float().abs().sum(0) * 32 * util.EPS32, "doffset")
+    alone = abi_rmsnorm(hotpath, x.to(DEV), dy.to(DEV), scale.to(DEV), offset.to(DEV), eps, mode, want_params=False)[2].cpu()
+    assert torch.equal(util.raw_bits(alone), util.raw_bits(dx)), "dx without parameter gradients"
 
 
 @pytest.mark.parametrize("mode", [0, 1])
